@@ -1,0 +1,439 @@
+"""anemone_amd -- Python bindings of libanemone_hip.so, the MI355X backend and operator prepare functions of the
+routed-expert path. Everything here goes through the library's C ABI (include/anemone_backend.h,
+include/anemone_ops.h, include/anemone_records.h); there is no CPU fallback: without the built library, or without
+a card, the calls fail."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(HERE, "libanemone_hip.so")
+
+STATUS_OK, STATUS_INVALID_ARGUMENT, STATUS_OUT_OF_MEMORY = 0, 1, 2
+STATUS_DEVICE_ERROR, STATUS_TIMED_OUT, STATUS_UNSUPPORTED, STATUS_BUSY = 5, 6, 7, 8
+WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED = 2, 3, 5
+ARITHMETIC_CLASS_GFX950 = 950
+BACKEND_NO_KERNEL = 0xFFFFFFFF
+EXL3_EXPERT_LAUNCHES, EXL3_TC_LAUNCHES = 5, 5
+EXL3_TC_GATE_UP_SLICES, EXL3_TC_DOWN_SLICES = 8, 4
+AFFINITY_SQRT_SOFTPLUS, AFFINITY_SIGMOID = 0, 1
+SECOND = 1_000_000_000
+
+u8, u32, u64, f32 = C.c_uint8, C.c_uint32, C.c_uint64, C.c_float
+
+
+class AnemoneError(RuntimeError):
+    def __init__(self, what, status):
+        super().__init__("%s: status %d (%s)" % (what, status, status_text(status)))
+        self.status = status
+
+
+class KernelLaunch(C.Structure):
+    _fields_ = [("kernel", u32), ("grid", u32 * 3), ("block", u32 * 3), ("dynamic_shared_byte_count", u32),
+                ("argument_byte_count", u32), ("branch", u32), ("argument", u8 * 192)]
+
+
+class CardDescription(C.Structure):
+    _fields_ = [("name", C.c_char * 96), ("bus_address", C.c_char * 32), ("arithmetic_class", u32),
+                ("link_generation", u32), ("link_lane_count", u32), ("reserved_zero", u32),
+                ("memory_total_bytes", u64), ("memory_free_bytes", u64), ("memory_reserved_bytes", u64)]
+
+
+class Range(C.Structure):
+    _fields_ = [("byte_offset", u64), ("byte_count", u64)]
+
+
+class Shape(C.Structure):
+    _fields_ = [("output_size", u32), ("input_size", u32), ("bits_per_weight", u32), ("reserved_must_be_zero", u32)]
+
+
+class Exl3ReconstructRecord(C.Structure):
+    _fields_ = [("matrix_offset", u64), ("output_offset", u64), ("input_size", u32), ("output_size", u32),
+                ("bits_per_weight", u32), ("reserved_zero", u32)]
+
+
+class Exl3ExpertRecord(C.Structure):
+    _fields_ = [("jobs_offset", u64), ("input_offset", u64), ("operands_offset", u64), ("products_offset", u64),
+                ("hidden_offset", u64), ("output_offset", u64), ("input_size", u32), ("inner_size", u32),
+                ("pair_count", u32), ("pairs_per_row", u32), ("job_count", u32), ("bits_per_weight", u32),
+                ("activation_limit", f32), ("reserved_zero", u32), ("widths_offset", u64)]
+
+
+class RowSumArguments(C.Structure):
+    _fields_ = [("pair_output_offset", u64), ("row_output_offset", u64), ("width", u32), ("pairs_per_row", u32)]
+
+
+class Exl3TcRecord(C.Structure):
+    _fields_ = [("jobs_offset", u64), ("hidden_offset", u64), ("workspace_offset", u64), ("output_offset", u64),
+                ("row_count", u32), ("job_capacity", u32), ("intermediate", u32), ("bits_x2", u32),
+                ("activation_limit", f32), ("pass_", u32), ("rotation", u32), ("shared_sum", u32),
+                ("shared_offset", u64), ("widths_offset", u64), ("hidden", u32), ("pairs_per_row", u32)]
+
+
+class RouterKernels(C.Structure):
+    _fields_ = [(name, u32) for name in ("select", "wide_select", "wide_count", "wide_place", "wide_jobs",
+                                         "wide_small", "select_draft", "projection")]
+
+
+class RoutedExpertsDescription(C.Structure):
+    _fields_ = [(name, Range) for name in ("jobs", "expert_weights", "codes", "exponents", "operands", "hidden",
+                                           "hidden_codes", "hidden_exponents", "hidden_operands", "pair_output",
+                                           "row_output")] + \
+               [("gate_up_shape", Shape), ("down_shape", Shape), ("weight_format", C.c_int), ("job_count", u32),
+                ("row_count", u32), ("pairs_per_row", u32), ("gate_up_slice_count", u32), ("down_slice_count", u32),
+                ("activation_limit", f32), ("reserved_zero", u32)]
+
+
+class RouterDescription(C.Structure):
+    _fields_ = [("experts", C.POINTER(RoutedExpertsDescription)), ("expert_offsets", C.POINTER(u64)),
+                ("expert_widths", C.POINTER(u32)), ("step", Range), ("scores", Range), ("bias", Range),
+                ("offsets", Range), ("affinities", Range), ("order", C.c_int), ("expert_count", u32),
+                ("pick_count", u32), ("affinity_kind", u32), ("route_scale", f32)]
+
+
+class RouterProjectionDescription(C.Structure):
+    _fields_ = [("weights", Range), ("rows", Range), ("output", Range), ("row_count", u32), ("hidden", u32),
+                ("expert_count", u32), ("reserved_zero", u32)]
+
+
+JOB_DTYPE = np.dtype([("gate_offset", "<u8"), ("up_offset", "<u8"), ("down_offset", "<u8"), ("row_count", "<u4"),
+                      ("expert", "<u4"), ("pair_index", "<u4", (8,)), ("route_weight", "<f4", (8,))])
+
+_lib = None
+
+
+def library():
+    """The loaded library. Raises if it was not built: there is no other implementation to fall back to."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIBRARY_PATH):
+            raise ImportError("%s is missing: run `python -m anemone_amd.build` (hipcc, gfx950)" % LIBRARY_PATH)
+        lib = C.CDLL(LIBRARY_PATH)
+        vp, launch_p = C.c_void_p, C.POINTER(KernelLaunch)
+        lib.status_text.restype = C.c_char_p
+        lib.status_text.argtypes = [C.c_int]
+        signatures = {
+            "backend_hip_card_count": [C.POINTER(u32)],
+            "backend_hip_card_describe": [u32, C.POINTER(CardDescription)],
+            "backend_hip_card_open": [u32, u64, C.POINTER(vp)],
+            "backend_hip_staging_allocate": [u64, C.POINTER(vp)],
+            "backend_hip_upload_begin": [vp, u64, vp, u64, C.POINTER(u64)],
+            "backend_hip_upload_wait": [vp, u64, u64],
+            "backend_hip_download_begin": [vp, u64, vp, u64, C.POINTER(u64)],
+            "backend_hip_kernel_prepare": [vp, C.c_char_p, C.c_char_p, u32, C.POINTER(u32)],
+            "backend_hip_launch_run": [vp, launch_p, u32],
+            "backend_hip_launch_run_timed": [vp, launch_p, u32, C.POINTER(C.c_double)],
+            "backend_hip_launch_wait": [vp, u64],
+            "backend_hip_graph_capture": [vp, launch_p, u32, C.POINTER(u32)],
+            "backend_hip_graph_run": [vp, u32],
+            "backend_hip_measure_begin": [vp],
+            "backend_hip_measure_end": [vp],
+            "backend_hip_measure_elapsed_us": [vp, u64, C.POINTER(C.c_double)],
+            "backend_hip_kernel_table_entry": [u32, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p), C.POINTER(u32)],
+            "exl3_reconstruct_prepare": [C.POINTER(Exl3ReconstructRecord), u64, u32, launch_p],
+            "exl3_experts_prepare": [C.POINTER(Exl3ExpertRecord), u64, vp, vp, u32, launch_p],
+            "exl3_experts_fast_prepare": [C.POINTER(Exl3ExpertRecord), u64, vp, vp, u32, launch_p],
+            "exl3_experts_relaxed_prepare": [C.POINTER(Exl3ExpertRecord), u64, vp, vp, u32, launch_p],
+            "exl3_row_sum_prepare": [C.POINTER(RowSumArguments), u32, u64, vp, vp, launch_p],
+            "exl3_tc_prepare": [C.POINTER(Exl3TcRecord), u64, vp, vp, launch_p],
+            "exl3_tc_prepare_short": [C.POINTER(Exl3TcRecord), u64, vp, vp, launch_p],
+            "exl3_tc_prepare_paired": [C.POINTER(Exl3TcRecord), u64, vp, vp, launch_p],
+            "router_kernels_prepare": [vp, vp, C.POINTER(RouterKernels)],
+            "router_select_prepare": [C.POINTER(RouterDescription), u64, C.POINTER(RouterKernels), launch_p],
+            "router_projection_prepare": [C.POINTER(RouterProjectionDescription), u64, C.POINTER(RouterKernels), launch_p],
+        }
+        for name, argtypes in signatures.items():
+            function = getattr(lib, name)
+            function.restype = C.c_int
+            function.argtypes = argtypes
+        lib.backend_hip_card_close.restype = None
+        lib.backend_hip_card_close.argtypes = [vp, u64]
+        lib.backend_hip_staging_free.restype = None
+        lib.backend_hip_staging_free.argtypes = [vp]
+        lib.backend_hip_format_supported.restype = C.c_bool
+        lib.backend_hip_format_supported.argtypes = [u32, C.c_int]
+        lib.backend_hip_kernel_table_count.restype = u32
+        lib.exl3_scratch_byte_count.restype = u64
+        lib.exl3_scratch_byte_count.argtypes = [u32, u32]
+        lib.exl3_width_name.restype = C.c_char_p
+        lib.exl3_width_name.argtypes = [u32]
+        _lib = lib
+    return _lib
+
+
+def status_text(status):
+    return library().status_text(status).decode()
+
+
+def check(status, what):
+    if status != STATUS_OK:
+        raise AnemoneError(what, status)
+
+
+def backend_table():
+    """Address of `backend_hip_value`, the table a prepare function takes as its backend."""
+    return C.addressof(C.c_char.in_dll(library(), "backend_hip_value"))
+
+
+def card_count():
+    count = u32(0)
+    check(library().backend_hip_card_count(C.byref(count)), "card_count")
+    return count.value
+
+
+def exl3_tc_workspace_bytes(pairs, hidden, intermediate):
+    align = lambda n: (n + 255) // 256 * 256
+    return (align(2 * pairs * hidden * 2) + align(EXL3_TC_GATE_UP_SLICES * 2 * pairs * intermediate * 4) +
+            align(EXL3_TC_DOWN_SLICES * pairs * hidden * 4))
+
+
+class Card:
+    """One open card: its arena, a staging block for copies, and a bump allocator over the arena."""
+
+    def __init__(self, arena_bytes, index=0, staging_bytes=64 << 20):
+        self.lib = library()
+        if card_count() <= index:
+            raise AnemoneError("no card %d on this machine" % index, STATUS_UNSUPPORTED)
+        self.arena_bytes = int(arena_bytes)
+        self.handle = C.c_void_p()
+        check(self.lib.backend_hip_card_open(index, self.arena_bytes, C.byref(self.handle)), "card_open")
+        self.staging = C.c_void_p()
+        self.staging_bytes = int(staging_bytes)
+        check(self.lib.backend_hip_staging_allocate(self.staging_bytes, C.byref(self.staging)), "staging_allocate")
+        self.staging_view = np.ctypeslib.as_array(C.cast(self.staging, C.POINTER(u8)), shape=(self.staging_bytes,))
+        self.cursor = 256
+
+    def close(self):
+        if self.handle:
+            self.lib.backend_hip_card_close(self.handle, 10 * SECOND)
+            self.lib.backend_hip_staging_free(self.staging)
+            self.handle = C.c_void_p()
+
+    def describe(self, index=0):
+        description = CardDescription()
+        check(self.lib.backend_hip_card_describe(index, C.byref(description)), "card_describe")
+        return description
+
+    def reserve(self, byte_count, alignment=256):
+        """A range of the arena: the planner's job in the reference, a bump allocation here."""
+        offset = (self.cursor + alignment - 1) // alignment * alignment
+        if offset + byte_count > self.arena_bytes:
+            raise AnemoneError("the arena is full", STATUS_OUT_OF_MEMORY)
+        self.cursor = offset + int(byte_count)
+        return offset
+
+    def upload(self, offset, array):
+        data = np.ascontiguousarray(array).view(np.uint8).reshape(-1)
+        ticket = u64(0)
+        for start in range(0, data.size, self.staging_bytes):
+            piece = data[start:start + self.staging_bytes]
+            self.staging_view[:piece.size] = piece
+            check(self.lib.backend_hip_upload_begin(self.handle, offset + start, self.staging, piece.size, C.byref(ticket)), "upload_begin")
+            check(self.lib.backend_hip_upload_wait(self.handle, ticket, 60 * SECOND), "upload_wait")
+
+    def place(self, array, alignment=256):
+        array = np.ascontiguousarray(array)
+        offset = self.reserve(array.nbytes, alignment)
+        self.upload(offset, array)
+        return offset
+
+    def download(self, offset, byte_count, dtype=np.uint8):
+        out = np.empty(int(byte_count), dtype=np.uint8)
+        ticket = u64(0)
+        for start in range(0, out.size, self.staging_bytes):
+            size = min(self.staging_bytes, out.size - start)
+            check(self.lib.backend_hip_download_begin(self.handle, offset + start, self.staging, size, C.byref(ticket)), "download_begin")
+            check(self.lib.backend_hip_upload_wait(self.handle, ticket, 60 * SECOND), "download wait")
+            out[start:start + size] = self.staging_view[:size]
+        return out.view(dtype)
+
+    def kernel(self, file, function, record_bytes):
+        handle = u32(BACKEND_NO_KERNEL)
+        check(self.lib.backend_hip_kernel_prepare(self.handle, file.encode(), function.encode(), record_bytes, C.byref(handle)),
+              "kernel_prepare %s" % function)
+        return handle.value
+
+    def run(self, launches, wait=True):
+        array = launches if isinstance(launches, C.Array) else (KernelLaunch * len(launches))(*launches)
+        check(self.lib.backend_hip_launch_run(self.handle, array, len(array)), "launch_run")
+        if wait:
+            self.wait()
+
+    def wait(self, seconds=60):
+        check(self.lib.backend_hip_launch_wait(self.handle, seconds * SECOND), "launch_wait")
+
+    def run_timed(self, launches):
+        array = launches if isinstance(launches, C.Array) else (KernelLaunch * len(launches))(*launches)
+        out = (C.c_double * len(array))()
+        check(self.lib.backend_hip_launch_run_timed(self.handle, array, len(array), out), "launch_run_timed")
+        return list(out)
+
+    def capture(self, launches):
+        array = launches if isinstance(launches, C.Array) else (KernelLaunch * len(launches))(*launches)
+        graph = u32(0)
+        check(self.lib.backend_hip_graph_capture(self.handle, array, len(array), C.byref(graph)), "graph_capture")
+        return graph.value
+
+    def run_graph(self, graph, wait=True):
+        check(self.lib.backend_hip_graph_run(self.handle, graph), "graph_run")
+        if wait:
+            self.wait()
+
+    def measure(self, body):
+        """Device microseconds of whatever `body()` queues on the card."""
+        check(self.lib.backend_hip_measure_begin(self.handle), "measure_begin")
+        body()
+        check(self.lib.backend_hip_measure_end(self.handle), "measure_end")
+        out = C.c_double(0)
+        check(self.lib.backend_hip_measure_elapsed_us(self.handle, 120 * SECOND, C.byref(out)), "measure_elapsed_us")
+        return out.value
+
+
+def step_block(live_rows):
+    """struct step_block {u64 sequence; u32 row_count; u32 flags} as bytes."""
+    return np.frombuffer(np.array([0], dtype="<u8").tobytes() + np.array([live_rows, 0], dtype="<u4").tobytes(), dtype=np.uint8)
+
+
+def launches_of(count):
+    return (KernelLaunch * count)()
+
+
+class Exl3Layer:
+    """One EXL3 MoE layer laid out in a card's arena the way the reference's loader lays one out: the experts'
+    stored matrices, the [E][3] offsets table, an optional per-matrix widths table, the router's weights and bias;
+    and the scratch ranges of a step of at most `rows` rows. Builds the prepared launches through the library's
+    prepare functions."""
+
+    def __init__(self, card, hidden, inner, expert_count, picks, rows, matrices, widths, router_weights_bf16=None,
+                 bias=None, affinity_kind=AFFINITY_SIGMOID, route_scale=1.5, limit=10.0):
+        self.card, self.H, self.I, self.E, self.P, self.rows = card, hidden, inner, expert_count, picks, rows
+        self.limit, self.affinity_kind, self.route_scale = limit, affinity_kind, route_scale
+        self.pairs = rows * picks
+        lib = card.lib
+        widths = np.asarray(widths, dtype=np.uint32).reshape(expert_count, 3)
+        self.widths = widths
+        self.uniform_width = int(widths[0, 0]) if np.all(widths == widths[0, 0]) else 0
+        total = sum(m.nbytes + 64 for trio in matrices for m in trio)
+        self.weights_offset = card.reserve(total, 256)
+        offsets = np.zeros((expert_count, 3), dtype=np.uint64)
+        cursor = self.weights_offset
+        blob = np.zeros(total, dtype=np.uint8)
+        for e, trio in enumerate(matrices):
+            for m, matrix in enumerate(trio):
+                cursor = (cursor + 63) // 64 * 64
+                offsets[e, m] = cursor
+                blob[cursor - self.weights_offset:cursor - self.weights_offset + matrix.nbytes] = matrix
+                cursor += matrix.nbytes
+        self.weights_bytes = total
+        card.upload(self.weights_offset, blob)
+        self.expert_offsets = offsets
+        self.offsets_offset = card.place(offsets)
+        packed = (widths[:, 0] | (widths[:, 1] << 8) | (widths[:, 2] << 16)).astype(np.uint32)
+        self.packed_widths = packed
+        self.widths_offset = card.place(packed) if self.uniform_width == 0 else 0
+        self.step_offset = card.place(step_block(rows))
+        self.x_offset = card.reserve(rows * hidden * 2)
+        self.scores_offset = card.reserve(rows * expert_count * 4)
+        self.affinities_offset = card.reserve(rows * expert_count * 4)
+        self.bias_offset = card.place(np.zeros(expert_count, dtype=np.float32) if bias is None else np.asarray(bias, dtype=np.float32))
+        self.router_offset = card.place(router_weights_bf16) if router_weights_bf16 is not None else 0
+        self.jobs_offset = card.reserve(self.pairs * 96)
+        self.out_offset = card.reserve(rows * hidden * 4)
+        # chain scratch
+        self.scratch_offset = card.reserve(int(lib.exl3_scratch_byte_count(self.pairs, hidden)))
+        self.hidden_offset = card.reserve(self.pairs * inner * 2)
+        # fused decode workspace
+        self.workspace_offset = card.reserve(exl3_tc_workspace_bytes(self.pairs, hidden, inner))
+        self.kernels = RouterKernels()
+        check(lib.router_kernels_prepare(backend_table(), card.handle, C.byref(self.kernels)), "router_kernels_prepare")
+
+    def set_rows(self, x_bf16, live_rows=None):
+        self.card.upload(self.x_offset, x_bf16)
+        live = self.rows if live_rows is None else live_rows
+        self.card.upload(self.step_offset, step_block(live))
+
+    def experts_description(self):
+        d = RoutedExpertsDescription()
+        d.jobs = Range(self.jobs_offset, self.pairs * 96)
+        d.expert_weights = Range(self.weights_offset, self.weights_bytes)
+        width = self.uniform_width if self.uniform_width else int(self.widths.max())
+        d.gate_up_shape = Shape(self.I, self.H, width, 0)
+        d.down_shape = Shape(self.H, self.I, width, 0)
+        d.weight_format = WEIGHT_FORMAT_EXL3
+        d.job_count, d.row_count, d.pairs_per_row = self.pairs, self.rows, self.P
+        d.activation_limit = self.limit
+        return d
+
+    def projection_launch(self):
+        d = RouterProjectionDescription(Range(self.router_offset, self.E * self.H * 2), Range(self.x_offset, self.rows * self.H * 2),
+                                        Range(self.scores_offset, self.rows * self.E * 4), self.rows, self.H, self.E, 0)
+        launch = launches_of(1)
+        check(self.card.lib.router_projection_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launch), "router_projection_prepare")
+        return launch
+
+    def select_launch(self, order=0):
+        experts = self.experts_description()
+        d = RouterDescription()
+        d.experts = C.pointer(experts)
+        d.expert_offsets = self.expert_offsets.ctypes.data_as(C.POINTER(u64))
+        d.expert_widths = self.packed_widths.ctypes.data_as(C.POINTER(u32)) if self.uniform_width == 0 else None
+        d.step = Range(self.step_offset, 16)
+        d.scores = Range(self.scores_offset, self.rows * self.E * 4)
+        d.bias = Range(self.bias_offset, self.E * 4)
+        d.offsets = Range(self.offsets_offset, self.E * 24)
+        d.affinities = Range(self.affinities_offset, self.rows * self.E * 4)
+        d.order, d.expert_count, d.pick_count = order, self.E, self.P
+        d.affinity_kind, d.route_scale = self.affinity_kind, self.route_scale
+        launch = launches_of(1)
+        check(self.card.lib.router_select_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launch), "router_select_prepare")
+        return launch
+
+    def chain_record(self):
+        r = Exl3ExpertRecord()
+        r.jobs_offset, r.input_offset = self.jobs_offset, self.x_offset
+        r.operands_offset = self.scratch_offset
+        r.products_offset = self.scratch_offset + self.pairs * self.H * 4
+        r.output_offset = r.products_offset
+        r.hidden_offset = self.hidden_offset
+        r.input_size, r.inner_size, r.pair_count, r.pairs_per_row = self.H, self.I, self.pairs, self.P
+        r.job_count = self.pairs
+        r.bits_per_weight = self.uniform_width if self.uniform_width else 4
+        r.activation_limit = self.limit
+        r.widths_offset = self.widths_offset
+        return r
+
+    def chain_launches(self):
+        """The reference's seven launches behind the select: five of the chain, then the row sum."""
+        record = self.chain_record()
+        launches = launches_of(EXL3_EXPERT_LAUNCHES + 1)
+        check(self.card.lib.exl3_experts_prepare(C.byref(record), self.card.arena_bytes, backend_table(), self.card.handle,
+                                                 ARITHMETIC_CLASS_GFX950, launches), "exl3_experts_prepare")
+        row_sum = RowSumArguments(record.output_offset, self.out_offset, self.H, self.P)
+        one = launches_of(1)
+        check(self.card.lib.exl3_row_sum_prepare(C.byref(row_sum), self.rows, self.card.arena_bytes, backend_table(),
+                                                 self.card.handle, one), "exl3_row_sum_prepare")
+        launches[EXL3_EXPERT_LAUNCHES] = one[0]
+        return launches
+
+    def tc_record(self):
+        r = Exl3TcRecord()
+        r.jobs_offset, r.hidden_offset = self.jobs_offset, self.x_offset
+        r.workspace_offset, r.output_offset = self.workspace_offset, self.out_offset
+        r.row_count, r.job_capacity, r.intermediate = self.rows, self.pairs, self.I
+        r.bits_x2 = {2: 4, 3: 6, 4: 8, 40: 5}.get(self.uniform_width, 8)
+        r.activation_limit = self.limit
+        r.widths_offset, r.hidden, r.pairs_per_row = self.widths_offset, self.H, self.P
+        return r
+
+    def tc_launches(self):
+        record = self.tc_record()
+        launches = launches_of(EXL3_TC_LAUNCHES)
+        check(self.card.lib.exl3_tc_prepare(C.byref(record), self.card.arena_bytes, backend_table(), self.card.handle, launches), "exl3_tc_prepare")
+        return launches
+
+    def jobs(self):
+        return self.card.download(self.jobs_offset, self.pairs * 96).view(JOB_DTYPE)
+
+    def output(self):
+        return self.card.download(self.out_offset, self.rows * self.H * 4, np.float32).reshape(self.rows, self.H)

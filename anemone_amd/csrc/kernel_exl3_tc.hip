@@ -1,0 +1,245 @@
+/*
+ * kernel_exl3_tc.hip -- the routed experts of one EXL3 layer for a decode-sized step (1 to 64 rows) on gfx950, from
+ * the router's job table: five launches (operands, gate/up products, activation, down products, combine), the
+ * counterpart of the reference's tensor-core MoE (source/kernel_exl3_tc.cu, include/anemone/exl3_tc_records.h).
+ *
+ * The arithmetic is the chain's (kernel_exl3.hip): fp16 operands from a float32 Hadamard transform, exactly decoded
+ * fp16 weights, float32 MFMA sums, SwiGLU in float32, the weighted pair outputs added in slot order. What differs is
+ * the work mapping: every (job, matrix, strip of eight output tiles, K slice) is an independent wavefront item that
+ * streams its bytes once; K-slice partial sums are kept apart in the workspace and added in slice order by the next
+ * launch, so a result does not depend on scheduling, on the other rows of the step or on the grid.
+ *
+ * Workspace (exl3_tc_workspace_bytes): fp16 operands [2][pairs][hidden], reused as [pairs][intermediate] for the
+ * down operands; float32 gate/up partials [GATE_UP_SLICES][2][pairs][intermediate]; float32 down partials
+ * [DOWN_SLICES][pairs][hidden].
+ */
+#include "exl3_device.cuh"
+#include "kernel_registry.h"
+
+#define STRIP_TILES 8u
+#define PRODUCT_WAVES 4u
+#define PRODUCT_THREADS (PRODUCT_WAVES * WAVE)
+
+struct tc_shape {
+    uint32_t hidden, intermediate, picks, pairs;
+};
+
+__device__ static __forceinline__ tc_shape tc_shape_of(const struct exl3_tc_record &record)
+{
+    tc_shape shape;
+    shape.hidden = record.hidden != 0u ? record.hidden : EXL3_TC_DEFAULT_HIDDEN;
+    shape.intermediate = record.intermediate;
+    shape.picks = record.pairs_per_row != 0u ? record.pairs_per_row : EXL3_TC_DEFAULT_PAIRS_PER_ROW;
+    shape.pairs = record.row_count * shape.picks;
+    return shape;
+}
+
+__device__ static __forceinline__ uint32_t tc_bits_x2(const struct exl3_tc_record &record, const unsigned char *arena,
+                                                      uint32_t expert, uint32_t matrix)
+{
+    if (record.widths_offset == 0u) {
+        return record.bits_x2;
+    }
+    return exl3_bits_x2(exl3_width_of(((const uint32_t *)(arena + record.widths_offset))[expert], matrix));
+}
+
+/* launch 0: grid (hidden / 128, job_capacity, 2), block 64 */
+extern "C" __global__ void exl3_tc_operands(struct exl3_tc_record record, unsigned char *arena)
+{
+    const struct expert_job_record *job = (const struct expert_job_record *)(arena + record.jobs_offset) + blockIdx.y;
+    if (job->row_count == 0u) {
+        return;
+    }
+    const tc_shape shape = tc_shape_of(record);
+    const uint32_t lane = threadIdx.x, projection = blockIdx.z, channel = blockIdx.x * EXL3_TRANSFORM + lane;
+    const uint64_t matrix = projection == 0u ? job->gate_offset : job->up_offset;
+    const uint16_t *suh = (const uint16_t *)(arena + matrix + exl3_code_bytes(shape.hidden, shape.intermediate,
+                                                                               tc_bits_x2(record, arena, job->expert, projection)));
+    const float s0 = half_bits_to_float(suh[channel]), s1 = half_bits_to_float(suh[channel + WAVE]);
+    const uint16_t *rows = (const uint16_t *)(arena + record.hidden_offset);
+    uint16_t *operands = (uint16_t *)(arena + record.workspace_offset);
+    for (uint32_t column = 0; column < job->row_count; column++) {
+        const uint32_t pair = job->pair_index[column];
+        const uint64_t row = pair / shape.picks;
+        float v0 = __fmul_rn(bf16_to_float(rows[row * shape.hidden + channel]), s0);
+        float v1 = __fmul_rn(bf16_to_float(rows[row * shape.hidden + channel + WAVE]), s1);
+        wave_hadamard128(v0, v1, lane);
+        uint16_t *out = operands + ((uint64_t)projection * shape.pairs + pair) * shape.hidden;
+        out[channel] = float_to_half_bits(__fmul_rn(v0, EXL3_NORMALIZATION));
+        out[channel + WAVE] = float_to_half_bits(__fmul_rn(v1, EXL3_NORMALIZATION));
+    }
+}
+ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_operands, exl3_tc_record);
+
+/* one wavefront item: a strip of eight output tiles by one K slice of one matrix of one job */
+template <uint32_t bits_x2>
+__device__ static __forceinline__ void tc_item(const uint32_t *codes, uint32_t inputs, uint32_t outputs,
+                                               uint32_t strip, uint32_t slice, uint32_t slices,
+                                               const struct expert_job_record *job, const half_t *operands,
+                                               float *partials, uint32_t *lds, uint32_t lane)
+{
+    const uint32_t column = lane % 16u;
+    const bool live = column < job->row_count;
+    const uint32_t pair = live ? job->pair_index[column] : 0u;
+    const half_t *operand = live ? operands + (uint64_t)pair * inputs : nullptr;
+    const uint32_t tiles = inputs / EXL3_TILE;
+    float4_t accumulator[STRIP_TILES];
+    exl3_wave_product<bits_x2, STRIP_TILES>(codes, outputs / EXL3_TILE, strip * STRIP_TILES, tiles * slice / slices,
+                                            tiles * (slice + 1u) / slices, operand, lds, lane, accumulator);
+    if (live) {
+        float *out = partials + (uint64_t)pair * outputs + strip * (STRIP_TILES * EXL3_TILE) + 4u * (lane / 16u);
+#pragma unroll
+        for (uint32_t n = 0; n < STRIP_TILES; n++) {
+            *(float4_t *)(out + n * EXL3_TILE) = accumulator[n];
+        }
+    }
+}
+
+/* launches 1 and 3: grid (outputs / 128, job_capacity, matrices * slices / 4), block 256: the block's four
+ * wavefronts take four consecutive (matrix, slice) items of one strip. pass 0: gate and up; pass 1: down. */
+extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS)
+    exl3_tc_products(struct exl3_tc_record record, unsigned char *arena)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t staging[PRODUCT_WAVES * 2u * STRIP_TILES * exl3_width<8>::tile_words];
+    const struct expert_job_record *job = (const struct expert_job_record *)(arena + record.jobs_offset) + blockIdx.y;
+    if (job->row_count == 0u) {
+        return;
+    }
+    const tc_shape shape = tc_shape_of(record);
+    const uint32_t lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const bool down = record.pass != 0u;
+    const uint32_t slices = down ? EXL3_TC_DOWN_SLICES : EXL3_TC_GATE_UP_SLICES;
+    const uint32_t item = blockIdx.z * PRODUCT_WAVES + wave; /* projection * slices + slice */
+    const uint32_t projection = item / slices, slice = item % slices;
+    const uint32_t inputs = down ? shape.intermediate : shape.hidden;
+    const uint32_t outputs = down ? shape.hidden : shape.intermediate;
+    const uint64_t matrix = down ? job->down_offset : projection == 0u ? job->gate_offset : job->up_offset;
+    const uint32_t bits_x2 = tc_bits_x2(record, arena, job->expert, down ? 2u : projection);
+    unsigned char *workspace = arena + record.workspace_offset;
+    const half_t *operands = (const half_t *)workspace + (down ? 0u : (uint64_t)projection * shape.pairs * inputs);
+    float *partials;
+    if (down) {
+        partials = (float *)(workspace + exl3_tc_operand_bytes(shape.pairs, shape.hidden) +
+                             exl3_tc_gate_up_bytes(shape.pairs, shape.intermediate)) +
+                   (uint64_t)slice * shape.pairs * outputs;
+    } else {
+        partials = (float *)(workspace + exl3_tc_operand_bytes(shape.pairs, shape.hidden)) +
+                   ((uint64_t)slice * 2u + projection) * shape.pairs * outputs;
+    }
+    uint32_t *lds = staging + wave * (2u * STRIP_TILES * exl3_width<8>::tile_words);
+    const uint32_t *codes = (const uint32_t *)(arena + matrix);
+    switch (bits_x2) {
+    case 4u: tc_item<4u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
+    case 5u: tc_item<5u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
+    case 6u: tc_item<6u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
+    case 8u: tc_item<8u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
+    default: break;
+    }
+}
+ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_products, exl3_tc_record);
+
+/* launch 2: grid (intermediate / 128, job_capacity), block 64 */
+extern "C" __global__ void exl3_tc_activate(struct exl3_tc_record record, unsigned char *arena)
+{
+    const struct expert_job_record *job = (const struct expert_job_record *)(arena + record.jobs_offset) + blockIdx.y;
+    if (job->row_count == 0u) {
+        return;
+    }
+    const tc_shape shape = tc_shape_of(record);
+    const uint32_t lane = threadIdx.x, channel = blockIdx.x * EXL3_TRANSFORM + lane;
+    const uint32_t H = shape.hidden, I = shape.intermediate;
+    const uint16_t *gate_svh = (const uint16_t *)(arena + job->gate_offset + exl3_code_bytes(H, I, tc_bits_x2(record, arena, job->expert, 0u))) + H;
+    const uint16_t *up_svh = (const uint16_t *)(arena + job->up_offset + exl3_code_bytes(H, I, tc_bits_x2(record, arena, job->expert, 1u))) + H;
+    const uint16_t *down_suh = (const uint16_t *)(arena + job->down_offset + exl3_code_bytes(I, H, tc_bits_x2(record, arena, job->expert, 2u)));
+    const float gs[2] = {half_bits_to_float(gate_svh[channel]), half_bits_to_float(gate_svh[channel + WAVE])};
+    const float us[2] = {half_bits_to_float(up_svh[channel]), half_bits_to_float(up_svh[channel + WAVE])};
+    const float ds[2] = {half_bits_to_float(down_suh[channel]), half_bits_to_float(down_suh[channel + WAVE])};
+    const float limit = record.activation_limit;
+    unsigned char *workspace = arena + record.workspace_offset;
+    const float *partials = (const float *)(workspace + exl3_tc_operand_bytes(shape.pairs, H));
+    for (uint32_t column = 0; column < job->row_count; column++) {
+        const uint32_t pair = job->pair_index[column];
+        float g[2] = {0.0f, 0.0f}, u[2] = {0.0f, 0.0f};
+        for (uint32_t slice = 0; slice < EXL3_TC_GATE_UP_SLICES; slice++) { /* in slice order from +0 */
+            const float *gate = partials + ((uint64_t)slice * 2u * shape.pairs + pair) * I;
+            const float *up = partials + (((uint64_t)slice * 2u + 1u) * shape.pairs + pair) * I;
+            g[0] = __fadd_rn(g[0], gate[channel]);
+            g[1] = __fadd_rn(g[1], gate[channel + WAVE]);
+            u[0] = __fadd_rn(u[0], up[channel]);
+            u[1] = __fadd_rn(u[1], up[channel + WAVE]);
+        }
+        wave_hadamard128(g[0], g[1], lane);
+        wave_hadamard128(u[0], u[1], lane);
+        float v[2];
+#pragma unroll
+        for (uint32_t i = 0; i < 2u; i++) {
+            const float gate = __fmul_rn(__fmul_rn(g[i], EXL3_NORMALIZATION), gs[i]);
+            const float up = __fmul_rn(__fmul_rn(u[i], EXL3_NORMALIZATION), us[i]);
+            const float bounded_gate = limit > 0.0f ? fminf(gate, limit) : gate;
+            const float bounded_up = limit > 0.0f ? fminf(fmaxf(up, -limit), limit) : up;
+            const float hidden = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
+            v[i] = __fmul_rn(hidden, ds[i]);
+        }
+        wave_hadamard128(v[0], v[1], lane);
+        uint16_t *operand = (uint16_t *)workspace + (uint64_t)pair * I;
+        operand[channel] = float_to_half_bits(__fmul_rn(v[0], EXL3_NORMALIZATION));
+        operand[channel + WAVE] = float_to_half_bits(__fmul_rn(v[1], EXL3_NORMALIZATION));
+    }
+}
+ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_activate, exl3_tc_record);
+
+/* launch 4: grid (hidden / 128, row_count), block 64: a row's pairs in slot order */
+extern "C" __global__ void exl3_tc_combine(struct exl3_tc_record record, unsigned char *arena)
+{
+    const tc_shape shape = tc_shape_of(record);
+    const uint32_t lane = threadIdx.x, channel = blockIdx.x * EXL3_TRANSFORM + lane, row = blockIdx.y;
+    const uint32_t H = shape.hidden, I = shape.intermediate;
+    const struct expert_job_record *jobs = (const struct expert_job_record *)(arena + record.jobs_offset);
+    const unsigned char *workspace = arena + record.workspace_offset;
+    const float *partials = (const float *)(workspace + exl3_tc_operand_bytes(shape.pairs, H) + exl3_tc_gate_up_bytes(shape.pairs, I));
+    float sum0 = 0.0f, sum1 = 0.0f;
+    for (uint32_t slot = 0; slot < shape.picks; slot++) {
+        const uint32_t pair = row * shape.picks + slot;
+        /* the job and column that hold this pair: every lane looks at jobs lane, lane + 64, ... */
+        uint32_t found = 0xFFFFFFFFu;
+        for (uint32_t base = 0; base < record.job_capacity; base += WAVE) {
+            const uint32_t index = base + lane;
+            uint32_t mine = 0xFFFFFFFFu;
+            if (index < record.job_capacity) {
+                const struct expert_job_record *job = jobs + index;
+                for (uint32_t column = 0; column < job->row_count; column++) {
+                    if (job->pair_index[column] == pair) {
+                        mine = index * LINEAR_MAXIMUM_ROWS + column;
+                    }
+                }
+            }
+#pragma unroll
+            for (uint32_t distance = WAVE / 2u; distance != 0u; distance >>= 1u) {
+                const uint32_t other = __shfl_xor(mine, (int)distance, WAVE);
+                mine = other < mine ? other : mine;
+            }
+            found = mine < found ? mine : found;
+        }
+        if (found == 0xFFFFFFFFu) {
+            continue; /* a pair no job holds (a row beyond the live ones) adds nothing */
+        }
+        const struct expert_job_record *job = jobs + found / LINEAR_MAXIMUM_ROWS;
+        const float weight = job->route_weight[found % LINEAR_MAXIMUM_ROWS];
+        const uint16_t *svh = (const uint16_t *)(arena + job->down_offset + exl3_code_bytes(I, H, tc_bits_x2(record, arena, job->expert, 2u))) + I;
+        float v0 = 0.0f, v1 = 0.0f;
+        for (uint32_t slice = 0; slice < EXL3_TC_DOWN_SLICES; slice++) {
+            const float *down = partials + ((uint64_t)slice * shape.pairs + pair) * H;
+            v0 = __fadd_rn(v0, down[channel]);
+            v1 = __fadd_rn(v1, down[channel + WAVE]);
+        }
+        wave_hadamard128(v0, v1, lane);
+        const float y0 = __fmul_rn(__fmul_rn(__fmul_rn(v0, EXL3_NORMALIZATION), half_bits_to_float(svh[channel])), weight);
+        const float y1 = __fmul_rn(__fmul_rn(__fmul_rn(v1, EXL3_NORMALIZATION), half_bits_to_float(svh[channel + WAVE])), weight);
+        sum0 = __fadd_rn(sum0, y0);
+        sum1 = __fadd_rn(sum1, y1);
+    }
+    float *out = (float *)(arena + record.output_offset) + (uint64_t)row * H;
+    out[channel] = sum0;
+    out[channel + WAVE] = sum1;
+}
+ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_combine, exl3_tc_record);

@@ -1,0 +1,125 @@
+/*
+ * exl3_tc.c -- load-time preparation of the fused EXL3 decode of one layer's routed experts (1 to 64 rows): five
+ * launches from the router's job table. Entry points follow the reference's source/exl3_tc.c:120-268 and
+ * include/anemone/exl3_tc.h:22-43; hidden size, picks a row and per-matrix widths are members of the record.
+ *
+ *   launch      kernel              grid                                            block
+ *   operands    exl3_tc_operands    (hidden / 128, job_capacity, 2)                 64
+ *   gate/up     exl3_tc_products    (intermediate / 128, job_capacity, 2 S_gu / 4)  256   pass 0
+ *   activate    exl3_tc_activate    (intermediate / 128, job_capacity, 1)           64
+ *   down        exl3_tc_products    (hidden / 128, job_capacity, S_d / 4)           256   pass 1
+ *   combine     exl3_tc_combine     (hidden / 128, row_count, 1)                    64
+ * S_gu = EXL3_TC_GATE_UP_SLICES and S_d = EXL3_TC_DOWN_SLICES K slices; every slice is a whole number of MFMA steps
+ * (32 inputs), which bounds the shapes: hidden a multiple of 32 S_gu, intermediate of 32 S_d, both of 128.
+ */
+#include <math.h>
+#include <string.h>
+
+#include "prepare_common.h"
+
+#define WAVE_THREADS 64u
+#define PRODUCT_THREADS 256u
+#define PRODUCT_WAVES 4u
+#define MOST_GRID_ROWS 65535u
+
+static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                const struct backend_operations *backend, struct device_card *card,
+                                struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
+{
+    static const char what[] = "EXL3 fused decode";
+    if (record == NULL || backend == NULL || backend->kernel_prepare == NULL || card == NULL || launches_out == NULL) {
+        REFUSE("%s: a missing argument", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint32_t hidden = record->hidden != 0 ? record->hidden : EXL3_TC_DEFAULT_HIDDEN;
+    const uint32_t picks = record->pairs_per_row != 0 ? record->pairs_per_row : EXL3_TC_DEFAULT_PAIRS_PER_ROW;
+    const uint32_t I = record->intermediate;
+    if (record->row_count == 0 || record->row_count > EXL3_TC_MOST_ROWS || record->job_capacity == 0 ||
+        record->job_capacity > MOST_GRID_ROWS || record->pass != 0 || picks > ROUTER_MOST_PICKS ||
+        !(record->activation_limit >= 0.0f) || !isfinite(record->activation_limit)) {
+        REFUSE("%s: 1 to %u rows, 1 to %u jobs, pass 0, an activation limit of zero (none) or above", what,
+               EXL3_TC_MOST_ROWS, MOST_GRID_ROWS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (record->rotation != 0 || record->shared_sum != 0) {
+        REFUSE("%s: expert rotation and the shared-expert sum are tensor-parallel forms this library does not build", what);
+        return STATUS_UNSUPPORTED;
+    }
+    if (I == 0 || I % EXL3_TRANSFORM != 0 || hidden % EXL3_TRANSFORM != 0 || hidden % (32u * EXL3_TC_GATE_UP_SLICES) != 0 ||
+        I % (32u * EXL3_TC_DOWN_SLICES) != 0 || I > hidden) {
+        REFUSE("%s: hidden %u and intermediate %u: multiples of 128, of %u and of %u", what, hidden, I,
+               32u * EXL3_TC_GATE_UP_SLICES, 32u * EXL3_TC_DOWN_SLICES);
+        return STATUS_UNSUPPORTED;
+    }
+    const bool mixed = record->widths_offset != 0;
+    if (!mixed && (record->bits_x2 != 4u && record->bits_x2 != 5u && record->bits_x2 != 6u && record->bits_x2 != 8u)) {
+        REFUSE("%s: bits_x2 %u: this build decodes 4, 5, 6 and 8", what, record->bits_x2);
+        return exl3_width_name(record->bits_x2) == NULL && (record->bits_x2 == 0 || record->bits_x2 > 16u)
+                   ? STATUS_INVALID_ARGUMENT
+                   : STATUS_UNSUPPORTED;
+    }
+    const uint64_t pairs = (uint64_t)record->row_count * picks;
+    const uint64_t workspace = exl3_tc_workspace_bytes(pairs, hidden, I);
+    const struct checked_range ranges[] = {
+        {"the jobs", {record->jobs_offset, (uint64_t)record->job_capacity * sizeof(struct expert_job_record)},
+         (uint64_t)record->job_capacity * sizeof(struct expert_job_record), false},
+        {"the rows", {record->hidden_offset, (uint64_t)record->row_count * hidden * 2u}, (uint64_t)record->row_count * hidden * 2u, false},
+        {"the workspace", {record->workspace_offset, workspace}, workspace, false},
+        {"the output", {record->output_offset, (uint64_t)record->row_count * hidden * 4u}, (uint64_t)record->row_count * hidden * 4u, false},
+    };
+    if (!ranges_are_valid(what, ranges, 4, arena_byte_count) || record->workspace_offset % 256u != 0 ||
+        (mixed && record->widths_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0)) {
+        if (record->workspace_offset % 256u != 0) {
+            REFUSE("%s: the workspace begins off a multiple of 256", what);
+        }
+        return STATUS_INVALID_ARGUMENT;
+    }
+    static const char *const names[EXL3_TC_LAUNCHES] = {"exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate",
+                                                        "exl3_tc_products", "exl3_tc_combine"};
+    const uint32_t grid_x[EXL3_TC_LAUNCHES] = {hidden / 128u, I / 128u, I / 128u, hidden / 128u, hidden / 128u};
+    const uint32_t grid_y[EXL3_TC_LAUNCHES] = {record->job_capacity, record->job_capacity, record->job_capacity,
+                                               record->job_capacity, record->row_count};
+    const uint32_t grid_z[EXL3_TC_LAUNCHES] = {2u, 2u * EXL3_TC_GATE_UP_SLICES / PRODUCT_WAVES, 1u,
+                                               EXL3_TC_DOWN_SLICES / PRODUCT_WAVES, 1u};
+    const uint32_t threads[EXL3_TC_LAUNCHES] = {WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS};
+    _Static_assert(2u * EXL3_TC_GATE_UP_SLICES % PRODUCT_WAVES == 0 && EXL3_TC_DOWN_SLICES % PRODUCT_WAVES == 0,
+                   "a block's four wavefronts take four whole items");
+    struct kernel_launch launches[EXL3_TC_LAUNCHES];
+    for (uint32_t index = 0; index < EXL3_TC_LAUNCHES; index++) {
+        uint32_t kernel = BACKEND_NO_KERNEL;
+        const result_status prepared = backend->kernel_prepare(card, EXL3_TC_KERNEL_FILE, names[index], sizeof *record, &kernel);
+        if (prepared != STATUS_OK) {
+            return prepared;
+        }
+        if (kernel == BACKEND_NO_KERNEL) {
+            return STATUS_UNSUPPORTED;
+        }
+        struct exl3_tc_record stamped = *record;
+        stamped.pass = index == 3u ? 1u : 0u;
+        launch_fill(&launches[index], kernel, grid_x[index], grid_y[index], grid_z[index], threads[index], 0, &stamped,
+                    sizeof stamped);
+    }
+    memcpy(launches_out, launches, sizeof launches);
+    return STATUS_OK;
+}
+
+result_status exl3_tc_prepare(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                              const struct backend_operations *backend, struct device_card *card,
+                              struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
+{
+    return tc_prepare(record, arena_byte_count, backend, card, launches_out);
+}
+
+result_status exl3_tc_prepare_short(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                    const struct backend_operations *backend, struct device_card *card,
+                                    struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
+{
+    return tc_prepare(record, arena_byte_count, backend, card, launches_out);
+}
+
+result_status exl3_tc_prepare_paired(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                     const struct backend_operations *backend, struct device_card *card,
+                                     struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
+{
+    return tc_prepare(record, arena_byte_count, backend, card, launches_out);
+}

@@ -1,0 +1,176 @@
+/*
+ * anemone_ops.h -- the host-side operator entry points of the routed-expert path: load-time "prepare" functions
+ * that check a description and fill immutable `struct kernel_launch` tables. C11, no device code, no allocation.
+ *
+ * Each function keeps the name, the argument meaning and the refusal rules of the reference function it replaces:
+ *   weight_format_operations_of          include/anemone/weight_format_seam.h:93-94   (source/weight_format.c)
+ *   exl3_*                               include/anemone/exl3.h:11-61                  (source/exl3.c)
+ *   exl3_row_sum_prepare                 include/anemone/exl3_tp.h:77-80 (bb_exl3_row_sum_prepare; source/exl3_tp.c:250-290)
+ *   exl3_tc_prepare, exl3_tcp_prepare    include/anemone/exl3_tc.h:22-59               (source/exl3_tc.c)
+ *   router_*                             include/anemone/router.h:50-124               (source/router.c)
+ *   linear_*                             include/anemone/linear.h:117-411              (source/linear.c, routed part)
+ *   expert_producer_prepare              include/anemone/expert_fused.h:51-101         (source/expert_fused.c)
+ * Contract of every prepare function (include/anemone/linear.h:17-48): arithmetic on a description, the arena is a
+ * number; pure and reentrant; a refusal is a status with one error line on stderr and the launch table untouched.
+ * What differs from the reference: shapes (experts, picks, hidden, widths) are run-time members instead of one
+ * model's compile-time constants, and the arithmetic class accepted is ARITHMETIC_CLASS_GFX950.
+ */
+#ifndef ANEMONE_OPS_H
+#define ANEMONE_OPS_H
+
+#include <stdbool.h>
+#include <stdint.h>
+
+#include "anemone_backend.h"
+#include "anemone_records.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- ranges, shapes, formats ---- */
+struct linear_range {
+    uint64_t byte_offset;
+    uint64_t byte_count;
+};
+struct matrix_shape_record {
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t bits_per_weight; /* EXL3: a stored width; a format of one width checks its figure */
+    uint32_t reserved_must_be_zero;
+};
+struct weight_format_operations {
+    const char *name;
+    MUST_CHECK result_status (*stored_byte_count)(const struct matrix_shape_record *shape, uint64_t *byte_count_out);
+};
+const struct weight_format_operations *weight_format_operations_of(enum weight_format_code format);
+extern const struct weight_format_operations exl3_weight_operations;
+
+enum linear_order_code { LINEAR_ORDER_FIXED = 0, LINEAR_ORDER_REFERENCE = 1 };
+
+/* ---- EXL3 chain ---- */
+const char *exl3_width_name(uint32_t bits_x2); /* "k2", "k2_5", "k3", "k4"; NULL for a width without entries */
+MUST_CHECK result_status exl3_reconstruct_prepare(const struct exl3_reconstruct_record *record,
+                                                  uint64_t arena_byte_count, uint32_t kernel,
+                                                  struct kernel_launch *launch_out);
+uint64_t exl3_scratch_byte_count(uint32_t pair_count, uint32_t input_size);
+/* launches_out: EXL3_EXPERT_LAUNCHES launches (input, gate/up, activate, down, finish) */
+MUST_CHECK result_status exl3_experts_prepare(const struct exl3_expert_record *record, uint64_t arena_byte_count,
+                                              const struct backend_operations *backend, struct device_card *card,
+                                              uint32_t arithmetic_class, struct kernel_launch *launches_out);
+/* the reference's alternative work mappings of the same words; on gfx950 there is one mapping, so fast == retained */
+MUST_CHECK result_status exl3_experts_fast_prepare(const struct exl3_expert_record *record,
+                                                   uint64_t arena_byte_count,
+                                                   const struct backend_operations *backend,
+                                                   struct device_card *card, uint32_t arithmetic_class,
+                                                   struct kernel_launch *launches_out);
+/* another association of the float32 sums, the CMP cards' own: STATUS_UNSUPPORTED on any other class, so here */
+MUST_CHECK result_status exl3_experts_relaxed_prepare(const struct exl3_expert_record *record,
+                                                      uint64_t arena_byte_count,
+                                                      const struct backend_operations *backend,
+                                                      struct device_card *card, uint32_t arithmetic_class,
+                                                      struct kernel_launch *launches_out);
+MUST_CHECK result_status exl3_row_sum_prepare(const struct expert_row_sum_arguments *record, uint32_t rows,
+                                              uint64_t arena_bytes, const struct backend_operations *backend,
+                                              struct device_card *card, struct kernel_launch *launch_out);
+
+/* ---- EXL3 fused decode (1 .. EXL3_TC_MOST_ROWS rows): EXL3_TC_LAUNCHES launches ---- */
+MUST_CHECK result_status exl3_tc_prepare(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                         const struct backend_operations *backend, struct device_card *card,
+                                         struct kernel_launch launches_out[EXL3_TC_LAUNCHES]);
+/* the reference's row-count-independent and paired forms: on gfx950 exl3_tc_prepare already is row-count
+ * independent (a row's bits do not depend on the other rows), so both are the same launches */
+MUST_CHECK result_status exl3_tc_prepare_short(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                               const struct backend_operations *backend, struct device_card *card,
+                                               struct kernel_launch launches_out[EXL3_TC_LAUNCHES]);
+MUST_CHECK result_status exl3_tc_prepare_paired(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                                const struct backend_operations *backend, struct device_card *card,
+                                                struct kernel_launch launches_out[EXL3_TC_LAUNCHES]);
+
+/* ---- router ---- */
+struct router_kernels_record {
+    uint32_t select;
+    uint32_t wide_select;
+    uint32_t wide_count;
+    uint32_t wide_place;
+    uint32_t wide_jobs;
+    uint32_t wide_small;
+    uint32_t select_draft; /* BACKEND_NO_KERNEL: the draft's router is outside this path */
+    uint32_t projection;   /* no counterpart: the router's score projection as its own launch */
+};
+MUST_CHECK result_status router_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                                struct router_kernels_record *kernels_out);
+
+/* the subset of the reference's linear_routed_experts_description the router checks its table against */
+struct linear_routed_experts_description {
+    struct linear_range jobs;           /* struct expert_job_record [job_count] */
+    struct linear_range expert_weights; /* holds every matrix a job names */
+    struct linear_range codes, exponents, operands;
+    struct linear_range hidden, hidden_codes, hidden_exponents, hidden_operands;
+    struct linear_range pair_output, row_output;
+    struct matrix_shape_record gate_up_shape;
+    struct matrix_shape_record down_shape;
+    enum weight_format_code weight_format; /* E2M1_SCALED, E4M3_SCALED or EXL3 */
+    uint32_t job_count;
+    uint32_t row_count;
+    uint32_t pairs_per_row;
+    uint32_t gate_up_slice_count;
+    uint32_t down_slice_count;
+    float activation_limit;
+    uint32_t reserved_zero;
+};
+
+struct router_description {
+    const struct linear_routed_experts_description *experts;
+    const uint64_t *expert_offsets; /* [E][3]: what the arena holds at offsets */
+    const uint32_t *expert_widths;  /* EXL3 with per-matrix widths: [E] packed as in the arena; else NULL */
+    struct linear_range step, scores, bias, offsets, affinities;
+    enum linear_order_code order;
+    uint32_t expert_count; /* 1 .. ROUTER_MOST_EXPERTS, a multiple of 64 */
+    uint32_t pick_count;   /* 1 .. ROUTER_MOST_PICKS */
+    uint32_t affinity_kind;
+    float route_scale;
+};
+MUST_CHECK result_status router_select_prepare(const struct router_description *description,
+                                               uint64_t arena_byte_count,
+                                               const struct router_kernels_record *kernels,
+                                               struct kernel_launch *launch_out);
+
+struct router_projection_description {
+    struct linear_range weights, rows, output;
+    uint32_t row_count, hidden, expert_count, reserved_zero;
+};
+MUST_CHECK result_status router_projection_prepare(const struct router_projection_description *description,
+                                                   uint64_t arena_byte_count,
+                                                   const struct router_kernels_record *kernels,
+                                                   struct kernel_launch *launch_out);
+
+enum router_wide_launch {
+    ROUTER_WIDE_SELECT_LAUNCH = 0,
+    ROUTER_WIDE_COUNT_LAUNCH = 1,
+    ROUTER_WIDE_PLACE_LAUNCH = 2,
+    ROUTER_WIDE_JOBS_LAUNCH = 3,
+    ROUTER_WIDE_LAUNCH_COUNT = 4
+};
+struct router_wide_description {
+    const uint64_t *expert_offsets;
+    const uint32_t *expert_widths;
+    struct linear_range step, scores, bias, offsets, expert_weights, affinities;
+    struct linear_range picks, counts, pairs, runs, tiles, jobs;
+    struct matrix_shape_record gate_up_shape, down_shape;
+    enum weight_format_code weight_format;
+    enum linear_order_code order;
+    uint32_t row_count;
+    uint32_t reserved_zero;
+    uint32_t expert_count, pick_count, affinity_kind;
+    float route_scale;
+};
+MUST_CHECK result_status router_wide_prepare(const struct router_wide_description *description,
+                                             uint64_t arena_byte_count,
+                                             const struct router_kernels_record *kernels,
+                                             struct kernel_launch *launches_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,370 @@
+/*
+ * anemone_records.h -- the by-value records of every kernel of the routed-expert path, and the arrays they name.
+ * Compiles as C11 (the host's prepare functions) and as HIP C++ (the kernels).
+ *
+ * The kernel ABI is the reference's (include/anemone/backend_seam.h:60-69): every kernel is
+ *     extern "C" __global__ void <name>(struct <record> record, unsigned char *arena)
+ * and a record names memory by BYTE OFFSETS into the card's one arena, never by address. Records are fixed-size,
+ * little-endian, without padding, at most LAUNCH_ARGUMENT_BYTES (192).
+ *
+ * Layout compatibility. Each struct below keeps the reference's members in the reference's order, so a caller that
+ * fills a record by member name fills the same leading bytes:
+ *     expert_job_record                 include/anemone/linear_records.h:245-253       (96 B)
+ *     router_pick, wide_pair/run/tile   include/anemone/router_records.h:112-115, wide_linear_records.h:62-78
+ *     step_block                        include/anemone/step_records.h:111-115         (16 B)
+ *     exl3_reconstruct_record           include/anemone/exl3_records.h:123-130         (32 B)
+ *     expert_row_sum_arguments          include/anemone/linear_records.h:300-305       (24 B)
+ *     activation_quantize_arguments     include/anemone/linear_records.h:222-229       (40 B)
+ *     expert_gate_up_arguments          include/anemone/linear_records.h:263-275       (64 B)
+ *     expert_down_arguments             include/anemone/linear_records.h:283-293       (56 B)
+ * Four records carry a TRAILING EXTENSION the reference does not have, because the reference fixes one model's
+ * shape at compile time (384 experts, 6 picks, hidden 5120, one width per layer) and this build takes them at run
+ * time. A zero extension means "the reference's behaviour":
+ *     router_select_arguments  80 B  (router_records.h:98-110)   + expert_count, pick_count, affinity_kind, route_scale
+ *     router_wide_arguments    120 B (router_records.h:117-134)  + the same four
+ *     exl3_expert_record       80 B  (exl3_records.h:144-159)    + widths_offset
+ *     exl3_tc_record           72 B  (exl3_tc_records.h:40-58)   + widths_offset, hidden, pairs_per_row
+ *     exl3_tcp_record          88 B  (exl3_tc_records.h:244-262) + widths_offset, hidden, pairs_per_row, expert_count
+ * widths_offset: 0, or the arena offset of uint32 [expert_count], entry e = gate | up << 8 | down << 16, the stored
+ * widths of expert e's three matrices (per-matrix widths: one layer mixes K = 2, 3, 4). When it is 0 every matrix
+ * has the record's one width, as in the reference.
+ */
+#ifndef ANEMONE_RECORDS_H
+#define ANEMONE_RECORDS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+#define ANEMONE_RECORD_HAS(record, bytes) static_assert(sizeof(struct record) == (bytes), #record " ABI")
+#else
+#define ANEMONE_RECORD_HAS(record, bytes) _Static_assert(sizeof(struct record) == (bytes), #record " ABI")
+#endif
+
+/* ---- shared geometry ---- */
+#define LINEAR_MAXIMUM_ROWS 8u          /* columns of one job */
+#define LINEAR_OUTPUTS_PER_TILE 16u
+#define LINEAR_VALUES_PER_BLOCK 32u     /* values that share one scale exponent */
+#define LINEAR_VALUES_PER_LOAD 64u
+#define LINEAR_OFFSET_ALIGNMENT_BYTES 16u
+#define LINEAR_ELEMENT_THREADS 256u
+#define WIDE_TILE_PAIRS 64u
+#define MODEL_EXPERT_MATRICES 3u        /* gate, up, down */
+#define ROUTER_DEFAULT_EXPERTS 384u     /* what a zero extension stands for */
+#define ROUTER_DEFAULT_PICKS 6u
+#define ROUTER_DEFAULT_SCALE 1.5f
+#define ROUTER_MOST_EXPERTS 512u
+#define ROUTER_MOST_PICKS 8u
+#define ROUTER_AFFINITY_SQRT_SOFTPLUS 0u
+#define ROUTER_AFFINITY_SIGMOID 1u
+
+/* ---- step ---- */
+struct step_block {
+    uint64_t sequence;
+    uint32_t row_count; /* the live rows of the step: the routers read it, not their record's */
+    uint32_t flags;
+};
+ANEMONE_RECORD_HAS(step_block, 16);
+
+/* ---- job table and the wide select's arrays ---- */
+struct expert_job_record {
+    uint64_t gate_offset;
+    uint64_t up_offset;
+    uint64_t down_offset;
+    uint32_t row_count; /* 0 .. 8; an empty job is read no further */
+    uint32_t expert;
+    uint32_t pair_index[LINEAR_MAXIMUM_ROWS]; /* row * pairs_per_row + slot */
+    float route_weight[LINEAR_MAXIMUM_ROWS];
+};
+ANEMONE_RECORD_HAS(expert_job_record, 96);
+
+struct router_pick {
+    uint32_t expert;
+    float route_weight;
+};
+struct wide_pair {
+    uint32_t pair_index;
+    float route_weight;
+};
+struct wide_run {
+    uint32_t first_pair;
+    uint32_t pair_count;
+};
+struct wide_expert_tile {
+    uint64_t gate_offset;
+    uint64_t up_offset;
+    uint64_t down_offset;
+    uint32_t first_pair;
+    uint32_t pair_count; /* at most WIDE_TILE_PAIRS */
+};
+ANEMONE_RECORD_HAS(router_pick, 8);
+ANEMONE_RECORD_HAS(wide_pair, 8);
+ANEMONE_RECORD_HAS(wide_run, 8);
+ANEMONE_RECORD_HAS(wide_expert_tile, 32);
+
+/* ---- router ---- */
+#define KERNEL_FILE_ROUTER "kernel_router"
+#define KERNEL_ROUTER_PROJECTION "router_projection"
+#define KERNEL_ROUTER_SELECT "router_select_entry"
+#define KERNEL_ROUTER_WIDE_SELECT "router_wide_select"
+#define KERNEL_ROUTER_WIDE_COUNT "router_wide_count"
+#define KERNEL_ROUTER_WIDE_PLACE "router_wide_place"
+#define KERNEL_ROUTER_WIDE_JOBS "router_wide_jobs"
+#define KERNEL_ROUTER_WIDE_SMALL "router_wide_small"
+#define ROUTER_THREADS 256u
+#define ROUTER_SORT_ROWS 384u
+
+struct router_projection_arguments { /* scores [rows][experts] = W x, bfloat16 in, float32 out */
+    uint64_t weights_offset;         /* read: bfloat16 [expert_count][hidden] */
+    uint64_t rows_offset;            /* read: bfloat16 [row_count][hidden] */
+    uint64_t output_offset;          /* written: float32 [row_count][expert_count] */
+    uint32_t row_count;
+    uint32_t hidden;
+    uint32_t expert_count;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(router_projection_arguments, 40);
+
+struct router_select_arguments {
+    uint64_t step_offset;            /* read: struct step_block */
+    uint64_t scores_offset;          /* read: float32 [row_count][E] */
+    uint64_t bias_offset;            /* read: float32 [E] */
+    uint64_t expert_offsets_offset;  /* read: uint64 [E][3] */
+    uint64_t affinities_offset;      /* written: float32 [row_count][E], live rows */
+    uint64_t jobs_offset;            /* written: struct expert_job_record [P row_count], every byte */
+    uint64_t weights_offset;         /* the experts' range: its first byte, */
+    uint64_t gate_up_last_offset;    /* the last a gate or up matrix may begin at, */
+    uint64_t down_last_offset;       /* the last a down matrix may begin at */
+    uint32_t row_count;              /* 1 .. LINEAR_MAXIMUM_ROWS */
+    uint32_t reference_order;        /* 0 or 1 (1: six picks alone) */
+    /* extension */
+    uint32_t expert_count;           /* 0: 384 */
+    uint32_t pick_count;             /* 0: 6 */
+    uint32_t affinity_kind;          /* ROUTER_AFFINITY_* */
+    float route_scale;               /* 0: 1.5 */
+};
+ANEMONE_RECORD_HAS(router_select_arguments, 96);
+
+struct router_wide_arguments {
+    uint64_t step_offset;
+    uint64_t scores_offset;
+    uint64_t bias_offset;
+    uint64_t expert_offsets_offset;
+    uint64_t affinities_offset;      /* written: float32 [row_count][E] */
+    uint64_t picks_offset;           /* scratch: struct router_pick [row_count][P] */
+    uint64_t counts_offset;          /* scratch: uint32 [ceil(row_count / ROUTER_SORT_ROWS)][E] */
+    uint64_t pairs_offset;           /* written: struct wide_pair [P row_count] */
+    uint64_t runs_offset;            /* written: struct wide_run [E] */
+    uint64_t tiles_offset;           /* written: struct wide_expert_tile [tiles of row_count] */
+    uint64_t jobs_offset;            /* written: struct expert_job_record [jobs of row_count] */
+    uint64_t weights_offset;
+    uint64_t gate_up_last_offset;
+    uint64_t down_last_offset;
+    uint32_t row_count;
+    uint32_t reference_order;
+    /* extension */
+    uint32_t expert_count;
+    uint32_t pick_count;
+    uint32_t affinity_kind;
+    float route_scale;
+};
+ANEMONE_RECORD_HAS(router_wide_arguments, 136);
+
+/* tiles / jobs of a wide select: each run cut in 64s (8s), the last ragged */
+#define ROUTER_WIDE_TILES_OF(row_count, picks, experts) \
+    (((row_count) * (picks) + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS + (experts))
+#define ROUTER_WIDE_JOB_BOUND_OF(row_count, picks, experts) \
+    (((row_count) * (picks) + (LINEAR_MAXIMUM_ROWS - 1u) * (experts)) / LINEAR_MAXIMUM_ROWS)
+#define ROUTER_WIDE_JOBS_OF(row_count, picks, experts)                                             \
+    ((row_count) * (picks) < ROUTER_WIDE_JOB_BOUND_OF(row_count, picks, experts) ? (row_count) * (picks) \
+                                                                                  : ROUTER_WIDE_JOB_BOUND_OF(row_count, picks, experts))
+
+/* ---- EXL3 ---- */
+#define EXL3_KERNEL_FILE "kernel_exl3"
+#define EXL3_RECONSTRUCT "exl3_reconstruct"
+#define EXL3_ROW_SUM "exl3_row_sum"
+#define EXL3_TILE 16u
+#define EXL3_TILE_VALUES 256u
+#define EXL3_TRANSFORM 128u
+#define EXL3_K2 2u   /* stored widths: K for a whole K, 16 K for a half K */
+#define EXL3_K2_5 40u
+#define EXL3_K3 3u
+#define EXL3_K4 4u
+#define EXL3_MUL1_MULTIPLIER 0x83DCD12Du
+#define EXL3_MUL1_BASE 0x6400u
+#define EXL3_MUL1_SCALE 0x1EEEu
+#define EXL3_MUL1_BIAS 0xC931u
+#define EXL3_NORMALIZATION 0.08838834764831845f
+#define EXL3_EXPERT_LAUNCHES 5u
+#define EXL3_PRODUCT_SLICES 4u
+
+#ifdef __cplusplus
+#define ANEMONE_INLINE __host__ __device__ static constexpr inline
+#else
+#define ANEMONE_INLINE static inline
+#endif
+
+/* bits_x2 = 2 K of a stored width; 0 for a value that is no width (whole 1-8, half 1.5-7.5) */
+ANEMONE_INLINE uint32_t exl3_bits_x2(uint32_t stored_width)
+{
+    return stored_width >= 1u && stored_width <= 8u ? 2u * stored_width
+           : stored_width % 16u == 8u && stored_width < 128u ? stored_width / 8u
+                                                             : 0u;
+}
+/* the widths this build has kernels for */
+ANEMONE_INLINE int exl3_width_supported(uint32_t stored_width)
+{
+    return stored_width == EXL3_K2 || stored_width == EXL3_K3 || stored_width == EXL3_K4 || stored_width == EXL3_K2_5;
+}
+/* S(i): ring bit where the window of position i ends */
+ANEMONE_INLINE uint32_t exl3_window_end(uint32_t position, uint32_t bits_x2)
+{
+    return (position + 1u) * bits_x2 / 2u;
+}
+ANEMONE_INLINE uint64_t exl3_code_bytes(uint64_t inputs, uint64_t outputs, uint32_t bits_x2)
+{
+    return inputs * outputs / 16u * bits_x2;
+}
+/* an expert's packed widths entry -> the stored width of matrix m (0 gate, 1 up, 2 down) */
+ANEMONE_INLINE uint32_t exl3_width_of(uint32_t packed, uint32_t matrix)
+{
+    return (packed >> (8u * matrix)) & 255u;
+}
+
+struct exl3_reconstruct_record {
+    uint64_t matrix_offset;
+    uint64_t output_offset; /* written: fp16 [input][output], before either transform or scale */
+    uint32_t input_size;
+    uint32_t output_size;
+    uint32_t bits_per_weight; /* stored width */
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(exl3_reconstruct_record, 32);
+
+/* The five-launch chain of one layer: input, gate/up products, activate, down products, finish (then exl3_row_sum).
+ * operands fp16 [2][pairs][input_size]; products float32 [2][pairs][inner_size], later [pairs][input_size];
+ * hidden bf16 [pairs][inner_size]; output float32 [pairs][input_size] == products (in place). */
+struct exl3_expert_record {
+    uint64_t jobs_offset;
+    uint64_t input_offset;    /* read: bf16 [rows][input_size] */
+    uint64_t operands_offset;
+    uint64_t products_offset;
+    uint64_t hidden_offset;
+    uint64_t output_offset;   /* == products_offset */
+    uint32_t input_size;
+    uint32_t inner_size;
+    uint32_t pair_count;
+    uint32_t pairs_per_row;
+    uint32_t job_count;
+    uint32_t bits_per_weight; /* the one stored width, unless widths_offset names per-matrix widths */
+    float activation_limit;
+    uint32_t reserved_zero;
+    /* extension */
+    uint64_t widths_offset;
+};
+ANEMONE_RECORD_HAS(exl3_expert_record, 88);
+
+struct expert_row_sum_arguments {
+    uint64_t pair_output_offset;
+    uint64_t row_output_offset;
+    uint32_t width;
+    uint32_t pairs_per_row;
+};
+ANEMONE_RECORD_HAS(expert_row_sum_arguments, 24);
+
+/* ---- EXL3 fused decode (at most EXL3_TC_MOST_ROWS rows) ---- */
+#define EXL3_TC_KERNEL_FILE "kernel_exl3_tc"
+#define EXL3_TC_LAUNCHES 5u
+#define EXL3_TC_MOST_ROWS 64u
+#define EXL3_TC_DEFAULT_HIDDEN 5120u
+#define EXL3_TC_DEFAULT_PAIRS_PER_ROW 6u
+#define EXL3_TC_GATE_UP_SLICES 8u /* K slices of a gate/up product: partial sums kept apart, added in order */
+#define EXL3_TC_DOWN_SLICES 4u
+
+struct exl3_tc_record {
+    uint64_t jobs_offset;      /* read: struct expert_job_record [job_capacity], empty ones anywhere */
+    uint64_t hidden_offset;    /* read: bf16 [row_count][hidden] */
+    uint64_t workspace_offset; /* scratch: exl3_tc_workspace_bytes(...), 256-aligned */
+    uint64_t output_offset;    /* written: float32 [row_count][hidden], each row's route-weighted expert sum */
+    uint32_t row_count;
+    uint32_t job_capacity;
+    uint32_t intermediate;
+    uint32_t bits_x2;          /* the one width as 2 K, unless widths_offset names per-matrix widths */
+    float activation_limit;    /* the SwiGLU limit; 0: none */
+    uint32_t pass;             /* the products launches: 0 gate and up, 1 down; the others 0 */
+    uint32_t rotation;         /* must be 0: a tensor-parallel feature, not built */
+    uint32_t shared_sum;       /* must be 0 */
+    uint64_t shared_offset;    /* unused */
+    /* extension */
+    uint64_t widths_offset;
+    uint32_t hidden;           /* 0: 5120 */
+    uint32_t pairs_per_row;    /* 0: 6 */
+};
+ANEMONE_RECORD_HAS(exl3_tc_record, 88);
+
+/* workspace of the fused decode: fp16 operands [2][pairs][hidden] (later [pairs][intermediate]), float32 gate/up
+ * partial products [GATE_UP_SLICES][2][pairs][intermediate], float32 down partials [DOWN_SLICES][pairs][hidden] */
+ANEMONE_INLINE uint64_t exl3_tc_operand_bytes(uint64_t pairs, uint64_t hidden)
+{
+    return (2u * pairs * hidden * 2u + 255u) / 256u * 256u;
+}
+ANEMONE_INLINE uint64_t exl3_tc_gate_up_bytes(uint64_t pairs, uint64_t intermediate)
+{
+    return (EXL3_TC_GATE_UP_SLICES * 2u * pairs * intermediate * 4u + 255u) / 256u * 256u;
+}
+ANEMONE_INLINE uint64_t exl3_tc_down_bytes(uint64_t pairs, uint64_t hidden)
+{
+    return (EXL3_TC_DOWN_SLICES * pairs * hidden * 4u + 255u) / 256u * 256u;
+}
+ANEMONE_INLINE uint64_t exl3_tc_workspace_bytes(uint64_t pairs, uint64_t hidden, uint64_t intermediate)
+{
+    return exl3_tc_operand_bytes(pairs, hidden) + exl3_tc_gate_up_bytes(pairs, intermediate) +
+           exl3_tc_down_bytes(pairs, hidden);
+}
+
+/* ---- FP4 / FP8 expert linears ---- */
+#define KERNEL_FILE_ACTIVATION_QUANTIZE "kernel_activation_quantize"
+#define KERNEL_FILE_EXPERT_LINEAR "kernel_expert_linear"
+#define KERNEL_ACTIVATION_QUANTIZE "activation_quantize_entry"
+#define KERNEL_EXPERT_GATE_UP_STEM "expert_gate_up_"
+#define KERNEL_EXPERT_DOWN_STEM "expert_down_"
+#define KERNEL_EXPERT_ROW_SUM "expert_row_sum_entry"
+
+struct activation_quantize_arguments {
+    uint64_t values_offset;    /* read: bf16 [V][width] */
+    uint64_t codes_offset;     /* written: E4M3 codes [V][width], lane order */
+    uint64_t exponents_offset; /* written: E8M0 [V][width / 32] */
+    uint64_t operands_offset;  /* written: bf16 x 2^100 [V][width], operand order */
+    uint32_t width;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(activation_quantize_arguments, 40);
+
+struct expert_gate_up_arguments {
+    uint64_t jobs_offset;
+    uint64_t codes_offset;     /* read: codes [R][input_size] */
+    uint64_t exponents_offset;
+    uint64_t operands_offset;
+    uint64_t hidden_offset;    /* written: bf16 [pair][output_size] */
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t pair_count;
+    uint32_t pairs_per_row;
+    float activation_limit;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(expert_gate_up_arguments, 64);
+
+struct expert_down_arguments {
+    uint64_t jobs_offset;
+    uint64_t codes_offset;     /* read: codes [pair][input_size] */
+    uint64_t exponents_offset;
+    uint64_t operands_offset;
+    uint64_t output_offset;    /* written: bf16 [pair][output_size] */
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t pair_count;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(expert_down_arguments, 56);
+
+#endif
