@@ -1,0 +1,73 @@
+"""Seeded synthetic tensors of the benchmark configurations: one generator (splitmix64) for everything, normals by
+Box-Muller in double precision, rounded once. Numpy only; used by bench.py, the smoke run and the tests."""
+import numpy as np
+
+SEED = 0x5EED0000
+
+
+def splitmix_words(seed, count):
+    with np.errstate(over="ignore"):
+        z = (np.arange(1, count + 1, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15)) + np.uint64(seed)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def uniform01(seed, count):
+    return (splitmix_words(seed, count) >> np.uint64(11)).astype(np.float64) * (1.0 / (1 << 53))
+
+
+def normals(seed, count):
+    n = (count + 1) // 2
+    u = uniform01(seed, 2 * n)
+    r = np.sqrt(-2.0 * np.log(np.maximum(u[:n], 1e-300)))
+    return np.concatenate([r * np.cos(2 * np.pi * u[n:]), r * np.sin(2 * np.pi * u[n:])])[:count]
+
+
+def to_bf16(values):
+    bits = np.asarray(values, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def bf16_to_f32(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def exl3_bits_x2(stored_width):
+    return 2 * stored_width if 1 <= stored_width <= 8 else stored_width // 8
+
+
+def exl3_matrix_bytes(inputs, outputs, stored_width):
+    return inputs * outputs // 16 * exl3_bits_x2(stored_width) + 2 * (inputs + outputs)
+
+
+def exl3_matrix(seed, inputs, outputs, stored_width):
+    """One stored EXL3 matrix: uniform random codes (every bit pattern is a tile), suh = +-1,
+    svh = +-U(0.5, 1.5) / 64 rounded to fp16."""
+    code_bytes = inputs * outputs // 16 * exl3_bits_x2(stored_width)
+    codes = splitmix_words(seed, code_bytes // 8).view(np.uint8)
+    signs = splitmix_words(seed ^ 0xABCDEF, inputs + outputs)
+    suh = np.where(signs[:inputs] & np.uint64(1), 1.0, -1.0).astype(np.float16)
+    magnitude = (0.5 + uniform01(seed ^ 0x123457, outputs)) / 64.0
+    svh = (np.where(signs[inputs:] & np.uint64(1), 1.0, -1.0) * magnitude).astype(np.float16)
+    return np.concatenate([codes, suh.view(np.uint8), svh.view(np.uint8)])
+
+
+def exl3_moe_layer(config, hidden, inner, expert_count, width_choices=(2, 3, 4), probabilities=(0.30, 0.50, 0.20)):
+    """Widths [E][3] drawn per tensor and the experts' stored matrices; router weights bf16 N(0, 0.02)."""
+    base = SEED + (config << 20)
+    draws = uniform01(base + 1, expert_count * 3)
+    edges = np.cumsum(probabilities)
+    widths = np.array(width_choices, dtype=np.uint32)[np.minimum(np.searchsorted(edges, draws, side="right"), len(width_choices) - 1)]
+    widths = widths.reshape(expert_count, 3)
+    matrices = []
+    for e in range(expert_count):
+        matrices.append([exl3_matrix(base + 16 + 3 * e + 0, hidden, inner, int(widths[e, 0])),
+                         exl3_matrix(base + 16 + 3 * e + 1, hidden, inner, int(widths[e, 1])),
+                         exl3_matrix(base + 16 + 3 * e + 2, inner, hidden, int(widths[e, 2]))])
+    router = to_bf16(normals(base + 2, expert_count * hidden) * 0.02).reshape(expert_count, hidden)
+    return widths, matrices, router
+
+
+def activations(config, rows, hidden):
+    return to_bf16(normals(SEED + (config << 20) + 3, rows * hidden)).reshape(rows, hidden)

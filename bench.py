@@ -1,0 +1,181 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed-expert hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload exl3_decode]
+
+Workload `exl3_decode` (the configuration the metric is quoted on): the routed MoE layer of a decode step of 8
+tokens: hidden 4096, 256 SwiGLU experts of intermediate 2048, sigmoid router choosing 8 experts a token, EXL3 expert
+weights with one width K in {2, 3, 4} drawn per tensor (about 2.9 bits a weight), seeded synthetic tensors, bf16
+activations N(0, 1). A step is one pass of the path over the batch: router projection, select (top-k, weights, job
+table) and the five launches of the fused EXL3 experts, with every input already resident in HBM.
+
+Prints ONE JSON line: tokens/s of the whole job, the roofline of the dominant kernel (the gate/up products: achieved
+HBM bytes/s of its algorithmic bytes against the published 8 TB/s) and the CPU oracle timed on this box's host cores
+on the same step. The oracle is used here as checker and baseline only; the measured path is the HIP library."""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
+CONFIG = 1
+
+
+def cpu_oracle_step(orc_module, layer, x, router, matrices, widths, threads):
+    """The same step on the host cores by the CPU oracle: routing, then the experts. Returns (seconds, output)."""
+    import ctypes as C
+    o = orc_module
+    orc, ptr = o.orc, o.ptr
+    start = time.perf_counter()
+    scores = np.zeros((ROWS, EXPERTS), dtype=np.float32)
+    orc.orc_router_projection(ptr(x, o.u16p), ptr(router, o.u16p), ROWS, HIDDEN, EXPERTS, ptr(scores, o.f32p))
+    affinities = np.array([[orc.orc_router_affinity(float(s), 1) for s in row] for row in scores], dtype=np.float32)
+    experts = np.zeros((ROWS, PICKS), dtype=np.uint32)
+    weights = np.zeros((ROWS, PICKS), dtype=np.float32)
+    bias = np.zeros(EXPERTS, dtype=np.float32)
+    for r in range(ROWS):
+        orc.orc_router_select(ptr(affinities[r], o.f32p), ptr(bias, o.f32p), EXPERTS, PICKS, 0, 1.5,
+                              ptr(experts[r], o.u32p), ptr(weights[r], o.f32p))
+    pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
+    out = np.zeros((ROWS, HIDDEN), dtype=np.float32)
+    widths8 = np.ascontiguousarray(widths.astype(np.uint8))
+    orc.orc_exl3_moe_layer(ptr(x, o.u16p), ROWS, HIDDEN, INNER, PICKS, ptr(experts, o.u32p), ptr(weights, o.f32p), EXPERTS,
+                           pointers, ptr(widths8, o.u8p), 10.0, ptr(out, o.f32p), None, None, threads)
+    return time.perf_counter() - start, out, experts
+
+
+def calibrate(amd):
+    """A copy of 1 GiB inside the arena (1 GiB read, 1 GiB written), five launches."""
+    import ctypes as C
+    size = 1 << 30
+    card = amd.Card(3 << 30)
+    source, destination = card.reserve(size), card.reserve(size)
+    record = (C.c_uint64 * 3)(source, destination, size)
+    launch = amd.launches_of(1)
+    launch[0].kernel = card.kernel("kernel_calibrate", "arena_copy", 24)
+    launch[0].grid[0], launch[0].grid[1], launch[0].grid[2] = 256 * 16, 1, 1
+    launch[0].block[0], launch[0].block[1], launch[0].block[2] = 256, 1, 1
+    launch[0].argument_byte_count = 24
+    C.memmove(launch[0].argument, record, 24)
+    times = [card.run_timed(launch)[0] for _ in range(5)]
+    card.close()
+    print(json.dumps({"calibrate": "arena_copy", "bytes_read": size, "bytes_written": size, "launch_us": times,
+                      "GBps_read_plus_write": 2 * size / (min(times) * 1e-6) / 1e9}))
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=20)
+    parser.add_argument("--workload", default="exl3_decode")
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--calibrate", action="store_true",
+                        help="run only a 1 GiB arena copy, five times: the yardstick of the traffic counters")
+    arguments = parser.parse_args()
+    if arguments.gpus != 1:
+        print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
+        sys.exit(2)
+    if arguments.workload != "exl3_decode":
+        print("unknown workload %s" % arguments.workload, file=sys.stderr)
+        sys.exit(2)
+
+    import anemone_amd as amd
+    from anemone_amd import workloads
+
+    if arguments.calibrate:
+        calibrate(amd)
+        return
+
+    widths, matrices, router = workloads.exl3_moe_layer(CONFIG, HIDDEN, INNER, EXPERTS)
+    x = workloads.activations(CONFIG, ROWS, HIDDEN)
+    card = amd.Card(4 << 30)
+    layer = amd.Exl3Layer(card, HIDDEN, INNER, EXPERTS, PICKS, ROWS, matrices, widths, router_weights_bf16=router,
+                          affinity_kind=amd.AFFINITY_SIGMOID, route_scale=1.5, limit=10.0)
+    layer.set_rows(x, ROWS)
+    step = amd.launches_of(2 + amd.EXL3_TC_LAUNCHES)
+    step[0] = layer.projection_launch()[0]
+    step[1] = layer.select_launch(0)[0]
+    fused = layer.tc_launches()
+    for i in range(amd.EXL3_TC_LAUNCHES):
+        step[2 + i] = fused[i]
+    names = ["router_projection", "router_select_entry", "exl3_tc_operands", "exl3_tc_products(gate/up)",
+             "exl3_tc_activate", "exl3_tc_products(down)", "exl3_tc_combine"]
+
+    for _ in range(arguments.warmup):
+        card.run(step, wait=False)
+    card.wait()
+    # the timed region: exactly K steps between two waits, on the card's own clock and on the host's
+    host_start = time.perf_counter()
+    device_us = card.measure(lambda: [card.run(step, wait=False) for _ in range(arguments.steps)])
+    host_seconds = time.perf_counter() - host_start
+    seconds = max(device_us * 1e-6, 1e-12)
+    ms_per_step = 1000.0 * seconds / arguments.steps
+
+    # per-launch durations with a device timestamp between launches, over the same K steps
+    per_launch = np.zeros(len(names))
+    for _ in range(arguments.steps):
+        per_launch += np.array(card.run_timed(step))
+    per_launch /= arguments.steps
+
+    # what one gate/up launch reads by the algorithm: the gate and up matrices of the distinct routed experts
+    jobs = layer.jobs()
+    distinct = jobs[jobs["row_count"] > 0]["expert"]
+    gate_up_bytes = sum(workloads.exl3_matrix_bytes(HIDDEN, INNER, int(widths[e, 0])) +
+                        workloads.exl3_matrix_bytes(HIDDEN, INNER, int(widths[e, 1])) for e in distinct)
+    down_bytes = sum(workloads.exl3_matrix_bytes(INNER, HIDDEN, int(widths[e, 2])) for e in distinct)
+    step_bytes = gate_up_bytes + down_bytes + ROWS * HIDDEN * 2 + ROWS * HIDDEN * 4
+    gate_up_us = float(per_launch[3])
+    achieved = gate_up_bytes / (gate_up_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "MoE layer tok/s; decode HBM GB/s & prefill MFMA % of peak, 1 GPU",
+        "value": ROWS * arguments.steps / seconds,
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": arguments.steps,
+        "warmup": arguments.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "exl3_moe_decode: 8 tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router, "
+                               "EXL3 K in {2,3,4} per tensor (%.2f bpw)" % float(np.mean(widths)),
+                   "distinct_experts": int(len(distinct)), "step_algorithmic_bytes": int(step_bytes),
+                   "step_GBps": step_bytes / seconds * arguments.steps / 1e9,
+                   "host_clock_ms_per_step": 1000.0 * host_seconds / arguments.steps,
+                   "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)}},
+        "roofline": {"bound": "hbm", "kernel": "exl3_tc_products (gate/up pass)", "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
+    }
+
+    got = layer.output()
+    if not arguments.no_cpu:
+        import _oracle
+        threads = min(os.cpu_count() or 1, 16)
+        cpu_seconds, want, experts = cpu_oracle_step(_oracle, layer, x, router, matrices, widths, threads)
+        rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+        error = float(np.max(np.abs(got - want))) / rms
+        assert sorted(set(experts.reshape(-1).tolist())) == sorted(distinct.tolist()), "expert ids differ from the oracle's"
+        assert error <= 4e-3, "GPU output differs from the oracle's: %g of rms" % error
+        result["cpu_baseline"] = {"value": ROWS / cpu_seconds, "unit": "tok/s", "cores": threads, "kind": "port",
+                                  "sample": "1 step of the same workload (8 tokens, %d experts) by the CPU oracle, "
+                                            "double-precision sums" % len(distinct),
+                                  "seconds": cpu_seconds, "gpu_vs_oracle_max_err_over_rms": error}
+    card.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
