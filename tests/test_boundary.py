@@ -1,0 +1,284 @@
+"""CPU tests of the boundary: the library loads without a card, exports every function its headers declare, lists its
+kernels with the record sizes of anemone_records.h, and the prepare functions (pure arithmetic on a description; the
+arena is a number) keep the refusal rules and launch geometry stated in anemone_ops.h. A fake backend table with a
+kernel registry of names only stands in for a card, as the reference's host tests do
+(tests/host_memory_backend.h:30-45 of the reference)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import anemone_amd as amd
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ARENA = 1 << 34
+
+
+def declared_functions():
+    names = set()
+    for header in ("anemone_backend.h", "anemone_ops.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        for match in re.finditer(r"\b([a-z][a-z0-9_]+)\s*\((?!\s*\*)[^;{}]*\)\s*;", text):
+            name = match.group(1)
+            if name not in ("__attribute__", "warn_unused_result") and not name.startswith("result_status"):
+                names.add(name)
+    return names
+
+
+def test_library_exports_every_declared_function():
+    lib = amd.library()
+    names = declared_functions()
+    assert {"backend_hip_card_open", "exl3_tc_prepare", "router_select_prepare", "status_text",
+            "weight_format_operations_of", "exl3_row_sum_prepare"} <= names
+    missing = [name for name in sorted(names) if not hasattr(lib, name)]
+    assert missing == []
+    assert C.c_void_p.in_dll(lib, "backend_hip_value") is not None
+    assert C.c_void_p.in_dll(lib, "exl3_weight_operations") is not None
+
+
+def test_status_text_and_card_count_without_a_card():
+    assert amd.status_text(0) == "ok" and amd.status_text(7) == "unsupported" and amd.status_text(99) == "unknown status"
+    count = C.c_uint32(77)
+    assert amd.library().backend_hip_card_count(C.byref(count)) == 0
+    assert amd.library().backend_hip_card_count(None) == amd.STATUS_INVALID_ARGUMENT
+
+
+def kernel_table():
+    lib = amd.library()
+    f, g, b = C.c_char_p(), C.c_char_p(), C.c_uint32()
+    table = {}
+    for i in range(lib.backend_hip_kernel_table_count()):
+        assert lib.backend_hip_kernel_table_entry(i, C.byref(f), C.byref(g), C.byref(b)) == 0
+        table[(f.value.decode(), g.value.decode())] = b.value
+    return table
+
+
+def test_kernel_table_matches_the_records():
+    table = kernel_table()
+    assert table[("kernel_exl3", "exl3_reconstruct")] == C.sizeof(amd.Exl3ReconstructRecord) == 32
+    assert table[("kernel_exl3", "exl3_input")] == C.sizeof(amd.Exl3ExpertRecord) == 88
+    assert table[("kernel_exl3", "exl3_row_sum")] == C.sizeof(amd.RowSumArguments) == 24
+    assert table[("kernel_exl3_tc", "exl3_tc_products")] == C.sizeof(amd.Exl3TcRecord) == 88
+    for width in ("k2", "k2_5", "k3", "k4", "mixed"):
+        assert ("kernel_exl3", "exl3_gate_up_" + width) in table and ("kernel_exl3", "exl3_down_" + width) in table
+    assert table[("kernel_router", "router_select_entry")] == 96
+    assert C.sizeof(amd.KernelLaunch) == 232
+
+
+# ---- a fake backend: kernel_prepare over the library's own kernel table, no card ----
+
+PREPARE = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_char_p, C.c_char_p, C.c_uint32, C.POINTER(C.c_uint32))
+
+
+class FakeBackend:
+    def __init__(self):
+        self.table = kernel_table()
+        self.handles = []
+        self.callback = PREPARE(self.prepare)
+        # struct backend_operations: name, then 27 function pointers; kernel_prepare is the 11th member
+        self.operations = (C.c_void_p * 28)()
+        self.operations[11] = C.cast(self.callback, C.c_void_p)
+        self.card = C.c_void_p(0x1000)  # never dereferenced by a prepare function
+
+    def prepare(self, card, file, function, record_bytes, out):
+        key = (file.decode(), function.decode())
+        if key not in self.table:
+            return amd.STATUS_INVALID_ARGUMENT
+        if self.table[key] != record_bytes:
+            return amd.STATUS_INVALID_ARGUMENT
+        if key not in self.handles:
+            self.handles.append(key)
+        out[0] = self.handles.index(key)
+        return 0
+
+    @property
+    def address(self):
+        return C.addressof(self.operations)
+
+
+@pytest.fixture()
+def fake():
+    return FakeBackend()
+
+
+def chain_record(**changes):
+    r = amd.Exl3ExpertRecord()
+    pairs, H, I = 64, 4096, 2048
+    r.jobs_offset, r.input_offset = 4096, 1 << 20
+    r.operands_offset = 2 << 20
+    r.products_offset = r.output_offset = (2 << 20) + pairs * H * 4
+    r.hidden_offset = 16 << 20
+    r.input_size, r.inner_size, r.pair_count, r.pairs_per_row, r.job_count = H, I, pairs, 8, pairs
+    r.bits_per_weight, r.activation_limit = 3, 10.0
+    for key, value in changes.items():
+        setattr(r, key, value)
+    return r
+
+
+def test_chain_prepare_geometry(fake):
+    lib = amd.library()
+    launches = amd.launches_of(5)
+    assert lib.exl3_experts_prepare(C.byref(chain_record()), ARENA, fake.address, fake.card, 950, launches) == 0
+    names = [fake.handles[launch.kernel][1] for launch in launches]
+    assert names == ["exl3_input", "exl3_gate_up_k3", "exl3_activate", "exl3_down_k3", "exl3_finish"]
+    assert [list(l.grid) for l in launches] == [[32, 64, 2], [16, 64, 2], [16, 64, 1], [32, 64, 1], [32, 64, 1]]
+    assert [l.block[0] for l in launches] == [64, 256, 64, 256, 64]
+    assert all(l.argument_byte_count == 88 and not any(l.argument[88:]) for l in launches)
+    mixed = amd.launches_of(5)
+    assert lib.exl3_experts_prepare(C.byref(chain_record(widths_offset=1 << 30)), ARENA, fake.address, fake.card, 950, mixed) == 0
+    assert fake.handles[mixed[1].kernel][1] == "exl3_gate_up_mixed" and fake.handles[mixed[3].kernel][1] == "exl3_down_mixed"
+    assert lib.exl3_scratch_byte_count(64, 4096) == 64 * 4096 * 12
+    assert lib.exl3_width_name(6) == b"k3" and lib.exl3_width_name(5) == b"k2_5" and lib.exl3_width_name(7) is None
+
+
+@pytest.mark.parametrize("changes,status", [
+    (dict(reserved_zero=1), 1), (dict(pair_count=0), 1), (dict(pair_count=63), 1), (dict(job_count=0), 1),
+    (dict(output_offset=64), 1), (dict(activation_limit=0.0), 1), (dict(activation_limit=float("nan")), 1),
+    (dict(inner_size=8192), 1), (dict(bits_per_weight=9), 1), (dict(bits_per_weight=5), 7),
+    (dict(hidden_offset=(2 << 20) + 64), 1),   # shares bytes with the operands
+    (dict(jobs_offset=4100), 1),               # off the 16-byte alignment
+    (dict(hidden_offset=ARENA - 4096), 1),     # leaves the arena
+])
+def test_chain_prepare_refusals_leave_the_launches_untouched(fake, changes, status):
+    lib = amd.library()
+    launches = amd.launches_of(5)
+    C.memset(launches, 0xAB, C.sizeof(launches))
+    before = bytes(launches)
+    assert lib.exl3_experts_prepare(C.byref(chain_record(**changes)), ARENA, fake.address, fake.card, 950, launches) == status
+    assert bytes(launches) == before
+
+
+def test_chain_prepare_other_refusals(fake):
+    lib = amd.library()
+    launches = amd.launches_of(5)
+    assert lib.exl3_experts_prepare(C.byref(chain_record()), ARENA, fake.address, fake.card, 80, launches) == 1  # another class
+    assert lib.exl3_experts_prepare(None, ARENA, fake.address, fake.card, 950, launches) == 1
+    assert lib.exl3_experts_relaxed_prepare(C.byref(chain_record()), ARENA, fake.address, fake.card, 950, launches) == 7
+    assert lib.exl3_experts_fast_prepare(C.byref(chain_record()), ARENA, fake.address, fake.card, 950, launches) == 0
+
+
+def tc_record(**changes):
+    r = amd.Exl3TcRecord()
+    r.jobs_offset, r.hidden_offset, r.workspace_offset, r.output_offset = 4096, 1 << 20, 2 << 20, 1 << 30
+    r.row_count, r.job_capacity, r.intermediate, r.bits_x2 = 8, 64, 2048, 6
+    r.activation_limit, r.hidden, r.pairs_per_row = 10.0, 4096, 8
+    for key, value in changes.items():
+        setattr(r, key, value)
+    return r
+
+
+def test_tc_prepare_geometry_and_refusals(fake):
+    lib = amd.library()
+    launches = amd.launches_of(5)
+    assert lib.exl3_tc_prepare(C.byref(tc_record()), ARENA, fake.address, fake.card, launches) == 0
+    assert [fake.handles[l.kernel][1] for l in launches] == ["exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate",
+                                                            "exl3_tc_products", "exl3_tc_combine"]
+    assert [list(l.grid) for l in launches] == [[32, 64, 2], [16, 64, 4], [16, 64, 1], [32, 64, 1], [32, 8, 1]]
+    passes = [amd.Exl3TcRecord.from_buffer_copy(bytes(l.argument)[:88]).pass_ for l in launches]
+    assert passes == [0, 0, 0, 1, 0]
+    assert amd.exl3_tc_workspace_bytes(64, 4096, 2048) == 64 * 4096 * 4 + 8 * 2 * 64 * 2048 * 4 + 4 * 64 * 4096 * 4
+    for changes, status in [(dict(row_count=0), 1), (dict(row_count=65), 1), (dict(rotation=1), 7), (dict(shared_sum=1), 7),
+                            (dict(intermediate=2000), 7), (dict(bits_x2=7), 7), (dict(bits_x2=0), 1), (dict(pass_=1), 1),
+                            (dict(workspace_offset=(2 << 20) + 16), 1), (dict(output_offset=2 << 20), 1),
+                            (dict(activation_limit=-1.0), 1)]:
+        untouched = amd.launches_of(5)
+        assert lib.exl3_tc_prepare(C.byref(tc_record(**changes)), ARENA, fake.address, fake.card, untouched) == status, changes
+        assert not any(bytes(untouched))
+    # hidden 0 and pairs_per_row 0 stand for the reference's 5120 and 6
+    default = amd.launches_of(5)
+    assert lib.exl3_tc_prepare(C.byref(tc_record(hidden=0, pairs_per_row=0, intermediate=640, job_capacity=48)), ARENA,
+                               fake.address, fake.card, default) == 0
+    assert list(default[0].grid) == [40, 48, 2]
+
+
+def test_reconstruct_and_row_sum_prepare(fake):
+    lib = amd.library()
+    record = amd.Exl3ReconstructRecord(4096, 1 << 24, 2304, 5120, 3, 0)
+    launch = amd.launches_of(1)
+    assert lib.exl3_reconstruct_prepare(C.byref(record), ARENA, 0, launch) == 0
+    assert list(launch[0].grid) == [2304 * 5120 // 256, 1, 1] and launch[0].block[0] == 256
+    # the output overlapping the matrix, and an arena too short: refused, the launch untouched
+    for bad in (amd.Exl3ReconstructRecord(4096, 4096 + 1024, 2304, 5120, 3, 0), ):
+        untouched = amd.launches_of(1)
+        assert lib.exl3_reconstruct_prepare(C.byref(bad), ARENA, 0, untouched) == 1 and not any(bytes(untouched))
+    untouched = amd.launches_of(1)
+    assert lib.exl3_reconstruct_prepare(C.byref(record), 1 << 20, 0, untouched) == 1 and not any(bytes(untouched))
+    assert lib.exl3_reconstruct_prepare(C.byref(record), ARENA, amd.BACKEND_NO_KERNEL, untouched) == 1
+    row_sum = amd.RowSumArguments(1 << 20, 1 << 28, 4096, 8)
+    assert lib.exl3_row_sum_prepare(C.byref(row_sum), 8, ARENA, fake.address, fake.card, launch) == 0
+    assert list(launch[0].grid) == [16, 8, 1]
+
+
+def test_stored_byte_counts():
+    lib = amd.library()
+    lib.weight_format_operations_of.restype = C.c_void_p
+
+    class Operations(C.Structure):
+        _fields_ = [("name", C.c_char_p), ("stored_byte_count", C.CFUNCTYPE(C.c_int, C.POINTER(amd.Shape), C.POINTER(C.c_uint64)))]
+
+    def count(fmt, shape):
+        operations = Operations.from_address(lib.weight_format_operations_of(fmt))
+        out = C.c_uint64(0)
+        return operations.stored_byte_count(C.byref(shape), C.byref(out)), out.value
+
+    # the reference's known byte counts of a 2304 x 5120 EXL3 matrix (tests/exl3_widths_test.c:67-88)
+    for stored, expected in ((2, 2963968), (40, 3701248), (3, 4438528), (4, 5913088)):
+        assert count(amd.WEIGHT_FORMAT_EXL3, amd.Shape(2304, 5120, stored, 0)) == (0, expected)
+    assert count(amd.WEIGHT_FORMAT_EXL3, amd.Shape(2304, 5120, 5, 0))[0] == 7       # defined, not decoded here
+    assert count(amd.WEIGHT_FORMAT_EXL3, amd.Shape(2304, 5120, 9, 0))[0] == 1
+    assert count(amd.WEIGHT_FORMAT_EXL3, amd.Shape(2300, 5120, 3, 0))[0] == 1
+    assert count(amd.WEIGHT_FORMAT_E2M1_SCALED, amd.Shape(2048, 4096, 4, 0)) == (0, 4194304 + 262144)
+    assert count(amd.WEIGHT_FORMAT_E4M3_SCALED, amd.Shape(48, 64, 8, 0)) == (0, 48 * 64 + 4)
+    assert lib.weight_format_operations_of(0) is None and lib.weight_format_operations_of(1) is None
+
+
+def router_description(fake, **changes):
+    E, P, rows = 256, 8, 8
+    experts = amd.RoutedExpertsDescription()
+    experts.jobs = amd.Range(1 << 20, rows * P * 96)
+    experts.expert_weights = amd.Range(1 << 24, 1 << 32)
+    experts.gate_up_shape, experts.down_shape = amd.Shape(2048, 4096, 3, 0), amd.Shape(4096, 2048, 3, 0)
+    experts.weight_format, experts.job_count, experts.row_count, experts.pairs_per_row = amd.WEIGHT_FORMAT_EXL3, rows * P, rows, P
+    offsets = ((1 << 24) + np.arange(E * 3, dtype=np.uint64) * np.uint64(4 << 20))
+    d = amd.RouterDescription()
+    d.experts = C.pointer(experts)
+    d.expert_offsets = offsets.ctypes.data_as(C.POINTER(C.c_uint64))
+    d.step, d.scores, d.bias = amd.Range(256, 16), amd.Range(4096, rows * E * 4), amd.Range(65536, E * 4)
+    d.offsets, d.affinities = amd.Range(131072, E * 24), amd.Range(262144, rows * E * 4)
+    d.order, d.expert_count, d.pick_count, d.affinity_kind, d.route_scale = 0, E, P, 1, 1.5
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d, experts, offsets
+
+
+def test_router_prepare(fake):
+    lib = amd.library()
+    kernels = amd.RouterKernels()
+    # the wide kernels may be absent: the select and the projection are required
+    assert lib.router_kernels_prepare(fake.address, fake.card, C.byref(kernels)) == 0
+    assert kernels.select != amd.BACKEND_NO_KERNEL and kernels.projection != amd.BACKEND_NO_KERNEL
+    d, experts, offsets = router_description(fake)
+    launch = amd.launches_of(1)
+    assert lib.router_select_prepare(C.byref(d), ARENA, C.byref(kernels), launch) == 0
+    assert list(launch[0].grid) == [1, 1, 1] and launch[0].block[0] == 512 and launch[0].argument_byte_count == 96
+    for changes in (dict(expert_count=250), dict(pick_count=9), dict(order=1), dict(affinity_kind=2), dict(route_scale=0.0)):
+        bad, keep, keep2 = router_description(fake, **changes)
+        untouched = amd.launches_of(1)
+        assert lib.router_select_prepare(C.byref(bad), ARENA, C.byref(kernels), untouched) == 1, changes
+        assert not any(bytes(untouched))
+    # an entry of the offsets table whose matrix leaves the experts' range
+    bad, keep, table = router_description(fake)
+    table[5] = (1 << 24) + (1 << 32) - 4096
+    assert lib.router_select_prepare(C.byref(bad), ARENA, C.byref(kernels), launch) == 1
+    # the reference order is the six-pick tree alone
+    six, keep, keep2 = router_description(fake, order=1, pick_count=6, expert_count=384)
+    keep.pairs_per_row, keep.job_count = 6, 48
+    keep.jobs = amd.Range(1 << 20, 48 * 96)
+    offsets384 = ((1 << 24) + np.arange(384 * 3, dtype=np.uint64) * np.uint64(1 << 20))
+    six.expert_offsets = offsets384.ctypes.data_as(C.POINTER(C.c_uint64))
+    six.scores, six.affinities, six.bias, six.offsets = amd.Range(4096, 8 * 384 * 4), amd.Range(262144, 8 * 384 * 4), amd.Range(65536, 384 * 4), amd.Range(131072, 384 * 24)
+    keep.gate_up_shape, keep.down_shape = amd.Shape(512, 1024, 3, 0), amd.Shape(1024, 512, 3, 0)
+    assert lib.router_select_prepare(C.byref(six), ARENA, C.byref(kernels), launch) == 0
