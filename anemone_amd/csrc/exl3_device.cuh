@@ -112,9 +112,10 @@ __device__ static __forceinline__ uint32_t exl3_decode_pair(uint32_t state_low, 
 {
     const uint32_t product_low = state_low * EXL3_MUL1_MULTIPLIER;
     const uint32_t product_high = state_high * EXL3_MUL1_MULTIPLIER;
-    /* byte sums with the codebook's base folded in: 0x6400 + b is the fp16 1024 + b */
-    const uint32_t low = __builtin_amdgcn_sad_u8(product_low, 0u, EXL3_MUL1_BASE);
-    const uint32_t packed = __builtin_amdgcn_sad_hi_u8(product_high, 0u, low + ((uint32_t)EXL3_MUL1_BASE << 16));
+    /* byte sums with the codebook's base folded in as the accumulator: 0x6400 + b is the fp16 1024 + b. The first
+     * sum lands in the low half on top of 0x64006400, the second is added into the high half. */
+    const uint32_t low = __builtin_amdgcn_sad_u8(product_low, 0u, (uint32_t)EXL3_MUL1_BASE * 0x10001u);
+    const uint32_t packed = __builtin_amdgcn_sad_hi_u8(product_high, 0u, low);
     const half2_t value = __builtin_bit_cast(half2_t, packed);
     const half2_t scale = __builtin_bit_cast(half2_t, (uint32_t)EXL3_MUL1_SCALE * 0x10001u);
     const half2_t bias = __builtin_bit_cast(half2_t, (uint32_t)EXL3_MUL1_BIAS * 0x10001u);

@@ -21,7 +21,7 @@
 
 #define SELECT_THREADS (LINEAR_MAXIMUM_ROWS * WAVE) /* a wavefront for each row */
 #define PROJECTION_CHAINS 32u
-#define PROJECTION_THREADS 256u
+#define PROJECTION_THREADS 128u
 #define JOB_WORDS (sizeof(struct expert_job_record) / 4u)
 
 __device__ static __forceinline__ float det_log1pf(float y) /* 0 <= y <= 1 */
@@ -61,26 +61,95 @@ __device__ static __forceinline__ float router_affinity(float score, uint32_t ki
     return sqrtf(__fadd_rn(positive, det_log1pf(det_expf(-fabsf(score)))));
 }
 
-/* scores[row][expert] = sum_k w[expert][k] x[row][k]: 32 fma chains owning k mod 32, then a halving fold
- * (source/kernel_official_router_projection.cu:33-57). Half a wavefront an output. */
-extern "C" __global__ void router_projection(struct router_projection_arguments arguments, unsigned char *arena)
+/* scores[row][expert] = sum_k w[expert][k] x[row][k]: 32 fma chains, chain c owning the inputs k = c mod 32 in
+ * ascending order, then a halving fold 16, 8, 4, 2, 1 (source/kernel_official_router_projection.cu:33-57).
+ * A block takes PROJECTION_EXPERTS experts and up to PROJECTION_ROWS rows: it stages the weights and the rows in
+ * chunks of PROJECTION_CHUNK inputs through LDS with 16-byte coalesced loads (the next chunk in flight while this
+ * one is consumed); a thread owns chains 2 j and 2 j + 1 of one expert for every row, so the fma order of a chain
+ * is the definition's whatever the staging. grid (ceil(E / 8), ceil(rows / 4)), block 128. */
+#define PROJECTION_ROWS 4u
+#define PROJECTION_EXPERTS 8u
+#define PROJECTION_CHUNK 1024u
+#define PROJECTION_W_LOADS (PROJECTION_EXPERTS * PROJECTION_CHUNK * 2u / 16u / PROJECTION_THREADS)
+#define PROJECTION_X_LOADS (PROJECTION_ROWS * PROJECTION_CHUNK * 2u / 16u / PROJECTION_THREADS)
+extern "C" __global__ void __launch_bounds__(PROJECTION_THREADS)
+    router_projection(struct router_projection_arguments arguments, unsigned char *arena)
 {
-    const uint32_t chain = threadIdx.x % PROJECTION_CHAINS;
-    const uint32_t expert = blockIdx.x * (PROJECTION_THREADS / PROJECTION_CHAINS) + threadIdx.x / PROJECTION_CHAINS;
-    const uint32_t row = blockIdx.y;
-    const bool live = expert < arguments.expert_count;
-    const uint16_t *weight = (const uint16_t *)(arena + arguments.weights_offset) + (uint64_t)(live ? expert : 0u) * arguments.hidden;
-    const uint16_t *input = (const uint16_t *)(arena + arguments.rows_offset) + (uint64_t)row * arguments.hidden;
-    float sum = 0.0f;
-    for (uint32_t k = chain; k < arguments.hidden; k += PROJECTION_CHAINS) {
-        sum = __fmaf_rn(bf16_to_float(weight[k]), bf16_to_float(input[k]), sum);
+    __shared__ __attribute__((aligned(16))) uint16_t w_tile[PROJECTION_EXPERTS][PROJECTION_CHUNK];
+    __shared__ __attribute__((aligned(16))) uint16_t x_tile[PROJECTION_ROWS][PROJECTION_CHUNK];
+    const uint32_t H = arguments.hidden, thread = threadIdx.x;
+    const uint32_t first_expert = blockIdx.x * PROJECTION_EXPERTS, first_row = blockIdx.y * PROJECTION_ROWS;
+    const uint16_t *weights = (const uint16_t *)(arena + arguments.weights_offset);
+    const uint16_t *rows = (const uint16_t *)(arena + arguments.rows_offset);
+    uint4_t w_next[PROJECTION_W_LOADS], x_next[PROJECTION_X_LOADS];
+    /* piece p of a tile: 8 values of line p / (CHUNK / 8) at column 8 (p % (CHUNK / 8)); out of range reads zero */
+    auto fetch = [&](uint32_t chunk) {
+#pragma unroll
+        for (uint32_t i = 0; i < PROJECTION_W_LOADS; i++) {
+            const uint32_t piece = i * PROJECTION_THREADS + thread, line = piece / (PROJECTION_CHUNK / 8u);
+            const uint32_t k = chunk + 8u * (piece % (PROJECTION_CHUNK / 8u)), expert = first_expert + line;
+            w_next[i] = (uint4_t){0, 0, 0, 0};
+            if (expert < arguments.expert_count && k < H) {
+                w_next[i] = *(const uint4_t *)(weights + (uint64_t)expert * H + k);
+            }
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < PROJECTION_X_LOADS; i++) {
+            const uint32_t piece = i * PROJECTION_THREADS + thread, line = piece / (PROJECTION_CHUNK / 8u);
+            const uint32_t k = chunk + 8u * (piece % (PROJECTION_CHUNK / 8u)), row = first_row + line;
+            x_next[i] = (uint4_t){0, 0, 0, 0};
+            if (row < arguments.row_count && k < H) {
+                x_next[i] = *(const uint4_t *)(rows + (uint64_t)row * H + k);
+            }
+        }
+    };
+    const uint32_t expert_in_block = thread / 16u, pair = thread % 16u; /* chains 2 pair, 2 pair + 1 */
+    float chain[PROJECTION_ROWS][2];
+#pragma unroll
+    for (uint32_t r = 0; r < PROJECTION_ROWS; r++) {
+        chain[r][0] = chain[r][1] = 0.0f;
     }
-    sum = __fadd_rn(0.0f, sum);
-    for (uint32_t distance = PROJECTION_CHAINS / 2u; distance != 0u; distance >>= 1u) {
-        sum = __fadd_rn(sum, __shfl_down(sum, distance, PROJECTION_CHAINS));
+    fetch(0u);
+    for (uint32_t chunk = 0; chunk < H; chunk += PROJECTION_CHUNK) {
+        __syncthreads(); /* the tile's readers of the chunk before are done */
+#pragma unroll
+        for (uint32_t i = 0; i < PROJECTION_W_LOADS; i++) {
+            ((uint4_t *)&w_tile[0][0])[i * PROJECTION_THREADS + thread] = w_next[i];
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < PROJECTION_X_LOADS; i++) {
+            ((uint4_t *)&x_tile[0][0])[i * PROJECTION_THREADS + thread] = x_next[i];
+        }
+        if (chunk + PROJECTION_CHUNK < H) {
+            fetch(chunk + PROJECTION_CHUNK);
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (uint32_t k = 0; k < PROJECTION_CHUNK; k += PROJECTION_CHAINS) {
+            const uint32_t w = *(const uint32_t *)&w_tile[expert_in_block][k + 2u * pair];
+            const float w0 = __uint_as_float(w << 16), w1 = __uint_as_float(w & 0xFFFF0000u);
+#pragma unroll
+            for (uint32_t r = 0; r < PROJECTION_ROWS; r++) {
+                const uint32_t x = *(const uint32_t *)&x_tile[r][k + 2u * pair];
+                chain[r][0] = __fmaf_rn(w0, __uint_as_float(x << 16), chain[r][0]);
+                chain[r][1] = __fmaf_rn(w1, __uint_as_float(x & 0xFFFF0000u), chain[r][1]);
+            }
+        }
     }
-    if (chain == 0u && live) {
-        ((float *)(arena + arguments.output_offset))[(uint64_t)row * arguments.expert_count + expert] = __fadd_rn(0.0f, sum);
+    const uint32_t expert = first_expert + expert_in_block;
+#pragma unroll
+    for (uint32_t r = 0; r < PROJECTION_ROWS; r++) {
+        float even = __fadd_rn(0.0f, chain[r][0]), odd = __fadd_rn(0.0f, chain[r][1]);
+        /* chain c + distance lies distance / 2 threads on, for the distances 16, 8, 4, 2 */
+#pragma unroll
+        for (uint32_t distance = 8u; distance != 0u; distance >>= 1u) {
+            even = __fadd_rn(even, __shfl_down(even, distance, 16));
+            odd = __fadd_rn(odd, __shfl_down(odd, distance, 16));
+        }
+        const float sum = __fadd_rn(even, odd); /* distance 1: chain 0 + chain 1 */
+        if (pair == 0u && expert < arguments.expert_count && first_row + r < arguments.row_count) {
+            ((float *)(arena + arguments.output_offset))[(uint64_t)(first_row + r) * arguments.expert_count + expert] = __fadd_rn(0.0f, sum);
+        }
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_projection, router_projection_arguments);
@@ -92,16 +161,28 @@ __device__ static __forceinline__ uint64_t router_key(float biased, uint32_t exp
     return ((uint64_t)ordered << 32) | (uint32_t)~expert;
 }
 
+/* The largest 64-bit key of a wavefront, in every lane: a data-parallel-primitive scan (shift by 1, 2, 4, 8 inside
+ * rows of 16 lanes, then the row broadcasts), no LDS round trip; lane 63 holds the maximum. */
+template <int control, int row_mask>
+__device__ static __forceinline__ uint64_t dpp_max_step(uint64_t value)
+{
+    const uint32_t low = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)value, control, row_mask, 0xF, false);
+    const uint32_t high = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(value >> 32), control, row_mask, 0xF, false);
+    const uint64_t other = ((uint64_t)high << 32) | low; /* lanes without a source keep 0, below every key */
+    return other > value ? other : value;
+}
+
 __device__ static __forceinline__ uint64_t wave_max_u64(uint64_t value)
 {
-#pragma unroll
-    for (uint32_t distance = WAVE / 2u; distance != 0u; distance >>= 1u) {
-        const uint32_t low = __shfl_xor((uint32_t)value, (int)distance, WAVE);
-        const uint32_t high = __shfl_xor((uint32_t)(value >> 32), (int)distance, WAVE);
-        const uint64_t other = ((uint64_t)high << 32) | low;
-        value = other > value ? other : value;
-    }
-    return value;
+    value = dpp_max_step<0x111, 0xF>(value); /* row_shr:1 */
+    value = dpp_max_step<0x112, 0xF>(value); /* row_shr:2 */
+    value = dpp_max_step<0x114, 0xF>(value); /* row_shr:4 */
+    value = dpp_max_step<0x118, 0xF>(value); /* row_shr:8: lane 15 of a row holds the row's maximum */
+    value = dpp_max_step<0x142, 0xA>(value); /* row_bcast:15 into rows 1 and 3 */
+    value = dpp_max_step<0x143, 0xC>(value); /* row_bcast:31 into rows 2 and 3 */
+    const uint32_t low = __builtin_amdgcn_readlane((int)(uint32_t)value, 63);
+    const uint32_t high = __builtin_amdgcn_readlane((int)(uint32_t)(value >> 32), 63);
+    return ((uint64_t)high << 32) | low;
 }
 
 /* One row by one wavefront: its picks by slot and their weights, written by lane 0. */

@@ -6,7 +6,7 @@
  * per-matrix widths table.
  *
  *   launch        kernel                grid                        block
- *   projection    router_projection     (ceil(E / 8), rows, 1)      256   half a wavefront an output
+ *   projection    router_projection     (ceil(E / 8), ceil(rows / 4), 1)   128   eight experts and four rows a block
  *   select        router_select_entry   (1, 1, 1)                   512   a wavefront a row
  */
 #include <inttypes.h>
@@ -15,8 +15,9 @@
 #include "prepare_common.h"
 
 #define SELECT_THREADS (LINEAR_MAXIMUM_ROWS * 64u)
-#define PROJECTION_THREADS 256u
-#define PROJECTION_OUTPUTS 8u
+#define PROJECTION_THREADS 128u
+#define PROJECTION_OUTPUTS 8u /* experts a block */
+#define PROJECTION_ROWS 4u    /* rows a block takes at once */
 
 result_status router_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                      struct router_kernels_record *kernels_out)
@@ -234,7 +235,7 @@ result_status router_projection_prepare(const struct router_projection_descripti
         .expert_count = description->expert_count,
     };
     launch_fill(launch_out, kernels->projection, (description->expert_count + PROJECTION_OUTPUTS - 1u) / PROJECTION_OUTPUTS,
-                description->row_count, 1, PROJECTION_THREADS, 0, &record, sizeof record);
+                (description->row_count + PROJECTION_ROWS - 1u) / PROJECTION_ROWS, 1, PROJECTION_THREADS, 0, &record, sizeof record);
     return STATUS_OK;
 }
 
