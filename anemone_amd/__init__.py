@@ -97,6 +97,18 @@ class RouterProjectionDescription(C.Structure):
                 ("expert_count", u32), ("reserved_zero", u32)]
 
 
+class LinearKernels(C.Structure):
+    _fields_ = [("activation_quantize", u32), ("expert_gate_up", u32 * 5), ("expert_down", u32 * 5), ("expert_row_sum", u32),
+                ("trunk_linear_quantized", u32 * 5), ("trunk_linear_bfloat16", u32 * 5), ("trunk_hidden", u32),
+                ("trunk_linear_quantized_wide", u32 * 5), ("trunk_linear_bfloat16_wide", u32 * 5),
+                ("trunk_linear_quantized_interleaved", u32)]
+
+
+class QuantizeDescription(C.Structure):
+    _fields_ = [("values", Range), ("codes", Range), ("exponents", Range), ("operands", Range), ("width", u32),
+                ("row_count", u32)]
+
+
 JOB_DTYPE = np.dtype([("gate_offset", "<u8"), ("up_offset", "<u8"), ("down_offset", "<u8"), ("row_count", "<u4"),
                       ("expert", "<u4"), ("pair_index", "<u4", (8,)), ("route_weight", "<f4", (8,))])
 
@@ -142,6 +154,10 @@ def library():
             "router_kernels_prepare": [vp, vp, C.POINTER(RouterKernels)],
             "router_select_prepare": [C.POINTER(RouterDescription), u64, C.POINTER(RouterKernels), launch_p],
             "router_projection_prepare": [C.POINTER(RouterProjectionDescription), u64, C.POINTER(RouterKernels), launch_p],
+            "linear_kernels_prepare": [vp, vp, u32, C.POINTER(LinearKernels)],
+            "linear_quantize_prepare": [C.POINTER(QuantizeDescription), u64, C.POINTER(LinearKernels), launch_p],
+            "linear_routed_experts_prepare": [C.POINTER(RoutedExpertsDescription), u64, C.POINTER(LinearKernels), launch_p],
+            "linear_default_slice_count": [C.c_int, C.c_int, C.c_int, C.POINTER(Shape), u32, C.POINTER(u32)],
         }
         for name, argtypes in signatures.items():
             function = getattr(lib, name)
@@ -437,3 +453,104 @@ class Exl3Layer:
 
     def output(self):
         return self.card.download(self.out_offset, self.rows * self.H * 4, np.float32).reshape(self.rows, self.H)
+
+
+class Fp4Layer:
+    """One MoE layer of the original FP4 weights (WEIGHT_FORMAT_E2M1_SCALED, stored bytes as the reference's packs
+    hold them) in a card's arena, with the scratch ranges of a step of at most `rows` rows: the quantizer of the rows,
+    the router's select, and the four launches of the routed experts."""
+
+    def __init__(self, card, hidden, inner, expert_count, picks, rows, matrices, router_weights_bf16=None,
+                 affinity_kind=AFFINITY_SIGMOID, route_scale=1.5, limit=10.0, gate_up_slices=4, down_slices=2):
+        self.card, self.H, self.I, self.E, self.P, self.rows = card, hidden, inner, expert_count, picks, rows
+        self.limit, self.affinity_kind, self.route_scale = limit, affinity_kind, route_scale
+        self.gate_up_slices, self.down_slices = gate_up_slices, down_slices
+        self.pairs = rows * picks
+        lib = card.lib
+        total = sum(m.nbytes + 64 for trio in matrices for m in trio)
+        self.weights_offset, self.weights_bytes = card.reserve(total, 256), total
+        offsets = np.zeros((expert_count, 3), dtype=np.uint64)
+        cursor, blob = self.weights_offset, np.zeros(total, dtype=np.uint8)
+        for e, trio in enumerate(matrices):
+            for m, matrix in enumerate(trio):
+                cursor = (cursor + 63) // 64 * 64
+                offsets[e, m] = cursor
+                blob[cursor - self.weights_offset:cursor - self.weights_offset + matrix.nbytes] = matrix
+                cursor += matrix.nbytes
+        card.upload(self.weights_offset, blob)
+        self.expert_offsets = offsets
+        self.offsets_offset = card.place(offsets)
+        self.step_offset = card.place(step_block(rows))
+        self.x_offset = card.reserve(rows * hidden * 2)
+        self.scores_offset = card.reserve(rows * expert_count * 4)
+        self.affinities_offset = card.reserve(rows * expert_count * 4)
+        self.bias_offset = card.place(np.zeros(expert_count, dtype=np.float32))
+        self.router_offset = card.place(router_weights_bf16) if router_weights_bf16 is not None else 0
+        self.jobs_offset = card.reserve(self.pairs * 96)
+        names = {"codes": rows * hidden, "exponents": rows * hidden // 32, "operands": rows * hidden * 2,
+                 "hidden": self.pairs * inner * 2, "hidden_codes": self.pairs * inner,
+                 "hidden_exponents": self.pairs * inner // 32, "hidden_operands": self.pairs * inner * 2,
+                 "pair_output": self.pairs * hidden * 2, "row_output": rows * hidden * 4}
+        self.ranges = {name: Range(card.reserve(size), size) for name, size in names.items()}
+        self.kernels, self.router_kernels = LinearKernels(), RouterKernels()
+        check(lib.linear_kernels_prepare(backend_table(), card.handle, ARITHMETIC_CLASS_GFX950, C.byref(self.kernels)), "linear_kernels_prepare")
+        check(lib.router_kernels_prepare(backend_table(), card.handle, C.byref(self.router_kernels)), "router_kernels_prepare")
+
+    def set_rows(self, x_bf16, live_rows=None):
+        self.card.upload(self.x_offset, x_bf16)
+        self.card.upload(self.step_offset, step_block(self.rows if live_rows is None else live_rows))
+
+    def experts_description(self):
+        d = RoutedExpertsDescription()
+        d.jobs = Range(self.jobs_offset, self.pairs * 96)
+        d.expert_weights = Range(self.weights_offset, self.weights_bytes)
+        for name, value in self.ranges.items():
+            setattr(d, name, value)
+        d.gate_up_shape, d.down_shape = Shape(self.I, self.H, 4, 0), Shape(self.H, self.I, 4, 0)
+        d.weight_format = WEIGHT_FORMAT_E2M1_SCALED
+        d.job_count, d.row_count, d.pairs_per_row = self.pairs, self.rows, self.P
+        d.gate_up_slice_count, d.down_slice_count = self.gate_up_slices, self.down_slices
+        d.activation_limit = self.limit
+        return d
+
+    def quantize_launch(self):
+        d = QuantizeDescription(Range(self.x_offset, self.rows * self.H * 2), self.ranges["codes"], self.ranges["exponents"],
+                                self.ranges["operands"], self.H, self.rows)
+        launch = launches_of(1)
+        check(self.card.lib.linear_quantize_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launch), "linear_quantize_prepare")
+        return launch
+
+    def projection_launch(self):
+        d = RouterProjectionDescription(Range(self.router_offset, self.E * self.H * 2), Range(self.x_offset, self.rows * self.H * 2),
+                                        Range(self.scores_offset, self.rows * self.E * 4), self.rows, self.H, self.E, 0)
+        launch = launches_of(1)
+        check(self.card.lib.router_projection_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.router_kernels), launch), "router_projection_prepare")
+        return launch
+
+    def select_launch(self, order=0):
+        experts = self.experts_description()
+        d = RouterDescription()
+        d.experts = C.pointer(experts)
+        d.expert_offsets = self.expert_offsets.ctypes.data_as(C.POINTER(u64))
+        d.expert_widths = None
+        d.step, d.scores = Range(self.step_offset, 16), Range(self.scores_offset, self.rows * self.E * 4)
+        d.bias, d.offsets = Range(self.bias_offset, self.E * 4), Range(self.offsets_offset, self.E * 24)
+        d.affinities = Range(self.affinities_offset, self.rows * self.E * 4)
+        d.order, d.expert_count, d.pick_count = order, self.E, self.P
+        d.affinity_kind, d.route_scale = self.affinity_kind, self.route_scale
+        launch = launches_of(1)
+        check(self.card.lib.router_select_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.router_kernels), launch), "router_select_prepare")
+        return launch
+
+    def expert_launches(self):
+        d = self.experts_description()
+        launches = launches_of(4)
+        check(self.card.lib.linear_routed_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launches), "linear_routed_experts_prepare")
+        return launches
+
+    def read(self, name, dtype=np.uint8):
+        r = self.ranges[name]
+        return self.card.download(r.byte_offset, r.byte_count, dtype)
+
+    def jobs(self):
+        return self.card.download(self.jobs_offset, self.pairs * 96).view(JOB_DTYPE)

@@ -1,0 +1,223 @@
+/*
+ * linear.c -- load-time preparation of the FP4 routed experts and of the activation quantizer: the routed part of
+ * the reference's source/linear.c (linear_kernels_prepare :292-311, linear_default_slice_count :567-593,
+ * linear_quantize_prepare :1088-1120, linear_routed_experts_prepare :1263-1390, the byte counts :716-724).
+ *
+ *   launch      kernel                      grid                                  block        shared
+ *   gate/up     expert_gate_up_<S>          (output_size / 16, jobs, 1)           128 S        static
+ *   quantize    activation_quantize_entry   (ceil(width / 256), pairs, 1)         256          0
+ *   down        expert_down_<S>             (output_size / 16, jobs, 1)           64 S         static
+ *   row sum     expert_row_sum_entry        (ceil(width / 256), rows, 1)          256          0
+ * A wavefront is 64 lanes, so a slice is a wavefront (gate with up: two); 16 slices would be a block of 2,048
+ * threads, which the card does not run: the instances are 1, 2, 4 and 8.
+ */
+#include <inttypes.h>
+#include <math.h>
+#include <string.h>
+
+#include "prepare_common.h"
+
+static const uint32_t slice_counts[LINEAR_SLICE_INSTANCES] = {1u, 2u, 4u, 8u, 16u};
+#define BUILT_INSTANCES 4u
+#define MOST_ROWS 4096u /* rows of one call: a wide step's chunk */
+
+uint64_t linear_values_byte_count(uint64_t vector_count, uint64_t width)
+{
+    return product_or_most(product_or_most(vector_count, width), 2u);
+}
+uint64_t linear_codes_byte_count(uint64_t vector_count, uint64_t width)
+{
+    return product_or_most(vector_count, width);
+}
+uint64_t linear_exponents_byte_count(uint64_t vector_count, uint64_t width)
+{
+    return product_or_most(vector_count, width / LINEAR_VALUES_PER_BLOCK);
+}
+uint64_t linear_sums_byte_count(uint64_t row_count, uint64_t width)
+{
+    return product_or_most(product_or_most(row_count, width), 4u);
+}
+uint64_t linear_jobs_byte_count(uint64_t job_count)
+{
+    return product_or_most(job_count, sizeof(struct expert_job_record));
+}
+
+result_status linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                     uint32_t arithmetic_class, struct linear_kernels_record *kernels_out)
+{
+    if (backend == NULL || backend->kernel_prepare == NULL || card == NULL || kernels_out == NULL ||
+        arithmetic_class != ARITHMETIC_CLASS_GFX950) {
+        REFUSE("the kernels of the linear: a missing argument, or a class other than %u", ARITHMETIC_CLASS_GFX950);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    struct linear_kernels_record kernels;
+    memset(&kernels, 0xFF, sizeof kernels); /* every handle BACKEND_NO_KERNEL */
+    result_status status = backend->kernel_prepare(card, KERNEL_FILE_ACTIVATION_QUANTIZE, KERNEL_ACTIVATION_QUANTIZE,
+                                                   sizeof(struct activation_quantize_arguments), &kernels.activation_quantize);
+    for (uint32_t instance = 0; status == STATUS_OK && instance < BUILT_INSTANCES; instance++) {
+        char name[40];
+        (void)snprintf(name, sizeof name, "%s%u", KERNEL_EXPERT_GATE_UP_STEM, slice_counts[instance]);
+        status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, name, sizeof(struct expert_gate_up_arguments),
+                                         &kernels.expert_gate_up[instance]);
+        if (status == STATUS_OK) {
+            (void)snprintf(name, sizeof name, "%s%u", KERNEL_EXPERT_DOWN_STEM, slice_counts[instance]);
+            status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, name, sizeof(struct expert_down_arguments),
+                                             &kernels.expert_down[instance]);
+        }
+    }
+    if (status == STATUS_OK) {
+        status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, KERNEL_EXPERT_ROW_SUM,
+                                         sizeof(struct expert_row_sum_arguments), &kernels.expert_row_sum);
+    }
+    if (status != STATUS_OK) {
+        REFUSE("the kernels of the linear: a kernel is not prepared: %s", status_text(status));
+        return status;
+    }
+    *kernels_out = kernels;
+    return STATUS_OK;
+}
+
+result_status linear_default_slice_count(enum linear_profile_code profile, enum linear_order_code order,
+                                         enum linear_family_code family, const struct matrix_shape_record *shape,
+                                         uint32_t arithmetic_class, uint32_t *slice_count_out)
+{
+    if (shape == NULL || slice_count_out == NULL || (profile != LINEAR_PROFILE_PRECISION && profile != LINEAR_PROFILE_SPEED) ||
+        (order != LINEAR_ORDER_FIXED && order != LINEAR_ORDER_REFERENCE) || arithmetic_class != ARITHMETIC_CLASS_GFX950 ||
+        (family != LINEAR_FAMILY_EXPERT_GATE_UP && family != LINEAR_FAMILY_EXPERT_DOWN) || shape->input_size == 0 ||
+        shape->input_size % 128u != 0) {
+        REFUSE("the default slice count: a profile, order, family, shape or class the table has no row for");
+        return STATUS_INVALID_ARGUMENT;
+    }
+    uint32_t count = order == LINEAR_ORDER_REFERENCE ? 1u : family == LINEAR_FAMILY_EXPERT_GATE_UP ? 4u : 2u;
+    while (count > shape->input_size / 128u) { /* at most one slice a K step of 128 inputs */
+        count /= 2u;
+    }
+    *slice_count_out = count;
+    return STATUS_OK;
+}
+
+result_status linear_quantize_prepare(const struct linear_quantize_description *description, uint64_t arena_byte_count,
+                                      const struct linear_kernels_record *kernels, struct kernel_launch *launch_out)
+{
+    static const char what[] = "the activation quantizer";
+    if (description == NULL || kernels == NULL || launch_out == NULL || kernels->activation_quantize == BACKEND_NO_KERNEL) {
+        REFUSE("%s: a missing argument or an unprepared kernel", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (description->width == 0 || description->width % LINEAR_VALUES_PER_LOAD != 0 || description->row_count == 0 ||
+        description->row_count > 65535u) {
+        REFUSE("%s: a width that is 0 or no multiple of %u, or a row count of 0 or above 65535", what, LINEAR_VALUES_PER_LOAD);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t rows = description->row_count, width = description->width;
+    const struct checked_range ranges[] = {
+        {"the values", description->values, linear_values_byte_count(rows, width), false},
+        {"the codes", description->codes, linear_codes_byte_count(rows, width), false},
+        {"the exponents", description->exponents, linear_exponents_byte_count(rows, width), false},
+        {"the operands", description->operands, linear_values_byte_count(rows, width), false},
+    };
+    if (!ranges_are_valid(what, ranges, 4, arena_byte_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct activation_quantize_arguments record = {description->values.byte_offset, description->codes.byte_offset,
+                                                         description->exponents.byte_offset,
+                                                         description->operands.byte_offset, description->width, 0};
+    launch_fill(launch_out, kernels->activation_quantize, (description->width + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS,
+                description->row_count, 1, LINEAR_ELEMENT_THREADS, 0, &record, sizeof record);
+    return STATUS_OK;
+}
+
+static bool instance_of(uint32_t slice_count, uint32_t input_size, uint32_t *instance_out)
+{
+    for (uint32_t instance = 0; instance < BUILT_INSTANCES; instance++) {
+        if (slice_counts[instance] == slice_count && slice_count <= input_size / 128u) {
+            *instance_out = instance;
+            return true;
+        }
+    }
+    return false;
+}
+
+result_status linear_routed_experts_prepare(const struct linear_routed_experts_description *description,
+                                            uint64_t arena_byte_count, const struct linear_kernels_record *kernels,
+                                            struct kernel_launch *launches_out)
+{
+    static const char what[] = "the routed experts";
+    if (description == NULL || kernels == NULL || launches_out == NULL) {
+        REFUSE("%s: a missing argument", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct matrix_shape_record *gate_up = &description->gate_up_shape, *down = &description->down_shape;
+    const struct weight_format_operations *format = weight_format_operations_of(description->weight_format);
+    uint64_t gate_up_bytes = 0, down_bytes = 0;
+    uint32_t gate_up_instance = 0, down_instance = 0;
+    if (description->reserved_zero != 0 || description->weight_format != WEIGHT_FORMAT_E2M1_SCALED || format == NULL ||
+        format->stored_byte_count(gate_up, &gate_up_bytes) != STATUS_OK ||
+        format->stored_byte_count(down, &down_bytes) != STATUS_OK || gate_up->input_size % 128u != 0 ||
+        down->input_size % 128u != 0 || down->input_size != gate_up->output_size) {
+        REFUSE("%s: matrices of format %u in shapes it stores, inputs a multiple of 128, down reading what gate and up "
+               "write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (!instance_of(description->gate_up_slice_count, gate_up->input_size, &gate_up_instance) ||
+        !instance_of(description->down_slice_count, down->input_size, &down_instance)) {
+        REFUSE("%s: slice counts %u and %u: 1, 2, 4 or 8, at most one a 128 inputs", what,
+               description->gate_up_slice_count, description->down_slice_count);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (kernels->expert_gate_up[gate_up_instance] == BACKEND_NO_KERNEL || kernels->expert_down[down_instance] == BACKEND_NO_KERNEL ||
+        kernels->activation_quantize == BACKEND_NO_KERNEL || kernels->expert_row_sum == BACKEND_NO_KERNEL) {
+        REFUSE("%s: a kernel of the chain is not prepared", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t rows = description->row_count, pairs = rows * description->pairs_per_row;
+    if (rows == 0 || rows > MOST_ROWS || description->pairs_per_row == 0 || pairs > UINT32_MAX || description->job_count == 0 ||
+        description->job_count > 65535u || pairs > 65535u || !(description->activation_limit > 0.0f)) {
+        REFUSE("%s: 1 to %u rows, pairs and jobs from 1 to 65535, an activation limit above zero", what, MOST_ROWS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t H = gate_up->input_size, I = gate_up->output_size, O = down->output_size;
+    const struct checked_range ranges[] = {
+        {"the job table", description->jobs, linear_jobs_byte_count(description->job_count), false},
+        {"the experts' matrices", description->expert_weights, gate_up_bytes > down_bytes ? gate_up_bytes : down_bytes, false},
+        {"the rows' codes", description->codes, linear_codes_byte_count(rows, H), false},
+        {"the rows' exponents", description->exponents, linear_exponents_byte_count(rows, H), false},
+        {"the rows' operands", description->operands, 0, false},
+        {"the hidden values", description->hidden, linear_values_byte_count(pairs, I), false},
+        {"the hidden codes", description->hidden_codes, linear_codes_byte_count(pairs, I), false},
+        {"the hidden exponents", description->hidden_exponents, linear_exponents_byte_count(pairs, I), false},
+        {"the hidden operands", description->hidden_operands, linear_values_byte_count(pairs, I), false},
+        {"the pair outputs", description->pair_output, linear_values_byte_count(pairs, O), false},
+        {"the row outputs", description->row_output, linear_sums_byte_count(rows, O), false},
+    };
+    if (!ranges_are_valid(what, ranges, sizeof ranges / sizeof ranges[0], arena_byte_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct expert_gate_up_arguments gate_up_record = {
+        description->jobs.byte_offset, description->codes.byte_offset, description->exponents.byte_offset,
+        description->operands.byte_offset, description->hidden.byte_offset, gate_up->output_size, gate_up->input_size,
+        (uint32_t)pairs, description->pairs_per_row, description->activation_limit, 0};
+    const struct activation_quantize_arguments quantize_record = {
+        description->hidden.byte_offset, description->hidden_codes.byte_offset, description->hidden_exponents.byte_offset,
+        description->hidden_operands.byte_offset, gate_up->output_size, 0};
+    const struct expert_down_arguments down_record = {
+        description->jobs.byte_offset, description->hidden_codes.byte_offset, description->hidden_exponents.byte_offset,
+        description->hidden_operands.byte_offset, description->pair_output.byte_offset, down->output_size, down->input_size,
+        (uint32_t)pairs, 0};
+    const struct expert_row_sum_arguments row_sum_record = {description->pair_output.byte_offset,
+                                                            description->row_output.byte_offset, down->output_size,
+                                                            description->pairs_per_row};
+    struct kernel_launch launches[LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT];
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_GATE_UP], kernels->expert_gate_up[gate_up_instance], gate_up->output_size / 16u,
+                description->job_count, 1, 128u * description->gate_up_slice_count, 0, &gate_up_record, sizeof gate_up_record);
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_QUANTIZE], kernels->activation_quantize,
+                (gate_up->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)pairs, 1,
+                LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_DOWN], kernels->expert_down[down_instance], down->output_size / 16u,
+                description->job_count, 1, 64u * description->down_slice_count, 0, &down_record, sizeof down_record);
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_ROW_SUM], kernels->expert_row_sum,
+                (down->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)rows, 1,
+                LINEAR_ELEMENT_THREADS, 0, &row_sum_record, sizeof row_sum_record);
+    memcpy(launches_out, launches, sizeof launches);
+    return STATUS_OK;
+}

@@ -71,3 +71,37 @@ def exl3_moe_layer(config, hidden, inner, expert_count, width_choices=(2, 3, 4),
 
 def activations(config, rows, hidden):
     return to_bf16(normals(SEED + (config << 20) + 3, rows * hidden)).reshape(rows, hidden)
+
+
+def e2m1_lay_out(codes, scales):
+    """codes uint8 [outputs][inputs] (0..15), scales uint8 [outputs][inputs / 32] -> the stored bytes of
+    WEIGHT_FORMAT_E2M1_SCALED: words [tile][load][lane][step] (nibble at bit 4 r + 16 h of a word is
+    W[16 tile + g + 8 (r % 2)][64 load + 16 step + 2 t + 8 (r / 2) + h], lane = 4 g + t), then the scales
+    [tile][load][g] (byte 2 q + r: inputs 64 load + 32 q.. of output 16 tile + g + 8 r)."""
+    outputs, inputs = codes.shape
+    tiles, loads = outputs // 16, inputs // 64
+    # w[tile, r%2, g, load, step, r/2, t, h]
+    w = codes.reshape(tiles, 2, 8, loads, 4, 2, 4, 2).astype(np.uint32)
+    words = np.zeros((tiles, loads, 8, 4, 4), dtype=np.uint32)  # [tile][load][g][t][step]
+    for r in range(4):
+        for h in range(2):
+            words |= w[:, r % 2, :, :, :, r // 2, :, h].transpose(0, 2, 1, 4, 3) << np.uint32(4 * r + 16 * h)
+    s = scales.reshape(tiles, 2, 8, loads, 2)  # [tile][r][g][load][q]
+    scale_bytes = s.transpose(0, 3, 2, 4, 1)    # [tile][load][g][q][r]
+    return np.concatenate([words.reshape(-1).view(np.uint8), np.ascontiguousarray(scale_bytes).reshape(-1)])
+
+
+def fp4_matrix(seed, outputs, inputs, scale_code=120):
+    """Uniform random E2M1 codes with E8M0 scales scale_code + {0, 1}: weights of standard deviation about 0.02."""
+    raw = splitmix_words(seed, outputs * inputs // 16)
+    codes = ((raw[:, None] >> (np.arange(16, dtype=np.uint64) * np.uint64(4))) & np.uint64(15)).astype(np.uint8).reshape(outputs, inputs)
+    scales = (scale_code + (splitmix_words(seed ^ 0x5CA1E, outputs * inputs // 32) & np.uint64(1))).astype(np.uint8).reshape(outputs, inputs // 32)
+    return e2m1_lay_out(codes, scales)
+
+
+def fp4_moe_layer(config, hidden, inner, expert_count):
+    base = SEED + (config << 20)
+    matrices = [[fp4_matrix(base + 16 + 3 * e + 0, inner, hidden), fp4_matrix(base + 16 + 3 * e + 1, inner, hidden),
+                 fp4_matrix(base + 16 + 3 * e + 2, hidden, inner)] for e in range(expert_count)]
+    router = to_bf16(normals(base + 2, expert_count * hidden) * 0.02).reshape(expert_count, hidden)
+    return matrices, router

@@ -170,6 +170,70 @@ MUST_CHECK result_status router_wide_prepare(const struct router_wide_descriptio
                                              const struct router_kernels_record *kernels,
                                              struct kernel_launch *launches_out);
 
+/* ---- FP4 / FP8 expert linears of the original weights (the routed part of the reference's linear.h) ---- */
+#define LINEAR_SLICE_INSTANCES 5u /* product kernels are stamped for 1, 2, 4, 8, 16 slices; gfx950 holds 1, 2, 4, 8 */
+#define LINEAR_MAXIMUM_SLICES 16u
+struct linear_kernels_record { /* include/anemone/linear.h:121-132 of the reference, member for member */
+    uint32_t activation_quantize;
+    uint32_t expert_gate_up[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_down[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_row_sum;
+    uint32_t trunk_linear_quantized[LINEAR_SLICE_INSTANCES]; /* the trunk families are outside this path: */
+    uint32_t trunk_linear_bfloat16[LINEAR_SLICE_INSTANCES];  /* every trunk handle is BACKEND_NO_KERNEL */
+    uint32_t trunk_hidden;
+    uint32_t trunk_linear_quantized_wide[LINEAR_SLICE_INSTANCES];
+    uint32_t trunk_linear_bfloat16_wide[LINEAR_SLICE_INSTANCES];
+    uint32_t trunk_linear_quantized_interleaved;
+};
+MUST_CHECK result_status linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                                uint32_t arithmetic_class, struct linear_kernels_record *kernels_out);
+
+enum linear_profile_code { LINEAR_PROFILE_PRECISION = 0, LINEAR_PROFILE_SPEED = 1 };
+enum linear_family_code {
+    LINEAR_FAMILY_EXPERT_GATE_UP = 0,
+    LINEAR_FAMILY_EXPERT_DOWN = 1,
+    LINEAR_FAMILY_TRUNK_QUANTIZED = 2,
+    LINEAR_FAMILY_TRUNK_BFLOAT16 = 3
+};
+/* the slice count of a product: 1 in the reference order; else gfx950's fixed counts (gate/up 4, down 2), never
+ * chosen by row count or timing */
+MUST_CHECK result_status linear_default_slice_count(enum linear_profile_code profile, enum linear_order_code order,
+                                                    enum linear_family_code family,
+                                                    const struct matrix_shape_record *shape,
+                                                    uint32_t arithmetic_class, uint32_t *slice_count_out);
+
+struct linear_quantize_description {
+    struct linear_range values;    /* read: bfloat16 [row_count][width] */
+    struct linear_range codes;     /* written: codes [row_count][width] */
+    struct linear_range exponents; /* written: exponents [row_count][width / 32] */
+    struct linear_range operands;  /* written: operands [row_count][width] */
+    uint32_t width;
+    uint32_t row_count;
+};
+MUST_CHECK result_status linear_quantize_prepare(const struct linear_quantize_description *description,
+                                                 uint64_t arena_byte_count,
+                                                 const struct linear_kernels_record *kernels,
+                                                 struct kernel_launch *launch_out);
+
+enum linear_routed_experts_launch {
+    LINEAR_ROUTED_EXPERTS_GATE_UP = 0,  /* expert_gate_up_<S>: jobs and the rows' arrays to hidden */
+    LINEAR_ROUTED_EXPERTS_QUANTIZE = 1, /* activation_quantize_entry: hidden of every pair to its arrays */
+    LINEAR_ROUTED_EXPERTS_DOWN = 2,     /* expert_down_<S>: jobs and the hidden arrays to pair_output */
+    LINEAR_ROUTED_EXPERTS_ROW_SUM = 3,  /* expert_row_sum_entry: pair_output to row_output */
+    LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT = 4
+};
+/* launches_out: LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT launches; weight_format E2M1_SCALED */
+MUST_CHECK result_status linear_routed_experts_prepare(const struct linear_routed_experts_description *description,
+                                                       uint64_t arena_byte_count,
+                                                       const struct linear_kernels_record *kernels,
+                                                       struct kernel_launch *launches_out);
+
+uint64_t linear_values_byte_count(uint64_t vector_count, uint64_t width);    /* bfloat16 [vector][width] */
+uint64_t linear_codes_byte_count(uint64_t vector_count, uint64_t width);     /* E4M3 [vector][width] */
+uint64_t linear_exponents_byte_count(uint64_t vector_count, uint64_t width); /* E8M0 [vector][width / 32] */
+uint64_t linear_sums_byte_count(uint64_t row_count, uint64_t width);         /* float32 [row][width] */
+uint64_t linear_jobs_byte_count(uint64_t job_count);                         /* struct expert_job_record */
+
 #ifdef __cplusplus
 }
 #endif

@@ -287,9 +287,15 @@ static double bf16_last_place(uint16_t bits)
 
 int orc_linear_within_tolerance(uint16_t output_bf16, double sum, double magnitude, uint32_t inputs, uint32_t slices)
 {
-    /* bound = (T + B + S) 2^-24 m + B 2^-149, T = 64; |c - y| <= last_place(c) / 2 + bound */
+    return orc_linear_within_allowance(output_bf16, sum, magnitude, inputs, slices, 64.0);
+}
+
+int orc_linear_within_allowance(uint16_t output_bf16, double sum, double magnitude, uint32_t inputs, uint32_t slices,
+                                double allowance)
+{
+    /* bound = (T + B + S) 2^-24 m + B 2^-149; |c - y| <= last_place(c) / 2 + bound */
     const double blocks = inputs / BLOCK;
-    const double bound = (64.0 + blocks + slices) * ldexp(1.0, -24) * magnitude + blocks * ldexp(1.0, -149);
+    const double bound = (allowance + blocks + slices) * ldexp(1.0, -24) * magnitude + blocks * ldexp(1.0, -149);
     const double c = (double)orc_bf16_to_float(output_bf16);
     if (c != c || sum != sum) {
         return c != c && sum != sum;

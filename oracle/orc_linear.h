@@ -56,6 +56,10 @@ int orc_linear_products(int format, uint32_t outputs, uint32_t inputs, const uin
                         double *sums_out, double *magnitude_out);
 /* the tolerance of a card's bf16 output against (sum, magnitude): |c - y| <= ulp_bf16(c)/2 + bound */
 int orc_linear_within_tolerance(uint16_t output_bf16, double sum, double magnitude, uint32_t inputs, uint32_t slices);
+/* the same with the allowance T for the rounding inside the matrix instructions given: the reference takes 64 for
+ * its cards' instructions of 16 products; a card whose instruction adds 128 scaled products has its own */
+int orc_linear_within_allowance(uint16_t output_bf16, double sum, double magnitude, uint32_t inputs, uint32_t slices,
+                                double allowance);
 
 /* hidden step in double (the definition) and in the kernels' float32 order with gate/up rounded to bf16 first */
 double orc_hidden_value(double gate, double up, double limit, double route_weight);

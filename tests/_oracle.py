@@ -69,6 +69,7 @@ def _load_oracle():
         "orc_operands_lay_out": (None, [u8p, u8p, u32, u16p]),
         "orc_linear_products": (i32, [i32, u32, u32, u8p, u32, u32, u8p, u8p, u32, f64p, f64p]),
         "orc_linear_within_tolerance": (i32, [C.c_uint16, C.c_double, C.c_double, u32, u32]),
+        "orc_linear_within_allowance": (i32, [C.c_uint16, C.c_double, C.c_double, u32, u32, C.c_double]),
         "orc_hidden_value": (C.c_double, [C.c_double] * 4),
         "orc_hidden_bits": (C.c_uint16, [f32] * 4),
         "orc_row_sum_bf16": (f32, [u16p, u32, u32, u32]),

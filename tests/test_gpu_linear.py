@@ -1,0 +1,189 @@
+"""GPU parity of the FP4 (E2M1 + E8M0 per 32) routed experts against the CPU oracle, through the C ABI: the activation
+quantizer byte for byte (codes in lane order, exponents, operands), the products within the reference's own bound
+(tests/linear_reference.h:43-58 of the reference: |c - y| <= ulp_bf16(c)/2 + (T + B + S) 2^-24 m + B 2^-149, T = 64),
+the hidden step, the row sum bit for bit, and whole layers.
+
+The allowance T for the rounding inside the matrix instructions is 64 in the reference (instructions of 16 products on
+its cards). gfx950's v_mfma_scale_f32_16x16x128_f8f6f4 adds 128 products of four scale blocks in one instruction and
+rounds inside it in a way no document defines; on outputs whose products cancel to a thousandth of their magnitudes
+the card was measured up to 1.5e2 x 2^-24 of the magnitude sum from the exact value, so T = 256 here."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+from _oracle import JOB_DTYPE, f32p, f64p, normals, orc, ptr, to_bf16, bf16_to_f32, u8p, u16p, u32p, u64p
+
+pytestmark = pytest.mark.gpu
+E2M1 = 3
+ALLOWANCE_GFX950 = 256.0
+
+
+def say(*words):
+    print(*words, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import anemone_amd
+    return anemone_amd
+
+
+@pytest.fixture(scope="module")
+def card(amd):
+    card = amd.Card(2 << 30)
+    yield card
+    card.close()
+
+
+@pytest.fixture(autouse=True)
+def fresh_arena(card):
+    card.cursor = 256
+    yield
+
+
+def build(amd, card, hidden, inner, experts_n, picks, rows, seed, **more):
+    from anemone_amd import workloads
+    matrices = [[workloads.fp4_matrix(seed * 1000 + 3 * e + 0, inner, hidden), workloads.fp4_matrix(seed * 1000 + 3 * e + 1, inner, hidden),
+                 workloads.fp4_matrix(seed * 1000 + 3 * e + 2, hidden, inner)] for e in range(experts_n)]
+    router = to_bf16(normals(seed + 5, experts_n * hidden) * 0.02).reshape(experts_n, hidden)
+    layer = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router, **more)
+    return layer, matrices, router
+
+
+def oracle_quantize(values):
+    rows, width = values.shape
+    codes = np.zeros((rows, width), dtype=np.uint8)
+    exps = np.zeros((rows, width // 32), dtype=np.uint8)
+    lane = np.zeros((rows, width), dtype=np.uint8)
+    operands = np.zeros((rows, width), dtype=np.uint16)
+    for r in range(rows):
+        assert orc.orc_act_quantize(ptr(values[r], u16p), width, ptr(codes[r], u8p), ptr(exps[r], u8p)) == 0
+        orc.orc_codes_lane_order(ptr(codes[r], u8p), width, ptr(lane[r], u8p))
+        orc.orc_operands_lay_out(ptr(codes[r], u8p), ptr(exps[r], u8p), width, ptr(operands[r], u16p))
+    return codes, exps, lane, operands
+
+
+def lane_to_value_order(lane_codes):
+    """Inverse of the lane order of a vector's codes."""
+    rows, width = lane_codes.shape
+    at = np.arange(width)
+    j, s, t, l = at % 4, (at // 4) % 4, (at // 16) % 4, at // 64
+    value = 64 * l + 16 * s + 2 * t + j // 2 + 8 * (j % 2)
+    out = np.zeros_like(lane_codes)
+    out[:, value] = lane_codes[:, at]
+    return out
+
+
+def test_quantizer_byte_for_byte(amd, card):
+    say("quantizer")
+    rows, width = 5, 1024
+    spread = np.repeat([1e-7, 1e-3, 0.2, 1.0, 30.0, 448.0, 5e3, 1e30], width // 8)
+    values = to_bf16(normals(3, rows * width).reshape(rows, width) * spread)
+    values[0, :32] = to_bf16(np.full(32, 448.0 * 2.0 ** -5))      # a block whose maximum is 448 x a power of two
+    values[1, 64:96] = 0                                            # an all-zero block: the floor 1e-4
+    values[2, 100] = 0x8000                                         # a negative zero keeps its sign
+    layer, _, _ = build(amd, card, width, 128, 64, 2, rows, 1)
+    layer.set_rows(values)
+    card.run(layer.quantize_launch())
+    codes, exps, lane, operands = oracle_quantize(values)
+    assert np.array_equal(layer.read("exponents").reshape(rows, -1), exps)
+    assert np.array_equal(layer.read("codes").reshape(rows, width), lane)
+    assert np.array_equal(layer.read("operands", np.uint16).reshape(rows, width), operands)
+
+
+@pytest.mark.parametrize("slices", [1, 2, 4, 8])
+def test_products_within_the_reference_bound(amd, card, slices):
+    """The down kernel is the plain product: each expert's gate matrix through it, against the exact block sums."""
+    say("products, slices", slices)
+    hidden, inner, experts_n, rows = 1024, 1024, 64, 6
+    layer, matrices, _ = build(amd, card, hidden, inner, experts_n, 1, rows, 2, gate_up_slices=1, down_slices=slices)
+    x = to_bf16(normals(7, rows * hidden).reshape(rows, hidden) * np.repeat([0.01, 1.0, 100.0, 1.0], hidden // 4))
+    codes, exps, lane, _ = oracle_quantize(x)
+    # pairs_per_row = 1: pair = row; three jobs over the first experts' GATE matrices (inner x hidden), as "down"
+    jobs = np.zeros(rows, dtype=JOB_DTYPE)
+    plan = [(0, [0, 1, 2]), (1, [3]), (2, [4, 5])]
+    for j, (expert, members) in enumerate(plan):
+        jobs[j]["down_offset"] = layer.expert_offsets[expert, 0]
+        jobs[j]["row_count"], jobs[j]["expert"] = len(members), expert
+        jobs[j]["pair_index"][:len(members)] = members
+    card.upload(layer.jobs_offset, jobs.view(np.uint8))
+    card.upload(layer.ranges["hidden_codes"].byte_offset, lane)
+    card.upload(layer.ranges["hidden_exponents"].byte_offset, exps)
+    launches = layer.expert_launches()
+    card.run(launches[2:3])
+    got = layer.read("pair_output", np.uint16).reshape(rows, hidden)
+    worst = 0.0
+    for expert, members in plan:
+        sums, mags = np.zeros((len(members), inner)), np.zeros((len(members), inner))
+        member_codes, member_exps = np.ascontiguousarray(codes[members]), np.ascontiguousarray(exps[members])
+        assert orc.orc_linear_products(E2M1, inner, hidden, ptr(matrices[expert][0], u8p), 0, inner, ptr(member_codes, u8p),
+                                       ptr(member_exps, u8p), len(members), ptr(sums, f64p), ptr(mags, f64p)) == 0
+        for i, row in enumerate(members):
+            for o in range(inner):
+                assert orc.orc_linear_within_allowance(int(got[row, o]), sums[i, o], mags[i, o], hidden, slices, ALLOWANCE_GFX950), (expert, row, o)
+            exact = to_bf16(sums[i].astype(np.float32))
+            worst = max(worst, float(np.mean(exact != got[row, :inner])))
+    say("  outputs that are not the exact sum rounded once: %.4f" % worst)
+    assert worst < 0.02
+
+
+@pytest.mark.parametrize("rows,live,picks", [(8, 8, 4), (3, 2, 8), (1, 1, 2)])
+def test_layer_against_oracle(amd, card, rows, live, picks):
+    say("layer", rows, live, picks)
+    hidden, inner, experts_n = 512, 256, 64
+    layer, matrices, router = build(amd, card, hidden, inner, experts_n, picks, rows, 4)
+    x = to_bf16(normals(9, rows * hidden)).reshape(rows, hidden)
+    layer.set_rows(x, live)
+    card.run(layer.projection_launch())
+    card.run(layer.select_launch(0))
+    card.run(layer.quantize_launch())
+    launches = layer.expert_launches()
+    card.run(launches)
+    jobs = layer.jobs()
+    # the oracle's routing (bit-exact with the card's, checked in test_gpu_exl3) rebuilt from the job table
+    experts = np.zeros((rows, picks), dtype=np.uint32)
+    weights = np.zeros((rows, picks), dtype=np.float32)
+    for job in jobs[jobs["row_count"] > 0]:
+        for c in range(job["row_count"]):
+            experts.reshape(-1)[job["pair_index"][c]] = job["expert"]
+            weights.reshape(-1)[job["pair_index"][c]] = job["route_weight"][c]
+    pointers = (C.c_void_p * (experts_n * 3))(*[m.ctypes.data for trio in matrices for m in trio])
+    want = np.zeros((live, hidden), dtype=np.float32)
+    want_hidden = np.zeros((live * picks, inner), dtype=np.uint16)
+    want_pairs = np.zeros((live * picks, hidden), dtype=np.uint16)
+    orc.orc_linear_moe_layer(E2M1, ptr(np.ascontiguousarray(x[:live]), u16p), live, hidden, inner, picks,
+                             ptr(np.ascontiguousarray(experts[:live]), u32p), ptr(np.ascontiguousarray(weights[:live]), f32p),
+                             experts_n, pointers, 10.0, ptr(want, f32p), ptr(want_hidden, u16p), ptr(want_pairs, u16p), 8)
+    live_pairs = live * picks
+    # hidden: the gate and up sums round to bfloat16 before the step; a flip of one last place there moves the
+    # hidden value by about 2^-7 of it
+    got_hidden = bf16_to_f32(layer.read("hidden", np.uint16).reshape(-1, inner)[:live_pairs]).astype(np.float64)
+    ref_hidden = bf16_to_f32(want_hidden).astype(np.float64)
+    assert np.all(np.abs(got_hidden - ref_hidden) <= 2.0 ** -6 * np.abs(ref_hidden) + 1e-6)
+    say("  hidden values equal to the oracle's: %.4f" % float(np.mean(got_hidden == ref_hidden)))
+    # down: exactly checked against the card's own hidden codes
+    hidden_lane = layer.read("hidden_codes").reshape(-1, inner)[:live_pairs]
+    hidden_exps = np.ascontiguousarray(layer.read("hidden_exponents").reshape(-1, inner // 32)[:live_pairs])
+    hidden_bits = np.ascontiguousarray(layer.read("hidden", np.uint16).reshape(-1, inner)[:live_pairs])
+    codes, exps, lane, _ = oracle_quantize(hidden_bits)
+    assert np.array_equal(lane, hidden_lane) and np.array_equal(exps, hidden_exps)
+    pair_out = layer.read("pair_output", np.uint16).reshape(-1, hidden)[:live_pairs]
+    for pair in range(0, live_pairs, max(1, live_pairs // 6)):
+        e = int(experts.reshape(-1)[pair])
+        sums, mags = np.zeros(hidden), np.zeros(hidden)
+        orc.orc_linear_products(E2M1, hidden, inner, ptr(matrices[e][2], u8p), 0, hidden, ptr(np.ascontiguousarray(codes[pair]), u8p),
+                                ptr(np.ascontiguousarray(exps[pair]), u8p), 1, ptr(sums, f64p), ptr(mags, f64p))
+        assert all(orc.orc_linear_within_allowance(int(pair_out[pair, o]), sums[o], mags[o], inner, 2, ALLOWANCE_GFX950) for o in range(hidden))
+    # row sum: bit for bit from the card's pair outputs
+    got = layer.read("row_output", np.float32).reshape(rows, hidden)[:live]
+    for r in range(live):
+        rows_pairs = np.ascontiguousarray(pair_out[r * picks:(r + 1) * picks])
+        for column in range(0, hidden, 37):
+            assert got[r, column] == orc.orc_row_sum_bf16(ptr(rows_pairs, u16p), picks, hidden, column)
+    # and the whole layer against the oracle's
+    error = np.sqrt(np.mean((got - want) ** 2) / np.mean(want.astype(np.float64) ** 2))
+    say("  layer rms error vs oracle: %.2e" % error)
+    assert error < 2e-2
