@@ -204,10 +204,21 @@ exl3_wave_product(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32
     const uint32_t *source = codes + (uint64_t)first_tile * row_stride + (uint64_t)strip_tile * W::tile_words +
                              lane * 4u;
     const bool carries = lane < row_lanes;
+    /* the operand's eight inputs of this lane in a step: 16 tau + 4 q + {0..3} and + {8..11}. They are asked for a
+     * step ahead with the weights: loads return in order, so an operand asked for inside the step that uses it would
+     * make that step wait for the weights prefetched just before it */
+    const half_t *x = operand == nullptr ? nullptr : operand + (first_tile * 16u + 16u * tau + 4u * q);
     uint4_t next0 = {0, 0, 0, 0}, next1 = {0, 0, 0, 0};
-    if (carries && first_tile < last_tile) {
-        next0 = *(const uint4_t *)source;
-        next1 = *(const uint4_t *)(source + row_stride);
+    uint2_t next_low = {0, 0}, next_high = {0, 0};
+    if (first_tile < last_tile) {
+        if (carries) {
+            next0 = *(const uint4_t *)source;
+            next1 = *(const uint4_t *)(source + row_stride);
+        }
+        if (x != nullptr) {
+            next_low = *(const uint2_t *)x;
+            next_high = *(const uint2_t *)(x + 8);
+        }
     }
 #pragma unroll
     for (uint32_t n = 0; n < NT; n++) {
@@ -215,17 +226,18 @@ exl3_wave_product(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32
     }
     for (uint32_t tile = first_tile; tile < last_tile; tile += 2u) {
         const uint4_t row0 = next0, row1 = next1;
+        const uint2_t b_low = next_low, b_high = next_high;
         source += 2u * row_stride;
-        if (carries && tile + 2u < last_tile) {
-            next0 = *(const uint4_t *)source;
-            next1 = *(const uint4_t *)(source + row_stride);
-        }
-        /* the operand's eight inputs of this lane: 16 tau + 4 q + {0..3} and + {8..11} */
-        uint2_t b_low = {0, 0}, b_high = {0, 0};
-        if (operand != nullptr) {
-            const half_t *x = operand + (tile * 16u + 16u * tau + 4u * q);
-            b_low = *(const uint2_t *)x;
-            b_high = *(const uint2_t *)(x + 8);
+        if (tile + 2u < last_tile) {
+            if (carries) {
+                next0 = *(const uint4_t *)source;
+                next1 = *(const uint4_t *)(source + row_stride);
+            }
+            if (x != nullptr) {
+                x += 32;
+                next_low = *(const uint2_t *)x;
+                next_high = *(const uint2_t *)(x + 8);
+            }
         }
         if (carries) {
             *(uint4_t *)(lds + lane * 4u) = row0;

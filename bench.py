@@ -71,12 +71,100 @@ def calibrate(amd):
                       "GBps_read_plus_write": 2 * size / (min(times) * 1e-6) / 1e9}))
 
 
+def fp4_decode(amd, workloads, arguments):
+    """Secondary workload: the same layer shape with the original FP4 weights (E2M1 codes, one E8M0 scale per 32
+    inputs), a decode step of `--rows` tokens (32 by default): quantizer, router, and the four launches of the routed
+    experts. Sixteen distinct seeded experts are generated and laid at 256 distinct places of the arena."""
+    import ctypes as C
+    rows = arguments.rows
+    distinct_generated = 16
+    base = workloads.SEED + (4 << 20)
+    trios = [[workloads.fp4_matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), workloads.fp4_matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
+              workloads.fp4_matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
+    matrices = [trios[e % distinct_generated] for e in range(EXPERTS)]
+    router = workloads.to_bf16(workloads.normals(base + 2, EXPERTS * HIDDEN) * 0.02).reshape(EXPERTS, HIDDEN)
+    x = workloads.activations(4, rows, HIDDEN)
+    card = amd.Card(5 << 30)
+    layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router,
+                         gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices)
+    layer.set_rows(x, rows)
+    step = amd.launches_of(7)
+    step[0] = layer.projection_launch()[0]
+    step[1] = layer.select_launch(0)[0]
+    step[2] = layer.quantize_launch()[0]
+    experts = layer.expert_launches()
+    for i in range(4):
+        step[3 + i] = experts[i]
+    names = ["router_projection", "router_select_entry", "activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
+             "expert_down", "expert_row_sum_entry"]
+    for _ in range(arguments.warmup):
+        card.run(step, wait=False)
+    card.wait()
+    device_us = card.measure(lambda: [card.run(step, wait=False) for _ in range(arguments.steps)])
+    seconds = device_us * 1e-6
+    per_launch = np.zeros(len(names))
+    for _ in range(arguments.steps):
+        per_launch += np.array(card.run_timed(step))
+    per_launch /= arguments.steps
+    jobs = layer.jobs()
+    live = jobs[jobs["row_count"] > 0]
+    distinct = np.unique(live["expert"])
+    matrix_bytes = HIDDEN * INNER // 2 + HIDDEN * INNER // 32
+    gate_up_bytes = 2 * matrix_bytes * len(distinct)
+    gate_up_us = float(per_launch[3])
+    down_us = float(per_launch[5])
+    result = {
+        "metric": "MoE layer tok/s; decode HBM GB/s & prefill MFMA % of peak, 1 GPU",
+        "value": rows * arguments.steps / seconds, "unit": "tok/s", "n_gpus": 1, "steps": arguments.steps,
+        "warmup": arguments.warmup, "ms_per_step": 1000.0 * seconds / arguments.steps, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp4 x fp8 -> f32", "data": "synthetic",
+        "config": {"workload": "fp4_moe_decode: %d tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router, "
+                               "E2M1 weights with E8M0 scales per 32" % rows,
+                   "distinct_experts": int(len(distinct)), "jobs": int(len(live)),
+                   "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
+                   "down_GBps": matrix_bytes * len(distinct) / (down_us * 1e-6) / 1e9},
+        "roofline": {"bound": "hbm", "kernel": "expert_gate_up_%d" % arguments.gate_up_slices,
+                     "achieved": gate_up_bytes / (gate_up_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
+    }
+    if not arguments.no_cpu:
+        import _oracle as o
+        threads = min(os.cpu_count() or 1, 16)
+        sample = min(rows, 4)
+        experts_of = np.zeros((rows, PICKS), dtype=np.uint32)
+        weights_of = np.zeros((rows, PICKS), dtype=np.float32)
+        for job in live:
+            for c in range(job["row_count"]):
+                experts_of.reshape(-1)[job["pair_index"][c]] = job["expert"]
+                weights_of.reshape(-1)[job["pair_index"][c]] = job["route_weight"][c]
+        pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
+        want = np.zeros((sample, HIDDEN), dtype=np.float32)
+        start = time.perf_counter()
+        o.orc.orc_linear_moe_layer(3, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS,
+                                   o.ptr(np.ascontiguousarray(experts_of[:sample]), o.u32p),
+                                   o.ptr(np.ascontiguousarray(weights_of[:sample]), o.f32p), EXPERTS, pointers, 10.0,
+                                   o.ptr(want, o.f32p), None, None, threads)
+        cpu_seconds = time.perf_counter() - start
+        got = layer.read("row_output", np.float32).reshape(rows, HIDDEN)[:sample]
+        error = float(np.sqrt(np.mean((got - want) ** 2) / np.mean(want.astype(np.float64) ** 2)))
+        assert error < 2e-2, "GPU output differs from the oracle's: rms %g" % error
+        result["cpu_baseline"] = {"value": sample / cpu_seconds, "unit": "tok/s", "cores": threads, "kind": "port",
+                                  "sample": "the first %d tokens of the same step by the CPU oracle" % sample,
+                                  "seconds": cpu_seconds, "gpu_vs_oracle_rms_err": error}
+    card.close()
+    print(json.dumps(result))
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=200)
     parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--workload", default="exl3_decode")
+    parser.add_argument("--rows", type=int, default=32, help="tokens of a step (fp4_decode)")
+    parser.add_argument("--gate-up-slices", type=int, default=4)
+    parser.add_argument("--down-slices", type=int, default=2)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--calibrate", action="store_true",
                         help="run only a 1 GiB arena copy, five times: the yardstick of the traffic counters")
@@ -84,7 +172,7 @@ def main():
     if arguments.gpus != 1:
         print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
         sys.exit(2)
-    if arguments.workload != "exl3_decode":
+    if arguments.workload not in ("exl3_decode", "fp4_decode"):
         print("unknown workload %s" % arguments.workload, file=sys.stderr)
         sys.exit(2)
 
@@ -93,6 +181,9 @@ def main():
 
     if arguments.calibrate:
         calibrate(amd)
+        return
+    if arguments.workload == "fp4_decode":
+        fp4_decode(amd, workloads, arguments)
         return
 
     widths, matrices, router = workloads.exl3_moe_layer(CONFIG, HIDDEN, INNER, EXPERTS)
