@@ -13,12 +13,20 @@
  * one v_mfma_scale_f32_16x16x128_f8f6f4 takes 128 inputs = four blocks of 32 with both E8M0 scale codes inside the
  * instruction and adds their terms to the running chain; E2M1 weights by E4M3 vector codes, no conversion.
  *
- * Work mapping (this build's own). A block is one tile of 16 outputs of one job; a wavefront is one slice of one
- * matrix. The 1,024 bytes of a tile's two consecutive loads are one 16-byte-per-lane load from memory straight into
- * a wavefront-private LDS window, whence they reach the MFMA's lanes: lane (o, g) needs output row o of inputs block g,
- * which the stored form spreads over four stored lanes (t = 0..3) as the even (o < 8) or odd (o >= 8) nibbles of two
- * words each. Compaction of eight nibbles into a register is two shifts, two ands and an or. The vector's codes are
- * brought into the same input order with two byte permutes a register.
+ * Work mapping (this build's own). What bounds a streaming kernel on this card, besides memory itself, is the number
+ * of memory instructions: a compute unit takes one wavefront-wide load every 16 cycles whatever its width, which at
+ * full memory speed leaves room for about six a KB of weights, and in practice far fewer. So:
+ *   - a block is one strip of STRIP tiles (64 outputs) of one job; a wavefront is one slice of the inputs, for the
+ *     gate AND the up matrix (their sums meet in one lane for the hidden step, no exchange);
+ *   - a stage is one K step (128 inputs) of all the wavefront's tiles: 1,024 bytes a tile go from memory straight
+ *     into the wavefront's LDS window with one 16-byte-a-lane load (no registers in between), the tiles' 64 scale
+ *     bytes each with one more load for every four tiles; two or three stages are on their way while one is used;
+ *   - the codes of the job's (at most eight) vectors for the step and their scale codes travel the same way, one load
+ *     each a stage, and serve every tile of the wavefront; nothing of the loop passes through registers, so the
+ *     compiler has no wait of its own to place and the waits are this file's constants;
+ *   - lane (o, g) of the MFMA needs output row o of inputs block g, which the stored form spreads over four stored
+ *     lanes (t = 0..3) as the even (o < 8) or odd (o >= 8) nibbles of two words each: four 8-byte LDS reads, and two
+ *     shifts, a shift and a bit-field insert a register.
  *
  * MFMA operand layout on gfx950, as measured on the card: A (fp4) lane l: row l % 16, element e = 8 v + n (register v,
  * nibble n) is k = 32 (l / 16) + e; B (fp8) lane l: column l % 16, element e = 4 v + b is k = 64 (e / 16) +
@@ -30,32 +38,36 @@
 
 typedef int int8_vector __attribute__((ext_vector_type(8)));
 
-#define TILE_LOAD_BYTES 512u     /* 16 outputs x 64 inputs x 4 bits */
+#define TILE_LOAD_BYTES 512u /* 16 outputs x 64 inputs x 4 bits */
 #define STEP_BYTES (2u * TILE_LOAD_BYTES)
-#define DEPTH 8u                 /* K steps in flight a wavefront */
-#define STAGE_WORDS (STEP_BYTES / 4u)
-#define WINDOW_WORDS (DEPTH * STAGE_WORDS) /* a wavefront's LDS window: DEPTH stages of one step's weights */
-#define STAGE_LOADS 7u           /* memory loads a stage issues: scale, four vector pieces, vector scale, weights */
+#define STRIP 4u             /* tiles of a strip */
 #define NIBBLE_MASK 0x0F0F0F0Fu
 
-typedef const __attribute__((address_space(1))) void *global_pointer;
 typedef __attribute__((address_space(3))) void *lds_pointer;
 
-/* 16 bytes a lane from memory straight into LDS: lane L's bytes land at `stage` + 16 L (the base travels in M0).
- * Written as assembly so that the compiler keeps no book on it: it would otherwise guard every LDS read that might
- * alias with a wait for all loads. The waits are this file's own (wait_loads). A fence for the compiler as well, so
- * the stages' loads keep their order, which the waits count on. */
-__device__ static __forceinline__ void load_to_lds(const unsigned char *source, uint32_t *stage)
+/* Memory straight into LDS, 16 or 4 bytes a lane: lane L's bytes land at lds_base + 16 L (4 L); the address is a
+ * base common to the wavefront plus the lane's own byte offset. Written as assembly so that the compiler keeps no
+ * book on these loads: it would guard every LDS read that might alias one with a wait for all of them. The waits
+ * are this file's own (wait_loads). A fence for the compiler as well, so the loads keep their order, which the waits
+ * count on. */
+__device__ static __forceinline__ void load_to_lds_16(const unsigned char *base, uint32_t lane_offset, uint32_t lds_base)
 {
-    const uint32_t base = (uint32_t)(uintptr_t)(lds_pointer)stage;
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(source), "s"(base)
+                 : "v"(lane_offset), "s"(base), "s"(lds_base)
+                 : "memory", "m0");
+}
+
+__device__ static __forceinline__ void load_to_lds_4(const unsigned char *base, uint32_t lane_offset, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(base), "s"(lds_base)
                  : "memory", "m0");
 }
 
 /* wait until at most `count` of the wavefront's memory loads are outstanding (they retire in order); also a fence
- * for the compiler: LDS reads of a stage stay behind the wait for the load that fills it */
+ * for the compiler: LDS reads of a stage stay behind the wait for the loads that fill it */
 template <uint32_t count>
 __device__ static __forceinline__ void wait_loads()
 {
@@ -63,172 +75,252 @@ __device__ static __forceinline__ void wait_loads()
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(count) : "memory");
 }
 
-/* What a lane keeps through a chain: where its loads start and where it reads its operands in a stage. */
-struct chain_lane {
-    const unsigned char *words;        /* this lane's 16-byte piece of the chain's first step */
-    const unsigned char *scales;       /* its weight scale byte of the first step */
-    const unsigned char *vector;       /* its 8-byte pieces of the vector's codes, first step */
-    const unsigned char *vector_scale; /* its vector scale byte, first step */
-    uint32_t *lds;                     /* the wavefront's window */
-    uint32_t read_at[4];               /* word offsets of its pieces T = 0..3 inside a stage */
-    uint32_t shift;                    /* 0: the even nibbles (outputs 0..7 of the tile), 4: the odd ones */
+/* A wavefront's part of a strip: MATRICES matrices (gate and up, or down alone) x STRIP tiles, K steps [first, last).
+ * LDS window of a wavefront: DEPTH stages; a stage: MATRICES x STRIP x 1,024 bytes of weights, MATRICES x 256 bytes
+ * of their scales (a matrix's STRIP tiles x 64), 1,024 bytes of the vectors' codes (8 columns x 128) and 256 bytes
+ * holding their scale words. */
+template <uint32_t MATRICES>
+struct strip_chain {
+    static constexpr uint32_t TILES = MATRICES * STRIP;
+    static constexpr uint32_t DEPTH = MATRICES == 2u ? 2u : 3u;
+    static constexpr uint32_t SCALES_AT = TILES * STEP_BYTES;
+    static constexpr uint32_t VECTOR_AT = SCALES_AT + MATRICES * 256u;
+    static constexpr uint32_t VECTOR_SCALE_AT = VECTOR_AT + 1024u;
+    static constexpr uint32_t STAGE_BYTES = VECTOR_SCALE_AT + 256u;
+    static constexpr uint32_t WINDOW_BYTES = DEPTH * STAGE_BYTES;
+    static constexpr uint32_t STAGE_LOADS = TILES + MATRICES + 2u;
+    static_assert(STAGE_LOADS * (DEPTH - 1u) < 64u, "vmcnt has six bits");
+
+    const unsigned char *words[MATRICES];  /* the strip's first tile, the chain's first step, of each matrix */
+    const unsigned char *scales[MATRICES]; /* the same of the scale words */
+    const unsigned char *codes;            /* the vectors' codes at the chain's first step (row 0) */
+    const unsigned char *exponents;        /* the vectors' scale codes at the chain's first step (row 0) */
+    uint32_t tile_bytes;                    /* from a tile to the next */
+    uint32_t window;                        /* LDS address of the wavefront's window */
+    uint32_t piece_offset;                  /* this lane's 16-byte piece of a step of a tile */
+    uint32_t scale_offset;                  /* this lane's scale word of a stage: tile lane / 16, word lane % 16 */
+    uint32_t codes_offset;                  /* this lane's 16-byte piece of the vectors' codes of a step */
+    uint32_t exponents_offset;              /* this lane's vector's scale word of a step */
+    uint32_t read_at[4];                    /* LDS byte offsets of its pieces T = 0..3 inside a tile of a stage */
+    uint32_t scale_at;                      /* LDS byte offset of its scale byte inside a matrix's scales of a stage */
+    uint32_t vector_at[4];                  /* LDS byte offsets of its four 8-byte pieces of its vector */
+    uint32_t vector_scale_at;               /* LDS byte offset of its vector's scale byte */
+    uint32_t shift;                         /* 0: the even nibbles (outputs 0..7 of a tile), 4: the odd ones */
+
+    __device__ __forceinline__ void issue(uint32_t stage, uint32_t at) const
+    {
+        const uint32_t base = window + stage * STAGE_BYTES;
+#pragma unroll
+        for (uint32_t m = 0; m < MATRICES; m++) {
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+                load_to_lds_16(words[m] + (uint64_t)n * tile_bytes + (uint64_t)at * STEP_BYTES, piece_offset,
+                               base + (m * STRIP + n) * STEP_BYTES);
+            }
+        }
+#pragma unroll
+        for (uint32_t m = 0; m < MATRICES; m++) {
+            load_to_lds_4(scales[m] + (uint64_t)at * 64u, scale_offset, base + SCALES_AT + m * 256u);
+        }
+        load_to_lds_16(codes + (uint64_t)at * 128u, codes_offset, base + VECTOR_AT);
+        load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT);
+    }
+
+    template <typename T>
+    __device__ static __forceinline__ T lds_read(uint32_t address)
+    {
+        return *(const __attribute__((address_space(3))) T *)(uintptr_t)address;
+    }
+
+    __device__ __forceinline__ void consume(uint32_t stage, float4_t (&chain)[TILES]) const
+    {
+        const uint32_t base = window + stage * STAGE_BYTES;
+        int8_vector b;
+#pragma unroll
+        for (uint32_t part = 0; part < 4u; part++) {
+            const uint2_t pair = lds_read<uint2_t>(base + VECTOR_AT + vector_at[part]);
+            b[2u * part] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x05010400u);
+            b[2u * part + 1u] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x07030602u);
+        }
+        const uint32_t scale_b = lds_read<unsigned char>(base + VECTOR_SCALE_AT + vector_scale_at);
+#pragma unroll
+        for (uint32_t tile = 0; tile < TILES; tile++) {
+            int8_vector a = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (uint32_t T = 0; T < 4u; T++) {
+                const uint2_t w = lds_read<uint2_t>(base + tile * STEP_BYTES + read_at[T]);
+                a[T] = (int)(((w.x >> shift) & NIBBLE_MASK) | (((w.y >> shift) & NIBBLE_MASK) << 4));
+            }
+            const uint32_t scale_a = lds_read<unsigned char>(base + SCALES_AT + (tile / STRIP) * 256u + (tile % STRIP) * 64u + scale_at);
+            chain[tile] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[tile], 4, 0, 0, (int)scale_a, 0, (int)scale_b);
+        }
+        /* the stage is read once its values are in registers; only then may it be filled again */
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+
+    /* The whole chain of `total` steps (the same in every lane). The window is idle on entry and on return. */
+    __device__ __forceinline__ void whole(uint32_t total, float4_t (&chain)[TILES]) const
+    {
+        uint32_t done = 0;
+        if (total >= 2u * DEPTH) {
+#pragma unroll
+            for (uint32_t i = 0; i < DEPTH; i++) {
+                issue(i, i);
+            }
+            /* the steady state: a step consumed has DEPTH - 1 whole stages asked for behind it, and asks for one more */
+            for (; done + 2u * DEPTH <= total; done += DEPTH) {
+#pragma unroll
+                for (uint32_t i = 0; i < DEPTH; i++) {
+                    wait_loads<STAGE_LOADS * (DEPTH - 1u)>();
+                    consume(i, chain);
+                    issue(i, done + i + DEPTH);
+                }
+            }
+        } else {
+#pragma unroll
+            for (uint32_t i = 0; i < DEPTH; i++) {
+                if (i < total) {
+                    issue(i, i);
+                }
+            }
+        }
+        /* the last steps, fewer than 2 DEPTH: the stages behind a step grow fewer */
+#pragma unroll
+        for (uint32_t round = 0; round < 2u; round++) {
+#pragma unroll
+            for (uint32_t i = 0; i < DEPTH; i++) {
+                const uint32_t at = done + round * DEPTH + i;
+                if (at < total) {
+                    const uint32_t behind = total - 1u - at;
+                    if (behind >= DEPTH - 1u) {
+                        wait_loads<STAGE_LOADS * (DEPTH - 1u)>();
+                    } else if (behind == 1u) {
+                        wait_loads<STAGE_LOADS>();
+                    } else {
+                        wait_loads<0>();
+                    }
+                    consume(i, chain);
+                    if (at + DEPTH < total) {
+                        issue(i, at + DEPTH);
+                    }
+                }
+            }
+        }
+    }
+
+    /* matrices: arena addresses of the MATRICES stored matrices; strip: the strip of tiles; first: the chain's first K
+     * step; vector_codes / vector_exponents: row 0 of the vectors' codes and scale codes; vector_rows: the rows of
+     * columns 0..7 (columns 8..15 never hold a row of a job: they mirror columns 0..7 and are not stored) */
+    __device__ __forceinline__ void place(const unsigned char *const (&matrices)[MATRICES], uint32_t outputs, uint32_t inputs,
+                                          uint32_t strip, uint32_t first, const unsigned char *vector_codes,
+                                          const unsigned char *vector_exponents, const uint32_t (&vector_rows)[8],
+                                          uint32_t window_address, uint32_t lane)
+    {
+        static_assert(DEPTH == 2u || DEPTH == 3u, "the waits of whole() are written out for two or three stages");
+        const uint32_t loads = inputs / 64u, tiles = outputs / 16u;
+        const uint32_t o = lane % 16u, g = lane / 16u, G = o % 8u, parity = o / 8u, ld = g / 2u, q = g % 2u;
+        /* a strip that reaches past the last tile reads the last tiles again; its surplus sums are not stored */
+        const uint32_t tile0 = strip * STRIP + STRIP <= tiles ? strip * STRIP : tiles - STRIP;
+        tile_bytes = loads * TILE_LOAD_BYTES;
+#pragma unroll
+        for (uint32_t m = 0; m < MATRICES; m++) {
+            words[m] = matrices[m] + ((uint64_t)tile0 * loads + 2u * first) * TILE_LOAD_BYTES;
+            scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + ((uint64_t)tile0 * loads + 2u * first) * 32u;
+        }
+        codes = vector_codes + 128u * first;
+        exponents = vector_exponents + 4u * first;
+        window = window_address;
+        /* lane L of a 16-byte load lands at bytes 16 L of the tile's stage and asks for the piece
+         * p = L ^ (2 bit4(L) + bit5(L)) of the step: the pieces of one T (p = 32 ld + 4 G + T) then lie in different
+         * LDS banks for the readers, and every 16 lanes still read 256 contiguous bytes of memory */
+        piece_offset = 16u * (lane ^ (2u * ((lane >> 4) & 1u) + ((lane >> 5) & 1u)));
+        /* scales: uint32 [tile][load][G]; lane L of the 4-byte load: tile L / 16, word L % 16 = 8 ld + G of the step */
+        scale_offset = (lane / 16u) * (loads * 32u) + (lane % 16u) * 4u;
+        /* the vectors: lane L of the 16-byte load holds slot L % 8 of column L / 8 and asks for that column's piece
+         * (L % 8) ^ (L / 8) of the step, so that one piece of all columns lies in different banks; lane L of the
+         * 4-byte load of their scale words serves column L % 8 (the readers take the copies of lanes 0..7) */
+        uint32_t row_of_codes = 0, row_of_exponents = 0;
+#pragma unroll
+        for (uint32_t c = 0; c < 8u; c++) {
+            row_of_codes = lane / 8u == c ? vector_rows[c] : row_of_codes;
+            row_of_exponents = lane % 8u == c ? vector_rows[c] : row_of_exponents;
+        }
+        codes_offset = row_of_codes * inputs + 16u * ((lane % 8u) ^ (lane / 8u));
+        exponents_offset = row_of_exponents * (inputs / 32u);
+#pragma unroll
+        for (uint32_t T = 0; T < 4u; T++) {
+            read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (2u * (G / 4u) + ld))) + 8u * q;
+        }
+        scale_at = (8u * ld + G) * 4u + 2u * q + parity;
+        /* the lane's vector pieces: piece 4 (part / 2) + part % 2 + 2 (g % 2) of its column, bytes 8 (g / 2) .. + 7 */
+        const uint32_t column = o % 8u;
+#pragma unroll
+        for (uint32_t part = 0; part < 4u; part++) {
+            const uint32_t piece = 4u * (part / 2u) + part % 2u + 2u * (g % 2u);
+            vector_at[part] = 16u * (8u * column + (piece ^ column)) + 8u * (g / 2u);
+        }
+        vector_scale_at = 4u * column + g;
+        shift = 4u * parity;
+    }
 };
 
-struct chain_stage { /* what a stage keeps in registers while its weights are on their way into LDS */
-    uint2_t vector[4];
-    uint32_t scale, vector_scale;
-};
-
-__device__ static __forceinline__ void stage_issue(const chain_lane &lane, uint32_t stage, uint32_t at, chain_stage &kept)
-{
-    kept.scale = lane.scales[(uint64_t)at * 64u];
-#pragma unroll
-    for (uint32_t part = 0; part < 4u; part++) {
-        kept.vector[part] = *(const uint2_t *)(lane.vector + (uint64_t)at * 128u + 64u * (part / 2u) + 16u * (part % 2u));
-    }
-    kept.vector_scale = lane.vector_scale[(uint64_t)at * 4u];
-    load_to_lds(lane.words + (uint64_t)at * STEP_BYTES, lane.lds + stage * STAGE_WORDS); /* the last of STAGE_LOADS */
-}
-
-__device__ static __forceinline__ float4_t stage_consume(const chain_lane &lane, uint32_t stage, chain_stage kept, float4_t chain)
-{
-    /* the stage's registers are first touched here, behind the wait: their uses may not drift to where an earlier
-     * wait would have to cover them */
-    asm volatile("" : "+v"(kept.scale), "+v"(kept.vector_scale));
-    int8_vector b;
-#pragma unroll
-    for (uint32_t part = 0; part < 4u; part++) {
-        uint2_t pair = kept.vector[part];
-        asm volatile("" : "+v"(pair.x), "+v"(pair.y));
-        b[2u * part] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x05010400u);
-        b[2u * part + 1u] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x07030602u);
-    }
-    int8_vector a = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-    for (uint32_t T = 0; T < 4u; T++) {
-        const uint2_t w = *(const uint2_t *)(lane.lds + stage * STAGE_WORDS + lane.read_at[T]);
-        a[T] = (int)(((w.x >> lane.shift) & NIBBLE_MASK) | (((w.y >> lane.shift) & NIBBLE_MASK) << 4));
-    }
-    /* the stage is read once its values are in registers; only then may it be filled again */
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain, 4, 0, 0, (int)kept.scale, 0, (int)kept.vector_scale);
-}
-
-/* N steps from `at` on, N known to the compiler (at most 2 DEPTH): straight-line code, so that every wait is a
- * constant: before step s, the stages asked for behind it number min(N, s + DEPTH) - 1 - s. The window must be idle
- * on entry (nothing of this wavefront on its way), and is idle again on return. */
-template <uint32_t N>
-__device__ static __forceinline__ float4_t chain_run(const chain_lane &lane, uint32_t at, float4_t chain)
-{
-    static_assert(N >= 1u && N <= 2u * DEPTH, "one or two rounds of the window");
-    chain_stage kept[DEPTH];
-#pragma unroll
-    for (uint32_t s = 0; s < (N < DEPTH ? N : DEPTH); s++) {
-        stage_issue(lane, s, at + s, kept[s]);
-    }
-#pragma unroll
-    for (uint32_t s = 0; s < N; s++) {
-        constexpr uint32_t none = 0;
-        const uint32_t asked = (s + DEPTH < N ? s + DEPTH : N) - 1u - s; /* folds: s is an unrolled constant */
-        switch (asked) {
-        case 7: wait_loads<STAGE_LOADS * 7u>(); break;
-        case 6: wait_loads<STAGE_LOADS * 6u>(); break;
-        case 5: wait_loads<STAGE_LOADS * 5u>(); break;
-        case 4: wait_loads<STAGE_LOADS * 4u>(); break;
-        case 3: wait_loads<STAGE_LOADS * 3u>(); break;
-        case 2: wait_loads<STAGE_LOADS * 2u>(); break;
-        case 1: wait_loads<STAGE_LOADS * 1u>(); break;
-        default: wait_loads<none>(); break;
-        }
-        chain = stage_consume(lane, s % DEPTH, kept[s % DEPTH], chain);
-        if (s + DEPTH < N) {
-            stage_issue(lane, s % DEPTH, at + s + DEPTH, kept[s % DEPTH]);
-        }
-    }
-    return chain;
-}
-
-/* One wavefront: the chain of K steps [first, last) of one tile of one matrix against up to 16 vector columns.
- *
- * The 1,024 bytes of a step go from memory straight into a stage of the wavefront's LDS window (no registers in
- * between), up to DEPTH stages ahead, so that a wavefront keeps DEPTH KB on their way. Lane L of the load lands at
- * bytes 16 L of the stage, and asks for the 16-byte piece p = L ^ (2 bit4(L) + bit5(L)) of the step: the pieces of
- * one T (p = 32 ld + 4 G + T) then lie in different LDS banks for the readers, and every 16 lanes still read 256
- * contiguous bytes of memory. The vector's codes and both scale codes of a stage are asked for together with its
- * weights and wait in registers: loads retire in order, so anything asked for later than the weights of a far stage
- * would have to wait for them. Columns without a row read the vector of row 0; their sums are never stored. */
-__device__ static __forceinline__ float4_t
-expert_chain(const unsigned char *matrix, uint32_t outputs, uint32_t inputs, uint32_t tile, uint32_t first,
-             uint32_t last, const unsigned char *codes, const unsigned char *exponents, uint32_t *lds, uint32_t lane_index)
-{
-    static_assert(DEPTH == 8u, "the waits of chain_run are written out for eight stages");
-    const uint32_t loads = inputs / 64u;
-    const uint32_t o = lane_index % 16u, g = lane_index / 16u, G = o % 8u, parity = o / 8u, ld = g / 2u, q = g % 2u;
-    const uint32_t piece = lane_index ^ (2u * ((lane_index >> 4) & 1u) + ((lane_index >> 5) & 1u));
-    chain_lane lane;
-    lane.words = matrix + ((uint64_t)tile * loads + 2u * first) * TILE_LOAD_BYTES + piece * 16u;
-    /* scales: uint32 [tile][load][G], byte 2 q + parity */
-    lane.scales = matrix + (uint64_t)outputs * inputs / 2u + (((uint64_t)tile * loads + 2u * first + ld) * 8u + G) * 4u + 2u * q + parity;
-    /* the vector: bytes 64 load + 16 T + 8 q .. + 7 for T = 2 (g % 2), 2 (g % 2) + 1 of both loads of the step */
-    lane.vector = codes + 128u * first + 32u * (g % 2u) + 8u * (g / 2u);
-    lane.vector_scale = exponents + 4u * first + g;
-    lane.lds = lds;
-    /* where this lane reads its piece T of a stage: slot 32 ld + 4 G + (T ^ (2 (G / 4) + ld)), half q */
-#pragma unroll
-    for (uint32_t T = 0; T < 4u; T++) {
-        lane.read_at[T] = (16u * (32u * ld + 4u * G + (T ^ (2u * (G / 4u) + ld))) + 8u * q) / 4u;
-    }
-    lane.shift = 4u * parity;
-    const uint32_t total = last - first; /* the same in every lane */
-    float4_t chain = {0.0f, 0.0f, 0.0f, 0.0f};
-    uint32_t at = 0;
-    for (; at + 2u * DEPTH <= total; at += 2u * DEPTH) {
-        chain = chain_run<2u * DEPTH>(lane, at, chain);
-    }
-    switch (total - at) {
-#define CHAIN_REST(n)                                                                                               \
-    case n: chain = chain_run<n>(lane, at, chain); break
-        CHAIN_REST(1); CHAIN_REST(2); CHAIN_REST(3); CHAIN_REST(4); CHAIN_REST(5); CHAIN_REST(6); CHAIN_REST(7); CHAIN_REST(8);
-        CHAIN_REST(9); CHAIN_REST(10); CHAIN_REST(11); CHAIN_REST(12); CHAIN_REST(13); CHAIN_REST(14); CHAIN_REST(15);
-#undef CHAIN_REST
-    default: break;
-    }
-    return chain;
-}
-
-/* gate and up: block = 2 S wavefronts (matrix = wave / S, slice = wave % S); grid (output_size / 16, jobs) */
+/* gate and up: block = S wavefronts (slices of the inputs); grid (ceil(output_size / 64), jobs) */
 template <uint32_t S>
 __device__ static __forceinline__ void expert_gate_up(const struct expert_gate_up_arguments &arguments,
                                                       unsigned char *arena)
 {
-    __shared__ __attribute__((aligned(16))) uint32_t window[2u * S][WINDOW_WORDS];
-    __shared__ __attribute__((aligned(16))) float partial[2u * S][WAVE * 4u];
+    typedef strip_chain<2> chain_type;
+    constexpr uint32_t TILES = chain_type::TILES;
+    __shared__ __attribute__((aligned(16))) unsigned char window[S][chain_type::WINDOW_BYTES];
+    static_assert(chain_type::WINDOW_BYTES >= TILES * WAVE * 16u, "a wavefront's sums fit its idle window");
     const struct expert_job_record *job = (const struct expert_job_record *)(arena + arguments.jobs_offset) + blockIdx.y;
     if (job->row_count == 0u) {
         return;
     }
-    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    const uint32_t matrix = wave / S, slice = wave % S;
+    const uint32_t lane = threadIdx.x % WAVE, slice = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const uint32_t column = lane % 16u;
-    const bool live = column < job->row_count;
+    const bool live = column < job->row_count; /* a job holds at most eight rows */
     const uint32_t pair = live ? job->pair_index[column] : 0u;
-    const uint64_t row = pair / arguments.pairs_per_row;
+    uint32_t rows[8]; /* the vectors' rows; columns without a row read row 0, and are never stored */
+#pragma unroll
+    for (uint32_t c = 0; c < 8u; c++) {
+        rows[c] = c < job->row_count ? job->pair_index[c] / arguments.pairs_per_row : 0u;
+    }
     const uint32_t steps = arguments.input_size / 128u;
-    const float4_t chain = expert_chain(arena + (matrix == 0u ? job->gate_offset : job->up_offset), arguments.output_size,
-                                        arguments.input_size, blockIdx.x, steps * slice / S, steps * (slice + 1u) / S,
-                                        arena + arguments.codes_offset + row * arguments.input_size,
-                                        arena + arguments.exponents_offset + row * (arguments.input_size / 32u),
-                                        window[wave], lane);
-    *(float4_t *)&partial[wave][lane * 4u] = chain;
+    const uint32_t first = steps * slice / S, last = steps * (slice + 1u) / S;
+    chain_type chain_of;
+    const unsigned char *const matrices[2] = {arena + job->gate_offset, arena + job->up_offset};
+    chain_of.place(matrices, arguments.output_size, arguments.input_size, blockIdx.x, first, arena + arguments.codes_offset,
+                   arena + arguments.exponents_offset, rows, (uint32_t)(uintptr_t)(lds_pointer)&window[slice][0], lane);
+    float4_t chain[TILES];
+#pragma unroll
+    for (uint32_t tile = 0; tile < TILES; tile++) {
+        chain[tile] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    chain_of.whole(last - first, chain);
+    /* the S chains meet in the windows, idle now: [slice][tile][lane] float4 */
+    float4_t *sums = (float4_t *)&window[slice][0];
+#pragma unroll
+    for (uint32_t tile = 0; tile < TILES; tile++) {
+        sums[tile * WAVE + lane] = chain[tile];
+    }
     __syncthreads();
-    if (wave == 0u && live) {
+    /* wavefront w finishes the tiles n = w, w + S, ..: the S chains from +0, in order, then the hidden step */
+    const uint32_t tiles = arguments.output_size / 16u;
+    const uint32_t tile0 = blockIdx.x * STRIP + STRIP <= tiles ? blockIdx.x * STRIP : tiles - STRIP;
+    for (uint32_t n = slice; n < STRIP; n += S) {
+        if (!live || tile0 + n < blockIdx.x * STRIP) { /* a tile the strip before this one stores */
+            continue;
+        }
         float gate[4] = {0.0f, 0.0f, 0.0f, 0.0f}, up[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (uint32_t part = 0; part < S; part++) { /* the S chains from +0, in order */
+        for (uint32_t part = 0; part < S; part++) {
+            const float4_t g4 = ((const float4_t *)&window[part][0])[n * WAVE + lane];
+            const float4_t u4 = ((const float4_t *)&window[part][0])[(STRIP + n) * WAVE + lane];
 #pragma unroll
             for (uint32_t v = 0; v < 4u; v++) {
-                gate[v] = __fadd_rn(gate[v], partial[part][lane * 4u + v]);
-                up[v] = __fadd_rn(up[v], partial[S + part][lane * 4u + v]);
+                gate[v] = __fadd_rn(gate[v], g4[v]);
+                up[v] = __fadd_rn(up[v], u4[v]);
             }
         }
         const float limit = arguments.activation_limit, weight = job->route_weight[column];
@@ -242,17 +334,19 @@ __device__ static __forceinline__ void expert_gate_up(const struct expert_gate_u
             hidden[v] = float_to_bf16(value);
         }
         uint16_t *out = (uint16_t *)(arena + arguments.hidden_offset) + (uint64_t)pair * arguments.output_size +
-                        blockIdx.x * 16u + 4u * (lane / 16u);
+                        (tile0 + n) * 16u + 4u * (lane / 16u);
         *(uint2_t *)out = (uint2_t){(uint32_t)hidden[0] | ((uint32_t)hidden[1] << 16), (uint32_t)hidden[2] | ((uint32_t)hidden[3] << 16)};
     }
 }
 
-/* down: block = S wavefronts; grid (output_size / 16, jobs) */
+/* down: block = S wavefronts; grid (ceil(output_size / 64), jobs) */
 template <uint32_t S>
 __device__ static __forceinline__ void expert_down(const struct expert_down_arguments &arguments, unsigned char *arena)
 {
-    __shared__ __attribute__((aligned(16))) uint32_t window[S][WINDOW_WORDS];
-    __shared__ __attribute__((aligned(16))) float partial[S][WAVE * 4u];
+    typedef strip_chain<1> chain_type;
+    constexpr uint32_t TILES = chain_type::TILES;
+    __shared__ __attribute__((aligned(16))) unsigned char window[S][chain_type::WINDOW_BYTES];
+    static_assert(chain_type::WINDOW_BYTES >= TILES * WAVE * 16u, "a wavefront's sums fit its idle window");
     const struct expert_job_record *job = (const struct expert_job_record *)(arena + arguments.jobs_offset) + blockIdx.y;
     if (job->row_count == 0u) {
         return;
@@ -260,37 +354,58 @@ __device__ static __forceinline__ void expert_down(const struct expert_down_argu
     const uint32_t lane = threadIdx.x % WAVE, slice = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), column = lane % 16u;
     const bool live = column < job->row_count;
     const uint64_t pair = live ? job->pair_index[column] : 0u;
+    uint32_t rows[8]; /* the vectors are the pairs' hidden vectors */
+#pragma unroll
+    for (uint32_t c = 0; c < 8u; c++) {
+        rows[c] = c < job->row_count ? job->pair_index[c] : 0u;
+    }
     const uint32_t steps = arguments.input_size / 128u;
-    const float4_t chain = expert_chain(arena + job->down_offset, arguments.output_size, arguments.input_size, blockIdx.x,
-                                        steps * slice / S, steps * (slice + 1u) / S,
-                                        arena + arguments.codes_offset + pair * arguments.input_size,
-                                        arena + arguments.exponents_offset + pair * (arguments.input_size / 32u),
-                                        window[slice], lane);
-    *(float4_t *)&partial[slice][lane * 4u] = chain;
+    const uint32_t first = steps * slice / S, last = steps * (slice + 1u) / S;
+    chain_type chain_of;
+    const unsigned char *const matrices[1] = {arena + job->down_offset};
+    chain_of.place(matrices, arguments.output_size, arguments.input_size, blockIdx.x, first, arena + arguments.codes_offset,
+                   arena + arguments.exponents_offset, rows, (uint32_t)(uintptr_t)(lds_pointer)&window[slice][0], lane);
+    float4_t chain[TILES];
+#pragma unroll
+    for (uint32_t tile = 0; tile < TILES; tile++) {
+        chain[tile] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    chain_of.whole(last - first, chain);
+    float4_t *sums = (float4_t *)&window[slice][0];
+#pragma unroll
+    for (uint32_t tile = 0; tile < TILES; tile++) {
+        sums[tile * WAVE + lane] = chain[tile];
+    }
     __syncthreads();
-    if (slice == 0u && live) {
+    const uint32_t tiles = arguments.output_size / 16u;
+    const uint32_t tile0 = blockIdx.x * STRIP + STRIP <= tiles ? blockIdx.x * STRIP : tiles - STRIP;
+    for (uint32_t n = slice; n < STRIP; n += S) {
+        if (!live || tile0 + n < blockIdx.x * STRIP) {
+            continue;
+        }
         float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (uint32_t part = 0; part < S; part++) {
+            const float4_t d4 = ((const float4_t *)&window[part][0])[n * WAVE + lane];
 #pragma unroll
             for (uint32_t v = 0; v < 4u; v++) {
-                sum[v] = __fadd_rn(sum[v], partial[part][lane * 4u + v]);
+                sum[v] = __fadd_rn(sum[v], d4[v]);
             }
         }
-        uint16_t *out = (uint16_t *)(arena + arguments.output_offset) + pair * arguments.output_size + blockIdx.x * 16u + 4u * (lane / 16u);
+        uint16_t *out = (uint16_t *)(arena + arguments.output_offset) + pair * arguments.output_size + (tile0 + n) * 16u + 4u * (lane / 16u);
         *(uint2_t *)out = (uint2_t){(uint32_t)float_to_bf16(sum[0]) | ((uint32_t)float_to_bf16(sum[1]) << 16),
                                     (uint32_t)float_to_bf16(sum[2]) | ((uint32_t)float_to_bf16(sum[3]) << 16)};
     }
 }
 
 #define EXPERT_ENTRIES(S)                                                                                         \
-    extern "C" __global__ void __launch_bounds__(2u * S * WAVE) __attribute__((amdgpu_waves_per_eu(4)))           \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
         expert_gate_up_##S(struct expert_gate_up_arguments arguments, unsigned char *arena)                      \
     {                                                                                                             \
         expert_gate_up<S>(arguments, arena);                                                                      \
     }                                                                                                             \
     ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_gate_up_##S, expert_gate_up_arguments);                      \
-    extern "C" __global__ void __launch_bounds__(S * WAVE) __attribute__((amdgpu_waves_per_eu(4)))                \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
         expert_down_##S(struct expert_down_arguments arguments, unsigned char *arena)                            \
     {                                                                                                             \
         expert_down<S>(arguments, arena);                                                                         \

@@ -17,6 +17,7 @@
 
 #include "prepare_common.h"
 
+#define LINEAR_STRIP_OUTPUTS 64u /* a block of the expert kernels: a strip of four tiles of 16 outputs */
 static const uint32_t slice_counts[LINEAR_SLICE_INSTANCES] = {1u, 2u, 4u, 8u, 16u};
 #define BUILT_INSTANCES 4u
 #define MOST_ROWS 4096u /* rows of one call: a wide step's chunk */
@@ -154,9 +155,10 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     if (description->reserved_zero != 0 || description->weight_format != WEIGHT_FORMAT_E2M1_SCALED || format == NULL ||
         format->stored_byte_count(gate_up, &gate_up_bytes) != STATUS_OK ||
         format->stored_byte_count(down, &down_bytes) != STATUS_OK || gate_up->input_size % 128u != 0 ||
-        down->input_size % 128u != 0 || down->input_size != gate_up->output_size) {
-        REFUSE("%s: matrices of format %u in shapes it stores, inputs a multiple of 128, down reading what gate and up "
-               "write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED);
+        down->input_size % 128u != 0 || down->input_size != gate_up->output_size ||
+        gate_up->output_size < LINEAR_STRIP_OUTPUTS || down->output_size < LINEAR_STRIP_OUTPUTS) {
+        REFUSE("%s: matrices of format %u in shapes it stores, inputs a multiple of 128, at least %u outputs, down "
+               "reading what gate and up write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, LINEAR_STRIP_OUTPUTS);
         return STATUS_INVALID_ARGUMENT;
     }
     if (!instance_of(description->gate_up_slice_count, gate_up->input_size, &gate_up_instance) ||
@@ -208,13 +210,14 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
                                                             description->row_output.byte_offset, down->output_size,
                                                             description->pairs_per_row};
     struct kernel_launch launches[LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT];
-    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_GATE_UP], kernels->expert_gate_up[gate_up_instance], gate_up->output_size / 16u,
-                description->job_count, 1, 128u * description->gate_up_slice_count, 0, &gate_up_record, sizeof gate_up_record);
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_GATE_UP], kernels->expert_gate_up[gate_up_instance],
+                (gate_up->output_size + LINEAR_STRIP_OUTPUTS - 1u) / LINEAR_STRIP_OUTPUTS,
+                description->job_count, 1, 64u * description->gate_up_slice_count, 0, &gate_up_record, sizeof gate_up_record);
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_QUANTIZE], kernels->activation_quantize,
                 (gate_up->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)pairs, 1,
                 LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
-    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_DOWN], kernels->expert_down[down_instance], down->output_size / 16u,
-                description->job_count, 1, 64u * description->down_slice_count, 0, &down_record, sizeof down_record);
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_DOWN], kernels->expert_down[down_instance],
+                (down->output_size + LINEAR_STRIP_OUTPUTS - 1u) / LINEAR_STRIP_OUTPUTS, description->job_count, 1, 64u * description->down_slice_count, 0, &down_record, sizeof down_record);
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_ROW_SUM], kernels->expert_row_sum,
                 (down->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)rows, 1,
                 LINEAR_ELEMENT_THREADS, 0, &row_sum_record, sizeof row_sum_record);
