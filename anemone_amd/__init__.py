@@ -92,6 +92,15 @@ class RouterDescription(C.Structure):
                 ("pick_count", u32), ("affinity_kind", u32), ("route_scale", f32)]
 
 
+class RouterWideDescription(C.Structure):
+    _fields_ = [("expert_offsets", C.POINTER(u64)), ("expert_widths", C.POINTER(u32)), ("step", Range), ("scores", Range),
+                ("bias", Range), ("offsets", Range), ("expert_weights", Range), ("affinities", Range), ("picks", Range),
+                ("counts", Range), ("pairs", Range), ("runs", Range), ("tiles", Range), ("jobs", Range),
+                ("gate_up_shape", Shape), ("down_shape", Shape), ("weight_format", C.c_int), ("order", C.c_int),
+                ("row_count", u32), ("reserved_zero", u32), ("expert_count", u32), ("pick_count", u32),
+                ("affinity_kind", u32), ("route_scale", f32)]
+
+
 class RouterProjectionDescription(C.Structure):
     _fields_ = [("weights", Range), ("rows", Range), ("output", Range), ("row_count", u32), ("hidden", u32),
                 ("expert_count", u32), ("reserved_zero", u32)]
@@ -154,6 +163,7 @@ def library():
             "router_kernels_prepare": [vp, vp, C.POINTER(RouterKernels)],
             "router_select_prepare": [C.POINTER(RouterDescription), u64, C.POINTER(RouterKernels), launch_p],
             "router_projection_prepare": [C.POINTER(RouterProjectionDescription), u64, C.POINTER(RouterKernels), launch_p],
+            "router_wide_prepare": [C.POINTER(RouterWideDescription), u64, C.POINTER(RouterKernels), launch_p],
             "linear_kernels_prepare": [vp, vp, u32, C.POINTER(LinearKernels)],
             "linear_quantize_prepare": [C.POINTER(QuantizeDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_routed_experts_prepare": [C.POINTER(RoutedExpertsDescription), u64, C.POINTER(LinearKernels), launch_p],
@@ -315,6 +325,60 @@ def launches_of(count):
     return (KernelLaunch * count)()
 
 
+ROUTER_SORT_ROWS = 384
+WIDE_PAIR_DTYPE = np.dtype([("pair_index", "<u4"), ("route_weight", "<f4")])
+WIDE_RUN_DTYPE = np.dtype([("first_pair", "<u4"), ("pair_count", "<u4")])
+WIDE_TILE_DTYPE = np.dtype([("gate_offset", "<u8"), ("up_offset", "<u8"), ("down_offset", "<u8"), ("first_pair", "<u4"),
+                            ("pair_count", "<u4")])
+
+
+def wide_tile_count(rows, picks, experts):
+    return (rows * picks + 63) // 64 + experts
+
+
+def wide_job_count(rows, picks, experts):
+    return min(rows * picks, (rows * picks + 7 * experts) // 8)
+
+
+class WideRouter:
+    """The wide select of a layer already laid out in a card's arena (its offsets table, bias, scores and step block):
+    reserves the picks, counts, sorted pairs, runs, tiles and the job table of `rows` rows, and prepares the four
+    launches."""
+
+    def __init__(self, layer, rows, weight_format, gate_up_shape, down_shape, widths=None, order=0):
+        card = layer.card
+        self.layer, self.card, self.rows = layer, card, rows
+        E, P = layer.E, layer.P
+        self.tile_count, self.job_count = wide_tile_count(rows, P, E), wide_job_count(rows, P, E)
+        sizes = {"picks": rows * P * 8, "counts": (rows + ROUTER_SORT_ROWS - 1) // ROUTER_SORT_ROWS * E * 4,
+                 "pairs": rows * P * 8, "runs": E * 8, "tiles": self.tile_count * 32, "jobs": self.job_count * 96}
+        self.ranges = {name: Range(card.reserve(size), size) for name, size in sizes.items()}
+        d = RouterWideDescription()
+        d.expert_offsets = layer.expert_offsets.ctypes.data_as(C.POINTER(u64))
+        self._widths = None if widths is None else np.ascontiguousarray(widths, dtype=np.uint32)
+        d.expert_widths = None if widths is None else self._widths.ctypes.data_as(C.POINTER(u32))
+        d.step, d.scores = Range(layer.step_offset, 16), Range(layer.scores_offset, rows * E * 4)
+        d.bias, d.offsets = Range(layer.bias_offset, E * 4), Range(layer.offsets_offset, E * 24)
+        d.expert_weights = Range(layer.weights_offset, layer.weights_bytes)
+        d.affinities = Range(layer.affinities_offset, rows * E * 4)
+        for name, value in self.ranges.items():
+            setattr(d, name, value)
+        d.gate_up_shape, d.down_shape, d.weight_format, d.order = gate_up_shape, down_shape, weight_format, order
+        d.row_count, d.expert_count, d.pick_count = rows, E, P
+        d.affinity_kind, d.route_scale = layer.affinity_kind, layer.route_scale
+        self.description = d
+
+    def launches(self):
+        launches = launches_of(4)
+        check(self.card.lib.router_wide_prepare(C.byref(self.description), self.card.arena_bytes, C.byref(self.layer.router_kernels), launches),
+              "router_wide_prepare")
+        return launches
+
+    def read(self, name, dtype):
+        r = self.ranges[name]
+        return self.card.download(r.byte_offset, r.byte_count).view(dtype)
+
+
 class Exl3Layer:
     """One EXL3 MoE layer laid out in a card's arena the way the reference's loader lays one out: the experts'
     stored matrices, the [E][3] offsets table, an optional per-matrix widths table, the router's weights and bias;
@@ -363,6 +427,7 @@ class Exl3Layer:
         self.workspace_offset = card.reserve(exl3_tc_workspace_bytes(self.pairs, hidden, inner))
         self.kernels = RouterKernels()
         check(lib.router_kernels_prepare(backend_table(), card.handle, C.byref(self.kernels)), "router_kernels_prepare")
+        self.router_kernels = self.kernels
 
     def set_rows(self, x_bf16, live_rows=None):
         self.card.upload(self.x_offset, x_bf16)
@@ -500,15 +565,16 @@ class Fp4Layer:
         self.card.upload(self.x_offset, x_bf16)
         self.card.upload(self.step_offset, step_block(self.rows if live_rows is None else live_rows))
 
-    def experts_description(self):
+    def experts_description(self, wide=None):
+        """wide: a WideRouter whose job table the experts read instead of the select's."""
         d = RoutedExpertsDescription()
-        d.jobs = Range(self.jobs_offset, self.pairs * 96)
+        d.jobs = Range(self.jobs_offset, self.pairs * 96) if wide is None else wide.ranges["jobs"]
         d.expert_weights = Range(self.weights_offset, self.weights_bytes)
         for name, value in self.ranges.items():
             setattr(d, name, value)
         d.gate_up_shape, d.down_shape = Shape(self.I, self.H, 4, 0), Shape(self.H, self.I, 4, 0)
         d.weight_format = WEIGHT_FORMAT_E2M1_SCALED
-        d.job_count, d.row_count, d.pairs_per_row = self.pairs, self.rows, self.P
+        d.job_count, d.row_count, d.pairs_per_row = self.pairs if wide is None else wide.job_count, self.rows, self.P
         d.gate_up_slice_count, d.down_slice_count = self.gate_up_slices, self.down_slices
         d.activation_limit = self.limit
         return d
@@ -542,8 +608,11 @@ class Fp4Layer:
         check(self.card.lib.router_select_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.router_kernels), launch), "router_select_prepare")
         return launch
 
-    def expert_launches(self):
-        d = self.experts_description()
+    def wide_router(self):
+        return WideRouter(self, self.rows, WEIGHT_FORMAT_E2M1_SCALED, Shape(self.I, self.H, 4, 0), Shape(self.H, self.I, 4, 0))
+
+    def expert_launches(self, wide=None):
+        d = self.experts_description(wide)
         launches = launches_of(4)
         check(self.card.lib.linear_routed_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launches), "linear_routed_experts_prepare")
         return launches

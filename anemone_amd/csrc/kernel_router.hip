@@ -329,3 +329,250 @@ extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_select_entry, router_select_arguments);
+
+/* ---- the wide select: rows of a prefill, sorted by expert ------------------------------------------------------
+ * Four launches of one record, in this order (include/anemone/router_records.h:31-47 of the reference; the kernels
+ * at source/kernel_router.cu:97-459 there): the picks of every live row; the pairs of each expert counted in blocks
+ * of ROUTER_SORT_ROWS rows; every pair placed (a pair's place: the pairs of lower experts, and of its expert in
+ * lower rows), the runs and the tiles of at most 64 pairs; the job table of at most 8 pairs a job. No atomic
+ * operation: a thread owns an expert and walks the block's picks in row order. */
+#define WIDE_SORT_THREADS 512u
+
+__device__ static __forceinline__ uint32_t wide_live_rows(const struct router_wide_arguments &arguments, const unsigned char *arena)
+{
+    const uint32_t step_rows = ((const struct step_block *)(arena + arguments.step_offset))->row_count;
+    return step_rows < arguments.row_count ? step_rows : arguments.row_count;
+}
+
+/* grid (ceil(row_count / 8)), a wavefront a row: its affinities, as the select writes them, and its picks by slot */
+extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
+    router_wide_select(struct router_wide_arguments arguments, unsigned char *arena)
+{
+    __shared__ float affinities[LINEAR_MAXIMUM_ROWS * ROUTER_MOST_EXPERTS];
+    __shared__ float pick_weights[LINEAR_MAXIMUM_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t pick_experts[LINEAR_MAXIMUM_ROWS * ROUTER_MOST_PICKS];
+    const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
+    const uint32_t live_rows = wide_live_rows(arguments, arena);
+    const uint32_t first_row = blockIdx.x * LINEAR_MAXIMUM_ROWS;
+    if (first_row >= live_rows) {
+        return;
+    }
+    const uint32_t rows = live_rows - first_row < LINEAR_MAXIMUM_ROWS ? live_rows - first_row : LINEAR_MAXIMUM_ROWS;
+    const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    for (uint32_t index = threadIdx.x; index < rows * experts; index += blockDim.x) {
+        const uint64_t at = (uint64_t)first_row * experts + index;
+        const float a = router_affinity(((const float *)(arena + arguments.scores_offset))[at], arguments.affinity_kind);
+        affinities[index] = a;
+        ((float *)(arena + arguments.affinities_offset))[at] = a;
+    }
+    __syncthreads();
+    if (wave < rows) {
+        router_row(affinities + wave * experts, (const float *)(arena + arguments.bias_offset), lane, experts, picks,
+                   arguments.reference_order, arguments.route_scale, pick_experts + wave * picks, pick_weights + wave * picks);
+    }
+    __syncthreads();
+    struct router_pick *out = (struct router_pick *)(arena + arguments.picks_offset) + (uint64_t)first_row * picks;
+    for (uint32_t index = threadIdx.x; index < rows * picks; index += blockDim.x) {
+        out[index] = (struct router_pick){pick_experts[index], pick_weights[index]};
+    }
+}
+ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_select, router_wide_arguments);
+
+/* the picked experts of the live rows of block `block` of ROUTER_SORT_ROWS rows, into LDS; returns their number */
+__device__ static __forceinline__ uint32_t wide_block_picks(const struct router_wide_arguments &arguments, const unsigned char *arena,
+                                                            uint32_t block, uint32_t live_rows, uint32_t *experts_out)
+{
+    const uint32_t first_row = block * ROUTER_SORT_ROWS;
+    const uint32_t rows = live_rows <= first_row ? 0u : live_rows - first_row < ROUTER_SORT_ROWS ? live_rows - first_row : ROUTER_SORT_ROWS;
+    const struct router_pick *picks = (const struct router_pick *)(arena + arguments.picks_offset) + (uint64_t)first_row * arguments.pick_count;
+    for (uint32_t index = threadIdx.x; index < rows * arguments.pick_count; index += blockDim.x) {
+        experts_out[index] = picks[index].expert;
+    }
+    return rows * arguments.pick_count;
+}
+
+/* grid (ceil(row_count / ROUTER_SORT_ROWS)): counts [block][E] */
+extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
+    router_wide_count(struct router_wide_arguments arguments, unsigned char *arena)
+{
+    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    const uint32_t live_rows = wide_live_rows(arguments, arena);
+    const uint32_t pairs = wide_block_picks(arguments, arena, blockIdx.x, live_rows, block_experts);
+    __syncthreads();
+    if (pairs == 0u) {
+        return; /* a block of no live row writes nothing; the place reads no count of it */
+    }
+    uint32_t *counts = (uint32_t *)(arena + arguments.counts_offset) + (uint64_t)blockIdx.x * arguments.expert_count;
+    for (uint32_t expert = threadIdx.x; expert < arguments.expert_count; expert += blockDim.x) {
+        uint32_t count = 0;
+        for (uint32_t index = 0; index < pairs; index++) {
+            count += block_experts[index] == expert ? 1u : 0u;
+        }
+        counts[expert] = count;
+    }
+}
+ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_count, router_wide_arguments);
+
+/* exclusive prefix sums of values[0 .. count) in LDS, count <= ROUTER_MOST_EXPERTS, by the whole block; total returned */
+__device__ static __forceinline__ uint32_t block_exclusive_scan(uint32_t *values, uint32_t count, uint32_t *scratch)
+{
+    /* count is small (at most 512): Hillis-Steele over two buffers */
+    uint32_t *from = values, *to = scratch;
+    for (uint32_t step = 1; step < count; step *= 2u) {
+        for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
+            to[i] = from[i] + (i >= step ? from[i - step] : 0u);
+        }
+        __syncthreads();
+        uint32_t *swap = from;
+        from = to;
+        to = swap;
+    }
+    const uint32_t total = count == 0u ? 0u : from[count - 1u];
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
+        to[i] = i == 0u ? 0u : from[i - 1u];
+    }
+    __syncthreads();
+    if (to != values) {
+        for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
+            values[i] = to[i];
+        }
+        __syncthreads();
+    }
+    return total;
+}
+
+/* grid as the count's: the sorted pairs of the block's rows; block 0 also the runs and every tile */
+extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
+    router_wide_place(struct router_wide_arguments arguments, unsigned char *arena)
+{
+    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
+    __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
+    const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
+    const uint32_t live_rows = wide_live_rows(arguments, arena);
+    const uint32_t live_blocks = (live_rows + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
+    const uint32_t pairs = wide_block_picks(arguments, arena, blockIdx.x, live_rows, block_experts);
+    if (pairs == 0u && blockIdx.x != 0u) {
+        return;
+    }
+    const uint32_t *counts = (const uint32_t *)(arena + arguments.counts_offset);
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        uint32_t total = 0, lower = 0;
+        for (uint32_t block = 0; block < live_blocks; block++) {
+            const uint32_t count = counts[(uint64_t)block * experts + expert];
+            total += count;
+            lower += block < blockIdx.x ? count : 0u;
+        }
+        totals[expert] = total;
+        starts[expert] = total;
+        before[expert] = lower;
+        tile_starts[expert] = (total + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS;
+    }
+    __syncthreads();
+    (void)block_exclusive_scan(starts, experts, scratch);
+    const struct router_pick *all_picks = (const struct router_pick *)(arena + arguments.picks_offset);
+    struct wide_pair *sorted = (struct wide_pair *)(arena + arguments.pairs_offset);
+    const uint32_t first_pair = blockIdx.x * ROUTER_SORT_ROWS * picks;
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        uint32_t place = starts[expert] + before[expert];
+        for (uint32_t index = 0; index < pairs; index++) {
+            if (block_experts[index] == expert) {
+                sorted[place] = (struct wide_pair){first_pair + index, all_picks[first_pair + index].route_weight};
+                place++;
+            }
+        }
+    }
+    if (blockIdx.x != 0u) {
+        return;
+    }
+    struct wide_run *runs = (struct wide_run *)(arena + arguments.runs_offset);
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        runs[expert] = (struct wide_run){starts[expert], totals[expert]};
+    }
+    const uint32_t used_tiles = block_exclusive_scan(tile_starts, experts, scratch);
+    if (threadIdx.x == 0u) {
+        tile_starts[experts] = used_tiles;
+    }
+    __syncthreads();
+    const uint32_t all_tiles = ROUTER_WIDE_TILES_OF(arguments.row_count, picks, experts);
+    struct wide_expert_tile *tiles = (struct wide_expert_tile *)(arena + arguments.tiles_offset);
+    const uint64_t *offsets = (const uint64_t *)(arena + arguments.expert_offsets_offset);
+    for (uint32_t tile = threadIdx.x; tile < all_tiles; tile += blockDim.x) {
+        struct wide_expert_tile value = {0, 0, 0, 0, 0};
+        if (tile < used_tiles) {
+            uint32_t low = 0, high = experts; /* the expert whose tiles hold this one: tile_starts[e] <= tile < [e + 1] */
+            while (high - low > 1u) {
+                const uint32_t middle = (low + high) / 2u;
+                if (tile_starts[middle] <= tile) {
+                    low = middle;
+                } else {
+                    high = middle;
+                }
+            }
+            const uint32_t taken = (tile - tile_starts[low]) * WIDE_TILE_PAIRS, left = totals[low] - taken;
+            value.gate_offset = offsets[(uint64_t)low * MODEL_EXPERT_MATRICES + 0u];
+            value.up_offset = offsets[(uint64_t)low * MODEL_EXPERT_MATRICES + 1u];
+            value.down_offset = offsets[(uint64_t)low * MODEL_EXPERT_MATRICES + 2u];
+            value.first_pair = starts[low] + taken;
+            value.pair_count = left < WIDE_TILE_PAIRS ? left : WIDE_TILE_PAIRS;
+        }
+        tiles[tile] = value;
+    }
+}
+ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_place, router_wide_arguments);
+
+/* grid (1): the job table of the runs, a thread a job */
+extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
+    router_wide_jobs(struct router_wide_arguments arguments, unsigned char *arena)
+{
+    __shared__ uint32_t job_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
+    const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
+    const struct wide_run *runs = (const struct wide_run *)(arena + arguments.runs_offset);
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        job_starts[expert] = (runs[expert].pair_count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS;
+    }
+    __syncthreads();
+    const uint32_t used_jobs = block_exclusive_scan(job_starts, experts, scratch);
+    if (threadIdx.x == 0u) {
+        job_starts[experts] = used_jobs;
+    }
+    __syncthreads();
+    const uint32_t all_jobs = ROUTER_WIDE_JOBS_OF(arguments.row_count, picks, experts);
+    const struct wide_pair *sorted = (const struct wide_pair *)(arena + arguments.pairs_offset);
+    const uint64_t *offsets = (const uint64_t *)(arena + arguments.expert_offsets_offset);
+    struct expert_job_record *jobs = (struct expert_job_record *)(arena + arguments.jobs_offset);
+    for (uint32_t job = threadIdx.x; job < all_jobs; job += blockDim.x) {
+        struct expert_job_record value;
+        uint32_t *words = (uint32_t *)&value;
+#pragma unroll
+        for (uint32_t word = 0; word < JOB_WORDS; word++) {
+            words[word] = 0u;
+        }
+        if (job < used_jobs) {
+            uint32_t low = 0, high = experts;
+            while (high - low > 1u) {
+                const uint32_t middle = (low + high) / 2u;
+                if (job_starts[middle] <= job) {
+                    low = middle;
+                } else {
+                    high = middle;
+                }
+            }
+            const struct wide_run run = runs[low];
+            const uint32_t taken = (job - job_starts[low]) * LINEAR_MAXIMUM_ROWS, left = run.pair_count - taken;
+            value.gate_offset = offsets[(uint64_t)low * MODEL_EXPERT_MATRICES + 0u];
+            value.up_offset = offsets[(uint64_t)low * MODEL_EXPERT_MATRICES + 1u];
+            value.down_offset = offsets[(uint64_t)low * MODEL_EXPERT_MATRICES + 2u];
+            value.row_count = left < LINEAR_MAXIMUM_ROWS ? left : LINEAR_MAXIMUM_ROWS;
+            value.expert = low;
+            for (uint32_t column = 0; column < value.row_count; column++) {
+                const struct wide_pair pair = sorted[run.first_pair + taken + column];
+                value.pair_index[column] = pair.pair_index;
+                value.route_weight[column] = pair.route_weight;
+            }
+        }
+        jobs[job] = value;
+    }
+}
+ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_jobs, router_wide_arguments);

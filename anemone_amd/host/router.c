@@ -8,6 +8,10 @@
  *   launch        kernel                grid                        block
  *   projection    router_projection     (ceil(E / 8), ceil(rows / 4), 1)   128   eight experts and four rows a block
  *   select        router_select_entry   (1, 1, 1)                   512   a wavefront a row
+ *   wide select   router_wide_select    (ceil(rows / 8), 1, 1)      512   a wavefront a row
+ *   wide count    router_wide_count     (ceil(rows / 384), 1, 1)    512   a thread an expert
+ *   wide place    router_wide_place     (ceil(rows / 384), 1, 1)    512   a thread an expert; block 0 the runs and tiles
+ *   wide jobs     router_wide_jobs      (1, 1, 1)                   512   a thread a job
  */
 #include <inttypes.h>
 #include <string.h>
@@ -15,6 +19,7 @@
 #include "prepare_common.h"
 
 #define SELECT_THREADS (LINEAR_MAXIMUM_ROWS * 64u)
+#define WIDE_SORT_THREADS 512u
 #define PROJECTION_THREADS 128u
 #define PROJECTION_OUTPUTS 8u /* experts a block */
 #define PROJECTION_ROWS 4u    /* rows a block takes at once */
@@ -242,10 +247,78 @@ result_status router_projection_prepare(const struct router_projection_descripti
 result_status router_wide_prepare(const struct router_wide_description *description, uint64_t arena_byte_count,
                                   const struct router_kernels_record *kernels, struct kernel_launch *launches_out)
 {
-    (void)arena_byte_count;
-    if (description == NULL || kernels == NULL || launches_out == NULL) {
+    static const char what[] = "the router's wide select";
+    if (description == NULL || kernels == NULL || launches_out == NULL || description->expert_offsets == NULL) {
+        REFUSE("%s: a missing argument", what);
         return STATUS_INVALID_ARGUMENT;
     }
-    REFUSE("the router's wide select: not built yet in this library");
-    return STATUS_UNSUPPORTED;
+    const uint32_t E = description->expert_count, P = description->pick_count, R = description->row_count;
+    if (description->reserved_zero != 0 || kernels->wide_select == BACKEND_NO_KERNEL || kernels->wide_count == BACKEND_NO_KERNEL ||
+        kernels->wide_place == BACKEND_NO_KERNEL || kernels->wide_jobs == BACKEND_NO_KERNEL) {
+        REFUSE("%s: a reserved field that is not zero, or a kernel of the four is not prepared", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (!shape_counts_are_valid(what, E, P, description->affinity_kind, description->order)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (R == 0 || R > ROUTER_WIDE_MOST_ROWS || !(description->route_scale > 0.0f) ||
+        (description->weight_format != WEIGHT_FORMAT_E2M1_SCALED && description->weight_format != WEIGHT_FORMAT_E4M3_SCALED &&
+         description->weight_format != WEIGHT_FORMAT_EXL3)) {
+        REFUSE("%s: 1 to %u rows, a route scale above zero, experts of a format the path holds", what, ROUTER_WIDE_MOST_ROWS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t row_bytes = (uint64_t)E * 4u, rows_bytes = R * row_bytes, pairs = (uint64_t)R * P;
+    const uint64_t blocks = (R + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
+    const struct checked_range ranges[] = {
+        {"the step block", description->step, sizeof(struct step_block), false},
+        {"the router scores", description->scores, rows_bytes, false},
+        {"the bias", description->bias, row_bytes, false},
+        {"the expert offsets", description->offsets, (uint64_t)E * MODEL_EXPERT_MATRICES * 8u, false},
+        {"the experts' matrices", description->expert_weights, 0, false},
+        {"the affinities", description->affinities, rows_bytes, false},
+        {"the picks", description->picks, pairs * sizeof(struct router_pick), false},
+        {"the counts", description->counts, blocks * row_bytes, false},
+        {"the sorted pairs", description->pairs, pairs * sizeof(struct wide_pair), false},
+        {"the runs", description->runs, (uint64_t)E * sizeof(struct wide_run), false},
+        {"the tiles", description->tiles, (uint64_t)ROUTER_WIDE_TILES_OF(R, P, E) * sizeof(struct wide_expert_tile), false},
+        {"the job table", description->jobs, (uint64_t)ROUTER_WIDE_JOBS_OF(R, P, E) * sizeof(struct expert_job_record), false},
+    };
+    uint64_t least_gate_up = 0, least_down = 0;
+    if (!ranges_are_valid(what, ranges, sizeof ranges / sizeof ranges[0], arena_byte_count) ||
+        !table_is_valid(what, description->weight_format, &description->gate_up_shape, &description->down_shape,
+                        description->expert_offsets, description->expert_widths, E, &description->expert_weights,
+                        &least_gate_up, &least_down)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t end = description->expert_weights.byte_offset + description->expert_weights.byte_count;
+    const struct router_wide_arguments record = {
+        .step_offset = description->step.byte_offset,
+        .scores_offset = description->scores.byte_offset,
+        .bias_offset = description->bias.byte_offset,
+        .expert_offsets_offset = description->offsets.byte_offset,
+        .affinities_offset = description->affinities.byte_offset,
+        .picks_offset = description->picks.byte_offset,
+        .counts_offset = description->counts.byte_offset,
+        .pairs_offset = description->pairs.byte_offset,
+        .runs_offset = description->runs.byte_offset,
+        .tiles_offset = description->tiles.byte_offset,
+        .jobs_offset = description->jobs.byte_offset,
+        .weights_offset = description->expert_weights.byte_offset,
+        .gate_up_last_offset = end - least_gate_up,
+        .down_last_offset = end - least_down,
+        .row_count = R,
+        .reference_order = description->order == LINEAR_ORDER_REFERENCE ? 1u : 0u,
+        .expert_count = E,
+        .pick_count = P,
+        .affinity_kind = description->affinity_kind,
+        .route_scale = description->route_scale,
+    };
+    struct kernel_launch launches[ROUTER_WIDE_LAUNCH_COUNT];
+    launch_fill(&launches[ROUTER_WIDE_SELECT_LAUNCH], kernels->wide_select, (R + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS, 1, 1,
+                SELECT_THREADS, 0, &record, sizeof record);
+    launch_fill(&launches[ROUTER_WIDE_COUNT_LAUNCH], kernels->wide_count, (uint32_t)blocks, 1, 1, WIDE_SORT_THREADS, 0, &record, sizeof record);
+    launch_fill(&launches[ROUTER_WIDE_PLACE_LAUNCH], kernels->wide_place, (uint32_t)blocks, 1, 1, WIDE_SORT_THREADS, 0, &record, sizeof record);
+    launch_fill(&launches[ROUTER_WIDE_JOBS_LAUNCH], kernels->wide_jobs, 1, 1, 1, WIDE_SORT_THREADS, 0, &record, sizeof record);
+    memcpy(launches_out, launches, sizeof launches);
+    return STATUS_OK;
 }

@@ -112,6 +112,7 @@ ANEMONE_RECORD_HAS(wide_expert_tile, 32);
 #define KERNEL_ROUTER_WIDE_SMALL "router_wide_small"
 #define ROUTER_THREADS 256u
 #define ROUTER_SORT_ROWS 384u
+#define ROUTER_WIDE_MOST_ROWS 65536u /* rows of one wide select */
 
 struct router_projection_arguments { /* scores [rows][experts] = W x, bfloat16 in, float32 out */
     uint64_t weights_offset;         /* read: bfloat16 [expert_count][hidden] */
