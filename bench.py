@@ -88,15 +88,16 @@ def fp4_decode(amd, workloads, arguments):
     layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router,
                          gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices)
     layer.set_rows(x, rows)
-    step = amd.launches_of(7)
-    step[0] = layer.projection_launch()[0]
-    step[1] = layer.select_launch(0)[0]
-    step[2] = layer.quantize_launch()[0]
-    experts = layer.expert_launches()
-    for i in range(4):
-        step[3 + i] = experts[i]
-    names = ["router_projection", "router_select_entry", "activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
-             "expert_down", "expert_row_sum_entry"]
+    wide = layer.wide_router() if rows > 8 else None  # more than eight rows: the wide select sorts the pairs by expert
+    routing = [layer.select_launch(0)[0]] if wide is None else list(wide.launches())
+    routing_names = ["router_select_entry"] if wide is None else ["router_wide_select", "router_wide_count", "router_wide_place", "router_wide_jobs"]
+    experts = layer.expert_launches(wide)
+    parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(4)]
+    step = amd.launches_of(len(parts))
+    for i, launch in enumerate(parts):
+        step[i] = launch
+    names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
+                                                     "expert_down", "expert_row_sum_entry"]
     for _ in range(arguments.warmup):
         card.run(step, wait=False)
     card.wait()
@@ -106,13 +107,13 @@ def fp4_decode(amd, workloads, arguments):
     for _ in range(arguments.steps):
         per_launch += np.array(card.run_timed(step))
     per_launch /= arguments.steps
-    jobs = layer.jobs()
+    jobs = layer.jobs() if wide is None else wide.read("jobs", amd.JOB_DTYPE)
     live = jobs[jobs["row_count"] > 0]
     distinct = np.unique(live["expert"])
     matrix_bytes = HIDDEN * INNER // 2 + HIDDEN * INNER // 32
     gate_up_bytes = 2 * matrix_bytes * len(distinct)
-    gate_up_us = float(per_launch[3])
-    down_us = float(per_launch[5])
+    gate_up_us = float(per_launch[names.index("expert_gate_up")])
+    down_us = float(per_launch[names.index("expert_down")])
     result = {
         "metric": "MoE layer tok/s; decode HBM GB/s & prefill MFMA % of peak, 1 GPU",
         "value": rows * arguments.steps / seconds, "unit": "tok/s", "n_gpus": 1, "steps": arguments.steps,
