@@ -110,7 +110,7 @@ class LinearKernels(C.Structure):
     _fields_ = [("activation_quantize", u32), ("expert_gate_up", u32 * 5), ("expert_down", u32 * 5), ("expert_row_sum", u32),
                 ("trunk_linear_quantized", u32 * 5), ("trunk_linear_bfloat16", u32 * 5), ("trunk_hidden", u32),
                 ("trunk_linear_quantized_wide", u32 * 5), ("trunk_linear_bfloat16_wide", u32 * 5),
-                ("trunk_linear_quantized_interleaved", u32)]
+                ("trunk_linear_quantized_interleaved", u32), ("expert_gate_up_e4m3", u32 * 5), ("expert_down_e4m3", u32 * 5)]
 
 
 class QuantizeDescription(C.Structure):
@@ -521,13 +521,16 @@ class Exl3Layer:
 
 
 class Fp4Layer:
-    """One MoE layer of the original FP4 weights (WEIGHT_FORMAT_E2M1_SCALED, stored bytes as the reference's packs
-    hold them) in a card's arena, with the scratch ranges of a step of at most `rows` rows: the quantizer of the rows,
+    """One MoE layer of the original FP4 weights (WEIGHT_FORMAT_E2M1_SCALED; or, with weight_format, of FP8 weights,
+    WEIGHT_FORMAT_E4M3_SCALED; stored bytes as the reference's packs hold them) in a card's arena, with the scratch ranges of a step of at most `rows` rows: the quantizer of the rows,
     the router's select, and the four launches of the routed experts."""
 
     def __init__(self, card, hidden, inner, expert_count, picks, rows, matrices, router_weights_bf16=None,
-                 affinity_kind=AFFINITY_SIGMOID, route_scale=1.5, limit=10.0, gate_up_slices=4, down_slices=2):
+                 affinity_kind=AFFINITY_SIGMOID, route_scale=1.5, limit=10.0, gate_up_slices=4, down_slices=2,
+                 weight_format=WEIGHT_FORMAT_E2M1_SCALED):
         self.card, self.H, self.I, self.E, self.P, self.rows = card, hidden, inner, expert_count, picks, rows
+        self.weight_format = weight_format
+        self.bits = 8 if weight_format == WEIGHT_FORMAT_E4M3_SCALED else 4
         self.limit, self.affinity_kind, self.route_scale = limit, affinity_kind, route_scale
         self.gate_up_slices, self.down_slices = gate_up_slices, down_slices
         self.pairs = rows * picks
@@ -572,8 +575,8 @@ class Fp4Layer:
         d.expert_weights = Range(self.weights_offset, self.weights_bytes)
         for name, value in self.ranges.items():
             setattr(d, name, value)
-        d.gate_up_shape, d.down_shape = Shape(self.I, self.H, 4, 0), Shape(self.H, self.I, 4, 0)
-        d.weight_format = WEIGHT_FORMAT_E2M1_SCALED
+        d.gate_up_shape, d.down_shape = Shape(self.I, self.H, self.bits, 0), Shape(self.H, self.I, self.bits, 0)
+        d.weight_format = self.weight_format
         d.job_count, d.row_count, d.pairs_per_row = self.pairs if wide is None else wide.job_count, self.rows, self.P
         d.gate_up_slice_count, d.down_slice_count = self.gate_up_slices, self.down_slices
         d.activation_limit = self.limit
@@ -609,7 +612,7 @@ class Fp4Layer:
         return launch
 
     def wide_router(self):
-        return WideRouter(self, self.rows, WEIGHT_FORMAT_E2M1_SCALED, Shape(self.I, self.H, 4, 0), Shape(self.H, self.I, 4, 0))
+        return WideRouter(self, self.rows, self.weight_format, Shape(self.I, self.H, self.bits, 0), Shape(self.H, self.I, self.bits, 0))
 
     def expert_launches(self, wide=None):
         d = self.experts_description(wide)

@@ -66,6 +66,17 @@ result_status linear_kernels_prepare(const struct backend_operations *backend, s
                                              &kernels.expert_down[instance]);
         }
     }
+    for (uint32_t instance = 0; status == STATUS_OK && instance < BUILT_INSTANCES; instance++) {
+        char name[48];
+        (void)snprintf(name, sizeof name, "%se4m3_%u", KERNEL_EXPERT_GATE_UP_STEM, slice_counts[instance]);
+        status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, name, sizeof(struct expert_gate_up_arguments),
+                                         &kernels.expert_gate_up_e4m3[instance]);
+        if (status == STATUS_OK) {
+            (void)snprintf(name, sizeof name, "%se4m3_%u", KERNEL_EXPERT_DOWN_STEM, slice_counts[instance]);
+            status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, name, sizeof(struct expert_down_arguments),
+                                             &kernels.expert_down_e4m3[instance]);
+        }
+    }
     if (status == STATUS_OK) {
         status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, KERNEL_EXPERT_ROW_SUM,
                                          sizeof(struct expert_row_sum_arguments), &kernels.expert_row_sum);
@@ -152,13 +163,16 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     const struct weight_format_operations *format = weight_format_operations_of(description->weight_format);
     uint64_t gate_up_bytes = 0, down_bytes = 0;
     uint32_t gate_up_instance = 0, down_instance = 0;
-    if (description->reserved_zero != 0 || description->weight_format != WEIGHT_FORMAT_E2M1_SCALED || format == NULL ||
+    const bool bytes = description->weight_format == WEIGHT_FORMAT_E4M3_SCALED;
+    const uint32_t strip_outputs = bytes ? LINEAR_STRIP_OUTPUTS / 2u : LINEAR_STRIP_OUTPUTS;
+    if (description->reserved_zero != 0 || (description->weight_format != WEIGHT_FORMAT_E2M1_SCALED && !bytes) || format == NULL ||
         format->stored_byte_count(gate_up, &gate_up_bytes) != STATUS_OK ||
         format->stored_byte_count(down, &down_bytes) != STATUS_OK || gate_up->input_size % 128u != 0 ||
         down->input_size % 128u != 0 || down->input_size != gate_up->output_size ||
-        gate_up->output_size < LINEAR_STRIP_OUTPUTS || down->output_size < LINEAR_STRIP_OUTPUTS) {
-        REFUSE("%s: matrices of format %u in shapes it stores, inputs a multiple of 128, at least %u outputs, down "
-               "reading what gate and up write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, LINEAR_STRIP_OUTPUTS);
+        gate_up->output_size < strip_outputs || down->output_size < strip_outputs) {
+        REFUSE("%s: matrices of format %u or %u in shapes it stores, inputs a multiple of 128, at least %u outputs, down "
+               "reading what gate and up write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, (uint32_t)WEIGHT_FORMAT_E4M3_SCALED,
+               strip_outputs);
         return STATUS_INVALID_ARGUMENT;
     }
     if (!instance_of(description->gate_up_slice_count, gate_up->input_size, &gate_up_instance) ||
@@ -167,7 +181,9 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
                description->gate_up_slice_count, description->down_slice_count);
         return STATUS_INVALID_ARGUMENT;
     }
-    if (kernels->expert_gate_up[gate_up_instance] == BACKEND_NO_KERNEL || kernels->expert_down[down_instance] == BACKEND_NO_KERNEL ||
+    const uint32_t gate_up_kernel = bytes ? kernels->expert_gate_up_e4m3[gate_up_instance] : kernels->expert_gate_up[gate_up_instance];
+    const uint32_t down_kernel = bytes ? kernels->expert_down_e4m3[down_instance] : kernels->expert_down[down_instance];
+    if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL ||
         kernels->activation_quantize == BACKEND_NO_KERNEL || kernels->expert_row_sum == BACKEND_NO_KERNEL) {
         REFUSE("%s: a kernel of the chain is not prepared", what);
         return STATUS_INVALID_ARGUMENT;
@@ -210,14 +226,14 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
                                                             description->row_output.byte_offset, down->output_size,
                                                             description->pairs_per_row};
     struct kernel_launch launches[LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT];
-    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_GATE_UP], kernels->expert_gate_up[gate_up_instance],
-                (gate_up->output_size + LINEAR_STRIP_OUTPUTS - 1u) / LINEAR_STRIP_OUTPUTS,
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_GATE_UP], gate_up_kernel,
+                (gate_up->output_size + strip_outputs - 1u) / strip_outputs,
                 description->job_count, 1, 64u * description->gate_up_slice_count, 0, &gate_up_record, sizeof gate_up_record);
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_QUANTIZE], kernels->activation_quantize,
                 (gate_up->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)pairs, 1,
                 LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
-    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_DOWN], kernels->expert_down[down_instance],
-                (down->output_size + LINEAR_STRIP_OUTPUTS - 1u) / LINEAR_STRIP_OUTPUTS, description->job_count, 1, 64u * description->down_slice_count, 0, &down_record, sizeof down_record);
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_DOWN], down_kernel,
+                (down->output_size + strip_outputs - 1u) / strip_outputs, description->job_count, 1, 64u * description->down_slice_count, 0, &down_record, sizeof down_record);
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_ROW_SUM], kernels->expert_row_sum,
                 (down->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)rows, 1,
                 LINEAR_ELEMENT_THREADS, 0, &row_sum_record, sizeof row_sum_record);

@@ -99,6 +99,53 @@ def fp4_matrix(seed, outputs, inputs, scale_code=120):
     return e2m1_lay_out(codes, scales)
 
 
+def e4m3_lay_out(codes, scales):
+    """codes uint8 [outputs][inputs] (E4M3 bytes), scales uint8 [ceil(outputs / 32)][inputs / 32] -> the stored bytes of
+    WEIGHT_FORMAT_E4M3_SCALED: bytes [tile][group][lane = 4 G + t][16], byte b of a lane is
+    W[16 tile + G + 8 (b % 2)][32 group + 8 (b / 4) + 2 t + (b / 2) % 2]; then the scales as they are."""
+    outputs, inputs = codes.shape
+    tiles, groups = outputs // 16, inputs // 32
+    # w[tile, b%2, G, group, b/4, t, (b/2)%2]
+    w = codes.reshape(tiles, 2, 8, groups, 4, 4, 2)
+    stored = w.transpose(0, 3, 2, 5, 4, 6, 1)  # [tile][group][G][t][b/4][(b/2)%2][b%2]
+    return np.concatenate([np.ascontiguousarray(stored).reshape(-1), np.ascontiguousarray(scales).reshape(-1)])
+
+
+def fp8_matrix_of_random_codes(seed, outputs, inputs, scale_code=113):
+    """Uniformly random E4M3 codes (every exponent as likely as any other; no NaN code) with E8M0 scales scale_code +
+    {0, 1} per 32 x 32 block: a stress of a sum's dynamic range, not a likeness of weights."""
+    raw = splitmix_words(seed, outputs * inputs // 8).view(np.uint8).reshape(outputs, inputs)
+    codes = np.where((raw & 0x7F) == 0x7F, raw & 0x80, raw).astype(np.uint8)
+    rows = (outputs + 31) // 32
+    scales = (scale_code + (splitmix_words(seed ^ 0x5CA1E, rows * inputs // 32) & np.uint64(1))).astype(np.uint8).reshape(rows, inputs // 32)
+    return e4m3_lay_out(codes, scales)
+
+
+E4M3_MAGNITUDES = np.array([(m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+                            for e in range(16) for m in range(8)][:127])
+
+
+def e4m3_nearest(values):
+    """Round-to-nearest-even E4M3 codes of float64 values, magnitudes clamped to 448."""
+    magnitudes = np.minimum(np.abs(values), 448.0)
+    middles = (E4M3_MAGNITUDES[:-1] + E4M3_MAGNITUDES[1:]) / 2.0
+    below = np.searchsorted(middles, magnitudes, side="left")   # a tie falls to the lower code here
+    tie = (below < 126) & (magnitudes == middles[np.minimum(below, 125)])
+    codes = np.where(tie & (below % 2 == 1), below + 1, below).astype(np.uint8)  # of two equally near, the even code
+    return codes | (np.signbit(values).astype(np.uint8) << 7)
+
+
+def fp8_matrix(seed, outputs, inputs, deviation=0.02):
+    """Weights N(0, deviation) as WEIGHT_FORMAT_E4M3_SCALED stores them: for every 32 x 32 block the smallest power of two
+    that brings the block's largest magnitude to at most 448, and the nearest E4M3 code of each weight over it."""
+    assert outputs % 32 == 0 and inputs % 32 == 0
+    weights = normals(seed, outputs * inputs).reshape(outputs // 32, 32, inputs // 32, 32) * deviation
+    largest = np.maximum(np.abs(weights).max(axis=(1, 3)), 1e-30)
+    exponents = np.ceil(np.log2(largest / 448.0)).astype(np.int64)
+    codes = e4m3_nearest(weights / (2.0 ** exponents)[:, None, :, None]).reshape(outputs, inputs)
+    return e4m3_lay_out(codes, (exponents + 127).astype(np.uint8))
+
+
 def fp4_moe_layer(config, hidden, inner, expert_count):
     base = SEED + (config << 20)
     matrices = [[fp4_matrix(base + 16 + 3 * e + 0, inner, hidden), fp4_matrix(base + 16 + 3 * e + 1, inner, hidden),

@@ -184,6 +184,10 @@ struct linear_kernels_record { /* include/anemone/linear.h:121-132 of the refere
     uint32_t trunk_linear_quantized_wide[LINEAR_SLICE_INSTANCES];
     uint32_t trunk_linear_bfloat16_wide[LINEAR_SLICE_INSTANCES];
     uint32_t trunk_linear_quantized_interleaved;
+    /* extension (no counterpart in the reference, whose expert kernels take E2M1 alone): the same two families
+     * for experts of WEIGHT_FORMAT_E4M3_SCALED */
+    uint32_t expert_gate_up_e4m3[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_down_e4m3[LINEAR_SLICE_INSTANCES];
 };
 MUST_CHECK result_status linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                 uint32_t arithmetic_class, struct linear_kernels_record *kernels_out);

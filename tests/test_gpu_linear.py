@@ -1,12 +1,16 @@
-"""GPU parity of the FP4 (E2M1 + E8M0 per 32) routed experts against the CPU oracle, through the C ABI: the activation
+"""GPU parity of the FP4 (E2M1 + E8M0 per 32) and FP8 (E4M3 + E8M0 per 32 x 32) routed experts against the CPU oracle, through the C ABI: the activation
 quantizer byte for byte (codes in lane order, exponents, operands), the products within the reference's own bound
 (tests/linear_reference.h:43-58 of the reference: |c - y| <= ulp_bf16(c)/2 + (T + B + S) 2^-24 m + B 2^-149, T = 64),
 the hidden step, the row sum bit for bit, and whole layers.
 
 The allowance T for the rounding inside the matrix instructions is 64 in the reference (instructions of 16 products on
-its cards). gfx950's v_mfma_scale_f32_16x16x128_f8f6f4 adds 128 products of four scale blocks in one instruction and
-rounds inside it in a way no document defines; on outputs whose products cancel to a thousandth of their magnitudes
-the card was measured up to 1.5e2 x 2^-24 of the magnitude sum from the exact value, so T = 256 here."""
+its cards). gfx950's v_mfma_scale_f32_16x16x128_f8f6f4 adds 128 products of four scale blocks in one instruction, and a
+probe of the instruction alone shows how: exact when the products' exponents lie close together, and up to 2.7e3 x 2^-24
+of the magnitude sum from the exact value (1.2e3 with E2M1 weights) when codes are drawn uniformly, every exponent as
+likely as any other: the products are cut a fixed number of places below the largest of the instruction, about
+2^-19 of it each. The sound bound of 128 products cut at 2^-19 of the largest is T = 4096, taken here for the stress
+of uniformly random E4M3 weights; weights and vectors of the benchmark's kind (Gaussian weights under their block
+scales, quantised Gaussian vectors) stay within T = 256."""
 import ctypes as C
 import sys
 
@@ -16,8 +20,9 @@ import pytest
 from _oracle import JOB_DTYPE, f32p, f64p, normals, orc, ptr, to_bf16, bf16_to_f32, u8p, u16p, u32p, u64p
 
 pytestmark = pytest.mark.gpu
-E2M1 = 3
-ALLOWANCE_GFX950 = 256.0
+E2M1, E4M3 = 3, 5
+ALLOWANCE_GFX950 = 256.0        # weights and vectors of the benchmark's kind
+ALLOWANCE_GFX950_STRESS = 4096.0  # uniformly random codes: 128 products cut at 2^-19 of the largest
 
 
 def say(*words):
@@ -44,12 +49,13 @@ def fresh_arena(card):
     yield
 
 
-def build(amd, card, hidden, inner, experts_n, picks, rows, seed, **more):
+def build(amd, card, hidden, inner, experts_n, picks, rows, seed, fmt=E2M1, stress=False, **more):
     from anemone_amd import workloads
-    matrices = [[workloads.fp4_matrix(seed * 1000 + 3 * e + 0, inner, hidden), workloads.fp4_matrix(seed * 1000 + 3 * e + 1, inner, hidden),
-                 workloads.fp4_matrix(seed * 1000 + 3 * e + 2, hidden, inner)] for e in range(experts_n)]
+    matrix = workloads.fp4_matrix if fmt == E2M1 else workloads.fp8_matrix_of_random_codes if stress else workloads.fp8_matrix
+    matrices = [[matrix(seed * 1000 + 3 * e + 0, inner, hidden), matrix(seed * 1000 + 3 * e + 1, inner, hidden),
+                 matrix(seed * 1000 + 3 * e + 2, hidden, inner)] for e in range(experts_n)]
     router = to_bf16(normals(seed + 5, experts_n * hidden) * 0.02).reshape(experts_n, hidden)
-    layer = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router, **more)
+    layer = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router, weight_format=fmt, **more)
     return layer, matrices, router
 
 
@@ -94,12 +100,14 @@ def test_quantizer_byte_for_byte(amd, card):
     assert np.array_equal(layer.read("operands", np.uint16).reshape(rows, width), operands)
 
 
-@pytest.mark.parametrize("slices", [1, 2, 4, 8])
-def test_products_within_the_reference_bound(amd, card, slices):
+@pytest.mark.parametrize("slices,fmt,stress", [(1, E2M1, False), (2, E2M1, False), (4, E2M1, False), (8, E2M1, False),
+                                               (1, E4M3, False), (2, E4M3, False), (8, E4M3, False), (4, E4M3, True)])
+def test_products_within_the_reference_bound(amd, card, slices, fmt, stress):
     """The down kernel is the plain product: each expert's gate matrix through it, against the exact block sums."""
-    say("products, slices", slices)
+    say("products, slices", slices, "format", fmt, "stress", stress)
     hidden, inner, experts_n, rows = 1024, 1024, 64, 6
-    layer, matrices, _ = build(amd, card, hidden, inner, experts_n, 1, rows, 2, gate_up_slices=1, down_slices=slices)
+    allowance = ALLOWANCE_GFX950_STRESS if stress else ALLOWANCE_GFX950
+    layer, matrices, _ = build(amd, card, hidden, inner, experts_n, 1, rows, 2, fmt=fmt, stress=stress, gate_up_slices=1, down_slices=slices)
     x = to_bf16(normals(7, rows * hidden).reshape(rows, hidden) * np.repeat([0.01, 1.0, 100.0, 1.0], hidden // 4))
     codes, exps, lane, _ = oracle_quantize(x)
     # pairs_per_row = 1: pair = row; three jobs over the first experts' GATE matrices (inner x hidden), as "down"
@@ -119,22 +127,22 @@ def test_products_within_the_reference_bound(amd, card, slices):
     for expert, members in plan:
         sums, mags = np.zeros((len(members), inner)), np.zeros((len(members), inner))
         member_codes, member_exps = np.ascontiguousarray(codes[members]), np.ascontiguousarray(exps[members])
-        assert orc.orc_linear_products(E2M1, inner, hidden, ptr(matrices[expert][0], u8p), 0, inner, ptr(member_codes, u8p),
+        assert orc.orc_linear_products(fmt, inner, hidden, ptr(matrices[expert][0], u8p), 0, inner, ptr(member_codes, u8p),
                                        ptr(member_exps, u8p), len(members), ptr(sums, f64p), ptr(mags, f64p)) == 0
         for i, row in enumerate(members):
             for o in range(inner):
-                assert orc.orc_linear_within_allowance(int(got[row, o]), sums[i, o], mags[i, o], hidden, slices, ALLOWANCE_GFX950), (expert, row, o)
+                assert orc.orc_linear_within_allowance(int(got[row, o]), sums[i, o], mags[i, o], hidden, slices, allowance), (expert, row, o)
             exact = to_bf16(sums[i].astype(np.float32))
             worst = max(worst, float(np.mean(exact != got[row, :inner])))
     say("  outputs that are not the exact sum rounded once: %.4f" % worst)
-    assert worst < 0.02
+    assert worst < (0.2 if stress else 0.02)
 
 
-@pytest.mark.parametrize("rows,live,picks", [(8, 8, 4), (3, 2, 8), (1, 1, 2)])
-def test_layer_against_oracle(amd, card, rows, live, picks):
-    say("layer", rows, live, picks)
+@pytest.mark.parametrize("rows,live,picks,fmt", [(8, 8, 4, E2M1), (3, 2, 8, E2M1), (1, 1, 2, E2M1), (8, 7, 4, E4M3), (2, 2, 8, E4M3)])
+def test_layer_against_oracle(amd, card, rows, live, picks, fmt):
+    say("layer", rows, live, picks, "format", fmt)
     hidden, inner, experts_n = 512, 256, 64
-    layer, matrices, router = build(amd, card, hidden, inner, experts_n, picks, rows, 4)
+    layer, matrices, router = build(amd, card, hidden, inner, experts_n, picks, rows, 4, fmt=fmt)
     x = to_bf16(normals(9, rows * hidden)).reshape(rows, hidden)
     layer.set_rows(x, live)
     card.run(layer.projection_launch())
@@ -154,7 +162,7 @@ def test_layer_against_oracle(amd, card, rows, live, picks):
     want = np.zeros((live, hidden), dtype=np.float32)
     want_hidden = np.zeros((live * picks, inner), dtype=np.uint16)
     want_pairs = np.zeros((live * picks, hidden), dtype=np.uint16)
-    orc.orc_linear_moe_layer(E2M1, ptr(np.ascontiguousarray(x[:live]), u16p), live, hidden, inner, picks,
+    orc.orc_linear_moe_layer(fmt, ptr(np.ascontiguousarray(x[:live]), u16p), live, hidden, inner, picks,
                              ptr(np.ascontiguousarray(experts[:live]), u32p), ptr(np.ascontiguousarray(weights[:live]), f32p),
                              experts_n, pointers, 10.0, ptr(want, f32p), ptr(want_hidden, u16p), ptr(want_pairs, u16p), 8)
     live_pairs = live * picks
@@ -174,7 +182,7 @@ def test_layer_against_oracle(amd, card, rows, live, picks):
     for pair in range(0, live_pairs, max(1, live_pairs // 6)):
         e = int(experts.reshape(-1)[pair])
         sums, mags = np.zeros(hidden), np.zeros(hidden)
-        orc.orc_linear_products(E2M1, hidden, inner, ptr(matrices[e][2], u8p), 0, hidden, ptr(np.ascontiguousarray(codes[pair]), u8p),
+        orc.orc_linear_products(fmt, hidden, inner, ptr(matrices[e][2], u8p), 0, hidden, ptr(np.ascontiguousarray(codes[pair]), u8p),
                                 ptr(np.ascontiguousarray(exps[pair]), u8p), 1, ptr(sums, f64p), ptr(mags, f64p))
         assert all(orc.orc_linear_within_allowance(int(pair_out[pair, o]), sums[o], mags[o], inner, 2, ALLOWANCE_GFX950) for o in range(hidden))
     # row sum: bit for bit from the card's pair outputs
