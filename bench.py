@@ -71,22 +71,25 @@ def calibrate(amd):
                       "GBps_read_plus_write": 2 * size / (min(times) * 1e-6) / 1e9}))
 
 
-def fp4_decode(amd, workloads, arguments):
-    """Secondary workload: the same layer shape with the original FP4 weights (E2M1 codes, one E8M0 scale per 32
-    inputs), a decode step of `--rows` tokens (32 by default): quantizer, router, and the four launches of the routed
-    experts. Sixteen distinct seeded experts are generated and laid at 256 distinct places of the arena."""
+def fp4_decode(amd, workloads, arguments, fp8=False):
+    """Secondary workloads: the same layer shape with the original FP4 weights (E2M1 codes, one E8M0 scale per 32
+    inputs) or FP8 weights (E4M3 codes, one E8M0 scale per 32 x 32), a decode step of `--rows` tokens (32 by default):
+    quantizer, router, and the four launches of the routed experts. A few distinct seeded experts are generated and laid
+    at 256 distinct places of the arena."""
     import ctypes as C
     rows = arguments.rows
-    distinct_generated = 16
-    base = workloads.SEED + (4 << 20)
-    trios = [[workloads.fp4_matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), workloads.fp4_matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
-              workloads.fp4_matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
+    distinct_generated = 4 if fp8 else 16
+    base = workloads.SEED + ((3 if fp8 else 4) << 20)
+    matrix = workloads.fp8_matrix if fp8 else workloads.fp4_matrix
+    trios = [[matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
+              matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
     matrices = [trios[e % distinct_generated] for e in range(EXPERTS)]
     router = workloads.to_bf16(workloads.normals(base + 2, EXPERTS * HIDDEN) * 0.02).reshape(EXPERTS, HIDDEN)
     x = workloads.activations(4, rows, HIDDEN)
-    card = amd.Card(5 << 30)
+    card = amd.Card((9 if fp8 else 5) << 30)
     layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router,
-                         gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices)
+                         gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices,
+                         weight_format=amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED)
     layer.set_rows(x, rows)
     wide = layer.wide_router() if rows > 8 else None  # more than eight rows: the wide select sorts the pairs by expert
     routing = [layer.select_launch(0)[0]] if wide is None else list(wide.launches())
@@ -110,7 +113,7 @@ def fp4_decode(amd, workloads, arguments):
     jobs = layer.jobs() if wide is None else wide.read("jobs", amd.JOB_DTYPE)
     live = jobs[jobs["row_count"] > 0]
     distinct = np.unique(live["expert"])
-    matrix_bytes = HIDDEN * INNER // 2 + HIDDEN * INNER // 32
+    matrix_bytes = HIDDEN * INNER + HIDDEN * INNER // 1024 if fp8 else HIDDEN * INNER // 2 + HIDDEN * INNER // 32
     gate_up_bytes = 2 * matrix_bytes * len(distinct)
     gate_up_us = float(per_launch[names.index("expert_gate_up")])
     down_us = float(per_launch[names.index("expert_down")])
@@ -118,13 +121,14 @@ def fp4_decode(amd, workloads, arguments):
         "metric": "MoE layer tok/s; decode HBM GB/s & prefill MFMA % of peak, 1 GPU",
         "value": rows * arguments.steps / seconds, "unit": "tok/s", "n_gpus": 1, "steps": arguments.steps,
         "warmup": arguments.warmup, "ms_per_step": 1000.0 * seconds / arguments.steps, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "fp4 x fp8 -> f32", "data": "synthetic",
-        "config": {"workload": "fp4_moe_decode: %d tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router, "
-                               "E2M1 weights with E8M0 scales per 32" % rows,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8 x fp8 -> f32" if fp8 else "fp4 x fp8 -> f32", "data": "synthetic",
+        "config": {"workload": "%s_moe_decode: %d tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router, %s"
+                               % ("fp8" if fp8 else "fp4", rows, "E4M3 weights with E8M0 scales per 32 x 32" if fp8 else
+                                  "E2M1 weights with E8M0 scales per 32"),
                    "distinct_experts": int(len(distinct)), "jobs": int(len(live)),
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "down_GBps": matrix_bytes * len(distinct) / (down_us * 1e-6) / 1e9},
-        "roofline": {"bound": "hbm", "kernel": "expert_gate_up_%d" % arguments.gate_up_slices,
+        "roofline": {"bound": "hbm", "kernel": "expert_gate_up_%s%d" % ("e4m3_" if fp8 else "", arguments.gate_up_slices),
                      "achieved": gate_up_bytes / (gate_up_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
@@ -142,7 +146,7 @@ def fp4_decode(amd, workloads, arguments):
         pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
         want = np.zeros((sample, HIDDEN), dtype=np.float32)
         start = time.perf_counter()
-        o.orc.orc_linear_moe_layer(3, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS,
+        o.orc.orc_linear_moe_layer(5 if fp8 else 3, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS,
                                    o.ptr(np.ascontiguousarray(experts_of[:sample]), o.u32p),
                                    o.ptr(np.ascontiguousarray(weights_of[:sample]), o.f32p), EXPERTS, pointers, 10.0,
                                    o.ptr(want, o.f32p), None, None, threads)
@@ -173,7 +177,7 @@ def main():
     if arguments.gpus != 1:
         print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
         sys.exit(2)
-    if arguments.workload not in ("exl3_decode", "fp4_decode"):
+    if arguments.workload not in ("exl3_decode", "fp4_decode", "fp8_decode"):
         print("unknown workload %s" % arguments.workload, file=sys.stderr)
         sys.exit(2)
 
@@ -183,8 +187,8 @@ def main():
     if arguments.calibrate:
         calibrate(amd)
         return
-    if arguments.workload == "fp4_decode":
-        fp4_decode(amd, workloads, arguments)
+    if arguments.workload in ("fp4_decode", "fp8_decode"):
+        fp4_decode(amd, workloads, arguments, fp8=arguments.workload == "fp8_decode")
         return
 
     widths, matrices, router = workloads.exl3_moe_layer(CONFIG, HIDDEN, INNER, EXPERTS)
