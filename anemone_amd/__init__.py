@@ -15,6 +15,7 @@ STATUS_DEVICE_ERROR, STATUS_TIMED_OUT, STATUS_UNSUPPORTED, STATUS_BUSY = 5, 6, 7
 WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED = 2, 3, 5
 ARITHMETIC_CLASS_GFX950 = 950
 BACKEND_NO_KERNEL = 0xFFFFFFFF
+ROUTER_SORT_ROWS = 384
 EXL3_EXPERT_LAUNCHES, EXL3_TC_LAUNCHES = 5, 5
 EXL3_TC_GATE_UP_SLICES, EXL3_TC_DOWN_SLICES = 8, 4
 AFFINITY_SQRT_SOFTPLUS, AFFINITY_SIGMOID = 0, 1
@@ -62,6 +63,14 @@ class Exl3ExpertRecord(C.Structure):
 
 class RowSumArguments(C.Structure):
     _fields_ = [("pair_output_offset", u64), ("row_output_offset", u64), ("width", u32), ("pairs_per_row", u32)]
+
+
+class Exl3TcpRecord(C.Structure):
+    _fields_ = [("picks_offset", u64), ("expert_offsets_offset", u64), ("hidden_offset", u64), ("workspace_offset", u64),
+                ("output_offset", u64), ("row_count", u32), ("intermediate", u32), ("bits_x2", u32), ("pass_", u32),
+                ("activation_limit", f32), ("rotation", u32), ("half_rows", u32), ("part", u32), ("step_offset", u64),
+                ("cone_layer", u32), ("two_blocks", u32), ("widths_offset", u64), ("hidden", u32), ("pairs_per_row", u32),
+                ("expert_count", u32), ("reserved_zero", u32)]
 
 
 class Exl3TcRecord(C.Structure):
@@ -160,6 +169,7 @@ def library():
             "exl3_tc_prepare": [C.POINTER(Exl3TcRecord), u64, vp, vp, launch_p],
             "exl3_tc_prepare_short": [C.POINTER(Exl3TcRecord), u64, vp, vp, launch_p],
             "exl3_tc_prepare_paired": [C.POINTER(Exl3TcRecord), u64, vp, vp, launch_p],
+            "exl3_tcp_prepare": [C.POINTER(Exl3TcpRecord), u64, vp, vp, launch_p, C.POINTER(u32)],
             "router_kernels_prepare": [vp, vp, C.POINTER(RouterKernels)],
             "router_select_prepare": [C.POINTER(RouterDescription), u64, C.POINTER(RouterKernels), launch_p],
             "router_projection_prepare": [C.POINTER(RouterProjectionDescription), u64, C.POINTER(RouterKernels), launch_p],
@@ -206,6 +216,23 @@ def card_count():
     count = u32(0)
     check(library().backend_hip_card_count(C.byref(count)), "card_count")
     return count.value
+
+
+def exl3_tcp_layout(rows, picks, experts, hidden, intermediate):
+    """The prefill workspace's parts (byte offsets) as exl3_tcp_layout_of of the library's records lays them."""
+    rounded = lambda n: (n + 255) // 256 * 256
+    pairs, blocks = rows * picks, (rows + ROUTER_SORT_ROWS - 1) // ROUTER_SORT_ROWS
+    layout = {"chunk_capacity": pairs // 128 + experts, "counts": 0}
+    layout["runs"] = layout["counts"] + rounded(blocks * experts * 4)
+    layout["header"] = layout["runs"] + rounded(experts * 8)
+    layout["chunks"] = layout["header"] + 256
+    layout["sorted"] = layout["chunks"] + rounded(layout["chunk_capacity"] * 16)
+    layout["place_of"] = layout["sorted"] + rounded(pairs * 4)
+    layout["operands"] = layout["place_of"] + rounded(pairs * 4)
+    layout["gate_up"] = layout["operands"] + rounded(2 * pairs * hidden * 2)
+    layout["down"] = layout["gate_up"] + rounded(2 * pairs * intermediate * 4)
+    layout["total"] = layout["down"] + rounded(pairs * hidden * 4)
+    return layout
 
 
 def exl3_tc_workspace_bytes(pairs, hidden, intermediate):
@@ -325,7 +352,6 @@ def launches_of(count):
     return (KernelLaunch * count)()
 
 
-ROUTER_SORT_ROWS = 384
 WIDE_PAIR_DTYPE = np.dtype([("pair_index", "<u4"), ("route_weight", "<f4")])
 WIDE_RUN_DTYPE = np.dtype([("first_pair", "<u4"), ("pair_count", "<u4")])
 WIDE_TILE_DTYPE = np.dtype([("gate_offset", "<u8"), ("up_offset", "<u8"), ("down_offset", "<u8"), ("first_pair", "<u4"),
@@ -420,11 +446,11 @@ class Exl3Layer:
         self.router_offset = card.place(router_weights_bf16) if router_weights_bf16 is not None else 0
         self.jobs_offset = card.reserve(self.pairs * 96)
         self.out_offset = card.reserve(rows * hidden * 4)
-        # chain scratch
-        self.scratch_offset = card.reserve(int(lib.exl3_scratch_byte_count(self.pairs, hidden)))
-        self.hidden_offset = card.reserve(self.pairs * inner * 2)
-        # fused decode workspace
-        self.workspace_offset = card.reserve(exl3_tc_workspace_bytes(self.pairs, hidden, inner))
+        if rows <= 64:  # the chain's scratch and the fused decode's workspace: steps of decode size
+            self.scratch_offset = card.reserve(int(lib.exl3_scratch_byte_count(self.pairs, hidden)))
+            self.hidden_offset = card.reserve(self.pairs * inner * 2)
+            self.workspace_offset = card.reserve(exl3_tc_workspace_bytes(self.pairs, hidden, inner))
+        self.tcp_workspace_offset = None
         self.kernels = RouterKernels()
         check(lib.router_kernels_prepare(backend_table(), card.handle, C.byref(self.kernels)), "router_kernels_prepare")
         self.router_kernels = self.kernels
@@ -512,6 +538,32 @@ class Exl3Layer:
         launches = launches_of(EXL3_TC_LAUNCHES)
         check(self.card.lib.exl3_tc_prepare(C.byref(record), self.card.arena_bytes, backend_table(), self.card.handle, launches), "exl3_tc_prepare")
         return launches
+
+    def wide_router(self):
+        width = self.uniform_width if self.uniform_width else int(self.widths.max())
+        return WideRouter(self, self.rows, WEIGHT_FORMAT_EXL3, Shape(self.I, self.H, width, 0), Shape(self.H, self.I, width, 0),
+                          widths=None if self.uniform_width else self.packed_widths)
+
+    def tcp_record(self, picks_offset):
+        if self.tcp_workspace_offset is None:
+            self.tcp_layout = exl3_tcp_layout(self.rows, self.P, self.E, self.H, self.I)
+            self.tcp_workspace_offset = self.card.reserve(self.tcp_layout["total"], 256)
+        r = Exl3TcpRecord()
+        r.picks_offset, r.expert_offsets_offset, r.hidden_offset = picks_offset, self.offsets_offset, self.x_offset
+        r.workspace_offset, r.output_offset = self.tcp_workspace_offset, self.out_offset
+        r.row_count, r.intermediate = self.rows, self.I
+        r.bits_x2 = {2: 4, 3: 6, 4: 8, 40: 5}.get(self.uniform_width, 8)
+        r.activation_limit = self.limit
+        r.widths_offset, r.hidden, r.pairs_per_row, r.expert_count = self.widths_offset, self.H, self.P, self.E
+        return r
+
+    def tcp_launches(self, picks_offset):
+        """The prefill form: seven launches from the picks [rows][P] of a wide select (or any table of that form)."""
+        record = self.tcp_record(picks_offset)
+        launches, count = launches_of(8), u32(0)
+        check(self.card.lib.exl3_tcp_prepare(C.byref(record), self.card.arena_bytes, backend_table(), self.card.handle, launches,
+                                             C.byref(count)), "exl3_tcp_prepare")
+        return (KernelLaunch * count.value)(*[launches[i] for i in range(count.value)])
 
     def jobs(self):
         return self.card.download(self.jobs_offset, self.pairs * 96).view(JOB_DTYPE)

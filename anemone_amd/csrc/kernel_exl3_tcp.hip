@@ -1,0 +1,449 @@
+/*
+ * kernel_exl3_tcp.hip -- the routed experts of one EXL3 layer for a prefill-sized call on gfx950: the pairs sorted by
+ * expert and the expert computation as a grouped GEMM on the matrix cores with the trellis decode fused into the
+ * weight tile loads. The counterpart of the reference's prefill form (source/kernel_exl3_tcp.cuh:7-15,
+ * include/anemone/exl3_tc_records.h:205-304): same record, same order of the work (route, operands, gate/up GEMM,
+ * activation and down operands, down GEMM, combine in route order).
+ *
+ * Arithmetic: the chain's (kernel_exl3.hip): fp16 operands from a float32 Hadamard transform, exactly decoded fp16
+ * weights, float32 MFMA sums over increasing k (one chain an output: the GEMM is not cut along k), SwiGLU in float32,
+ * a row's weighted pair outputs added in slot order. A pair's result does not depend on the other pairs of the call.
+ *
+ * The GEMM block: 256 outputs (four wavefronts of four 16 x 16 tiles) by one chunk of at most 128 pairs of one expert.
+ * A K step is 32 inputs: the chunk's operand columns (128 x 32 fp16, 8 KB) go from memory straight into LDS once a
+ * block and serve all four wavefronts; each wavefront streams the two tile rows of its own strip through a private LDS
+ * window, decodes each 16 x 32 weight tile once (eight weights a lane) and feeds it to eight MFMAs, one for every
+ * sixteen columns. Decoding is the vector unit's work (about 4.4 instructions a weight) and the products the matrix
+ * unit's (16 cycles an MFMA): at 128 columns the two take about the same time and overlap across the wavefronts of a
+ * SIMD.
+ */
+#include "exl3_device.cuh"
+#include "kernel_registry.h"
+#include "sort_device.cuh"
+
+#define TCP_SORT_THREADS 512u
+#define TCP_GEMM_WAVES 4u
+#define TCP_GEMM_THREADS (TCP_GEMM_WAVES * WAVE)
+#define TCP_WAVE_TILES 4u  /* output tiles of a wavefront: 64 outputs */
+#define TCP_COLUMN_BLOCKS (EXL3_TCP_CHUNK_PAIRS / 16u)
+#define TCP_STEP_INPUTS 32u
+#define TCP_STAGE_BYTES (EXL3_TCP_CHUNK_PAIRS * TCP_STEP_INPUTS * 2u) /* a K step of the chunk's operand columns */
+
+struct tcp_shape {
+    uint32_t hidden, intermediate, picks, pairs, experts;
+    struct exl3_tcp_layout layout;
+};
+
+__device__ static __forceinline__ tcp_shape tcp_shape_of(const struct exl3_tcp_record &record)
+{
+    tcp_shape shape;
+    shape.hidden = record.hidden;
+    shape.intermediate = record.intermediate;
+    shape.picks = record.pairs_per_row;
+    shape.pairs = record.row_count * record.pairs_per_row;
+    shape.experts = record.expert_count;
+    shape.layout = exl3_tcp_layout_of(record.row_count, record.pairs_per_row, record.expert_count, record.hidden, record.intermediate);
+    return shape;
+}
+
+__device__ static __forceinline__ uint32_t tcp_bits_x2(const struct exl3_tcp_record &record, const unsigned char *arena,
+                                                       uint32_t expert, uint32_t matrix)
+{
+    if (record.widths_offset == 0u) {
+        return record.bits_x2;
+    }
+    return exl3_bits_x2(exl3_width_of(((const uint32_t *)(arena + record.widths_offset))[expert], matrix));
+}
+
+__device__ static __forceinline__ uint64_t tcp_matrix_of(const struct exl3_tcp_record &record, const unsigned char *arena,
+                                                         uint32_t expert, uint32_t matrix)
+{
+    return ((const uint64_t *)(arena + record.expert_offsets_offset))[(uint64_t)expert * MODEL_EXPERT_MATRICES + matrix];
+}
+
+/* launch 0: grid (ceil(row_count / ROUTER_SORT_ROWS)): counts [block][experts] */
+extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_count(struct exl3_tcp_record record, unsigned char *arena)
+{
+    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    const tcp_shape shape = tcp_shape_of(record);
+    const uint32_t pairs = sort_block_picks((const struct router_pick *)(arena + record.picks_offset), shape.picks, blockIdx.x,
+                                            record.row_count, block_experts);
+    __syncthreads();
+    uint32_t *counts = (uint32_t *)(arena + record.workspace_offset + shape.layout.counts) + (uint64_t)blockIdx.x * shape.experts;
+    for (uint32_t expert = threadIdx.x; expert < shape.experts; expert += blockDim.x) {
+        uint32_t count = 0;
+        for (uint32_t index = 0; index < pairs; index++) {
+            count += block_experts[index] == expert ? 1u : 0u;
+        }
+        counts[expert] = count;
+    }
+}
+ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_count, exl3_tcp_record);
+
+/* launch 1: the same grid: the block's pairs placed (sorted [place] and place_of [pair]); block 0 also the runs, the
+ * chunks and their number */
+extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_place(struct exl3_tcp_record record, unsigned char *arena)
+{
+    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
+    __shared__ uint32_t chunk_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
+    const tcp_shape shape = tcp_shape_of(record);
+    const uint32_t experts = shape.experts;
+    const uint32_t blocks = (record.row_count + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
+    unsigned char *workspace = arena + record.workspace_offset;
+    const uint32_t pairs = sort_block_picks((const struct router_pick *)(arena + record.picks_offset), shape.picks, blockIdx.x,
+                                            record.row_count, block_experts);
+    const uint32_t *counts = (const uint32_t *)(workspace + shape.layout.counts);
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        uint32_t total = 0, lower = 0;
+        for (uint32_t block = 0; block < blocks; block++) {
+            const uint32_t count = counts[(uint64_t)block * experts + expert];
+            total += count;
+            lower += block < blockIdx.x ? count : 0u;
+        }
+        totals[expert] = total;
+        starts[expert] = total;
+        before[expert] = lower;
+        chunk_starts[expert] = (total + EXL3_TCP_CHUNK_PAIRS - 1u) / EXL3_TCP_CHUNK_PAIRS;
+    }
+    __syncthreads();
+    (void)block_exclusive_scan(starts, experts, scratch);
+    uint32_t *sorted = (uint32_t *)(workspace + shape.layout.sorted), *place_of = (uint32_t *)(workspace + shape.layout.place_of);
+    const uint32_t first_pair = blockIdx.x * ROUTER_SORT_ROWS * shape.picks;
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        uint32_t place = starts[expert] + before[expert];
+        for (uint32_t index = 0; index < pairs; index++) {
+            if (block_experts[index] == expert) {
+                sorted[place] = first_pair + index;
+                place_of[first_pair + index] = place;
+                place++;
+            }
+        }
+    }
+    if (blockIdx.x != 0u) {
+        return;
+    }
+    struct wide_run *runs = (struct wide_run *)(workspace + shape.layout.runs);
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        runs[expert] = (struct wide_run){starts[expert], totals[expert]};
+    }
+    const uint32_t used = block_exclusive_scan(chunk_starts, experts, scratch);
+    if (threadIdx.x == 0u) {
+        chunk_starts[experts] = used;
+        uint32_t *header = (uint32_t *)(workspace + shape.layout.header);
+        header[0] = used;
+        header[1] = header[2] = header[3] = 0u;
+    }
+    __syncthreads();
+    struct exl3_tcp_chunk *chunks = (struct exl3_tcp_chunk *)(workspace + shape.layout.chunks);
+    for (uint32_t chunk = threadIdx.x; chunk < shape.layout.chunk_capacity; chunk += blockDim.x) {
+        struct exl3_tcp_chunk value = {0, 0, 0, 0};
+        if (chunk < used) {
+            uint32_t low = 0, high = experts; /* the expert whose chunks hold this one */
+            while (high - low > 1u) {
+                const uint32_t middle = (low + high) / 2u;
+                if (chunk_starts[middle] <= chunk) {
+                    low = middle;
+                } else {
+                    high = middle;
+                }
+            }
+            const uint32_t taken = (chunk - chunk_starts[low]) * EXL3_TCP_CHUNK_PAIRS, left = totals[low] - taken;
+            value.expert = low;
+            value.first_pair = starts[low] + taken;
+            value.pair_count = left < EXL3_TCP_CHUNK_PAIRS ? left : EXL3_TCP_CHUNK_PAIRS;
+        }
+        chunks[chunk] = value;
+    }
+}
+ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_place, exl3_tcp_record);
+
+__device__ static __forceinline__ struct exl3_tcp_chunk tcp_chunk_of(const tcp_shape &shape, const unsigned char *workspace, uint32_t index)
+{
+    const uint32_t used = ((const uint32_t *)(workspace + shape.layout.header))[0];
+    struct exl3_tcp_chunk chunk = {0, 0, 0, 0};
+    if (index < used) {
+        chunk = ((const struct exl3_tcp_chunk *)(workspace + shape.layout.chunks))[index];
+    }
+    return chunk;
+}
+
+/* launch 2: grid (hidden / 128, chunk capacity, 2), block 64: the gate (z = 0) and up (z = 1) operands of a chunk's
+ * pairs, by place: fp16(H128(x suh) / sqrt(128)) */
+extern "C" __global__ void exl3_tcp_operands(struct exl3_tcp_record record, unsigned char *arena)
+{
+    const tcp_shape shape = tcp_shape_of(record);
+    unsigned char *workspace = arena + record.workspace_offset;
+    const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, blockIdx.y);
+    if (chunk.pair_count == 0u) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x, projection = blockIdx.z, channel = blockIdx.x * EXL3_TRANSFORM + lane;
+    const uint64_t matrix = tcp_matrix_of(record, arena, chunk.expert, projection);
+    const uint16_t *suh = (const uint16_t *)(arena + matrix + exl3_code_bytes(shape.hidden, shape.intermediate,
+                                                                               tcp_bits_x2(record, arena, chunk.expert, projection)));
+    const float s0 = half_bits_to_float(suh[channel]), s1 = half_bits_to_float(suh[channel + WAVE]);
+    const uint16_t *rows = (const uint16_t *)(arena + record.hidden_offset);
+    const uint32_t *sorted = (const uint32_t *)(workspace + shape.layout.sorted);
+    uint16_t *operands = (uint16_t *)(workspace + shape.layout.operands) + (uint64_t)projection * shape.pairs * shape.hidden;
+    for (uint32_t column = 0; column < chunk.pair_count; column++) {
+        const uint32_t place = chunk.first_pair + column;
+        const uint64_t row = sorted[place] / shape.picks;
+        float v0 = __fmul_rn(bf16_to_float(rows[row * shape.hidden + channel]), s0);
+        float v1 = __fmul_rn(bf16_to_float(rows[row * shape.hidden + channel + WAVE]), s1);
+        wave_hadamard128(v0, v1, lane);
+        uint16_t *out = operands + (uint64_t)place * shape.hidden;
+        out[channel] = float_to_half_bits(__fmul_rn(v0, EXL3_NORMALIZATION));
+        out[channel + WAVE] = float_to_half_bits(__fmul_rn(v1, EXL3_NORMALIZATION));
+    }
+}
+ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_operands, exl3_tcp_record);
+
+/* 16 bytes a lane from memory straight into LDS (lane L lands at lds_base + 16 L). Written as assembly so that the
+ * compiler keeps no book on it; the waits are this file's own. */
+__device__ static __forceinline__ void tcp_load_to_lds(const void *lane_address, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_address), "s"(lds_base) : "memory", "m0");
+}
+
+template <uint32_t count>
+__device__ static __forceinline__ void tcp_wait_loads()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(count) : "memory");
+}
+
+/* One wavefront of a GEMM block: its strip of TCP_WAVE_TILES output tiles against the chunk's columns, every K step.
+ *   codes      the matrix's trellis, [inputs / 16][out_tiles][tile_words] uint32; strip_tile: the strip's first tile
+ *   columns    the chunk's first operand row (fp16 [pair][inputs], rows of the chunk consecutive), count of them
+ *   stage      LDS address of the block's two operand stages; window: of this wavefront's two weight windows
+ * Lane L of an operand load lands at bytes 16 L of a 16-column group: column L / 4, slot L % 4, and asks for that
+ * column's 16-byte piece (L % 4) ^ ((column / 2) % 4) of the step, so that the readers of one piece of sixteen columns
+ * meet different banks. */
+template <uint32_t bits_x2>
+__device__ static __forceinline__ void
+tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t strip_tile, uint32_t inputs,
+              const half_t *__restrict__ columns, uint32_t column_count, uint32_t stage, uint32_t window, uint32_t wave,
+              uint32_t lane, bool strip_is_live, float4_t (&accumulator)[TCP_WAVE_TILES][TCP_COLUMN_BLOCKS])
+{
+    typedef exl3_width<bits_x2> W;
+    constexpr uint32_t row_bytes = TCP_WAVE_TILES * W::tile_bytes, row_lanes = row_bytes / 16u;
+    constexpr uint32_t window_bytes = 2u * row_bytes; /* the two tile rows of a K step */
+    static_assert(row_bytes % 16u == 0u && 2u * row_lanes <= WAVE, "a step's two strip rows are one load of the wavefront");
+    const uint32_t o = lane % 16u, g = lane / 16u, tau = g / 2u, q = g % 2u;
+    const exl3_run_place run0 = exl3_run_of<bits_x2>(o, 2u * q), run1 = exl3_run_of<bits_x2>(o, 2u * q + 1u);
+    const uint64_t row_stride = (uint64_t)out_tiles * W::tile_bytes; /* bytes between K tile rows */
+    /* weights: lanes 0 .. row_lanes - 1 carry the step's first tile row, the next row_lanes its second */
+    const bool carries = lane < 2u * row_lanes && strip_is_live;
+    const unsigned char *weight_source = (const unsigned char *)codes + (uint64_t)strip_tile * W::tile_bytes +
+                                         (lane / row_lanes) * row_stride + (lane % row_lanes) * 16u;
+    /* operands: this wavefront brings two of the step's eight 16-column groups: wave, wave + 4 */
+    const uint32_t load_column = lane / 4u, load_piece = (lane % 4u) ^ ((load_column / 2u) % 4u);
+    const unsigned char *operand_source[2]; /* a column past the chunk's last reads the first again: never stored */
+#pragma unroll
+    for (uint32_t part = 0; part < 2u; part++) {
+        const uint32_t column = 16u * (wave + TCP_GEMM_WAVES * part) + load_column;
+        operand_source[part] = (const unsigned char *)(columns + (uint64_t)(column < column_count ? column : 0u) * inputs) + load_piece * 16u;
+    }
+    /* where this lane reads its operand halves of column block j: column o, pieces 2 tau and 2 tau + 1, bytes 8 q .. */
+    const uint32_t swizzle = (o / 2u) % 4u;
+    const uint32_t read_low = o * 64u + ((2u * tau) ^ swizzle) * 16u + 8u * q, read_high = o * 64u + ((2u * tau + 1u) ^ swizzle) * 16u + 8u * q;
+#pragma unroll
+    for (uint32_t n = 0; n < TCP_WAVE_TILES; n++) {
+#pragma unroll
+        for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
+            accumulator[n][j] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+    const uint32_t steps = inputs / TCP_STEP_INPUTS;
+#define TCP_ISSUE(step, buffer)                                                                                       \
+    do {                                                                                                              \
+        _Pragma("unroll") for (uint32_t part = 0; part < 2u; part++)                                                  \
+        {                                                                                                             \
+            tcp_load_to_lds(operand_source[part] + (uint64_t)(step) * (TCP_STEP_INPUTS * 2u),                         \
+                            stage + (buffer) * TCP_STAGE_BYTES + (wave + TCP_GEMM_WAVES * part) * 1024u);             \
+        }                                                                                                             \
+        if (carries) {                                                                                                \
+            tcp_load_to_lds(weight_source + (uint64_t)(step) * 2u * row_stride, window + (buffer) * window_bytes);    \
+        }                                                                                                             \
+    } while (0)
+    TCP_ISSUE(0u, 0u);
+    for (uint32_t step = 0; step < steps; step++) {
+        const uint32_t buffer = step % 2u;
+        if (step + 1u < steps) {
+            TCP_ISSUE(step + 1u, buffer ^ 1u);
+        }
+        /* a wavefront asks for three loads a step (two column groups and its weights), two when its strip lies past
+         * the matrix: this step's have landed once nothing but the next step's is outstanding */
+        if (step + 1u >= steps) {
+            tcp_wait_loads<0>();
+        } else if (strip_is_live) {
+            tcp_wait_loads<3>();
+        } else {
+            tcp_wait_loads<2>();
+        }
+        __syncthreads(); /* the other wavefronts' column groups of this step have landed as well */
+        uint2_t b_low[TCP_COLUMN_BLOCKS], b_high[TCP_COLUMN_BLOCKS];
+        const uint32_t stage_base = stage + buffer * TCP_STAGE_BYTES;
+#pragma unroll
+        for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
+            b_low[j] = *(const __attribute__((address_space(3))) uint2_t *)(uintptr_t)(stage_base + j * 1024u + read_low);
+            b_high[j] = *(const __attribute__((address_space(3))) uint2_t *)(uintptr_t)(stage_base + j * 1024u + read_high);
+        }
+        if (strip_is_live) {
+            const uint32_t window_base = window + buffer * window_bytes + tau * row_bytes;
+#pragma unroll
+            for (uint32_t n = 0; n < TCP_WAVE_TILES; n++) {
+                const uint32_t tile_base = window_base + n * W::tile_bytes;
+                const uint32_t w00 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run0.word0);
+                const uint32_t w01 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run0.word1);
+                const uint32_t w10 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run1.word0);
+                const uint32_t w11 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run1.word1);
+                const uint32_t f0 = __builtin_amdgcn_alignbit(w00, w01, run0.shift);
+                const uint32_t f1 = __builtin_amdgcn_alignbit(w10, w11, run1.shift);
+                uint32_t a[4];
+                exl3_decode_run<bits_x2>(f0, a[0], a[2]); /* run 0: inputs 4 q + {0, 1} and {8, 9} */
+                exl3_decode_run<bits_x2>(f1, a[1], a[3]); /* run 1: inputs 4 q + {2, 3} and {10, 11} */
+                const half8_t weights = __builtin_bit_cast(half8_t, *(const uint4_t *)a);
+#pragma unroll
+                for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
+                    const uint32_t b[4] = {b_low[j].x, b_low[j].y, b_high[j].x, b_high[j].y};
+                    accumulator[n][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(weights, __builtin_bit_cast(half8_t, *(const uint4_t *)b),
+                                                                               accumulator[n][j], 0, 0, 0);
+                }
+            }
+        }
+        /* this step's stage and window are read (their values are in registers or used); the step after the next may
+         * fill them once every wavefront is past this point */
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+#undef TCP_ISSUE
+}
+
+/* launches 3 and 5: grid (ceil(outputs / 256), chunk capacity, projections), block 256.
+ * pass EXL3_TCP_GATE_AND_UP: z = 0 gate, 1 up, products [z][place][intermediate]; pass EXL3_TCP_DOWN: down,
+ * products [place][hidden]. */
+extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS) exl3_tcp_gemm(struct exl3_tcp_record record, unsigned char *arena)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char stages[2u * TCP_STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char windows[TCP_GEMM_WAVES][2u * 2u * TCP_WAVE_TILES * exl3_width<8>::tile_bytes];
+    const tcp_shape shape = tcp_shape_of(record);
+    unsigned char *workspace = arena + record.workspace_offset;
+    const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, blockIdx.y);
+    if (chunk.pair_count == 0u) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const bool down = record.pass == EXL3_TCP_DOWN;
+    const uint32_t projection = down ? 2u : blockIdx.z;
+    const uint32_t inputs = down ? shape.intermediate : shape.hidden, outputs = down ? shape.hidden : shape.intermediate;
+    const uint32_t bits_x2 = tcp_bits_x2(record, arena, chunk.expert, projection);
+    const uint32_t *codes = (const uint32_t *)(arena + tcp_matrix_of(record, arena, chunk.expert, projection));
+    const half_t *columns = (const half_t *)(workspace + shape.layout.operands) +
+                            ((uint64_t)(down ? 0u : projection) * shape.pairs + chunk.first_pair) * inputs;
+    float *products = down ? (float *)(workspace + shape.layout.down) + (uint64_t)chunk.first_pair * outputs
+                           : (float *)(workspace + shape.layout.gate_up) + ((uint64_t)projection * shape.pairs + chunk.first_pair) * outputs;
+    const uint32_t strip_tile = (blockIdx.x * EXL3_TCP_BLOCK_OUTPUTS) / EXL3_TILE + wave * TCP_WAVE_TILES;
+    const bool strip_is_live = strip_tile * EXL3_TILE < outputs;
+    const uint32_t stage = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)stages;
+    const uint32_t window = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)&windows[wave][0];
+    float4_t accumulator[TCP_WAVE_TILES][TCP_COLUMN_BLOCKS];
+    switch (bits_x2) {
+    case 4u: tcp_wave_gemm<4u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
+    case 5u: tcp_wave_gemm<5u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
+    case 6u: tcp_wave_gemm<6u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
+    case 8u: tcp_wave_gemm<8u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
+    default: return; /* no width of the format: the prepare refuses such a record */
+    }
+    if (!strip_is_live) {
+        return;
+    }
+    /* lane l of an accumulator: column l % 16 of its block, outputs 4 (l / 16) + i of its tile */
+#pragma unroll
+    for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
+        const uint32_t column = 16u * j + lane % 16u;
+        if (column < chunk.pair_count) {
+            float *out = products + (uint64_t)column * outputs + strip_tile * EXL3_TILE + 4u * (lane / 16u);
+#pragma unroll
+            for (uint32_t n = 0; n < TCP_WAVE_TILES; n++) {
+                *(float4_t *)(out + n * EXL3_TILE) = accumulator[n][j];
+            }
+        }
+    }
+}
+ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_gemm, exl3_tcp_record);
+
+/* launch 4: grid (intermediate / 128, chunk capacity), block 64: per pair of the chunk, gate = H128(gate products) /
+ * sqrt(128) x svh, up the same, the SwiGLU with its limit, x the down matrix's suh, H128 -> the fp16 down operand */
+extern "C" __global__ void exl3_tcp_activate(struct exl3_tcp_record record, unsigned char *arena)
+{
+    const tcp_shape shape = tcp_shape_of(record);
+    unsigned char *workspace = arena + record.workspace_offset;
+    const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, blockIdx.y);
+    if (chunk.pair_count == 0u) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x, channel = blockIdx.x * EXL3_TRANSFORM + lane;
+    const uint32_t H = shape.hidden, I = shape.intermediate, e = chunk.expert;
+    const uint16_t *gate_svh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, e, 0u) + exl3_code_bytes(H, I, tcp_bits_x2(record, arena, e, 0u))) + H;
+    const uint16_t *up_svh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, e, 1u) + exl3_code_bytes(H, I, tcp_bits_x2(record, arena, e, 1u))) + H;
+    const uint16_t *down_suh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, e, 2u) + exl3_code_bytes(I, H, tcp_bits_x2(record, arena, e, 2u)));
+    const float gs[2] = {half_bits_to_float(gate_svh[channel]), half_bits_to_float(gate_svh[channel + WAVE])};
+    const float us[2] = {half_bits_to_float(up_svh[channel]), half_bits_to_float(up_svh[channel + WAVE])};
+    const float ds[2] = {half_bits_to_float(down_suh[channel]), half_bits_to_float(down_suh[channel + WAVE])};
+    const float limit = record.activation_limit;
+    const float *gate_products = (const float *)(workspace + shape.layout.gate_up);
+    const float *up_products = gate_products + (uint64_t)shape.pairs * I;
+    uint16_t *operands = (uint16_t *)(workspace + shape.layout.operands);
+    for (uint32_t column = 0; column < chunk.pair_count; column++) {
+        const uint64_t place = chunk.first_pair + column;
+        float g[2] = {gate_products[place * I + channel], gate_products[place * I + channel + WAVE]};
+        float u[2] = {up_products[place * I + channel], up_products[place * I + channel + WAVE]};
+        wave_hadamard128(g[0], g[1], lane);
+        wave_hadamard128(u[0], u[1], lane);
+        float v[2];
+#pragma unroll
+        for (uint32_t i = 0; i < 2u; i++) {
+            const float gate = __fmul_rn(__fmul_rn(g[i], EXL3_NORMALIZATION), gs[i]);
+            const float up = __fmul_rn(__fmul_rn(u[i], EXL3_NORMALIZATION), us[i]);
+            const float bounded_gate = limit > 0.0f ? fminf(gate, limit) : gate;
+            const float bounded_up = limit > 0.0f ? fminf(fmaxf(up, -limit), limit) : up;
+            const float hidden = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
+            v[i] = __fmul_rn(hidden, ds[i]);
+        }
+        wave_hadamard128(v[0], v[1], lane);
+        uint16_t *operand = operands + place * I;
+        operand[channel] = float_to_half_bits(__fmul_rn(v[0], EXL3_NORMALIZATION));
+        operand[channel + WAVE] = float_to_half_bits(__fmul_rn(v[1], EXL3_NORMALIZATION));
+    }
+}
+ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_activate, exl3_tcp_record);
+
+/* launch 6: grid (hidden / 128, row_count), block 64: a row's pairs in slot order */
+extern "C" __global__ void exl3_tcp_combine(struct exl3_tcp_record record, unsigned char *arena)
+{
+    const tcp_shape shape = tcp_shape_of(record);
+    const unsigned char *workspace = arena + record.workspace_offset;
+    const uint32_t lane = threadIdx.x, channel = blockIdx.x * EXL3_TRANSFORM + lane, row = blockIdx.y;
+    const uint32_t H = shape.hidden, I = shape.intermediate;
+    const struct router_pick *picks = (const struct router_pick *)(arena + record.picks_offset) + (uint64_t)row * shape.picks;
+    const uint32_t *place_of = (const uint32_t *)(workspace + shape.layout.place_of);
+    const float *down = (const float *)(workspace + shape.layout.down);
+    float sum0 = 0.0f, sum1 = 0.0f;
+    for (uint32_t slot = 0; slot < shape.picks; slot++) {
+        const struct router_pick pick = picks[slot];
+        const uint64_t place = place_of[row * shape.picks + slot];
+        const uint16_t *svh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, pick.expert, 2u) +
+                                                 exl3_code_bytes(I, H, tcp_bits_x2(record, arena, pick.expert, 2u))) + I;
+        float v0 = down[place * H + channel], v1 = down[place * H + channel + WAVE];
+        wave_hadamard128(v0, v1, lane);
+        const float y0 = __fmul_rn(__fmul_rn(__fmul_rn(v0, EXL3_NORMALIZATION), half_bits_to_float(svh[channel])), pick.route_weight);
+        const float y1 = __fmul_rn(__fmul_rn(__fmul_rn(v1, EXL3_NORMALIZATION), half_bits_to_float(svh[channel + WAVE])), pick.route_weight);
+        sum0 = __fadd_rn(sum0, y0);
+        sum1 = __fadd_rn(sum1, y1);
+    }
+    float *out = (float *)(arena + record.output_offset) + (uint64_t)row * H;
+    out[channel] = sum0;
+    out[channel + WAVE] = sum1;
+}
+ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_combine, exl3_tcp_record);

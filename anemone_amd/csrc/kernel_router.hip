@@ -18,6 +18,7 @@
  */
 #include "exl3_device.cuh" /* det_expf, bf16_to_float */
 #include "kernel_registry.h"
+#include "sort_device.cuh"
 
 #define SELECT_THREADS (LINEAR_MAXIMUM_ROWS * WAVE) /* a wavefront for each row */
 #define PROJECTION_CHAINS 32u
@@ -382,13 +383,7 @@ ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_select, router_wide_arguments);
 __device__ static __forceinline__ uint32_t wide_block_picks(const struct router_wide_arguments &arguments, const unsigned char *arena,
                                                             uint32_t block, uint32_t live_rows, uint32_t *experts_out)
 {
-    const uint32_t first_row = block * ROUTER_SORT_ROWS;
-    const uint32_t rows = live_rows <= first_row ? 0u : live_rows - first_row < ROUTER_SORT_ROWS ? live_rows - first_row : ROUTER_SORT_ROWS;
-    const struct router_pick *picks = (const struct router_pick *)(arena + arguments.picks_offset) + (uint64_t)first_row * arguments.pick_count;
-    for (uint32_t index = threadIdx.x; index < rows * arguments.pick_count; index += blockDim.x) {
-        experts_out[index] = picks[index].expert;
-    }
-    return rows * arguments.pick_count;
+    return sort_block_picks((const struct router_pick *)(arena + arguments.picks_offset), arguments.pick_count, block, live_rows, experts_out);
 }
 
 /* grid (ceil(row_count / ROUTER_SORT_ROWS)): counts [block][E] */
@@ -412,35 +407,6 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_count, router_wide_arguments);
-
-/* exclusive prefix sums of values[0 .. count) in LDS, count <= ROUTER_MOST_EXPERTS, by the whole block; total returned */
-__device__ static __forceinline__ uint32_t block_exclusive_scan(uint32_t *values, uint32_t count, uint32_t *scratch)
-{
-    /* count is small (at most 512): Hillis-Steele over two buffers */
-    uint32_t *from = values, *to = scratch;
-    for (uint32_t step = 1; step < count; step *= 2u) {
-        for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
-            to[i] = from[i] + (i >= step ? from[i - step] : 0u);
-        }
-        __syncthreads();
-        uint32_t *swap = from;
-        from = to;
-        to = swap;
-    }
-    const uint32_t total = count == 0u ? 0u : from[count - 1u];
-    __syncthreads();
-    for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
-        to[i] = i == 0u ? 0u : from[i - 1u];
-    }
-    __syncthreads();
-    if (to != values) {
-        for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
-            values[i] = to[i];
-        }
-        __syncthreads();
-    }
-    return total;
-}
 
 /* grid as the count's: the sorted pairs of the block's rows; block 0 also the runs and every tile */
 extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)

@@ -1,0 +1,56 @@
+/*
+ * sort_device.cuh -- what the sorts of pairs by expert share (the router's wide select and the prefill form of the
+ * EXL3 experts): a block's picked experts into LDS, and a block-wide exclusive prefix sum. No atomic operation
+ * anywhere: a thread owns an expert and walks the block's picks in row order.
+ */
+#ifndef SORT_DEVICE_CUH
+#define SORT_DEVICE_CUH
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "anemone_records.h"
+
+/* the picked experts of the live rows of block `block` of ROUTER_SORT_ROWS rows, into LDS; returns their number */
+__device__ static __forceinline__ uint32_t sort_block_picks(const struct router_pick *all_picks, uint32_t picks_per_row,
+                                                            uint32_t block, uint32_t live_rows, uint32_t *experts_out)
+{
+    const uint32_t first_row = block * ROUTER_SORT_ROWS;
+    const uint32_t rows = live_rows <= first_row ? 0u : live_rows - first_row < ROUTER_SORT_ROWS ? live_rows - first_row : ROUTER_SORT_ROWS;
+    const struct router_pick *picks = all_picks + (uint64_t)first_row * picks_per_row;
+    for (uint32_t index = threadIdx.x; index < rows * picks_per_row; index += blockDim.x) {
+        experts_out[index] = picks[index].expert;
+    }
+    return rows * picks_per_row;
+}
+
+/* exclusive prefix sums of values[0 .. count) in LDS, count <= ROUTER_MOST_EXPERTS, by the whole block; total returned */
+__device__ static __forceinline__ uint32_t block_exclusive_scan(uint32_t *values, uint32_t count, uint32_t *scratch)
+{
+    /* count is small (at most 512): Hillis-Steele over two buffers */
+    uint32_t *from = values, *to = scratch;
+    for (uint32_t step = 1; step < count; step *= 2u) {
+        for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
+            to[i] = from[i] + (i >= step ? from[i - step] : 0u);
+        }
+        __syncthreads();
+        uint32_t *swap = from;
+        from = to;
+        to = swap;
+    }
+    const uint32_t total = count == 0u ? 0u : from[count - 1u];
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
+        to[i] = i == 0u ? 0u : from[i - 1u];
+    }
+    __syncthreads();
+    if (to != values) {
+        for (uint32_t i = threadIdx.x; i < count; i += blockDim.x) {
+            values[i] = to[i];
+        }
+        __syncthreads();
+    }
+    return total;
+}
+
+#endif

@@ -123,3 +123,120 @@ result_status exl3_tc_prepare_paired(const struct exl3_tc_record *record, uint64
 {
     return tc_prepare(record, arena_byte_count, backend, card, launches_out);
 }
+
+/*
+ * The prefill form (include/anemone/exl3_tc.h:40-59 of the reference): seven launches of one record.
+ *
+ *   launch      kernel              grid                                             block
+ *   count       exl3_tcp_count      (ceil(rows / 384), 1, 1)                         512
+ *   place       exl3_tcp_place      (ceil(rows / 384), 1, 1)                         512
+ *   operands    exl3_tcp_operands   (hidden / 128, chunk capacity, 2)                64
+ *   gate/up     exl3_tcp_gemm       (ceil(intermediate / 256), chunk capacity, 2)    256   pass EXL3_TCP_GATE_AND_UP
+ *   activate    exl3_tcp_activate   (intermediate / 128, chunk capacity, 1)          64
+ *   down        exl3_tcp_gemm       (ceil(hidden / 256), chunk capacity, 1)          256   pass EXL3_TCP_DOWN
+ *   combine     exl3_tcp_combine    (hidden / 128, rows, 1)                          64
+ * chunk capacity = pairs / 128 + experts: an expert's pairs cut in chunks of 128, the last ragged.
+ */
+static result_status tcp_prepare(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
+                                 const struct backend_operations *backend, struct device_card *card,
+                                 struct kernel_launch launches_out[EXL3_TCP_MOST_LAUNCHES], uint32_t *launch_count_out)
+{
+    static const char what[] = "EXL3 prefill";
+    if (record == NULL || backend == NULL || backend->kernel_prepare == NULL || card == NULL || launches_out == NULL ||
+        launch_count_out == NULL) {
+        REFUSE("%s: a missing argument", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint32_t H = record->hidden, I = record->intermediate, P = record->pairs_per_row, E = record->expert_count;
+    if (record->row_count == 0 || record->row_count > EXL3_TCP_MOST_ROWS || record->pass != 0 || record->reserved_zero != 0 ||
+        P == 0 || P > ROUTER_MOST_PICKS || E == 0 || E > ROUTER_MOST_EXPERTS || !(record->activation_limit >= 0.0f) ||
+        !isfinite(record->activation_limit)) {
+        REFUSE("%s: 1 to %u rows of 1 to %u pairs, 1 to %u experts, pass 0, an activation limit of zero (none) or above", what,
+               EXL3_TCP_MOST_ROWS, ROUTER_MOST_PICKS, ROUTER_MOST_EXPERTS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (record->rotation != 0 || record->half_rows != 0 || record->part != 0 || record->cone_layer != 0 || record->two_blocks != 0) {
+        REFUSE("%s: rotation, halves of rows, cone layers and the two-blocks forms are forms this library does not build", what);
+        return STATUS_UNSUPPORTED;
+    }
+    if (H == 0 || I == 0 || I % EXL3_TRANSFORM != 0 || H % EXL3_TRANSFORM != 0) {
+        REFUSE("%s: hidden %u and intermediate %u: multiples of 128", what, H, I);
+        return STATUS_UNSUPPORTED;
+    }
+    const bool mixed = record->widths_offset != 0;
+    if (!mixed && (record->bits_x2 != 4u && record->bits_x2 != 5u && record->bits_x2 != 6u && record->bits_x2 != 8u)) {
+        REFUSE("%s: bits_x2 %u: this build decodes 4, 5, 6 and 8", what, record->bits_x2);
+        return exl3_width_name(record->bits_x2) == NULL && (record->bits_x2 == 0 || record->bits_x2 > 16u)
+                   ? STATUS_INVALID_ARGUMENT
+                   : STATUS_UNSUPPORTED;
+    }
+    const uint64_t rows = record->row_count, pairs = rows * P;
+    const struct exl3_tcp_layout layout = exl3_tcp_layout_of(rows, P, E, H, I);
+    if (layout.chunk_capacity > MOST_GRID_ROWS) {
+        REFUSE("%s: %u chunks of pairs are more than a grid holds", what, layout.chunk_capacity);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct checked_range ranges[] = {
+        {"the picks", {record->picks_offset, pairs * sizeof(struct router_pick)}, pairs * sizeof(struct router_pick), false},
+        {"the expert offsets", {record->expert_offsets_offset, (uint64_t)E * MODEL_EXPERT_MATRICES * 8u},
+         (uint64_t)E * MODEL_EXPERT_MATRICES * 8u, false},
+        {"the rows", {record->hidden_offset, rows * H * 2u}, rows * H * 2u, false},
+        {"the workspace", {record->workspace_offset, layout.total}, layout.total, false},
+        {"the output", {record->output_offset, rows * H * 4u}, rows * H * 4u, false},
+    };
+    if (!ranges_are_valid(what, ranges, 5, arena_byte_count) || record->workspace_offset % 256u != 0 ||
+        (mixed && record->widths_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0)) {
+        if (record->workspace_offset % 256u != 0) {
+            REFUSE("%s: the workspace begins off a multiple of 256", what);
+        }
+        return STATUS_INVALID_ARGUMENT;
+    }
+    static const char *const names[EXL3_TCP_LAUNCHES] = {"exl3_tcp_count",    "exl3_tcp_place", "exl3_tcp_operands", "exl3_tcp_gemm",
+                                                         "exl3_tcp_activate", "exl3_tcp_gemm",  "exl3_tcp_combine"};
+    const uint32_t blocks = (uint32_t)((rows + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS), capacity = layout.chunk_capacity;
+    const uint32_t grid_x[EXL3_TCP_LAUNCHES] = {blocks, blocks, H / 128u, (I + EXL3_TCP_BLOCK_OUTPUTS - 1u) / EXL3_TCP_BLOCK_OUTPUTS,
+                                                I / 128u, (H + EXL3_TCP_BLOCK_OUTPUTS - 1u) / EXL3_TCP_BLOCK_OUTPUTS, H / 128u};
+    const uint32_t grid_y[EXL3_TCP_LAUNCHES] = {1u, 1u, capacity, capacity, capacity, capacity, record->row_count};
+    const uint32_t grid_z[EXL3_TCP_LAUNCHES] = {1u, 1u, 2u, 2u, 1u, 1u, 1u};
+    const uint32_t threads[EXL3_TCP_LAUNCHES] = {512u, 512u, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS};
+    struct kernel_launch launches[EXL3_TCP_LAUNCHES];
+    for (uint32_t index = 0; index < EXL3_TCP_LAUNCHES; index++) {
+        uint32_t kernel = BACKEND_NO_KERNEL;
+        const result_status prepared = backend->kernel_prepare(card, EXL3_TCP_KERNEL_FILE, names[index], sizeof *record, &kernel);
+        if (prepared != STATUS_OK) {
+            return prepared;
+        }
+        if (kernel == BACKEND_NO_KERNEL) {
+            return STATUS_UNSUPPORTED;
+        }
+        struct exl3_tcp_record stamped = *record;
+        stamped.pass = index == EXL3_TCP_DOWN_LAUNCH ? EXL3_TCP_DOWN : EXL3_TCP_GATE_AND_UP;
+        launch_fill(&launches[index], kernel, grid_x[index], grid_y[index], grid_z[index], threads[index], 0, &stamped, sizeof stamped);
+    }
+    memcpy(launches_out, launches, sizeof launches);
+    *launch_count_out = EXL3_TCP_LAUNCHES;
+    return STATUS_OK;
+}
+
+result_status exl3_tcp_prepare(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
+                               const struct backend_operations *backend, struct device_card *card,
+                               struct kernel_launch launches_out[EXL3_TCP_MOST_LAUNCHES], uint32_t *launch_count_out)
+{
+    return tcp_prepare(record, arena_byte_count, backend, card, launches_out, launch_count_out);
+}
+
+/* the reference's _base and _hybrid forms pick between two GEMM forms of its 640-column geometry that give the same
+ * bits; here there is one form */
+result_status exl3_tcp_prepare_base(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
+                                    const struct backend_operations *backend, struct device_card *card,
+                                    struct kernel_launch launches_out[EXL3_TCP_MOST_LAUNCHES], uint32_t *launch_count_out)
+{
+    return tcp_prepare(record, arena_byte_count, backend, card, launches_out, launch_count_out);
+}
+
+result_status exl3_tcp_prepare_hybrid(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
+                                      const struct backend_operations *backend, struct device_card *card,
+                                      struct kernel_launch launches_out[EXL3_TCP_MOST_LAUNCHES], uint32_t *launch_count_out)
+{
+    return tcp_prepare(record, arena_byte_count, backend, card, launches_out, launch_count_out);
+}

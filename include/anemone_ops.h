@@ -87,6 +87,22 @@ MUST_CHECK result_status exl3_tc_prepare_paired(const struct exl3_tc_record *rec
                                                 const struct backend_operations *backend, struct device_card *card,
                                                 struct kernel_launch launches_out[EXL3_TC_LAUNCHES]);
 
+/* The prefill form (include/anemone/exl3_tc.h:40-59 of the reference): fills launches_out and *launch_count_out
+ * (EXL3_TCP_LAUNCHES here). The reference's _base and _hybrid choose between two GEMM forms of the same bits; this
+ * library has one form behind all three names. */
+MUST_CHECK result_status exl3_tcp_prepare(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
+                                          const struct backend_operations *backend, struct device_card *card,
+                                          struct kernel_launch launches_out[EXL3_TCP_MOST_LAUNCHES],
+                                          uint32_t *launch_count_out);
+MUST_CHECK result_status exl3_tcp_prepare_base(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
+                                               const struct backend_operations *backend, struct device_card *card,
+                                               struct kernel_launch launches_out[EXL3_TCP_MOST_LAUNCHES],
+                                               uint32_t *launch_count_out);
+MUST_CHECK result_status exl3_tcp_prepare_hybrid(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
+                                                 const struct backend_operations *backend, struct device_card *card,
+                                                 struct kernel_launch launches_out[EXL3_TCP_MOST_LAUNCHES],
+                                                 uint32_t *launch_count_out);
+
 /* ---- router ---- */
 struct router_kernels_record {
     uint32_t select;

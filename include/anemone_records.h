@@ -322,6 +322,95 @@ ANEMONE_INLINE uint64_t exl3_tc_workspace_bytes(uint64_t pairs, uint64_t hidden,
            exl3_tc_down_bytes(pairs, hidden);
 }
 
+/* ---- EXL3 prefill: the routed experts as a grouped GEMM (include/anemone/exl3_tc_records.h:205-304 of the
+ * reference: struct exl3_tcp_record and its workspace) ----
+ * Seven launches of one record: the pairs of each expert counted in blocks of ROUTER_SORT_ROWS rows; every pair placed
+ * (sorted by expert, rows ascending), the runs and the chunks of at most EXL3_TCP_CHUNK_PAIRS pairs of one expert; the
+ * gate and up operands of every placed pair; the gate/up GEMM; the activation and the down operands; the down GEMM;
+ * the combine of a row's pairs in slot order. */
+#define EXL3_TCP_KERNEL_FILE "kernel_exl3_tcp"
+#define EXL3_TCP_CHUNK_PAIRS 128u  /* columns of one GEMM block: pairs of one expert */
+#define EXL3_TCP_BLOCK_OUTPUTS 256u /* outputs of one GEMM block: four wavefronts of four tiles */
+#define EXL3_TCP_LAUNCHES 7u
+#define EXL3_TCP_MOST_LAUNCHES 8u  /* the reference's bound of its own forms */
+#define EXL3_TCP_MOST_ROWS 16384u
+enum exl3_tcp_pass { EXL3_TCP_GATE_AND_UP = 0, EXL3_TCP_GATE = 1, EXL3_TCP_UP = 2, EXL3_TCP_DOWN = 3 };
+enum exl3_tcp_launch {
+    EXL3_TCP_COUNT_LAUNCH = 0,
+    EXL3_TCP_PLACE_LAUNCH = 1,
+    EXL3_TCP_OPERANDS_LAUNCH = 2,
+    EXL3_TCP_GATE_UP_LAUNCH = 3,
+    EXL3_TCP_ACTIVATE_LAUNCH = 4,
+    EXL3_TCP_DOWN_LAUNCH = 5,
+    EXL3_TCP_COMBINE_LAUNCH = 6
+};
+
+struct exl3_tcp_record {
+    uint64_t picks_offset;          /* read: struct router_pick [row_count][pairs_per_row] */
+    uint64_t expert_offsets_offset; /* read: uint64 [expert_count][3] */
+    uint64_t hidden_offset;         /* read: bf16 [row_count][hidden] */
+    uint64_t workspace_offset;      /* scratch: exl3_tcp_layout_of(...).total bytes, 256-aligned */
+    uint64_t output_offset;         /* written: float32 [row_count][hidden] */
+    uint32_t row_count;
+    uint32_t intermediate;
+    uint32_t bits_x2;               /* the one width as 2 K, unless widths_offset names per-matrix widths */
+    uint32_t pass;                  /* the GEMM launches: enum exl3_tcp_pass; the others 0 */
+    float activation_limit;
+    uint32_t rotation;              /* must be 0: tensor-parallel features of the reference, not built */
+    uint32_t half_rows;             /* must be 0 */
+    uint32_t part;                  /* must be 0 */
+    uint64_t step_offset;           /* unused (cone layers are outside this path) */
+    uint32_t cone_layer;            /* must be 0 */
+    uint32_t two_blocks;            /* must be 0 */
+    /* extension */
+    uint64_t widths_offset;
+    uint32_t hidden;
+    uint32_t pairs_per_row;
+    uint32_t expert_count;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(exl3_tcp_record, 112);
+
+struct exl3_tcp_chunk {
+    uint32_t expert;
+    uint32_t first_pair; /* place of its first pair among the sorted pairs */
+    uint32_t pair_count; /* 1 to EXL3_TCP_CHUNK_PAIRS */
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(exl3_tcp_chunk, 16);
+
+/* The workspace, byte offsets from its start, every part 256-aligned: uint32 counts [blocks][experts]; struct wide_run
+ * runs [experts]; a header of four uint32 (the chunks in use first); struct exl3_tcp_chunk chunks [capacity]; uint32
+ * sorted [pairs] (the pair at each place); uint32 place_of [pairs]; fp16 operands [2][pairs][hidden], by place (later
+ * the down operands [pairs][intermediate]); float32 gate and up products [2][pairs][intermediate]; float32 down
+ * products [pairs][hidden]. */
+struct exl3_tcp_layout {
+    uint64_t counts, runs, header, chunks, sorted, place_of, operands, gate_up, down, total;
+    uint32_t chunk_capacity, reserved;
+};
+ANEMONE_INLINE uint64_t exl3_tcp_rounded(uint64_t bytes)
+{
+    return (bytes + 255u) / 256u * 256u;
+}
+ANEMONE_INLINE struct exl3_tcp_layout exl3_tcp_layout_of(uint64_t rows, uint64_t picks, uint64_t experts, uint64_t hidden,
+                                                         uint64_t intermediate)
+{
+    struct exl3_tcp_layout layout = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const uint64_t pairs = rows * picks, blocks = (rows + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
+    layout.chunk_capacity = (uint32_t)(pairs / EXL3_TCP_CHUNK_PAIRS + experts);
+    layout.counts = 0;
+    layout.runs = layout.counts + exl3_tcp_rounded(blocks * experts * 4u);
+    layout.header = layout.runs + exl3_tcp_rounded(experts * 8u);
+    layout.chunks = layout.header + 256u;
+    layout.sorted = layout.chunks + exl3_tcp_rounded((uint64_t)layout.chunk_capacity * 16u);
+    layout.place_of = layout.sorted + exl3_tcp_rounded(pairs * 4u);
+    layout.operands = layout.place_of + exl3_tcp_rounded(pairs * 4u);
+    layout.gate_up = layout.operands + exl3_tcp_rounded(2u * pairs * hidden * 2u);
+    layout.down = layout.gate_up + exl3_tcp_rounded(2u * pairs * intermediate * 4u);
+    layout.total = layout.down + exl3_tcp_rounded(pairs * hidden * 4u);
+    return layout;
+}
+
 /* ---- FP4 / FP8 expert linears ---- */
 #define KERNEL_FILE_ACTIVATION_QUANTIZE "kernel_activation_quantize"
 #define KERNEL_FILE_EXPERT_LINEAR "kernel_expert_linear"
