@@ -16,6 +16,7 @@ WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED = 2, 3,
 ARITHMETIC_CLASS_GFX950 = 950
 BACKEND_NO_KERNEL = 0xFFFFFFFF
 ROUTER_SORT_ROWS = 384
+EXL3_TCP_CHUNK_PAIRS = 128
 EXL3_EXPERT_LAUNCHES, EXL3_TC_LAUNCHES = 5, 5
 EXL3_TC_GATE_UP_SLICES, EXL3_TC_DOWN_SLICES = 8, 4
 AFFINITY_SQRT_SOFTPLUS, AFFINITY_SIGMOID = 0, 1
@@ -222,7 +223,7 @@ def exl3_tcp_layout(rows, picks, experts, hidden, intermediate):
     """The prefill workspace's parts (byte offsets) as exl3_tcp_layout_of of the library's records lays them."""
     rounded = lambda n: (n + 255) // 256 * 256
     pairs, blocks = rows * picks, (rows + ROUTER_SORT_ROWS - 1) // ROUTER_SORT_ROWS
-    layout = {"chunk_capacity": pairs // 128 + experts, "counts": 0}
+    layout = {"chunk_capacity": pairs // EXL3_TCP_CHUNK_PAIRS + experts, "counts": 0}
     layout["runs"] = layout["counts"] + rounded(blocks * experts * 4)
     layout["header"] = layout["runs"] + rounded(experts * 8)
     layout["chunks"] = layout["header"] + 256

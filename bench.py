@@ -161,12 +161,100 @@ def fp4_decode(amd, workloads, arguments, fp8=False):
     print(json.dumps(result))
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def exl3_prefill(amd, workloads, arguments):
+    """Secondary workload: the EXL3 layer of the main workload for a prefill of `--rows` tokens (4096 by default), the
+    router biased so that the experts' load is Zipf-skewed (s = 1.1 over a seeded permutation of the experts; the bias
+    is zipf_strength x ln(pmf), scaled to the spread of the sigmoid affinities so that load, not only rank, is skewed):
+    router projection, the picks of every row, and the seven launches of the prefill form (sort by expert, operands,
+    gate/up GEMM with the trellis decode fused into the tile loads, activation, down GEMM, combine)."""
+    rows = arguments.rows if arguments.rows != 32 else 4096
+    widths, matrices, router = workloads.exl3_moe_layer(CONFIG, HIDDEN, INNER, EXPERTS)
+    x = workloads.activations(2, rows, HIDDEN)
+    ranks = np.argsort(workloads.uniform01(workloads.SEED + (2 << 20) + 7, EXPERTS))
+    bias = np.zeros(EXPERTS, dtype=np.float32)
+    pmf = (1.0 + np.arange(EXPERTS)) ** -1.1
+    bias[ranks] = (arguments.zipf_strength * np.log(pmf / pmf.max())).astype(np.float32)
+    card = amd.Card(10 << 30)
+    layer = amd.Exl3Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, widths, router_weights_bf16=router, bias=bias,
+                          affinity_kind=amd.AFFINITY_SIGMOID, route_scale=1.5, limit=10.0)
+    layer.set_rows(x, rows)
+    wide = layer.wide_router()
+    parts = [layer.projection_launch()[0], wide.launches()[0]] + list(layer.tcp_launches(wide.ranges["picks"].byte_offset))
+    step = amd.launches_of(len(parts))
+    for i, launch in enumerate(parts):
+        step[i] = launch
+    names = ["router_projection", "router_wide_select", "exl3_tcp_count", "exl3_tcp_place", "exl3_tcp_operands", "exl3_tcp_gemm(gate/up)",
+             "exl3_tcp_activate", "exl3_tcp_gemm(down)", "exl3_tcp_combine"]
+    for _ in range(arguments.warmup):
+        card.run(step, wait=False)
+    card.wait()
+    device_us = card.measure(lambda: [card.run(step, wait=False) for _ in range(arguments.steps)])
+    seconds = device_us * 1e-6
+    per_launch = np.zeros(len(names))
+    for _ in range(arguments.steps):
+        per_launch += np.array(card.run_timed(step))
+    per_launch /= arguments.steps
+    pairs = rows * PICKS
+    gate_up_flops, down_flops = 2.0 * pairs * 2 * HIDDEN * INNER, 2.0 * pairs * HIDDEN * INNER
+    gate_up_us, down_us = float(per_launch[5]), float(per_launch[7])
+    picks = wide.read("picks", np.dtype([("expert", "<u4"), ("route_weight", "<f4")])).reshape(rows, PICKS)
+    counts = np.bincount(picks["expert"].reshape(-1), minlength=EXPERTS)
+    achieved = gate_up_flops / (gate_up_us * 1e-6) / 1e12
+    chunk = amd.EXL3_TCP_CHUNK_PAIRS
+    result = {
+        "metric": "MoE layer tok/s; decode HBM GB/s & prefill MFMA % of peak, 1 GPU",
+        "value": rows * arguments.steps / seconds, "unit": "tok/s", "n_gpus": 1, "steps": arguments.steps,
+        "warmup": arguments.warmup, "ms_per_step": 1000.0 * seconds / arguments.steps, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "exl3_moe_prefill: %d tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router "
+                               "with a Zipf (s = 1.1) bias of strength %.2f, EXL3 K in {2,3,4} per tensor (%.2f bpw)"
+                               % (rows, arguments.zipf_strength, float(np.mean(widths))),
+                   "pairs_of_the_busiest_expert": int(counts.max()), "experts_without_a_pair": int((counts == 0).sum()),
+                   "chunks": int(((counts + chunk - 1) // chunk).sum()),
+                   "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
+                   "down_TFLOPs": down_flops / (down_us * 1e-6) / 1e12,
+                   "step_TFLOPs": (gate_up_flops + down_flops) / (seconds / arguments.steps) / 1e12},
+        "roofline": {"bound": "mfma", "kernel": "exl3_tcp_gemm (gate/up pass)", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": None,
+                     "algorithmic_flops_per_launch": gate_up_flops, "launch_us": gate_up_us},
+    }
+    if not arguments.no_cpu:
+        import ctypes as C
+        import _oracle as o
+        threads = min(os.cpu_count() or 1, 16)
+        sample = min(rows, 8)
+        experts_of = np.ascontiguousarray(picks["expert"][:sample])
+        weights_of = np.ascontiguousarray(picks["route_weight"][:sample])
+        pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
+        want = np.zeros((sample, HIDDEN), dtype=np.float32)
+        widths8 = np.ascontiguousarray(widths.astype(np.uint8))
+        start = time.perf_counter()
+        o.orc.orc_exl3_moe_layer(o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS, o.ptr(experts_of, o.u32p),
+                                 o.ptr(weights_of, o.f32p), EXPERTS, pointers, o.ptr(widths8, o.u8p), 10.0, o.ptr(want, o.f32p), None, None,
+                                 threads)
+        cpu_seconds = time.perf_counter() - start
+        got = layer.output()[:sample]
+        rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+        error = float(np.max(np.abs(got - want))) / rms
+        assert error <= 4e-3, "GPU output differs from the oracle's: %g of rms" % error
+        result["cpu_baseline"] = {"value": sample / cpu_seconds, "unit": "tok/s", "cores": threads, "kind": "port",
+                                  "sample": "the first %d tokens of the same call by the CPU oracle, double-precision sums" % sample,
+                                  "seconds": cpu_seconds, "gpu_vs_oracle_max_err_over_rms": error}
+    card.close()
+    print(json.dumps(result))
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=200)
     parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--workload", default="exl3_decode")
+    parser.add_argument("--zipf-strength", type=float, default=0.2,
+                        help="exl3_prefill: the router's bias is this times ln(Zipf pmf); 0.2 matches the spread of sigmoid affinities")
     parser.add_argument("--rows", type=int, default=32, help="tokens of a step (fp4_decode)")
     parser.add_argument("--gate-up-slices", type=int, default=4)
     parser.add_argument("--down-slices", type=int, default=2)
@@ -177,7 +265,7 @@ def main():
     if arguments.gpus != 1:
         print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
         sys.exit(2)
-    if arguments.workload not in ("exl3_decode", "fp4_decode", "fp8_decode"):
+    if arguments.workload not in ("exl3_decode", "fp4_decode", "fp8_decode", "exl3_prefill"):
         print("unknown workload %s" % arguments.workload, file=sys.stderr)
         sys.exit(2)
 
@@ -186,6 +274,9 @@ def main():
 
     if arguments.calibrate:
         calibrate(amd)
+        return
+    if arguments.workload == "exl3_prefill":
+        exl3_prefill(amd, workloads, arguments)
         return
     if arguments.workload in ("fp4_decode", "fp8_decode"):
         fp4_decode(amd, workloads, arguments, fp8=arguments.workload == "fp8_decode")
