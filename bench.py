@@ -253,8 +253,9 @@ def main():
     parser.add_argument("--steps", type=int, default=200)
     parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--workload", default="exl3_decode")
-    parser.add_argument("--zipf-strength", type=float, default=0.2,
-                        help="exl3_prefill: the router's bias is this times ln(Zipf pmf); 0.2 matches the spread of sigmoid affinities")
+    parser.add_argument("--zipf-strength", type=float, default=0.05,
+                        help="exl3_prefill: the router's bias is this times ln(Zipf pmf): 0.05 gives loads close to Zipf (s = 1.1) "
+                             "under sigmoid affinities with no idle expert; 0.2 leaves three quarters of the experts idle")
     parser.add_argument("--rows", type=int, default=32, help="tokens of a step (fp4_decode)")
     parser.add_argument("--gate-up-slices", type=int, default=4)
     parser.add_argument("--down-slices", type=int, default=2)
