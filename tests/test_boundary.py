@@ -282,3 +282,148 @@ def test_router_prepare(fake):
     six.scores, six.affinities, six.bias, six.offsets = amd.Range(4096, 8 * 384 * 4), amd.Range(262144, 8 * 384 * 4), amd.Range(65536, 384 * 4), amd.Range(131072, 384 * 24)
     keep.gate_up_shape, keep.down_shape = amd.Shape(512, 1024, 3, 0), amd.Shape(1024, 512, 3, 0)
     assert lib.router_select_prepare(C.byref(six), ARENA, C.byref(kernels), launch) == 0
+
+
+# ---- the wide select, the prefill form, the FP4 / FP8 experts: geometry and refusals ----
+
+def wide_description(**changes):
+    E, P, rows = 256, 8, 4096
+    offsets = ((1 << 28) + np.arange(E * 3, dtype=np.uint64) * np.uint64(4 << 20))
+    d = amd.RouterWideDescription()
+    d.expert_offsets = offsets.ctypes.data_as(C.POINTER(C.c_uint64))
+    d.expert_weights = amd.Range(1 << 28, 1 << 32)
+    d.gate_up_shape, d.down_shape, d.weight_format = amd.Shape(2048, 4096, 3, 0), amd.Shape(4096, 2048, 3, 0), amd.WEIGHT_FORMAT_EXL3
+    cursor = [4096]
+
+    def take(size):
+        at = cursor[0]
+        cursor[0] = (at + size + 255) // 256 * 256
+        return amd.Range(at, size)
+    d.step, d.scores, d.bias, d.offsets = take(16), take(rows * E * 4), take(E * 4), take(E * 24)
+    d.affinities, d.picks, d.counts = take(rows * E * 4), take(rows * P * 8), take((rows + 383) // 384 * E * 4)
+    d.pairs, d.runs = take(rows * P * 8), take(E * 8)
+    d.tiles, d.jobs = take(amd.wide_tile_count(rows, P, E) * 32), take(amd.wide_job_count(rows, P, E) * 96)
+    d.order, d.row_count, d.expert_count, d.pick_count, d.affinity_kind, d.route_scale = 0, rows, E, P, 1, 1.5
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d, offsets
+
+
+def test_wide_router_prepare(fake):
+    lib = amd.library()
+    kernels = amd.RouterKernels()
+    assert lib.router_kernels_prepare(fake.address, fake.card, C.byref(kernels)) == 0
+    assert amd.BACKEND_NO_KERNEL not in (kernels.wide_select, kernels.wide_count, kernels.wide_place, kernels.wide_jobs)
+    assert kernels.wide_small == amd.BACKEND_NO_KERNEL  # the one-launch form is not built
+    d, keep = wide_description()
+    launches = amd.launches_of(4)
+    assert lib.router_wide_prepare(C.byref(d), ARENA, C.byref(kernels), launches) == 0
+    names = [fake.handles[l.kernel][1] for l in launches]
+    assert names == ["router_wide_select", "router_wide_count", "router_wide_place", "router_wide_jobs"]
+    assert [list(l.grid) for l in launches] == [[512, 1, 1], [11, 1, 1], [11, 1, 1], [1, 1, 1]]
+    assert all(l.block[0] == 512 and l.argument_byte_count == 136 for l in launches)
+    assert amd.wide_tile_count(4096, 8, 256) == 768 and amd.wide_job_count(4096, 8, 256) == 4320  # the survey's figures
+    for changes in (dict(row_count=0), dict(row_count=70000), dict(expert_count=100), dict(pick_count=0), dict(route_scale=-1.0),
+                    dict(reserved_zero=1), dict(weight_format=1), dict(jobs=amd.Range(1 << 27, 96))):
+        bad, keep = wide_description(**changes)
+        untouched = amd.launches_of(4)
+        assert lib.router_wide_prepare(C.byref(bad), ARENA, C.byref(kernels), untouched) == 1, changes
+        assert not any(bytes(untouched))
+    # two ranges of one description that share a byte
+    bad, keep = wide_description()
+    bad.runs = amd.Range(bad.pairs.byte_offset, 256 * 8)
+    assert lib.router_wide_prepare(C.byref(bad), ARENA, C.byref(kernels), amd.launches_of(4)) == 1
+
+
+def tcp_record(**changes):
+    r = amd.Exl3TcpRecord()
+    rows, H, I, P, E = 4096, 4096, 2048, 8, 256
+    r.picks_offset, r.expert_offsets_offset, r.hidden_offset = 4096, 1 << 20, 2 << 20
+    r.output_offset, r.workspace_offset = 64 << 20, 256 << 20
+    r.row_count, r.intermediate, r.bits_x2, r.activation_limit = rows, I, 6, 10.0
+    r.hidden, r.pairs_per_row, r.expert_count = H, P, E
+    for key, value in changes.items():
+        setattr(r, key, value)
+    return r
+
+
+def test_tcp_prepare_geometry_and_refusals(fake):
+    lib = amd.library()
+    launches, count = amd.launches_of(8), C.c_uint32(0)
+    assert lib.exl3_tcp_prepare(C.byref(tcp_record()), ARENA, fake.address, fake.card, launches, C.byref(count)) == 0
+    assert count.value == 7
+    names = [fake.handles[launches[i].kernel][1] for i in range(7)]
+    assert names == ["exl3_tcp_count", "exl3_tcp_place", "exl3_tcp_operands", "exl3_tcp_gemm", "exl3_tcp_activate", "exl3_tcp_gemm",
+                     "exl3_tcp_combine"]
+    capacity = 4096 * 8 // amd.EXL3_TCP_CHUNK_PAIRS + 256
+    assert [list(launches[i].grid) for i in range(7)] == [[11, 1, 1], [11, 1, 1], [32, capacity, 2], [8, capacity, 2], [16, capacity, 1],
+                                                           [16, capacity, 1], [32, 4096, 1]]
+    assert [launches[i].block[0] for i in range(7)] == [512, 512, 64, 256, 64, 256, 64]
+    records = [amd.Exl3TcpRecord.from_buffer_copy(bytes(launches[i].argument)[:112]) for i in range(7)]
+    assert [r.pass_ for r in records] == [0, 0, 0, 0, 0, 3, 0] and all(launches[i].argument_byte_count == 112 for i in range(7))
+    layout = amd.exl3_tcp_layout(4096, 8, 256, 4096, 2048)
+    assert layout["total"] % 256 == 0 and layout["down"] - layout["gate_up"] == 2 * 32768 * 2048 * 4
+    for changes, status in ((dict(row_count=0), 1), (dict(pairs_per_row=9), 1), (dict(expert_count=0), 1), (dict(pass_=1), 1),
+                            (dict(rotation=1), 7), (dict(half_rows=5), 7), (dict(cone_layer=3), 7), (dict(intermediate=2000), 7),
+                            (dict(bits_x2=7), 7), (dict(bits_x2=40), 1), (dict(workspace_offset=(256 << 20) + 16), 1),
+                            (dict(workspace_offset=ARENA - 4096), 1), (dict(output_offset=2 << 20), 1)):
+        untouched, n = amd.launches_of(8), C.c_uint32(99)
+        assert lib.exl3_tcp_prepare(C.byref(tcp_record(**changes)), ARENA, fake.address, fake.card, untouched, C.byref(n)) == status, changes
+        assert not any(bytes(untouched)) and n.value == 99
+
+
+def experts_description(fmt=amd.WEIGHT_FORMAT_E2M1_SCALED, **changes):
+    rows, P, H, I = 8, 8, 4096, 2048
+    pairs = rows * P
+    bits = 8 if fmt == amd.WEIGHT_FORMAT_E4M3_SCALED else 4
+    d = amd.RoutedExpertsDescription()
+    cursor = [4096]
+
+    def take(size):
+        at = cursor[0]
+        cursor[0] = (at + size + 255) // 256 * 256
+        return amd.Range(at, size)
+    d.jobs, d.expert_weights = take(pairs * 96), take(1 << 30)
+    d.codes, d.exponents, d.operands = take(rows * H), take(rows * H // 32), take(rows * H * 2)
+    d.hidden, d.hidden_codes, d.hidden_exponents, d.hidden_operands = take(pairs * I * 2), take(pairs * I), take(pairs * I // 32), take(pairs * I * 2)
+    d.pair_output, d.row_output = take(pairs * H * 2), take(rows * H * 4)
+    d.gate_up_shape, d.down_shape, d.weight_format = amd.Shape(I, H, bits, 0), amd.Shape(H, I, bits, 0), fmt
+    d.job_count, d.row_count, d.pairs_per_row = pairs, rows, P
+    d.gate_up_slice_count, d.down_slice_count, d.activation_limit = 4, 2, 10.0
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d
+
+
+def test_linear_prepare_geometry_and_refusals(fake):
+    lib = amd.library()
+    kernels = amd.LinearKernels()
+    assert lib.linear_kernels_prepare(fake.address, fake.card, 80, C.byref(kernels)) == 1  # a class of another card
+    assert lib.linear_kernels_prepare(fake.address, fake.card, 950, C.byref(kernels)) == 0
+    assert kernels.expert_gate_up[4] == amd.BACKEND_NO_KERNEL and kernels.trunk_hidden == amd.BACKEND_NO_KERNEL  # 16 slices; the trunk
+    launches = amd.launches_of(4)
+    assert lib.linear_routed_experts_prepare(C.byref(experts_description()), ARENA, C.byref(kernels), launches) == 0
+    names = [fake.handles[l.kernel][1] for l in launches]
+    assert names == ["expert_gate_up_4", "activation_quantize_entry", "expert_down_2", "expert_row_sum_entry"]
+    assert [list(l.grid) for l in launches] == [[32, 64, 1], [8, 64, 1], [64, 64, 1], [16, 8, 1]]
+    assert [l.block[0] for l in launches] == [256, 256, 128, 256]
+    assert [l.argument_byte_count for l in launches] == [64, 40, 56, 24]
+    fp8 = amd.launches_of(4)
+    assert lib.linear_routed_experts_prepare(C.byref(experts_description(amd.WEIGHT_FORMAT_E4M3_SCALED)), ARENA, C.byref(kernels), fp8) == 0
+    assert [fake.handles[l.kernel][1] for l in fp8][::2] == ["expert_gate_up_e4m3_4", "expert_down_e4m3_2"]
+    assert [list(l.grid) for l in fp8][::2] == [[64, 64, 1], [128, 64, 1]]  # strips of 32 outputs
+    for changes in (dict(gate_up_slice_count=3), dict(down_slice_count=16), dict(row_count=0), dict(activation_limit=0.0),
+                    dict(weight_format=amd.WEIGHT_FORMAT_EXL3), dict(reserved_zero=1), dict(gate_up_shape=amd.Shape(2048, 4000, 4, 0)),
+                    dict(down_shape=amd.Shape(4096, 1024, 4, 0)), dict(gate_up_shape=amd.Shape(32, 4096, 4, 0))):
+        untouched = amd.launches_of(4)
+        assert lib.linear_routed_experts_prepare(C.byref(experts_description(**changes)), ARENA, C.byref(kernels), untouched) == 1, changes
+        assert not any(bytes(untouched))
+    quantize = amd.QuantizeDescription(amd.Range(4096, 8 * 4096 * 2), amd.Range(1 << 20, 8 * 4096), amd.Range(2 << 20, 8 * 128),
+                                       amd.Range(3 << 20, 8 * 4096 * 2), 4096, 8)
+    one = amd.launches_of(1)
+    assert lib.linear_quantize_prepare(C.byref(quantize), ARENA, C.byref(kernels), one) == 0
+    assert list(one[0].grid) == [16, 8, 1] and one[0].argument_byte_count == 40
+    quantize.width = 4100
+    assert lib.linear_quantize_prepare(C.byref(quantize), ARENA, C.byref(kernels), one) == 1
+    shape, count = amd.Shape(2048, 4096, 4, 0), C.c_uint32(0)
+    assert lib.linear_default_slice_count(1, 0, 0, C.byref(shape), 950, C.byref(count)) == 0 and count.value in (1, 2, 4, 8)
