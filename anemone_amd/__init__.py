@@ -123,6 +123,10 @@ class LinearKernels(C.Structure):
                 ("trunk_linear_quantized_interleaved", u32), ("expert_gate_up_e4m3", u32 * 5), ("expert_down_e4m3", u32 * 5)]
 
 
+class ExpertFusedKernels(C.Structure):
+    _fields_ = [("gate_up_quantize", u32 * 5), ("shared_join", u32 * 5), ("join", u32), ("gate_up_quantize_e4m3", u32 * 5)]
+
+
 class QuantizeDescription(C.Structure):
     _fields_ = [("values", Range), ("codes", Range), ("exponents", Range), ("operands", Range), ("width", u32),
                 ("row_count", u32)]
@@ -179,6 +183,9 @@ def library():
             "linear_quantize_prepare": [C.POINTER(QuantizeDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_routed_experts_prepare": [C.POINTER(RoutedExpertsDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_default_slice_count": [C.c_int, C.c_int, C.c_int, C.POINTER(Shape), u32, C.POINTER(u32)],
+            "expert_fused_kernels_prepare": [vp, vp, u32, C.POINTER(ExpertFusedKernels)],
+            "expert_producer_prepare": [C.POINTER(RoutedExpertsDescription), Range, u64, C.POINTER(LinearKernels),
+                                        C.POINTER(ExpertFusedKernels), launch_p],
         }
         for name, argtypes in signatures.items():
             function = getattr(lib, name)
@@ -672,6 +679,20 @@ class Fp4Layer:
         launches = launches_of(4)
         check(self.card.lib.linear_routed_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launches), "linear_routed_experts_prepare")
         return launches
+
+    def producer_launch(self):
+        """One launch in place of the first two of expert_launches(): gate with up, and the hidden vectors' quantization."""
+        if not hasattr(self, "fused_kernels"):
+            self.fused_kernels = ExpertFusedKernels()
+            check(self.card.lib.expert_fused_kernels_prepare(backend_table(), self.card.handle, ARITHMETIC_CLASS_GFX950,
+                                                             C.byref(self.fused_kernels)), "expert_fused_kernels_prepare")
+            size = self.pairs * (self.I // 32) * 4
+            self.arrivals = Range(self.card.place(np.zeros(size, dtype=np.uint8)), size)
+        d = self.experts_description()
+        launch = launches_of(1)
+        check(self.card.lib.expert_producer_prepare(C.byref(d), self.arrivals, self.card.arena_bytes, C.byref(self.kernels),
+                                                    C.byref(self.fused_kernels), launch), "expert_producer_prepare")
+        return launch
 
     def read(self, name, dtype=np.uint8):
         r = self.ranges[name]

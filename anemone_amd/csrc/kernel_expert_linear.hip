@@ -35,6 +35,7 @@
  */
 #include "exl3_device.cuh" /* det_expf, bf16 helpers, vector types */
 #include "kernel_registry.h"
+#include "quantize_device.cuh"
 
 typedef int int8_vector __attribute__((ext_vector_type(8)));
 
@@ -333,7 +334,7 @@ struct strip_chain {
 /* gate and up: block = S wavefronts (slices of the inputs); grid (ceil(output_size / 64), jobs) */
 template <uint32_t S, bool BYTES>
 __device__ static __forceinline__ void expert_gate_up(const struct expert_gate_up_arguments &arguments,
-                                                      unsigned char *arena)
+                                                      unsigned char *arena, uint16_t *strip_hidden = nullptr)
 {
     typedef strip_chain<2, BYTES> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP;
@@ -402,6 +403,85 @@ __device__ static __forceinline__ void expert_gate_up(const struct expert_gate_u
         uint16_t *out = (uint16_t *)(arena + arguments.hidden_offset) + (uint64_t)pair * arguments.output_size +
                         (tile0 + n) * 16u + 4u * (lane / 16u);
         *(uint2_t *)out = (uint2_t){(uint32_t)hidden[0] | ((uint32_t)hidden[1] << 16), (uint32_t)hidden[2] | ((uint32_t)hidden[3] << 16)};
+        if (strip_hidden != nullptr) { /* the producer's copy: [column][the strip's outputs] */
+            uint16_t *copy = strip_hidden + column * (STRIP * 16u) + n * 16u + 4u * (lane / 16u);
+#pragma unroll
+            for (uint32_t v = 0; v < 4u; v++) {
+                copy[v] = hidden[v];
+            }
+        }
+    }
+}
+
+/* The producer: gate with up, then the quantization of the strip's hidden values, in one launch. A block of the
+ * quantization is 32 consecutive outputs and a strip holds whole blocks (64 outputs of 4-bit weights, 32 of one-byte
+ * weights), so the second step needs nothing of another block: the hidden values pass through LDS. One more row of
+ * blocks (blockIdx.y = the jobs' number) quantizes, from memory, the pairs that stand in no job, as the quantizer's
+ * own launch does. Grid (ceil(output_size / strip), jobs + 1). */
+template <uint32_t S, bool BYTES>
+__device__ static __forceinline__ void expert_gate_up_quantize(const struct expert_gate_up_quantize_arguments &arguments,
+                                                               unsigned char *arena)
+{
+    typedef strip_chain<2, BYTES> chain_type;
+    constexpr uint32_t STRIP_OUTPUTS = chain_type::STRIP * 16u;
+    __shared__ uint16_t strip_hidden[LINEAR_MAXIMUM_ROWS][STRIP_OUTPUTS];
+    __shared__ uint32_t routed[EXPERT_PRODUCER_MOST_PAIRS / 32u];
+    const uint32_t tiles = arguments.output_size / 16u;
+    const uint32_t tile0 = blockIdx.x * chain_type::STRIP + chain_type::STRIP <= tiles ? blockIdx.x * chain_type::STRIP : tiles - chain_type::STRIP;
+    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t width = arguments.output_size;
+    const uint32_t first_output = blockIdx.x * STRIP_OUTPUTS; /* a last strip that reaches past the matrix starts earlier */
+    if (blockIdx.y + 1u == gridDim.y) {
+        /* the pairs no job holds: a bit a pair from the job table (a job a pair at most), then the quantizer's work */
+        const struct expert_job_record *jobs = (const struct expert_job_record *)(arena + arguments.jobs_offset);
+        if (threadIdx.x < EXPERT_PRODUCER_MOST_PAIRS / 32u) {
+            uint32_t bits = 0;
+            for (uint32_t job = 0; job < arguments.pair_count; job++) {
+                for (uint32_t column = 0; column < jobs[job].row_count; column++) {
+                    const uint32_t pair = jobs[job].pair_index[column];
+                    bits |= pair / 32u == threadIdx.x ? 1u << (pair % 32u) : 0u;
+                }
+            }
+            routed[threadIdx.x] = bits;
+        }
+        __syncthreads();
+        for (uint32_t pair = wave; pair < arguments.pair_count; pair += S) {
+            if ((routed[pair / 32u] >> (pair % 32u)) & 1u) {
+                continue;
+            }
+            for (uint32_t at = lane; at < STRIP_OUTPUTS; at += WAVE) {
+                const uint32_t index = tile0 * 16u + at;
+                if (index < first_output) { /* whole blocks of 32 that the strip before this one takes */
+                    continue;
+                }
+                const uint32_t bits = ((const uint16_t *)(arena + arguments.hidden_offset))[(uint64_t)pair * width + index];
+                quantize_value(bits, index, arena + arguments.hidden_codes_offset + (uint64_t)pair * width,
+                               arena + arguments.hidden_exponents_offset + (uint64_t)pair * (width / 32u),
+                               (uint16_t *)(arena + arguments.hidden_operands_offset) + (uint64_t)pair * width);
+            }
+        }
+        return;
+    }
+    const struct expert_gate_up_arguments plain = {arguments.jobs_offset, arguments.codes_offset, arguments.exponents_offset,
+                                                   arguments.operands_offset, arguments.hidden_offset, arguments.output_size,
+                                                   arguments.input_size, arguments.pair_count, arguments.pairs_per_row,
+                                                   arguments.activation_limit, 0u};
+    const struct expert_job_record *job = (const struct expert_job_record *)(arena + arguments.jobs_offset) + blockIdx.y;
+    if (job->row_count == 0u) {
+        return;
+    }
+    expert_gate_up<S, BYTES>(plain, arena, &strip_hidden[0][0]);
+    __syncthreads();
+    for (uint32_t column = wave; column < job->row_count; column += S) {
+        const uint64_t pair = job->pair_index[column];
+        for (uint32_t at = lane; at < STRIP_OUTPUTS; at += WAVE) {
+            if (tile0 * 16u + at < first_output) {
+                continue;
+            }
+            quantize_value(strip_hidden[column][at], tile0 * 16u + at, arena + arguments.hidden_codes_offset + pair * width,
+                           arena + arguments.hidden_exponents_offset + pair * (width / 32u),
+                           (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width);
+        }
     }
 }
 
@@ -491,7 +571,19 @@ __device__ static __forceinline__ void expert_down(const struct expert_down_argu
     {                                                                                                             \
         expert_down<S, true>(arguments, arena);                                                                   \
     }                                                                                                             \
-    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_e4m3_##S, expert_down_arguments)
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_e4m3_##S, expert_down_arguments);                       \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_gate_up_quantize_##S(struct expert_gate_up_quantize_arguments arguments, unsigned char *arena)    \
+    {                                                                                                             \
+        expert_gate_up_quantize<S, false>(arguments, arena);                                                      \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_gate_up_quantize_##S, expert_gate_up_quantize_arguments);    \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_gate_up_quantize_e4m3_##S(struct expert_gate_up_quantize_arguments arguments, unsigned char *arena) \
+    {                                                                                                             \
+        expert_gate_up_quantize<S, true>(arguments, arena);                                                       \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_gate_up_quantize_e4m3_##S, expert_gate_up_quantize_arguments)
 EXPERT_ENTRIES(1);
 EXPERT_ENTRIES(2);
 EXPERT_ENTRIES(4);

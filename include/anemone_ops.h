@@ -248,6 +248,27 @@ MUST_CHECK result_status linear_routed_experts_prepare(const struct linear_route
                                                        const struct linear_kernels_record *kernels,
                                                        struct kernel_launch *launches_out);
 
+/* ---- the producer (include/anemone/expert_fused.h:37-60 of the reference): one launch in place of the first two of
+ * the routed experts. The join and the shared join of that header belong to the layer's next step, outside this
+ * path: their handles are BACKEND_NO_KERNEL. ---- */
+struct expert_fused_kernels {
+    uint32_t gate_up_quantize[LINEAR_SLICE_INSTANCES];
+    uint32_t shared_join[LINEAR_SLICE_INSTANCES];
+    uint32_t join;
+    uint32_t gate_up_quantize_e4m3[LINEAR_SLICE_INSTANCES]; /* extension: experts of WEIGHT_FORMAT_E4M3_SCALED */
+};
+MUST_CHECK result_status expert_fused_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                                      uint32_t arithmetic_class, struct expert_fused_kernels *kernels_out);
+/* One launch of expert_gate_up_quantize_<gate_up_slice_count>: it stands for launches LINEAR_ROUTED_EXPERTS_GATE_UP and
+ * _QUANTIZE of linear_routed_experts_prepare and writes what they write, byte for byte. arrivals: uint32
+ * [job_count][gate_up_shape.output_size / 32], holding zeros (left so). Refused besides what the routed experts'
+ * prepare refuses: more than LINEAR_MAXIMUM_ROWS rows, more than EXPERT_PRODUCER_MOST_PAIRS pairs, an output size
+ * that is no multiple of 32, an arrivals range that is too small or shares a byte with another range. */
+MUST_CHECK result_status expert_producer_prepare(const struct linear_routed_experts_description *description,
+                                                 struct linear_range arrivals, uint64_t arena_byte_count,
+                                                 const struct linear_kernels_record *linear_kernels,
+                                                 const struct expert_fused_kernels *kernels, struct kernel_launch *launch_out);
+
 uint64_t linear_values_byte_count(uint64_t vector_count, uint64_t width);    /* bfloat16 [vector][width] */
 uint64_t linear_codes_byte_count(uint64_t vector_count, uint64_t width);     /* E4M3 [vector][width] */
 uint64_t linear_exponents_byte_count(uint64_t vector_count, uint64_t width); /* E8M0 [vector][width / 32] */

@@ -444,6 +444,29 @@ struct expert_gate_up_arguments {
 };
 ANEMONE_RECORD_HAS(expert_gate_up_arguments, 64);
 
+/* expert_gate_up_quantize_<S> (include/anemone/expert_fused_records.h:87-103 of the reference): gate with up and the
+ * quantization of the hidden vectors in one launch */
+#define KERNEL_EXPERT_GATE_UP_QUANTIZE_STEM "expert_gate_up_quantize_"
+#define EXPERT_PRODUCER_MOST_PAIRS (LINEAR_MAXIMUM_ROWS * ROUTER_MOST_PICKS)
+struct expert_gate_up_quantize_arguments {
+    uint64_t jobs_offset;
+    uint64_t codes_offset;            /* the rows' quantized input: as expert_gate_up_arguments */
+    uint64_t exponents_offset;
+    uint64_t operands_offset;
+    uint64_t hidden_offset;           /* written (pairs that stand in a job); read (the others) */
+    uint64_t hidden_codes_offset;     /* written, of every pair */
+    uint64_t hidden_exponents_offset; /* written */
+    uint64_t hidden_operands_offset;  /* written */
+    uint64_t arrivals_offset;         /* uint32 [jobs][output_size / 32], zeros: not touched by this build's kernels */
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t pair_count;
+    uint32_t pairs_per_row;
+    float activation_limit;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(expert_gate_up_quantize_arguments, 96);
+
 struct expert_down_arguments {
     uint64_t jobs_offset;
     uint64_t codes_offset;     /* read: codes [pair][input_size] */

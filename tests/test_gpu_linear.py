@@ -195,3 +195,35 @@ def test_layer_against_oracle(amd, card, rows, live, picks, fmt):
     error = np.sqrt(np.mean((got - want) ** 2) / np.mean(want.astype(np.float64) ** 2))
     say("  layer rms error vs oracle: %.2e" % error)
     assert error < 2e-2
+
+
+@pytest.mark.parametrize("rows,live,picks,fmt,slices", [(8, 6, 4, E2M1, 4), (8, 8, 8, E2M1, 1), (4, 3, 8, E4M3, 2), (1, 1, 2, E2M1, 2)])
+def test_producer_equals_the_two_launches_byte_for_byte(amd, card, rows, live, picks, fmt, slices):
+    """expert_gate_up_quantize_<S> against expert_gate_up_<S> followed by the quantizer (the reference's own bar for its
+    producer, tests/expert_fused_card_test.c:2-4): the hidden values, their codes, exponents and operands of every pair,
+    those of the rows beyond the live ones among them (quantized from what the hidden range holds)."""
+    say("producer", rows, live, picks, fmt, slices)
+    hidden, inner, experts_n = 512, 256, 64
+    layer, _, _ = build(amd, card, hidden, inner, experts_n, picks, rows, 6, fmt=fmt, gate_up_slices=slices, down_slices=1)
+    x = to_bf16(normals(13, rows * hidden)).reshape(rows, hidden)
+    layer.set_rows(x, live)
+    card.run(layer.projection_launch())
+    card.run(layer.select_launch(0))
+    card.run(layer.quantize_launch())
+    stale = to_bf16(normals(14, rows * picks * inner) * 3.0)  # what the hidden range holds for pairs no job writes
+    names = ("hidden", "hidden_codes", "hidden_exponents", "hidden_operands")
+
+    def run(launches):
+        card.upload(layer.ranges["hidden"].byte_offset, stale)
+        for name in names[1:]:
+            card.upload(layer.ranges[name].byte_offset, np.full(layer.ranges[name].byte_count, 0xEE, dtype=np.uint8))
+        card.run(launches)
+        return [layer.read(name).copy() for name in names]
+    apart = run(layer.expert_launches()[0:2])
+    fused = run(layer.producer_launch())
+    for name, a, b in zip(names, apart, fused):
+        assert np.array_equal(a, b), name
+    assert not np.any(card.download(layer.arrivals.byte_offset, layer.arrivals.byte_count))  # the arrival counters stay zero
+    if live < rows:  # the pairs of the rows beyond the live ones were quantized from the stale values
+        want = oracle_quantize(stale.reshape(rows * picks, inner)[live * picks:])[2]
+        assert np.array_equal(fused[1].reshape(rows * picks, inner)[live * picks:], want)
