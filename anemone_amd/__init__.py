@@ -95,6 +95,21 @@ class RoutedExpertsDescription(C.Structure):
                 ("activation_limit", f32), ("reserved_zero", u32)]
 
 
+class WideExpertGateUpArguments(C.Structure):
+    _fields_ = [("tiles_offset", u64), ("pairs_offset", u64), ("codes_offset", u64), ("exponents_offset", u64), ("operands_offset", u64),
+                ("hidden_codes_offset", u64), ("hidden_exponents_offset", u64), ("hidden_operands_offset", u64), ("output_size", u32),
+                ("input_size", u32), ("tile_count", u32), ("pairs_per_row", u32), ("activation_limit", f32), ("pair_count", u32)]
+
+
+class WideExpertDownArguments(C.Structure):
+    _fields_ = [("tiles_offset", u64), ("pairs_offset", u64), ("codes_offset", u64), ("exponents_offset", u64), ("operands_offset", u64),
+                ("output_offset", u64), ("output_size", u32), ("input_size", u32), ("tile_count", u32), ("pair_count", u32)]
+
+
+class LinearWideExpertsDescription(C.Structure):
+    _fields_ = [("experts", RoutedExpertsDescription), ("tiles", Range), ("pairs", Range), ("tile_count", u32), ("reserved_zero", u32)]
+
+
 class RouterDescription(C.Structure):
     _fields_ = [("experts", C.POINTER(RoutedExpertsDescription)), ("expert_offsets", C.POINTER(u64)),
                 ("expert_widths", C.POINTER(u32)), ("step", Range), ("scores", Range), ("bias", Range),
@@ -125,6 +140,10 @@ class LinearKernels(C.Structure):
 
 class ExpertFusedKernels(C.Structure):
     _fields_ = [("gate_up_quantize", u32 * 5), ("shared_join", u32 * 5), ("join", u32), ("gate_up_quantize_e4m3", u32 * 5)]
+
+
+class LinearWideKernels(C.Structure):
+    _fields_ = [("wide_expert_gate_up", u32), ("wide_expert_down", u32), ("wide_expert_gate_up_e4m3", u32), ("wide_expert_down_e4m3", u32)]
 
 
 class QuantizeDescription(C.Structure):
@@ -183,6 +202,9 @@ def library():
             "linear_quantize_prepare": [C.POINTER(QuantizeDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_routed_experts_prepare": [C.POINTER(RoutedExpertsDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_default_slice_count": [C.c_int, C.c_int, C.c_int, C.POINTER(Shape), u32, C.POINTER(u32)],
+            "linear_wide_kernels_prepare": [vp, vp, u32, C.POINTER(LinearWideKernels)],
+            "linear_wide_experts_prepare": [C.POINTER(LinearWideExpertsDescription), u64, C.POINTER(LinearKernels),
+                                            C.POINTER(LinearWideKernels), launch_p],
             "expert_fused_kernels_prepare": [vp, vp, u32, C.POINTER(ExpertFusedKernels)],
             "expert_producer_prepare": [C.POINTER(RoutedExpertsDescription), Range, u64, C.POINTER(LinearKernels),
                                         C.POINTER(ExpertFusedKernels), launch_p],
@@ -678,6 +700,21 @@ class Fp4Layer:
         d = self.experts_description(wide)
         launches = launches_of(4)
         check(self.card.lib.linear_routed_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launches), "linear_routed_experts_prepare")
+        return launches
+
+    def wide_expert_launches(self, wide):
+        """The wide form over the tiles and sorted pairs of a WideRouter: gate/up with the quantization, down, row sum."""
+        if not hasattr(self, "wide_kernels"):
+            self.wide_kernels = LinearWideKernels()
+            check(self.card.lib.linear_wide_kernels_prepare(backend_table(), self.card.handle, ARITHMETIC_CLASS_GFX950,
+                                                            C.byref(self.wide_kernels)), "linear_wide_kernels_prepare")
+        d = LinearWideExpertsDescription()
+        d.experts = self.experts_description(wide)
+        d.experts.gate_up_slice_count = d.experts.down_slice_count = 1
+        d.tiles, d.pairs, d.tile_count = wide.ranges["tiles"], wide.ranges["pairs"], wide.tile_count
+        launches = launches_of(3)
+        check(self.card.lib.linear_wide_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), C.byref(self.wide_kernels),
+                                                        launches), "linear_wide_experts_prepare")
         return launches
 
     def producer_launch(self):

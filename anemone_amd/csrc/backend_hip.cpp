@@ -331,7 +331,10 @@ result_status backend_hip_card_open(uint32_t card_index, uint64_t arena_byte_cou
         return STATUS_DEVICE_ERROR;
     }
     card->max_threads = properties.maxThreadsPerBlock;
-    card->max_shared = (int)properties.sharedMemPerBlock;
+    /* what a block may take with the limit raised at kernel_prepare: the whole LDS of a compute unit on gfx950 */
+    card->max_shared = (int)(properties.maxSharedMemoryPerMultiProcessor > properties.sharedMemPerBlock
+                                 ? properties.maxSharedMemoryPerMultiProcessor
+                                 : properties.sharedMemPerBlock);
     if (hipMalloc((void **)&card->arena, arena_byte_count) != hipSuccess) {
         (void)hipGetLastError();
         delete card;
@@ -490,6 +493,12 @@ result_status backend_hip_kernel_prepare(struct device_card *card, const char *k
         if (card->prepared.size() >= BACKEND_MAXIMUM_KERNELS) {
             log_error(function_name, "more kernels than a card prepares");
             return STATUS_INVALID_ARGUMENT;
+        }
+        /* as the reference's backend does behind its parameter check (source/backend_cuda_launch.c:160-186): raise
+         * the kernel's limit of dynamic shared memory to what the card holds; a refusal shows at the launch that asks */
+        if (hipSetDevice(card->device) == hipSuccess) {
+            (void)hipFuncSetAttribute(table[index].host_function, hipFuncAttributeMaxDynamicSharedMemorySize, card->max_shared);
+            (void)hipGetLastError();
         }
         card->prepared.push_back(index);
         *kernel_out = (uint32_t)card->prepared.size() - 1u;

@@ -33,47 +33,9 @@
  * 16 (l / 16) + e % 16; scale of lane l: row or column l % 16, inputs block l / 16; D lane l: column l % 16, rows
  * 4 (l / 16) + v.
  */
-#include "exl3_device.cuh" /* det_expf, bf16 helpers, vector types */
 #include "kernel_registry.h"
+#include "linear_device.cuh"
 #include "quantize_device.cuh"
-
-typedef int int8_vector __attribute__((ext_vector_type(8)));
-
-#define NIBBLE_STEP_BYTES 1024u /* a tile's K step of 128 inputs: 16 outputs x 128 inputs x 4 bits */
-#define BYTE_STEP_BYTES 2048u   /* the same of one-byte weights */
-#define NIBBLE_MASK 0x0F0F0F0Fu
-
-typedef __attribute__((address_space(3))) void *lds_pointer;
-
-/* Memory straight into LDS, 16 or 4 bytes a lane: lane L's bytes land at lds_base + 16 L (4 L); the address is a
- * base common to the wavefront plus the lane's own byte offset. Written as assembly so that the compiler keeps no
- * book on these loads: it would guard every LDS read that might alias one with a wait for all of them. The waits
- * are this file's own (wait_loads). A fence for the compiler as well, so the loads keep their order, which the waits
- * count on. */
-__device__ static __forceinline__ void load_to_lds_16(const unsigned char *base, uint32_t lane_offset, uint32_t lds_base)
-{
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(lane_offset), "s"(base), "s"(lds_base)
-                 : "memory", "m0");
-}
-
-__device__ static __forceinline__ void load_to_lds_4(const unsigned char *base, uint32_t lane_offset, uint32_t lds_base)
-{
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                 :
-                 : "v"(lane_offset), "s"(base), "s"(lds_base)
-                 : "memory", "m0");
-}
-
-/* wait until at most `count` of the wavefront's memory loads are outstanding (they retire in order); also a fence
- * for the compiler: LDS reads of a stage stay behind the wait for the loads that fill it */
-template <uint32_t count>
-__device__ static __forceinline__ void wait_loads()
-{
-    static_assert(count < 64u, "vmcnt has six bits");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(count) : "memory");
-}
 
 /* A wavefront's part of a strip: MATRICES matrices (gate and up, or down alone) x STRIP tiles, K steps [first, last).
  * LDS window of a wavefront: DEPTH stages; a stage: MATRICES x STRIP x 1,024 bytes of weights, MATRICES x 256 bytes

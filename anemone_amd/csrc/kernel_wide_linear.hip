@@ -1,0 +1,413 @@
+/*
+ * kernel_wide_linear.hip -- the routed experts of the original FP4 / FP8 weights for a prefill-sized step on gfx950:
+ * a grouped GEMM over the tiles of at most 64 pairs of one expert that the router's wide select writes. Entry names,
+ * records and what is written follow the reference (include/anemone/wide_linear_records.h:80-118,
+ * source/kernel_wide_linear.cu): wide_expert_gate_up_<S> writes, for each pair of a tile, what the quantizer writes
+ * from the hidden values expert_gate_up_<S> computes (codes, exponents, operands, not the values);
+ * wide_expert_down_<S> writes a pair's output at its pair_index. An output's bits depend on its matrix, its pair's
+ * input and S alone (the reference's class R): here they are expert_gate_up_<S>'s and expert_down_<S>'s of
+ * kernel_expert_linear.hip bit for bit, because a column's sum is the same chain of the same MFMAs in the same order.
+ * Built for S = 1 (one chain an output).
+ *
+ * Work mapping (this build's own). A block is one tile of pairs (64 columns: four MFMA column blocks of 16) by 256
+ * outputs: four wavefronts, each a strip of tiles of 16 outputs (64 outputs of 4-bit weights, 32 of one-byte
+ * weights; gate AND up of the strip in the gate/up kernel). A stage is one K step (128 inputs): each wavefront's
+ * weights and their scales go from memory straight into its part of the stage in LDS; the 64 columns' codes (8 KB)
+ * and scale words go there once a block, two column groups a wavefront, and serve all four. Three stages are on
+ * their way or in use; one barrier a step. A weight tile's operand is prepared once (four 8-byte LDS reads and
+ * sixteen vector instructions for 4-bit weights) and feeds four MFMAs of 128 inputs each.
+ */
+#include "kernel_registry.h"
+#include "linear_device.cuh"
+#include "quantize_device.cuh"
+
+#define WIDE_WAVES 4u
+#define WIDE_THREADS (WIDE_WAVES * WAVE)
+#define WIDE_COLUMN_BLOCKS (WIDE_TILE_PAIRS / 16u)
+#define WIDE_DEPTH 3u
+#define WIDE_VECTOR_BYTES (WIDE_TILE_PAIRS * 128u) /* a K step of the tile's columns' codes */
+
+/* One block's pipeline: MATRICES matrices x STRIP tiles a wavefront, the tile's columns shared. */
+template <uint32_t MATRICES, bool BYTES>
+struct wide_chain {
+    static constexpr uint32_t STRIP = BYTES ? 2u : 4u;
+    static constexpr uint32_t STEP_BYTES = BYTES ? BYTE_STEP_BYTES : NIBBLE_STEP_BYTES;
+    static constexpr uint32_t TILE_LOADS = STEP_BYTES / 1024u;
+    static constexpr uint32_t TILES = MATRICES * STRIP;
+    static constexpr uint32_t SCALES_AT = TILES * STEP_BYTES;                    /* inside a wavefront's part */
+    static constexpr uint32_t WAVE_BYTES = SCALES_AT + MATRICES * 256u;          /* a wavefront's part of a stage */
+    static constexpr uint32_t VECTOR_AT = WIDE_WAVES * WAVE_BYTES;               /* inside a stage */
+    static constexpr uint32_t VECTOR_SCALE_AT = VECTOR_AT + WIDE_VECTOR_BYTES;
+    static constexpr uint32_t STAGE_BYTES = VECTOR_SCALE_AT + 256u;
+    static constexpr uint32_t WINDOW_BYTES = WIDE_DEPTH * STAGE_BYTES;
+    static constexpr uint32_t STAGE_LOADS = TILES * TILE_LOADS + MATRICES + 2u + 1u; /* a wavefront's loads a stage */
+    static_assert(STAGE_LOADS * (WIDE_DEPTH - 1u) < 64u && WINDOW_BYTES <= 160u * 1024u, "vmcnt has six bits; LDS 160 KB");
+
+    const unsigned char *words[MATRICES], *scales[MATRICES], *codes, *exponents;
+    uint32_t tile_bytes, window, wave, piece_offset, scale_offset, codes_offset[2], exponents_offset;
+    uint32_t read_at[BYTES ? 8 : 4], scale_at[STRIP], vector_at[BYTES ? 8 : 4], vector_scale_at, shift;
+
+    __device__ __forceinline__ void issue(uint32_t stage, uint32_t at) const
+    {
+        const uint32_t base = window + stage * STAGE_BYTES, mine = base + wave * WAVE_BYTES;
+#pragma unroll
+        for (uint32_t m = 0; m < MATRICES; m++) {
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+#pragma unroll
+                for (uint32_t part = 0; part < TILE_LOADS; part++) {
+                    load_to_lds_16(words[m] + (uint64_t)n * tile_bytes + (uint64_t)at * STEP_BYTES + part * 1024u, piece_offset,
+                                   mine + (m * STRIP + n) * STEP_BYTES + part * 1024u);
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t m = 0; m < MATRICES; m++) {
+            load_to_lds_4(scales[m] + (uint64_t)at * (BYTES ? 4u : 64u), scale_offset, mine + SCALES_AT + m * 256u);
+        }
+        /* the tile's columns: eight groups of eight columns, two a wavefront; every wavefront brings the scale words
+         * (the same bytes to the same place: one load more a wavefront, and all wavefronts count alike) */
+#pragma unroll
+        for (uint32_t part = 0; part < 2u; part++) {
+            load_to_lds_16(codes + (uint64_t)at * 128u, codes_offset[part], base + VECTOR_AT + (2u * wave + part) * 1024u);
+        }
+        load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT);
+    }
+
+    template <typename T>
+    __device__ static __forceinline__ T lds_read(uint32_t address)
+    {
+        return *(const __attribute__((address_space(3))) T *)(uintptr_t)address;
+    }
+
+    __device__ __forceinline__ void consume(uint32_t stage, uint32_t live_blocks, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
+    {
+        const uint32_t base = window + stage * STAGE_BYTES, mine = base + wave * WAVE_BYTES;
+        int8_vector b[WIDE_COLUMN_BLOCKS];
+        uint32_t scale_b[WIDE_COLUMN_BLOCKS];
+#pragma unroll
+        for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+            if (j < live_blocks) { /* the same in every lane */
+                if constexpr (BYTES) {
+#pragma unroll
+                    for (uint32_t v = 0; v < 8u; v++) {
+                        b[j][v] = (int)lds_read<uint32_t>(base + VECTOR_AT + j * 2048u + vector_at[v]);
+                    }
+                } else {
+#pragma unroll
+                    for (uint32_t part = 0; part < 4u; part++) {
+                        const uint2_t pair = lds_read<uint2_t>(base + VECTOR_AT + j * 2048u + vector_at[part]);
+                        b[j][2u * part] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x05010400u);
+                        b[j][2u * part + 1u] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x07030602u);
+                    }
+                }
+                scale_b[j] = lds_read<unsigned char>(base + VECTOR_SCALE_AT + j * 64u + vector_scale_at);
+            }
+        }
+#pragma unroll
+        for (uint32_t tile = 0; tile < TILES; tile++) {
+            int8_vector a = {0, 0, 0, 0, 0, 0, 0, 0};
+            const uint32_t scale_a = lds_read<unsigned char>(mine + SCALES_AT + (tile / STRIP) * 256u + scale_at[tile % STRIP]);
+            if constexpr (BYTES) {
+#pragma unroll
+                for (uint32_t v = 0; v < 8u; v++) {
+                    const uint2_t w = lds_read<uint2_t>(mine + tile * STEP_BYTES + read_at[v]);
+                    a[v] = (int)__builtin_amdgcn_perm(w.y, w.x, shift);
+                }
+            } else {
+#pragma unroll
+                for (uint32_t T = 0; T < 4u; T++) {
+                    const uint2_t w = lds_read<uint2_t>(mine + tile * STEP_BYTES + read_at[T]);
+                    a[T] = (int)(((w.x >> shift) & NIBBLE_MASK) | (((w.y >> shift) & NIBBLE_MASK) << 4));
+                }
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+                if (j < live_blocks) {
+                    if constexpr (BYTES) {
+                        chain[tile][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b[j], chain[tile][j], 0, 0, 0, (int)scale_a, 0, (int)scale_b[j]);
+                    } else {
+                        chain[tile][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b[j], chain[tile][j], 4, 0, 0, (int)scale_a, 0, (int)scale_b[j]);
+                    }
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stage is read before the next barrier */
+    }
+
+    /* all `total` K steps; every wavefront of the block calls it (barriers inside) */
+    __device__ __forceinline__ void whole(uint32_t total, uint32_t live_blocks, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
+    {
+        static_assert(WIDE_DEPTH == 3u, "the waits are written out for two stages ahead");
+#pragma unroll
+        for (uint32_t ahead = 0; ahead + 1u < WIDE_DEPTH; ahead++) {
+            if (ahead < total) {
+                issue(ahead, ahead);
+            }
+        }
+        for (uint32_t step = 0; step < total; step++) {
+            /* this step's loads have landed once nothing but the later steps' (one stage at most here) is outstanding */
+            if (step + 1u < total) {
+                wait_loads<STAGE_LOADS>();
+            } else {
+                wait_loads<0>();
+            }
+            /* behind this barrier every wavefront's column groups of this step have landed, and every wavefront has
+             * read the step before: its stage may be asked for again */
+            __syncthreads();
+            if (step + WIDE_DEPTH - 1u < total) {
+                issue((step + WIDE_DEPTH - 1u) % WIDE_DEPTH, step + WIDE_DEPTH - 1u);
+            }
+            consume(step % WIDE_DEPTH, live_blocks, chain);
+        }
+    }
+
+    /* matrices: arena addresses of the stored matrices; block_strip: the block's first strip (of STRIP tiles) is
+     * WIDE_WAVES block_strip; vector_codes / vector_exponents: vector 0's codes and scale codes; vectors: this lane's
+     * two columns' vectors for the codes' loads (lane / 8 of groups 2 wave, 2 wave + 1) and its column's for the scale
+     * words' load (lane) */
+    __device__ __forceinline__ void place(const unsigned char *const (&matrices)[MATRICES], uint32_t outputs, uint32_t inputs,
+                                          uint32_t block_strip, const unsigned char *vector_codes, const unsigned char *vector_exponents,
+                                          const uint32_t (&code_vectors)[2], uint32_t exponent_vector, uint32_t window_address,
+                                          uint32_t wave_index, uint32_t lane, uint32_t &tile0_out)
+    {
+        const uint32_t tiles = outputs / 16u;
+        const uint32_t o = lane % 16u, g = lane / 16u, G = o % 8u, parity = o / 8u, ld = g / 2u, q = g % 2u;
+        const uint32_t strip = block_strip * WIDE_WAVES + wave_index;
+        /* a strip that reaches past the last tile reads the last tiles again; its surplus sums are not stored */
+        const uint32_t tile0 = strip * STRIP + STRIP <= tiles ? strip * STRIP : tiles - STRIP;
+        tile0_out = tile0;
+        const uint32_t steps = inputs / 128u;
+        tile_bytes = steps * STEP_BYTES;
+        window = window_address;
+        wave = wave_index;
+        codes = vector_codes;
+        exponents = vector_exponents;
+        if constexpr (BYTES) {
+            const uint32_t scale_rows = (outputs + 31u) / 32u, row0 = tile0 / 2u;
+#pragma unroll
+            for (uint32_t m = 0; m < MATRICES; m++) {
+                words[m] = matrices[m] + (uint64_t)tile0 * steps * STEP_BYTES;
+                scales[m] = matrices[m] + (uint64_t)outputs * inputs + (uint64_t)row0 * (inputs / 32u);
+            }
+            piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
+            const uint32_t rows_left = scale_rows - 1u - row0;
+            scale_offset = (lane < rows_left ? lane : rows_left) * (inputs / 32u);
+#pragma unroll
+            for (uint32_t v = 0; v < 8u; v++) {
+                const uint32_t group = 2u * (v / 4u) + g / 2u, t = v % 4u;
+                read_at[v] = 16u * (32u * group + 4u * G + (t ^ (G / 2u))) + 8u * (g % 2u);
+            }
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+                scale_at[n] = 4u * ((tile0 + n) / 2u - row0) + g;
+            }
+            shift = parity == 0u ? 0x06020400u : 0x07030501u;
+        } else {
+            const uint32_t loads = inputs / 64u;
+#pragma unroll
+            for (uint32_t m = 0; m < MATRICES; m++) {
+                words[m] = matrices[m] + (uint64_t)tile0 * steps * STEP_BYTES;
+                scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + (uint64_t)tile0 * loads * 32u;
+            }
+            piece_offset = 16u * (lane ^ (2u * ((lane >> 4) & 1u) + ((lane >> 5) & 1u)));
+            scale_offset = (lane / 16u) * (loads * 32u) + (lane % 16u) * 4u;
+#pragma unroll
+            for (uint32_t T = 0; T < 4u; T++) {
+                read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (2u * (G / 4u) + ld))) + 8u * q;
+            }
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+                scale_at[n] = n * 64u + (8u * ld + G) * 4u + 2u * q + parity;
+            }
+            shift = 4u * parity;
+        }
+        /* the columns' codes: lane L of a load holds slot L % 8 of column L / 8 of its group of eight and asks for
+         * that column's piece (L % 8) ^ (L / 8); a column block of 16 columns is two groups (2,048 bytes) */
+#pragma unroll
+        for (uint32_t part = 0; part < 2u; part++) {
+            codes_offset[part] = code_vectors[part] * inputs + 16u * ((lane % 8u) ^ (lane / 8u));
+        }
+        exponents_offset = exponent_vector * (inputs / 32u);
+        const uint32_t column = o % 8u, group_bytes = (o / 8u) * 1024u;
+        if constexpr (BYTES) {
+#pragma unroll
+            for (uint32_t v = 0; v < 8u; v++) {
+                vector_at[v] = group_bytes + 16u * (8u * column + (v ^ column)) + 4u * g;
+            }
+        } else {
+#pragma unroll
+            for (uint32_t part = 0; part < 4u; part++) {
+                const uint32_t piece = 4u * (part / 2u) + part % 2u + 2u * (g % 2u);
+                vector_at[part] = group_bytes + 16u * (8u * column + (piece ^ column)) + 8u * (g / 2u);
+            }
+        }
+        vector_scale_at = 4u * o + g;
+    }
+};
+
+/* grid (ceil(output_size / (4 strips)), tile_count), block 256 */
+template <bool BYTES>
+__device__ static __forceinline__ void wide_expert_gate_up(const struct wide_expert_gate_up_arguments &arguments, unsigned char *arena)
+{
+    typedef wide_chain<2, BYTES> chain_type;
+    constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
+    extern __shared__ __attribute__((aligned(16))) unsigned char window[];
+    static_assert(chain_type::WAVE_BYTES >= WIDE_TILE_PAIRS * STRIP_OUTPUTS * 2u, "a wavefront's hidden values fit its idle part of a stage");
+    const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
+    if (tile.pair_count == 0u) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const struct wide_pair *pairs = (const struct wide_pair *)(arena + arguments.pairs_offset) + tile.first_pair;
+    /* columns past the tile's last pair read its first pair's vector; their sums are never stored */
+    uint32_t code_vectors[2];
+#pragma unroll
+    for (uint32_t part = 0; part < 2u; part++) {
+        const uint32_t column = 8u * (2u * wave + part) + lane / 8u;
+        code_vectors[part] = pairs[column < tile.pair_count ? column : 0u].pair_index / arguments.pairs_per_row;
+    }
+    const uint32_t exponent_vector = pairs[lane < tile.pair_count ? lane : 0u].pair_index / arguments.pairs_per_row;
+    chain_type chain_of;
+    const unsigned char *const matrices[2] = {arena + tile.gate_offset, arena + tile.up_offset};
+    const uint32_t window_address = (uint32_t)(uintptr_t)(lds_pointer)window;
+    uint32_t tile0 = 0;
+    chain_of.place(matrices, arguments.output_size, arguments.input_size, blockIdx.x, arena + arguments.codes_offset,
+                   arena + arguments.exponents_offset, code_vectors, exponent_vector, window_address, wave, lane, tile0);
+    float4_t chain[TILES][WIDE_COLUMN_BLOCKS];
+#pragma unroll
+    for (uint32_t t = 0; t < TILES; t++) {
+#pragma unroll
+        for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+            chain[t][j] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+    const uint32_t live_blocks = (tile.pair_count + 15u) / 16u;
+    chain_of.whole(arguments.input_size / 128u, live_blocks, chain);
+    __syncthreads(); /* every wavefront is done with the stages: each takes its part of stage 0 for its hidden values */
+    /* the hidden step, as expert_gate_up_1 rounds it (the one chain is added to +0 first, as S chains are) */
+    uint16_t *strip_hidden = (uint16_t *)(window + wave * chain_type::WAVE_BYTES); /* [column][the strip's outputs] */
+    const float limit = arguments.activation_limit;
+#pragma unroll
+    for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+        const uint32_t column = 16u * j + lane % 16u;
+        if (column < tile.pair_count) {
+            const float weight = pairs[column].route_weight;
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+#pragma unroll
+                for (uint32_t v = 0; v < 4u; v++) {
+                    const float gate_sum = __fadd_rn(0.0f, chain[n][j][v]), up_sum = __fadd_rn(0.0f, chain[STRIP + n][j][v]);
+                    const float g = bf16_to_float(float_to_bf16(gate_sum)), u = bf16_to_float(float_to_bf16(up_sum));
+                    const float bounded_gate = fminf(g, limit);
+                    const float bounded_up = fminf(fmaxf(u, -limit), limit);
+                    const float value = __fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), weight);
+                    strip_hidden[column * STRIP_OUTPUTS + n * 16u + 4u * (lane / 16u) + v] = float_to_bf16(value);
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f); /* the wavefront's own LDS writes have landed */
+    __builtin_amdgcn_wave_barrier();
+    const uint32_t width = arguments.output_size, first_output = (blockIdx.x * WIDE_WAVES + wave) * STRIP_OUTPUTS;
+    if (first_output >= width) {
+        return; /* a strip wholly past the matrix */
+    }
+    for (uint32_t column = 0; column < tile.pair_count; column++) {
+        const uint64_t pair = pairs[column].pair_index;
+        for (uint32_t at = lane; at < STRIP_OUTPUTS; at += WAVE) {
+            if (tile0 * 16u + at < first_output) {
+                continue; /* whole blocks of 32 that the strip before this one takes */
+            }
+            quantize_value(strip_hidden[column * STRIP_OUTPUTS + at], tile0 * 16u + at, arena + arguments.hidden_codes_offset + pair * width,
+                           arena + arguments.hidden_exponents_offset + pair * (width / 32u),
+                           (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width);
+        }
+    }
+}
+
+template <bool BYTES>
+__device__ static __forceinline__ void wide_expert_down(const struct wide_expert_down_arguments &arguments, unsigned char *arena)
+{
+    typedef wide_chain<1, BYTES> chain_type;
+    constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
+    extern __shared__ __attribute__((aligned(16))) unsigned char window[];
+    const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
+    if (tile.pair_count == 0u) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const struct wide_pair *pairs = (const struct wide_pair *)(arena + arguments.pairs_offset) + tile.first_pair;
+    uint32_t code_vectors[2]; /* the vectors are the pairs' hidden vectors */
+#pragma unroll
+    for (uint32_t part = 0; part < 2u; part++) {
+        const uint32_t column = 8u * (2u * wave + part) + lane / 8u;
+        code_vectors[part] = pairs[column < tile.pair_count ? column : 0u].pair_index;
+    }
+    const uint32_t exponent_vector = pairs[lane < tile.pair_count ? lane : 0u].pair_index;
+    chain_type chain_of;
+    const unsigned char *const matrices[1] = {arena + tile.down_offset};
+    uint32_t tile0 = 0;
+    chain_of.place(matrices, arguments.output_size, arguments.input_size, blockIdx.x, arena + arguments.codes_offset,
+                   arena + arguments.exponents_offset, code_vectors, exponent_vector, (uint32_t)(uintptr_t)(lds_pointer)window, wave, lane, tile0);
+    float4_t chain[TILES][WIDE_COLUMN_BLOCKS];
+#pragma unroll
+    for (uint32_t t = 0; t < TILES; t++) {
+#pragma unroll
+        for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+            chain[t][j] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+    chain_of.whole(arguments.input_size / 128u, (tile.pair_count + 15u) / 16u, chain);
+    const uint32_t first_output = (blockIdx.x * WIDE_WAVES + wave) * STRIP_OUTPUTS;
+    if (first_output >= arguments.output_size) {
+        return;
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+        const uint32_t column = 16u * j + lane % 16u;
+        if (column < tile.pair_count) {
+            const uint64_t pair = pairs[column].pair_index;
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+                if ((tile0 + n) * 16u < first_output) {
+                    continue; /* a tile the strip before this one stores */
+                }
+                uint16_t *out = (uint16_t *)(arena + arguments.output_offset) + pair * arguments.output_size + (tile0 + n) * 16u + 4u * (lane / 16u);
+                const float s0 = __fadd_rn(0.0f, chain[n][j][0]), s1 = __fadd_rn(0.0f, chain[n][j][1]);
+                const float s2 = __fadd_rn(0.0f, chain[n][j][2]), s3 = __fadd_rn(0.0f, chain[n][j][3]);
+                *(uint2_t *)out = (uint2_t){(uint32_t)float_to_bf16(s0) | ((uint32_t)float_to_bf16(s1) << 16),
+                                            (uint32_t)float_to_bf16(s2) | ((uint32_t)float_to_bf16(s3) << 16)};
+            }
+        }
+    }
+}
+
+/* wide_expert_gate_up_1, wide_expert_down_1: the reference's entries, of WEIGHT_FORMAT_E2M1_SCALED experts; the _e4m3_
+ * entries take WEIGHT_FORMAT_E4M3_SCALED experts (no counterpart among the reference's expert kernels). The LDS window
+ * is dynamic shared memory (more than the 64 KB a kernel may declare): wide_gate_up_window_bytes and
+ * wide_down_window_bytes of anemone_records.h. */
+extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_gate_up_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
+{
+    wide_expert_gate_up<false>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_gate_up_1, wide_expert_gate_up_arguments);
+extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
+{
+    wide_expert_down<false>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_1, wide_expert_down_arguments);
+extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_gate_up_e4m3_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
+{
+    wide_expert_gate_up<true>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_gate_up_e4m3_1, wide_expert_gate_up_arguments);
+extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_e4m3_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
+{
+    wide_expert_down<true>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_e4m3_1, wide_expert_down_arguments);
+
+static_assert(wide_chain<2, false>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES &&
+                  wide_chain<1, false>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES && wide_chain<1, true>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES,
+              "the windows the host asks for are the kernels'");

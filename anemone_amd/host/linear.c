@@ -240,3 +240,123 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     memcpy(launches_out, launches, sizeof launches);
     return STATUS_OK;
 }
+
+/*
+ * The wide form: a grouped GEMM over the tiles of a wide select.
+ *
+ *   launch      kernel                       grid                                       block   dynamic LDS
+ *   gate/up     wide_expert_gate_up_1        (ceil(I / (4 strips)), tile_count, 1)      256     WIDE_GATE_UP_WINDOW_BYTES
+ *   down        wide_expert_down_1           (ceil(H / (4 strips)), tile_count, 1)      256     WIDE_DOWN_WINDOW_BYTES
+ *   row sum     expert_row_sum_entry         (ceil(H / 256), rows, 1)                   256
+ * strip = 64 outputs of E2M1 weights, 32 of E4M3.
+ */
+#define WIDE_MOST_ROWS 16384u
+
+result_status linear_wide_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                          uint32_t arithmetic_class, struct linear_wide_kernels_record *kernels_out)
+{
+    if (backend == NULL || backend->kernel_prepare == NULL || card == NULL || kernels_out == NULL ||
+        arithmetic_class != ARITHMETIC_CLASS_GFX950) {
+        REFUSE("the kernels of the wide linear: a missing argument, or a class other than %u", ARITHMETIC_CLASS_GFX950);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    static const struct {
+        const char *name;
+        uint32_t record_bytes;
+    } wanted[4] = {{KERNEL_WIDE_EXPERT_GATE_UP_STEM "1", sizeof(struct wide_expert_gate_up_arguments)},
+                   {KERNEL_WIDE_EXPERT_DOWN_STEM "1", sizeof(struct wide_expert_down_arguments)},
+                   {KERNEL_WIDE_EXPERT_GATE_UP_STEM "e4m3_1", sizeof(struct wide_expert_gate_up_arguments)},
+                   {KERNEL_WIDE_EXPERT_DOWN_STEM "e4m3_1", sizeof(struct wide_expert_down_arguments)}};
+    uint32_t handles[4];
+    for (uint32_t i = 0; i < 4u; i++) {
+        const result_status status = backend->kernel_prepare(card, KERNEL_FILE_WIDE_LINEAR, wanted[i].name, wanted[i].record_bytes, &handles[i]);
+        if (status != STATUS_OK) {
+            REFUSE("the kernels of the wide linear: %s is not prepared: %s", wanted[i].name, status_text(status));
+            return status;
+        }
+    }
+    memcpy(kernels_out, handles, sizeof handles);
+    return STATUS_OK;
+}
+
+result_status linear_wide_experts_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
+                                          const struct linear_kernels_record *linear_kernels,
+                                          const struct linear_wide_kernels_record *kernels, struct kernel_launch *launches_out)
+{
+    static const char what[] = "the wide routed experts";
+    if (description == NULL || linear_kernels == NULL || kernels == NULL || launches_out == NULL) {
+        REFUSE("%s: a missing argument", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct linear_routed_experts_description *experts = &description->experts;
+    const struct matrix_shape_record *gate_up = &experts->gate_up_shape, *down = &experts->down_shape;
+    const struct weight_format_operations *format = weight_format_operations_of(experts->weight_format);
+    const bool bytes = experts->weight_format == WEIGHT_FORMAT_E4M3_SCALED;
+    const uint32_t strip_outputs = bytes ? LINEAR_STRIP_OUTPUTS / 2u : LINEAR_STRIP_OUTPUTS;
+    uint64_t gate_up_bytes = 0, down_bytes = 0;
+    if (description->reserved_zero != 0 || experts->reserved_zero != 0 || (experts->weight_format != WEIGHT_FORMAT_E2M1_SCALED && !bytes) ||
+        format == NULL || format->stored_byte_count(gate_up, &gate_up_bytes) != STATUS_OK ||
+        format->stored_byte_count(down, &down_bytes) != STATUS_OK || gate_up->input_size % 128u != 0 || down->input_size % 128u != 0 ||
+        down->input_size != gate_up->output_size || gate_up->output_size < strip_outputs || down->output_size < strip_outputs ||
+        gate_up->output_size % 32u != 0) {
+        REFUSE("%s: matrices of format %u or %u in shapes it stores, inputs a multiple of 128, gate/up outputs of 32, at least %u outputs, "
+               "down reading what gate and up write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, (uint32_t)WEIGHT_FORMAT_E4M3_SCALED, strip_outputs);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (experts->gate_up_slice_count != 1u || experts->down_slice_count != 1u) {
+        REFUSE("%s: slice counts %u and %u: the wide products are built for one slice", what, experts->gate_up_slice_count,
+               experts->down_slice_count);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint32_t gate_up_kernel = bytes ? kernels->wide_expert_gate_up_e4m3 : kernels->wide_expert_gate_up;
+    const uint32_t down_kernel = bytes ? kernels->wide_expert_down_e4m3 : kernels->wide_expert_down;
+    if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL || linear_kernels->expert_row_sum == BACKEND_NO_KERNEL) {
+        REFUSE("%s: a kernel of the chain is not prepared", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t rows = experts->row_count, pairs = rows * experts->pairs_per_row;
+    if (rows == 0 || rows > WIDE_MOST_ROWS || experts->pairs_per_row == 0 || pairs > UINT32_MAX || description->tile_count == 0 ||
+        description->tile_count > 65535u || !(experts->activation_limit > 0.0f)) {
+        REFUSE("%s: 1 to %u rows, 1 to 65535 tiles, an activation limit above zero", what, WIDE_MOST_ROWS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t H = gate_up->input_size, I = gate_up->output_size, O = down->output_size;
+    const struct checked_range ranges[] = {
+        {"the tiles", description->tiles, (uint64_t)description->tile_count * sizeof(struct wide_expert_tile), false},
+        {"the sorted pairs", description->pairs, pairs * sizeof(struct wide_pair), false},
+        {"the experts' matrices", experts->expert_weights, gate_up_bytes > down_bytes ? gate_up_bytes : down_bytes, false},
+        {"the rows' codes", experts->codes, linear_codes_byte_count(rows, H), false},
+        {"the rows' exponents", experts->exponents, linear_exponents_byte_count(rows, H), false},
+        {"the rows' operands", experts->operands, 0, false},
+        {"the hidden codes", experts->hidden_codes, linear_codes_byte_count(pairs, I), false},
+        {"the hidden exponents", experts->hidden_exponents, linear_exponents_byte_count(pairs, I), false},
+        {"the hidden operands", experts->hidden_operands, linear_values_byte_count(pairs, I), false},
+        {"the pair outputs", experts->pair_output, linear_values_byte_count(pairs, O), false},
+        {"the row outputs", experts->row_output, linear_sums_byte_count(rows, O), false},
+    };
+    if (!ranges_are_valid(what, ranges, sizeof ranges / sizeof ranges[0], arena_byte_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct wide_expert_gate_up_arguments gate_up_record = {
+        description->tiles.byte_offset, description->pairs.byte_offset, experts->codes.byte_offset, experts->exponents.byte_offset,
+        experts->operands.byte_offset, experts->hidden_codes.byte_offset, experts->hidden_exponents.byte_offset,
+        experts->hidden_operands.byte_offset, gate_up->output_size, gate_up->input_size, description->tile_count,
+        experts->pairs_per_row, experts->activation_limit, (uint32_t)pairs};
+    const struct wide_expert_down_arguments down_record = {
+        description->tiles.byte_offset, description->pairs.byte_offset, experts->hidden_codes.byte_offset,
+        experts->hidden_exponents.byte_offset, experts->hidden_operands.byte_offset, experts->pair_output.byte_offset,
+        down->output_size, down->input_size, description->tile_count, (uint32_t)pairs};
+    const struct expert_row_sum_arguments row_sum_record = {experts->pair_output.byte_offset, experts->row_output.byte_offset,
+                                                            down->output_size, experts->pairs_per_row};
+    const uint32_t block_outputs = 4u * strip_outputs;
+    struct kernel_launch launches[LINEAR_WIDE_EXPERTS_LAUNCH_COUNT];
+    launch_fill(&launches[LINEAR_WIDE_EXPERTS_GATE_UP], gate_up_kernel, (gate_up->output_size + block_outputs - 1u) / block_outputs,
+                description->tile_count, 1, WIDE_BLOCK_THREADS, WIDE_GATE_UP_WINDOW_BYTES, &gate_up_record, sizeof gate_up_record);
+    launch_fill(&launches[LINEAR_WIDE_EXPERTS_DOWN], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
+                description->tile_count, 1, WIDE_BLOCK_THREADS, WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);
+    launch_fill(&launches[LINEAR_WIDE_EXPERTS_ROW_SUM], linear_kernels->expert_row_sum,
+                (down->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)rows, 1, LINEAR_ELEMENT_THREADS, 0,
+                &row_sum_record, sizeof row_sum_record);
+    memcpy(launches_out, launches, sizeof launches);
+    return STATUS_OK;
+}

@@ -269,6 +269,39 @@ MUST_CHECK result_status expert_producer_prepare(const struct linear_routed_expe
                                                  const struct linear_kernels_record *linear_kernels,
                                                  const struct expert_fused_kernels *kernels, struct kernel_launch *launch_out);
 
+/* ---- the wide form of the routed experts: a grouped GEMM over the tiles of a wide select ----
+ * The reference prepares its wide products from a description of the routed experts plus the tiles and sorted pairs
+ * of the router's wide select (struct expert_relaxed_description, include/anemone/expert_relaxed.h:79-99, for its
+ * class-80 order; the kernels of the reference order are source/kernel_wide_linear.cu). Here: the same description,
+ * three launches: wide_expert_gate_up_1 (gate with up, hidden step, quantization), wide_expert_down_1,
+ * expert_row_sum_entry. Slice counts must be 1 (the only instance built); the outputs are those of the job-table
+ * kernels of one slice, bit for bit. */
+struct linear_wide_kernels_record {
+    uint32_t wide_expert_gate_up; /* of one slice */
+    uint32_t wide_expert_down;
+    uint32_t wide_expert_gate_up_e4m3; /* extension: experts of WEIGHT_FORMAT_E4M3_SCALED */
+    uint32_t wide_expert_down_e4m3;
+};
+MUST_CHECK result_status linear_wide_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                                     uint32_t arithmetic_class, struct linear_wide_kernels_record *kernels_out);
+enum linear_wide_experts_launch {
+    LINEAR_WIDE_EXPERTS_GATE_UP = 0,
+    LINEAR_WIDE_EXPERTS_DOWN = 1,
+    LINEAR_WIDE_EXPERTS_ROW_SUM = 2,
+    LINEAR_WIDE_EXPERTS_LAUNCH_COUNT = 3
+};
+struct linear_wide_experts_description {
+    struct linear_routed_experts_description experts; /* the chain's arrays; jobs is not read (its range may be empty) */
+    struct linear_range tiles;                        /* read: struct wide_expert_tile [tile_count] */
+    struct linear_range pairs;                        /* read: struct wide_pair [row_count * pairs_per_row] */
+    uint32_t tile_count;                              /* grid[1] of the two products */
+    uint32_t reserved_zero;
+};
+MUST_CHECK result_status linear_wide_experts_prepare(const struct linear_wide_experts_description *description,
+                                                     uint64_t arena_byte_count, const struct linear_kernels_record *linear_kernels,
+                                                     const struct linear_wide_kernels_record *kernels,
+                                                     struct kernel_launch *launches_out);
+
 uint64_t linear_values_byte_count(uint64_t vector_count, uint64_t width);    /* bfloat16 [vector][width] */
 uint64_t linear_codes_byte_count(uint64_t vector_count, uint64_t width);     /* E4M3 [vector][width] */
 uint64_t linear_exponents_byte_count(uint64_t vector_count, uint64_t width); /* E8M0 [vector][width / 32] */

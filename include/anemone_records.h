@@ -467,6 +467,45 @@ struct expert_gate_up_quantize_arguments {
 };
 ANEMONE_RECORD_HAS(expert_gate_up_quantize_arguments, 96);
 
+/* ---- the wide products of the routed experts (include/anemone/wide_linear_records.h:80-118 of the reference) ---- */
+#define KERNEL_FILE_WIDE_LINEAR "kernel_wide_linear"
+#define KERNEL_WIDE_EXPERT_GATE_UP_STEM "wide_expert_gate_up_"
+#define KERNEL_WIDE_EXPERT_DOWN_STEM "wide_expert_down_"
+#define WIDE_BLOCK_THREADS 256u          /* four wavefronts: four strips of one tile of pairs */
+#define WIDE_GATE_UP_WINDOW_BYTES 129792u /* dynamic LDS of wide_expert_gate_up_<S>: three stages */
+#define WIDE_DOWN_WINDOW_BYTES 77568u     /* of wide_expert_down_<S> */
+struct wide_expert_gate_up_arguments {
+    uint64_t tiles_offset;            /* read: struct wide_expert_tile [tile_count] */
+    uint64_t pairs_offset;            /* read: struct wide_pair [pair_count] */
+    uint64_t codes_offset;            /* read: the rows' quantized input [row][input_size] */
+    uint64_t exponents_offset;
+    uint64_t operands_offset;
+    uint64_t hidden_codes_offset;     /* written [pair][output_size], of the tiles' pairs only */
+    uint64_t hidden_exponents_offset; /* written [pair][output_size / 32] */
+    uint64_t hidden_operands_offset;  /* written [pair][output_size] */
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t tile_count;
+    uint32_t pairs_per_row;
+    float activation_limit;
+    uint32_t pair_count;
+};
+ANEMONE_RECORD_HAS(wide_expert_gate_up_arguments, 88);
+
+struct wide_expert_down_arguments {
+    uint64_t tiles_offset;
+    uint64_t pairs_offset;
+    uint64_t codes_offset;     /* read: the pairs' quantized hidden [pair][input_size] */
+    uint64_t exponents_offset;
+    uint64_t operands_offset;
+    uint64_t output_offset;    /* written: bf16 [pair][output_size], of the tiles' pairs only */
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t tile_count;
+    uint32_t pair_count;
+};
+ANEMONE_RECORD_HAS(wide_expert_down_arguments, 64);
+
 struct expert_down_arguments {
     uint64_t jobs_offset;
     uint64_t codes_offset;     /* read: codes [pair][input_size] */

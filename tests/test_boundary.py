@@ -427,3 +427,63 @@ def test_linear_prepare_geometry_and_refusals(fake):
     assert lib.linear_quantize_prepare(C.byref(quantize), ARENA, C.byref(kernels), one) == 1
     shape, count = amd.Shape(2048, 4096, 4, 0), C.c_uint32(0)
     assert lib.linear_default_slice_count(1, 0, 0, C.byref(shape), 950, C.byref(count)) == 0 and count.value in (1, 2, 4, 8)
+
+
+def wide_experts_description(fmt=amd.WEIGHT_FORMAT_E2M1_SCALED, **changes):
+    rows, P, E = 1024, 8, 256
+    tile_count = amd.wide_tile_count(rows, P, E)
+    d = amd.LinearWideExpertsDescription()
+    d.experts = experts_description(fmt, row_count=rows, gate_up_slice_count=1, down_slice_count=1)
+    pairs, H, I = rows * P, 4096, 2048
+    cursor = [3 << 30]
+
+    def take(size):
+        at = cursor[0]
+        cursor[0] = (at + size + 255) // 256 * 256
+        return amd.Range(at, size)
+    e = d.experts
+    e.codes, e.exponents = take(rows * H), take(rows * H // 32)
+    e.hidden_codes, e.hidden_exponents, e.hidden_operands = take(pairs * I), take(pairs * I // 32), take(pairs * I * 2)
+    e.pair_output, e.row_output = take(pairs * H * 2), take(rows * H * 4)
+    d.tiles, d.pairs, d.tile_count = take(tile_count * 32), take(pairs * 8), tile_count
+    for key, value in changes.items():
+        if hasattr(d, key):
+            setattr(d, key, value)
+        else:
+            setattr(d.experts, key, value)
+    return d
+
+
+def test_wide_linear_prepare_geometry_and_refusals(fake):
+    lib = amd.library()
+    arena = 8 << 30
+    linear, kernels = amd.LinearKernels(), amd.LinearWideKernels()
+    assert lib.linear_kernels_prepare(fake.address, fake.card, 950, C.byref(linear)) == 0
+    assert lib.linear_wide_kernels_prepare(fake.address, fake.card, 90, C.byref(kernels)) == 1
+    assert lib.linear_wide_kernels_prepare(fake.address, fake.card, 950, C.byref(kernels)) == 0
+    table = kernel_table()
+    assert table[("kernel_wide_linear", "wide_expert_gate_up_1")] == C.sizeof(amd.WideExpertGateUpArguments) == 88
+    assert table[("kernel_wide_linear", "wide_expert_down_1")] == C.sizeof(amd.WideExpertDownArguments) == 64
+    launches = amd.launches_of(3)
+    assert lib.linear_wide_experts_prepare(C.byref(wide_experts_description()), arena, C.byref(linear), C.byref(kernels), launches) == 0
+    assert [fake.handles[l.kernel][1] for l in launches] == ["wide_expert_gate_up_1", "wide_expert_down_1", "expert_row_sum_entry"]
+    tiles = 1024 * 8 // 64 + 256
+    assert [list(l.grid) for l in launches] == [[8, tiles, 1], [16, tiles, 1], [16, 1024, 1]]
+    assert [l.block[0] for l in launches] == [256, 256, 256]
+    assert [l.dynamic_shared_byte_count for l in launches] == [129792, 77568, 0]
+    assert [l.argument_byte_count for l in launches] == [88, 64, 24]
+    record = amd.WideExpertGateUpArguments.from_buffer_copy(bytes(launches[0].argument)[:88])
+    assert (record.output_size, record.input_size, record.tile_count, record.pairs_per_row, record.pair_count) == (2048, 4096, tiles, 8, 8192)
+    fp8 = amd.launches_of(3)
+    description = wide_experts_description(amd.WEIGHT_FORMAT_E4M3_SCALED)
+    assert lib.linear_wide_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(kernels), fp8) == 0
+    assert [fake.handles[l.kernel][1] for l in fp8][:2] == ["wide_expert_gate_up_e4m3_1", "wide_expert_down_e4m3_1"]
+    assert [list(l.grid) for l in fp8][:2] == [[16, tiles, 1], [32, tiles, 1]]  # strips of 32 outputs
+    for changes in (dict(gate_up_slice_count=2), dict(down_slice_count=4), dict(tile_count=0), dict(tile_count=70000), dict(reserved_zero=1),
+                    dict(row_count=0), dict(row_count=20000), dict(activation_limit=0.0), dict(weight_format=amd.WEIGHT_FORMAT_EXL3),
+                    dict(tiles=amd.Range(3 << 30, 64)), dict(pairs=amd.Range((8 << 30) - 256, 65536)),
+                    dict(gate_up_shape=amd.Shape(2048, 4000, 4, 0)), dict(down_shape=amd.Shape(4096, 1024, 4, 0))):
+        untouched = amd.launches_of(3)
+        status = lib.linear_wide_experts_prepare(C.byref(wide_experts_description(**changes)), arena, C.byref(linear), C.byref(kernels), untouched)
+        assert status == 1, changes
+        assert not any(bytes(untouched))
