@@ -28,9 +28,9 @@
 #define WIDE_VECTOR_BYTES (WIDE_TILE_PAIRS * 128u) /* a K step of the tile's columns' codes */
 
 /* One block's pipeline: MATRICES matrices x STRIP tiles a wavefront, the tile's columns shared. */
-template <uint32_t MATRICES, bool BYTES>
+template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES>
 struct wide_chain {
-    static constexpr uint32_t STRIP = BYTES ? 2u : 4u;
+    static constexpr uint32_t STRIP = STRIP_TILES;
     static constexpr uint32_t STEP_BYTES = BYTES ? BYTE_STEP_BYTES : NIBBLE_STEP_BYTES;
     static constexpr uint32_t TILE_LOADS = STEP_BYTES / 1024u;
     static constexpr uint32_t TILES = MATRICES * STRIP;
@@ -40,16 +40,26 @@ struct wide_chain {
     static constexpr uint32_t VECTOR_SCALE_AT = VECTOR_AT + WIDE_VECTOR_BYTES;
     static constexpr uint32_t STAGE_BYTES = VECTOR_SCALE_AT + 256u;
     static constexpr uint32_t WINDOW_BYTES = WIDE_DEPTH * STAGE_BYTES;
-    static constexpr uint32_t STAGE_LOADS = TILES * TILE_LOADS + MATRICES + 2u + 1u; /* a wavefront's loads a stage */
+    static constexpr uint32_t VECTOR_LOADS = 2u + 1u;                            /* issued first: two column groups, the scale words */
+    static constexpr uint32_t WEIGHT_LOADS = TILES * TILE_LOADS + MATRICES;
+    static constexpr uint32_t STAGE_LOADS = VECTOR_LOADS + WEIGHT_LOADS;         /* a wavefront's loads a stage */
     static_assert(STAGE_LOADS * (WIDE_DEPTH - 1u) < 64u && WINDOW_BYTES <= 160u * 1024u, "vmcnt has six bits; LDS 160 KB");
 
     const unsigned char *words[MATRICES], *scales[MATRICES], *codes, *exponents;
     uint32_t tile_bytes, window, wave, piece_offset, scale_offset, codes_offset[2], exponents_offset;
-    uint32_t read_at[BYTES ? 8 : 4], scale_at[STRIP], vector_at[BYTES ? 8 : 4], vector_scale_at, shift;
+    uint32_t read_at[BYTES ? 8 : 4], scale_at[STRIP], vector_at[BYTES ? 8 : 4], vector_scale_at, operand_at, shift;
 
     __device__ __forceinline__ void issue(uint32_t stage, uint32_t at) const
     {
         const uint32_t base = window + stage * STAGE_BYTES, mine = base + wave * WAVE_BYTES;
+        /* first the tile's columns (this wavefront waits for them a step before the weights): eight groups of eight
+         * columns, two a wavefront: the column block it prepares; every wavefront brings the scale words (the same
+         * bytes to the same place: one load more a wavefront, and all wavefronts count alike) */
+#pragma unroll
+        for (uint32_t part = 0; part < 2u; part++) {
+            load_to_lds_16(codes + (uint64_t)at * 128u, codes_offset[part], base + VECTOR_AT + (2u * wave + part) * 1024u);
+        }
+        load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT);
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
 #pragma unroll
@@ -65,13 +75,6 @@ struct wide_chain {
         for (uint32_t m = 0; m < MATRICES; m++) {
             load_to_lds_4(scales[m] + (uint64_t)at * (BYTES ? 4u : 64u), scale_offset, mine + SCALES_AT + m * 256u);
         }
-        /* the tile's columns: eight groups of eight columns, two a wavefront; every wavefront brings the scale words
-         * (the same bytes to the same place: one load more a wavefront, and all wavefronts count alike) */
-#pragma unroll
-        for (uint32_t part = 0; part < 2u; part++) {
-            load_to_lds_16(codes + (uint64_t)at * 128u, codes_offset[part], base + VECTOR_AT + (2u * wave + part) * 1024u);
-        }
-        load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT);
     }
 
     template <typename T>
@@ -80,85 +83,164 @@ struct wide_chain {
         return *(const __attribute__((address_space(3))) T *)(uintptr_t)address;
     }
 
-    __device__ __forceinline__ void consume(uint32_t stage, uint32_t live_blocks, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
+    template <typename T>
+    __device__ static __forceinline__ void lds_write(uint32_t address, T value)
     {
-        const uint32_t base = window + stage * STAGE_BYTES, mine = base + wave * WAVE_BYTES;
-        int8_vector b[WIDE_COLUMN_BLOCKS];
-        uint32_t scale_b[WIDE_COLUMN_BLOCKS];
+        *(__attribute__((address_space(3))) T *)(uintptr_t)address = value;
+    }
+
+    /* The wavefront's own column block of a stage, from the codes as they landed (a column's 128 bytes in the order the
+     * quantizer writes them) to the MFMA's operand, in place: [half of the operand][lane][16 bytes], which every
+     * wavefront then reads with two 16-byte reads a lane and no bank conflict. Only this wavefront touches the block
+     * before the next barrier. */
+    __device__ __forceinline__ void prepare_columns(uint32_t stage) const
+    {
+        uint32_t at = window + stage * STAGE_BYTES + VECTOR_AT + wave * 2048u;
+        asm volatile("" : "+s"(at));
+        int8_vector b;
+        if constexpr (BYTES) {
 #pragma unroll
-        for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
-            if (j < live_blocks) { /* the same in every lane */
-                if constexpr (BYTES) {
-#pragma unroll
-                    for (uint32_t v = 0; v < 8u; v++) {
-                        b[j][v] = (int)lds_read<uint32_t>(base + VECTOR_AT + j * 2048u + vector_at[v]);
-                    }
-                } else {
-#pragma unroll
-                    for (uint32_t part = 0; part < 4u; part++) {
-                        const uint2_t pair = lds_read<uint2_t>(base + VECTOR_AT + j * 2048u + vector_at[part]);
-                        b[j][2u * part] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x05010400u);
-                        b[j][2u * part + 1u] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x07030602u);
-                    }
-                }
-                scale_b[j] = lds_read<unsigned char>(base + VECTOR_SCALE_AT + j * 64u + vector_scale_at);
+            for (uint32_t v = 0; v < 8u; v++) {
+                b[v] = (int)lds_read<uint32_t>(at + vector_at[v]);
             }
+        } else {
+#pragma unroll
+            for (uint32_t part = 0; part < 4u; part++) {
+                const uint2_t pair = lds_read<uint2_t>(at + vector_at[part]);
+                b[2u * part] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x05010400u);
+                b[2u * part + 1u] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x07030602u);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* every lane has read before any lane writes */
+        lds_write<uint4_t>(at + operand_at, (uint4_t){(uint32_t)b[0], (uint32_t)b[1], (uint32_t)b[2], (uint32_t)b[3]});
+        lds_write<uint4_t>(at + operand_at + 1024u, (uint4_t){(uint32_t)b[4], (uint32_t)b[5], (uint32_t)b[6], (uint32_t)b[7]});
+    }
+
+    /* one K step of LIVE column blocks (a constant: the MFMAs of a step stay one straight line) */
+    template <uint32_t LIVE>
+    __device__ __forceinline__ void consume(uint32_t stage, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
+    {
+        /* the stage's addresses, once a step: every read below is one of them plus a constant */
+        uint32_t base = window + stage * STAGE_BYTES, mine = base + wave * WAVE_BYTES;
+        asm volatile("" : "+s"(base), "+s"(mine));
+        uint32_t a_at[BYTES ? 8 : 4], a_scale_at[STRIP], b_at = base + operand_at, b_scale_at = base + vector_scale_at;
+#pragma unroll
+        for (uint32_t v = 0; v < (BYTES ? 8u : 4u); v++) {
+            a_at[v] = mine + read_at[v];
+            asm volatile("" : "+v"(a_at[v]));
+        }
+#pragma unroll
+        for (uint32_t n = 0; n < STRIP; n++) {
+            a_scale_at[n] = mine + scale_at[n];
+            asm volatile("" : "+v"(a_scale_at[n]));
+        }
+        asm volatile("" : "+v"(b_at), "+v"(b_scale_at));
+        int8_vector b[LIVE];
+        uint32_t scale_b[LIVE];
+#pragma unroll
+        for (uint32_t j = 0; j < LIVE; j++) {
+            const uint4_t low = lds_read<uint4_t>(b_at + VECTOR_AT + j * 2048u), high = lds_read<uint4_t>(b_at + VECTOR_AT + j * 2048u + 1024u);
+            b[j] = (int8_vector){(int)low.x, (int)low.y, (int)low.z, (int)low.w, (int)high.x, (int)high.y, (int)high.z, (int)high.w};
+            scale_b[j] = lds_read<unsigned char>(b_scale_at + VECTOR_SCALE_AT + j * 64u);
         }
 #pragma unroll
         for (uint32_t tile = 0; tile < TILES; tile++) {
             int8_vector a = {0, 0, 0, 0, 0, 0, 0, 0};
-            const uint32_t scale_a = lds_read<unsigned char>(mine + SCALES_AT + (tile / STRIP) * 256u + scale_at[tile % STRIP]);
+            const uint32_t scale_a = lds_read<unsigned char>(a_scale_at[tile % STRIP] + SCALES_AT + (tile / STRIP) * 256u);
             if constexpr (BYTES) {
 #pragma unroll
                 for (uint32_t v = 0; v < 8u; v++) {
-                    const uint2_t w = lds_read<uint2_t>(mine + tile * STEP_BYTES + read_at[v]);
+                    const uint2_t w = lds_read<uint2_t>(a_at[v] + tile * STEP_BYTES);
                     a[v] = (int)__builtin_amdgcn_perm(w.y, w.x, shift);
                 }
             } else {
 #pragma unroll
                 for (uint32_t T = 0; T < 4u; T++) {
-                    const uint2_t w = lds_read<uint2_t>(mine + tile * STEP_BYTES + read_at[T]);
-                    a[T] = (int)(((w.x >> shift) & NIBBLE_MASK) | (((w.y >> shift) & NIBBLE_MASK) << 4));
+                    /* a byte of the result: the output's nibble of w.x below that of w.y. Rotating w.x right by 0 or 4
+                     * and w.y left by 4 or 0 puts them there; the mask picks */
+                    const uint2_t w = lds_read<uint2_t>(a_at[T] + tile * STEP_BYTES);
+                    const uint32_t low = __builtin_amdgcn_alignbit(w.x, w.x, shift), high = __builtin_amdgcn_alignbit(w.y, w.y, 28u + shift);
+                    a[T] = (int)((low & NIBBLE_MASK) | (high & ~NIBBLE_MASK));
                 }
             }
 #pragma unroll
-            for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
-                if (j < live_blocks) {
-                    if constexpr (BYTES) {
-                        chain[tile][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b[j], chain[tile][j], 0, 0, 0, (int)scale_a, 0, (int)scale_b[j]);
-                    } else {
-                        chain[tile][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b[j], chain[tile][j], 4, 0, 0, (int)scale_a, 0, (int)scale_b[j]);
-                    }
+            for (uint32_t j = 0; j < LIVE; j++) {
+                if constexpr (BYTES) {
+                    chain[tile][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b[j], chain[tile][j], 0, 0, 0, (int)scale_a, 0, (int)scale_b[j]);
+                } else {
+                    chain[tile][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b[j], chain[tile][j], 4, 0, 0, (int)scale_a, 0, (int)scale_b[j]);
                 }
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stage is read before the next barrier */
     }
 
-    /* all `total` K steps; every wavefront of the block calls it (barriers inside) */
-    __device__ __forceinline__ void whole(uint32_t total, uint32_t live_blocks, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
+    /* K step `step` of `total`, in stage `stage`; AHEAD = how many steps follow it, capped at 2 (a constant, so that
+     * the steady loop carries no test) */
+    template <uint32_t LIVE, uint32_t AHEAD>
+    __device__ __forceinline__ void one_step(uint32_t step, uint32_t stage, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
+    {
+        /* loads complete in the order they are issued: "at most N outstanding" names the oldest that have landed.
+         * This step's have landed once nothing but the later step's is outstanding */
+        wait_loads<AHEAD >= 1u ? STAGE_LOADS : 0u>();
+        /* behind this barrier every wavefront's weights and prepared column block of this step are in LDS, and
+         * every wavefront has read the step before: its stage may be asked for again */
+        __syncthreads();
+        const uint32_t behind = stage == 0u ? WIDE_DEPTH - 1u : stage - 1u, ahead = stage + 1u == WIDE_DEPTH ? 0u : stage + 1u;
+        if constexpr (AHEAD >= 2u) {
+            issue(behind, step + 2u);
+        }
+        consume<LIVE>(stage, chain);
+        if constexpr (AHEAD >= 1u) { /* the next step's columns, which this wavefront asked for, have landed: prepare them */
+            wait_loads<WEIGHT_LOADS + (AHEAD >= 2u ? STAGE_LOADS : 0u)>();
+            prepare_columns(ahead);
+        }
+    }
+
+    /* all `total` K steps of LIVE live column blocks; every wavefront of the block calls it (barriers inside) */
+    template <uint32_t LIVE>
+    __device__ __forceinline__ void steps(uint32_t total, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
     {
         static_assert(WIDE_DEPTH == 3u, "the waits are written out for two stages ahead");
-#pragma unroll
-        for (uint32_t ahead = 0; ahead + 1u < WIDE_DEPTH; ahead++) {
-            if (ahead < total) {
-                issue(ahead, ahead);
-            }
+        issue(0u, 0u);
+        if (total > 1u) {
+            issue(1u, 1u);
+            wait_loads<WEIGHT_LOADS + STAGE_LOADS>();
+        } else {
+            wait_loads<WEIGHT_LOADS>();
         }
-        for (uint32_t step = 0; step < total; step++) {
-            /* this step's loads have landed once nothing but the later steps' (one stage at most here) is outstanding */
-            if (step + 1u < total) {
-                wait_loads<STAGE_LOADS>();
-            } else {
-                wait_loads<0>();
-            }
-            /* behind this barrier every wavefront's column groups of this step have landed, and every wavefront has
-             * read the step before: its stage may be asked for again */
-            __syncthreads();
-            if (step + WIDE_DEPTH - 1u < total) {
-                issue((step + WIDE_DEPTH - 1u) % WIDE_DEPTH, step + WIDE_DEPTH - 1u);
-            }
-            consume(step % WIDE_DEPTH, live_blocks, chain);
+        prepare_columns(0u);
+        uint32_t stage = 0, step = 0;
+        for (; step + 2u < total; step++) {
+            one_step<LIVE, 2u>(step, stage, chain);
+            stage = stage + 1u == WIDE_DEPTH ? 0u : stage + 1u;
+        }
+        if (step + 1u < total) {
+            one_step<LIVE, 1u>(step, stage, chain);
+            stage = stage + 1u == WIDE_DEPTH ? 0u : stage + 1u;
+            step++;
+        }
+        one_step<LIVE, 0u>(step, stage, chain);
+    }
+
+    /* live_blocks: the tile's column blocks that hold a pair, the same in every lane of the block; the sums of the
+     * others stay what they were */
+    __device__ __forceinline__ void whole(uint32_t total, uint32_t live_blocks, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
+    {
+        static_assert(WIDE_COLUMN_BLOCKS == 4u, "one instance a count of live column blocks");
+        switch (live_blocks) {
+        case 1u:
+            steps<1>(total, chain);
+            break;
+        case 2u:
+            steps<2>(total, chain);
+            break;
+        case 3u:
+            steps<3>(total, chain);
+            break;
+        default:
+            steps<4>(total, chain);
+            break;
         }
     }
 
@@ -211,7 +293,8 @@ struct wide_chain {
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + (uint64_t)tile0 * loads * 32u;
             }
             piece_offset = 16u * (lane ^ (2u * ((lane >> 4) & 1u) + ((lane >> 5) & 1u)));
-            scale_offset = (lane / 16u) * (loads * 32u) + (lane % 16u) * 4u;
+            /* lanes past the strip's tiles read its last tile's words again */
+            scale_offset = (lane / 16u < STRIP ? lane / 16u : STRIP - 1u) * (loads * 32u) + (lane % 16u) * 4u;
 #pragma unroll
             for (uint32_t T = 0; T < 4u; T++) {
                 read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (2u * (G / 4u) + ld))) + 8u * q;
@@ -243,6 +326,7 @@ struct wide_chain {
             }
         }
         vector_scale_at = 4u * o + g;
+        operand_at = 16u * lane;
     }
 };
 
@@ -250,7 +334,7 @@ struct wide_chain {
 template <bool BYTES>
 __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_expert_gate_up_arguments &arguments, unsigned char *arena)
 {
-    typedef wide_chain<2, BYTES> chain_type;
+    typedef wide_chain<2, BYTES, 2u> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     static_assert(chain_type::WAVE_BYTES >= WIDE_TILE_PAIRS * STRIP_OUTPUTS * 2u, "a wavefront's hidden values fit its idle part of a stage");
@@ -313,23 +397,26 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
     if (first_output >= width) {
         return; /* a strip wholly past the matrix */
     }
-    for (uint32_t column = 0; column < tile.pair_count; column++) {
+    /* a column's strip is STRIP_OUTPUTS values: a wavefront quantizes WAVE / STRIP_OUTPUTS columns at a time, a block
+     * of 32 outputs in 32 consecutive lanes */
+    static_assert(STRIP_OUTPUTS == 32u || STRIP_OUTPUTS == 64u, "whole columns a pass of the wavefront");
+    constexpr uint32_t TOGETHER = WAVE / STRIP_OUTPUTS;
+    const uint32_t at = lane % STRIP_OUTPUTS;
+    if (tile0 * 16u + at < first_output) {
+        return; /* whole blocks of 32 that the strip before this one takes (the same in the 32 lanes of a block) */
+    }
+    for (uint32_t column = lane / STRIP_OUTPUTS; column < tile.pair_count; column += TOGETHER) {
         const uint64_t pair = pairs[column].pair_index;
-        for (uint32_t at = lane; at < STRIP_OUTPUTS; at += WAVE) {
-            if (tile0 * 16u + at < first_output) {
-                continue; /* whole blocks of 32 that the strip before this one takes */
-            }
-            quantize_value(strip_hidden[column * STRIP_OUTPUTS + at], tile0 * 16u + at, arena + arguments.hidden_codes_offset + pair * width,
-                           arena + arguments.hidden_exponents_offset + pair * (width / 32u),
-                           (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width);
-        }
+        quantize_value(strip_hidden[column * STRIP_OUTPUTS + at], tile0 * 16u + at, arena + arguments.hidden_codes_offset + pair * width,
+                       arena + arguments.hidden_exponents_offset + pair * (width / 32u),
+                       (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width);
     }
 }
 
 template <bool BYTES>
 __device__ static __forceinline__ void wide_expert_down(const struct wide_expert_down_arguments &arguments, unsigned char *arena)
 {
-    typedef wide_chain<1, BYTES> chain_type;
+    typedef wide_chain<1, BYTES, (BYTES ? 2u : 4u)> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
@@ -408,6 +495,6 @@ extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_e4m3
 }
 ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_e4m3_1, wide_expert_down_arguments);
 
-static_assert(wide_chain<2, false>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES &&
-                  wide_chain<1, false>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES && wide_chain<1, true>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES,
+static_assert(wide_chain<2, false, 2u>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true, 2u>::WINDOW_BYTES == WIDE_GATE_UP_E4M3_WINDOW_BYTES &&
+                  wide_chain<1, false, 4u>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES && wide_chain<1, true, 2u>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES,
               "the windows the host asks for are the kernels'");

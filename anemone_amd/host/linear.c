@@ -245,7 +245,7 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
  * The wide form: a grouped GEMM over the tiles of a wide select.
  *
  *   launch      kernel                       grid                                       block   dynamic LDS
- *   gate/up     wide_expert_gate_up_1        (ceil(I / (4 strips)), tile_count, 1)      256     WIDE_GATE_UP_WINDOW_BYTES
+ *   gate/up     wide_expert_gate_up_1        (ceil(I / 128), tile_count, 1)             256     WIDE_GATE_UP_WINDOW_BYTES
  *   down        wide_expert_down_1           (ceil(H / (4 strips)), tile_count, 1)      256     WIDE_DOWN_WINDOW_BYTES
  *   row sum     expert_row_sum_entry         (ceil(H / 256), rows, 1)                   256
  * strip = 64 outputs of E2M1 weights, 32 of E4M3.
@@ -350,8 +350,9 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
                                                             down->output_size, experts->pairs_per_row};
     const uint32_t block_outputs = 4u * strip_outputs;
     struct kernel_launch launches[LINEAR_WIDE_EXPERTS_LAUNCH_COUNT];
-    launch_fill(&launches[LINEAR_WIDE_EXPERTS_GATE_UP], gate_up_kernel, (gate_up->output_size + block_outputs - 1u) / block_outputs,
-                description->tile_count, 1, WIDE_BLOCK_THREADS, WIDE_GATE_UP_WINDOW_BYTES, &gate_up_record, sizeof gate_up_record);
+    launch_fill(&launches[LINEAR_WIDE_EXPERTS_GATE_UP], gate_up_kernel,
+                (gate_up->output_size + WIDE_GATE_UP_BLOCK_OUTPUTS - 1u) / WIDE_GATE_UP_BLOCK_OUTPUTS, description->tile_count, 1,
+                WIDE_BLOCK_THREADS, bytes ? WIDE_GATE_UP_E4M3_WINDOW_BYTES : WIDE_GATE_UP_WINDOW_BYTES, &gate_up_record, sizeof gate_up_record);
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_DOWN], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
                 description->tile_count, 1, WIDE_BLOCK_THREADS, WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_ROW_SUM], linear_kernels->expert_row_sum,

@@ -71,13 +71,14 @@ def calibrate(amd):
                       "GBps_read_plus_write": 2 * size / (min(times) * 1e-6) / 1e9}))
 
 
-def fp4_decode(amd, workloads, arguments, fp8=False):
-    """Secondary workloads: the same layer shape with the original FP4 weights (E2M1 codes, one E8M0 scale per 32
+def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
+    """Secondary workloads (with `prefill`, the wide form: --rows defaults to 8192 tokens of FP4 weights, 2048 of FP8;
+    the wide select's tiles, wide gate/up with the quantization fused, wide down, row sum; the roofline is the MFMA's): the same layer shape with the original FP4 weights (E2M1 codes, one E8M0 scale per 32
     inputs) or FP8 weights (E4M3 codes, one E8M0 scale per 32 x 32), a decode step of `--rows` tokens (32 by default):
     quantizer, router, and the four launches of the routed experts. A few distinct seeded experts are generated and laid
     at 256 distinct places of the arena."""
     import ctypes as C
-    rows = arguments.rows
+    rows = arguments.rows if not prefill or arguments.rows != 32 else 2048 if fp8 else 8192
     distinct_generated = 4 if fp8 else 16
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
     matrix = workloads.fp8_matrix if fp8 else workloads.fp4_matrix
@@ -86,21 +87,27 @@ def fp4_decode(amd, workloads, arguments, fp8=False):
     matrices = [trios[e % distinct_generated] for e in range(EXPERTS)]
     router = workloads.to_bf16(workloads.normals(base + 2, EXPERTS * HIDDEN) * 0.02).reshape(EXPERTS, HIDDEN)
     x = workloads.activations(4, rows, HIDDEN)
-    card = amd.Card((9 if fp8 else 5) << 30)
+    card = amd.Card(((9 if fp8 else 5) << 30) + rows * (1 << 18))
     layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router,
                          gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices,
                          weight_format=amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED)
     layer.set_rows(x, rows)
-    wide = layer.wide_router() if rows > 8 else None  # more than eight rows: the wide select sorts the pairs by expert
+    wide = layer.wide_router() if rows > 8 or prefill else None  # more than eight rows: the wide select sorts the pairs by expert
     routing = [layer.select_launch(0)[0]] if wide is None else list(wide.launches())
     routing_names = ["router_select_entry"] if wide is None else ["router_wide_select", "router_wide_count", "router_wide_place", "router_wide_jobs"]
-    experts = layer.expert_launches(wide)
-    parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(4)]
+    if prefill:
+        routing, routing_names = routing[:3], routing_names[:3]  # the tiles are the place's; no job table
+        experts = layer.wide_expert_launches(wide)
+        parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(3)]
+        names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "expert_down", "expert_row_sum_entry"]
+    else:
+        experts = layer.expert_launches(wide)
+        parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(4)]
+        names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
+                                                         "expert_down", "expert_row_sum_entry"]
     step = amd.launches_of(len(parts))
     for i, launch in enumerate(parts):
         step[i] = launch
-    names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
-                                                     "expert_down", "expert_row_sum_entry"]
     for _ in range(arguments.warmup):
         card.run(step, wait=False)
     card.wait()
@@ -110,9 +117,15 @@ def fp4_decode(amd, workloads, arguments, fp8=False):
     for _ in range(arguments.steps):
         per_launch += np.array(card.run_timed(step))
     per_launch /= arguments.steps
-    jobs = layer.jobs() if wide is None else wide.read("jobs", amd.JOB_DTYPE)
-    live = jobs[jobs["row_count"] > 0]
-    distinct = np.unique(live["expert"])
+    if prefill:
+        picks = wide.read("picks", np.dtype([("expert", "<u4"), ("route_weight", "<f4")])).reshape(rows, PICKS)
+        tiles = wide.read("tiles", amd.WIDE_TILE_DTYPE)
+        live = tiles[tiles["pair_count"] > 0]
+        distinct = np.unique(picks["expert"])
+    else:
+        jobs = layer.jobs() if wide is None else wide.read("jobs", amd.JOB_DTYPE)
+        live = jobs[jobs["row_count"] > 0]
+        distinct = np.unique(live["expert"])
     matrix_bytes = HIDDEN * INNER + HIDDEN * INNER // 1024 if fp8 else HIDDEN * INNER // 2 + HIDDEN * INNER // 32
     gate_up_bytes = 2 * matrix_bytes * len(distinct)
     gate_up_us = float(per_launch[names.index("expert_gate_up")])
@@ -133,13 +146,28 @@ def fp4_decode(amd, workloads, arguments, fp8=False):
                      "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
     }
+    if prefill:
+        pairs = rows * PICKS
+        gate_up_flops, down_flops = 2.0 * pairs * 2 * HIDDEN * INNER, 2.0 * pairs * HIDDEN * INNER
+        achieved = gate_up_flops / (gate_up_us * 1e-6) / 1e12
+        result["config"]["workload"] = result["config"]["workload"].replace("_moe_decode", "_moe_prefill")
+        result["config"]["tiles"] = result["config"].pop("jobs")
+        result["config"].pop("down_GBps")
+        result["config"]["down_TFLOPs"] = down_flops / (down_us * 1e-6) / 1e12
+        result["config"]["step_TFLOPs"] = (gate_up_flops + down_flops) / (seconds / arguments.steps) / 1e12
+        # the products are MFMAs of FP8 activations (with FP4 or FP8 weights): the FP8 rate is the instruction's peak
+        result["roofline"] = {"bound": "mfma", "kernel": "wide_expert_gate_up_%s1" % ("e4m3_" if fp8 else ""), "achieved": achieved,
+                              "peak": MFMA_F8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": None,
+                              "algorithmic_flops_per_launch": gate_up_flops, "launch_us": gate_up_us}
     if not arguments.no_cpu:
         import _oracle as o
         threads = min(os.cpu_count() or 1, 16)
         sample = min(rows, 4)
         experts_of = np.zeros((rows, PICKS), dtype=np.uint32)
         weights_of = np.zeros((rows, PICKS), dtype=np.float32)
-        for job in live:
+        if prefill:
+            experts_of[:], weights_of[:] = picks["expert"], picks["route_weight"]
+        for job in ([] if prefill else live):
             for c in range(job["row_count"]):
                 experts_of.reshape(-1)[job["pair_index"][c]] = job["expert"]
                 weights_of.reshape(-1)[job["pair_index"][c]] = job["route_weight"][c]
@@ -162,6 +190,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False):
 
 
 MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_F8_PEAK_TFLOPS = 5000.0
 
 
 def exl3_prefill(amd, workloads, arguments):
@@ -266,7 +295,7 @@ def main():
     if arguments.gpus != 1:
         print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
         sys.exit(2)
-    if arguments.workload not in ("exl3_decode", "fp4_decode", "fp8_decode", "exl3_prefill"):
+    if arguments.workload not in ("exl3_decode", "fp4_decode", "fp8_decode", "exl3_prefill", "fp4_prefill", "fp8_prefill"):
         print("unknown workload %s" % arguments.workload, file=sys.stderr)
         sys.exit(2)
 
@@ -279,8 +308,8 @@ def main():
     if arguments.workload == "exl3_prefill":
         exl3_prefill(amd, workloads, arguments)
         return
-    if arguments.workload in ("fp4_decode", "fp8_decode"):
-        fp4_decode(amd, workloads, arguments, fp8=arguments.workload == "fp8_decode")
+    if arguments.workload in ("fp4_decode", "fp8_decode", "fp4_prefill", "fp8_prefill"):
+        fp4_decode(amd, workloads, arguments, fp8=arguments.workload.startswith("fp8"), prefill=arguments.workload.endswith("prefill"))
         return
 
     widths, matrices, router = workloads.exl3_moe_layer(CONFIG, HIDDEN, INNER, EXPERTS)
