@@ -306,23 +306,25 @@ struct wide_chain {
             shift = 4u * parity;
         }
         /* the columns' codes: lane L of a load holds slot L % 8 of column L / 8 of its group of eight and asks for
-         * that column's piece (L % 8) ^ (L / 8); a column block of 16 columns is two groups (2,048 bytes) */
+         * that column's piece (L % 8) ^ (L / 8) ^ (the group's parity); a column block of 16 columns is two groups
+         * (2,048 bytes). With the parity the 32 lanes of a pass of prepare_columns' reads fall on every bank pair of
+         * their half twice, not four times */
 #pragma unroll
         for (uint32_t part = 0; part < 2u; part++) {
-            codes_offset[part] = code_vectors[part] * inputs + 16u * ((lane % 8u) ^ (lane / 8u));
+            codes_offset[part] = code_vectors[part] * inputs + 16u * ((lane % 8u) ^ (lane / 8u) ^ part);
         }
         exponents_offset = exponent_vector * (inputs / 32u);
         const uint32_t column = o % 8u, group_bytes = (o / 8u) * 1024u;
         if constexpr (BYTES) {
 #pragma unroll
             for (uint32_t v = 0; v < 8u; v++) {
-                vector_at[v] = group_bytes + 16u * (8u * column + (v ^ column)) + 4u * g;
+                vector_at[v] = group_bytes + 16u * (8u * column + (v ^ column ^ (o / 8u))) + 4u * g;
             }
         } else {
 #pragma unroll
             for (uint32_t part = 0; part < 4u; part++) {
                 const uint32_t piece = 4u * (part / 2u) + part % 2u + 2u * (g % 2u);
-                vector_at[part] = group_bytes + 16u * (8u * column + (piece ^ column)) + 8u * (g / 2u);
+                vector_at[part] = group_bytes + 16u * (8u * column + (piece ^ column ^ (o / 8u))) + 8u * (g / 2u);
             }
         }
         vector_scale_at = 4u * o + g;

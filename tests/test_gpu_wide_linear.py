@@ -57,7 +57,10 @@ def build(amd, card, hidden, inner, experts_n, picks, rows, seed, fmt, distinct=
     (512, 256, 64, 8, 40, 40, E2M1),      # most tiles hold a few pairs
     (512, 256, 64, 4, 300, 300, E4M3),
     (640, 384, 64, 2, 450, 449, E4M3),
-    (512, 256, 64, 1, 700, 700, E2M1),    # long runs: experts of several full tiles
+    (512, 256, 64, 1, 700, 700, E2M1),    # one pick a row
+    (512, 256, 64, 8, 1500, 1500, E2M1),  # runs of three tiles and more: blocks of two tiles of one expert, and a run's odd last tile
+    (640, 384, 64, 8, 1100, 1003, E2M1),
+    (512, 256, 64, 8, 1500, 1401, E4M3),
 ])
 def test_wide_equals_the_job_table_kernels_byte_for_byte(amd, card, hidden, inner, experts_n, picks, rows, live, fmt):
     say("wide experts", hidden, inner, experts_n, picks, rows, live, fmt)
