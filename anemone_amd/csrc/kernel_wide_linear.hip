@@ -339,7 +339,6 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
     typedef wide_chain<2, BYTES, 2u> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
-    static_assert(chain_type::WAVE_BYTES >= WIDE_TILE_PAIRS * STRIP_OUTPUTS * 2u, "a wavefront's hidden values fit its idle part of a stage");
     const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
     if (tile.pair_count == 0u) {
         return;
@@ -370,48 +369,62 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
     }
     const uint32_t live_blocks = (tile.pair_count + 15u) / 16u;
     chain_of.whole(arguments.input_size / 128u, live_blocks, chain);
-    __syncthreads(); /* every wavefront is done with the stages: each takes its part of stage 0 for its hidden values */
-    /* the hidden step, as expert_gate_up_1 rounds it (the one chain is added to +0 first, as S chains are) */
-    uint16_t *strip_hidden = (uint16_t *)(window + wave * chain_type::WAVE_BYTES); /* [column][the strip's outputs] */
+    /* The hidden step, as expert_gate_up_1 rounds it (the one chain is added to +0 first, as S chains are), and the
+     * quantizer's step on it, from the registers the sums are in. A lane holds, of a column of every column block, rows
+     * 4 (lane / 16) .. + 3 of the strip's two tiles: the 32 outputs of one quantizer block are the 8 values of each
+     * of the 4 lanes of a column. Codes are bytes 2 (v % 2) + g / 2 of a word, so the lanes g and g ^ 2 of a column
+     * hold the halves of the same two words: one exchange, and each writes one whole word. */
+    static_assert(STRIP == 2u, "a strip is one block of 32 outputs");
+    const uint32_t width = arguments.output_size, first_output = (blockIdx.x * WIDE_WAVES + wave) * STRIP_OUTPUTS;
+    if (first_output >= width) {
+        return; /* a strip wholly past the matrix (its tiles were the strip's before it) */
+    }
     const float limit = arguments.activation_limit;
+    const uint32_t g = lane / 16u, upper = g / 2u;
 #pragma unroll
     for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
         const uint32_t column = 16u * j + lane % 16u;
-        if (column < tile.pair_count) {
-            const float weight = pairs[column].route_weight;
+        if (column < tile.pair_count) { /* the same in the four lanes of a column */
+            const struct wide_pair pair = pairs[column];
+            uint32_t bits[STRIP][4];
+            float largest = 0.0f;
 #pragma unroll
             for (uint32_t n = 0; n < STRIP; n++) {
 #pragma unroll
                 for (uint32_t v = 0; v < 4u; v++) {
                     const float gate_sum = __fadd_rn(0.0f, chain[n][j][v]), up_sum = __fadd_rn(0.0f, chain[STRIP + n][j][v]);
-                    const float g = bf16_to_float(float_to_bf16(gate_sum)), u = bf16_to_float(float_to_bf16(up_sum));
-                    const float bounded_gate = fminf(g, limit);
-                    const float bounded_up = fminf(fmaxf(u, -limit), limit);
-                    const float value = __fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), weight);
-                    strip_hidden[column * STRIP_OUTPUTS + n * 16u + 4u * (lane / 16u) + v] = float_to_bf16(value);
+                    const float gate = bf16_to_float(float_to_bf16(gate_sum)), up = bf16_to_float(float_to_bf16(up_sum));
+                    const float bounded_gate = fminf(gate, limit);
+                    const float bounded_up = fminf(fmaxf(up, -limit), limit);
+                    const float value = __fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), pair.route_weight);
+                    bits[n][v] = float_to_bf16(value);
+                    largest = fmaxf(largest, fabsf(bf16_to_float((uint16_t)bits[n][v])));
                 }
             }
+            largest = fmaxf(largest, __shfl_xor(largest, 16, WAVE));
+            largest = fmaxf(largest, __shfl_xor(largest, 32, WAVE));
+            const uint32_t code_exponent = quantize_exponent_code(largest);
+            unsigned char *codes = arena + arguments.hidden_codes_offset + (uint64_t)pair.pair_index * width;
+            uint16_t *operands = (uint16_t *)(arena + arguments.hidden_operands_offset) + (uint64_t)pair.pair_index * width;
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+                uint32_t code[4], operand[4];
+#pragma unroll
+                for (uint32_t v = 0; v < 4u; v++) {
+                    quantize_code(bits[n][v], code_exponent, code[v], operand[v]);
+                }
+                const uint32_t load = (tile0 + n) / 4u, step = (tile0 + n) % 4u, t = 2u * (g % 2u);
+                const uint32_t word0 = quantize_word_of(load, step, t), word1 = quantize_word_of(load, step, t + 1u);
+                const uint32_t half0 = (code[0] | (code[1] << 16)) << (8u * upper), half1 = (code[2] | (code[3] << 16)) << (8u * upper);
+                const uint32_t other = (uint32_t)__shfl_xor((int)(upper != 0u ? half0 : half1), 32, WAVE);
+                *(uint32_t *)(codes + (upper != 0u ? word1 : word0)) = (upper != 0u ? half1 : half0) | other;
+                *(uint32_t *)(operands + word0 + 2u * upper) = operand[0] | (operand[1] << 16);
+                *(uint32_t *)(operands + word1 + 2u * upper) = operand[2] | (operand[3] << 16);
+            }
+            if (g == 0u) {
+                (arena + arguments.hidden_exponents_offset)[(uint64_t)pair.pair_index * (width / 32u) + first_output / 32u] = (unsigned char)code_exponent;
+            }
         }
-    }
-    __builtin_amdgcn_s_waitcnt(0xc07f); /* the wavefront's own LDS writes have landed */
-    __builtin_amdgcn_wave_barrier();
-    const uint32_t width = arguments.output_size, first_output = (blockIdx.x * WIDE_WAVES + wave) * STRIP_OUTPUTS;
-    if (first_output >= width) {
-        return; /* a strip wholly past the matrix */
-    }
-    /* a column's strip is STRIP_OUTPUTS values: a wavefront quantizes WAVE / STRIP_OUTPUTS columns at a time, a block
-     * of 32 outputs in 32 consecutive lanes */
-    static_assert(STRIP_OUTPUTS == 32u || STRIP_OUTPUTS == 64u, "whole columns a pass of the wavefront");
-    constexpr uint32_t TOGETHER = WAVE / STRIP_OUTPUTS;
-    const uint32_t at = lane % STRIP_OUTPUTS;
-    if (tile0 * 16u + at < first_output) {
-        return; /* whole blocks of 32 that the strip before this one takes (the same in the 32 lanes of a block) */
-    }
-    for (uint32_t column = lane / STRIP_OUTPUTS; column < tile.pair_count; column += TOGETHER) {
-        const uint64_t pair = pairs[column].pair_index;
-        quantize_value(strip_hidden[column * STRIP_OUTPUTS + at], tile0 * 16u + at, arena + arguments.hidden_codes_offset + pair * width,
-                       arena + arguments.hidden_exponents_offset + pair * (width / 32u),
-                       (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width);
     }
 }
 
