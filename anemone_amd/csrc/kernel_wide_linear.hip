@@ -28,7 +28,7 @@
 #define WIDE_VECTOR_BYTES (WIDE_TILE_PAIRS * 128u) /* a K step of the tile's columns' codes */
 
 /* One block's pipeline: MATRICES matrices x STRIP tiles a wavefront, the tile's columns shared. */
-template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES>
+template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES, uint32_t DEPTH = WIDE_DEPTH>
 struct wide_chain {
     static constexpr uint32_t STRIP = STRIP_TILES;
     static constexpr uint32_t STEP_BYTES = BYTES ? BYTE_STEP_BYTES : NIBBLE_STEP_BYTES;
@@ -39,11 +39,11 @@ struct wide_chain {
     static constexpr uint32_t VECTOR_AT = WIDE_WAVES * WAVE_BYTES;               /* inside a stage */
     static constexpr uint32_t VECTOR_SCALE_AT = VECTOR_AT + WIDE_VECTOR_BYTES;
     static constexpr uint32_t STAGE_BYTES = VECTOR_SCALE_AT + 256u;
-    static constexpr uint32_t WINDOW_BYTES = WIDE_DEPTH * STAGE_BYTES;
+    static constexpr uint32_t WINDOW_BYTES = DEPTH * STAGE_BYTES;
     static constexpr uint32_t VECTOR_LOADS = 2u + 1u;                            /* issued first: two column groups, the scale words */
     static constexpr uint32_t WEIGHT_LOADS = TILES * TILE_LOADS + MATRICES;
     static constexpr uint32_t STAGE_LOADS = VECTOR_LOADS + WEIGHT_LOADS;         /* a wavefront's loads a stage */
-    static_assert(STAGE_LOADS * (WIDE_DEPTH - 1u) < 64u && WINDOW_BYTES <= 160u * 1024u, "vmcnt has six bits; LDS 160 KB");
+    static_assert(STAGE_LOADS * (DEPTH - 1u) < 64u && WINDOW_BYTES <= 160u * 1024u, "vmcnt has six bits; LDS 160 KB");
 
     const unsigned char *words[MATRICES], *scales[MATRICES], *codes, *exponents;
     uint32_t tile_bytes, window, wave, piece_offset, scale_offset, codes_offset[2], exponents_offset;
@@ -186,7 +186,7 @@ struct wide_chain {
         /* behind this barrier every wavefront's weights and prepared column block of this step are in LDS, and
          * every wavefront has read the step before: its stage may be asked for again */
         __syncthreads();
-        const uint32_t behind = stage == 0u ? WIDE_DEPTH - 1u : stage - 1u, ahead = stage + 1u == WIDE_DEPTH ? 0u : stage + 1u;
+        const uint32_t behind = stage == 0u ? DEPTH - 1u : stage - 1u, ahead = stage + 1u == DEPTH ? 0u : stage + 1u;
         if constexpr (AHEAD >= 2u) {
             issue(behind, step + 2u);
         }
@@ -201,7 +201,22 @@ struct wide_chain {
     template <uint32_t LIVE>
     __device__ __forceinline__ void steps(uint32_t total, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
     {
-        static_assert(WIDE_DEPTH == 3u, "the waits are written out for two stages ahead");
+        if constexpr (DEPTH == 2u) {
+            /* two stages: a step's loads are asked for a step ahead, and its columns prepared once they have landed,
+             * before the barrier that opens the step */
+            issue(0u, 0u);
+            for (uint32_t step = 0; step < total; step++) {
+                wait_loads<0>();
+                prepare_columns(step % 2u);
+                __syncthreads(); /* every wavefront has read the step before and brought and prepared its part of this one */
+                if (step + 1u < total) {
+                    issue((step + 1u) % 2u, step + 1u);
+                }
+                consume<LIVE>(step % 2u, chain);
+            }
+            return;
+        }
+        static_assert(DEPTH == 2u || DEPTH == 3u, "the waits are written out for one or two stages ahead");
         issue(0u, 0u);
         if (total > 1u) {
             issue(1u, 1u);
@@ -213,11 +228,11 @@ struct wide_chain {
         uint32_t stage = 0, step = 0;
         for (; step + 2u < total; step++) {
             one_step<LIVE, 2u>(step, stage, chain);
-            stage = stage + 1u == WIDE_DEPTH ? 0u : stage + 1u;
+            stage = stage + 1u == DEPTH ? 0u : stage + 1u;
         }
         if (step + 1u < total) {
             one_step<LIVE, 1u>(step, stage, chain);
-            stage = stage + 1u == WIDE_DEPTH ? 0u : stage + 1u;
+            stage = stage + 1u == DEPTH ? 0u : stage + 1u;
             step++;
         }
         one_step<LIVE, 0u>(step, stage, chain);
@@ -336,7 +351,7 @@ struct wide_chain {
 template <bool BYTES>
 __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_expert_gate_up_arguments &arguments, unsigned char *arena)
 {
-    typedef wide_chain<2, BYTES, 2u> chain_type;
+    typedef wide_chain<2, BYTES, 2u, (BYTES ? 3u : 2u)> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
@@ -431,7 +446,7 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
 template <bool BYTES>
 __device__ static __forceinline__ void wide_expert_down(const struct wide_expert_down_arguments &arguments, unsigned char *arena)
 {
-    typedef wide_chain<1, BYTES, (BYTES ? 2u : 4u)> chain_type;
+    typedef wide_chain<1, BYTES, (BYTES ? 2u : 4u), 2u> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
@@ -510,6 +525,6 @@ extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_e4m3
 }
 ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_e4m3_1, wide_expert_down_arguments);
 
-static_assert(wide_chain<2, false, 2u>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true, 2u>::WINDOW_BYTES == WIDE_GATE_UP_E4M3_WINDOW_BYTES &&
-                  wide_chain<1, false, 4u>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES && wide_chain<1, true, 2u>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES,
+static_assert(wide_chain<2, false, 2u, 2u>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true, 2u, 3u>::WINDOW_BYTES == WIDE_GATE_UP_E4M3_WINDOW_BYTES &&
+                  wide_chain<1, false, 4u, 2u>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES && wide_chain<1, true, 2u, 2u>::WINDOW_BYTES == WIDE_DOWN_E4M3_WINDOW_BYTES,
               "the windows the host asks for are the kernels'");

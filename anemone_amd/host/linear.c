@@ -354,7 +354,7 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
                 (gate_up->output_size + WIDE_GATE_UP_BLOCK_OUTPUTS - 1u) / WIDE_GATE_UP_BLOCK_OUTPUTS, description->tile_count, 1,
                 WIDE_BLOCK_THREADS, bytes ? WIDE_GATE_UP_E4M3_WINDOW_BYTES : WIDE_GATE_UP_WINDOW_BYTES, &gate_up_record, sizeof gate_up_record);
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_DOWN], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
-                description->tile_count, 1, WIDE_BLOCK_THREADS, WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);
+                description->tile_count, 1, WIDE_BLOCK_THREADS, bytes ? WIDE_DOWN_E4M3_WINDOW_BYTES : WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_ROW_SUM], linear_kernels->expert_row_sum,
                 (down->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)rows, 1, LINEAR_ELEMENT_THREADS, 0,
                 &row_sum_record, sizeof row_sum_record);

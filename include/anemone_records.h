@@ -473,9 +473,10 @@ ANEMONE_RECORD_HAS(expert_gate_up_quantize_arguments, 96);
 #define KERNEL_WIDE_EXPERT_DOWN_STEM "wide_expert_down_"
 #define WIDE_BLOCK_THREADS 256u          /* four wavefronts: four strips of one tile of pairs */
 #define WIDE_GATE_UP_BLOCK_OUTPUTS 128u   /* of gate and of up: a wavefront takes 32 of each */
-#define WIDE_GATE_UP_WINDOW_BYTES 80640u  /* dynamic LDS of wide_expert_gate_up_<S>: three stages; two blocks fit a CU */
+#define WIDE_GATE_UP_WINDOW_BYTES 53760u  /* dynamic LDS of wide_expert_gate_up_<S>: two stages; three blocks fit a CU */
 #define WIDE_GATE_UP_E4M3_WINDOW_BYTES 129792u /* of wide_expert_gate_up_e4m3_<S> */
-#define WIDE_DOWN_WINDOW_BYTES 77568u     /* of wide_expert_down_<S> */
+#define WIDE_DOWN_WINDOW_BYTES 51712u     /* of wide_expert_down_<S>: two stages */
+#define WIDE_DOWN_E4M3_WINDOW_BYTES 51712u /* of wide_expert_down_e4m3_<S>: two stages */
 struct wide_expert_gate_up_arguments {
     uint64_t tiles_offset;            /* read: struct wide_expert_tile [tile_count] */
     uint64_t pairs_offset;            /* read: struct wide_pair [pair_count] */

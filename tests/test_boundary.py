@@ -470,7 +470,7 @@ def test_wide_linear_prepare_geometry_and_refusals(fake):
     tiles = 1024 * 8 // 64 + 256
     assert [list(l.grid) for l in launches] == [[16, tiles, 1], [16, tiles, 1], [16, 1024, 1]]
     assert [l.block[0] for l in launches] == [256, 256, 256]
-    assert [l.dynamic_shared_byte_count for l in launches] == [80640, 77568, 0]  # two blocks of either fit a CU's 160 KB
+    assert [l.dynamic_shared_byte_count for l in launches] == [53760, 51712, 0]  # three blocks of either fit a CU's 160 KB
     assert [l.argument_byte_count for l in launches] == [88, 64, 24]
     record = amd.WideExpertGateUpArguments.from_buffer_copy(bytes(launches[0].argument)[:88])
     assert (record.output_size, record.input_size, record.tile_count, record.pairs_per_row, record.pair_count) == (2048, 4096, tiles, 8, 8192)
@@ -479,7 +479,7 @@ def test_wide_linear_prepare_geometry_and_refusals(fake):
     assert lib.linear_wide_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(kernels), fp8) == 0
     assert [fake.handles[l.kernel][1] for l in fp8][:2] == ["wide_expert_gate_up_e4m3_1", "wide_expert_down_e4m3_1"]
     assert [list(l.grid) for l in fp8][:2] == [[16, tiles, 1], [32, tiles, 1]]  # strips of 32 outputs
-    assert [l.dynamic_shared_byte_count for l in fp8] == [129792, 77568, 0]
+    assert [l.dynamic_shared_byte_count for l in fp8] == [129792, 51712, 0]
     for changes in (dict(gate_up_slice_count=2), dict(down_slice_count=4), dict(tile_count=0), dict(tile_count=70000), dict(reserved_zero=1),
                     dict(row_count=0), dict(row_count=20000), dict(activation_limit=0.0), dict(weight_format=amd.WEIGHT_FORMAT_EXL3),
                     dict(tiles=amd.Range(3 << 30, 64)), dict(pairs=amd.Range((8 << 30) - 256, 65536)),
