@@ -155,10 +155,17 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         result["config"].pop("down_GBps")
         result["config"]["down_TFLOPs"] = down_flops / (down_us * 1e-6) / 1e12
         result["config"]["step_TFLOPs"] = (gate_up_flops + down_flops) / (seconds / arguments.steps) / 1e12
-        # the products are MFMAs of FP8 activations (with FP4 or FP8 weights): the FP8 rate is the instruction's peak
-        result["roofline"] = {"bound": "mfma", "kernel": "wide_expert_gate_up_%s1" % ("e4m3_" if fp8 else ""), "achieved": achieved,
-                              "peak": MFMA_F8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": None,
-                              "algorithmic_flops_per_launch": gate_up_flops, "launch_us": gate_up_us}
+        # the products are MFMAs of FP8 activations (with FP4 or FP8 weights): the FP8 rate is the instruction's peak.
+        # What bounds the launch is read off its arithmetic intensity against the card's balance of the two peaks.
+        kernel = "wide_expert_gate_up_%s1" % ("e4m3_" if fp8 else "")
+        if gate_up_flops / gate_up_bytes >= MFMA_F8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
+            result["roofline"] = {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_F8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                  "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": None, "algorithmic_flops_per_launch": gate_up_flops,
+                                  "launch_us": gate_up_us}
+        else:
+            result["roofline"]["kernel"] = kernel  # the matrices' bytes of the distinct experts against the memory's peak
+            result["roofline"]["TFLOPs"] = achieved
+            result["roofline"]["flop_per_byte"] = gate_up_flops / gate_up_bytes
     if not arguments.no_cpu:
         import _oracle as o
         threads = min(os.cpu_count() or 1, 16)
