@@ -198,6 +198,7 @@ def library():
             "router_select_prepare": [C.POINTER(RouterDescription), u64, C.POINTER(RouterKernels), launch_p],
             "router_projection_prepare": [C.POINTER(RouterProjectionDescription), u64, C.POINTER(RouterKernels), launch_p],
             "router_wide_prepare": [C.POINTER(RouterWideDescription), u64, C.POINTER(RouterKernels), launch_p],
+            "router_wide_small_prepare": [C.POINTER(RouterWideDescription), u64, C.POINTER(RouterKernels), launch_p],
             "linear_kernels_prepare": [vp, vp, u32, C.POINTER(LinearKernels)],
             "linear_quantize_prepare": [C.POINTER(QuantizeDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_routed_experts_prepare": [C.POINTER(RoutedExpertsDescription), u64, C.POINTER(LinearKernels), launch_p],
@@ -424,10 +425,12 @@ class WideRouter:
         d.affinity_kind, d.route_scale = layer.affinity_kind, layer.route_scale
         self.description = d
 
-    def launches(self):
-        launches = launches_of(4)
-        check(self.card.lib.router_wide_prepare(C.byref(self.description), self.card.arena_bytes, C.byref(self.layer.router_kernels), launches),
-              "router_wide_prepare")
+    def launches(self, small=False):
+        """The four launches of any row count; small: the two of at most ROUTER_SORT_ROWS rows (select, router_wide_small)."""
+        launches = launches_of(2 if small else 4)
+        prepare = self.card.lib.router_wide_small_prepare if small else self.card.lib.router_wide_prepare
+        check(prepare(C.byref(self.description), self.card.arena_bytes, C.byref(self.layer.router_kernels), launches),
+              "router_wide_small_prepare" if small else "router_wide_prepare")
         return launches
 
     def read(self, name, dtype):

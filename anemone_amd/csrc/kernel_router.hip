@@ -408,38 +408,19 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_count, router_wide_arguments);
 
-/* grid as the count's: the sorted pairs of the block's rows; block 0 also the runs and every tile */
-extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
-    router_wide_place(struct router_wide_arguments arguments, unsigned char *arena)
+/* What a block of the place does once it holds, in LDS, its picks (block_experts, `pairs` of them) and of every expert
+ * the pairs of all blocks (totals; starts a copy of them), those of the blocks before this one (before) and its
+ * tiles (tile_starts): the sorted pairs of the block's rows; block 0 also the runs and every tile. The whole block
+ * calls it after a barrier. */
+__device__ static __forceinline__ void wide_place_block(const struct router_wide_arguments &arguments, unsigned char *arena, uint32_t block,
+                                                        const uint32_t *block_experts, uint32_t pairs, uint32_t *totals, uint32_t *starts,
+                                                        const uint32_t *before, uint32_t *tile_starts, uint32_t *scratch)
 {
-    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
-    __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
-    __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
     const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
-    const uint32_t live_rows = wide_live_rows(arguments, arena);
-    const uint32_t live_blocks = (live_rows + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
-    const uint32_t pairs = wide_block_picks(arguments, arena, blockIdx.x, live_rows, block_experts);
-    if (pairs == 0u && blockIdx.x != 0u) {
-        return;
-    }
-    const uint32_t *counts = (const uint32_t *)(arena + arguments.counts_offset);
-    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
-        uint32_t total = 0, lower = 0;
-        for (uint32_t block = 0; block < live_blocks; block++) {
-            const uint32_t count = counts[(uint64_t)block * experts + expert];
-            total += count;
-            lower += block < blockIdx.x ? count : 0u;
-        }
-        totals[expert] = total;
-        starts[expert] = total;
-        before[expert] = lower;
-        tile_starts[expert] = (total + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS;
-    }
-    __syncthreads();
     (void)block_exclusive_scan(starts, experts, scratch);
     const struct router_pick *all_picks = (const struct router_pick *)(arena + arguments.picks_offset);
     struct wide_pair *sorted = (struct wide_pair *)(arena + arguments.pairs_offset);
-    const uint32_t first_pair = blockIdx.x * ROUTER_SORT_ROWS * picks;
+    const uint32_t first_pair = block * ROUTER_SORT_ROWS * picks;
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
         uint32_t place = starts[expert] + before[expert];
         for (uint32_t index = 0; index < pairs; index++) {
@@ -449,7 +430,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
             }
         }
     }
-    if (blockIdx.x != 0u) {
+    if (block != 0u) {
         return;
     }
     struct wide_run *runs = (struct wide_run *)(arena + arguments.runs_offset);
@@ -486,19 +467,46 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
         tiles[tile] = value;
     }
 }
-ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_place, router_wide_arguments);
 
-/* grid (1): the job table of the runs, a thread a job */
+/* grid as the count's: the sorted pairs of the block's rows; block 0 also the runs and every tile */
 extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
-    router_wide_jobs(struct router_wide_arguments arguments, unsigned char *arena)
+    router_wide_place(struct router_wide_arguments arguments, unsigned char *arena)
 {
-    __shared__ uint32_t job_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
-    const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
-    const struct wide_run *runs = (const struct wide_run *)(arena + arguments.runs_offset);
+    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
+    __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
+    const uint32_t experts = arguments.expert_count;
+    const uint32_t live_rows = wide_live_rows(arguments, arena);
+    const uint32_t live_blocks = (live_rows + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
+    const uint32_t pairs = wide_block_picks(arguments, arena, blockIdx.x, live_rows, block_experts);
+    if (pairs == 0u && blockIdx.x != 0u) {
+        return;
+    }
+    const uint32_t *counts = (const uint32_t *)(arena + arguments.counts_offset);
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
-        job_starts[expert] = (runs[expert].pair_count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS;
+        uint32_t total = 0, lower = 0;
+        for (uint32_t block = 0; block < live_blocks; block++) {
+            const uint32_t count = counts[(uint64_t)block * experts + expert];
+            total += count;
+            lower += block < blockIdx.x ? count : 0u;
+        }
+        totals[expert] = total;
+        starts[expert] = total;
+        before[expert] = lower;
+        tile_starts[expert] = (total + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS;
     }
     __syncthreads();
+    wide_place_block(arguments, arena, blockIdx.x, block_experts, pairs, totals, starts, before, tile_starts, scratch);
+}
+ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_place, router_wide_arguments);
+
+/* The job table of the runs, a thread a job; job_starts holds every expert's jobs. The whole block calls it after a
+ * barrier that follows the writing of the runs and the sorted pairs. */
+__device__ static __forceinline__ void wide_jobs_block(const struct router_wide_arguments &arguments, unsigned char *arena,
+                                                       uint32_t *job_starts, uint32_t *scratch)
+{
+    const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
+    const struct wide_run *runs = (const struct wide_run *)(arena + arguments.runs_offset);
     const uint32_t used_jobs = block_exclusive_scan(job_starts, experts, scratch);
     if (threadIdx.x == 0u) {
         job_starts[experts] = used_jobs;
@@ -541,4 +549,49 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
         jobs[job] = value;
     }
 }
+
+/* grid (1): the job table of the runs, a thread a job */
+extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
+    router_wide_jobs(struct router_wide_arguments arguments, unsigned char *arena)
+{
+    __shared__ uint32_t job_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
+    const struct wide_run *runs = (const struct wide_run *)(arena + arguments.runs_offset);
+    for (uint32_t expert = threadIdx.x; expert < arguments.expert_count; expert += blockDim.x) {
+        job_starts[expert] = (runs[expert].pair_count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS;
+    }
+    __syncthreads();
+    wide_jobs_block(arguments, arena, job_starts, scratch);
+}
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_jobs, router_wide_arguments);
+
+/* grid (1): the count, the place and the jobs of at most ROUTER_SORT_ROWS rows in one block (the reference's
+ * router_wide_small, source/kernel_router.cu there): the same pairs, runs, tiles and jobs; the counts scratch is
+ * not written */
+extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
+    router_wide_small(struct router_wide_arguments arguments, unsigned char *arena)
+{
+    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
+    __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS], job_starts[ROUTER_MOST_EXPERTS + 1u];
+    const uint32_t experts = arguments.expert_count;
+    const uint32_t live_rows = wide_live_rows(arguments, arena);
+    const uint32_t pairs = wide_block_picks(arguments, arena, 0u, live_rows, block_experts);
+    __syncthreads();
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        uint32_t count = 0;
+        for (uint32_t index = 0; index < pairs; index++) {
+            count += block_experts[index] == expert ? 1u : 0u;
+        }
+        totals[expert] = count;
+        starts[expert] = count;
+        before[expert] = 0u;
+        tile_starts[expert] = (count + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS;
+        job_starts[expert] = (count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS;
+    }
+    __syncthreads();
+    wide_place_block(arguments, arena, 0u, block_experts, pairs, totals, starts, before, tile_starts, scratch);
+    __threadfence_block();
+    __syncthreads(); /* the runs and the sorted pairs, written by this block, are read by its jobs */
+    wide_jobs_block(arguments, arena, job_starts, scratch);
+}
+ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_small, router_wide_arguments);

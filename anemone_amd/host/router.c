@@ -12,6 +12,7 @@
  *   wide count    router_wide_count     (ceil(rows / 384), 1, 1)    512   a thread an expert
  *   wide place    router_wide_place     (ceil(rows / 384), 1, 1)    512   a thread an expert; block 0 the runs and tiles
  *   wide jobs     router_wide_jobs      (1, 1, 1)                   512   a thread a job
+ *   wide small    router_wide_small     (1, 1, 1)                   512   count, place and jobs of at most 384 rows
  */
 #include <inttypes.h>
 #include <string.h>
@@ -244,18 +245,24 @@ result_status router_projection_prepare(const struct router_projection_descripti
     return STATUS_OK;
 }
 
-result_status router_wide_prepare(const struct router_wide_description *description, uint64_t arena_byte_count,
-                                  const struct router_kernels_record *kernels, struct kernel_launch *launches_out)
+/* the wide select's launches: the four of any row count, or (small) the select and router_wide_small */
+static result_status wide_launches(const struct router_wide_description *description, uint64_t arena_byte_count,
+                                   const struct router_kernels_record *kernels, bool small, struct kernel_launch *launches_out)
 {
-    static const char what[] = "the router's wide select";
+    const char *what = small ? "the router's wide select in one block" : "the router's wide select";
     if (description == NULL || kernels == NULL || launches_out == NULL || description->expert_offsets == NULL) {
         REFUSE("%s: a missing argument", what);
         return STATUS_INVALID_ARGUMENT;
     }
     const uint32_t E = description->expert_count, P = description->pick_count, R = description->row_count;
-    if (description->reserved_zero != 0 || kernels->wide_select == BACKEND_NO_KERNEL || kernels->wide_count == BACKEND_NO_KERNEL ||
-        kernels->wide_place == BACKEND_NO_KERNEL || kernels->wide_jobs == BACKEND_NO_KERNEL) {
-        REFUSE("%s: a reserved field that is not zero, or a kernel of the four is not prepared", what);
+    if (description->reserved_zero != 0 || kernels->wide_select == BACKEND_NO_KERNEL ||
+        (small ? kernels->wide_small == BACKEND_NO_KERNEL
+               : kernels->wide_count == BACKEND_NO_KERNEL || kernels->wide_place == BACKEND_NO_KERNEL || kernels->wide_jobs == BACKEND_NO_KERNEL)) {
+        REFUSE("%s: a reserved field that is not zero, or a kernel of its launches is not prepared", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (small && description->row_count > ROUTER_SORT_ROWS) {
+        REFUSE("%s: %u rows, at most %u", what, description->row_count, ROUTER_SORT_ROWS);
         return STATUS_INVALID_ARGUMENT;
     }
     if (!shape_counts_are_valid(what, E, P, description->affinity_kind, description->order)) {
@@ -316,9 +323,26 @@ result_status router_wide_prepare(const struct router_wide_description *descript
     struct kernel_launch launches[ROUTER_WIDE_LAUNCH_COUNT];
     launch_fill(&launches[ROUTER_WIDE_SELECT_LAUNCH], kernels->wide_select, (R + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS, 1, 1,
                 SELECT_THREADS, 0, &record, sizeof record);
+    if (small) {
+        launch_fill(&launches[1], kernels->wide_small, 1, 1, 1, WIDE_SORT_THREADS, 0, &record, sizeof record);
+        memcpy(launches_out, launches, ROUTER_WIDE_SMALL_LAUNCH_COUNT * sizeof launches[0]);
+        return STATUS_OK;
+    }
     launch_fill(&launches[ROUTER_WIDE_COUNT_LAUNCH], kernels->wide_count, (uint32_t)blocks, 1, 1, WIDE_SORT_THREADS, 0, &record, sizeof record);
     launch_fill(&launches[ROUTER_WIDE_PLACE_LAUNCH], kernels->wide_place, (uint32_t)blocks, 1, 1, WIDE_SORT_THREADS, 0, &record, sizeof record);
     launch_fill(&launches[ROUTER_WIDE_JOBS_LAUNCH], kernels->wide_jobs, 1, 1, 1, WIDE_SORT_THREADS, 0, &record, sizeof record);
     memcpy(launches_out, launches, sizeof launches);
     return STATUS_OK;
+}
+
+result_status router_wide_prepare(const struct router_wide_description *description, uint64_t arena_byte_count,
+                                  const struct router_kernels_record *kernels, struct kernel_launch *launches_out)
+{
+    return wide_launches(description, arena_byte_count, kernels, false, launches_out);
+}
+
+result_status router_wide_small_prepare(const struct router_wide_description *description, uint64_t arena_byte_count,
+                                        const struct router_kernels_record *kernels, struct kernel_launch *launches_out)
+{
+    return wide_launches(description, arena_byte_count, kernels, true, launches_out);
 }

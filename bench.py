@@ -93,8 +93,10 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                          weight_format=amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED)
     layer.set_rows(x, rows)
     wide = layer.wide_router() if rows > 8 or prefill else None  # more than eight rows: the wide select sorts the pairs by expert
-    routing = [layer.select_launch(0)[0]] if wide is None else list(wide.launches())
-    routing_names = ["router_select_entry"] if wide is None else ["router_wide_select", "router_wide_count", "router_wide_place", "router_wide_jobs"]
+    small = wide is not None and rows <= amd.ROUTER_SORT_ROWS and not prefill  # count, place and jobs in one block
+    routing = [layer.select_launch(0)[0]] if wide is None else list(wide.launches(small=small))
+    routing_names = ["router_select_entry"] if wide is None else ["router_wide_select", "router_wide_small"] if small else \
+        ["router_wide_select", "router_wide_count", "router_wide_place", "router_wide_jobs"]
     if prefill:
         routing, routing_names = routing[:3], routing_names[:3]  # the tiles are the place's; no job table
         experts = layer.wide_expert_launches(wide)

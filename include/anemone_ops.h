@@ -185,6 +185,14 @@ MUST_CHECK result_status router_wide_prepare(const struct router_wide_descriptio
                                              uint64_t arena_byte_count,
                                              const struct router_kernels_record *kernels,
                                              struct kernel_launch *launches_out);
+/* include/anemone/router.h:117-124 of the reference: the same of at most ROUTER_SORT_ROWS rows in two launches, the
+ * select and router_wide_small (the count, the place and the jobs in one block: the same picks, affinities, pairs,
+ * runs, tiles and jobs; the counts scratch unwritten). More rows: STATUS_INVALID_ARGUMENT. */
+#define ROUTER_WIDE_SMALL_LAUNCH_COUNT 2u
+MUST_CHECK result_status router_wide_small_prepare(const struct router_wide_description *description,
+                                                   uint64_t arena_byte_count,
+                                                   const struct router_kernels_record *kernels,
+                                                   struct kernel_launch *launches_out);
 
 /* ---- FP4 / FP8 expert linears of the original weights (the routed part of the reference's linear.h) ---- */
 #define LINEAR_SLICE_INSTANCES 5u /* product kernels are stamped for 1, 2, 4, 8, 16 slices; gfx950 holds 1, 2, 4, 8 */

@@ -314,7 +314,7 @@ def test_wide_router_prepare(fake):
     kernels = amd.RouterKernels()
     assert lib.router_kernels_prepare(fake.address, fake.card, C.byref(kernels)) == 0
     assert amd.BACKEND_NO_KERNEL not in (kernels.wide_select, kernels.wide_count, kernels.wide_place, kernels.wide_jobs)
-    assert kernels.wide_small == amd.BACKEND_NO_KERNEL  # the one-launch form is not built
+    assert kernels.wide_small != amd.BACKEND_NO_KERNEL
     d, keep = wide_description()
     launches = amd.launches_of(4)
     assert lib.router_wide_prepare(C.byref(d), ARENA, C.byref(kernels), launches) == 0
@@ -333,6 +333,17 @@ def test_wide_router_prepare(fake):
     bad, keep = wide_description()
     bad.runs = amd.Range(bad.pairs.byte_offset, 256 * 8)
     assert lib.router_wide_prepare(C.byref(bad), ARENA, C.byref(kernels), amd.launches_of(4)) == 1
+    # the form of at most 384 rows: the select and one block
+    two = amd.launches_of(2)
+    d, keep = wide_description()
+    assert lib.router_wide_small_prepare(C.byref(d), ARENA, C.byref(kernels), two) == 1  # 4096 rows
+    assert not any(bytes(two))
+    d, keep = wide_description(row_count=384)
+    assert lib.router_wide_small_prepare(C.byref(d), ARENA, C.byref(kernels), two) == 0
+    assert [fake.handles[l.kernel][1] for l in two] == ["router_wide_select", "router_wide_small"]
+    assert [list(l.grid) for l in two] == [[48, 1, 1], [1, 1, 1]] and two[1].block[0] == 512 and two[1].argument_byte_count == 136
+    d, keep = wide_description(row_count=385)
+    assert lib.router_wide_small_prepare(C.byref(d), ARENA, C.byref(kernels), amd.launches_of(2)) == 1
 
 
 def tcp_record(**changes):

@@ -127,6 +127,35 @@ def test_wide_select_skewed_and_hand_case(amd, card):
     assert counts.max() > 400
 
 
+@pytest.mark.parametrize("experts_n,picks,rows,live", [(64, 4, 40, 37), (256, 8, 384, 384), (384, 6, 130, 130), (128, 3, 1, 1)])
+def test_wide_small_equals_the_four_launches(amd, card, experts_n, picks, rows, live):
+    """router_wide_small (count, place and jobs of at most 384 rows in one block) writes the pairs, runs, tiles and
+    jobs of the four launches, byte for byte (include/anemone/router.h:117-119 of the reference), and those are held to
+    the oracle by the tests above."""
+    say("wide small", experts_n, picks, rows, live)
+    layer, _ = small_layer(amd, card, experts_n, picks, rows)
+    scores = (normals(123, rows * experts_n) * 1.5).astype(np.float32).reshape(rows, experts_n)
+    card.upload(layer.scores_offset, scores)
+    card.upload(layer.bias_offset, np.zeros(experts_n, dtype=np.float32))
+    card.upload(layer.step_offset, amd.step_block(live))
+    wide = layer.wide_router()
+    names = ("pairs", "runs", "tiles", "jobs")
+
+    def run(launches):
+        for name in names:
+            card.upload(wide.ranges[name].byte_offset, np.full(wide.ranges[name].byte_count, 0xEE, dtype=np.uint8))
+        card.run(launches)
+        return [wide.read(name, np.uint8).copy() for name in names]
+    four = run(wide.launches())
+    card.upload(wide.ranges["counts"].byte_offset, np.full(wide.ranges["counts"].byte_count, 0xEE, dtype=np.uint8))
+    two = run(wide.launches(small=True))
+    live_pairs = live * picks
+    for name, a, b in zip(names, four, two):
+        count = live_pairs * 8 if name == "pairs" else a.size  # the pairs past the live rows' are not written
+        assert np.array_equal(a[:count], b[:count]), name
+    assert np.all(wide.read("counts", np.uint8) == 0xEE)  # the counts scratch stays unwritten
+
+
 def test_fp4_layer_through_the_wide_job_table(amd, card):
     """40 rows (37 live) routed by the wide select, then the FP4 experts over its job table, against the oracle."""
     say("fp4 layer, wide")
