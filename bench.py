@@ -25,6 +25,16 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes of the roofline kernel's launch as rocprofv3 counted them (FETCH_SIZE + WRITE_SIZE, each scaled by what the
+# same counter reads for a 1 GiB copy), for the workloads at the sizes profiled: constants of those runs (the summaries
+# under profiles/ hold the commands and the counts), reported as roofline.traffic when a run has the same sizes
+MEASURED_TRAFFIC_BYTES = {
+    ("exl3_decode", 8): 375.2e6 + 8.4e6,      # profiles/exl3_tc_products_decode8.md
+    ("fp4_decode", 32): 1434.7e6 + 1.0e6,     # profiles/expert_gate_up_fp4_fp8_decode32.md
+    ("fp8_decode", 32): 2768.4e6 + 1.0e6,
+    ("fp4_prefill", 8192): 5444e6 + 444e6,    # profiles/wide_expert_fp4_fp8_prefill.md
+    ("fp8_prefill", 2048): 5801e6 + 111e6,
+}
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
 CONFIG = 1
 
@@ -148,6 +158,9 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                      "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
     }
+    key = ("%s_%s" % ("fp8" if fp8 else "fp4", "prefill" if prefill else "decode"), rows)
+    if key in MEASURED_TRAFFIC_BYTES and (prefill or (arguments.gate_up_slices, arguments.down_slices) == (4, 2)):
+        result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES[key]
     if prefill:
         pairs = rows * PICKS
         gate_up_flops, down_flops = 2.0 * pairs * 2 * HIDDEN * INNER, 2.0 * pairs * HIDDEN * INNER
@@ -162,7 +175,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         kernel = "wide_expert_gate_up_%s1" % ("e4m3_" if fp8 else "")
         if gate_up_flops / gate_up_bytes >= MFMA_F8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
             result["roofline"] = {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_F8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                  "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": None, "algorithmic_flops_per_launch": gate_up_flops,
+                                  "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": result["roofline"]["traffic"],
+                                  "algorithmic_flops_per_launch": gate_up_flops,
                                   "launch_us": gate_up_us}
         else:
             result["roofline"]["kernel"] = kernel  # the matrices' bytes of the distinct experts against the memory's peak
@@ -382,7 +396,8 @@ def main():
                    "host_clock_ms_per_step": 1000.0 * host_seconds / arguments.steps,
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)}},
         "roofline": {"bound": "hbm", "kernel": "exl3_tc_products (gate/up pass)", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES[("exl3_decode", ROWS)],
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
     }
 
