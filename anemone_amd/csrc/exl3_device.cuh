@@ -38,14 +38,13 @@ __device__ static __forceinline__ float bf16_to_float(uint16_t bits)
     return __uint_as_float((uint32_t)bits << 16);
 }
 
-/* float32 -> bfloat16, to nearest, ties to even; a NaN becomes 0x7FC0 */
+/* float32 -> bfloat16, to nearest, ties to even; a NaN becomes 0x7FC0. The card's own conversion
+ * (v_cvt_pk_bf16_f32) gives, for every float32 that is a number, the bits of (bits + 0x7FFF + ((bits >> 16) & 1)) >> 16
+ * (compared over all 2^32 inputs); it keeps a NaN's payload, hence the select. */
 __device__ static __forceinline__ uint16_t float_to_bf16(float value)
 {
-    const uint32_t bits = __float_as_uint(value);
-    if (value != value) {
-        return 0x7FC0u;
-    }
-    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+    const uint16_t rounded = __builtin_bit_cast(uint16_t, (__bf16)value);
+    return value != value ? (uint16_t)0x7FC0u : rounded;
 }
 
 __device__ static __forceinline__ float half_bits_to_float(uint16_t bits)
