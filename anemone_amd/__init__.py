@@ -16,7 +16,7 @@ WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED = 2, 3,
 ARITHMETIC_CLASS_GFX950 = 950
 BACKEND_NO_KERNEL = 0xFFFFFFFF
 ROUTER_SORT_ROWS = 384
-EXL3_TCP_CHUNK_PAIRS = 128
+EXL3_TCP_CHUNK_PAIRS = 160
 EXL3_EXPERT_LAUNCHES, EXL3_TC_LAUNCHES = 5, 5
 EXL3_TC_GATE_UP_SLICES, EXL3_TC_DOWN_SLICES = 8, 4
 AFFINITY_SQRT_SOFTPLUS, AFFINITY_SIGMOID = 0, 1

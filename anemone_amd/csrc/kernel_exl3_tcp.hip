@@ -27,7 +27,8 @@
 #define TCP_WAVE_TILES 4u  /* output tiles of a wavefront: 64 outputs */
 #define TCP_COLUMN_BLOCKS (EXL3_TCP_CHUNK_PAIRS / 16u)
 #define TCP_STEP_INPUTS 32u
-#define TCP_STAGE_BYTES (EXL3_TCP_CHUNK_PAIRS * TCP_STEP_INPUTS * 2u) /* a K step of the chunk's operand columns */
+#define TCP_OPERAND_PARTS ((TCP_COLUMN_BLOCKS + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES) /* 16-column groups a wavefront brings a step */
+#define TCP_STAGE_BYTES (TCP_OPERAND_PARTS * TCP_GEMM_WAVES * 1024u) /* a K step of the chunk's operand columns, in whole groups */
 
 struct tcp_shape {
     uint32_t hidden, intermediate, picks, pairs, experts;
@@ -219,7 +220,7 @@ __device__ static __forceinline__ void tcp_wait_loads()
  * Lane L of an operand load lands at bytes 16 L of a 16-column group: column L / 4, slot L % 4, and asks for that
  * column's 16-byte piece (L % 4) ^ ((column / 2) % 4) of the step, so that the readers of one piece of sixteen columns
  * meet different banks. */
-template <uint32_t bits_x2>
+template <uint32_t bits_x2, uint32_t LIVE>
 __device__ static __forceinline__ void
 tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t strip_tile, uint32_t inputs,
               const half_t *__restrict__ columns, uint32_t column_count, uint32_t stage, uint32_t window, uint32_t wave,
@@ -236,11 +237,12 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
     const bool carries = lane < 2u * row_lanes && strip_is_live;
     const unsigned char *weight_source = (const unsigned char *)codes + (uint64_t)strip_tile * W::tile_bytes +
                                          (lane / row_lanes) * row_stride + (lane % row_lanes) * 16u;
-    /* operands: this wavefront brings two of the step's eight 16-column groups: wave, wave + 4 */
+    /* operands: this wavefront brings TCP_OPERAND_PARTS of the step's 16-column groups: wave, wave + 4, ... (a group
+     * past the chunk's columns lands in the stage's spare room) */
     const uint32_t load_column = lane / 4u, load_piece = (lane % 4u) ^ ((load_column / 2u) % 4u);
-    const unsigned char *operand_source[2]; /* a column past the chunk's last reads the first again: never stored */
+    const unsigned char *operand_source[TCP_OPERAND_PARTS]; /* a column past the chunk's last reads the first again: never stored */
 #pragma unroll
-    for (uint32_t part = 0; part < 2u; part++) {
+    for (uint32_t part = 0; part < TCP_OPERAND_PARTS; part++) {
         const uint32_t column = 16u * (wave + TCP_GEMM_WAVES * part) + load_column;
         operand_source[part] = (const unsigned char *)(columns + (uint64_t)(column < column_count ? column : 0u) * inputs) + load_piece * 16u;
     }
@@ -257,7 +259,7 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
     const uint32_t steps = inputs / TCP_STEP_INPUTS;
 #define TCP_ISSUE(step, buffer)                                                                                       \
     do {                                                                                                              \
-        _Pragma("unroll") for (uint32_t part = 0; part < 2u; part++)                                                  \
+        _Pragma("unroll") for (uint32_t part = 0; part < TCP_OPERAND_PARTS; part++)                                   \
         {                                                                                                             \
             tcp_load_to_lds(operand_source[part] + (uint64_t)(step) * (TCP_STEP_INPUTS * 2u),                         \
                             stage + (buffer) * TCP_STAGE_BYTES + (wave + TCP_GEMM_WAVES * part) * 1024u);             \
@@ -272,20 +274,20 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
         if (step + 1u < steps) {
             TCP_ISSUE(step + 1u, buffer ^ 1u);
         }
-        /* a wavefront asks for three loads a step (two column groups and its weights), two when its strip lies past
+        /* a wavefront asks for its column groups and its weights a step, the groups alone when its strip lies past
          * the matrix: this step's have landed once nothing but the next step's is outstanding */
         if (step + 1u >= steps) {
             tcp_wait_loads<0>();
         } else if (strip_is_live) {
-            tcp_wait_loads<3>();
+            tcp_wait_loads<TCP_OPERAND_PARTS + 1u>();
         } else {
-            tcp_wait_loads<2>();
+            tcp_wait_loads<TCP_OPERAND_PARTS>();
         }
         __syncthreads(); /* the other wavefronts' column groups of this step have landed as well */
-        uint2_t b_low[TCP_COLUMN_BLOCKS], b_high[TCP_COLUMN_BLOCKS];
+        uint2_t b_low[LIVE], b_high[LIVE]; /* the column blocks that hold a pair (LIVE of them: a constant) */
         const uint32_t stage_base = stage + buffer * TCP_STAGE_BYTES;
 #pragma unroll
-        for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
+        for (uint32_t j = 0; j < LIVE; j++) {
             b_low[j] = *(const __attribute__((address_space(3))) uint2_t *)(uintptr_t)(stage_base + j * 1024u + read_low);
             b_high[j] = *(const __attribute__((address_space(3))) uint2_t *)(uintptr_t)(stage_base + j * 1024u + read_high);
         }
@@ -305,7 +307,7 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
                 exl3_decode_run<bits_x2>(f1, a[1], a[3]); /* run 1: inputs 4 q + {2, 3} and {10, 11} */
                 const half8_t weights = __builtin_bit_cast(half8_t, *(const uint4_t *)a);
 #pragma unroll
-                for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
+                for (uint32_t j = 0; j < LIVE; j++) {
                     const uint32_t b[4] = {b_low[j].x, b_low[j].y, b_high[j].x, b_high[j].y};
                     accumulator[n][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(weights, __builtin_bit_cast(half8_t, *(const uint4_t *)b),
                                                                                accumulator[n][j], 0, 0, 0);
@@ -348,13 +350,26 @@ extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS) exl3_tcp_gemm(str
     const uint32_t stage = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)stages;
     const uint32_t window = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)&windows[wave][0];
     float4_t accumulator[TCP_WAVE_TILES][TCP_COLUMN_BLOCKS];
+    /* one instance a width and a count of live column blocks (4, 8 or all): the blocks past the count keep their zeros */
+    const uint32_t live_blocks = (chunk.pair_count + 15u) / 16u;
+#define TCP_GEMM_OF(bits, live) tcp_wave_gemm<bits, live>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator)
+#define TCP_GEMM_WIDTH(bits)                \
+    if (live_blocks <= 4u) {                \
+        TCP_GEMM_OF(bits, 4u);              \
+    } else if (live_blocks <= 8u) {         \
+        TCP_GEMM_OF(bits, 8u);              \
+    } else {                                \
+        TCP_GEMM_OF(bits, TCP_COLUMN_BLOCKS); \
+    }
     switch (bits_x2) {
-    case 4u: tcp_wave_gemm<4u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
-    case 5u: tcp_wave_gemm<5u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
-    case 6u: tcp_wave_gemm<6u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
-    case 8u: tcp_wave_gemm<8u>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator); break;
+    case 4u: TCP_GEMM_WIDTH(4u) break;
+    case 5u: TCP_GEMM_WIDTH(5u) break;
+    case 6u: TCP_GEMM_WIDTH(6u) break;
+    case 8u: TCP_GEMM_WIDTH(8u) break;
     default: return; /* no width of the format: the prepare refuses such a record */
     }
+#undef TCP_GEMM_WIDTH
+#undef TCP_GEMM_OF
     if (!strip_is_live) {
         return;
     }

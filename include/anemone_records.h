@@ -329,7 +329,7 @@ ANEMONE_INLINE uint64_t exl3_tc_workspace_bytes(uint64_t pairs, uint64_t hidden,
  * gate and up operands of every placed pair; the gate/up GEMM; the activation and the down operands; the down GEMM;
  * the combine of a row's pairs in slot order. */
 #define EXL3_TCP_KERNEL_FILE "kernel_exl3_tcp"
-#define EXL3_TCP_CHUNK_PAIRS 128u  /* columns of one GEMM block: pairs of one expert */
+#define EXL3_TCP_CHUNK_PAIRS 160u  /* columns of one GEMM block: pairs of one expert (ten MFMA column blocks) */
 #define EXL3_TCP_BLOCK_OUTPUTS 256u /* outputs of one GEMM block: four wavefronts of four tiles */
 #define EXL3_TCP_LAUNCHES 7u
 #define EXL3_TCP_MOST_LAUNCHES 8u  /* the reference's bound of its own forms */

@@ -61,7 +61,7 @@ def oracle_layer(layer, x, experts, weights, matrices, widths, threads=8):
 
 
 @pytest.mark.parametrize("hidden,inner,experts_n,picks,rows,width_choices,skew", [
-    (512, 256, 64, 4, 300, [2, 3, 4], 1.5),   # a few experts with more than one chunk of 128 pairs, others ragged
+    (512, 256, 64, 4, 300, [2, 3, 4], 1.5),   # a few experts with more than one chunk of pairs, others ragged
     (512, 384, 64, 8, 70, [3], 0.0),          # one width; 384 outputs: a GEMM block whose last wavefronts lie past the matrix
     (256, 128, 64, 2, 9, [40, 4], 0.0),       # K = 2.5 among the widths; chunks of one or two pairs, experts without any
 ])
@@ -85,7 +85,7 @@ def test_prefill_layer_against_oracle(amd, card, hidden, inner, experts_n, picks
     card.upload(layer.tcp_workspace_offset, np.full(layout["operands"], 0xA5, dtype=np.uint8))
     card.upload(layer.out_offset, np.full(rows * hidden * 4, 0xFF, dtype=np.uint8))
     card.run(launches)
-    # the route: sorted by expert, rows ascending; place_of its inverse; chunks of at most 128 of one expert
+    # the route: sorted by expert, rows ascending; place_of its inverse; chunks of at most EXL3_TCP_CHUNK_PAIRS of one expert
     pairs = rows * picks
     sorted_pairs = card.download(layer.tcp_workspace_offset + layout["sorted"], pairs * 4, np.uint32)
     place_of = card.download(layer.tcp_workspace_offset + layout["place_of"], pairs * 4, np.uint32)
@@ -95,8 +95,9 @@ def test_prefill_layer_against_oracle(amd, card, hidden, inner, experts_n, picks
     used = int(card.download(layer.tcp_workspace_offset + layout["header"], 4, np.uint32)[0])
     chunks = card.download(layer.tcp_workspace_offset + layout["chunks"], layout["chunk_capacity"] * 16, np.uint32).reshape(-1, 4)
     counts = np.bincount(experts.reshape(-1), minlength=experts_n)
-    assert used == int(((counts + 127) // 128).sum()) and not chunks[used:].any()
-    assert int(chunks[:used, 2].sum()) == pairs and chunks[:used, 2].max() <= 128
+    most = amd.EXL3_TCP_CHUNK_PAIRS
+    assert used == int(((counts + most - 1) // most).sum()) and not chunks[used:].any()
+    assert int(chunks[:used, 2].sum()) == pairs and chunks[:used, 2].max() <= most
     assert np.array_equal(chunks[:used, 1], np.concatenate([[0], np.cumsum(chunks[:used, 2])[:-1]]))
     say("  chunks %d, the longest run %d pairs" % (used, counts.max()))
     got = layer.output()
