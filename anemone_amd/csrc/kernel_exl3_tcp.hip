@@ -27,6 +27,7 @@
 #define TCP_WAVE_TILES 4u  /* output tiles of a wavefront: 64 outputs */
 #define TCP_COLUMN_BLOCKS (EXL3_TCP_CHUNK_PAIRS / 16u)
 #define TCP_STEP_INPUTS 32u
+#define TCP_BATCH 4u        /* columns the element-wise launches take at a time */
 #define TCP_OPERAND_PARTS ((TCP_COLUMN_BLOCKS + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES) /* 16-column groups a wavefront brings a step */
 #define TCP_STAGE_BYTES (TCP_OPERAND_PARTS * TCP_GEMM_WAVES * 1024u) /* a K step of the chunk's operand columns, in whole groups */
 
@@ -65,7 +66,7 @@ __device__ static __forceinline__ uint64_t tcp_matrix_of(const struct exl3_tcp_r
 /* launch 0: grid (ceil(row_count / ROUTER_SORT_ROWS)): counts [block][experts] */
 extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_count(struct exl3_tcp_record record, unsigned char *arena)
 {
-    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     const tcp_shape shape = tcp_shape_of(record);
     const uint32_t pairs = sort_block_picks((const struct router_pick *)(arena + record.picks_offset), shape.picks, blockIdx.x,
                                             record.row_count, block_experts);
@@ -73,9 +74,7 @@ extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_count(st
     uint32_t *counts = (uint32_t *)(arena + record.workspace_offset + shape.layout.counts) + (uint64_t)blockIdx.x * shape.experts;
     for (uint32_t expert = threadIdx.x; expert < shape.experts; expert += blockDim.x) {
         uint32_t count = 0;
-        for (uint32_t index = 0; index < pairs; index++) {
-            count += block_experts[index] == expert ? 1u : 0u;
-        }
+        sort_walk_picks(block_experts, pairs, [&](uint32_t, uint32_t picked) { count += picked == expert ? 1u : 0u; });
         counts[expert] = count;
     }
 }
@@ -85,7 +84,7 @@ ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_count, exl3_tcp_record);
  * chunks and their number */
 extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_place(struct exl3_tcp_record record, unsigned char *arena)
 {
-    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t chunk_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
     const tcp_shape shape = tcp_shape_of(record);
@@ -113,13 +112,13 @@ extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_place(st
     const uint32_t first_pair = blockIdx.x * ROUTER_SORT_ROWS * shape.picks;
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
         uint32_t place = starts[expert] + before[expert];
-        for (uint32_t index = 0; index < pairs; index++) {
-            if (block_experts[index] == expert) {
+        sort_walk_picks(block_experts, pairs, [&](uint32_t index, uint32_t picked) {
+            if (picked == expert) {
                 sorted[place] = first_pair + index;
                 place_of[first_pair + index] = place;
                 place++;
             }
-        }
+        });
     }
     if (blockIdx.x != 0u) {
         return;
@@ -187,15 +186,30 @@ extern "C" __global__ void exl3_tcp_operands(struct exl3_tcp_record record, unsi
     const uint16_t *rows = (const uint16_t *)(arena + record.hidden_offset);
     const uint32_t *sorted = (const uint32_t *)(workspace + shape.layout.sorted);
     uint16_t *operands = (uint16_t *)(workspace + shape.layout.operands) + (uint64_t)projection * shape.pairs * shape.hidden;
-    for (uint32_t column = 0; column < chunk.pair_count; column++) {
-        const uint32_t place = chunk.first_pair + column;
-        const uint64_t row = sorted[place] / shape.picks;
-        float v0 = __fmul_rn(bf16_to_float(rows[row * shape.hidden + channel]), s0);
-        float v1 = __fmul_rn(bf16_to_float(rows[row * shape.hidden + channel + WAVE]), s1);
-        wave_hadamard128(v0, v1, lane);
-        uint16_t *out = operands + (uint64_t)place * shape.hidden;
-        out[channel] = float_to_half_bits(__fmul_rn(v0, EXL3_NORMALIZATION));
-        out[channel + WAVE] = float_to_half_bits(__fmul_rn(v1, EXL3_NORMALIZATION));
+    /* TCP_BATCH columns at a time: their loads are asked for together, so that one column's latency hides behind
+     * the others' (a column past the chunk's last repeats it and is not stored) */
+    for (uint32_t first = 0; first < chunk.pair_count; first += TCP_BATCH) {
+        float v0[TCP_BATCH], v1[TCP_BATCH];
+        uint32_t place[TCP_BATCH];
+#pragma unroll
+        for (uint32_t i = 0; i < TCP_BATCH; i++) {
+            const uint32_t column = first + i < chunk.pair_count ? first + i : chunk.pair_count - 1u;
+            place[i] = chunk.first_pair + column;
+            const uint64_t row = sorted[place[i]] / shape.picks;
+            v0[i] = bf16_to_float(rows[row * shape.hidden + channel]);
+            v1[i] = bf16_to_float(rows[row * shape.hidden + channel + WAVE]);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < TCP_BATCH; i++) {
+            v0[i] = __fmul_rn(v0[i], s0);
+            v1[i] = __fmul_rn(v1[i], s1);
+            wave_hadamard128(v0[i], v1[i], lane);
+            if (first + i < chunk.pair_count) {
+                uint16_t *out = operands + (uint64_t)place[i] * shape.hidden;
+                out[channel] = float_to_half_bits(__fmul_rn(v0[i], EXL3_NORMALIZATION));
+                out[channel + WAVE] = float_to_half_bits(__fmul_rn(v1[i], EXL3_NORMALIZATION));
+            }
+        }
     }
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_operands, exl3_tcp_record);
@@ -410,26 +424,39 @@ extern "C" __global__ void exl3_tcp_activate(struct exl3_tcp_record record, unsi
     const float *gate_products = (const float *)(workspace + shape.layout.gate_up);
     const float *up_products = gate_products + (uint64_t)shape.pairs * I;
     uint16_t *operands = (uint16_t *)(workspace + shape.layout.operands);
-    for (uint32_t column = 0; column < chunk.pair_count; column++) {
-        const uint64_t place = chunk.first_pair + column;
-        float g[2] = {gate_products[place * I + channel], gate_products[place * I + channel + WAVE]};
-        float u[2] = {up_products[place * I + channel], up_products[place * I + channel + WAVE]};
-        wave_hadamard128(g[0], g[1], lane);
-        wave_hadamard128(u[0], u[1], lane);
-        float v[2];
+    for (uint32_t first = 0; first < chunk.pair_count; first += TCP_BATCH) { /* batched as the operands' loop */
+        float g[TCP_BATCH][2], u[TCP_BATCH][2];
+        uint64_t place[TCP_BATCH];
 #pragma unroll
-        for (uint32_t i = 0; i < 2u; i++) {
-            const float gate = __fmul_rn(__fmul_rn(g[i], EXL3_NORMALIZATION), gs[i]);
-            const float up = __fmul_rn(__fmul_rn(u[i], EXL3_NORMALIZATION), us[i]);
-            const float bounded_gate = limit > 0.0f ? fminf(gate, limit) : gate;
-            const float bounded_up = limit > 0.0f ? fminf(fmaxf(up, -limit), limit) : up;
-            const float hidden = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
-            v[i] = __fmul_rn(hidden, ds[i]);
+        for (uint32_t i = 0; i < TCP_BATCH; i++) {
+            const uint32_t column = first + i < chunk.pair_count ? first + i : chunk.pair_count - 1u;
+            place[i] = chunk.first_pair + column;
+            g[i][0] = gate_products[place[i] * I + channel];
+            g[i][1] = gate_products[place[i] * I + channel + WAVE];
+            u[i][0] = up_products[place[i] * I + channel];
+            u[i][1] = up_products[place[i] * I + channel + WAVE];
         }
-        wave_hadamard128(v[0], v[1], lane);
-        uint16_t *operand = operands + place * I;
-        operand[channel] = float_to_half_bits(__fmul_rn(v[0], EXL3_NORMALIZATION));
-        operand[channel + WAVE] = float_to_half_bits(__fmul_rn(v[1], EXL3_NORMALIZATION));
+#pragma unroll
+        for (uint32_t i = 0; i < TCP_BATCH; i++) {
+            wave_hadamard128(g[i][0], g[i][1], lane);
+            wave_hadamard128(u[i][0], u[i][1], lane);
+            float v[2];
+#pragma unroll
+            for (uint32_t half = 0; half < 2u; half++) {
+                const float gate = __fmul_rn(__fmul_rn(g[i][half], EXL3_NORMALIZATION), gs[half]);
+                const float up = __fmul_rn(__fmul_rn(u[i][half], EXL3_NORMALIZATION), us[half]);
+                const float bounded_gate = limit > 0.0f ? fminf(gate, limit) : gate;
+                const float bounded_up = limit > 0.0f ? fminf(fmaxf(up, -limit), limit) : up;
+                const float hidden = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
+                v[half] = __fmul_rn(hidden, ds[half]);
+            }
+            wave_hadamard128(v[0], v[1], lane);
+            if (first + i < chunk.pair_count) {
+                uint16_t *operand = operands + place[i] * I;
+                operand[channel] = float_to_half_bits(__fmul_rn(v[0], EXL3_NORMALIZATION));
+                operand[channel + WAVE] = float_to_half_bits(__fmul_rn(v[1], EXL3_NORMALIZATION));
+            }
+        }
     }
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_activate, exl3_tcp_record);

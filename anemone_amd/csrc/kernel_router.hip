@@ -390,7 +390,7 @@ __device__ static __forceinline__ uint32_t wide_block_picks(const struct router_
 extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     router_wide_count(struct router_wide_arguments arguments, unsigned char *arena)
 {
-    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     const uint32_t live_rows = wide_live_rows(arguments, arena);
     const uint32_t pairs = wide_block_picks(arguments, arena, blockIdx.x, live_rows, block_experts);
     __syncthreads();
@@ -400,9 +400,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     uint32_t *counts = (uint32_t *)(arena + arguments.counts_offset) + (uint64_t)blockIdx.x * arguments.expert_count;
     for (uint32_t expert = threadIdx.x; expert < arguments.expert_count; expert += blockDim.x) {
         uint32_t count = 0;
-        for (uint32_t index = 0; index < pairs; index++) {
-            count += block_experts[index] == expert ? 1u : 0u;
-        }
+        sort_walk_picks(block_experts, pairs, [&](uint32_t, uint32_t picked) { count += picked == expert ? 1u : 0u; });
         counts[expert] = count;
     }
 }
@@ -423,12 +421,12 @@ __device__ static __forceinline__ void wide_place_block(const struct router_wide
     const uint32_t first_pair = block * ROUTER_SORT_ROWS * picks;
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
         uint32_t place = starts[expert] + before[expert];
-        for (uint32_t index = 0; index < pairs; index++) {
-            if (block_experts[index] == expert) {
+        sort_walk_picks(block_experts, pairs, [&](uint32_t index, uint32_t picked) {
+            if (picked == expert) {
                 sorted[place] = (struct wide_pair){first_pair + index, all_picks[first_pair + index].route_weight};
                 place++;
             }
-        }
+        });
     }
     if (block != 0u) {
         return;
@@ -472,7 +470,7 @@ __device__ static __forceinline__ void wide_place_block(const struct router_wide
 extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     router_wide_place(struct router_wide_arguments arguments, unsigned char *arena)
 {
-    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
     const uint32_t experts = arguments.expert_count;
@@ -570,7 +568,7 @@ ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_jobs, router_wide_arguments);
 extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     router_wide_small(struct router_wide_arguments arguments, unsigned char *arena)
 {
-    __shared__ uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS], job_starts[ROUTER_MOST_EXPERTS + 1u];
     const uint32_t experts = arguments.expert_count;
@@ -579,9 +577,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     __syncthreads();
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
         uint32_t count = 0;
-        for (uint32_t index = 0; index < pairs; index++) {
-            count += block_experts[index] == expert ? 1u : 0u;
-        }
+        sort_walk_picks(block_experts, pairs, [&](uint32_t, uint32_t picked) { count += picked == expert ? 1u : 0u; });
         totals[expert] = count;
         starts[expert] = count;
         before[expert] = 0u;

@@ -24,6 +24,29 @@ __device__ static __forceinline__ uint32_t sort_block_picks(const struct router_
     return rows * picks_per_row;
 }
 
+/* Every pick of a block in order, eight at a time (two 16-byte LDS reads in flight, not one 4-byte read a step):
+ * visit(index, expert). block_experts is 16-byte aligned. */
+template <typename Visit>
+__device__ static __forceinline__ void sort_walk_picks(const uint32_t *block_experts, uint32_t pairs, Visit visit)
+{
+    typedef __attribute__((ext_vector_type(4))) uint32_t four_words;
+    uint32_t index = 0;
+    for (; index + 8u <= pairs; index += 8u) {
+        const four_words low = *(const four_words *)(block_experts + index), high = *(const four_words *)(block_experts + index + 4u);
+        visit(index, low.x);
+        visit(index + 1u, low.y);
+        visit(index + 2u, low.z);
+        visit(index + 3u, low.w);
+        visit(index + 4u, high.x);
+        visit(index + 5u, high.y);
+        visit(index + 6u, high.z);
+        visit(index + 7u, high.w);
+    }
+    for (; index < pairs; index++) {
+        visit(index, block_experts[index]);
+    }
+}
+
 /* exclusive prefix sums of values[0 .. count) in LDS, count <= ROUTER_MOST_EXPERTS, by the whole block; total returned */
 __device__ static __forceinline__ uint32_t block_exclusive_scan(uint32_t *values, uint32_t count, uint32_t *scratch)
 {
