@@ -83,7 +83,7 @@ class Exl3TcRecord(C.Structure):
 
 class RouterKernels(C.Structure):
     _fields_ = [(name, u32) for name in ("select", "wide_select", "wide_count", "wide_place", "wide_jobs",
-                                         "wide_small", "select_draft", "projection")]
+                                         "wide_small", "select_draft", "projection", "projection_tiles")]
 
 
 class RoutedExpertsDescription(C.Structure):

@@ -155,6 +155,95 @@ extern "C" __global__ void __launch_bounds__(PROJECTION_THREADS)
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_projection, router_projection_arguments);
 
+/* The same scores on the matrix unit, for steps of many rows. v_mfma_f32_16x16x1_4b_f32 adds, to each of four 16 x 16
+ * blocks of sums, one product a sum, each a fused multiply-add of float32 rounded once (compared bit for bit with
+ * fmaf over wide exponent ranges, subnormal products and infinities): a block is a chain, its 16 x 16 sums the chains
+ * of 16 experts by 16 rows, and the eight instructions of a group of 32 inputs advance the 32 chains by one input
+ * each, in the definition's order. Instruction q takes the chains 8 b + q of the blocks b = 0 .. 3, so that lane
+ * (b, n) needs the inputs 32 i + 8 b + {0 .. 7} of expert n (and of row n): one 16-byte load each a group. The fold is
+ * inside a lane. grid (E / 16, ceil(rows / 64)), block 256: a wavefront 16 rows. */
+typedef __attribute__((ext_vector_type(16))) float float16_t;
+extern "C" __global__ void __launch_bounds__(PROJECTION_TILE_THREADS, 2) /* two blocks a CU: two wavefronts a SIMD */
+    router_projection_tiles(struct router_projection_arguments arguments, unsigned char *arena)
+{
+    const uint32_t lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, block = lane / 16u, index = lane % 16u;
+    const uint32_t H = arguments.hidden, groups = H / PROJECTION_CHAINS;
+    const uint32_t first_expert = blockIdx.x * 16u, first_row = (blockIdx.y * (PROJECTION_TILE_THREADS / WAVE) + wave) * 16u;
+    if (first_row >= arguments.row_count) {
+        return; /* the whole wavefront */
+    }
+    /* a row past the last repeats the last: its sums are not stored */
+    const uint32_t row = first_row + index < arguments.row_count ? first_row + index : arguments.row_count - 1u;
+    const uint4_t *w = (const uint4_t *)((const uint16_t *)(arena + arguments.weights_offset) + (uint64_t)(first_expert + index) * H + 8u * block);
+    const uint4_t *x = (const uint4_t *)((const uint16_t *)(arena + arguments.rows_offset) + (uint64_t)row * H + 8u * block);
+    float16_t chain[8];
+#pragma unroll
+    for (uint32_t q = 0; q < 8u; q++) {
+#pragma unroll
+        for (uint32_t v = 0; v < 16u; v++) {
+            chain[q][v] = 0.0f;
+        }
+    }
+    /* PROJECTION_TILE_AHEAD groups are asked for ahead of the one in use (a group is 32 bfloat16: four 16-byte pieces
+     * on); the ring is indexed by constants: the loop is unrolled by its length */
+    uint4_t w_ring[PROJECTION_TILE_AHEAD], x_ring[PROJECTION_TILE_AHEAD];
+#pragma unroll
+    for (uint32_t ahead = 0; ahead < PROJECTION_TILE_AHEAD; ahead++) {
+        const uint32_t group = ahead < groups ? ahead : groups - 1u;
+        w_ring[ahead] = w[4u * group];
+        x_ring[ahead] = x[4u * group];
+    }
+    for (uint32_t first = 0; first < groups; first += PROJECTION_TILE_AHEAD) {
+#pragma unroll
+        for (uint32_t slot = 0; slot < PROJECTION_TILE_AHEAD; slot++) {
+            const uint32_t group = first + slot;
+            if (group >= groups) { /* the same in every lane */
+                break;
+            }
+            const uint4_t w_now = w_ring[slot], x_now = x_ring[slot];
+            const uint32_t next = group + PROJECTION_TILE_AHEAD < groups ? group + PROJECTION_TILE_AHEAD : groups - 1u;
+            w_ring[slot] = w[4u * next];
+            x_ring[slot] = x[4u * next];
+            const uint32_t w_words[4] = {w_now.x, w_now.y, w_now.z, w_now.w}, x_words[4] = {x_now.x, x_now.y, x_now.z, x_now.w};
+#pragma unroll
+            for (uint32_t q = 0; q < 8u; q++) {
+                const float a = __uint_as_float(q % 2u == 0u ? w_words[q / 2u] << 16 : w_words[q / 2u] & 0xFFFF0000u);
+                const float b = __uint_as_float(q % 2u == 0u ? x_words[q / 2u] << 16 : x_words[q / 2u] & 0xFFFF0000u);
+                chain[q] = __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, chain[q], 0, 0, 0);
+            }
+        }
+    }
+    /* register v = 4 b + r of chain[q] is chain 8 b + q of expert 4 (lane / 16) + r and row lane % 16. The fold, as the
+     * definition orders it: + 0 first, then the distances 16 and 8 (blocks), 4, 2 and 1 (instructions) */
+    float sums[8][8];
+#pragma unroll
+    for (uint32_t q = 0; q < 8u; q++) {
+#pragma unroll
+        for (uint32_t v = 0; v < 8u; v++) {
+            sums[q][v] = __fadd_rn(__fadd_rn(0.0f, chain[q][v]), __fadd_rn(0.0f, chain[q][v + 8u]));
+        }
+#pragma unroll
+        for (uint32_t r = 0; r < 4u; r++) {
+            sums[q][r] = __fadd_rn(sums[q][r], sums[q][r + 4u]);
+        }
+    }
+#pragma unroll
+    for (uint32_t distance = 4u; distance != 0u; distance >>= 1u) {
+#pragma unroll
+        for (uint32_t q = 0; q < distance; q++) {
+#pragma unroll
+            for (uint32_t r = 0; r < 4u; r++) {
+                sums[q][r] = __fadd_rn(sums[q][r], sums[q + distance][r]);
+            }
+        }
+    }
+    if (first_row + index < arguments.row_count) {
+        float *out = (float *)(arena + arguments.output_offset) + (uint64_t)(first_row + index) * arguments.expert_count + first_expert + 4u * block;
+        *(float4_t *)out = (float4_t){__fadd_rn(0.0f, sums[0][0]), __fadd_rn(0.0f, sums[0][1]), __fadd_rn(0.0f, sums[0][2]), __fadd_rn(0.0f, sums[0][3])};
+    }
+}
+ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_projection_tiles, router_projection_arguments);
+
 __device__ static __forceinline__ uint64_t router_key(float biased, uint32_t expert)
 {
     const uint32_t bits = __float_as_uint(biased);

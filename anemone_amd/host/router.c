@@ -7,6 +7,7 @@
  *
  *   launch        kernel                grid                        block
  *   projection    router_projection     (ceil(E / 8), ceil(rows / 4), 1)   128   eight experts and four rows a block
+ *                 router_projection_tiles (E / 16, ceil(rows / 64), 1)     256   257 rows and more: 16 experts by 64 rows a block
  *   select        router_select_entry   (1, 1, 1)                   512   a wavefront a row
  *   wide select   router_wide_select    (ceil(rows / 8), 1, 1)      512   a wavefront a row
  *   wide count    router_wide_count     (ceil(rows / 384), 1, 1)    512   a thread an expert
@@ -64,7 +65,13 @@ result_status router_kernels_prepare(const struct backend_operations *backend, s
     if (projected != STATUS_OK) {
         return projected;
     }
-    memcpy(kernels_out, handles, sizeof *kernels_out);
+    uint32_t tiles = BACKEND_NO_KERNEL;
+    if (backend->kernel_prepare(card, KERNEL_FILE_ROUTER, KERNEL_ROUTER_PROJECTION_TILES, sizeof(struct router_projection_arguments),
+                                &tiles) != STATUS_OK) {
+        tiles = BACKEND_NO_KERNEL; /* every row count then takes router_projection */
+    }
+    memcpy(kernels_out, handles, sizeof handles);
+    kernels_out->projection_tiles = tiles;
     return STATUS_OK;
 }
 
@@ -240,6 +247,13 @@ result_status router_projection_prepare(const struct router_projection_descripti
         .hidden = description->hidden,
         .expert_count = description->expert_count,
     };
+    if (kernels->projection_tiles != BACKEND_NO_KERNEL && description->row_count >= PROJECTION_TILE_LEAST_ROWS &&
+        description->expert_count % 16u == 0) { /* many rows: the chains on the matrix unit, 16 experts by 64 rows a block */
+        launch_fill(launch_out, kernels->projection_tiles, description->expert_count / 16u,
+                    (description->row_count + PROJECTION_TILE_ROWS - 1u) / PROJECTION_TILE_ROWS, 1, PROJECTION_TILE_THREADS, 0, &record,
+                    sizeof record);
+        return STATUS_OK;
+    }
     launch_fill(launch_out, kernels->projection, (description->expert_count + PROJECTION_OUTPUTS - 1u) / PROJECTION_OUTPUTS,
                 (description->row_count + PROJECTION_ROWS - 1u) / PROJECTION_ROWS, 1, PROJECTION_THREADS, 0, &record, sizeof record);
     return STATUS_OK;

@@ -113,6 +113,7 @@ struct router_kernels_record {
     uint32_t wide_small;
     uint32_t select_draft; /* BACKEND_NO_KERNEL: the draft's router is outside this path */
     uint32_t projection;   /* no counterpart: the router's score projection as its own launch */
+    uint32_t projection_tiles; /* no counterpart: the same scores for steps of 257 rows and more, on the matrix unit */
 };
 MUST_CHECK result_status router_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                 struct router_kernels_record *kernels_out);

@@ -104,6 +104,11 @@ ANEMONE_RECORD_HAS(wide_expert_tile, 32);
 /* ---- router ---- */
 #define KERNEL_FILE_ROUTER "kernel_router"
 #define KERNEL_ROUTER_PROJECTION "router_projection"
+#define KERNEL_ROUTER_PROJECTION_TILES "router_projection_tiles" /* the same scores on the matrix unit: steps of many rows */
+#define PROJECTION_TILE_THREADS 256u
+#define PROJECTION_TILE_ROWS 64u   /* rows of a block of router_projection_tiles: 16 a wavefront */
+#define PROJECTION_TILE_LEAST_ROWS 257u /* fewer rows take router_projection: its blocks are smaller and more */
+#define PROJECTION_TILE_AHEAD 4u        /* groups of 32 inputs asked for ahead */
 #define KERNEL_ROUTER_SELECT "router_select_entry"
 #define KERNEL_ROUTER_WIDE_SELECT "router_wide_select"
 #define KERNEL_ROUTER_WIDE_COUNT "router_wide_count"

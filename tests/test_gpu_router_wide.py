@@ -156,6 +156,29 @@ def test_wide_small_equals_the_four_launches(amd, card, experts_n, picks, rows, 
     assert np.all(wide.read("counts", np.uint8) == 0xEE)  # the counts scratch stays unwritten
 
 
+@pytest.mark.parametrize("experts_n,rows,hidden,scale", [(64, 300, 512, 1.0), (256, 257, 1024, 1.0), (64, 321, 128, 1e-18), (128, 1000, 256, 3e18), (64, 700, 384, 1.0)])
+def test_projection_of_many_rows_bit_exact(amd, card, experts_n, rows, hidden, scale):
+    """router_projection_tiles (257 rows and more: the 32 chains of a score as matrix-unit products of one input each)
+    against the oracle's chains, every bit; scales that put products among the subnormals and near overflow among
+    the cases."""
+    say("projection, many rows", experts_n, rows, hidden, scale)
+    layer, _ = small_layer(amd, card, experts_n, 2, rows, hidden=hidden)
+    router = to_bf16(normals(41, experts_n * hidden) * scale).reshape(experts_n, hidden)
+    x = to_bf16(normals(42, rows * hidden) * scale).reshape(rows, hidden)
+    card.upload(layer.router_offset, router)
+    layer.set_rows(x, rows)
+    launch = layer.projection_launch()
+    assert list(launch[0].block)[0] == 256 and list(launch[0].grid) == [experts_n // 16, (rows + 63) // 64, 1]
+    card.upload(layer.scores_offset, np.full(rows * experts_n * 4, 0xEE, dtype=np.uint8))
+    card.run(launch)
+    got = card.download(layer.scores_offset, rows * experts_n * 4, np.float32).reshape(rows, experts_n)
+    want = np.zeros((rows, experts_n), dtype=np.float32)
+    orc.orc_router_projection(ptr(x, u16p), ptr(router, u16p), rows, hidden, experts_n, ptr(want, f32p))
+    differing = np.flatnonzero(got.view(np.uint32) != want.view(np.uint32))
+    say("  %d of %d scores differ" % (differing.size, got.size))
+    assert differing.size == 0
+
+
 def test_fp4_layer_through_the_wide_job_table(amd, card):
     """40 rows (37 live) routed by the wide select, then the FP4 experts over its job table, against the oracle."""
     say("fp4 layer, wide")
