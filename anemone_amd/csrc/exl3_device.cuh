@@ -97,9 +97,11 @@ __device__ static __forceinline__ void wave_hadamard128(float &v0, float &v1, ui
     for (uint32_t distance = 1; distance < WAVE; distance *= 2u) {
         const float o0 = __shfl_xor(v0, (int)distance, WAVE);
         const float o1 = __shfl_xor(v1, (int)distance, WAVE);
-        const bool lower = (lane & distance) == 0u;
-        v0 = lower ? __fadd_rn(v0, o0) : __fsub_rn(o0, v0);
-        v1 = lower ? __fadd_rn(v1, o1) : __fsub_rn(o1, v1);
+        /* the lower of a pair becomes lower + upper, the upper lower - upper: other + own or other - own, one
+         * rounding either way: a fused multiply-add of own by +1 or -1 (the product is exact) */
+        const float sign = (lane & distance) == 0u ? 1.0f : -1.0f;
+        v0 = __fmaf_rn(sign, v0, o0);
+        v1 = __fmaf_rn(sign, v1, o1);
     }
     const float sum = __fadd_rn(v0, v1), difference = __fsub_rn(v0, v1);
     v0 = sum;

@@ -551,19 +551,41 @@ EXPERT_ENTRIES(2);
 EXPERT_ENTRIES(4);
 EXPERT_ENTRIES(8);
 
-/* float32 sum of a row's bfloat16 pair outputs from +0 in ascending slot order; grid (ceil(width / 256), rows) */
+/* float32 sum of a row's bfloat16 pair outputs from +0 in ascending slot order; a thread takes
+ * EXPERT_ROW_SUM_CHANNELS consecutive outputs (one 16-byte load a slot); grid (ceil(width / (8 x 256)), rows) */
 extern "C" __global__ void expert_row_sum_entry(struct expert_row_sum_arguments arguments, unsigned char *arena)
 {
-    const uint32_t channel = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t channel = (blockIdx.x * blockDim.x + threadIdx.x) * EXPERT_ROW_SUM_CHANNELS;
     if (channel >= arguments.width) {
         return;
     }
     const uint64_t row = blockIdx.y;
-    const uint16_t *pairs = (const uint16_t *)(arena + arguments.pair_output_offset);
-    float sum = 0.0f;
-    for (uint32_t slot = 0; slot < arguments.pairs_per_row; slot++) {
-        sum = __fadd_rn(sum, bf16_to_float(pairs[(row * arguments.pairs_per_row + slot) * arguments.width + channel]));
+    const uint16_t *pairs = (const uint16_t *)(arena + arguments.pair_output_offset) + row * arguments.pairs_per_row * arguments.width + channel;
+    float *out = (float *)(arena + arguments.row_output_offset) + row * arguments.width + channel;
+    float sum[EXPERT_ROW_SUM_CHANNELS];
+#pragma unroll
+    for (uint32_t i = 0; i < EXPERT_ROW_SUM_CHANNELS; i++) {
+        sum[i] = 0.0f;
     }
-    ((float *)(arena + arguments.row_output_offset))[row * arguments.width + channel] = sum;
+    if (arguments.width % EXPERT_ROW_SUM_CHANNELS == 0u) {
+        for (uint32_t slot = 0; slot < arguments.pairs_per_row; slot++) {
+            const uint4_t eight = *(const uint4_t *)(pairs + (uint64_t)slot * arguments.width);
+            const uint32_t words[4] = {eight.x, eight.y, eight.z, eight.w};
+#pragma unroll
+            for (uint32_t i = 0; i < EXPERT_ROW_SUM_CHANNELS; i++) {
+                sum[i] = __fadd_rn(sum[i], __uint_as_float(i % 2u == 0u ? words[i / 2u] << 16 : words[i / 2u] & 0xFFFF0000u));
+            }
+        }
+        *(float4_t *)out = (float4_t){sum[0], sum[1], sum[2], sum[3]};
+        *(float4_t *)(out + 4) = (float4_t){sum[4], sum[5], sum[6], sum[7]};
+        return;
+    }
+    for (uint32_t i = 0; i < EXPERT_ROW_SUM_CHANNELS && channel + i < arguments.width; i++) { /* a width that is no multiple of 8 */
+        float one = 0.0f;
+        for (uint32_t slot = 0; slot < arguments.pairs_per_row; slot++) {
+            one = __fadd_rn(one, bf16_to_float(pairs[(uint64_t)slot * arguments.width + i]));
+        }
+        out[i] = one;
+    }
 }
 ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_row_sum_entry, expert_row_sum_arguments);

@@ -7,7 +7,7 @@
  *   gate/up     expert_gate_up_<S>          (output_size / 16, jobs, 1)           128 S        static
  *   quantize    activation_quantize_entry   (ceil(width / 256), pairs, 1)         256          0
  *   down        expert_down_<S>             (output_size / 16, jobs, 1)           64 S         static
- *   row sum     expert_row_sum_entry        (ceil(width / 256), rows, 1)          256          0
+ *   row sum     expert_row_sum_entry        (ceil(width / 2048), rows, 1)         256          0
  * A wavefront is 64 lanes, so a slice is a wavefront (gate with up: two); 16 slices would be a block of 2,048
  * threads, which the card does not run: the instances are 1, 2, 4 and 8.
  */
@@ -17,6 +17,7 @@
 
 #include "prepare_common.h"
 
+#define ROW_SUM_BLOCK_OUTPUTS (EXPERT_ROW_SUM_CHANNELS * LINEAR_ELEMENT_THREADS) /* outputs a block of the row sum takes */
 #define LINEAR_STRIP_OUTPUTS 64u /* a block of the expert kernels: a strip of four tiles of 16 outputs */
 static const uint32_t slice_counts[LINEAR_SLICE_INSTANCES] = {1u, 2u, 4u, 8u, 16u};
 #define BUILT_INSTANCES 4u
@@ -235,7 +236,7 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_DOWN], down_kernel,
                 (down->output_size + strip_outputs - 1u) / strip_outputs, description->job_count, 1, 64u * description->down_slice_count, 0, &down_record, sizeof down_record);
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_ROW_SUM], kernels->expert_row_sum,
-                (down->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)rows, 1,
+                (down->output_size + ROW_SUM_BLOCK_OUTPUTS - 1u) / ROW_SUM_BLOCK_OUTPUTS, (uint32_t)rows, 1,
                 LINEAR_ELEMENT_THREADS, 0, &row_sum_record, sizeof row_sum_record);
     memcpy(launches_out, launches, sizeof launches);
     return STATUS_OK;
@@ -247,7 +248,7 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
  *   launch      kernel                       grid                                       block   dynamic LDS
  *   gate/up     wide_expert_gate_up_1        (ceil(I / 128), tile_count, 1)             256     WIDE_GATE_UP_WINDOW_BYTES
  *   down        wide_expert_down_1           (ceil(H / (4 strips)), tile_count, 1)      256     WIDE_DOWN_WINDOW_BYTES
- *   row sum     expert_row_sum_entry         (ceil(H / 256), rows, 1)                   256
+ *   row sum     expert_row_sum_entry         (ceil(H / 2048), rows, 1)                  256
  * strip = 64 outputs of E2M1 weights, 32 of E4M3.
  */
 #define WIDE_MOST_ROWS 16384u
@@ -356,7 +357,7 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_DOWN], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
                 description->tile_count, 1, WIDE_BLOCK_THREADS, bytes ? WIDE_DOWN_E4M3_WINDOW_BYTES : WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_ROW_SUM], linear_kernels->expert_row_sum,
-                (down->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)rows, 1, LINEAR_ELEMENT_THREADS, 0,
+                (down->output_size + ROW_SUM_BLOCK_OUTPUTS - 1u) / ROW_SUM_BLOCK_OUTPUTS, (uint32_t)rows, 1, LINEAR_ELEMENT_THREADS, 0,
                 &row_sum_record, sizeof row_sum_record);
     memcpy(launches_out, launches, sizeof launches);
     return STATUS_OK;

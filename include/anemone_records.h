@@ -269,6 +269,7 @@ struct exl3_expert_record {
 };
 ANEMONE_RECORD_HAS(exl3_expert_record, 88);
 
+#define EXPERT_ROW_SUM_CHANNELS 8u /* consecutive outputs a thread of expert_row_sum_entry sums */
 struct expert_row_sum_arguments {
     uint64_t pair_output_offset;
     uint64_t row_output_offset;

@@ -416,7 +416,7 @@ def test_linear_prepare_geometry_and_refusals(fake):
     assert lib.linear_routed_experts_prepare(C.byref(experts_description()), ARENA, C.byref(kernels), launches) == 0
     names = [fake.handles[l.kernel][1] for l in launches]
     assert names == ["expert_gate_up_4", "activation_quantize_entry", "expert_down_2", "expert_row_sum_entry"]
-    assert [list(l.grid) for l in launches] == [[32, 64, 1], [8, 64, 1], [64, 64, 1], [16, 8, 1]]
+    assert [list(l.grid) for l in launches] == [[32, 64, 1], [8, 64, 1], [64, 64, 1], [2, 8, 1]]
     assert [l.block[0] for l in launches] == [256, 256, 128, 256]
     assert [l.argument_byte_count for l in launches] == [64, 40, 56, 24]
     fp8 = amd.launches_of(4)
@@ -479,7 +479,7 @@ def test_wide_linear_prepare_geometry_and_refusals(fake):
     assert lib.linear_wide_experts_prepare(C.byref(wide_experts_description()), arena, C.byref(linear), C.byref(kernels), launches) == 0
     assert [fake.handles[l.kernel][1] for l in launches] == ["wide_expert_gate_up_1", "wide_expert_down_1", "expert_row_sum_entry"]
     tiles = 1024 * 8 // 64 + 256
-    assert [list(l.grid) for l in launches] == [[16, tiles, 1], [16, tiles, 1], [16, 1024, 1]]
+    assert [list(l.grid) for l in launches] == [[16, tiles, 1], [16, tiles, 1], [2, 1024, 1]]
     assert [l.block[0] for l in launches] == [256, 256, 256]
     assert [l.dynamic_shared_byte_count for l in launches] == [53760, 51712, 0]  # three blocks of either fit a CU's 160 KB
     assert [l.argument_byte_count for l in launches] == [88, 64, 24]
