@@ -143,6 +143,7 @@ struct wide_chain {
             b[j] = (int8_vector){(int)low.x, (int)low.y, (int)low.z, (int)low.w, (int)high.x, (int)high.y, (int)high.z, (int)high.w};
             scale_b[j] = lds_read<unsigned char>(b_scale_at + VECTOR_SCALE_AT + j * 64u);
         }
+        __builtin_amdgcn_s_setprio(1); /* the wavefront that feeds the matrix unit goes first at the issue */
 #pragma unroll
         for (uint32_t tile = 0; tile < TILES; tile++) {
             int8_vector a = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -172,6 +173,7 @@ struct wide_chain {
                 }
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stage is read before the next barrier */
     }
 
@@ -347,12 +349,13 @@ struct wide_chain {
     }
 };
 
-/* grid (ceil(output_size / (4 strips)), tile_count), block 256 */
-template <bool BYTES>
+/* grid (ceil(output_size / (4 strips)), tile_count), block 256; a strip is STRIP tiles of gate and STRIP of up */
+template <bool BYTES, uint32_t STRIP, uint32_t DEPTH>
 __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_expert_gate_up_arguments &arguments, unsigned char *arena)
 {
-    typedef wide_chain<2, BYTES, 2u, (BYTES ? 3u : 2u)> chain_type;
-    constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
+    typedef wide_chain<2, BYTES, STRIP, DEPTH> chain_type;
+    constexpr uint32_t TILES = chain_type::TILES, STRIP_OUTPUTS = STRIP * 16u;
+    static_assert(STRIP == 1u || STRIP == 2u, "a quantizer block of 32 outputs is one strip or two");
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
     if (tile.pair_count == 0u) {
@@ -386,23 +389,23 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
     chain_of.whole(arguments.input_size / 128u, live_blocks, chain);
     /* The hidden step, as expert_gate_up_1 rounds it (the one chain is added to +0 first, as S chains are), and the
      * quantizer's step on it, from the registers the sums are in. A lane holds, of a column of every column block, rows
-     * 4 (lane / 16) .. + 3 of the strip's two tiles: the 32 outputs of one quantizer block are the 8 values of each
-     * of the 4 lanes of a column. Codes are bytes 2 (v % 2) + g / 2 of a word, so the lanes g and g ^ 2 of a column
-     * hold the halves of the same two words: one exchange, and each writes one whole word. */
-    static_assert(STRIP == 2u, "a strip is one block of 32 outputs");
+     * 4 (lane / 16) .. + 3 of the strip's tiles. Two tiles a strip: the 32 outputs of one quantizer block are the 8
+     * values of each of the 4 lanes of a column. One tile a strip: the block is the strips of the wavefronts 2 p and
+     * 2 p + 1 (the matrix holds whole blocks of 32 outputs: both are inside it or neither), which pass each other the
+     * largest magnitude of their halves through LDS. Codes are bytes 2 (v % 2) + g / 2 of a word, so the lanes g and
+     * g ^ 2 of a column hold the halves of the same two words: one exchange, and each writes one whole word. */
     const uint32_t width = arguments.output_size, first_output = (blockIdx.x * WIDE_WAVES + wave) * STRIP_OUTPUTS;
-    if (first_output >= width) {
-        return; /* a strip wholly past the matrix (its tiles were the strip's before it) */
-    }
+    const bool strip_is_live = first_output < width; /* else: a strip wholly past the matrix (its tiles were the strip's before it) */
     const float limit = arguments.activation_limit;
     const uint32_t g = lane / 16u, upper = g / 2u;
+    uint32_t bits[WIDE_COLUMN_BLOCKS][STRIP][4];
+    float largest[WIDE_COLUMN_BLOCKS];
 #pragma unroll
     for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
         const uint32_t column = 16u * j + lane % 16u;
-        if (column < tile.pair_count) { /* the same in the four lanes of a column */
-            const struct wide_pair pair = pairs[column];
-            uint32_t bits[STRIP][4];
-            float largest = 0.0f;
+        largest[j] = 0.0f;
+        if (column < tile.pair_count && strip_is_live) { /* the same in the four lanes of a column */
+            const float weight = pairs[column].route_weight;
 #pragma unroll
             for (uint32_t n = 0; n < STRIP; n++) {
 #pragma unroll
@@ -411,22 +414,47 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
                     const float gate = bf16_to_float(float_to_bf16(gate_sum)), up = bf16_to_float(float_to_bf16(up_sum));
                     const float bounded_gate = fminf(gate, limit);
                     const float bounded_up = fminf(fmaxf(up, -limit), limit);
-                    const float value = __fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), pair.route_weight);
-                    bits[n][v] = float_to_bf16(value);
-                    largest = fmaxf(largest, fabsf(bf16_to_float((uint16_t)bits[n][v])));
+                    const float value = __fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), weight);
+                    bits[j][n][v] = float_to_bf16(value);
+                    largest[j] = fmaxf(largest[j], fabsf(bf16_to_float((uint16_t)bits[j][n][v])));
                 }
             }
-            largest = fmaxf(largest, __shfl_xor(largest, 16, WAVE));
-            largest = fmaxf(largest, __shfl_xor(largest, 32, WAVE));
-            const uint32_t code_exponent = quantize_exponent_code(largest);
-            unsigned char *codes = arena + arguments.hidden_codes_offset + (uint64_t)pair.pair_index * width;
-            uint16_t *operands = (uint16_t *)(arena + arguments.hidden_operands_offset) + (uint64_t)pair.pair_index * width;
+            largest[j] = fmaxf(largest[j], __shfl_xor(largest[j], 16, WAVE));
+            largest[j] = fmaxf(largest[j], __shfl_xor(largest[j], 32, WAVE));
+        }
+    }
+    if constexpr (STRIP == 1u) {
+        float *halves = (float *)window; /* [wavefront][column]: the stages are done with */
+        __syncthreads();
+#pragma unroll
+        for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+            if (g == 0u) {
+                halves[wave * WIDE_TILE_PAIRS + 16u * j + lane] = largest[j];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+            largest[j] = fmaxf(largest[j], halves[(wave ^ 1u) * WIDE_TILE_PAIRS + 16u * j + lane % 16u]);
+        }
+    }
+    if (!strip_is_live) {
+        return;
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < WIDE_COLUMN_BLOCKS; j++) {
+        const uint32_t column = 16u * j + lane % 16u;
+        if (column < tile.pair_count) {
+            const uint64_t pair = pairs[column].pair_index;
+            const uint32_t code_exponent = quantize_exponent_code(largest[j]);
+            unsigned char *codes = arena + arguments.hidden_codes_offset + pair * width;
+            uint16_t *operands = (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width;
 #pragma unroll
             for (uint32_t n = 0; n < STRIP; n++) {
                 uint32_t code[4], operand[4];
 #pragma unroll
                 for (uint32_t v = 0; v < 4u; v++) {
-                    quantize_code(bits[n][v], code_exponent, code[v], operand[v]);
+                    quantize_code(bits[j][n][v], code_exponent, code[v], operand[v]);
                 }
                 const uint32_t load = (tile0 + n) / 4u, step = (tile0 + n) % 4u, t = 2u * (g % 2u);
                 const uint32_t word0 = quantize_word_of(load, step, t), word1 = quantize_word_of(load, step, t + 1u);
@@ -436,8 +464,8 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
                 *(uint32_t *)(operands + word0 + 2u * upper) = operand[0] | (operand[1] << 16);
                 *(uint32_t *)(operands + word1 + 2u * upper) = operand[2] | (operand[3] << 16);
             }
-            if (g == 0u) {
-                (arena + arguments.hidden_exponents_offset)[(uint64_t)pair.pair_index * (width / 32u) + first_output / 32u] = (unsigned char)code_exponent;
+            if (g == 0u && first_output % 32u == 0u) {
+                (arena + arguments.hidden_exponents_offset)[pair * (width / 32u) + first_output / 32u] = (unsigned char)code_exponent;
             }
         }
     }
@@ -506,7 +534,7 @@ __device__ static __forceinline__ void wide_expert_down(const struct wide_expert
  * wide_down_window_bytes of anemone_records.h. */
 extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_gate_up_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
 {
-    wide_expert_gate_up<false>(arguments, arena);
+    wide_expert_gate_up<false, 2u, 2u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_gate_up_1, wide_expert_gate_up_arguments);
 extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
@@ -516,7 +544,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_1(st
 ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_1, wide_expert_down_arguments);
 extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_gate_up_e4m3_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
 {
-    wide_expert_gate_up<true>(arguments, arena);
+    wide_expert_gate_up<true, 1u, 2u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_gate_up_e4m3_1, wide_expert_gate_up_arguments);
 extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_e4m3_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
@@ -525,6 +553,6 @@ extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_e4m3
 }
 ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_e4m3_1, wide_expert_down_arguments);
 
-static_assert(wide_chain<2, false, 2u, 2u>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true, 2u, 3u>::WINDOW_BYTES == WIDE_GATE_UP_E4M3_WINDOW_BYTES &&
+static_assert(wide_chain<2, false, 2u, 2u>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true, 1u, 2u>::WINDOW_BYTES == WIDE_GATE_UP_E4M3_WINDOW_BYTES &&
                   wide_chain<1, false, 4u, 2u>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES && wide_chain<1, true, 2u, 2u>::WINDOW_BYTES == WIDE_DOWN_E4M3_WINDOW_BYTES,
               "the windows the host asks for are the kernels'");

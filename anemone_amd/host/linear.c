@@ -350,9 +350,10 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
     const struct expert_row_sum_arguments row_sum_record = {experts->pair_output.byte_offset, experts->row_output.byte_offset,
                                                             down->output_size, experts->pairs_per_row};
     const uint32_t block_outputs = 4u * strip_outputs;
+    const uint32_t gate_up_outputs = bytes ? WIDE_GATE_UP_E4M3_BLOCK_OUTPUTS : WIDE_GATE_UP_BLOCK_OUTPUTS;
     struct kernel_launch launches[LINEAR_WIDE_EXPERTS_LAUNCH_COUNT];
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_GATE_UP], gate_up_kernel,
-                (gate_up->output_size + WIDE_GATE_UP_BLOCK_OUTPUTS - 1u) / WIDE_GATE_UP_BLOCK_OUTPUTS, description->tile_count, 1,
+                (gate_up->output_size + gate_up_outputs - 1u) / gate_up_outputs, description->tile_count, 1,
                 WIDE_BLOCK_THREADS, bytes ? WIDE_GATE_UP_E4M3_WINDOW_BYTES : WIDE_GATE_UP_WINDOW_BYTES, &gate_up_record, sizeof gate_up_record);
     launch_fill(&launches[LINEAR_WIDE_EXPERTS_DOWN], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
                 description->tile_count, 1, WIDE_BLOCK_THREADS, bytes ? WIDE_DOWN_E4M3_WINDOW_BYTES : WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);

@@ -480,7 +480,8 @@ ANEMONE_RECORD_HAS(expert_gate_up_quantize_arguments, 96);
 #define WIDE_BLOCK_THREADS 256u          /* four wavefronts: four strips of one tile of pairs */
 #define WIDE_GATE_UP_BLOCK_OUTPUTS 128u   /* of gate and of up: a wavefront takes 32 of each */
 #define WIDE_GATE_UP_WINDOW_BYTES 53760u  /* dynamic LDS of wide_expert_gate_up_<S>: two stages; three blocks fit a CU */
-#define WIDE_GATE_UP_E4M3_WINDOW_BYTES 129792u /* of wide_expert_gate_up_e4m3_<S> */
+#define WIDE_GATE_UP_E4M3_BLOCK_OUTPUTS 64u /* of wide_expert_gate_up_e4m3_<S>: a wavefront takes 16 of gate and of up */
+#define WIDE_GATE_UP_E4M3_WINDOW_BYTES 53760u /* of wide_expert_gate_up_e4m3_<S>: two stages */
 #define WIDE_DOWN_WINDOW_BYTES 51712u     /* of wide_expert_down_<S>: two stages */
 #define WIDE_DOWN_E4M3_WINDOW_BYTES 51712u /* of wide_expert_down_e4m3_<S>: two stages */
 struct wide_expert_gate_up_arguments {

@@ -489,8 +489,8 @@ def test_wide_linear_prepare_geometry_and_refusals(fake):
     description = wide_experts_description(amd.WEIGHT_FORMAT_E4M3_SCALED)
     assert lib.linear_wide_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(kernels), fp8) == 0
     assert [fake.handles[l.kernel][1] for l in fp8][:2] == ["wide_expert_gate_up_e4m3_1", "wide_expert_down_e4m3_1"]
-    assert [list(l.grid) for l in fp8][:2] == [[16, tiles, 1], [32, tiles, 1]]  # strips of 32 outputs
-    assert [l.dynamic_shared_byte_count for l in fp8] == [129792, 51712, 0]
+    assert [list(l.grid) for l in fp8][:2] == [[32, tiles, 1], [32, tiles, 1]]  # strips of 16 hidden outputs, of 32 outputs
+    assert [l.dynamic_shared_byte_count for l in fp8] == [53760, 51712, 0]
     for changes in (dict(gate_up_slice_count=2), dict(down_slice_count=4), dict(tile_count=0), dict(tile_count=70000), dict(reserved_zero=1),
                     dict(row_count=0), dict(row_count=20000), dict(activation_limit=0.0), dict(weight_format=amd.WEIGHT_FORMAT_EXL3),
                     dict(tiles=amd.Range(3 << 30, 64)), dict(pairs=amd.Range((8 << 30) - 256, 65536)),
