@@ -320,12 +320,14 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
                 exl3_decode_run<bits_x2>(f0, a[0], a[2]); /* run 0: inputs 4 q + {0, 1} and {8, 9} */
                 exl3_decode_run<bits_x2>(f1, a[1], a[3]); /* run 1: inputs 4 q + {2, 3} and {10, 11} */
                 const half8_t weights = __builtin_bit_cast(half8_t, *(const uint4_t *)a);
+                __builtin_amdgcn_s_setprio(1); /* the wavefront that feeds the matrix unit goes first at the issue */
 #pragma unroll
                 for (uint32_t j = 0; j < LIVE; j++) {
                     const uint32_t b[4] = {b_low[j].x, b_low[j].y, b_high[j].x, b_high[j].y};
                     accumulator[n][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(weights, __builtin_bit_cast(half8_t, *(const uint4_t *)b),
                                                                                accumulator[n][j], 0, 0, 0);
                 }
+                __builtin_amdgcn_s_setprio(0);
             }
         }
         /* this step's stage and window are read (their values are in registers or used); the step after the next may
