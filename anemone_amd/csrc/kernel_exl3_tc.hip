@@ -197,44 +197,81 @@ extern "C" __global__ void exl3_tc_combine(struct exl3_tc_record record, unsigne
     const struct expert_job_record *jobs = (const struct expert_job_record *)(arena + record.jobs_offset);
     const unsigned char *workspace = arena + record.workspace_offset;
     const float *partials = (const float *)(workspace + exl3_tc_operand_bytes(shape.pairs, H) + exl3_tc_gate_up_bytes(shape.pairs, I));
-    float sum0 = 0.0f, sum1 = 0.0f;
-    for (uint32_t slot = 0; slot < shape.picks; slot++) {
-        const uint32_t pair = row * shape.picks + slot;
-        /* the job and column that hold this pair: every lane looks at jobs lane, lane + 64, ... */
-        uint32_t found = 0xFFFFFFFFu;
-        for (uint32_t base = 0; base < record.job_capacity; base += WAVE) {
-            const uint32_t index = base + lane;
-            uint32_t mine = 0xFFFFFFFFu;
-            if (index < record.job_capacity) {
-                const struct expert_job_record *job = jobs + index;
-                for (uint32_t column = 0; column < job->row_count; column++) {
-                    if (job->pair_index[column] == pair) {
-                        mine = index * LINEAR_MAXIMUM_ROWS + column;
+    /* the job and column that hold each of the row's pairs: every lane looks once at the jobs lane, lane + 64, ...
+     * (the eight pair indexes of a job as two 16-byte loads); a pair is held at most once, so the lane that found a
+     * slot's is read off a ballot */
+    uint32_t found[ROUTER_MOST_PICKS];
+#pragma unroll
+    for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
+        found[slot] = 0xFFFFFFFFu;
+    }
+    static_assert(LINEAR_MAXIMUM_ROWS == 8u, "a job's pair indexes are two loads of four");
+    for (uint32_t base = 0; base < record.job_capacity; base += WAVE) {
+        const uint32_t index = base + lane;
+        uint32_t mine[ROUTER_MOST_PICKS];
+#pragma unroll
+        for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
+            mine[slot] = 0xFFFFFFFFu;
+        }
+        if (index < record.job_capacity) {
+            const struct expert_job_record *job = jobs + index;
+            const uint32_t count = job->row_count;
+            const uint4_t low = *(const uint4_t *)&job->pair_index[0], high = *(const uint4_t *)&job->pair_index[4];
+            const uint32_t held[LINEAR_MAXIMUM_ROWS] = {low.x, low.y, low.z, low.w, high.x, high.y, high.z, high.w};
+#pragma unroll
+            for (uint32_t column = 0; column < LINEAR_MAXIMUM_ROWS; column++) {
+                if (column < count && held[column] / shape.picks == row) {
+                    const uint32_t slot = held[column] % shape.picks;
+#pragma unroll
+                    for (uint32_t target = 0; target < ROUTER_MOST_PICKS; target++) {
+                        mine[target] = target == slot ? index * LINEAR_MAXIMUM_ROWS + column : mine[target];
                     }
                 }
             }
-#pragma unroll
-            for (uint32_t distance = WAVE / 2u; distance != 0u; distance >>= 1u) {
-                const uint32_t other = __shfl_xor(mine, (int)distance, WAVE);
-                mine = other < mine ? other : mine;
-            }
-            found = mine < found ? mine : found;
         }
-        if (found == 0xFFFFFFFFu) {
+#pragma unroll
+        for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
+            const uint64_t holders = __builtin_amdgcn_ballot_w64(mine[slot] != 0xFFFFFFFFu);
+            if (holders != 0u) { /* the same in every lane */
+                found[slot] = (uint32_t)__builtin_amdgcn_readlane((int)mine[slot], (int)__builtin_ctzll(holders));
+            }
+        }
+    }
+    /* every slot's loads are asked for before the first is used; the sums then run in slot order */
+    float partial0[ROUTER_MOST_PICKS][EXL3_TC_DOWN_SLICES], partial1[ROUTER_MOST_PICKS][EXL3_TC_DOWN_SLICES];
+    float weight[ROUTER_MOST_PICKS], scale0[ROUTER_MOST_PICKS], scale1[ROUTER_MOST_PICKS];
+#pragma unroll
+    for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
+        if (slot < shape.picks && found[slot] != 0xFFFFFFFFu) {
+            const uint32_t pair = row * shape.picks + slot;
+            const struct expert_job_record *job = jobs + found[slot] / LINEAR_MAXIMUM_ROWS;
+            weight[slot] = job->route_weight[found[slot] % LINEAR_MAXIMUM_ROWS];
+            const uint16_t *svh = (const uint16_t *)(arena + job->down_offset + exl3_code_bytes(I, H, tc_bits_x2(record, arena, job->expert, 2u))) + I;
+            scale0[slot] = half_bits_to_float(svh[channel]);
+            scale1[slot] = half_bits_to_float(svh[channel + WAVE]);
+#pragma unroll
+            for (uint32_t slice = 0; slice < EXL3_TC_DOWN_SLICES; slice++) {
+                const float *down = partials + ((uint64_t)slice * shape.pairs + pair) * H;
+                partial0[slot][slice] = down[channel];
+                partial1[slot][slice] = down[channel + WAVE];
+            }
+        }
+    }
+    float sum0 = 0.0f, sum1 = 0.0f;
+#pragma unroll
+    for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
+        if (slot >= shape.picks || found[slot] == 0xFFFFFFFFu) {
             continue; /* a pair no job holds (a row beyond the live ones) adds nothing */
         }
-        const struct expert_job_record *job = jobs + found / LINEAR_MAXIMUM_ROWS;
-        const float weight = job->route_weight[found % LINEAR_MAXIMUM_ROWS];
-        const uint16_t *svh = (const uint16_t *)(arena + job->down_offset + exl3_code_bytes(I, H, tc_bits_x2(record, arena, job->expert, 2u))) + I;
         float v0 = 0.0f, v1 = 0.0f;
+#pragma unroll
         for (uint32_t slice = 0; slice < EXL3_TC_DOWN_SLICES; slice++) {
-            const float *down = partials + ((uint64_t)slice * shape.pairs + pair) * H;
-            v0 = __fadd_rn(v0, down[channel]);
-            v1 = __fadd_rn(v1, down[channel + WAVE]);
+            v0 = __fadd_rn(v0, partial0[slot][slice]);
+            v1 = __fadd_rn(v1, partial1[slot][slice]);
         }
         wave_hadamard128(v0, v1, lane);
-        const float y0 = __fmul_rn(__fmul_rn(__fmul_rn(v0, EXL3_NORMALIZATION), half_bits_to_float(svh[channel])), weight);
-        const float y1 = __fmul_rn(__fmul_rn(__fmul_rn(v1, EXL3_NORMALIZATION), half_bits_to_float(svh[channel + WAVE])), weight);
+        const float y0 = __fmul_rn(__fmul_rn(__fmul_rn(v0, EXL3_NORMALIZATION), scale0[slot]), weight[slot]);
+        const float y1 = __fmul_rn(__fmul_rn(__fmul_rn(v1, EXL3_NORMALIZATION), scale1[slot]), weight[slot]);
         sum0 = __fadd_rn(sum0, y0);
         sum1 = __fadd_rn(sum1, y1);
     }
