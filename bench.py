@@ -62,6 +62,17 @@ def cpu_oracle_step(orc_module, layer, x, router, matrices, widths, threads):
     return time.perf_counter() - start, out, experts
 
 
+def queue_steps(card, step, count, graph):
+    """`count` steps queued without waiting: launch by launch, or (graph) as replays of the step captured once with
+    the backend's graph_capture, as the reference's model runs its steps."""
+    if graph is None:
+        for _ in range(count):
+            card.run(step, wait=False)
+    else:
+        for _ in range(count):
+            card.run_graph(graph, wait=False)
+
+
 def calibrate(amd):
     """A copy of 1 GiB inside the arena (1 GiB read, 1 GiB written), five launches."""
     import ctypes as C
@@ -120,10 +131,10 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     step = amd.launches_of(len(parts))
     for i, launch in enumerate(parts):
         step[i] = launch
-    for _ in range(arguments.warmup):
-        card.run(step, wait=False)
+    graph = card.capture(step) if arguments.graph else None
+    queue_steps(card, step, arguments.warmup, graph)
     card.wait()
-    device_us = card.measure(lambda: [card.run(step, wait=False) for _ in range(arguments.steps)])
+    device_us = card.measure(lambda: queue_steps(card, step, arguments.steps, graph))
     seconds = device_us * 1e-6
     per_launch = np.zeros(len(names))
     for _ in range(arguments.steps):
@@ -240,10 +251,10 @@ def exl3_prefill(amd, workloads, arguments):
         step[i] = launch
     names = ["router_projection", "router_wide_select", "exl3_tcp_count", "exl3_tcp_place", "exl3_tcp_operands", "exl3_tcp_gemm(gate/up)",
              "exl3_tcp_activate", "exl3_tcp_gemm(down)", "exl3_tcp_combine"]
-    for _ in range(arguments.warmup):
-        card.run(step, wait=False)
+    graph = card.capture(step) if arguments.graph else None
+    queue_steps(card, step, arguments.warmup, graph)
     card.wait()
-    device_us = card.measure(lambda: [card.run(step, wait=False) for _ in range(arguments.steps)])
+    device_us = card.measure(lambda: queue_steps(card, step, arguments.steps, graph))
     seconds = device_us * 1e-6
     per_launch = np.zeros(len(names))
     for _ in range(arguments.steps):
@@ -312,6 +323,7 @@ def main():
     parser.add_argument("--gate-up-slices", type=int, default=4)
     parser.add_argument("--down-slices", type=int, default=2)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--graph", action="store_true", help="time replays of the step captured as one graph (graph_capture / graph_run)")
     parser.add_argument("--calibrate", action="store_true",
                         help="run only a 1 GiB arena copy, five times: the yardstick of the traffic counters")
     arguments = parser.parse_args()
@@ -350,12 +362,12 @@ def main():
     names = ["router_projection", "router_select_entry", "exl3_tc_operands", "exl3_tc_products(gate/up)",
              "exl3_tc_activate", "exl3_tc_products(down)", "exl3_tc_combine"]
 
-    for _ in range(arguments.warmup):
-        card.run(step, wait=False)
+    graph = card.capture(step) if arguments.graph else None
+    queue_steps(card, step, arguments.warmup, graph)
     card.wait()
     # the timed region: exactly K steps between two waits, on the card's own clock and on the host's
     host_start = time.perf_counter()
-    device_us = card.measure(lambda: [card.run(step, wait=False) for _ in range(arguments.steps)])
+    device_us = card.measure(lambda: queue_steps(card, step, arguments.steps, graph))
     host_seconds = time.perf_counter() - host_start
     seconds = max(device_us * 1e-6, 1e-12)
     ms_per_step = 1000.0 * seconds / arguments.steps
