@@ -32,8 +32,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("exl3_decode", 8): 375.2e6 + 8.4e6,      # profiles/exl3_tc_products_decode8.md
     ("fp4_decode", 32): 1434.7e6 + 1.0e6,     # profiles/expert_gate_up_fp4_fp8_decode32.md
     ("fp8_decode", 32): 2768.4e6 + 1.0e6,
-    ("fp4_prefill", 8192): 5444e6 + 444e6,    # profiles/wide_expert_fp4_fp8_prefill.md
-    ("fp8_prefill", 2048): 5801e6 + 111e6,
+    ("fp4_prefill", 8192): 5044.9e6 + 443.2e6,  # profiles/wide_expert_fp4_fp8_prefill.md
+    ("fp8_prefill", 2048): 5642.4e6 + 117.0e6,
 }
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
 CONFIG = 1
