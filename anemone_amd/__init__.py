@@ -15,6 +15,7 @@ STATUS_DEVICE_ERROR, STATUS_TIMED_OUT, STATUS_UNSUPPORTED, STATUS_BUSY = 5, 6, 7
 WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED = 2, 3, 5
 ARITHMETIC_CLASS_GFX950 = 950
 BACKEND_NO_KERNEL = 0xFFFFFFFF
+LAUNCH_CHAIN, LAUNCH_SIDE, LAUNCH_RESUME, LAUNCH_JOIN, LAUNCH_SIDE_MORE = 0, 1, 2, 3, 4  # kernel_launch.branch
 ROUTER_SORT_ROWS = 384
 EXL3_TCP_CHUNK_PAIRS = 160
 EXL3_EXPERT_LAUNCHES, EXL3_TC_LAUNCHES = 5, 5

@@ -69,8 +69,10 @@ struct device_card {
     /* copies */
     uint64_t next_ticket, finished_ticket;
     copy_slot slots[BACKEND_MAXIMUM_UPLOADS_IN_FLIGHT];
-    /* graphs */
+    /* graphs; the streams and events that carry a graph's side runs while it is captured */
     std::vector<hipGraphExec_t> graphs;
+    hipStream_t side_streams[LAUNCH_MOST_SIDE_RUNS];
+    hipEvent_t fork_event, side_events[LAUNCH_MOST_SIDE_RUNS];
     /* one timing interval */
     hipEvent_t measure_start, measure_stop;
     int measure_state; /* 0 idle, 1 begun, 2 ended */
@@ -186,9 +188,8 @@ result_status launches_check(device_card *card, const kernel_launch *launches, u
             threads *= launch.block[d];
         }
         if (launch.argument_byte_count != entry.record_bytes || launch.argument_byte_count > LAUNCH_ARGUMENT_BYTES ||
-            threads > (uint64_t)card->max_threads || launch.dynamic_shared_byte_count > (uint32_t)card->max_shared ||
-            launch.branch != LAUNCH_CHAIN) {
-            log_error(entry.function, "a record size, block size, shared memory size or branch the card refuses");
+            threads > (uint64_t)card->max_threads || launch.dynamic_shared_byte_count > (uint32_t)card->max_shared) {
+            log_error(entry.function, "a record size, block size or shared memory size the card refuses");
             return STATUS_INVALID_ARGUMENT;
         }
         for (uint32_t byte = launch.argument_byte_count; byte < LAUNCH_ARGUMENT_BYTES; byte++) {
@@ -198,17 +199,115 @@ result_status launches_check(device_card *card, const kernel_launch *launches, u
             }
         }
     }
+    /* the branches: side runs open behind a fork (a launch on the main line, or the root), at most
+     * LAUNCH_MOST_SIDE_RUNS of them; the main line goes on with RESUME or JOIN, never with a CHAIN behind a side launch */
+    uint32_t open_runs = 0;
+    bool last_is_side = false;
+    for (uint32_t index = 0; index < count; index++) {
+        const uint32_t branch = launches[index].branch;
+        bool fine = true;
+        switch (branch) {
+        case LAUNCH_CHAIN:
+            fine = !last_is_side;
+            last_is_side = false;
+            break;
+        case LAUNCH_SIDE:
+            if (!last_is_side) {
+                fine = open_runs == 0; /* one fork at a time: further runs behind it are SIDE_MORE */
+                open_runs++;
+            }
+            last_is_side = true;
+            break;
+        case LAUNCH_SIDE_MORE:
+            fine = open_runs != 0 && open_runs < LAUNCH_MOST_SIDE_RUNS && last_is_side;
+            open_runs++;
+            last_is_side = true;
+            break;
+        case LAUNCH_RESUME:
+            fine = open_runs != 0 && last_is_side;
+            last_is_side = false;
+            break;
+        case LAUNCH_JOIN:
+            fine = open_runs != 0;
+            open_runs = 0;
+            last_is_side = false;
+            break;
+        default:
+            fine = false;
+        }
+        if (!fine) {
+            log_error("launch", "a branch that does not fit the launches before it");
+            return STATUS_INVALID_ARGUMENT;
+        }
+    }
     return STATUS_OK;
 }
 
-hipError_t launch_one(device_card *card, const kernel_launch &launch)
+hipError_t launch_on(device_card *card, const kernel_launch &launch, hipStream_t stream)
 {
     const kernel_entry &entry = kernel_table()[card->prepared[launch.kernel]];
     /* the record travels by value: the runtime copies record_bytes from the launch's own bytes */
     void *arguments[2] = {(void *)launch.argument, (void *)&card->arena};
     return hipLaunchKernel(entry.host_function, dim3(launch.grid[0], launch.grid[1], launch.grid[2]),
                            dim3(launch.block[0], launch.block[1], launch.block[2]), arguments,
-                           launch.dynamic_shared_byte_count, card->stream);
+                           launch.dynamic_shared_byte_count, stream);
+}
+
+hipError_t launch_one(device_card *card, const kernel_launch &launch)
+{
+    return launch_on(card, launch, card->stream);
+}
+
+/* A checked list under capture on the card's stream: side runs go to side streams that wait for the fork's event, a
+ * JOIN (and the list's end) makes the main line wait for theirs. Every stream keeps the default priority. */
+hipError_t capture_branches(device_card *card, const kernel_launch *launches, uint32_t count)
+{
+    hipError_t status = hipSuccess;
+    uint32_t open_runs = 0;
+    bool last_is_side = false;
+    auto join = [&]() {
+        for (uint32_t run = 0; run < open_runs && status == hipSuccess; run++) {
+            status = hipEventRecord(card->side_events[run], card->side_streams[run]);
+            if (status == hipSuccess) {
+                status = hipStreamWaitEvent(card->stream, card->side_events[run], 0);
+            }
+        }
+        open_runs = 0;
+    };
+    for (uint32_t index = 0; index < count && status == hipSuccess; index++) {
+        const kernel_launch &launch = launches[index];
+        switch (launch.branch) {
+        case LAUNCH_SIDE:
+        case LAUNCH_SIDE_MORE:
+            if (!last_is_side || launch.branch == LAUNCH_SIDE_MORE) { /* a new run behind the fork */
+                if (open_runs == 0) {
+                    status = hipEventRecord(card->fork_event, card->stream);
+                }
+                if (status == hipSuccess) {
+                    status = hipStreamWaitEvent(card->side_streams[open_runs], card->fork_event, 0);
+                }
+                open_runs++;
+            }
+            if (status == hipSuccess) {
+                status = launch_on(card, launch, card->side_streams[open_runs - 1u]);
+            }
+            last_is_side = true;
+            break;
+        case LAUNCH_JOIN:
+            join();
+            /* fall through: the launch itself stands on the main line */
+        default: /* CHAIN, RESUME: the main line, which stands at the fork while side runs are open */
+            if (status == hipSuccess) {
+                status = launch_on(card, launch, card->stream);
+            }
+            last_is_side = false;
+            break;
+        }
+    }
+    if (status == hipSuccess) {
+        join(); /* a capture ends with every stream back on the main line */
+    }
+    return status;
 }
 
 result_status wait_for(device_card *card, hipEvent_t event, uint64_t limit_ns)
@@ -346,6 +445,11 @@ result_status backend_hip_card_open(uint32_t card_index, uint64_t arena_byte_cou
         ok = ok && hipEventCreateWithFlags(&slot.event, hipEventDisableTiming) == hipSuccess;
     }
     ok = ok && hipEventCreate(&card->measure_start) == hipSuccess && hipEventCreate(&card->measure_stop) == hipSuccess;
+    ok = ok && hipEventCreateWithFlags(&card->fork_event, hipEventDisableTiming) == hipSuccess;
+    for (uint32_t run = 0; run < LAUNCH_MOST_SIDE_RUNS; run++) {
+        ok = ok && hipStreamCreateWithFlags(&card->side_streams[run], hipStreamNonBlocking) == hipSuccess &&
+             hipEventCreateWithFlags(&card->side_events[run], hipEventDisableTiming) == hipSuccess;
+    }
     if (!ok) {
         (void)hipFree(card->arena);
         delete card;
@@ -377,6 +481,11 @@ void backend_hip_card_close(struct device_card *card, uint64_t wait_limit_nanose
         }
         (void)hipEventDestroy(card->measure_start);
         (void)hipEventDestroy(card->measure_stop);
+        for (uint32_t run = 0; run < LAUNCH_MOST_SIDE_RUNS; run++) {
+            (void)hipStreamDestroy(card->side_streams[run]);
+            (void)hipEventDestroy(card->side_events[run]);
+        }
+        (void)hipEventDestroy(card->fork_event);
         (void)hipStreamDestroy(card->stream);
         (void)hipFree(card->arena);
     }
@@ -640,10 +749,7 @@ result_status backend_hip_graph_capture(struct device_card *card, const struct k
         card_fail(card, "hipStreamBeginCapture", hipStreamBeginCapture(card->stream, hipStreamCaptureModeThreadLocal))) {
         return STATUS_DEVICE_ERROR;
     }
-    hipError_t launched = hipSuccess;
-    for (uint32_t index = 0; index < launch_count && launched == hipSuccess; index++) {
-        launched = launch_one(card, launches[index]); /* kernels only: no memset node enters a graph */
-    }
+    const hipError_t launched = capture_branches(card, launches, launch_count); /* kernels only: no memset node enters a graph */
     hipGraph_t graph = nullptr;
     const hipError_t ended = hipStreamEndCapture(card->stream, &graph);
     if (card_fail(card, "a launch under capture", launched) || card_fail(card, "hipStreamEndCapture", ended)) {

@@ -131,7 +131,16 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     step = amd.launches_of(len(parts))
     for i, launch in enumerate(parts):
         step[i] = launch
-    graph = card.capture(step) if arguments.graph else None
+    graph = None
+    if arguments.graph:
+        # the rows' quantizer reads the rows alone: a side run beside the router's launches, joined by the gate/up launch
+        at = names.index("activation_quantize")
+        order = [parts[at]] + parts[:at] + parts[at + 1:]
+        branched = amd.launches_of(len(order))
+        for i, launch in enumerate(order):
+            branched[i] = launch
+        branched[0].branch, branched[1].branch, branched[at + 1].branch = amd.LAUNCH_SIDE, amd.LAUNCH_RESUME, amd.LAUNCH_JOIN
+        graph = card.capture(branched)
     queue_steps(card, step, arguments.warmup, graph)
     card.wait()
     device_us = card.measure(lambda: queue_steps(card, step, arguments.steps, graph))

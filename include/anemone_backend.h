@@ -80,7 +80,17 @@ struct card_description_record { /* backend_seam.h:165-179 */
 
 struct device_card;
 
-#define LAUNCH_CHAIN 0u /* the only branch kind this backend runs: each launch behind the one before it */
+/* backend_seam.h:184-195 of the reference: where a launch stands in a captured graph. CHAIN: behind the launch before
+ * it. A run of SIDE launches stands behind the launch before the run (the fork), each behind the one before it;
+ * SIDE_MORE is another side run, of one launch, behind the same fork; RESUME stands behind the fork, not the side runs;
+ * JOIN behind the launch before it and every side run's last. A list's first launch may open a side run: its fork is
+ * then the graph's root. launch_run runs a list in its serial order whatever the branches say. */
+#define LAUNCH_CHAIN 0u
+#define LAUNCH_SIDE 1u
+#define LAUNCH_RESUME 2u
+#define LAUNCH_JOIN 3u
+#define LAUNCH_SIDE_MORE 4u
+#define LAUNCH_MOST_SIDE_RUNS 4u
 struct kernel_launch { /* backend_seam.h:196-204 */
     uint32_t kernel;
     uint32_t grid[LAUNCH_DIMENSIONS];

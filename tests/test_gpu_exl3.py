@@ -239,3 +239,4 @@ def test_single_linear_config0_shape(amd, card):
     rms = np.sqrt(np.mean(want ** 2))
     say("  max err / rms", float(np.max(np.abs(got - want)) / rms))
     assert np.max(np.abs(got - want)) <= 2e-3 * rms  # fp16 operand rounding (2^-11 a value) dominates
+

@@ -227,3 +227,61 @@ def test_producer_equals_the_two_launches_byte_for_byte(amd, card, rows, live, p
     if live < rows:  # the pairs of the rows beyond the live ones were quantized from the stale values
         want = oracle_quantize(stale.reshape(rows * picks, inner)[live * picks:])[2]
         assert np.array_equal(fused[1].reshape(rows * picks, inner)[live * picks:], want)
+
+
+def branched_step(amd, layer, wide, branches):
+    """A decode step of the FP4 layer through the wide select's one-block form: the rows' quantizer reads the rows alone
+    and stands first; with `branches` it is a side run that opens the graph, the router's launches the main line behind
+    the root, the gate/up launch the join. (Every other launch of the step reads what the one before it wrote.)"""
+    routing = wide.launches(small=True)
+    experts = layer.expert_launches(wide)
+    order = [layer.quantize_launch()[0], layer.projection_launch()[0], routing[0], routing[1]] + [experts[i] for i in range(4)]
+    step = amd.launches_of(len(order))
+    for i, launch in enumerate(order):
+        step[i] = launch
+    if branches:
+        step[0].branch, step[1].branch, step[4].branch = amd.LAUNCH_SIDE, amd.LAUNCH_RESUME, amd.LAUNCH_JOIN
+    return step
+
+
+def test_graph_with_a_side_run_replays_the_serial_step(amd, card):
+    """A step captured with graph_capture, the rows' quantizer on a side run beside the router (LAUNCH_SIDE, RESUME,
+    JOIN: include/anemone/backend_seam.h:184-195 of the reference), replayed three times with other work and waits of
+    the card between the replays: every replay writes the bits of the serial launch_run; lists whose branches do not
+    fit are refused before anything is captured."""
+    say("graph with a side run")
+    hidden, inner, experts_n, picks, rows = 512, 256, 64, 4, 32
+    layer, _, _ = build(amd, card, hidden, inner, experts_n, picks, rows, 8, gate_up_slices=2, down_slices=1)
+    x = to_bf16(normals(29, rows * hidden)).reshape(rows, hidden)
+    other = to_bf16(normals(30, rows * hidden)).reshape(rows, hidden)
+    wide = layer.wide_router()
+    layer.set_rows(x, rows)
+    card.run(branched_step(amd, layer, wide, False))
+    serial = layer.read("row_output", np.float32).copy()
+    assert np.any(serial != 0.0)
+    graph = card.capture(branched_step(amd, layer, wide, True))
+    for replay in range(3):
+        layer.set_rows(other, rows)  # other work between the replays: a step on other rows, run launch by launch
+        card.run(branched_step(amd, layer, wide, False))
+        assert np.any(layer.read("row_output", np.float32) != serial)
+        layer.set_rows(x, rows)
+        card.run_graph(graph)
+        assert np.array_equal(layer.read("row_output", np.float32).view(np.uint32), serial.view(np.uint32)), replay
+    # launch_run takes the same list in its serial order
+    layer.set_rows(other, rows)
+    card.run(branched_step(amd, layer, wide, False))
+    layer.set_rows(x, rows)
+    card.run(branched_step(amd, layer, wide, True))
+    assert np.array_equal(layer.read("row_output", np.float32).view(np.uint32), serial.view(np.uint32))
+    for spoil in ("join without a side run", "chain behind a side launch", "resume without a side run", "unknown branch"):
+        step = branched_step(amd, layer, wide, spoil == "chain behind a side launch")
+        if spoil == "join without a side run":
+            step[4].branch = amd.LAUNCH_JOIN
+        elif spoil == "chain behind a side launch":
+            step[1].branch = amd.LAUNCH_CHAIN
+        elif spoil == "resume without a side run":
+            step[1].branch = amd.LAUNCH_RESUME
+        else:
+            step[2].branch = 9
+        with pytest.raises(amd.AnemoneError):
+            card.capture(step)
