@@ -379,22 +379,34 @@ extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
                    arguments.reference_order, scale, pair_experts + wave * picks, pair_weights + wave * picks);
     }
     __syncthreads();
+    /* The job table: at most 64 pairs, one a lane of the first wavefront. A pair's column is the number of earlier
+     * pairs of its expert, its job the number of distinct experts below its own, a job's rows the pairs of its expert:
+     * counted over the other lanes' experts read lane by lane (no LDS round trip a step). */
+    static_assert(LINEAR_MAXIMUM_ROWS * ROUTER_MOST_PICKS <= WAVE, "a step's pairs fit one wavefront");
     const bool mine = pair < pair_count;
-    const uint32_t expert = mine ? pair_experts[pair] : 0u;
-    uint32_t column = 0;
-    for (uint32_t earlier = 0; mine && earlier < pair; earlier++) {
-        column += pair_experts[earlier] == expert ? 1u : 0u;
-    }
-    if (mine) {
-        pair_is_first[pair] = column == 0u ? 1u : 0u;
+    uint32_t used_jobs = 0, job = 0, rows = 0, column = 0;
+    const uint32_t expert = mine ? pair_experts[pair] : 0xFFFFFFFFu; /* no expert: equal to none that is picked */
+    if (wave == 0u) {
+#pragma unroll
+        for (uint32_t other = 0; other < WAVE; other++) {
+            const uint32_t theirs = (uint32_t)__builtin_amdgcn_readlane((int)expert, (int)other);
+            const bool same = theirs == expert;
+            rows += same ? 1u : 0u;
+            column += same && other < lane ? 1u : 0u;
+        }
+        const uint64_t firsts = __builtin_amdgcn_ballot_w64(mine && column == 0u); /* the first pair of every picked expert */
+        used_jobs = (uint32_t)__builtin_popcountll(firsts);
+#pragma unroll
+        for (uint32_t other = 0; other < WAVE; other++) {
+            const uint32_t theirs = (uint32_t)__builtin_amdgcn_readlane((int)expert, (int)other);
+            job += ((firsts >> other) & 1u) != 0u && theirs < expert ? 1u : 0u;
+        }
+        if (lane == 0u) {
+            pair_is_first[0] = used_jobs; /* for the wavefronts that clear the table's unused jobs */
+        }
     }
     __syncthreads();
-    uint32_t used_jobs = 0, job = 0, rows = 0;
-    for (uint32_t other = 0; other < pair_count; other++) {
-        used_jobs += pair_is_first[other];
-        job += pair_is_first[other] != 0u && pair_experts[other] < expert ? 1u : 0u;
-        rows += pair_experts[other] == expert ? 1u : 0u;
-    }
+    used_jobs = pair_is_first[0];
     struct expert_job_record *jobs = (struct expert_job_record *)(arena + arguments.jobs_offset);
     if (mine) {
         jobs[job].pair_index[column] = pair;
