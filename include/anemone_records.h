@@ -41,7 +41,7 @@
 #endif
 
 /* ---- shared geometry ---- */
-#define LINEAR_MAXIMUM_ROWS 8u          /* columns of one job */
+#define LINEAR_MAXIMUM_ROWS 8u          /* columns of one job; rows of one thin trunk launch, a group of a wide one */
 #define LINEAR_OUTPUTS_PER_TILE 16u
 #define LINEAR_VALUES_PER_BLOCK 32u     /* values that share one scale exponent */
 #define LINEAR_VALUES_PER_LOAD 64u
@@ -528,5 +528,91 @@ struct expert_down_arguments {
     uint32_t reserved_zero;
 };
 ANEMONE_RECORD_HAS(expert_down_arguments, 56);
+
+/* ---- the shared expert and the FFN site's join: the step behind the routed experts ----
+ * Records of the reference member for member (include/anemone/linear_records.h:307-356,
+ * include/anemone/expert_fused_records.h:100-131, include/anemone/hyper_connection_records.h:79-89). The reference
+ * fixes the streams' width at its model's 5,120; here a join's width is what its grid covers: grid[0] x block[0]
+ * threads of HYPER_VALUES_PER_THREAD values each. */
+#define KERNEL_FILE_TRUNK_LINEAR "kernel_trunk_linear"
+#define KERNEL_TRUNK_LINEAR_QUANTIZED_STEM "trunk_linear_quantized_"
+#define KERNEL_TRUNK_LINEAR_QUANTIZED_WIDE_STEM "trunk_linear_quantized_wide_"
+#define KERNEL_TRUNK_LINEAR_QUANTIZED_INTERLEAVED "trunk_linear_quantized_interleaved_1"
+#define KERNEL_TRUNK_HIDDEN "trunk_hidden_entry"
+#define KERNEL_EXPERT_SHARED_JOIN_STEM "expert_shared_join_"
+#define KERNEL_FILE_HYPER_CONNECTION "kernel_hyper_connection"
+#define KERNEL_HYPER_POST "hyper_post_entry"
+#define KERNEL_EXPERT_JOIN "expert_join"
+#define LINEAR_MERGED_MATRICES 2u /* the most matrices one trunk launch reads */
+#define TRUNK_STRIP_OUTPUTS 32u   /* outputs of a block of the thin and the wide trunk kernels: two tiles of one-byte weights */
+#define TRUNK_INTERLEAVED_ROWS 64u          /* rows of a block of the interleaved instance: one tile of vectors */
+#define TRUNK_INTERLEAVED_BLOCK_OUTPUTS 128u /* its outputs: four wavefronts' strips of two tiles */
+#define TRUNK_INTERLEAVED_WINDOW_BYTES 51712u
+#define MODEL_STREAMS 4u
+#define HYPER_VALUES_PER_THREAD 8u /* one 16-byte load of bfloat16 */
+#define HYPER_PIECE_THREADS 128u
+#define EXPERT_JOIN_NO_ROW_SUMS UINT64_MAX /* in place of row_sums_offset: the sums are not stored */
+
+struct trunk_linear_quantized_arguments {
+    uint64_t weights_offset[LINEAR_MERGED_MATRICES]; /* read: WEIGHT_FORMAT_E4M3_SCALED matrices of one input_size */
+    uint64_t output_offset[LINEAR_MERGED_MATRICES];  /* written: bf16 [row_count][output_size[m]] */
+    uint64_t codes_offset;                           /* read: the rows' codes, exponents, operands */
+    uint64_t exponents_offset;
+    uint64_t operands_offset;
+    uint32_t output_size[LINEAR_MERGED_MATRICES];    /* [1] is 0 where there is one matrix */
+    uint32_t input_size;
+    uint32_t row_count;
+};
+ANEMONE_RECORD_HAS(trunk_linear_quantized_arguments, 72);
+
+struct trunk_hidden_arguments { /* the hidden step alone, route weight 1; grid[1] vectors */
+    uint64_t gate_offset;   /* read: bf16 [V][width] */
+    uint64_t up_offset;
+    uint64_t hidden_offset; /* written: bf16 [V][width] */
+    uint32_t width;
+    float activation_limit;
+};
+ANEMONE_RECORD_HAS(trunk_hidden_arguments, 32);
+
+struct hyper_post_arguments {
+    uint64_t streams_offset; /* read and written: bf16 [row][4][width] */
+    uint64_t post_offset;    /* read: float32 [row][4] */
+    uint64_t comb_offset;    /* read: float32 [row][4 sources][4 targets] */
+    uint64_t output_offset;  /* read: bf16 [row][width], the sublayer's or the shared expert's */
+    uint64_t sums_offset;    /* read with the combine alone: float32 [row][width] */
+    uint32_t is_combined;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(hyper_post_arguments, 48);
+
+struct expert_join_arguments {
+    uint64_t pair_output_offset;   /* read: bf16 [row * pairs_per_row + slot][width] */
+    uint64_t shared_output_offset; /* read: bf16 [row][width] */
+    uint64_t streams_offset;       /* read and written */
+    uint64_t post_offset;
+    uint64_t comb_offset;
+    uint64_t row_sums_offset;      /* written: float32 [row][width], or EXPERT_JOIN_NO_ROW_SUMS */
+    uint32_t pairs_per_row;
+    uint32_t reserved_zero;
+};
+ANEMONE_RECORD_HAS(expert_join_arguments, 56);
+
+struct expert_shared_join_arguments {
+    uint64_t weights_offset;     /* the shared expert's down: E4M3_SCALED, the streams' width by input_size */
+    uint64_t codes_offset;       /* its quantized input, as trunk_linear_quantized_arguments */
+    uint64_t exponents_offset;
+    uint64_t operands_offset;
+    uint64_t output_offset;      /* written: the shared expert's output, bf16 [row][width] */
+    uint64_t pair_output_offset; /* the join's, as expert_join_arguments */
+    uint64_t streams_offset;
+    uint64_t post_offset;
+    uint64_t comb_offset;
+    uint64_t row_sums_offset;
+    uint32_t input_size;
+    uint32_t row_count;
+    uint32_t pairs_per_row;
+    uint32_t reserved_zero;      /* extension: the streams' width (the down matrix's outputs); 0 stands for 5,120 */
+};
+ANEMONE_RECORD_HAS(expert_shared_join_arguments, 96);
 
 #endif

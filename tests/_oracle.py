@@ -77,6 +77,9 @@ def _load_oracle():
         "orc_fp8_block128_products": (None, [u32, u32, u8p, f32p, u8p, f32p, u32, f64p]),
         "orc_linear_moe_layer": (None, [i32, u16p, u32, u32, u32, u32, u32p, f32p, u32, C.POINTER(vp), f32, f32p,
                                         u16p, u16p, u32]),
+        "orc_hyper_post": (None, [u16p, f32p, f32p, u16p, f32p, u32, u16p]),
+        "orc_expert_join": (None, [u16p, u16p, u16p, f32p, f32p, f32p, u32, u32, u32]),
+        "orc_trunk_hidden": (None, [u16p, u16p, f32, u32, u16p]),
     }
     for name, (restype, argtypes) in sig.items():
         fn = getattr(lib, name)
@@ -134,6 +137,9 @@ def _load_ref():
     lib.test_linear_row_sum.argtypes = [u16p, u32, u32, u32]
     lib.test_linear_output_is_within_tolerance.restype = C.c_bool
     lib.test_linear_output_is_within_tolerance.argtypes = [C.c_uint16, C.c_void_p, u32, u32]
+    if hasattr(lib, "test_hyper_post"):
+        lib.test_hyper_post.restype = None
+        lib.test_hyper_post.argtypes = [u16p, f32p, f32p, u16p, f32p, u16p]
     return lib
 
 
