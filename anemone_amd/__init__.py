@@ -140,7 +140,43 @@ class LinearKernels(C.Structure):
 
 
 class ExpertFusedKernels(C.Structure):
-    _fields_ = [("gate_up_quantize", u32 * 5), ("shared_join", u32 * 5), ("join", u32), ("gate_up_quantize_e4m3", u32 * 5)]
+    _fields_ = [("gate_up_quantize", u32 * 5), ("shared_join", u32 * 5), ("join", u32), ("gate_up_quantize_e4m3", u32 * 5), ("post", u32)]
+
+
+class LinearMatrix(C.Structure):
+    _fields_ = [("stored", Range), ("shape", Shape), ("weight_format", C.c_int), ("slice_count", u32), ("wide_form", C.c_int),
+                ("reserved_zero", u32)]
+
+
+class TrunkQuantizedDescription(C.Structure):
+    _fields_ = [("matrices", LinearMatrix * 2), ("codes", Range), ("exponents", Range), ("operands", Range), ("outputs", Range * 2),
+                ("matrix_count", u32), ("row_count", u32)]
+
+
+class SharedExpertDescription(C.Structure):
+    _fields_ = [("gate", LinearMatrix), ("up", LinearMatrix), ("down", LinearMatrix)] + \
+               [(name, Range) for name in ("codes", "exponents", "operands", "gate_output", "up_output", "hidden", "hidden_codes",
+                                           "hidden_exponents", "hidden_operands", "output")] + \
+               [("row_count", u32), ("activation_limit", f32)]
+
+
+class ExpertJoinDescription(C.Structure):
+    _fields_ = [(name, Range) for name in ("pair_output", "shared_output", "streams", "post", "comb", "row_sums")] + \
+               [("pairs_per_row", u32), ("row_count", u32), ("width", u32)]
+
+
+class ExpertSharedJoinDescription(C.Structure):
+    _fields_ = [("down", LinearMatrix), ("codes", Range), ("exponents", Range), ("operands", Range), ("join", ExpertJoinDescription)]
+
+
+class TrunkLinearQuantizedArguments(C.Structure):
+    _fields_ = [("weights_offset", u64 * 2), ("output_offset", u64 * 2), ("codes_offset", u64), ("exponents_offset", u64),
+                ("operands_offset", u64), ("output_size", u32 * 2), ("input_size", u32), ("row_count", u32)]
+
+
+class ExpertJoinArguments(C.Structure):
+    _fields_ = [("pair_output_offset", u64), ("shared_output_offset", u64), ("streams_offset", u64), ("post_offset", u64),
+                ("comb_offset", u64), ("row_sums_offset", u64), ("pairs_per_row", u32), ("reserved_zero", u32)]
 
 
 class LinearWideKernels(C.Structure):
@@ -210,6 +246,12 @@ def library():
             "expert_fused_kernels_prepare": [vp, vp, u32, C.POINTER(ExpertFusedKernels)],
             "expert_producer_prepare": [C.POINTER(RoutedExpertsDescription), Range, u64, C.POINTER(LinearKernels),
                                         C.POINTER(ExpertFusedKernels), launch_p],
+            "linear_trunk_quantized_prepare": [C.POINTER(TrunkQuantizedDescription), u64, C.POINTER(LinearKernels), launch_p],
+            "linear_shared_expert_prepare": [C.POINTER(SharedExpertDescription), u64, C.POINTER(LinearKernels), launch_p],
+            "expert_join_prepare": [C.POINTER(ExpertJoinDescription), u64, C.POINTER(ExpertFusedKernels), launch_p],
+            "expert_post_prepare": [C.POINTER(ExpertJoinDescription), u64, u32, launch_p],
+            "expert_shared_join_prepare": [C.POINTER(ExpertSharedJoinDescription), u64, C.POINTER(LinearKernels),
+                                           C.POINTER(ExpertFusedKernels), launch_p],
         }
         for name, argtypes in signatures.items():
             function = getattr(lib, name)
@@ -741,3 +783,94 @@ class Fp4Layer:
 
     def jobs(self):
         return self.card.download(self.jobs_offset, self.pairs * 96).view(JOB_DTYPE)
+
+
+LINEAR_WIDE_GROUP_BLOCKS, LINEAR_WIDE_TILE_BLOCKS, LINEAR_INTERLEAVED_CHUNK_BLOCKS, LINEAR_INTERLEAVED_TILE_BLOCKS = 0, 1, 2, 3
+LINEAR_MAXIMUM_ROWS = 8
+MODEL_STREAMS = 4
+
+
+class SharedExpert:
+    """The step behind a layer's routed experts: the shared expert (three WEIGHT_FORMAT_E4M3_SCALED matrices applied to
+    every row: gate with up, the hidden step, the quantizer, down) and the FFN site's join (a row's routed sum, the
+    shared expert's output added to it, the post of the four residual streams). Reads the rows' codes and the pair
+    outputs of `layer` (an Fp4Layer); holds its own scratch, the streams, post and comb in the layer's arena."""
+
+    def __init__(self, layer, matrices, gate_up_slices=1, down_slices=1, wide_form=LINEAR_INTERLEAVED_CHUNK_BLOCKS, inner=None):
+        self.layer, self.card = layer, layer.card
+        card, rows, hidden = layer.card, layer.rows, layer.H
+        self.inner = inner = layer.I if inner is None else inner
+        self.gate_up_slices, self.down_slices, self.wide_form = gate_up_slices, down_slices, wide_form
+        self.matrix_ranges = [Range(card.place(matrix, 256), matrix.nbytes) for matrix in matrices]
+        names = {"gate_output": rows * inner * 2, "up_output": rows * inner * 2, "hidden": rows * inner * 2,
+                 "hidden_codes": rows * inner, "hidden_exponents": rows * inner // 32, "hidden_operands": rows * inner * 2,
+                 "output": rows * hidden * 2, "streams": rows * MODEL_STREAMS * hidden * 2, "post": rows * MODEL_STREAMS * 4,
+                 "comb": rows * MODEL_STREAMS * MODEL_STREAMS * 4, "row_sums": rows * hidden * 4}
+        self.ranges = {name: Range(card.reserve(size), size) for name, size in names.items()}
+        self.fused_kernels = ExpertFusedKernels()
+        check(card.lib.expert_fused_kernels_prepare(backend_table(), card.handle, ARITHMETIC_CLASS_GFX950, C.byref(self.fused_kernels)),
+              "expert_fused_kernels_prepare")
+
+    def matrix(self, index, slices):
+        outputs, inputs = (self.layer.H, self.inner) if index == 2 else (self.inner, self.layer.H)
+        return LinearMatrix(self.matrix_ranges[index], Shape(outputs, inputs, 8, 0), WEIGHT_FORMAT_E4M3_SCALED, slices, self.wide_form, 0)
+
+    def set_site(self, streams_bf16, post, comb):
+        self.card.upload(self.ranges["streams"].byte_offset, streams_bf16)
+        self.card.upload(self.ranges["post"].byte_offset, np.ascontiguousarray(post, dtype=np.float32))
+        self.card.upload(self.ranges["comb"].byte_offset, np.ascontiguousarray(comb, dtype=np.float32))
+
+    def description(self, rows=None):
+        d = SharedExpertDescription()
+        d.gate, d.up, d.down = self.matrix(0, self.gate_up_slices), self.matrix(1, self.gate_up_slices), self.matrix(2, self.down_slices)
+        d.codes, d.exponents, d.operands = (self.layer.ranges[name] for name in ("codes", "exponents", "operands"))
+        for name in ("gate_output", "up_output", "hidden", "hidden_codes", "hidden_exponents", "hidden_operands", "output"):
+            setattr(d, name, self.ranges[name])
+        d.row_count, d.activation_limit = self.layer.rows if rows is None else rows, self.layer.limit
+        return d
+
+    def launches(self, rows=None):
+        """The shared expert's four launches: gate with up, the hidden step, the quantizer, down."""
+        d = self.description(rows)
+        launches = launches_of(4)
+        check(self.card.lib.linear_shared_expert_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.layer.kernels), launches),
+              "linear_shared_expert_prepare")
+        return launches
+
+    def join_description(self, rows=None, row_sums=True):
+        d = ExpertJoinDescription()
+        d.pair_output, d.shared_output = self.layer.ranges["pair_output"], self.ranges["output"]
+        d.streams, d.post, d.comb = self.ranges["streams"], self.ranges["post"], self.ranges["comb"]
+        d.row_sums = self.ranges["row_sums"] if row_sums else Range(0, 0)
+        d.pairs_per_row, d.row_count, d.width = self.layer.P, self.layer.rows if rows is None else rows, self.layer.H
+        return d
+
+    def join_launch(self, rows=None, row_sums=True):
+        d = self.join_description(rows, row_sums)
+        launch = launches_of(1)
+        check(self.card.lib.expert_join_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.fused_kernels), launch), "expert_join_prepare")
+        return launch
+
+    def post_launch(self, rows=None):
+        """hyper_post_entry with the combine, reading the layer's row outputs (what expert_row_sum_entry, the last of the
+        routed experts' launches, wrote): the second of the two launches a join stands for."""
+        d = self.join_description(rows, True)
+        d.row_sums = self.layer.ranges["row_output"]
+        launch = launches_of(1)
+        check(self.card.lib.expert_post_prepare(C.byref(d), self.card.arena_bytes, self.fused_kernels.post, launch), "expert_post_prepare")
+        return launch
+
+    def shared_join_launch(self, rows=None, row_sums=True):
+        """The shared expert's down and the join in one launch (at most LINEAR_MAXIMUM_ROWS rows)."""
+        d = ExpertSharedJoinDescription()
+        d.down = self.matrix(2, self.down_slices)
+        d.codes, d.exponents, d.operands = self.ranges["hidden_codes"], self.ranges["hidden_exponents"], self.ranges["hidden_operands"]
+        d.join = self.join_description(rows, row_sums)
+        launch = launches_of(1)
+        check(self.card.lib.expert_shared_join_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.layer.kernels),
+                                                       C.byref(self.fused_kernels), launch), "expert_shared_join_prepare")
+        return launch
+
+    def read(self, name, dtype=np.uint8):
+        r = self.ranges[name]
+        return self.card.download(r.byte_offset, r.byte_count, dtype)

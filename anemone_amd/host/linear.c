@@ -82,6 +82,25 @@ result_status linear_kernels_prepare(const struct backend_operations *backend, s
         status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, KERNEL_EXPERT_ROW_SUM,
                                          sizeof(struct expert_row_sum_arguments), &kernels.expert_row_sum);
     }
+    for (uint32_t instance = 0; status == STATUS_OK && instance < BUILT_INSTANCES; instance++) {
+        char name[48];
+        (void)snprintf(name, sizeof name, "%s%u", KERNEL_TRUNK_LINEAR_QUANTIZED_STEM, slice_counts[instance]);
+        status = backend->kernel_prepare(card, KERNEL_FILE_TRUNK_LINEAR, name, sizeof(struct trunk_linear_quantized_arguments),
+                                         &kernels.trunk_linear_quantized[instance]);
+        if (status == STATUS_OK) {
+            (void)snprintf(name, sizeof name, "%s%u", KERNEL_TRUNK_LINEAR_QUANTIZED_WIDE_STEM, slice_counts[instance]);
+            status = backend->kernel_prepare(card, KERNEL_FILE_TRUNK_LINEAR, name, sizeof(struct trunk_linear_quantized_arguments),
+                                             &kernels.trunk_linear_quantized_wide[instance]);
+        }
+    }
+    if (status == STATUS_OK) {
+        status = backend->kernel_prepare(card, KERNEL_FILE_TRUNK_LINEAR, KERNEL_TRUNK_LINEAR_QUANTIZED_INTERLEAVED,
+                                         sizeof(struct trunk_linear_quantized_arguments), &kernels.trunk_linear_quantized_interleaved);
+    }
+    if (status == STATUS_OK) {
+        status = backend->kernel_prepare(card, KERNEL_FILE_TRUNK_LINEAR, KERNEL_TRUNK_HIDDEN, sizeof(struct trunk_hidden_arguments),
+                                         &kernels.trunk_hidden);
+    }
     if (status != STATUS_OK) {
         REFUSE("the kernels of the linear: a kernel is not prepared: %s", status_text(status));
         return status;
@@ -238,6 +257,211 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_ROW_SUM], kernels->expert_row_sum,
                 (down->output_size + ROW_SUM_BLOCK_OUTPUTS - 1u) / ROW_SUM_BLOCK_OUTPUTS, (uint32_t)rows, 1,
                 LINEAR_ELEMENT_THREADS, 0, &row_sum_record, sizeof row_sum_record);
+    memcpy(launches_out, launches, sizeof launches);
+    return STATUS_OK;
+}
+
+/*
+ * The shared expert: trunk products of quantized rows by E4M3_SCALED matrices (the reference's source/linear.c:
+ * linear_trunk_quantized_prepare, linear_shared_expert_prepare :1392-1506).
+ *
+ *   rows      kernel                                  grid                                             block   LDS
+ *   1..8      trunk_linear_quantized_<S>              (strips of both matrices, 1, 1)                  64 S    static
+ *   9..       trunk_linear_quantized_wide_<S>         (strips x n, 1, 1), n = groups of 8 rows or 1    64 S    static
+ *   9..       trunk_linear_quantized_interleaved_1    (blocks of both matrices, ceil(rows / 64), 1)    256     TRUNK_INTERLEAVED_WINDOW_BYTES
+ *   hidden    trunk_hidden_entry                      (ceil(width / 2048), rows, 1)                    256     0
+ * strip = TRUNK_STRIP_OUTPUTS outputs of one matrix, block = TRUNK_INTERLEAVED_BLOCK_OUTPUTS.
+ */
+static bool trunk_matrix_is_valid(const char *what, const struct linear_matrix *matrix, uint64_t *bytes_out, uint32_t *instance_out)
+{
+    const struct weight_format_operations *format = weight_format_operations_of(matrix->weight_format);
+    if (matrix->weight_format != WEIGHT_FORMAT_E4M3_SCALED || format == NULL || matrix->reserved_zero != 0 ||
+        format->stored_byte_count(&matrix->shape, bytes_out) != STATUS_OK || matrix->shape.input_size % 128u != 0 ||
+        matrix->shape.output_size < TRUNK_STRIP_OUTPUTS || matrix->shape.output_size % 16u != 0) {
+        REFUSE("%s: a matrix of format %u in a shape it stores, inputs a multiple of 128, outputs a multiple of 16 and at least %u",
+               what, (uint32_t)WEIGHT_FORMAT_E4M3_SCALED, TRUNK_STRIP_OUTPUTS);
+        return false;
+    }
+    if (!instance_of(matrix->slice_count, matrix->shape.input_size, instance_out)) {
+        REFUSE("%s: a slice count of %u: 1, 2, 4 or 8, at most one a 128 inputs", what, matrix->slice_count);
+        return false;
+    }
+    if ((uint32_t)matrix->wide_form >= (uint32_t)LINEAR_WIDE_FORM_COUNT) {
+        REFUSE("%s: a wide form of %u", what, (uint32_t)matrix->wide_form);
+        return false;
+    }
+    return true;
+}
+
+/* the launch of a trunk product whose description is checked: thin up to LINEAR_MAXIMUM_ROWS rows, else the
+ * first matrix's wide form; false where that form's kernel is not prepared or takes no such matrix */
+static bool trunk_launch_fill(const char *what, struct kernel_launch *launch, const struct linear_kernels_record *kernels,
+                              uint32_t instance, const struct linear_matrix *matrices, uint32_t matrix_count,
+                              const struct linear_range *codes, const struct linear_range *exponents,
+                              const struct linear_range *operands, const struct linear_range *outputs, uint32_t row_count)
+{
+    struct trunk_linear_quantized_arguments record;
+    memset(&record, 0, sizeof record);
+    uint32_t strips = 0, blocks = 0;
+    for (uint32_t m = 0; m < matrix_count; m++) {
+        record.weights_offset[m] = matrices[m].stored.byte_offset;
+        record.output_offset[m] = outputs[m].byte_offset;
+        record.output_size[m] = matrices[m].shape.output_size;
+        strips += (matrices[m].shape.output_size + TRUNK_STRIP_OUTPUTS - 1u) / TRUNK_STRIP_OUTPUTS;
+        blocks += (matrices[m].shape.output_size + TRUNK_INTERLEAVED_BLOCK_OUTPUTS - 1u) / TRUNK_INTERLEAVED_BLOCK_OUTPUTS;
+    }
+    record.codes_offset = codes->byte_offset;
+    record.exponents_offset = exponents->byte_offset;
+    record.operands_offset = operands->byte_offset;
+    record.input_size = matrices[0].shape.input_size;
+    record.row_count = row_count;
+    const uint32_t threads = 64u * matrices[0].slice_count;
+    const enum linear_wide_form form = matrices[0].wide_form;
+    uint32_t kernel;
+    if (row_count <= LINEAR_MAXIMUM_ROWS) {
+        kernel = kernels->trunk_linear_quantized[instance];
+        launch_fill(launch, kernel, strips, 1, 1, threads, 0, &record, sizeof record);
+    } else if (form == LINEAR_WIDE_GROUP_BLOCKS || form == LINEAR_WIDE_TILE_BLOCKS) {
+        const uint32_t groups = (row_count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS;
+        kernel = kernels->trunk_linear_quantized_wide[instance];
+        launch_fill(launch, kernel, strips * (form == LINEAR_WIDE_GROUP_BLOCKS ? groups : 1u), 1, 1, threads, 0, &record, sizeof record);
+    } else {
+        if (matrices[0].slice_count != 1u) {
+            REFUSE("%s: the interleaved form takes a matrix of one slice, not %u", what, matrices[0].slice_count);
+            return false;
+        }
+        kernel = kernels->trunk_linear_quantized_interleaved;
+        launch_fill(launch, kernel, blocks, (row_count + TRUNK_INTERLEAVED_ROWS - 1u) / TRUNK_INTERLEAVED_ROWS, 1, WIDE_BLOCK_THREADS,
+                    TRUNK_INTERLEAVED_WINDOW_BYTES, &record, sizeof record);
+    }
+    if (kernel == BACKEND_NO_KERNEL) {
+        REFUSE("%s: the kernel of its rows and form is not prepared", what);
+        return false;
+    }
+    return true;
+}
+
+result_status linear_trunk_quantized_prepare(const struct linear_trunk_quantized_description *description, uint64_t arena_byte_count,
+                                             const struct linear_kernels_record *kernels, struct kernel_launch *launch_out)
+{
+    static const char what[] = "a trunk product of quantized rows";
+    if (description == NULL || kernels == NULL || launch_out == NULL) {
+        REFUSE("%s: a missing argument", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (description->matrix_count == 0 || description->matrix_count > LINEAR_MERGED_MATRICES || description->row_count == 0 ||
+        description->row_count > LINEAR_TRUNK_MOST_ROWS) {
+        REFUSE("%s: one or two matrices, 1 to %u rows", what, LINEAR_TRUNK_MOST_ROWS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    uint64_t bytes[LINEAR_MERGED_MATRICES] = {0, 0};
+    uint32_t instance = 0;
+    const struct linear_matrix *first = &description->matrices[0];
+    for (uint32_t m = 0; m < description->matrix_count; m++) {
+        const struct linear_matrix *matrix = &description->matrices[m];
+        if (!trunk_matrix_is_valid(what, matrix, &bytes[m], &instance)) {
+            return STATUS_INVALID_ARGUMENT;
+        }
+        if (matrix->shape.input_size != first->shape.input_size || matrix->slice_count != first->slice_count ||
+            matrix->wide_form != first->wide_form) {
+            REFUSE("%s: two matrices of one launch are of one input size, slice count and wide form", what);
+            return STATUS_INVALID_ARGUMENT;
+        }
+    }
+    const uint64_t rows = description->row_count, inputs = first->shape.input_size;
+    struct checked_range ranges[3 + 2 * LINEAR_MERGED_MATRICES] = {
+        {"the rows' codes", description->codes, linear_codes_byte_count(rows, inputs), false},
+        {"the rows' exponents", description->exponents, linear_exponents_byte_count(rows, inputs), false},
+        {"the rows' operands", description->operands, 0, false},
+    };
+    uint32_t count = 3;
+    for (uint32_t m = 0; m < description->matrix_count; m++) {
+        ranges[count++] = (struct checked_range){"a matrix", description->matrices[m].stored, bytes[m], true};
+        ranges[count++] = (struct checked_range){"an output", description->outputs[m],
+                                                 linear_values_byte_count(rows, description->matrices[m].shape.output_size), false};
+    }
+    if (!ranges_are_valid(what, ranges, count, arena_byte_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    struct kernel_launch launch;
+    if (!trunk_launch_fill(what, &launch, kernels, instance, description->matrices, description->matrix_count, &description->codes,
+                           &description->exponents, &description->operands, description->outputs, description->row_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    *launch_out = launch;
+    return STATUS_OK;
+}
+
+result_status linear_shared_expert_prepare(const struct linear_shared_expert_description *description, uint64_t arena_byte_count,
+                                           const struct linear_kernels_record *kernels, struct kernel_launch *launches_out)
+{
+    static const char what[] = "the shared expert";
+    if (description == NULL || kernels == NULL || launches_out == NULL) {
+        REFUSE("%s: a missing argument", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct linear_matrix gate_up[LINEAR_MERGED_MATRICES] = {description->gate, description->up};
+    const struct linear_range gate_up_outputs[LINEAR_MERGED_MATRICES] = {description->gate_output, description->up_output};
+    const struct matrix_shape_record *gate = &description->gate.shape, *up = &description->up.shape, *down = &description->down.shape;
+    uint64_t gate_bytes = 0, up_bytes = 0, down_bytes = 0;
+    uint32_t gate_up_instance = 0, up_instance = 0, down_instance = 0;
+    if (!trunk_matrix_is_valid(what, &description->gate, &gate_bytes, &gate_up_instance) ||
+        !trunk_matrix_is_valid(what, &description->up, &up_bytes, &up_instance) ||
+        !trunk_matrix_is_valid(what, &description->down, &down_bytes, &down_instance)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (up->output_size != gate->output_size || up->input_size != gate->input_size || up_instance != gate_up_instance ||
+        description->up.wide_form != description->gate.wide_form || down->input_size != gate->output_size) {
+        REFUSE("%s: up is of gate's shape, slice count and wide form; down reads what they write", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t rows = description->row_count;
+    if (rows == 0 || rows > LINEAR_TRUNK_MOST_ROWS || !(description->activation_limit > 0.0f)) {
+        REFUSE("%s: 1 to %u rows, an activation limit above zero", what, LINEAR_TRUNK_MOST_ROWS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (kernels->trunk_hidden == BACKEND_NO_KERNEL || kernels->activation_quantize == BACKEND_NO_KERNEL) {
+        REFUSE("%s: a kernel of the chain is not prepared", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t H = gate->input_size, I = gate->output_size, hidden_bytes = linear_values_byte_count(rows, I);
+    const struct checked_range ranges[] = {
+        {"gate", description->gate.stored, gate_bytes, true},
+        {"up", description->up.stored, up_bytes, true},
+        {"down", description->down.stored, down_bytes, true},
+        {"the rows' codes", description->codes, linear_codes_byte_count(rows, H), false},
+        {"the rows' exponents", description->exponents, linear_exponents_byte_count(rows, H), false},
+        {"the rows' operands", description->operands, 0, false},
+        {"the output of gate", description->gate_output, hidden_bytes, false},
+        {"the output of up", description->up_output, hidden_bytes, false},
+        {"the hidden values", description->hidden, hidden_bytes, false},
+        {"the hidden codes", description->hidden_codes, linear_codes_byte_count(rows, I), false},
+        {"the hidden exponents", description->hidden_exponents, linear_exponents_byte_count(rows, I), false},
+        {"the hidden operands", description->hidden_operands, hidden_bytes, false},
+        {"the output", description->output, linear_values_byte_count(rows, down->output_size), false},
+    };
+    if (!ranges_are_valid(what, ranges, sizeof ranges / sizeof ranges[0], arena_byte_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    struct kernel_launch launches[LINEAR_SHARED_EXPERT_LAUNCH_COUNT];
+    if (!trunk_launch_fill(what, &launches[LINEAR_SHARED_EXPERT_GATE_UP], kernels, gate_up_instance, gate_up, LINEAR_MERGED_MATRICES,
+                           &description->codes, &description->exponents, &description->operands, gate_up_outputs, description->row_count) ||
+        !trunk_launch_fill(what, &launches[LINEAR_SHARED_EXPERT_DOWN], kernels, down_instance, &description->down, 1,
+                           &description->hidden_codes, &description->hidden_exponents, &description->hidden_operands,
+                           &description->output, description->row_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct trunk_hidden_arguments hidden_record = {description->gate_output.byte_offset, description->up_output.byte_offset,
+                                                         description->hidden.byte_offset, gate->output_size, description->activation_limit};
+    const struct activation_quantize_arguments quantize_record = {
+        description->hidden.byte_offset, description->hidden_codes.byte_offset, description->hidden_exponents.byte_offset,
+        description->hidden_operands.byte_offset, gate->output_size, 0};
+    launch_fill(&launches[LINEAR_SHARED_EXPERT_HIDDEN], kernels->trunk_hidden,
+                (gate->output_size + ROW_SUM_BLOCK_OUTPUTS - 1u) / ROW_SUM_BLOCK_OUTPUTS, description->row_count, 1,
+                LINEAR_ELEMENT_THREADS, 0, &hidden_record, sizeof hidden_record);
+    launch_fill(&launches[LINEAR_SHARED_EXPERT_QUANTIZE], kernels->activation_quantize,
+                (gate->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, description->row_count, 1,
+                LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
     memcpy(launches_out, launches, sizeof launches);
     return STATUS_OK;
 }

@@ -203,11 +203,11 @@ struct linear_kernels_record { /* include/anemone/linear.h:121-132 of the refere
     uint32_t expert_gate_up[LINEAR_SLICE_INSTANCES];
     uint32_t expert_down[LINEAR_SLICE_INSTANCES];
     uint32_t expert_row_sum;
-    uint32_t trunk_linear_quantized[LINEAR_SLICE_INSTANCES]; /* the trunk families are outside this path: */
-    uint32_t trunk_linear_bfloat16[LINEAR_SLICE_INSTANCES];  /* every trunk handle is BACKEND_NO_KERNEL */
+    uint32_t trunk_linear_quantized[LINEAR_SLICE_INSTANCES]; /* the shared expert's products: 1, 2, 4, 8 slices */
+    uint32_t trunk_linear_bfloat16[LINEAR_SLICE_INSTANCES];  /* rows that are not quantized: outside this path, BACKEND_NO_KERNEL */
     uint32_t trunk_hidden;
-    uint32_t trunk_linear_quantized_wide[LINEAR_SLICE_INSTANCES];
-    uint32_t trunk_linear_bfloat16_wide[LINEAR_SLICE_INSTANCES];
+    uint32_t trunk_linear_quantized_wide[LINEAR_SLICE_INSTANCES]; /* prepared by linear_kernels_prepare too (the reference prepares them apart) */
+    uint32_t trunk_linear_bfloat16_wide[LINEAR_SLICE_INSTANCES];  /* BACKEND_NO_KERNEL */
     uint32_t trunk_linear_quantized_interleaved;
     /* extension (no counterpart in the reference, whose expert kernels take E2M1 alone): the same two families
      * for experts of WEIGHT_FORMAT_E4M3_SCALED */
@@ -257,14 +257,75 @@ MUST_CHECK result_status linear_routed_experts_prepare(const struct linear_route
                                                        const struct linear_kernels_record *kernels,
                                                        struct kernel_launch *launches_out);
 
-/* ---- the producer (include/anemone/expert_fused.h:37-60 of the reference): one launch in place of the first two of
- * the routed experts. The join and the shared join of that header belong to the layer's next step, outside this
- * path: their handles are BACKEND_NO_KERNEL. ---- */
+/* ---- the shared expert (include/anemone/linear.h:161-262, 323-367 of the reference): trunk products of quantized
+ * rows by WEIGHT_FORMAT_E4M3_SCALED matrices ---- */
+/* The form of a trunk launch of more than LINEAR_MAXIMUM_ROWS rows. Every form gives the thin instance's bits.
+ * Here: GROUP_BLOCKS the wide instance with a block for each group of 8 rows of each strip, TILE_BLOCKS one block a
+ * strip that takes the groups in turn; both INTERLEAVED forms the interleaved instance of one slice (a block a tile of
+ * 64 rows by 128 outputs, the card's grouped-GEMM form: what a step of many rows takes). */
+enum linear_wide_form {
+    LINEAR_WIDE_GROUP_BLOCKS = 0,
+    LINEAR_WIDE_TILE_BLOCKS = 1,
+    LINEAR_INTERLEAVED_CHUNK_BLOCKS = 2,
+    LINEAR_INTERLEAVED_TILE_BLOCKS = 3,
+    LINEAR_WIDE_FORM_COUNT = 4
+};
+struct linear_matrix {
+    struct linear_range stored; /* read: exactly the bytes its format stores for its shape */
+    struct matrix_shape_record shape;
+    enum weight_format_code weight_format;
+    uint32_t slice_count;
+    enum linear_wide_form wide_form;
+    uint32_t reserved_zero;
+};
+#define LINEAR_TRUNK_MOST_ROWS 16384u /* rows of one trunk launch (the reference: 1,024, a wide step's chunk) */
+/* y = W x for quantized rows, of one matrix or of two that read the same rows (gate and up of the shared expert):
+ * one launch of trunk_linear_quantized_<S>, of its wide instance or of the interleaved one. Refused: a format other
+ * than E4M3_SCALED, a shape it does not store, inputs no multiple of 128, fewer than 32 outputs or no multiple of 16,
+ * a slice count no kernel is built for or above inputs / 128, two matrices that differ in input_size, slice_count or
+ * wide form, an interleaved form of more than one slice, 0 rows or more than LINEAR_TRUNK_MOST_ROWS, a bad range. */
+struct linear_trunk_quantized_description {
+    struct linear_matrix matrices[LINEAR_MERGED_MATRICES];
+    struct linear_range codes;     /* read: codes [row_count][input_size] */
+    struct linear_range exponents; /* read: exponents [row_count][input_size / 32] */
+    struct linear_range operands;  /* read: operands [row_count][input_size] */
+    struct linear_range outputs[LINEAR_MERGED_MATRICES]; /* written: bf16 [row_count][output_size] */
+    uint32_t matrix_count; /* 1 or 2 */
+    uint32_t row_count;
+};
+MUST_CHECK result_status linear_trunk_quantized_prepare(const struct linear_trunk_quantized_description *description,
+                                                        uint64_t arena_byte_count, const struct linear_kernels_record *kernels,
+                                                        struct kernel_launch *launch_out);
+
+enum linear_shared_expert_launch {
+    LINEAR_SHARED_EXPERT_GATE_UP = 0,  /* trunk_linear_quantized, two matrices: to gate_output and up_output */
+    LINEAR_SHARED_EXPERT_HIDDEN = 1,   /* trunk_hidden_entry: gate_output and up_output to hidden */
+    LINEAR_SHARED_EXPERT_QUANTIZE = 2, /* activation_quantize_entry: hidden to its arrays */
+    LINEAR_SHARED_EXPERT_DOWN = 3,     /* trunk_linear_quantized: the hidden arrays to output */
+    LINEAR_SHARED_EXPERT_LAUNCH_COUNT = 4
+};
+struct linear_shared_expert_description {
+    struct linear_matrix gate, up, down; /* E4M3_SCALED; gate and up of one shape, slice_count and wide form */
+    struct linear_range codes, exponents, operands;                     /* read: the rows' arrays, [row_count][gate.input_size] */
+    struct linear_range gate_output, up_output, hidden;                 /* scratch: bf16 [row_count][gate.output_size] each */
+    struct linear_range hidden_codes, hidden_exponents, hidden_operands; /* scratch: the hidden vectors' arrays */
+    struct linear_range output;                                         /* written: bf16 [row_count][down.output_size] */
+    uint32_t row_count;
+    float activation_limit;
+};
+/* launches_out: LINEAR_SHARED_EXPERT_LAUNCH_COUNT launches */
+MUST_CHECK result_status linear_shared_expert_prepare(const struct linear_shared_expert_description *description,
+                                                      uint64_t arena_byte_count, const struct linear_kernels_record *kernels,
+                                                      struct kernel_launch *launches_out);
+
+/* ---- the producer, the join and the shared join (include/anemone/expert_fused.h:37-101 of the reference): the
+ * routed experts' phase in fewer launches ---- */
 struct expert_fused_kernels {
     uint32_t gate_up_quantize[LINEAR_SLICE_INSTANCES];
     uint32_t shared_join[LINEAR_SLICE_INSTANCES];
     uint32_t join;
     uint32_t gate_up_quantize_e4m3[LINEAR_SLICE_INSTANCES]; /* extension: experts of WEIGHT_FORMAT_E4M3_SCALED */
+    uint32_t post;                                          /* extension: hyper_post_entry, the join's second half alone */
 };
 MUST_CHECK result_status expert_fused_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                       uint32_t arithmetic_class, struct expert_fused_kernels *kernels_out);
@@ -277,6 +338,40 @@ MUST_CHECK result_status expert_producer_prepare(const struct linear_routed_expe
                                                  struct linear_range arrivals, uint64_t arena_byte_count,
                                                  const struct linear_kernels_record *linear_kernels,
                                                  const struct expert_fused_kernels *kernels, struct kernel_launch *launch_out);
+
+/* A layer's FFN join: a row's routed sum (as expert_row_sum_entry), the shared expert's output added to it, and the
+ * post of the four residual streams, one launch of expert_join. The reference takes 1 to LINEAR_MAXIMUM_ROWS rows (a
+ * thin step, or a slab of a wide one) of its model's width; here 1 to 65535 rows of `width` values, a multiple of
+ * HYPER_VALUES_PER_THREAD x HYPER_PIECE_THREADS = 1,024 (0 stands for the reference's 5,120). */
+struct expert_join_description {
+    struct linear_range pair_output;   /* read: bf16 [row_count * pairs_per_row][width] */
+    struct linear_range shared_output; /* read: bf16 [row_count][width] */
+    struct linear_range streams;       /* read and written: bf16 [row_count][4][width] */
+    struct linear_range post;          /* read: float32 [row_count][4] */
+    struct linear_range comb;          /* read: float32 [row_count][4][4] */
+    struct linear_range row_sums;      /* written: float32 [row_count][width], or no bytes */
+    uint32_t pairs_per_row;
+    uint32_t row_count;
+    uint32_t width;                    /* extension */
+};
+MUST_CHECK result_status expert_join_prepare(const struct expert_join_description *description, uint64_t arena_byte_count,
+                                             const struct expert_fused_kernels *kernels, struct kernel_launch *launch_out);
+/* The post alone (hyper_post_entry with the combine: the sums read from join.row_sums, which must have bytes, the
+ * output from join.shared_output): the second of the two launches an expert_join stands for, behind
+ * expert_row_sum_entry. kernel: a handle of KERNEL_HYPER_POST. */
+MUST_CHECK result_status expert_post_prepare(const struct expert_join_description *join, uint64_t arena_byte_count,
+                                             uint32_t kernel, struct kernel_launch *launch_out);
+
+/* The same join behind the shared expert's down, one launch of expert_shared_join_<down.slice_count>: at most
+ * LINEAR_MAXIMUM_ROWS rows; down's outputs are the join's width; its output is written to join.shared_output. */
+struct expert_shared_join_description {
+    struct linear_matrix down;
+    struct linear_range codes, exponents, operands; /* read: the hidden vectors' arrays, [row_count][down.input_size] */
+    struct expert_join_description join;
+};
+MUST_CHECK result_status expert_shared_join_prepare(const struct expert_shared_join_description *description,
+                                                    uint64_t arena_byte_count, const struct linear_kernels_record *linear_kernels,
+                                                    const struct expert_fused_kernels *kernels, struct kernel_launch *launch_out);
 
 /* ---- the wide form of the routed experts: a grouped GEMM over the tiles of a wide select ----
  * The reference prepares its wide products from a description of the routed experts plus the tiles and sorted pairs

@@ -411,7 +411,10 @@ def test_linear_prepare_geometry_and_refusals(fake):
     kernels = amd.LinearKernels()
     assert lib.linear_kernels_prepare(fake.address, fake.card, 80, C.byref(kernels)) == 1  # a class of another card
     assert lib.linear_kernels_prepare(fake.address, fake.card, 950, C.byref(kernels)) == 0
-    assert kernels.expert_gate_up[4] == amd.BACKEND_NO_KERNEL and kernels.trunk_hidden == amd.BACKEND_NO_KERNEL  # 16 slices; the trunk
+    assert kernels.expert_gate_up[4] == amd.BACKEND_NO_KERNEL and kernels.trunk_linear_bfloat16[0] == amd.BACKEND_NO_KERNEL  # 16 slices; rows that are not quantized
+    assert fake.handles[kernels.trunk_hidden][1] == "trunk_hidden_entry" and kernels.trunk_linear_quantized[4] == amd.BACKEND_NO_KERNEL
+    assert fake.handles[kernels.trunk_linear_quantized_wide[2]] == ("kernel_trunk_linear", "trunk_linear_quantized_wide_4")
+    assert fake.handles[kernels.trunk_linear_quantized_interleaved][1] == "trunk_linear_quantized_interleaved_1"
     launches = amd.launches_of(4)
     assert lib.linear_routed_experts_prepare(C.byref(experts_description()), ARENA, C.byref(kernels), launches) == 0
     names = [fake.handles[l.kernel][1] for l in launches]
@@ -499,3 +502,152 @@ def test_wide_linear_prepare_geometry_and_refusals(fake):
         status = lib.linear_wide_experts_prepare(C.byref(wide_experts_description(**changes)), arena, C.byref(linear), C.byref(kernels), untouched)
         assert status == 1, changes
         assert not any(bytes(untouched))
+
+
+# ---- the shared expert and the FFN site's join ----
+
+def shared_description(rows=8, gate_up_slices=4, down_slices=2, form=amd.LINEAR_WIDE_GROUP_BLOCKS, **changes):
+    H, I = 4096, 2048
+    cursor = [4096]
+
+    def take(size):
+        at = cursor[0]
+        cursor[0] = (at + size + 255) // 256 * 256
+        return amd.Range(at, size)
+
+    def matrix(outputs, inputs, slices):
+        return amd.LinearMatrix(take(outputs * inputs + (outputs + 31) // 32 * (inputs // 32)), amd.Shape(outputs, inputs, 8, 0),
+                                amd.WEIGHT_FORMAT_E4M3_SCALED, slices, form, 0)
+    d = amd.SharedExpertDescription()
+    d.gate, d.up, d.down = matrix(I, H, gate_up_slices), matrix(I, H, gate_up_slices), matrix(H, I, down_slices)
+    d.codes, d.exponents, d.operands = take(rows * H), take(rows * H // 32), take(rows * H * 2)
+    d.gate_output, d.up_output, d.hidden = take(rows * I * 2), take(rows * I * 2), take(rows * I * 2)
+    d.hidden_codes, d.hidden_exponents, d.hidden_operands = take(rows * I), take(rows * I // 32), take(rows * I * 2)
+    d.output = take(rows * H * 2)
+    d.row_count, d.activation_limit = rows, 10.0
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d, cursor[0]
+
+
+def join_description(rows=8, picks=8, width=4096, first=1 << 30, row_sums=True, **changes):
+    cursor = [first]
+
+    def take(size):
+        at = cursor[0]
+        cursor[0] = (at + size + 255) // 256 * 256
+        return amd.Range(at, size)
+    d = amd.ExpertJoinDescription()
+    wide = 5120 if width == 0 else width
+    d.pair_output, d.shared_output, d.streams = take(rows * picks * wide * 2), take(rows * wide * 2), take(rows * 4 * wide * 2)
+    d.post, d.comb = take(rows * 16), take(rows * 64)
+    d.row_sums = take(rows * wide * 4) if row_sums else amd.Range(0, 0)
+    d.pairs_per_row, d.row_count, d.width = picks, rows, width
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d
+
+
+def test_shared_expert_prepare_geometry_and_refusals(fake):
+    lib = amd.library()
+    arena = 8 << 30
+    kernels = amd.LinearKernels()
+    assert lib.linear_kernels_prepare(fake.address, fake.card, 950, C.byref(kernels)) == 0
+    table = kernel_table()
+    assert table[("kernel_trunk_linear", "trunk_linear_quantized_1")] == C.sizeof(amd.TrunkLinearQuantizedArguments) == 72
+    assert table[("kernel_trunk_linear", "trunk_hidden_entry")] == 32
+    launches = amd.launches_of(4)
+    d, _ = shared_description()
+    assert lib.linear_shared_expert_prepare(C.byref(d), arena, C.byref(kernels), launches) == 0
+    assert [fake.handles[l.kernel][1] for l in launches] == ["trunk_linear_quantized_4", "trunk_hidden_entry", "activation_quantize_entry",
+                                                             "trunk_linear_quantized_2"]
+    assert [list(l.grid) for l in launches] == [[128, 1, 1], [1, 8, 1], [8, 8, 1], [128, 1, 1]]  # strips of 32 outputs of both matrices
+    assert [l.block[0] for l in launches] == [256, 256, 256, 128]
+    assert [l.argument_byte_count for l in launches] == [72, 32, 40, 72]
+    record = amd.TrunkLinearQuantizedArguments.from_buffer_copy(bytes(launches[0].argument)[:72])
+    assert list(record.output_size) == [2048, 2048] and (record.input_size, record.row_count) == (4096, 8)
+    assert list(record.weights_offset) == [d.gate.stored.byte_offset, d.up.stored.byte_offset]
+    down = amd.TrunkLinearQuantizedArguments.from_buffer_copy(bytes(launches[3].argument)[:72])
+    assert list(down.output_size) == [4096, 0] and down.codes_offset == d.hidden_codes.byte_offset
+    # more than eight rows: the matrix's wide form
+    for form, names, grids, blocks, shared_bytes in (
+            (amd.LINEAR_WIDE_GROUP_BLOCKS, ["trunk_linear_quantized_wide_4", "trunk_linear_quantized_wide_2"], [[128 * 13, 1, 1], [128 * 13, 1, 1]], [256, 128], 0),
+            (amd.LINEAR_WIDE_TILE_BLOCKS, ["trunk_linear_quantized_wide_4", "trunk_linear_quantized_wide_2"], [[128, 1, 1], [128, 1, 1]], [256, 128], 0)):
+        wide, _ = shared_description(rows=100, form=form)
+        assert lib.linear_shared_expert_prepare(C.byref(wide), arena, C.byref(kernels), launches) == 0
+        assert [fake.handles[l.kernel][1] for l in launches][::3] == names
+        assert [list(l.grid) for l in launches][::3] == grids and [l.block[0] for l in launches][::3] == blocks
+        assert launches[0].dynamic_shared_byte_count == shared_bytes
+    many, _ = shared_description(rows=8192, gate_up_slices=1, down_slices=1, form=amd.LINEAR_INTERLEAVED_CHUNK_BLOCKS)
+    assert lib.linear_shared_expert_prepare(C.byref(many), arena, C.byref(kernels), launches) == 0
+    assert [fake.handles[l.kernel][1] for l in launches][::3] == ["trunk_linear_quantized_interleaved_1"] * 2
+    assert [list(l.grid) for l in launches] == [[32, 128, 1], [1, 8192, 1], [8, 8192, 1], [32, 128, 1]]
+    assert [l.dynamic_shared_byte_count for l in launches] == [51712, 0, 0, 51712] and launches[0].block[0] == 256
+    sliced, _ = shared_description(rows=100, form=amd.LINEAR_INTERLEAVED_CHUNK_BLOCKS)  # the interleaved form is of one slice
+    untouched = amd.launches_of(4)
+    assert lib.linear_shared_expert_prepare(C.byref(sliced), arena, C.byref(kernels), untouched) == 1 and not any(bytes(untouched))
+    for changes in (dict(row_count=0), dict(row_count=20000), dict(activation_limit=0.0), dict(output=amd.Range((8 << 30) - 256, 1 << 20)),
+                    dict(hidden=amd.Range(4096, 1 << 16))):
+        bad, _ = shared_description(**changes)
+        assert lib.linear_shared_expert_prepare(C.byref(bad), arena, C.byref(kernels), untouched) == 1, changes
+        assert not any(bytes(untouched))
+    for mutate in (lambda d: setattr(d.gate, "weight_format", amd.WEIGHT_FORMAT_E2M1_SCALED), lambda d: setattr(d.up, "slice_count", 2),
+                   lambda d: setattr(d.down, "slice_count", 3), lambda d: setattr(d.down, "wide_form", 7),
+                   lambda d: setattr(d.up, "shape", amd.Shape(1024, 4096, 8, 0)), lambda d: setattr(d.gate, "reserved_zero", 1)):
+        bad, _ = shared_description()
+        mutate(bad)
+        assert lib.linear_shared_expert_prepare(C.byref(bad), arena, C.byref(kernels), untouched) == 1
+        assert not any(bytes(untouched))
+    # a trunk launch of one matrix
+    one = amd.TrunkQuantizedDescription()
+    one.matrices[0], one.codes, one.exponents, one.operands, one.outputs[0] = d.down, d.hidden_codes, d.hidden_exponents, d.hidden_operands, d.output
+    one.matrix_count, one.row_count = 1, 8
+    launch = amd.launches_of(1)
+    assert lib.linear_trunk_quantized_prepare(C.byref(one), arena, C.byref(kernels), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "trunk_linear_quantized_2" and list(launch[0].grid) == [128, 1, 1]
+    one.matrix_count = 3
+    assert lib.linear_trunk_quantized_prepare(C.byref(one), arena, C.byref(kernels), launch) == 1
+
+
+def test_join_prepare_geometry_and_refusals(fake):
+    lib = amd.library()
+    arena = 8 << 30
+    linear, kernels = amd.LinearKernels(), amd.ExpertFusedKernels()
+    assert lib.linear_kernels_prepare(fake.address, fake.card, 950, C.byref(linear)) == 0
+    assert lib.expert_fused_kernels_prepare(fake.address, fake.card, 950, C.byref(kernels)) == 0
+    assert fake.handles[kernels.join] == ("kernel_hyper_connection", "expert_join")
+    assert fake.handles[kernels.shared_join[1]] == ("kernel_trunk_linear", "expert_shared_join_2") and kernels.shared_join[4] == amd.BACKEND_NO_KERNEL
+    table = kernel_table()
+    assert table[("kernel_hyper_connection", "expert_join")] == C.sizeof(amd.ExpertJoinArguments) == 56
+    assert table[("kernel_hyper_connection", "hyper_post_entry")] == 48 and table[("kernel_trunk_linear", "expert_shared_join_1")] == 96
+    launch = amd.launches_of(1)
+    d = join_description()
+    assert lib.expert_join_prepare(C.byref(d), arena, C.byref(kernels), launch) == 0
+    assert list(launch[0].grid) == [4, 8, 1] and launch[0].block[0] == 128 and launch[0].argument_byte_count == 56
+    record = amd.ExpertJoinArguments.from_buffer_copy(bytes(launch[0].argument)[:56])
+    assert (record.pair_output_offset, record.row_sums_offset, record.pairs_per_row) == (d.pair_output.byte_offset, d.row_sums.byte_offset, 8)
+    none = join_description(row_sums=False)
+    assert lib.expert_join_prepare(C.byref(none), arena, C.byref(kernels), launch) == 0
+    assert amd.ExpertJoinArguments.from_buffer_copy(bytes(launch[0].argument)[:56]).row_sums_offset == 0xFFFFFFFFFFFFFFFF
+    default = join_description(width=0, rows=3000, picks=6)  # the reference's width
+    assert lib.expert_join_prepare(C.byref(default), arena, C.byref(kernels), launch) == 0 and list(launch[0].grid) == [5, 3000, 1]
+    assert lib.expert_post_prepare(C.byref(d), arena, kernels.post, launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "hyper_post_entry" and launch[0].argument_byte_count == 48 and list(launch[0].grid) == [4, 8, 1]
+    untouched = amd.launches_of(1)
+    assert lib.expert_post_prepare(C.byref(none), arena, kernels.post, untouched) == 1
+    for changes in (dict(row_count=0), dict(pairs_per_row=0), dict(width=4100), dict(width=512), dict(streams=amd.Range(1 << 30, 1 << 20)),
+                    dict(post=amd.Range((8 << 30) - 64, 128)), dict(comb=amd.Range((1 << 30) + 8, 512))):
+        assert lib.expert_join_prepare(C.byref(join_description(**changes)), arena, C.byref(kernels), untouched) == 1, changes
+        assert not any(bytes(untouched))
+    # the shared join: the down of a shared expert with the join behind it
+    shared, end = shared_description(down_slices=2)
+    s = amd.ExpertSharedJoinDescription()
+    s.down, s.codes, s.exponents, s.operands = shared.down, shared.hidden_codes, shared.hidden_exponents, shared.hidden_operands
+    s.join = join_description()
+    assert lib.expert_shared_join_prepare(C.byref(s), arena, C.byref(linear), C.byref(kernels), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "expert_shared_join_2" and list(launch[0].grid) == [128, 1, 1] and launch[0].block[0] == 128
+    assert launch[0].argument_byte_count == 96
+    s.join = join_description(rows=9)
+    assert lib.expert_shared_join_prepare(C.byref(s), arena, C.byref(linear), C.byref(kernels), untouched) == 1 and not any(bytes(untouched))
+    s.join = join_description(width=5120)
+    assert lib.expert_shared_join_prepare(C.byref(s), arena, C.byref(linear), C.byref(kernels), untouched) == 1  # down has 4,096 outputs
