@@ -34,6 +34,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("fp8_decode", 32): 2768.4e6 + 1.0e6,
     ("fp4_prefill", 8192): 5044.9e6 + 443.2e6,  # profiles/wide_expert_fp4_fp8_prefill.md
     ("fp8_prefill", 2048): 5642.4e6 + 117.0e6,
+    ("expert_join", 8192): 877.7e6 + 402.7e6,  # profiles/expert_join_trunk_linear_ffn_site.md
 }
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
 CONFIG = 1
@@ -128,6 +129,25 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(4)]
         names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
                                                          "expert_down", "expert_row_sum_entry"]
+    shared = None
+    if arguments.site:
+        # the whole FFN site: the shared expert (three E4M3 matrices applied to every row) and the join in place of the
+        # row sum (a row's routed sum, which it also stores, the shared output added, the post of the four streams)
+        shared_matrices = [workloads.fp8_matrix(base + 900, INNER, HIDDEN), workloads.fp8_matrix(base + 901, INNER, HIDDEN),
+                           workloads.fp8_matrix(base + 902, HIDDEN, INNER)]
+        many = rows > 64
+        shared = amd.SharedExpert(layer, shared_matrices, gate_up_slices=1 if many else 4, down_slices=1 if many else 2,
+                                  wide_form=amd.LINEAR_INTERLEAVED_CHUNK_BLOCKS if many else amd.LINEAR_WIDE_GROUP_BLOCKS)
+        site_streams = workloads.to_bf16(workloads.normals(base + 903, rows * 4 * HIDDEN)).reshape(rows, 4, HIDDEN)
+        site_post, site_comb = np.ones((rows, 4), dtype=np.float32), np.full((rows, 4, 4), 0.25, dtype=np.float32)
+        shared.set_site(site_streams, site_post, site_comb)
+        four = shared.launches()
+        if rows <= amd.LINEAR_MAXIMUM_ROWS:  # a thin step: the shared expert's down and the join in one launch
+            parts = parts[:-1] + [four[i] for i in range(3)] + [shared.shared_join_launch()[0]]
+            names = names[:-1] + ["trunk_gate_up", "trunk_hidden", "activation_quantize(shared)", "expert_shared_join"]
+        else:
+            parts = parts[:-1] + [four[i] for i in range(4)] + [shared.join_launch()[0]]
+            names = names[:-1] + ["trunk_gate_up", "trunk_hidden", "activation_quantize(shared)", "trunk_down", "expert_join"]
     step = amd.launches_of(len(parts))
     for i, launch in enumerate(parts):
         step[i] = launch
@@ -178,6 +198,21 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                      "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
     }
+    if shared is not None:
+        # the join moves (pairs_per_row + 1 + 4) bf16 values in and 4 bf16 values and a float32 sum out, a value
+        join_name = "expert_shared_join" if rows <= amd.LINEAR_MAXIMUM_ROWS else "expert_join"
+        join_us = float(per_launch[names.index(join_name)])
+        join_bytes = rows * HIDDEN * ((PICKS + 1 + 4) * 2 + 4 * 2 + 4)
+        trunk_us = float(per_launch[names.index("trunk_gate_up")])
+        shared_matrix_bytes = HIDDEN * INNER + HIDDEN * INNER // 1024
+        result["config"]["site"] = {
+            "launches": "the shared expert (E4M3 weights) and the join in place of the row sum",
+            "join_us": join_us, "join_algorithmic_bytes": int(join_bytes),
+            "join_GBps": None if join_name == "expert_shared_join" else join_bytes / (join_us * 1e-6) / 1e9,
+            "join_frac_of_hbm_peak": None if join_name == "expert_shared_join" else join_bytes / (join_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "join_traffic": MEASURED_TRAFFIC_BYTES.get(("expert_join", rows)),
+            "trunk_gate_up_us": trunk_us, "trunk_gate_up_GBps": 2 * shared_matrix_bytes / (trunk_us * 1e-6) / 1e9,
+            "trunk_gate_up_TFLOPs": 2.0 * rows * 2 * HIDDEN * INNER / (trunk_us * 1e-6) / 1e12}
     key = ("%s_%s" % ("fp8" if fp8 else "fp4", "prefill" if prefill else "decode"), rows)
     if key in MEASURED_TRAFFIC_BYTES and (prefill or (arguments.gate_up_slices, arguments.down_slices) == (4, 2)):
         result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES[key]
@@ -216,13 +251,34 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                 weights_of.reshape(-1)[job["pair_index"][c]] = job["route_weight"][c]
         pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
         want = np.zeros((sample, HIDDEN), dtype=np.float32)
+        want_pairs = np.zeros((sample * PICKS, HIDDEN), dtype=np.uint16)
         start = time.perf_counter()
         o.orc.orc_linear_moe_layer(5 if fp8 else 3, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS,
                                    o.ptr(np.ascontiguousarray(experts_of[:sample]), o.u32p),
                                    o.ptr(np.ascontiguousarray(weights_of[:sample]), o.f32p), EXPERTS, pointers, 10.0,
-                                   o.ptr(want, o.f32p), None, None, threads)
+                                   o.ptr(want, o.f32p), None, o.ptr(want_pairs, o.u16p), threads)
+        if shared is not None:  # the shared expert of the same sample, and the join of the two
+            shared_pointers = (C.c_void_p * 3)(*[m.ctypes.data for m in shared_matrices])
+            zero, one = np.zeros((sample, 1), dtype=np.uint32), np.ones((sample, 1), dtype=np.float32)
+            unused, shared_want = np.zeros((sample, HIDDEN), dtype=np.float32), np.zeros((sample, HIDDEN), dtype=np.uint16)
+            o.orc.orc_linear_moe_layer(5, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, 1, o.ptr(zero, o.u32p),
+                                       o.ptr(one, o.f32p), 1, shared_pointers, 10.0, o.ptr(unused, o.f32p), None, o.ptr(shared_want, o.u16p),
+                                       threads)
+            want_streams = site_streams[:sample].copy()  # joined in place
+            o.orc.orc_expert_join(o.ptr(want_pairs, o.u16p), o.ptr(shared_want, o.u16p), o.ptr(want_streams, o.u16p),
+                                  o.ptr(site_post, o.f32p), o.ptr(site_comb, o.f32p), None, sample, PICKS, HIDDEN)
         cpu_seconds = time.perf_counter() - start
-        got = layer.read("row_output", np.float32).reshape(rows, HIDDEN)[:sample]
+        if shared is None:
+            got = layer.read("row_output", np.float32).reshape(rows, HIDDEN)[:sample]
+        else:  # one step from the streams' first values
+            shared.set_site(site_streams, site_post, site_comb)
+            card.run(step)
+            got = shared.read("row_sums", np.float32).reshape(rows, HIDDEN)[:sample]
+            got_streams = o.bf16_to_f32(shared.read("streams", np.uint16).reshape(rows, 4, HIDDEN)[:sample].reshape(-1)).astype(np.float64)
+            wanted = o.bf16_to_f32(want_streams.reshape(-1)).astype(np.float64)
+            stream_error = float(np.sqrt(np.mean((got_streams - wanted) ** 2) / np.mean(wanted ** 2)))
+            assert stream_error < 2e-2, "the streams differ from the oracle's: rms %g" % stream_error
+            result["config"]["site"]["streams_vs_oracle_rms_err"] = stream_error
         error = float(np.sqrt(np.mean((got - want) ** 2) / np.mean(want.astype(np.float64) ** 2)))
         assert error < 2e-2, "GPU output differs from the oracle's: rms %g" % error
         result["cpu_baseline"] = {"value": sample / cpu_seconds, "unit": "tok/s", "cores": threads, "kind": "port",
@@ -332,6 +388,8 @@ def main():
     parser.add_argument("--gate-up-slices", type=int, default=4)
     parser.add_argument("--down-slices", type=int, default=2)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--site", action="store_true",
+                        help="fp4/fp8 workloads: the whole FFN site, with the shared expert and the join in place of the row sum")
     parser.add_argument("--graph", action="store_true", help="time replays of the step captured as one graph (graph_capture / graph_run)")
     parser.add_argument("--calibrate", action="store_true",
                         help="run only a 1 GiB arena copy, five times: the yardstick of the traffic counters")
