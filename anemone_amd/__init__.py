@@ -12,7 +12,7 @@ LIBRARY_PATH = os.path.join(HERE, "libanemone_hip.so")
 
 STATUS_OK, STATUS_INVALID_ARGUMENT, STATUS_OUT_OF_MEMORY = 0, 1, 2
 STATUS_DEVICE_ERROR, STATUS_TIMED_OUT, STATUS_UNSUPPORTED, STATUS_BUSY = 5, 6, 7, 8
-WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED = 2, 3, 5
+WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED, WEIGHT_FORMAT_E4M3_BLOCK128 = 2, 3, 5, 6
 ARITHMETIC_CLASS_GFX950 = 950
 BACKEND_NO_KERNEL = 0xFFFFFFFF
 LAUNCH_CHAIN, LAUNCH_SIDE, LAUNCH_RESUME, LAUNCH_JOIN, LAUNCH_SIDE_MORE = 0, 1, 2, 3, 4  # kernel_launch.branch
@@ -136,7 +136,8 @@ class LinearKernels(C.Structure):
     _fields_ = [("activation_quantize", u32), ("expert_gate_up", u32 * 5), ("expert_down", u32 * 5), ("expert_row_sum", u32),
                 ("trunk_linear_quantized", u32 * 5), ("trunk_linear_bfloat16", u32 * 5), ("trunk_hidden", u32),
                 ("trunk_linear_quantized_wide", u32 * 5), ("trunk_linear_bfloat16_wide", u32 * 5),
-                ("trunk_linear_quantized_interleaved", u32), ("expert_gate_up_e4m3", u32 * 5), ("expert_down_e4m3", u32 * 5)]
+                ("trunk_linear_quantized_interleaved", u32), ("expert_gate_up_e4m3", u32 * 5), ("expert_down_e4m3", u32 * 5),
+                ("expert_gate_up_b128", u32 * 5), ("expert_down_b128", u32 * 5), ("activation_quantize_128", u32)]
 
 
 class ExpertFusedKernels(C.Structure):
@@ -180,7 +181,8 @@ class ExpertJoinArguments(C.Structure):
 
 
 class LinearWideKernels(C.Structure):
-    _fields_ = [("wide_expert_gate_up", u32), ("wide_expert_down", u32), ("wide_expert_gate_up_e4m3", u32), ("wide_expert_down_e4m3", u32)]
+    _fields_ = [("wide_expert_gate_up", u32), ("wide_expert_down", u32), ("wide_expert_gate_up_e4m3", u32), ("wide_expert_down_e4m3", u32),
+                ("wide_expert_gate_up_b128", u32), ("wide_expert_down_b128", u32)]
 
 
 class QuantizeDescription(C.Structure):
@@ -238,6 +240,9 @@ def library():
             "router_wide_small_prepare": [C.POINTER(RouterWideDescription), u64, C.POINTER(RouterKernels), launch_p],
             "linear_kernels_prepare": [vp, vp, u32, C.POINTER(LinearKernels)],
             "linear_quantize_prepare": [C.POINTER(QuantizeDescription), u64, C.POINTER(LinearKernels), launch_p],
+            "linear_quantize_128_prepare": [C.POINTER(QuantizeDescription), u64, C.POINTER(LinearKernels), launch_p],
+            "linear_wide_experts_block128_prepare": [C.POINTER(LinearWideExpertsDescription), u64, C.POINTER(LinearKernels),
+                                                     C.POINTER(LinearWideKernels), launch_p],
             "linear_routed_experts_prepare": [C.POINTER(RoutedExpertsDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_default_slice_count": [C.c_int, C.c_int, C.c_int, C.POINTER(Shape), u32, C.POINTER(u32)],
             "linear_wide_kernels_prepare": [vp, vp, u32, C.POINTER(LinearWideKernels)],
@@ -658,7 +663,8 @@ class Fp4Layer:
                  weight_format=WEIGHT_FORMAT_E2M1_SCALED):
         self.card, self.H, self.I, self.E, self.P, self.rows = card, hidden, inner, expert_count, picks, rows
         self.weight_format = weight_format
-        self.bits = 8 if weight_format == WEIGHT_FORMAT_E4M3_SCALED else 4
+        self.bits = 8 if weight_format in (WEIGHT_FORMAT_E4M3_SCALED, WEIGHT_FORMAT_E4M3_BLOCK128) else 4
+        self.block128 = weight_format == WEIGHT_FORMAT_E4M3_BLOCK128
         self.limit, self.affinity_kind, self.route_scale = limit, affinity_kind, route_scale
         self.gate_up_slices, self.down_slices = gate_up_slices, down_slices
         self.pairs = rows * picks
@@ -714,7 +720,8 @@ class Fp4Layer:
         d = QuantizeDescription(Range(self.x_offset, self.rows * self.H * 2), self.ranges["codes"], self.ranges["exponents"],
                                 self.ranges["operands"], self.H, self.rows)
         launch = launches_of(1)
-        check(self.card.lib.linear_quantize_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launch), "linear_quantize_prepare")
+        prepare = self.card.lib.linear_quantize_128_prepare if self.block128 else self.card.lib.linear_quantize_prepare
+        check(prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), launch), "linear_quantize_prepare")
         return launch
 
     def projection_launch(self):
@@ -758,9 +765,9 @@ class Fp4Layer:
         d.experts = self.experts_description(wide)
         d.experts.gate_up_slice_count = d.experts.down_slice_count = 1
         d.tiles, d.pairs, d.tile_count = wide.ranges["tiles"], wide.ranges["pairs"], wide.tile_count
-        launches = launches_of(3)
-        check(self.card.lib.linear_wide_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), C.byref(self.wide_kernels),
-                                                        launches), "linear_wide_experts_prepare")
+        launches = launches_of(4 if self.block128 else 3)
+        prepare = self.card.lib.linear_wide_experts_block128_prepare if self.block128 else self.card.lib.linear_wide_experts_prepare
+        check(prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), C.byref(self.wide_kernels), launches), "linear_wide_experts_prepare")
         return launches
 
     def producer_launch(self):

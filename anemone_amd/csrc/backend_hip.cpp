@@ -725,7 +725,8 @@ bool backend_hip_format_supported(uint32_t card_index, enum weight_format_code f
     if (backend_hip_card_count(&count) != STATUS_OK || card_index >= count) {
         return false;
     }
-    return format == WEIGHT_FORMAT_EXL3 || format == WEIGHT_FORMAT_E2M1_SCALED || format == WEIGHT_FORMAT_E4M3_SCALED;
+    return format == WEIGHT_FORMAT_EXL3 || format == WEIGHT_FORMAT_E2M1_SCALED || format == WEIGHT_FORMAT_E4M3_SCALED ||
+           format == WEIGHT_FORMAT_E4M3_BLOCK128;
 }
 
 result_status backend_hip_graph_capture(struct device_card *card, const struct kernel_launch *launches,

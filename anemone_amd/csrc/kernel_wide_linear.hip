@@ -24,10 +24,10 @@
 #include "wide_device.cuh"
 
 /* grid (ceil(output_size / (4 strips)), tile_count), block 256; a strip is STRIP tiles of gate and STRIP of up */
-template <bool BYTES, uint32_t STRIP, uint32_t DEPTH>
+template <bool BYTES, uint32_t STRIP, uint32_t DEPTH, bool B128 = false>
 __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_expert_gate_up_arguments &arguments, unsigned char *arena)
 {
-    typedef wide_chain<2, BYTES, STRIP, DEPTH> chain_type;
+    typedef wide_chain<2, BYTES, STRIP, DEPTH, B128> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP_OUTPUTS = STRIP * 16u;
     static_assert(STRIP == 1u || STRIP == 2u, "a quantizer block of 32 outputs is one strip or two");
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
@@ -93,9 +93,21 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
                     largest[j] = fmaxf(largest[j], fabsf(bf16_to_float((uint16_t)bits[j][n][v])));
                 }
             }
+            if constexpr (B128) {
+                /* the hidden values themselves, where the record names the hidden operands (bfloat16 [pair][width]
+                 * either way): this format's quantizer takes 128 values a scale, in a launch of its own */
+                uint16_t *values = (uint16_t *)(arena + arguments.hidden_operands_offset) + (uint64_t)pairs[column].pair_index * width;
+#pragma unroll
+                for (uint32_t n = 0; n < STRIP; n++) {
+                    *(uint2_t *)(values + (tile0 + n) * 16u + 4u * g) = (uint2_t){bits[j][n][0] | (bits[j][n][1] << 16), bits[j][n][2] | (bits[j][n][3] << 16)};
+                }
+            }
             largest[j] = fmaxf(largest[j], __shfl_xor(largest[j], 16, WAVE));
             largest[j] = fmaxf(largest[j], __shfl_xor(largest[j], 32, WAVE));
         }
+    }
+    if constexpr (B128) {
+        return;
     }
     if constexpr (STRIP == 1u) {
         float *halves = (float *)window; /* [wavefront][column]: the stages are done with */
@@ -145,10 +157,10 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
     }
 }
 
-template <bool BYTES>
+template <bool BYTES, bool B128 = false>
 __device__ static __forceinline__ void wide_expert_down(const struct wide_expert_down_arguments &arguments, unsigned char *arena)
 {
-    typedef wide_chain<1, BYTES, (BYTES ? 2u : 4u), 2u> chain_type;
+    typedef wide_chain<1, BYTES, (BYTES ? 2u : 4u), 2u, B128> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP, STRIP_OUTPUTS = STRIP * 16u;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     const struct wide_expert_tile tile = ((const struct wide_expert_tile *)(arena + arguments.tiles_offset))[blockIdx.y];
@@ -226,6 +238,18 @@ extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_e4m3
     wide_expert_down<true>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_e4m3_1, wide_expert_down_arguments);
+/* WEIGHT_FORMAT_E4M3_BLOCK128 experts (float32 scales of 128 x 128 blocks; no counterpart in the reference): the
+ * gate/up entry writes the hidden VALUES at hidden_operands_offset and no codes */
+extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_gate_up_b128_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
+{
+    wide_expert_gate_up<true, 1u, 2u, true>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_gate_up_b128_1, wide_expert_gate_up_arguments);
+extern "C" __global__ void __launch_bounds__(WIDE_THREADS) wide_expert_down_b128_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
+{
+    wide_expert_down<true, true>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_WIDE_LINEAR, wide_expert_down_b128_1, wide_expert_down_arguments);
 
 static_assert(wide_chain<2, false, 2u, 2u>::WINDOW_BYTES == WIDE_GATE_UP_WINDOW_BYTES && wide_chain<2, true, 1u, 2u>::WINDOW_BYTES == WIDE_GATE_UP_E4M3_WINDOW_BYTES &&
                   wide_chain<1, false, 4u, 2u>::WINDOW_BYTES == WIDE_DOWN_WINDOW_BYTES && wide_chain<1, true, 2u, 2u>::WINDOW_BYTES == WIDE_DOWN_E4M3_WINDOW_BYTES,

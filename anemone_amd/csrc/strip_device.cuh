@@ -14,8 +14,12 @@
  * LDS window of a wavefront: DEPTH stages; a stage: MATRICES x STRIP x 1,024 bytes of weights, MATRICES x 256 bytes
  * of their scales (a matrix's STRIP tiles x 64), 1,024 bytes of the vectors' codes (8 columns x 128) and 256 bytes
  * holding their scale words. */
-template <uint32_t MATRICES, bool BYTES>
+/* B128 (one-byte weights alone): the scales are float32, one for every 128 outputs x 128 inputs of a matrix and one for
+ * every 128 values of a vector, in place of the E8M0 codes; a K step's MFMA then runs from zero with scales of one and its
+ * sums enter the chain by one fused multiply-add with the product of the two scales. */
+template <uint32_t MATRICES, bool BYTES, bool B128 = false>
 struct strip_chain {
+    static_assert(BYTES || !B128, "float32 scales go with one-byte weights");
     static constexpr uint32_t STRIP = BYTES ? 2u : 4u; /* tiles of a strip: 4 KB of every matrix a stage either way */
     static constexpr uint32_t STEP_BYTES = BYTES ? BYTE_STEP_BYTES : NIBBLE_STEP_BYTES;
     static constexpr uint32_t TILE_LOADS = STEP_BYTES / 1024u; /* 16-byte-a-lane loads of a tile's step */
@@ -91,10 +95,30 @@ struct strip_chain {
                 b[2u * part + 1u] = (int)__builtin_amdgcn_perm(pair.y, pair.x, 0x07030602u);
             }
         }
-        const uint32_t scale_b = lds_read<unsigned char>(base + VECTOR_SCALE_AT + vector_scale_at);
+        uint32_t scale_b = 0;
+        float float_scale_b = 0.0f;
+        if constexpr (B128) {
+            float_scale_b = lds_read<float>(base + VECTOR_SCALE_AT + vector_scale_at);
+        } else {
+            scale_b = lds_read<unsigned char>(base + VECTOR_SCALE_AT + vector_scale_at);
+        }
 #pragma unroll
         for (uint32_t tile = 0; tile < TILES; tile++) {
             int8_vector a = {0, 0, 0, 0, 0, 0, 0, 0};
+            if constexpr (B128) {
+                const float scale = __fmul_rn(lds_read<float>(base + SCALES_AT + (tile / STRIP) * 256u), float_scale_b);
+#pragma unroll
+                for (uint32_t v = 0; v < 8u; v++) {
+                    const uint2_t w = lds_read<uint2_t>(base + tile * STEP_BYTES + read_at[v]);
+                    a[v] = (int)__builtin_amdgcn_perm(w.y, w.x, shift);
+                }
+                const float4_t step = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, (float4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0, 127, 0, 127);
+#pragma unroll
+                for (uint32_t v = 0; v < 4u; v++) {
+                    chain[tile][v] = __fmaf_rn(step[v], scale, chain[tile][v]);
+                }
+                continue;
+            }
             const uint32_t scale_a = lds_read<unsigned char>(base + SCALES_AT + (tile / STRIP) * 256u + scale_at[tile % STRIP]);
             if constexpr (BYTES) {
 #pragma unroll
@@ -189,7 +213,9 @@ struct strip_chain {
              * [tile][group of 32 inputs][lane = 4 G + t][16], byte b of a lane: output 16 tile + G + 8 (b % 2), input
              * 32 group + 8 (b / 4) + 2 t + (b / 2) % 2; then one scale code for every 32 outputs x 32 inputs,
              * [ceil(outputs / 32)][inputs / 32]. A step is four groups, 128 pieces of 16 bytes. */
-            const uint32_t scale_rows = (outputs + 31u) / 32u, row0 = tile0 / 2u;
+            /* B128: float32 [outputs / 128][inputs / 128] behind the codes: the strip's row of them, a word a K step (a row
+             * of either kind of scales is inputs / 32 bytes) */
+            const uint32_t scale_rows = (outputs + 31u) / 32u, row0 = B128 ? tile0 / 8u : tile0 / 2u;
 #pragma unroll
             for (uint32_t m = 0; m < MATRICES; m++) {
                 words[m] = matrices[m] + ((uint64_t)tile0 * steps + first) * STEP_BYTES;
@@ -200,7 +226,7 @@ struct strip_chain {
             piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
             /* the scale words of the step: lane L asks for scale row row0 + min(L, rows left) */
             const uint32_t rows_left = scale_rows - 1u - row0;
-            scale_offset = (lane < rows_left ? lane : rows_left) * (inputs / 32u);
+            scale_offset = B128 ? 0u : (lane < rows_left ? lane : rows_left) * (inputs / 32u);
             /* this lane's operand registers 4 L + t: group 2 L + g / 2, piece t of output row G, its half g % 2 */
 #pragma unroll
             for (uint32_t v = 0; v < 8u; v++) {
@@ -262,7 +288,7 @@ struct strip_chain {
                 vector_at[part] = 16u * (8u * column + (piece ^ column)) + 8u * (g / 2u);
             }
         }
-        vector_scale_at = 4u * column + g;
+        vector_scale_at = B128 ? 4u * column : 4u * column + g;
     }
 };
 

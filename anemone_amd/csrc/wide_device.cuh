@@ -14,8 +14,10 @@
 #define WIDE_VECTOR_BYTES (WIDE_TILE_PAIRS * 128u) /* a K step of the tile's columns' codes */
 
 /* One block's pipeline: MATRICES matrices x STRIP tiles a wavefront, the tile's columns shared. */
-template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES, uint32_t DEPTH = WIDE_DEPTH>
+/* B128: float32 scales of 128 x 128 blocks and of 128 values in place of the E8M0 codes, as in strip_device.cuh. */
+template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES, uint32_t DEPTH = WIDE_DEPTH, bool B128 = false>
 struct wide_chain {
+    static_assert(BYTES || !B128, "float32 scales go with one-byte weights");
     static constexpr uint32_t STRIP = STRIP_TILES;
     static constexpr uint32_t STEP_BYTES = BYTES ? BYTE_STEP_BYTES : NIBBLE_STEP_BYTES;
     static constexpr uint32_t TILE_LOADS = STEP_BYTES / 1024u;
@@ -123,16 +125,39 @@ struct wide_chain {
         asm volatile("" : "+v"(b_at), "+v"(b_scale_at));
         int8_vector b[LIVE];
         uint32_t scale_b[LIVE];
+        float float_scale_b[LIVE];
 #pragma unroll
         for (uint32_t j = 0; j < LIVE; j++) {
             const uint4_t low = lds_read<uint4_t>(b_at + VECTOR_AT + j * 2048u), high = lds_read<uint4_t>(b_at + VECTOR_AT + j * 2048u + 1024u);
             b[j] = (int8_vector){(int)low.x, (int)low.y, (int)low.z, (int)low.w, (int)high.x, (int)high.y, (int)high.z, (int)high.w};
-            scale_b[j] = lds_read<unsigned char>(b_scale_at + VECTOR_SCALE_AT + j * 64u);
+            if constexpr (B128) {
+                float_scale_b[j] = lds_read<float>(b_scale_at + VECTOR_SCALE_AT + j * 64u);
+            } else {
+                scale_b[j] = lds_read<unsigned char>(b_scale_at + VECTOR_SCALE_AT + j * 64u);
+            }
         }
         __builtin_amdgcn_s_setprio(1); /* the wavefront that feeds the matrix unit goes first at the issue */
 #pragma unroll
         for (uint32_t tile = 0; tile < TILES; tile++) {
             int8_vector a = {0, 0, 0, 0, 0, 0, 0, 0};
+            if constexpr (B128) {
+                const float float_scale_a = lds_read<float>(mine + SCALES_AT + (tile / STRIP) * 256u);
+#pragma unroll
+                for (uint32_t v = 0; v < 8u; v++) {
+                    const uint2_t w = lds_read<uint2_t>(a_at[v] + tile * STEP_BYTES);
+                    a[v] = (int)__builtin_amdgcn_perm(w.y, w.x, shift);
+                }
+#pragma unroll
+                for (uint32_t j = 0; j < LIVE; j++) {
+                    const float scale = __fmul_rn(float_scale_a, float_scale_b[j]);
+                    const float4_t step = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b[j], (float4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0, 127, 0, 127);
+#pragma unroll
+                    for (uint32_t v = 0; v < 4u; v++) {
+                        chain[tile][j][v] = __fmaf_rn(step[v], scale, chain[tile][j][v]);
+                    }
+                }
+                continue;
+            }
             const uint32_t scale_a = lds_read<unsigned char>(a_scale_at[tile % STRIP] + SCALES_AT + (tile / STRIP) * 256u);
             if constexpr (BYTES) {
 #pragma unroll
@@ -269,7 +294,7 @@ struct wide_chain {
         codes = vector_codes;
         exponents = vector_exponents;
         if constexpr (BYTES) {
-            const uint32_t scale_rows = (outputs + 31u) / 32u, row0 = tile0 / 2u;
+            const uint32_t scale_rows = (outputs + 31u) / 32u, row0 = B128 ? tile0 / 8u : tile0 / 2u;
 #pragma unroll
             for (uint32_t m = 0; m < MATRICES; m++) {
                 words[m] = matrices[m] + (uint64_t)tile0 * steps * STEP_BYTES;
@@ -277,7 +302,7 @@ struct wide_chain {
             }
             piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
             const uint32_t rows_left = scale_rows - 1u - row0;
-            scale_offset = (lane < rows_left ? lane : rows_left) * (inputs / 32u);
+            scale_offset = B128 ? 0u : (lane < rows_left ? lane : rows_left) * (inputs / 32u);
 #pragma unroll
             for (uint32_t v = 0; v < 8u; v++) {
                 const uint32_t group = 2u * (v / 4u) + g / 2u, t = v % 4u;
@@ -330,7 +355,7 @@ struct wide_chain {
                 vector_at[part] = group_bytes + 16u * (8u * column + (piece ^ column ^ (o / 8u))) + 8u * (g / 2u);
             }
         }
-        vector_scale_at = 4u * o + g;
+        vector_scale_at = B128 ? 4u * o : 4u * o + g;
         operand_at = 16u * lane;
     }
 };

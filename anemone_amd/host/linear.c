@@ -78,6 +78,21 @@ result_status linear_kernels_prepare(const struct backend_operations *backend, s
                                              &kernels.expert_down_e4m3[instance]);
         }
     }
+    for (uint32_t instance = 0; status == STATUS_OK && instance < BUILT_INSTANCES; instance++) {
+        char name[48];
+        (void)snprintf(name, sizeof name, "%sb128_%u", KERNEL_EXPERT_GATE_UP_STEM, slice_counts[instance]);
+        status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, name, sizeof(struct expert_gate_up_arguments),
+                                         &kernels.expert_gate_up_b128[instance]);
+        if (status == STATUS_OK) {
+            (void)snprintf(name, sizeof name, "%sb128_%u", KERNEL_EXPERT_DOWN_STEM, slice_counts[instance]);
+            status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, name, sizeof(struct expert_down_arguments),
+                                             &kernels.expert_down_b128[instance]);
+        }
+    }
+    if (status == STATUS_OK) {
+        status = backend->kernel_prepare(card, KERNEL_FILE_ACTIVATION_QUANTIZE, KERNEL_ACTIVATION_QUANTIZE_128,
+                                         sizeof(struct activation_quantize_arguments), &kernels.activation_quantize_128);
+    }
     if (status == STATUS_OK) {
         status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, KERNEL_EXPERT_ROW_SUM,
                                          sizeof(struct expert_row_sum_arguments), &kernels.expert_row_sum);
@@ -159,6 +174,37 @@ result_status linear_quantize_prepare(const struct linear_quantize_description *
     return STATUS_OK;
 }
 
+#define QUANTIZE_128_BLOCK_VALUES (2u * LINEAR_ELEMENT_THREADS) /* a lane of activation_quantize_128_entry takes two values */
+
+result_status linear_quantize_128_prepare(const struct linear_quantize_description *description, uint64_t arena_byte_count,
+                                          const struct linear_kernels_record *kernels, struct kernel_launch *launch_out)
+{
+    static const char what[] = "the activation quantizer of 128 values a scale";
+    if (description == NULL || kernels == NULL || launch_out == NULL || kernels->activation_quantize_128 == BACKEND_NO_KERNEL) {
+        REFUSE("%s: a missing argument or an unprepared kernel", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (description->width == 0 || description->width % 128u != 0 || description->row_count == 0 || description->row_count > 65535u) {
+        REFUSE("%s: a width that is 0 or no multiple of 128, or a row count of 0 or above 65535", what);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint64_t rows = description->row_count, width = description->width;
+    const struct checked_range ranges[] = {
+        {"the values", description->values, linear_values_byte_count(rows, width), false},
+        {"the codes", description->codes, linear_codes_byte_count(rows, width), false},
+        {"the scales", description->exponents, linear_exponents_byte_count(rows, width), false},
+    };
+    if (!ranges_are_valid(what, ranges, 3, arena_byte_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const struct activation_quantize_arguments record = {description->values.byte_offset, description->codes.byte_offset,
+                                                         description->exponents.byte_offset, description->operands.byte_offset,
+                                                         description->width, 0};
+    launch_fill(launch_out, kernels->activation_quantize_128, (description->width + QUANTIZE_128_BLOCK_VALUES - 1u) / QUANTIZE_128_BLOCK_VALUES,
+                description->row_count, 1, LINEAR_ELEMENT_THREADS, 0, &record, sizeof record);
+    return STATUS_OK;
+}
+
 static bool instance_of(uint32_t slice_count, uint32_t input_size, uint32_t *instance_out)
 {
     for (uint32_t instance = 0; instance < BUILT_INSTANCES; instance++) {
@@ -183,7 +229,8 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     const struct weight_format_operations *format = weight_format_operations_of(description->weight_format);
     uint64_t gate_up_bytes = 0, down_bytes = 0;
     uint32_t gate_up_instance = 0, down_instance = 0;
-    const bool bytes = description->weight_format == WEIGHT_FORMAT_E4M3_SCALED;
+    const bool block128 = description->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128;
+    const bool bytes = description->weight_format == WEIGHT_FORMAT_E4M3_SCALED || block128;
     const uint32_t strip_outputs = bytes ? LINEAR_STRIP_OUTPUTS / 2u : LINEAR_STRIP_OUTPUTS;
     if (description->reserved_zero != 0 || (description->weight_format != WEIGHT_FORMAT_E2M1_SCALED && !bytes) || format == NULL ||
         format->stored_byte_count(gate_up, &gate_up_bytes) != STATUS_OK ||
@@ -201,10 +248,16 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
                description->gate_up_slice_count, description->down_slice_count);
         return STATUS_INVALID_ARGUMENT;
     }
-    const uint32_t gate_up_kernel = bytes ? kernels->expert_gate_up_e4m3[gate_up_instance] : kernels->expert_gate_up[gate_up_instance];
-    const uint32_t down_kernel = bytes ? kernels->expert_down_e4m3[down_instance] : kernels->expert_down[down_instance];
+    const uint32_t gate_up_kernel = block128 ? kernels->expert_gate_up_b128[gate_up_instance]
+                                    : bytes  ? kernels->expert_gate_up_e4m3[gate_up_instance]
+                                             : kernels->expert_gate_up[gate_up_instance];
+    const uint32_t down_kernel = block128 ? kernels->expert_down_b128[down_instance]
+                                 : bytes  ? kernels->expert_down_e4m3[down_instance]
+                                          : kernels->expert_down[down_instance];
+    const uint32_t quantize_kernel = block128 ? kernels->activation_quantize_128 : kernels->activation_quantize;
+    const uint32_t quantize_block_values = block128 ? QUANTIZE_128_BLOCK_VALUES : LINEAR_ELEMENT_THREADS;
     if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL ||
-        kernels->activation_quantize == BACKEND_NO_KERNEL || kernels->expert_row_sum == BACKEND_NO_KERNEL) {
+        quantize_kernel == BACKEND_NO_KERNEL || kernels->expert_row_sum == BACKEND_NO_KERNEL) {
         REFUSE("%s: a kernel of the chain is not prepared", what);
         return STATUS_INVALID_ARGUMENT;
     }
@@ -249,8 +302,8 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_GATE_UP], gate_up_kernel,
                 (gate_up->output_size + strip_outputs - 1u) / strip_outputs,
                 description->job_count, 1, 64u * description->gate_up_slice_count, 0, &gate_up_record, sizeof gate_up_record);
-    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_QUANTIZE], kernels->activation_quantize,
-                (gate_up->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, (uint32_t)pairs, 1,
+    launch_fill(&launches[LINEAR_ROUTED_EXPERTS_QUANTIZE], quantize_kernel,
+                (gate_up->output_size + quantize_block_values - 1u) / quantize_block_values, (uint32_t)pairs, 1,
                 LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
     launch_fill(&launches[LINEAR_ROUTED_EXPERTS_DOWN], down_kernel,
                 (down->output_size + strip_outputs - 1u) / strip_outputs, description->job_count, 1, 64u * description->down_slice_count, 0, &down_record, sizeof down_record);
@@ -488,12 +541,15 @@ result_status linear_wide_kernels_prepare(const struct backend_operations *backe
     static const struct {
         const char *name;
         uint32_t record_bytes;
-    } wanted[4] = {{KERNEL_WIDE_EXPERT_GATE_UP_STEM "1", sizeof(struct wide_expert_gate_up_arguments)},
+    } wanted[6] = {{KERNEL_WIDE_EXPERT_GATE_UP_STEM "1", sizeof(struct wide_expert_gate_up_arguments)},
                    {KERNEL_WIDE_EXPERT_DOWN_STEM "1", sizeof(struct wide_expert_down_arguments)},
                    {KERNEL_WIDE_EXPERT_GATE_UP_STEM "e4m3_1", sizeof(struct wide_expert_gate_up_arguments)},
-                   {KERNEL_WIDE_EXPERT_DOWN_STEM "e4m3_1", sizeof(struct wide_expert_down_arguments)}};
-    uint32_t handles[4];
-    for (uint32_t i = 0; i < 4u; i++) {
+                   {KERNEL_WIDE_EXPERT_DOWN_STEM "e4m3_1", sizeof(struct wide_expert_down_arguments)},
+                   {KERNEL_WIDE_EXPERT_GATE_UP_STEM "b128_1", sizeof(struct wide_expert_gate_up_arguments)},
+                   {KERNEL_WIDE_EXPERT_DOWN_STEM "b128_1", sizeof(struct wide_expert_down_arguments)}};
+    uint32_t handles[6];
+    _Static_assert(sizeof(struct linear_wide_kernels_record) == sizeof handles, "a handle a member, in the members' order");
+    for (uint32_t i = 0; i < 6u; i++) {
         const result_status status = backend->kernel_prepare(card, KERNEL_FILE_WIDE_LINEAR, wanted[i].name, wanted[i].record_bytes, &handles[i]);
         if (status != STATUS_OK) {
             REFUSE("the kernels of the wide linear: %s is not prepared: %s", wanted[i].name, status_text(status));
@@ -504,11 +560,14 @@ result_status linear_wide_kernels_prepare(const struct backend_operations *backe
     return STATUS_OK;
 }
 
-result_status linear_wide_experts_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
+/* block128: the launches of WEIGHT_FORMAT_E4M3_BLOCK128 experts (four: the hidden vectors' quantizer is a launch of its
+ * own between the products); else those of the reference's formats (three) */
+static result_status wide_experts_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
                                           const struct linear_kernels_record *linear_kernels,
-                                          const struct linear_wide_kernels_record *kernels, struct kernel_launch *launches_out)
+                                          const struct linear_wide_kernels_record *kernels, bool block128,
+                                          struct kernel_launch *launches_out)
 {
-    static const char what[] = "the wide routed experts";
+    const char *what = block128 ? "the wide routed experts of float32 block scales" : "the wide routed experts";
     if (description == NULL || linear_kernels == NULL || kernels == NULL || launches_out == NULL) {
         REFUSE("%s: a missing argument", what);
         return STATUS_INVALID_ARGUMENT;
@@ -516,7 +575,11 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
     const struct linear_routed_experts_description *experts = &description->experts;
     const struct matrix_shape_record *gate_up = &experts->gate_up_shape, *down = &experts->down_shape;
     const struct weight_format_operations *format = weight_format_operations_of(experts->weight_format);
-    const bool bytes = experts->weight_format == WEIGHT_FORMAT_E4M3_SCALED;
+    if (block128 != (experts->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128)) {
+        REFUSE("%s: a weight format of %u", what, (uint32_t)experts->weight_format);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const bool bytes = experts->weight_format == WEIGHT_FORMAT_E4M3_SCALED || block128;
     const uint32_t strip_outputs = bytes ? LINEAR_STRIP_OUTPUTS / 2u : LINEAR_STRIP_OUTPUTS;
     uint64_t gate_up_bytes = 0, down_bytes = 0;
     if (description->reserved_zero != 0 || experts->reserved_zero != 0 || (experts->weight_format != WEIGHT_FORMAT_E2M1_SCALED && !bytes) ||
@@ -533,9 +596,10 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
                experts->down_slice_count);
         return STATUS_INVALID_ARGUMENT;
     }
-    const uint32_t gate_up_kernel = bytes ? kernels->wide_expert_gate_up_e4m3 : kernels->wide_expert_gate_up;
-    const uint32_t down_kernel = bytes ? kernels->wide_expert_down_e4m3 : kernels->wide_expert_down;
-    if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL || linear_kernels->expert_row_sum == BACKEND_NO_KERNEL) {
+    const uint32_t gate_up_kernel = block128 ? kernels->wide_expert_gate_up_b128 : bytes ? kernels->wide_expert_gate_up_e4m3 : kernels->wide_expert_gate_up;
+    const uint32_t down_kernel = block128 ? kernels->wide_expert_down_b128 : bytes ? kernels->wide_expert_down_e4m3 : kernels->wide_expert_down;
+    if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL || linear_kernels->expert_row_sum == BACKEND_NO_KERNEL ||
+        (block128 && linear_kernels->activation_quantize_128 == BACKEND_NO_KERNEL)) {
         REFUSE("%s: a kernel of the chain is not prepared", what);
         return STATUS_INVALID_ARGUMENT;
     }
@@ -575,15 +639,38 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
                                                             down->output_size, experts->pairs_per_row};
     const uint32_t block_outputs = 4u * strip_outputs;
     const uint32_t gate_up_outputs = bytes ? WIDE_GATE_UP_E4M3_BLOCK_OUTPUTS : WIDE_GATE_UP_BLOCK_OUTPUTS;
-    struct kernel_launch launches[LINEAR_WIDE_EXPERTS_LAUNCH_COUNT];
-    launch_fill(&launches[LINEAR_WIDE_EXPERTS_GATE_UP], gate_up_kernel,
+    struct kernel_launch launches[LINEAR_WIDE_EXPERTS_BLOCK128_LAUNCH_COUNT];
+    uint32_t at = 0;
+    launch_fill(&launches[at++], gate_up_kernel,
                 (gate_up->output_size + gate_up_outputs - 1u) / gate_up_outputs, description->tile_count, 1,
                 WIDE_BLOCK_THREADS, bytes ? WIDE_GATE_UP_E4M3_WINDOW_BYTES : WIDE_GATE_UP_WINDOW_BYTES, &gate_up_record, sizeof gate_up_record);
-    launch_fill(&launches[LINEAR_WIDE_EXPERTS_DOWN], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
+    if (block128) { /* the hidden values, which the gate/up launch left where the operands go, to their codes and scales */
+        const struct activation_quantize_arguments quantize_record = {
+            experts->hidden_operands.byte_offset, experts->hidden_codes.byte_offset, experts->hidden_exponents.byte_offset,
+            experts->hidden_operands.byte_offset, gate_up->output_size, 0};
+        launch_fill(&launches[at++], linear_kernels->activation_quantize_128,
+                    (gate_up->output_size + QUANTIZE_128_BLOCK_VALUES - 1u) / QUANTIZE_128_BLOCK_VALUES, (uint32_t)pairs, 1,
+                    LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
+    }
+    launch_fill(&launches[at++], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
                 description->tile_count, 1, WIDE_BLOCK_THREADS, bytes ? WIDE_DOWN_E4M3_WINDOW_BYTES : WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);
-    launch_fill(&launches[LINEAR_WIDE_EXPERTS_ROW_SUM], linear_kernels->expert_row_sum,
+    launch_fill(&launches[at++], linear_kernels->expert_row_sum,
                 (down->output_size + ROW_SUM_BLOCK_OUTPUTS - 1u) / ROW_SUM_BLOCK_OUTPUTS, (uint32_t)rows, 1, LINEAR_ELEMENT_THREADS, 0,
                 &row_sum_record, sizeof row_sum_record);
-    memcpy(launches_out, launches, sizeof launches);
+    memcpy(launches_out, launches, at * sizeof launches[0]);
     return STATUS_OK;
+}
+
+result_status linear_wide_experts_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
+                                          const struct linear_kernels_record *linear_kernels,
+                                          const struct linear_wide_kernels_record *kernels, struct kernel_launch *launches_out)
+{
+    return wide_experts_prepare(description, arena_byte_count, linear_kernels, kernels, false, launches_out);
+}
+
+result_status linear_wide_experts_block128_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
+                                                   const struct linear_kernels_record *linear_kernels,
+                                                   const struct linear_wide_kernels_record *kernels, struct kernel_launch *launches_out)
+{
+    return wide_experts_prepare(description, arena_byte_count, linear_kernels, kernels, true, launches_out);
 }

@@ -1,7 +1,7 @@
 /*
  * weight_format.c -- how many bytes a matrix of a shape occupies, per format, exactly as the kernels read it.
  * Byte counts follow include/anemone/weight_format_seam.h:22-46 (E2M1_SCALED, E4M3_SCALED) and
- * include/anemone/exl3_records.h:2-9 with source/exl3.c:10-37 (EXL3) of the reference.
+ * include/anemone/exl3_records.h:2-9 with source/exl3.c:10-37 (EXL3) of the reference; E4M3_BLOCK128 is this build's own.
  */
 #include "anemone_ops.h"
 
@@ -31,6 +31,16 @@ static result_status e4m3_bytes(const struct matrix_shape_record *shape, uint64_
     return STATUS_OK;
 }
 
+static result_status e4m3_block128_bytes(const struct matrix_shape_record *shape, uint64_t *out)
+{
+    if (shape == NULL || out == NULL || shape->reserved_must_be_zero != 0 || shape->bits_per_weight != 8 ||
+        shape->output_size == 0 || shape->input_size == 0 || shape->output_size % 128u != 0 || shape->input_size % 128u != 0) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    *out = (uint64_t)shape->output_size * shape->input_size + (uint64_t)(shape->output_size / 128u) * (shape->input_size / 128u) * 4u;
+    return STATUS_OK;
+}
+
 static result_status exl3_bytes(const struct matrix_shape_record *shape, uint64_t *out)
 {
     /* whole 128-wide transforms on both sides; a width the format defines but this build has no kernels for is
@@ -50,6 +60,7 @@ static result_status exl3_bytes(const struct matrix_shape_record *shape, uint64_
 
 static const struct weight_format_operations e2m1_operations = {"e2m1_scaled", e2m1_bytes};
 static const struct weight_format_operations e4m3_operations = {"e4m3_scaled", e4m3_bytes};
+static const struct weight_format_operations e4m3_block128_operations = {"e4m3_block128", e4m3_block128_bytes};
 const struct weight_format_operations exl3_weight_operations = {"exl3", exl3_bytes};
 
 const struct weight_format_operations *weight_format_operations_of(enum weight_format_code format)
@@ -58,6 +69,7 @@ const struct weight_format_operations *weight_format_operations_of(enum weight_f
     case WEIGHT_FORMAT_E2M1_SCALED: return &e2m1_operations;
     case WEIGHT_FORMAT_E4M3_SCALED: return &e4m3_operations;
     case WEIGHT_FORMAT_EXL3: return &exl3_weight_operations;
+    case WEIGHT_FORMAT_E4M3_BLOCK128: return &e4m3_block128_operations;
     default: return NULL;
     }
 }

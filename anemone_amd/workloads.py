@@ -146,6 +146,18 @@ def fp8_matrix(seed, outputs, inputs, deviation=0.02):
     return e4m3_lay_out(codes, (exponents + 127).astype(np.uint8))
 
 
+def fp8_block128_matrix(seed, outputs, inputs, deviation=0.02):
+    """Weights N(0, deviation) as WEIGHT_FORMAT_E4M3_BLOCK128 stores them: for every 128 x 128 block one float32 scale,
+    the block's largest magnitude over 448, and the nearest E4M3 code of each weight over it (a float32 division); the
+    codes in WEIGHT_FORMAT_E4M3_SCALED's lane order, the scales float32 [outputs / 128][inputs / 128] behind them."""
+    assert outputs % 128 == 0 and inputs % 128 == 0
+    weights = (normals(seed, outputs * inputs).reshape(outputs // 128, 128, inputs // 128, 128) * deviation).astype(np.float32)
+    scales = (np.maximum(np.abs(weights).max(axis=(1, 3)), np.float32(1e-30)) / np.float32(448.0)).astype(np.float32)
+    scaled = (weights / scales[:, None, :, None]).astype(np.float32)
+    codes = e4m3_nearest(scaled.astype(np.float64)).reshape(outputs, inputs)
+    return e4m3_lay_out(codes, scales.view(np.uint8))
+
+
 def fp4_moe_layer(config, hidden, inner, expert_count):
     base = SEED + (config << 20)
     matrices = [[fp4_matrix(base + 16 + 3 * e + 0, inner, hidden), fp4_matrix(base + 16 + 3 * e + 1, inner, hidden),

@@ -48,7 +48,11 @@ enum weight_format_code {
     WEIGHT_FORMAT_E2M1_SCALED = 3,
     WEIGHT_FORMAT_INT4_SCALED = 4,
     WEIGHT_FORMAT_E4M3_SCALED = 5,
-    WEIGHT_FORMAT_COUNT = 6
+    WEIGHT_FORMAT_COUNT = 6, /* the reference's formats end here */
+    /* extension, no counterpart in the reference: E4M3 codes in E4M3_SCALED's lane order [out/16][in/32][lane][16], then
+     * one float32 scale for every 128 outputs x 128 inputs, [out/128][in/128]; its vectors are quantized 128 values a
+     * float32 scale */
+    WEIGHT_FORMAT_E4M3_BLOCK128 = 6
 };
 
 #define BACKEND_MAXIMUM_CARDS 16

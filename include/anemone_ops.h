@@ -213,6 +213,10 @@ struct linear_kernels_record { /* include/anemone/linear.h:121-132 of the refere
      * for experts of WEIGHT_FORMAT_E4M3_SCALED */
     uint32_t expert_gate_up_e4m3[LINEAR_SLICE_INSTANCES];
     uint32_t expert_down_e4m3[LINEAR_SLICE_INSTANCES];
+    /* extension: experts of WEIGHT_FORMAT_E4M3_BLOCK128 and the quantizer of their vectors (128 values a float32 scale) */
+    uint32_t expert_gate_up_b128[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_down_b128[LINEAR_SLICE_INSTANCES];
+    uint32_t activation_quantize_128;
 };
 MUST_CHECK result_status linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                 uint32_t arithmetic_class, struct linear_kernels_record *kernels_out);
@@ -244,6 +248,14 @@ MUST_CHECK result_status linear_quantize_prepare(const struct linear_quantize_de
                                                  const struct linear_kernels_record *kernels,
                                                  struct kernel_launch *launch_out);
 
+/* The same for the vectors of WEIGHT_FORMAT_E4M3_BLOCK128 matrices (no counterpart in the reference): one launch of
+ * activation_quantize_128_entry. `exponents` receives the float32 scales [row_count][width / 128] (the same bytes);
+ * `operands` is not written and may be empty; width a multiple of 128. */
+MUST_CHECK result_status linear_quantize_128_prepare(const struct linear_quantize_description *description,
+                                                     uint64_t arena_byte_count,
+                                                     const struct linear_kernels_record *kernels,
+                                                     struct kernel_launch *launch_out);
+
 enum linear_routed_experts_launch {
     LINEAR_ROUTED_EXPERTS_GATE_UP = 0,  /* expert_gate_up_<S>: jobs and the rows' arrays to hidden */
     LINEAR_ROUTED_EXPERTS_QUANTIZE = 1, /* activation_quantize_entry: hidden of every pair to its arrays */
@@ -251,7 +263,9 @@ enum linear_routed_experts_launch {
     LINEAR_ROUTED_EXPERTS_ROW_SUM = 3,  /* expert_row_sum_entry: pair_output to row_output */
     LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT = 4
 };
-/* launches_out: LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT launches; weight_format E2M1_SCALED */
+/* launches_out: LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT launches; weight_format E2M1_SCALED, or (extensions) E4M3_SCALED or
+ * E4M3_BLOCK128: the latter's exponent ranges hold float32 scales of 128 values (the same bytes), its quantizer launch
+ * is activation_quantize_128_entry, its shapes are multiples of 128 */
 MUST_CHECK result_status linear_routed_experts_prepare(const struct linear_routed_experts_description *description,
                                                        uint64_t arena_byte_count,
                                                        const struct linear_kernels_record *kernels,
@@ -385,6 +399,8 @@ struct linear_wide_kernels_record {
     uint32_t wide_expert_down;
     uint32_t wide_expert_gate_up_e4m3; /* extension: experts of WEIGHT_FORMAT_E4M3_SCALED */
     uint32_t wide_expert_down_e4m3;
+    uint32_t wide_expert_gate_up_b128; /* extension: experts of WEIGHT_FORMAT_E4M3_BLOCK128 */
+    uint32_t wide_expert_down_b128;
 };
 MUST_CHECK result_status linear_wide_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                      uint32_t arithmetic_class, struct linear_wide_kernels_record *kernels_out);
@@ -405,6 +421,16 @@ MUST_CHECK result_status linear_wide_experts_prepare(const struct linear_wide_ex
                                                      uint64_t arena_byte_count, const struct linear_kernels_record *linear_kernels,
                                                      const struct linear_wide_kernels_record *kernels,
                                                      struct kernel_launch *launches_out);
+
+/* The wide form of WEIGHT_FORMAT_E4M3_BLOCK128 experts (no counterpart in the reference): four launches, the gate/up
+ * product (which leaves the hidden VALUES where hidden_operands names: the same bytes), activation_quantize_128_entry of
+ * them (codes and float32 scales), the down product, the row sum. Refusals as linear_wide_experts_prepare's, which
+ * refuses this format as this function refuses the others. */
+enum { LINEAR_WIDE_EXPERTS_BLOCK128_LAUNCH_COUNT = 4 };
+MUST_CHECK result_status linear_wide_experts_block128_prepare(const struct linear_wide_experts_description *description,
+                                                              uint64_t arena_byte_count, const struct linear_kernels_record *linear_kernels,
+                                                              const struct linear_wide_kernels_record *kernels,
+                                                              struct kernel_launch *launches_out);
 
 uint64_t linear_values_byte_count(uint64_t vector_count, uint64_t width);    /* bfloat16 [vector][width] */
 uint64_t linear_codes_byte_count(uint64_t vector_count, uint64_t width);     /* E4M3 [vector][width] */

@@ -421,6 +421,7 @@ ANEMONE_INLINE struct exl3_tcp_layout exl3_tcp_layout_of(uint64_t rows, uint64_t
 #define KERNEL_FILE_ACTIVATION_QUANTIZE "kernel_activation_quantize"
 #define KERNEL_FILE_EXPERT_LINEAR "kernel_expert_linear"
 #define KERNEL_ACTIVATION_QUANTIZE "activation_quantize_entry"
+#define KERNEL_ACTIVATION_QUANTIZE_128 "activation_quantize_128_entry" /* no counterpart in the reference: 128 values a float32 scale */
 #define KERNEL_EXPERT_GATE_UP_STEM "expert_gate_up_"
 #define KERNEL_EXPERT_DOWN_STEM "expert_down_"
 #define KERNEL_EXPERT_ROW_SUM "expert_row_sum_entry"

@@ -25,6 +25,9 @@ static int shape_is_stored(int format, uint32_t outputs, uint32_t inputs)
     if (format == ORC_FORMAT_E4M3_SCALED) {
         return inputs % 32u == 0u;
     }
+    if (format == ORC_FORMAT_E4M3_BLOCK128) {
+        return inputs % 128u == 0u && outputs % 128u == 0u;
+    }
     return 0;
 }
 
@@ -32,6 +35,9 @@ uint64_t orc_linear_scale_count(int format, uint32_t outputs, uint32_t inputs)
 {
     if (format == ORC_FORMAT_E2M1_SCALED) {
         return (uint64_t)outputs * (inputs / BLOCK);
+    }
+    if (format == ORC_FORMAT_E4M3_BLOCK128) {
+        return (uint64_t)(outputs / 128u) * (inputs / 128u) * 4u; /* float32 scales, counted in bytes */
     }
     return (uint64_t)((outputs + 31u) / 32u) * (inputs / BLOCK);
 }
@@ -133,6 +139,10 @@ int orc_linear_read(int format, uint32_t outputs, uint32_t inputs, const uint8_t
     const uint32_t t = (within % 8u) / 2u;
     const uint32_t b = 4u * (within / 8u) + 2u * (within % 2u) + far_output;
     *code_out = stored[(((uint64_t)tile * groups + group) * 32u + 4u * g + t) * 16u + b];
+    if (format == ORC_FORMAT_E4M3_BLOCK128) { /* the float32 scale of the weight's 128 x 128 block, as its bits */
+        memcpy(scale_out, stored + (uint64_t)outputs * inputs + ((uint64_t)(output / 128u) * (inputs / 128u) + input / 128u) * 4u, 4u);
+        return 0;
+    }
     *scale_out = stored[(uint64_t)outputs * inputs + (uint64_t)(output / 32u) * groups + group];
     return 0;
 }
@@ -279,6 +289,49 @@ int orc_linear_products(int format, uint32_t outputs, uint32_t inputs, const uin
     return 0;
 }
 
+int orc_linear_products_128(uint32_t outputs, uint32_t inputs, const uint8_t *stored, uint32_t first, uint32_t count,
+                            const uint8_t *fed_codes, const float *fed_scales, uint32_t vectors, double *sums_out,
+                            double *magnitude_out)
+{
+    const int format = ORC_FORMAT_E4M3_BLOCK128;
+    if (!shape_is_stored(format, outputs, inputs) || first + count > outputs) {
+        return -1;
+    }
+    const uint32_t blocks = inputs / 128u;
+    float *values = malloc((size_t)inputs * sizeof *values), *scales = malloc((size_t)blocks * sizeof *scales);
+    for (uint32_t o = first; o < first + count; o++) {
+        for (uint32_t input = 0; input < inputs; input++) {
+            uint32_t code, scale;
+            (void)orc_linear_read(format, outputs, inputs, stored, o, input, &code, &scale);
+            values[input] = (float)orc_e4m3_value(code);
+            if (input % 128u == 0u) {
+                scales[input / 128u] = orc_f32_from_bits(scale);
+            }
+        }
+        for (uint32_t v = 0; v < vectors; v++) {
+            double sum = 0.0, magnitude = 0.0;
+            for (uint32_t block = 0; block < blocks; block++) {
+                double block_sum = 0.0, block_magnitude = 0.0; /* exact */
+                for (uint32_t i = 0; i < 128u; i++) {
+                    const double product = (double)values[block * 128u + i] * orc_e4m3_value(fed_codes[(uint64_t)v * inputs + block * 128u + i]);
+                    block_sum += product;
+                    block_magnitude += fabs(product);
+                }
+                const double w_scale = (double)scales[block], a_scale = (double)fed_scales[(uint64_t)v * blocks + block];
+                sum += block_sum * w_scale * a_scale;
+                magnitude += block_magnitude * fabs(w_scale) * fabs(a_scale);
+            }
+            sums_out[(uint64_t)v * count + (o - first)] = sum;
+            if (magnitude_out != NULL) {
+                magnitude_out[(uint64_t)v * count + (o - first)] = magnitude;
+            }
+        }
+    }
+    free(values);
+    free(scales);
+    return 0;
+}
+
 static double bf16_last_place(uint16_t bits)
 {
     const int exponent = (int)((bits >> 7) & 255u);
@@ -404,6 +457,27 @@ struct linear_layer {
     pthread_mutex_t lock;
 };
 
+/* the quantizer and the product of the layer's format: E8M0 scale codes a 32 values, or float32 scales a 128 (the
+ * scale arrays have the same bytes either way: width / 32 a vector) */
+static void layer_quantize(int format, const uint16_t *values, uint32_t width, uint8_t *codes, uint8_t *scales)
+{
+    if (format == ORC_FORMAT_E4M3_BLOCK128) {
+        orc_act_quantize_128(values, width, codes, (float *)(void *)scales);
+    } else {
+        (void)orc_act_quantize(values, width, codes, scales);
+    }
+}
+
+static void layer_products(int format, uint32_t outputs, uint32_t inputs, const uint8_t *stored, const uint8_t *codes,
+                           const uint8_t *scales, uint32_t vectors, double *sums)
+{
+    if (format == ORC_FORMAT_E4M3_BLOCK128) {
+        (void)orc_linear_products_128(outputs, inputs, stored, 0, outputs, codes, (const float *)(const void *)scales, vectors, sums, NULL);
+    } else {
+        (void)orc_linear_products(format, outputs, inputs, stored, 0, outputs, codes, scales, vectors, sums, NULL);
+    }
+}
+
 static void linear_expert(struct linear_layer *layer, uint32_t expert)
 {
     const uint32_t H = layer->hidden, I = layer->inner, total = layer->rows * layer->picks;
@@ -426,8 +500,8 @@ static void linear_expert(struct linear_layer *layer, uint32_t expert)
         memcpy(codes + (uint64_t)c * H, layer->x_codes + (uint64_t)row * H, H);
         memcpy(exponents + (uint64_t)c * (H / BLOCK), layer->x_exponents + (uint64_t)row * (H / BLOCK), H / BLOCK);
     }
-    (void)orc_linear_products(layer->format, I, H, layer->matrices[expert * 3u + 0u], 0, I, codes, exponents, count, gate, NULL);
-    (void)orc_linear_products(layer->format, I, H, layer->matrices[expert * 3u + 1u], 0, I, codes, exponents, count, up, NULL);
+    layer_products(layer->format, I, H, layer->matrices[expert * 3u + 0u], codes, exponents, count, gate);
+    layer_products(layer->format, I, H, layer->matrices[expert * 3u + 1u], codes, exponents, count, up);
     for (uint32_t c = 0; c < count; c++) {
         for (uint32_t i = 0; i < I; i++) {
             /* the products are rounded once to bfloat16, then the hidden step in float32 */
@@ -438,9 +512,9 @@ static void linear_expert(struct linear_layer *layer, uint32_t expert)
         if (layer->hidden_out != NULL) {
             memcpy(layer->hidden_out + (uint64_t)pairs[c] * I, hidden + (uint64_t)c * I, I * sizeof(uint16_t));
         }
-        (void)orc_act_quantize(hidden + (uint64_t)c * I, I, codes + (uint64_t)c * I, exponents + (uint64_t)c * (I / BLOCK));
+        layer_quantize(layer->format, hidden + (uint64_t)c * I, I, codes + (uint64_t)c * I, exponents + (uint64_t)c * (I / BLOCK));
     }
-    (void)orc_linear_products(layer->format, H, I, layer->matrices[expert * 3u + 2u], 0, H, codes, exponents, count, down, NULL);
+    layer_products(layer->format, H, I, layer->matrices[expert * 3u + 2u], codes, exponents, count, down);
     for (uint32_t c = 0; c < count; c++) {
         for (uint32_t i = 0; i < H; i++) {
             layer->pair_out[(uint64_t)pairs[c] * H + i] = orc_bf16_from_float((float)down[(uint64_t)c * H + i]);
@@ -488,8 +562,8 @@ void orc_linear_moe_layer(int format, const uint16_t *x_bf16, uint32_t rows, uin
     layer.x_codes = malloc((size_t)rows * hidden);
     layer.x_exponents = malloc((size_t)rows * hidden / BLOCK);
     for (uint32_t row = 0; row < rows; row++) {
-        (void)orc_act_quantize(x_bf16 + (uint64_t)row * hidden, hidden, layer.x_codes + (uint64_t)row * hidden,
-                               layer.x_exponents + (uint64_t)row * (hidden / BLOCK));
+        layer_quantize(format, x_bf16 + (uint64_t)row * hidden, hidden, layer.x_codes + (uint64_t)row * hidden,
+                       layer.x_exponents + (uint64_t)row * (hidden / BLOCK));
     }
     pthread_mutex_init(&layer.lock, NULL);
     threads = threads < 1u ? 1u : (threads > 64u ? 64u : threads);

@@ -30,6 +30,8 @@
 
 #define ORC_FORMAT_E2M1_SCALED 3 /* enum weight_format_code values of the reference */
 #define ORC_FORMAT_E4M3_SCALED 5
+#define ORC_FORMAT_E4M3_BLOCK128 6 /* no reference counterpart: E4M3 codes in E4M3_SCALED's lane order, then one float32
+                                    * scale for every 128 outputs x 128 inputs, [outputs / 128][inputs / 128] */
 
 uint64_t orc_linear_stored_bytes(int format, uint32_t outputs, uint32_t inputs);
 uint64_t orc_linear_scale_count(int format, uint32_t outputs, uint32_t inputs);
@@ -75,8 +77,14 @@ void orc_act_quantize_128(const uint16_t *values_bf16, uint32_t width, uint8_t *
 void orc_fp8_block128_products(uint32_t outputs, uint32_t inputs, const uint8_t *w_codes, const float *w_scales,
                                const uint8_t *a_codes, const float *a_scales, uint32_t vectors, double *sums_out);
 
+/* the same for a matrix stored as ORC_FORMAT_E4M3_BLOCK128 and vectors quantized by orc_act_quantize_128
+ * (fed_scales float32 [vectors][inputs / 128]): blocks of 128 inputs; any first and count */
+int orc_linear_products_128(uint32_t outputs, uint32_t inputs, const uint8_t *stored, uint32_t first, uint32_t count,
+                            const uint8_t *fed_codes, const float *fed_scales, uint32_t vectors, double *sums_out,
+                            double *magnitude_out);
+
 /* One whole FP4/FP8 routed-expert layer (formats of the reference, per-32 scales), double-precision products with
- * the kernels' rounding points: quantize x per row, gate/up products -> bf16, hidden step -> bf16, quantize the
+ * the kernels' rounding points (format 6: float32 scales per 128, quantizer orc_act_quantize_128): quantize x per row, gate/up products -> bf16, hidden step -> bf16, quantize the
  * hidden vector, down product -> bf16 pair output, float32 row sum. matrices [expert_count][3] stored pointers. */
 void orc_linear_moe_layer(int format, const uint16_t *x_bf16, uint32_t rows, uint32_t hidden, uint32_t inner,
                           uint32_t picks, const uint32_t *experts, const float *weights, uint32_t expert_count,

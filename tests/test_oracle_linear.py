@@ -187,6 +187,37 @@ def test_block128_mode_against_numpy():
     assert np.allclose(sums, xq @ wq.T, rtol=1e-11)
 
 
+def test_block128_stored_format_against_the_plain_arrays():
+    """Format 6 (codes in E4M3_SCALED's lane order, float32 scales behind them): laid out and read back, and its
+    products equal the products of the plain row-major arrays, which numpy pins above."""
+    B128 = 6
+    outputs, inputs, vectors = 256, 384, 3
+    rng = np.random.default_rng(3)
+    w_codes = rng.integers(0, 256, size=(outputs, inputs)).astype(np.uint8)
+    w_codes[(w_codes & 0x7F) == 0x7F] = 0x7E
+    w_scales = (rng.random((outputs // 128, inputs // 128)) * 1e-3 + 1e-5).astype(np.float32)
+    assert orc.orc_linear_stored_bytes(B128, outputs, inputs) == outputs * inputs + w_scales.nbytes
+    stored = np.zeros(outputs * inputs + w_scales.nbytes, dtype=np.uint8)
+    assert orc.orc_linear_lay_out(B128, outputs, inputs, ptr(w_codes, u8p), ptr(w_scales.view(np.uint8).reshape(-1), u8p), ptr(stored, u8p)) == 0
+    assert orc.orc_linear_lay_out(B128, 192, 384, ptr(w_codes, u8p), ptr(w_scales.view(np.uint8).reshape(-1), u8p), ptr(stored, u8p)) == -1
+    same = np.zeros(outputs * inputs + outputs // 32 * (inputs // 32), dtype=np.uint8)  # the codes lie as E4M3_SCALED lays them
+    assert orc.orc_linear_lay_out(E4M3, outputs, inputs, ptr(w_codes, u8p), ptr(np.zeros(outputs // 32 * inputs // 32, dtype=np.uint8), u8p), ptr(same, u8p)) == 0
+    assert np.array_equal(stored[:outputs * inputs], same[:outputs * inputs])
+    code, scale = C.c_uint32(0), C.c_uint32(0)
+    for o, i in ((0, 0), (130, 5), (255, 383), (127, 128), (128, 127)):
+        assert orc.orc_linear_read(B128, outputs, inputs, ptr(stored, u8p), o, i, C.byref(code), C.byref(scale)) == 0
+        assert code.value == w_codes[o, i] and scale.value == w_scales[o // 128, i // 128].view(np.uint32)
+    x = to_bf16(normals(12, vectors * inputs) * 3.0).reshape(vectors, inputs)
+    a_codes, a_scales = np.zeros((vectors, inputs), dtype=np.uint8), np.zeros((vectors, inputs // 128), dtype=np.float32)
+    for v in range(vectors):
+        orc.orc_act_quantize_128(ptr(x[v], u16p), inputs, ptr(a_codes[v], u8p), ptr(a_scales[v], f32p))
+    want, got, mags = np.zeros((vectors, outputs)), np.zeros((vectors, outputs)), np.zeros((vectors, outputs))
+    orc.orc_fp8_block128_products(outputs, inputs, ptr(w_codes, u8p), ptr(w_scales, f32p), ptr(a_codes, u8p), ptr(a_scales, f32p), vectors, ptr(want, f64p))
+    assert orc.orc_linear_products_128(outputs, inputs, ptr(stored, u8p), 0, outputs, ptr(a_codes, u8p), ptr(a_scales, f32p), vectors,
+                                       ptr(got, f64p), ptr(mags, f64p)) == 0
+    assert np.array_equal(got, want) and np.all(mags >= np.abs(got))
+
+
 def test_layer_runs_and_matches_dequantised_matmul():
     rows, hidden, inner, picks, experts_n = 2, 128, 64, 2, 3
     mats, dense = [], []
