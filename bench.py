@@ -35,6 +35,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("fp4_prefill", 8192): 5044.9e6 + 443.2e6,  # profiles/wide_expert_fp4_fp8_prefill.md
     ("fp8_prefill", 2048): 5642.4e6 + 117.0e6,
     ("expert_join", 8192): 877.7e6 + 402.7e6,  # profiles/expert_join_trunk_linear_ffn_site.md
+    ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,  # profiles/expert_b128_fp8_block128_decode64_prefill2048.md
+    ("fp8_prefill_block128", 2048): 5707.3e6 + 67.2e6,
 }
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
 CONFIG = 1
@@ -103,7 +105,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     rows = arguments.rows if not prefill or arguments.rows != 32 else 2048 if fp8 else 8192
     distinct_generated = 4 if fp8 else 16
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
-    matrix = workloads.fp8_matrix if fp8 else workloads.fp4_matrix
+    block128 = fp8 and arguments.block128  # float32 scales of 128 x 128 blocks and of 128 values: BASELINE config 3's wording
+    matrix = workloads.fp8_block128_matrix if block128 else workloads.fp8_matrix if fp8 else workloads.fp4_matrix
     trios = [[matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
               matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
     matrices = [trios[e % distinct_generated] for e in range(EXPERTS)]
@@ -112,7 +115,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     card = amd.Card(((9 if fp8 else 5) << 30) + rows * (1 << 18))
     layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router,
                          gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices,
-                         weight_format=amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED)
+                         weight_format=amd.WEIGHT_FORMAT_E4M3_BLOCK128 if block128 else amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else
+                         amd.WEIGHT_FORMAT_E2M1_SCALED)
     layer.set_rows(x, rows)
     wide = layer.wide_router() if rows > 8 or prefill else None  # more than eight rows: the wide select sorts the pairs by expert
     small = wide is not None and rows <= amd.ROUTER_SORT_ROWS and not prefill  # count, place and jobs in one block
@@ -122,14 +126,17 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     if prefill:
         routing, routing_names = routing[:3], routing_names[:3]  # the tiles are the place's; no job table
         experts = layer.wide_expert_launches(wide)
-        parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(3)]
-        names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "expert_down", "expert_row_sum_entry"]
+        parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(len(experts))]
+        names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up"] + \
+            (["activation_quantize(hidden)"] if block128 else []) + ["expert_down", "expert_row_sum_entry"]
     else:
         experts = layer.expert_launches(wide)
         parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(4)]
         names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
                                                          "expert_down", "expert_row_sum_entry"]
     shared = None
+    if arguments.site and block128:
+        raise SystemExit("--site takes the reference's scaling: the shared expert's kernels read E8M0 scales of 32 values")
     if arguments.site:
         # the whole FFN site: the shared expert (three E4M3 matrices applied to every row) and the join in place of the
         # row sum (a row's routed sum, which it also stores, the shared output added, the post of the four streams)
@@ -178,7 +185,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         jobs = layer.jobs() if wide is None else wide.read("jobs", amd.JOB_DTYPE)
         live = jobs[jobs["row_count"] > 0]
         distinct = np.unique(live["expert"])
-    matrix_bytes = HIDDEN * INNER + HIDDEN * INNER // 1024 if fp8 else HIDDEN * INNER // 2 + HIDDEN * INNER // 32
+    matrix_bytes = HIDDEN * INNER + HIDDEN * INNER // 16384 * 4 if block128 else HIDDEN * INNER + HIDDEN * INNER // 1024 if fp8 else \
+        HIDDEN * INNER // 2 + HIDDEN * INNER // 32
     gate_up_bytes = 2 * matrix_bytes * len(distinct)
     gate_up_us = float(per_launch[names.index("expert_gate_up")])
     down_us = float(per_launch[names.index("expert_down")])
@@ -193,7 +201,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                    "distinct_experts": int(len(distinct)), "jobs": int(len(live)),
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "down_GBps": matrix_bytes * len(distinct) / (down_us * 1e-6) / 1e9},
-        "roofline": {"bound": "hbm", "kernel": "expert_gate_up_%s%d" % ("e4m3_" if fp8 else "", arguments.gate_up_slices),
+        "roofline": {"bound": "hbm", "kernel": "expert_gate_up_%s%d" % ("b128_" if block128 else "e4m3_" if fp8 else "", arguments.gate_up_slices),
                      "achieved": gate_up_bytes / (gate_up_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
@@ -214,6 +222,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
             "trunk_gate_up_us": trunk_us, "trunk_gate_up_GBps": 2 * shared_matrix_bytes / (trunk_us * 1e-6) / 1e9,
             "trunk_gate_up_TFLOPs": 2.0 * rows * 2 * HIDDEN * INNER / (trunk_us * 1e-6) / 1e12}
     key = ("%s_%s" % ("fp8" if fp8 else "fp4", "prefill" if prefill else "decode"), rows)
+    if block128:
+        key = (key[0] + "_block128", rows)
     if key in MEASURED_TRAFFIC_BYTES and (prefill or (arguments.gate_up_slices, arguments.down_slices) == (4, 2)):
         result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES[key]
     if prefill:
@@ -227,7 +237,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         result["config"]["step_TFLOPs"] = (gate_up_flops + down_flops) / (seconds / arguments.steps) / 1e12
         # the products are MFMAs of FP8 activations (with FP4 or FP8 weights): the FP8 rate is the instruction's peak.
         # What bounds the launch is read off its arithmetic intensity against the card's balance of the two peaks.
-        kernel = "wide_expert_gate_up_%s1" % ("e4m3_" if fp8 else "")
+        kernel = "wide_expert_gate_up_%s1" % ("b128_" if block128 else "e4m3_" if fp8 else "")
         if gate_up_flops / gate_up_bytes >= MFMA_F8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
             result["roofline"] = {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_F8_PEAK_TFLOPS, "unit": "TFLOP/s",
                                   "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": result["roofline"]["traffic"],
@@ -253,7 +263,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         want = np.zeros((sample, HIDDEN), dtype=np.float32)
         want_pairs = np.zeros((sample * PICKS, HIDDEN), dtype=np.uint16)
         start = time.perf_counter()
-        o.orc.orc_linear_moe_layer(5 if fp8 else 3, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS,
+        o.orc.orc_linear_moe_layer(6 if block128 else 5 if fp8 else 3, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS,
                                    o.ptr(np.ascontiguousarray(experts_of[:sample]), o.u32p),
                                    o.ptr(np.ascontiguousarray(weights_of[:sample]), o.f32p), EXPERTS, pointers, 10.0,
                                    o.ptr(want, o.f32p), None, o.ptr(want_pairs, o.u16p), threads)
@@ -388,6 +398,8 @@ def main():
     parser.add_argument("--gate-up-slices", type=int, default=4)
     parser.add_argument("--down-slices", type=int, default=2)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--block128", action="store_true",
+                        help="fp8 workloads: float32 scales of 128 x 128 weight blocks and of 128 activation values in place of the reference's E8M0 scales")
     parser.add_argument("--site", action="store_true",
                         help="fp4/fp8 workloads: the whole FFN site, with the shared expert and the join in place of the row sum")
     parser.add_argument("--graph", action="store_true", help="time replays of the step captured as one graph (graph_capture / graph_run)")

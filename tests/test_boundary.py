@@ -386,7 +386,7 @@ def test_tcp_prepare_geometry_and_refusals(fake):
 def experts_description(fmt=amd.WEIGHT_FORMAT_E2M1_SCALED, **changes):
     rows, P, H, I = 8, 8, 4096, 2048
     pairs = rows * P
-    bits = 8 if fmt == amd.WEIGHT_FORMAT_E4M3_SCALED else 4
+    bits = 8 if fmt in (amd.WEIGHT_FORMAT_E4M3_SCALED, amd.WEIGHT_FORMAT_E4M3_BLOCK128) else 4
     d = amd.RoutedExpertsDescription()
     cursor = [4096]
 
@@ -651,3 +651,52 @@ def test_join_prepare_geometry_and_refusals(fake):
     assert lib.expert_shared_join_prepare(C.byref(s), arena, C.byref(linear), C.byref(kernels), untouched) == 1 and not any(bytes(untouched))
     s.join = join_description(width=5120)
     assert lib.expert_shared_join_prepare(C.byref(s), arena, C.byref(linear), C.byref(kernels), untouched) == 1  # down has 4,096 outputs
+
+
+# ---- the FP8 experts with float32 scales of 128 x 128 blocks (an extension) ----
+
+def test_block128_prepare_geometry_and_refusals(fake):
+    lib = amd.library()
+    arena = 8 << 30
+    B128 = amd.WEIGHT_FORMAT_E4M3_BLOCK128
+    count = C.c_uint64(0)
+    operations = lib.weight_format_operations_of
+    operations.restype = C.c_void_p
+    linear, wide_kernels = amd.LinearKernels(), amd.LinearWideKernels()
+    assert lib.linear_kernels_prepare(fake.address, fake.card, 950, C.byref(linear)) == 0
+    assert lib.linear_wide_kernels_prepare(fake.address, fake.card, 950, C.byref(wide_kernels)) == 0
+    assert fake.handles[linear.expert_gate_up_b128[2]][1] == "expert_gate_up_b128_4" and linear.expert_down_b128[4] == amd.BACKEND_NO_KERNEL
+    assert fake.handles[linear.activation_quantize_128] == ("kernel_activation_quantize", "activation_quantize_128_entry")
+    assert fake.handles[wide_kernels.wide_expert_down_b128][1] == "wide_expert_down_b128_1"
+    launches = amd.launches_of(4)
+    assert lib.linear_routed_experts_prepare(C.byref(experts_description(B128)), ARENA, C.byref(linear), launches) == 0
+    assert [fake.handles[l.kernel][1] for l in launches] == ["expert_gate_up_b128_4", "activation_quantize_128_entry", "expert_down_b128_2",
+                                                             "expert_row_sum_entry"]
+    assert [list(l.grid) for l in launches] == [[64, 64, 1], [4, 64, 1], [128, 64, 1], [2, 8, 1]]  # the quantizer: 512 values a block
+    untouched = amd.launches_of(4)
+    for changes in (dict(gate_up_shape=amd.Shape(2048 + 64, 4096, 8, 0)), dict(down_shape=amd.Shape(4096, 2048 + 64, 8, 0))):  # whole blocks of 128
+        assert lib.linear_routed_experts_prepare(C.byref(experts_description(B128, **changes)), ARENA, C.byref(linear), untouched) == 1, changes
+        assert not any(bytes(untouched))
+    quantize = amd.QuantizeDescription(amd.Range(4096, 8 * 4096 * 2), amd.Range(1 << 20, 8 * 4096), amd.Range(2 << 20, 8 * 128), amd.Range(0, 0), 4096, 8)
+    one = amd.launches_of(1)
+    assert lib.linear_quantize_128_prepare(C.byref(quantize), ARENA, C.byref(linear), one) == 0
+    assert fake.handles[one[0].kernel][1] == "activation_quantize_128_entry" and list(one[0].grid) == [8, 8, 1] and one[0].block[0] == 256
+    quantize.width = 4096 + 64
+    assert lib.linear_quantize_128_prepare(C.byref(quantize), ARENA, C.byref(linear), one) == 1
+    # the wide form: four launches, from a prepare of its own; each prepare refuses the other's formats
+    four = amd.launches_of(4)
+    description = wide_experts_description(B128)
+    assert lib.linear_wide_experts_block128_prepare(C.byref(description), arena, C.byref(linear), C.byref(wide_kernels), four) == 0
+    assert [fake.handles[l.kernel][1] for l in four] == ["wide_expert_gate_up_b128_1", "activation_quantize_128_entry", "wide_expert_down_b128_1",
+                                                         "expert_row_sum_entry"]
+    tiles = 1024 * 8 // 64 + 256
+    assert [list(l.grid) for l in four] == [[32, tiles, 1], [4, 8192, 1], [32, tiles, 1], [2, 1024, 1]]
+    assert [l.dynamic_shared_byte_count for l in four] == [53760, 0, 51712, 0]
+    quantizer = bytes(four[1].argument)[:40]
+    assert int.from_bytes(quantizer[0:8], "little") == description.experts.hidden_operands.byte_offset  # the values the gate/up launch left
+    assert int.from_bytes(quantizer[8:16], "little") == description.experts.hidden_codes.byte_offset
+    three = amd.launches_of(4)
+    assert lib.linear_wide_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(wide_kernels), three) == 1
+    assert lib.linear_wide_experts_block128_prepare(C.byref(wide_experts_description(amd.WEIGHT_FORMAT_E4M3_SCALED)), arena, C.byref(linear),
+                                                    C.byref(wide_kernels), three) == 1
+    assert not any(bytes(three))
