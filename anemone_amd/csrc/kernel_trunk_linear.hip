@@ -148,7 +148,8 @@ __device__ static __forceinline__ void trunk_linear_quantized_interleaved(const 
         const uint32_t column = 8u * (2u * wave + part) + lane / 8u;
         code_vectors[part] = first_row + (column < row_count ? column : 0u);
     }
-    const uint32_t exponent_vector = first_row + (lane < row_count ? lane : 0u);
+    const uint32_t scale_column = 16u * wave + lane % 16u;
+    const uint32_t exponent_vector = first_row + (scale_column < row_count ? scale_column : 0u);
     chain_type chain_of;
     const unsigned char *const matrices[1] = {arena + arguments.weights_offset[matrix]};
     uint32_t tile0 = 0;

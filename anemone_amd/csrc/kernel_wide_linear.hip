@@ -44,7 +44,8 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
         const uint32_t column = 8u * (2u * wave + part) + lane / 8u;
         code_vectors[part] = pairs[column < tile.pair_count ? column : 0u].pair_index / arguments.pairs_per_row;
     }
-    const uint32_t exponent_vector = pairs[lane < tile.pair_count ? lane : 0u].pair_index / arguments.pairs_per_row;
+    const uint32_t scale_column = 16u * wave + lane % 16u;
+    const uint32_t exponent_vector = pairs[scale_column < tile.pair_count ? scale_column : 0u].pair_index / arguments.pairs_per_row;
     chain_type chain_of;
     const unsigned char *const matrices[2] = {arena + tile.gate_offset, arena + tile.up_offset};
     const uint32_t window_address = (uint32_t)(uintptr_t)(lds_pointer)window;
@@ -175,7 +176,8 @@ __device__ static __forceinline__ void wide_expert_down(const struct wide_expert
         const uint32_t column = 8u * (2u * wave + part) + lane / 8u;
         code_vectors[part] = pairs[column < tile.pair_count ? column : 0u].pair_index;
     }
-    const uint32_t exponent_vector = pairs[lane < tile.pair_count ? lane : 0u].pair_index;
+    const uint32_t scale_column = 16u * wave + lane % 16u;
+    const uint32_t exponent_vector = pairs[scale_column < tile.pair_count ? scale_column : 0u].pair_index;
     chain_type chain_of;
     const unsigned char *const matrices[1] = {arena + tile.down_offset};
     uint32_t tile0 = 0;

@@ -224,9 +224,12 @@ struct strip_chain {
             /* lane L of a load lands at slot L and asks for the piece L ^ (bits 3, 4 of L, as a number): the pieces
              * (group, G, t) of one t then lie in different banks for the readers */
             piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
-            /* the scale words of the step: lane L asks for scale row row0 + min(L, rows left) */
-            const uint32_t rows_left = scale_rows - 1u - row0;
-            scale_offset = B128 ? 0u : (lane < rows_left ? lane : rows_left) * (inputs / 32u);
+            /* the strip's tiles lie in one or two rows of scales (32 outputs a row): lanes past them ask for the last again,
+             * so that a load touches two cache lines and not one a lane */
+            const uint32_t rows_needed = (tile0 + STRIP - 1u) / 2u - row0;
+            static_assert(STRIP <= 2u, "a strip of one-byte weights spans two rows of scales at most");
+            (void)scale_rows;
+            scale_offset = B128 ? 0u : (lane < rows_needed ? lane : rows_needed) * (inputs / 32u);
             /* this lane's operand registers 4 L + t: group 2 L + g / 2, piece t of output row G, its half g % 2 */
 #pragma unroll
             for (uint32_t v = 0; v < 8u; v++) {

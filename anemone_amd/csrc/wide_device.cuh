@@ -35,19 +35,22 @@ struct wide_chain {
 
     const unsigned char *words[MATRICES], *scales[MATRICES], *codes, *exponents;
     uint32_t tile_bytes, window, wave, piece_offset, scale_offset, codes_offset[2], exponents_offset;
+    bool scale_lane; /* lanes 0..15: the ones that bring the scale words of the wavefront's own column block */
     uint32_t read_at[BYTES ? 8 : 4], scale_at[STRIP], vector_at[BYTES ? 8 : 4], vector_scale_at, operand_at, shift;
 
     __device__ __forceinline__ void issue(uint32_t stage, uint32_t at) const
     {
         const uint32_t base = window + stage * STAGE_BYTES, mine = base + wave * WAVE_BYTES;
         /* first the tile's columns (this wavefront waits for them a step before the weights): eight groups of eight
-         * columns, two a wavefront: the column block it prepares; every wavefront brings the scale words (the same
-         * bytes to the same place: one load more a wavefront, and all wavefronts count alike) */
+         * columns, two a wavefront: the column block it prepares, and that block's scale words (every wavefront issues
+         * the same number of loads: the waits count them) */
 #pragma unroll
         for (uint32_t part = 0; part < 2u; part++) {
             load_to_lds_16(codes + (uint64_t)at * 128u, codes_offset[part], base + VECTOR_AT + (2u * wave + part) * 1024u);
         }
-        load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT);
+        if (scale_lane) { /* its own sixteen columns' scale words, a lane a column: sixteen cache lines a wavefront, not 64 */
+            load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT + wave * 64u);
+        }
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
 #pragma unroll
@@ -275,7 +278,7 @@ struct wide_chain {
     /* matrices: arena addresses of the stored matrices; block_strip: the block's first strip (of STRIP tiles) is
      * WIDE_WAVES block_strip; vector_codes / vector_exponents: vector 0's codes and scale codes; vectors: this lane's
      * two columns' vectors for the codes' loads (lane / 8 of groups 2 wave, 2 wave + 1) and its column's for the scale
-     * words' load (lane) */
+     * words' load (column 16 wave + lane % 16: lanes 0..15 bring them) */
     __device__ __forceinline__ void place(const unsigned char *const (&matrices)[MATRICES], uint32_t outputs, uint32_t inputs,
                                           uint32_t block_strip, const unsigned char *vector_codes, const unsigned char *vector_exponents,
                                           const uint32_t (&code_vectors)[2], uint32_t exponent_vector, uint32_t window_address,
@@ -301,8 +304,12 @@ struct wide_chain {
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs + (uint64_t)row0 * (inputs / 32u);
             }
             piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
-            const uint32_t rows_left = scale_rows - 1u - row0;
-            scale_offset = B128 ? 0u : (lane < rows_left ? lane : rows_left) * (inputs / 32u);
+            /* the strip's tiles lie in one or two rows of scales (32 outputs a row): lanes past them ask for the last again,
+             * so that a load touches two cache lines and not one a lane */
+            const uint32_t rows_needed = (tile0 + STRIP - 1u) / 2u - row0;
+            static_assert(STRIP <= 2u, "a strip of one-byte weights spans two rows of scales at most");
+            (void)scale_rows;
+            scale_offset = B128 ? 0u : (lane < rows_needed ? lane : rows_needed) * (inputs / 32u);
 #pragma unroll
             for (uint32_t v = 0; v < 8u; v++) {
                 const uint32_t group = 2u * (v / 4u) + g / 2u, t = v % 4u;
@@ -342,6 +349,7 @@ struct wide_chain {
             codes_offset[part] = code_vectors[part] * inputs + 16u * ((lane % 8u) ^ (lane / 8u) ^ part);
         }
         exponents_offset = exponent_vector * (inputs / 32u);
+        scale_lane = lane < 16u;
         const uint32_t column = o % 8u, group_bytes = (o / 8u) * 1024u;
         if constexpr (BYTES) {
 #pragma unroll
