@@ -31,9 +31,9 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     ("exl3_decode", 8): 375.2e6 + 8.4e6,      # profiles/exl3_tc_products_decode8.md
     ("fp4_decode", 32): 1434.7e6 + 1.0e6,     # profiles/expert_gate_up_fp4_fp8_decode32.md
-    ("fp8_decode", 32): 2768.4e6 + 1.0e6,
-    ("fp4_prefill", 8192): 5044.9e6 + 443.2e6,  # profiles/wide_expert_fp4_fp8_prefill.md
-    ("fp8_prefill", 2048): 5642.4e6 + 117.0e6,
+    ("fp8_decode", 32): 2746.9e6 + 1.0e6,
+    ("fp4_prefill", 8192): 4820.4e6 + 442.9e6,  # profiles/wide_expert_fp4_fp8_prefill.md
+    ("fp8_prefill", 2048): 5214.7e6 + 115.7e6,
     ("expert_join", 8192): 877.7e6 + 402.7e6,  # profiles/expert_join_trunk_linear_ffn_site.md
     ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,  # profiles/expert_b128_fp8_block128_decode64_prefill2048.md
     ("fp8_prefill_block128", 2048): 5707.3e6 + 67.2e6,
