@@ -512,22 +512,28 @@ ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_count, router_wide_arguments);
  * tiles (tile_starts): the sorted pairs of the block's rows; block 0 also the runs and every tile. The whole block
  * calls it after a barrier. */
 __device__ static __forceinline__ void wide_place_block(const struct router_wide_arguments &arguments, unsigned char *arena, uint32_t block,
-                                                        const uint32_t *block_experts, uint32_t pairs, uint32_t *totals, uint32_t *starts,
-                                                        const uint32_t *before, uint32_t *tile_starts, uint32_t *scratch)
+                                                        const uint32_t *block_experts, uint32_t *place_of, uint32_t pairs, uint32_t *totals,
+                                                        uint32_t *starts, const uint32_t *before, uint32_t *tile_starts, uint32_t *scratch)
 {
     const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
     (void)block_exclusive_scan(starts, experts, scratch);
     const struct router_pick *all_picks = (const struct router_pick *)(arena + arguments.picks_offset);
     struct wide_pair *sorted = (struct wide_pair *)(arena + arguments.pairs_offset);
     const uint32_t first_pair = block * ROUTER_SORT_ROWS * picks;
+    /* the walk writes a pick's place into LDS and nothing else: a load of the pick's weight inside it would make every
+     * match wait for memory, one after the other; the pairs are written behind it, a thread a pick */
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
         uint32_t place = starts[expert] + before[expert];
         sort_walk_picks(block_experts, pairs, [&](uint32_t index, uint32_t picked) {
             if (picked == expert) {
-                sorted[place] = (struct wide_pair){first_pair + index, all_picks[first_pair + index].route_weight};
+                place_of[index] = place;
                 place++;
             }
         });
+    }
+    __syncthreads();
+    for (uint32_t index = threadIdx.x; index < pairs; index += blockDim.x) {
+        sorted[place_of[index]] = (struct wide_pair){first_pair + index, all_picks[first_pair + index].route_weight};
     }
     if (block != 0u) {
         return;
@@ -572,6 +578,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     router_wide_place(struct router_wide_arguments arguments, unsigned char *arena)
 {
     __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t place_of[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
     const uint32_t experts = arguments.expert_count;
@@ -595,7 +602,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
         tile_starts[expert] = (total + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS;
     }
     __syncthreads();
-    wide_place_block(arguments, arena, blockIdx.x, block_experts, pairs, totals, starts, before, tile_starts, scratch);
+    wide_place_block(arguments, arena, blockIdx.x, block_experts, place_of, pairs, totals, starts, before, tile_starts, scratch);
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_place, router_wide_arguments);
 
@@ -670,6 +677,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     router_wide_small(struct router_wide_arguments arguments, unsigned char *arena)
 {
     __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t place_of[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS], job_starts[ROUTER_MOST_EXPERTS + 1u];
     const uint32_t experts = arguments.expert_count;
@@ -686,7 +694,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
         job_starts[expert] = (count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS;
     }
     __syncthreads();
-    wide_place_block(arguments, arena, 0u, block_experts, pairs, totals, starts, before, tile_starts, scratch);
+    wide_place_block(arguments, arena, 0u, block_experts, place_of, pairs, totals, starts, before, tile_starts, scratch);
     __threadfence_block();
     __syncthreads(); /* the runs and the sorted pairs, written by this block, are read by its jobs */
     wide_jobs_block(arguments, arena, job_starts, scratch);
