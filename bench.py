@@ -29,13 +29,13 @@ HBM_PEAK_GBS = 8000.0
 # same counter reads for a 1 GiB copy), for the workloads at the sizes profiled: constants of those runs (the summaries
 # under profiles/ hold the commands and the counts), reported as roofline.traffic when a run has the same sizes
 MEASURED_TRAFFIC_BYTES = {
-    ("exl3_decode", 8): 375.2e6 + 8.4e6,      # profiles/exl3_tc_products_decode8.md
-    ("fp4_decode", 32): 1434.7e6 + 1.0e6,     # profiles/expert_gate_up_fp4_fp8_decode32.md
+    ("exl3_decode", 8): 375.2e6 + 8.4e6,
+    ("fp4_decode", 32): 1434.7e6 + 1.0e6,
     ("fp8_decode", 32): 2746.9e6 + 1.0e6,
-    ("fp4_prefill", 8192): 4820.4e6 + 442.9e6,  # profiles/wide_expert_fp4_fp8_prefill.md
+    ("fp4_prefill", 8192): 4820.4e6 + 442.9e6,
     ("fp8_prefill", 2048): 5214.7e6 + 115.7e6,
-    ("expert_join", 8192): 877.7e6 + 402.7e6,  # profiles/expert_join_trunk_linear_ffn_site.md
-    ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,  # profiles/expert_b128_fp8_block128_decode64_prefill2048.md
+    ("expert_join", 8192): 877.7e6 + 402.7e6,
+    ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,
     ("fp8_prefill_block128", 2048): 5707.3e6 + 67.2e6,
 }
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
@@ -105,7 +105,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     rows = arguments.rows if not prefill or arguments.rows != 32 else 2048 if fp8 else 8192
     distinct_generated = 4 if fp8 else 16
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
-    block128 = fp8 and arguments.block128  # float32 scales of 128 x 128 blocks and of 128 values: BASELINE config 3's wording
+    block128 = fp8 and arguments.block128  # float32 scales of 128 x 128 blocks and of 128 values (the usual FP8 block scaling)
     matrix = workloads.fp8_block128_matrix if block128 else workloads.fp8_matrix if fp8 else workloads.fp4_matrix
     trios = [[matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
               matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]

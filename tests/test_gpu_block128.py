@@ -1,6 +1,6 @@
 """GPU checks, through the C ABI, of the FP8 experts with float32 block scales (WEIGHT_FORMAT_E4M3_BLOCK128: E4M3
-weights with one float32 scale for every 128 x 128 block, vectors quantized 128 values a float32 scale: the scaling
-BASELINE's FP8 configuration words). PARITY UNPINNED against the reference, which has no function of this scaling: the
+weights with one float32 scale for every 128 x 128 block, vectors quantized 128 values a float32 scale: the usual
+block scaling of FP8 checkpoints). PARITY UNPINNED against the reference, which has no function of this scaling: the
 checker is the CPU oracle's closed form (oracle/orc_linear.c: orc_act_quantize_128, orc_linear_products_128, which
 tests/test_oracle_linear.py pins against numpy). The quantizer is held byte for byte, the products to the bound the
 reference states for its own formats (tests/linear_reference.h:43-58 of the reference, with this card's allowance), the
