@@ -9,7 +9,8 @@
  * 8 (j % 2)), exponents [v][width / 32], operands [v][width] (bfloat16 of the value's code x scale x 2^100, in
  * OPERAND ORDER; an infinity of the sign where c is above 146). The operands are not read by this library's own
  * kernels; they are written because the record's contract writes them on every card.
- * Launch: grid (ceil(width / 256), vectors), block 256; a thread a value, 32 lanes a block of values.
+ * Launch: grid (ceil(width / 1024), vectors), block 256; a thread four values (a word of codes), eight threads a block
+ * of 32 values.
  */
 #include "kernel_registry.h"
 #include "quantize_device.cuh"
@@ -17,15 +18,39 @@
 extern "C" __global__ void __launch_bounds__(LINEAR_ELEMENT_THREADS)
     activation_quantize_entry(struct activation_quantize_arguments arguments, unsigned char *arena)
 {
-    const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
-    if (index >= arguments.width) {
-        return; /* the width is a multiple of 64: whole groups of 32 lanes leave together */
+    /* thread q = (16 l + 4 s + t) takes the four values 64 l + 16 s + 2 t + {0, 1, 8, 9}: the four codes of one word of
+     * the lane order and the four operands of one pair of words; the 32 values of a block of the quantization are those
+     * of eight neighbouring threads (s = 2 b, 2 b + 1; t = 0 .. 3) */
+    const uint32_t q = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t l = q / 16u, s = (q / 4u) % 4u, t = q % 4u, first = 64u * l + 16u * s + 2u * t;
+    if (first >= arguments.width) {
+        return; /* the width is a multiple of 64: whole groups of sixteen threads leave together */
     }
     const uint64_t vector = blockIdx.y;
-    const uint32_t bits = ((const uint16_t *)(arena + arguments.values_offset))[vector * arguments.width + index];
-    quantize_value(bits, index, arena + arguments.codes_offset + vector * arguments.width,
-                   arena + arguments.exponents_offset + vector * (arguments.width / 32u),
-                   (uint16_t *)(arena + arguments.operands_offset) + vector * arguments.width);
+    const uint16_t *values = (const uint16_t *)(arena + arguments.values_offset) + vector * arguments.width + first;
+    const uint32_t near_pair = *(const uint32_t *)values, far_pair = *(const uint32_t *)(values + 8);
+    const uint32_t bits[4] = {near_pair & 0xFFFFu, near_pair >> 16, far_pair & 0xFFFFu, far_pair >> 16}; /* values +0, +1, +8, +9 */
+    float largest = fmaxf(fmaxf(fabsf(bf16_to_float((uint16_t)bits[0])), fabsf(bf16_to_float((uint16_t)bits[1]))),
+                          fmaxf(fabsf(bf16_to_float((uint16_t)bits[2])), fabsf(bf16_to_float((uint16_t)bits[3]))));
+#pragma unroll
+    for (uint32_t distance = 4u; distance != 0u; distance >>= 1u) {
+        largest = fmaxf(largest, __shfl_xor(largest, (int)distance, 8));
+    }
+    const uint32_t code_exponent = quantize_exponent_code(largest);
+    uint32_t code[4], operand[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; i++) {
+        quantize_code(bits[i], code_exponent, code[i], operand[i]);
+    }
+    /* the word's bytes j = 0 .. 3 hold values +0 (j = 0), +8 (1), +1 (2), +9 (3); its operands' halfwords 2 r + h hold
+     * value + h + 8 r */
+    const uint32_t word = quantize_word_of(l, s, t);
+    *(uint32_t *)(arena + arguments.codes_offset + vector * arguments.width + word) = code[0] | (code[2] << 8) | (code[1] << 16) | (code[3] << 24);
+    *(uint2_t *)((uint16_t *)(arena + arguments.operands_offset) + vector * arguments.width + word) =
+        (uint2_t){operand[0] | (operand[1] << 16), operand[2] | (operand[3] << 16)};
+    if (q % 8u == 0u) {
+        (arena + arguments.exponents_offset)[vector * (arguments.width / 32u) + first / 32u] = (unsigned char)code_exponent;
+    }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ACTIVATION_QUANTIZE, activation_quantize_entry, activation_quantize_arguments);
 
@@ -34,36 +59,41 @@ ANEMONE_KERNEL(KERNEL_FILE_ACTIVATION_QUANTIZE, activation_quantize_entry, activ
  * (one rounding), limited to 448 and rounded to the nearest E4M3 number, a tie to the even code, the sign kept.
  * Written: codes [v][width] in the same lane order; the scales, float32 [v][width / 128], where the record names the
  * exponents (the same bytes a vector: width / 32); the operands are not written.
- * Launch: grid (ceil(width / 512), vectors), block 256: a wavefront 128 values, a lane two neighbours. */
+ * Launch: grid (ceil(width / 1024), vectors), block 256: a thread four values (a word of codes), 32 threads a scale. */
 extern "C" __global__ void __launch_bounds__(LINEAR_ELEMENT_THREADS)
     activation_quantize_128_entry(struct activation_quantize_arguments arguments, unsigned char *arena)
 {
-    const uint32_t index = 2u * (blockIdx.x * blockDim.x + threadIdx.x);
-    if (index >= arguments.width) {
-        return; /* the width is a multiple of 128: whole wavefronts leave together */
+    /* the threads' values as in activation_quantize_entry: thread q = 16 l + 4 s + t takes 64 l + 16 s + 2 t + {0, 1, 8, 9},
+     * one word of codes; the 128 values of a scale are those of 32 neighbouring threads */
+    const uint32_t q = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t l = q / 16u, s = (q / 4u) % 4u, t = q % 4u, first = 64u * l + 16u * s + 2u * t;
+    if (first >= arguments.width) {
+        return; /* the width is a multiple of 128: whole groups of 32 threads leave together */
     }
     const uint64_t vector = blockIdx.y;
-    const uint32_t two = *(const uint32_t *)((const uint16_t *)(arena + arguments.values_offset) + vector * arguments.width + index);
-    const uint32_t bits[2] = {two & 0xFFFFu, two >> 16};
-    float largest = fmaxf(fabsf(bf16_to_float((uint16_t)bits[0])), fabsf(bf16_to_float((uint16_t)bits[1])));
+    const uint16_t *values = (const uint16_t *)(arena + arguments.values_offset) + vector * arguments.width + first;
+    const uint32_t near_pair = *(const uint32_t *)values, far_pair = *(const uint32_t *)(values + 8);
+    const uint32_t bits[4] = {near_pair & 0xFFFFu, near_pair >> 16, far_pair & 0xFFFFu, far_pair >> 16};
+    float largest = fmaxf(fmaxf(fabsf(bf16_to_float((uint16_t)bits[0])), fabsf(bf16_to_float((uint16_t)bits[1]))),
+                          fmaxf(fabsf(bf16_to_float((uint16_t)bits[2])), fabsf(bf16_to_float((uint16_t)bits[3]))));
 #pragma unroll
-    for (uint32_t distance = 32u; distance != 0u; distance >>= 1u) {
-        largest = fmaxf(largest, __shfl_xor(largest, (int)distance, WAVE));
+    for (uint32_t distance = 16u; distance != 0u; distance >>= 1u) {
+        largest = fmaxf(largest, __shfl_xor(largest, (int)distance, 32));
     }
     const float scale = __fdiv_rn(fmaxf(largest, 1e-4f), 448.0f);
-    unsigned char *codes = arena + arguments.codes_offset + vector * arguments.width;
+    uint32_t code[4];
 #pragma unroll
-    for (uint32_t i = 0; i < 2u; i++) {
+    for (uint32_t i = 0; i < 4u; i++) {
         const float scaled = __fdiv_rn(bf16_to_float((uint16_t)bits[i]), scale);
         const float magnitude = fminf(fabsf(scaled), 448.0f);
         const uint32_t field = __float_as_uint(fmaxf(magnitude, 0.015625f)) >> 23;
         const uint32_t units = (uint32_t)__builtin_rintf(__fmul_rn(magnitude, __uint_as_float((257u - field) << 23)));
-        const uint32_t code = (((field - 120u) << 3) + units - 8u) | ((bits[i] >> 8) & 0x80u);
-        const uint32_t at = index + i, u = at % 16u;
-        codes[quantize_word_of(at / 64u, (at % 64u) / 16u, (u % 8u) / 2u) + 2u * (u % 2u) + u / 8u] = (unsigned char)code;
+        code[i] = (((field - 120u) << 3) + units - 8u) | ((bits[i] >> 8) & 0x80u);
     }
-    if (index % 128u == 0u) {
-        ((float *)(arena + arguments.exponents_offset))[vector * (arguments.width / 128u) + index / 128u] = scale;
+    *(uint32_t *)(arena + arguments.codes_offset + vector * arguments.width + quantize_word_of(l, s, t)) =
+        code[0] | (code[2] << 8) | (code[1] << 16) | (code[3] << 24); /* bytes: values +0, +8, +1, +9 */
+    if (q % 32u == 0u) {
+        ((float *)(arena + arguments.exponents_offset))[vector * (arguments.width / 128u) + first / 128u] = scale;
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ACTIVATION_QUANTIZE, activation_quantize_128_entry, activation_quantize_arguments);

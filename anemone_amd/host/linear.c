@@ -5,7 +5,7 @@
  *
  *   launch      kernel                      grid                                  block        shared
  *   gate/up     expert_gate_up_<S>          (output_size / 16, jobs, 1)           128 S        static
- *   quantize    activation_quantize_entry   (ceil(width / 256), pairs, 1)         256          0
+ *   quantize    activation_quantize_entry   (ceil(width / 1024), pairs, 1)        256          0
  *   down        expert_down_<S>             (output_size / 16, jobs, 1)           64 S         static
  *   row sum     expert_row_sum_entry        (ceil(width / 2048), rows, 1)         256          0
  * A wavefront is 64 lanes, so a slice is a wavefront (gate with up: two); 16 slices would be a block of 2,048
@@ -18,6 +18,7 @@
 #include "prepare_common.h"
 
 #define ROW_SUM_BLOCK_OUTPUTS (EXPERT_ROW_SUM_CHANNELS * LINEAR_ELEMENT_THREADS) /* outputs a block of the row sum takes */
+#define QUANTIZE_BLOCK_VALUES (4u * LINEAR_ELEMENT_THREADS) /* a thread of activation_quantize_entry takes four values */
 #define LINEAR_STRIP_OUTPUTS 64u /* a block of the expert kernels: a strip of four tiles of 16 outputs */
 static const uint32_t slice_counts[LINEAR_SLICE_INSTANCES] = {1u, 2u, 4u, 8u, 16u};
 #define BUILT_INSTANCES 4u
@@ -169,12 +170,12 @@ result_status linear_quantize_prepare(const struct linear_quantize_description *
     const struct activation_quantize_arguments record = {description->values.byte_offset, description->codes.byte_offset,
                                                          description->exponents.byte_offset,
                                                          description->operands.byte_offset, description->width, 0};
-    launch_fill(launch_out, kernels->activation_quantize, (description->width + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS,
+    launch_fill(launch_out, kernels->activation_quantize, (description->width + QUANTIZE_BLOCK_VALUES - 1u) / QUANTIZE_BLOCK_VALUES,
                 description->row_count, 1, LINEAR_ELEMENT_THREADS, 0, &record, sizeof record);
     return STATUS_OK;
 }
 
-#define QUANTIZE_128_BLOCK_VALUES (2u * LINEAR_ELEMENT_THREADS) /* a lane of activation_quantize_128_entry takes two values */
+#define QUANTIZE_128_BLOCK_VALUES (4u * LINEAR_ELEMENT_THREADS) /* a thread of activation_quantize_128_entry takes four values */
 
 result_status linear_quantize_128_prepare(const struct linear_quantize_description *description, uint64_t arena_byte_count,
                                           const struct linear_kernels_record *kernels, struct kernel_launch *launch_out)
@@ -255,7 +256,7 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
                                  : bytes  ? kernels->expert_down_e4m3[down_instance]
                                           : kernels->expert_down[down_instance];
     const uint32_t quantize_kernel = block128 ? kernels->activation_quantize_128 : kernels->activation_quantize;
-    const uint32_t quantize_block_values = block128 ? QUANTIZE_128_BLOCK_VALUES : LINEAR_ELEMENT_THREADS;
+    const uint32_t quantize_block_values = block128 ? QUANTIZE_128_BLOCK_VALUES : QUANTIZE_BLOCK_VALUES;
     if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL ||
         quantize_kernel == BACKEND_NO_KERNEL || kernels->expert_row_sum == BACKEND_NO_KERNEL) {
         REFUSE("%s: a kernel of the chain is not prepared", what);
@@ -513,7 +514,7 @@ result_status linear_shared_expert_prepare(const struct linear_shared_expert_des
                 (gate->output_size + ROW_SUM_BLOCK_OUTPUTS - 1u) / ROW_SUM_BLOCK_OUTPUTS, description->row_count, 1,
                 LINEAR_ELEMENT_THREADS, 0, &hidden_record, sizeof hidden_record);
     launch_fill(&launches[LINEAR_SHARED_EXPERT_QUANTIZE], kernels->activation_quantize,
-                (gate->output_size + LINEAR_ELEMENT_THREADS - 1u) / LINEAR_ELEMENT_THREADS, description->row_count, 1,
+                (gate->output_size + QUANTIZE_BLOCK_VALUES - 1u) / QUANTIZE_BLOCK_VALUES, description->row_count, 1,
                 LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
     memcpy(launches_out, launches, sizeof launches);
     return STATUS_OK;

@@ -419,7 +419,7 @@ def test_linear_prepare_geometry_and_refusals(fake):
     assert lib.linear_routed_experts_prepare(C.byref(experts_description()), ARENA, C.byref(kernels), launches) == 0
     names = [fake.handles[l.kernel][1] for l in launches]
     assert names == ["expert_gate_up_4", "activation_quantize_entry", "expert_down_2", "expert_row_sum_entry"]
-    assert [list(l.grid) for l in launches] == [[32, 64, 1], [8, 64, 1], [64, 64, 1], [2, 8, 1]]
+    assert [list(l.grid) for l in launches] == [[32, 64, 1], [2, 64, 1], [64, 64, 1], [2, 8, 1]]  # the quantizer: 1,024 values a block
     assert [l.block[0] for l in launches] == [256, 256, 128, 256]
     assert [l.argument_byte_count for l in launches] == [64, 40, 56, 24]
     fp8 = amd.launches_of(4)
@@ -436,7 +436,7 @@ def test_linear_prepare_geometry_and_refusals(fake):
                                        amd.Range(3 << 20, 8 * 4096 * 2), 4096, 8)
     one = amd.launches_of(1)
     assert lib.linear_quantize_prepare(C.byref(quantize), ARENA, C.byref(kernels), one) == 0
-    assert list(one[0].grid) == [16, 8, 1] and one[0].argument_byte_count == 40
+    assert list(one[0].grid) == [4, 8, 1] and one[0].argument_byte_count == 40
     quantize.width = 4100
     assert lib.linear_quantize_prepare(C.byref(quantize), ARENA, C.byref(kernels), one) == 1
     shape, count = amd.Shape(2048, 4096, 4, 0), C.c_uint32(0)
@@ -561,7 +561,7 @@ def test_shared_expert_prepare_geometry_and_refusals(fake):
     assert lib.linear_shared_expert_prepare(C.byref(d), arena, C.byref(kernels), launches) == 0
     assert [fake.handles[l.kernel][1] for l in launches] == ["trunk_linear_quantized_4", "trunk_hidden_entry", "activation_quantize_entry",
                                                              "trunk_linear_quantized_2"]
-    assert [list(l.grid) for l in launches] == [[128, 1, 1], [1, 8, 1], [8, 8, 1], [128, 1, 1]]  # strips of 32 outputs of both matrices
+    assert [list(l.grid) for l in launches] == [[128, 1, 1], [1, 8, 1], [2, 8, 1], [128, 1, 1]]  # strips of 32 outputs of both matrices
     assert [l.block[0] for l in launches] == [256, 256, 256, 128]
     assert [l.argument_byte_count for l in launches] == [72, 32, 40, 72]
     record = amd.TrunkLinearQuantizedArguments.from_buffer_copy(bytes(launches[0].argument)[:72])
@@ -581,7 +581,7 @@ def test_shared_expert_prepare_geometry_and_refusals(fake):
     many, _ = shared_description(rows=8192, gate_up_slices=1, down_slices=1, form=amd.LINEAR_INTERLEAVED_CHUNK_BLOCKS)
     assert lib.linear_shared_expert_prepare(C.byref(many), arena, C.byref(kernels), launches) == 0
     assert [fake.handles[l.kernel][1] for l in launches][::3] == ["trunk_linear_quantized_interleaved_1"] * 2
-    assert [list(l.grid) for l in launches] == [[32, 128, 1], [1, 8192, 1], [8, 8192, 1], [32, 128, 1]]
+    assert [list(l.grid) for l in launches] == [[32, 128, 1], [1, 8192, 1], [2, 8192, 1], [32, 128, 1]]
     assert [l.dynamic_shared_byte_count for l in launches] == [51712, 0, 0, 51712] and launches[0].block[0] == 256
     sliced, _ = shared_description(rows=100, form=amd.LINEAR_INTERLEAVED_CHUNK_BLOCKS)  # the interleaved form is of one slice
     untouched = amd.launches_of(4)
@@ -672,7 +672,7 @@ def test_block128_prepare_geometry_and_refusals(fake):
     assert lib.linear_routed_experts_prepare(C.byref(experts_description(B128)), ARENA, C.byref(linear), launches) == 0
     assert [fake.handles[l.kernel][1] for l in launches] == ["expert_gate_up_b128_4", "activation_quantize_128_entry", "expert_down_b128_2",
                                                              "expert_row_sum_entry"]
-    assert [list(l.grid) for l in launches] == [[64, 64, 1], [4, 64, 1], [128, 64, 1], [2, 8, 1]]  # the quantizer: 512 values a block
+    assert [list(l.grid) for l in launches] == [[64, 64, 1], [2, 64, 1], [128, 64, 1], [2, 8, 1]]  # the quantizer: 1,024 values a block
     untouched = amd.launches_of(4)
     for changes in (dict(gate_up_shape=amd.Shape(2048 + 64, 4096, 8, 0)), dict(down_shape=amd.Shape(4096, 2048 + 64, 8, 0))):  # whole blocks of 128
         assert lib.linear_routed_experts_prepare(C.byref(experts_description(B128, **changes)), ARENA, C.byref(linear), untouched) == 1, changes
@@ -680,7 +680,7 @@ def test_block128_prepare_geometry_and_refusals(fake):
     quantize = amd.QuantizeDescription(amd.Range(4096, 8 * 4096 * 2), amd.Range(1 << 20, 8 * 4096), amd.Range(2 << 20, 8 * 128), amd.Range(0, 0), 4096, 8)
     one = amd.launches_of(1)
     assert lib.linear_quantize_128_prepare(C.byref(quantize), ARENA, C.byref(linear), one) == 0
-    assert fake.handles[one[0].kernel][1] == "activation_quantize_128_entry" and list(one[0].grid) == [8, 8, 1] and one[0].block[0] == 256
+    assert fake.handles[one[0].kernel][1] == "activation_quantize_128_entry" and list(one[0].grid) == [4, 8, 1] and one[0].block[0] == 256
     quantize.width = 4096 + 64
     assert lib.linear_quantize_128_prepare(C.byref(quantize), ARENA, C.byref(linear), one) == 1
     # the wide form: four launches, from a prepare of its own; each prepare refuses the other's formats
@@ -690,7 +690,7 @@ def test_block128_prepare_geometry_and_refusals(fake):
     assert [fake.handles[l.kernel][1] for l in four] == ["wide_expert_gate_up_b128_1", "activation_quantize_128_entry", "wide_expert_down_b128_1",
                                                          "expert_row_sum_entry"]
     tiles = 1024 * 8 // 64 + 256
-    assert [list(l.grid) for l in four] == [[32, tiles, 1], [4, 8192, 1], [32, tiles, 1], [2, 1024, 1]]
+    assert [list(l.grid) for l in four] == [[32, tiles, 1], [2, 8192, 1], [32, tiles, 1], [2, 1024, 1]]
     assert [l.dynamic_shared_byte_count for l in four] == [53760, 0, 51712, 0]
     quantizer = bytes(four[1].argument)[:40]
     assert int.from_bytes(quantizer[0:8], "little") == description.experts.hidden_operands.byte_offset  # the values the gate/up launch left
