@@ -108,6 +108,83 @@ __device__ static __forceinline__ void wave_hadamard128(float &v0, float &v1, ui
     v1 = difference;
 }
 
+/* The same transform with a block of 128 values across SIXTEEN lanes (a row of the wavefront): lane r of the row holds
+ * values 8 r .. 8 r + 7. Distances 1, 2, 4 stay inside the lane; 8, 16, 32, 64 pair lane r with r ^ 1, ^ 2, ^ 4, ^ 8 of
+ * the row, which the data-parallel primitives of a vector instruction reach without LDS: a permutation of four lanes
+ * (^ 1, ^ 2), the mirror of eight lanes followed by the reversal of four (^ 4), the mirror of sixteen followed by the
+ * mirror of eight (^ 8). Every pair (lower, upper) becomes (lower + upper, lower - upper), each one rounding: the bits of
+ * wave_hadamard128. A row's sixteen lanes are all active or all idle. */
+template <int control>
+__device__ static __forceinline__ float row_lane_of(float value)
+{
+    /* every lane of an active row has a source lane in it: what a lane without one would keep is never read */
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, value), control, 0xF, 0xF, true));
+}
+
+__device__ static __forceinline__ void row_hadamard128(float (&v)[8], uint32_t lane)
+{
+    constexpr int SWAP_PAIRS = 0xB1 /* lanes 1, 0, 3, 2 of four */, SWAP_TWOS = 0x4E /* 2, 3, 0, 1 */, REVERSE_FOUR = 0x1B /* 3, 2, 1, 0 */,
+                  MIRROR_SIXTEEN = 0x140, MIRROR_EIGHT = 0x141;
+#pragma unroll
+    for (uint32_t distance = 1; distance < 8u; distance *= 2u) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; i++) {
+            if ((i & distance) == 0u) {
+                const float lower = v[i], upper = v[i + distance];
+                v[i] = __fadd_rn(lower, upper);
+                v[i + distance] = __fsub_rn(lower, upper);
+            }
+        }
+    }
+    /* other + own for the lower lane of a pair, other - own for the upper: own by +1 or -1 (exact), then one addition
+     * whose first operand comes from the other lane inside the instruction */
+    const float sign1 = (lane & 1u) == 0u ? 1.0f : -1.0f, sign2 = (lane & 2u) == 0u ? 1.0f : -1.0f;
+    const float sign4 = (lane & 4u) == 0u ? 1.0f : -1.0f, sign8 = (lane & 8u) == 0u ? 1.0f : -1.0f;
+#pragma unroll
+    for (uint32_t i = 0; i < 8u; i++) {
+        v[i] = __fadd_rn(row_lane_of<SWAP_PAIRS>(v[i]), __fmul_rn(sign1, v[i]));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 8u; i++) {
+        v[i] = __fadd_rn(row_lane_of<SWAP_TWOS>(v[i]), __fmul_rn(sign2, v[i]));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 8u; i++) {
+        v[i] = __fadd_rn(row_lane_of<REVERSE_FOUR>(row_lane_of<MIRROR_EIGHT>(v[i])), __fmul_rn(sign4, v[i]));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 8u; i++) {
+        v[i] = __fadd_rn(row_lane_of<MIRROR_EIGHT>(row_lane_of<MIRROR_SIXTEEN>(v[i])), __fmul_rn(sign8, v[i]));
+    }
+}
+
+/* eight bfloat16 or fp16 values of a 16-byte load as float32; eight float32 as fp16, one rounding each */
+__device__ static __forceinline__ void unpack_bf16x8(uint4_t load, float (&values)[8])
+{
+#pragma unroll
+    for (uint32_t i = 0; i < 8u; i++) {
+        values[i] = __uint_as_float(i % 2u == 0u ? load[i / 2u] << 16 : load[i / 2u] & 0xFFFF0000u);
+    }
+}
+
+__device__ static __forceinline__ void unpack_half8(uint4_t load, float (&values)[8])
+{
+#pragma unroll
+    for (uint32_t i = 0; i < 8u; i++) {
+        values[i] = half_bits_to_float((uint16_t)(i % 2u == 0u ? load[i / 2u] & 0xFFFFu : load[i / 2u] >> 16));
+    }
+}
+
+__device__ static __forceinline__ uint4_t pack_half8(const float (&values)[8])
+{
+    uint4_t packed;
+#pragma unroll
+    for (uint32_t word = 0; word < 4u; word++) {
+        packed[word] = (uint32_t)float_to_half_bits(values[2u * word]) | ((uint32_t)float_to_half_bits(values[2u * word + 1u]) << 16);
+    }
+    return packed;
+}
+
 /* mul1: two 16-bit states -> two fp16 weights in one register (low half: first) */
 __device__ static __forceinline__ uint32_t exl3_decode_pair(uint32_t state_low, uint32_t state_high)
 {

@@ -28,6 +28,7 @@
 #define TCP_COLUMN_BLOCKS (EXL3_TCP_CHUNK_PAIRS / 16u)
 #define TCP_STEP_INPUTS 32u
 #define TCP_BATCH 4u        /* columns the element-wise launches take at a time */
+#define TCP_WAVE_BLOCKS 4u  /* blocks of 128 channels a wavefront of an element-wise launch takes: a row of sixteen lanes each */
 #define TCP_OPERAND_PARTS ((TCP_COLUMN_BLOCKS + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES) /* 16-column groups a wavefront brings a step */
 #define TCP_STAGE_BYTES (TCP_OPERAND_PARTS * TCP_GEMM_WAVES * 1024u) /* a K step of the chunk's operand columns, in whole groups */
 
@@ -168,46 +169,72 @@ __device__ static __forceinline__ struct exl3_tcp_chunk tcp_chunk_of(const tcp_s
     return chunk;
 }
 
-/* launch 2: grid (hidden / 128, chunk capacity, 2), block 64: the gate (z = 0) and up (z = 1) operands of a chunk's
- * pairs, by place: fp16(H128(x suh) / sqrt(128)) */
+/* The element-wise launches take a block of 128 values in a row of sixteen lanes, eight consecutive values a lane
+ * (one 16-byte load of bfloat16 or fp16, two of float32): a wavefront is four adjacent blocks of one vector, 1 KB of
+ * bfloat16 a load. this lane's block of 128 channels and its first channel, or false past the width */
+__device__ static __forceinline__ bool tcp_lane_channels(uint32_t width, uint32_t &channel)
+{
+    const uint32_t lane = threadIdx.x;
+    channel = (blockIdx.x * TCP_WAVE_BLOCKS + lane / 16u) * EXL3_TRANSFORM + 8u * (lane % 16u);
+    return channel < width;
+}
+
+/* launch 2: grid (ceil(hidden / 512), chunk capacity, EXL3_TCP_COLUMN_PARTS), block 64: the gate and the up operands of
+ * a part of a chunk's pairs, by place: fp16(H128(x suh) / sqrt(128)); a row is read once for both */
 extern "C" __global__ void exl3_tcp_operands(struct exl3_tcp_record record, unsigned char *arena)
 {
     const tcp_shape shape = tcp_shape_of(record);
     unsigned char *workspace = arena + record.workspace_offset;
     const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, blockIdx.y);
-    if (chunk.pair_count == 0u) {
+    const uint32_t first_column = blockIdx.z * EXL3_TCP_PART_COLUMNS;
+    uint32_t channel;
+    if (first_column >= chunk.pair_count || !tcp_lane_channels(shape.hidden, channel)) {
         return;
     }
-    const uint32_t lane = threadIdx.x, projection = blockIdx.z, channel = blockIdx.x * EXL3_TRANSFORM + lane;
-    const uint64_t matrix = tcp_matrix_of(record, arena, chunk.expert, projection);
-    const uint16_t *suh = (const uint16_t *)(arena + matrix + exl3_code_bytes(shape.hidden, shape.intermediate,
-                                                                               tcp_bits_x2(record, arena, chunk.expert, projection)));
-    const float s0 = half_bits_to_float(suh[channel]), s1 = half_bits_to_float(suh[channel + WAVE]);
+    const uint32_t lane = threadIdx.x;
+    const uint32_t last_column = first_column + EXL3_TCP_PART_COLUMNS < chunk.pair_count ? first_column + EXL3_TCP_PART_COLUMNS : chunk.pair_count;
+    float scale[2][8];
+#pragma unroll
+    for (uint32_t projection = 0; projection < 2u; projection++) {
+        const uint64_t matrix = tcp_matrix_of(record, arena, chunk.expert, projection);
+        const uint16_t *suh = (const uint16_t *)(arena + matrix + exl3_code_bytes(shape.hidden, shape.intermediate,
+                                                                                   tcp_bits_x2(record, arena, chunk.expert, projection)));
+        unpack_half8(*(const uint4_t *)(suh + channel), scale[projection]);
+    }
     const uint16_t *rows = (const uint16_t *)(arena + record.hidden_offset);
     const uint32_t *sorted = (const uint32_t *)(workspace + shape.layout.sorted);
-    uint16_t *operands = (uint16_t *)(workspace + shape.layout.operands) + (uint64_t)projection * shape.pairs * shape.hidden;
+    uint16_t *operands = (uint16_t *)(workspace + shape.layout.operands);
     /* TCP_BATCH columns at a time: their loads are asked for together, so that one column's latency hides behind
-     * the others' (a column past the chunk's last repeats it and is not stored) */
-    for (uint32_t first = 0; first < chunk.pair_count; first += TCP_BATCH) {
-        float v0[TCP_BATCH], v1[TCP_BATCH];
+     * the others' (a column past the part's last repeats it and is not stored) */
+    for (uint32_t first = first_column; first < last_column; first += TCP_BATCH) {
+        uint4_t loads[TCP_BATCH];
         uint32_t place[TCP_BATCH];
 #pragma unroll
         for (uint32_t i = 0; i < TCP_BATCH; i++) {
-            const uint32_t column = first + i < chunk.pair_count ? first + i : chunk.pair_count - 1u;
+            const uint32_t column = first + i < last_column ? first + i : last_column - 1u;
             place[i] = chunk.first_pair + column;
             const uint64_t row = sorted[place[i]] / shape.picks;
-            v0[i] = bf16_to_float(rows[row * shape.hidden + channel]);
-            v1[i] = bf16_to_float(rows[row * shape.hidden + channel + WAVE]);
+            loads[i] = *(const uint4_t *)(rows + row * shape.hidden + channel);
         }
 #pragma unroll
         for (uint32_t i = 0; i < TCP_BATCH; i++) {
-            v0[i] = __fmul_rn(v0[i], s0);
-            v1[i] = __fmul_rn(v1[i], s1);
-            wave_hadamard128(v0[i], v1[i], lane);
-            if (first + i < chunk.pair_count) {
-                uint16_t *out = operands + (uint64_t)place[i] * shape.hidden;
-                out[channel] = float_to_half_bits(__fmul_rn(v0[i], EXL3_NORMALIZATION));
-                out[channel + WAVE] = float_to_half_bits(__fmul_rn(v1[i], EXL3_NORMALIZATION));
+            float x[8];
+            unpack_bf16x8(loads[i], x);
+#pragma unroll
+            for (uint32_t projection = 0; projection < 2u; projection++) {
+                float v[8];
+#pragma unroll
+                for (uint32_t j = 0; j < 8u; j++) {
+                    v[j] = __fmul_rn(x[j], scale[projection][j]);
+                }
+                row_hadamard128(v, lane);
+#pragma unroll
+                for (uint32_t j = 0; j < 8u; j++) {
+                    v[j] = __fmul_rn(v[j], EXL3_NORMALIZATION);
+                }
+                if (first + i < last_column) {
+                    *(uint4_t *)(operands + ((uint64_t)projection * shape.pairs + place[i]) * shape.hidden + channel) = pack_half8(v);
+                }
             }
         }
     }
@@ -404,90 +431,110 @@ extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS) exl3_tcp_gemm(str
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_gemm, exl3_tcp_record);
 
-/* launch 4: grid (intermediate / 128, chunk capacity), block 64: per pair of the chunk, gate = H128(gate products) /
+/* launch 4: grid (ceil(intermediate / 512), chunk capacity, EXL3_TCP_COLUMN_PARTS), block 64: per pair of a part of the chunk, gate = H128(gate products) /
  * sqrt(128) x svh, up the same, the SwiGLU with its limit, x the down matrix's suh, H128 -> the fp16 down operand */
 extern "C" __global__ void exl3_tcp_activate(struct exl3_tcp_record record, unsigned char *arena)
 {
     const tcp_shape shape = tcp_shape_of(record);
     unsigned char *workspace = arena + record.workspace_offset;
     const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, blockIdx.y);
-    if (chunk.pair_count == 0u) {
+    const uint32_t first_column = blockIdx.z * EXL3_TCP_PART_COLUMNS;
+    uint32_t channel;
+    if (first_column >= chunk.pair_count || !tcp_lane_channels(shape.intermediate, channel)) {
         return;
     }
-    const uint32_t lane = threadIdx.x, channel = blockIdx.x * EXL3_TRANSFORM + lane;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t last_column = first_column + EXL3_TCP_PART_COLUMNS < chunk.pair_count ? first_column + EXL3_TCP_PART_COLUMNS : chunk.pair_count;
     const uint32_t H = shape.hidden, I = shape.intermediate, e = chunk.expert;
     const uint16_t *gate_svh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, e, 0u) + exl3_code_bytes(H, I, tcp_bits_x2(record, arena, e, 0u))) + H;
     const uint16_t *up_svh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, e, 1u) + exl3_code_bytes(H, I, tcp_bits_x2(record, arena, e, 1u))) + H;
     const uint16_t *down_suh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, e, 2u) + exl3_code_bytes(I, H, tcp_bits_x2(record, arena, e, 2u)));
-    const float gs[2] = {half_bits_to_float(gate_svh[channel]), half_bits_to_float(gate_svh[channel + WAVE])};
-    const float us[2] = {half_bits_to_float(up_svh[channel]), half_bits_to_float(up_svh[channel + WAVE])};
-    const float ds[2] = {half_bits_to_float(down_suh[channel]), half_bits_to_float(down_suh[channel + WAVE])};
+    float gs[8], us[8], ds[8];
+    unpack_half8(*(const uint4_t *)(gate_svh + channel), gs);
+    unpack_half8(*(const uint4_t *)(up_svh + channel), us);
+    unpack_half8(*(const uint4_t *)(down_suh + channel), ds);
     const float limit = record.activation_limit;
     const float *gate_products = (const float *)(workspace + shape.layout.gate_up);
     const float *up_products = gate_products + (uint64_t)shape.pairs * I;
     uint16_t *operands = (uint16_t *)(workspace + shape.layout.operands);
-    for (uint32_t first = 0; first < chunk.pair_count; first += TCP_BATCH) { /* batched as the operands' loop */
-        float g[TCP_BATCH][2], u[TCP_BATCH][2];
-        uint64_t place[TCP_BATCH];
+    constexpr uint32_t BATCH = 2u; /* two columns' eight loads together */
+    for (uint32_t first = first_column; first < last_column; first += BATCH) {
+        float4_t loads[BATCH][4];
+        uint64_t place[BATCH];
 #pragma unroll
-        for (uint32_t i = 0; i < TCP_BATCH; i++) {
-            const uint32_t column = first + i < chunk.pair_count ? first + i : chunk.pair_count - 1u;
+        for (uint32_t i = 0; i < BATCH; i++) {
+            const uint32_t column = first + i < last_column ? first + i : last_column - 1u;
             place[i] = chunk.first_pair + column;
-            g[i][0] = gate_products[place[i] * I + channel];
-            g[i][1] = gate_products[place[i] * I + channel + WAVE];
-            u[i][0] = up_products[place[i] * I + channel];
-            u[i][1] = up_products[place[i] * I + channel + WAVE];
+            const float4_t *gate = (const float4_t *)(gate_products + place[i] * I + channel), *up = (const float4_t *)(up_products + place[i] * I + channel);
+            loads[i][0] = gate[0];
+            loads[i][1] = gate[1];
+            loads[i][2] = up[0];
+            loads[i][3] = up[1];
         }
 #pragma unroll
-        for (uint32_t i = 0; i < TCP_BATCH; i++) {
-            wave_hadamard128(g[i][0], g[i][1], lane);
-            wave_hadamard128(u[i][0], u[i][1], lane);
-            float v[2];
+        for (uint32_t i = 0; i < BATCH; i++) {
+            float g[8], u[8], v[8];
 #pragma unroll
-            for (uint32_t half = 0; half < 2u; half++) {
-                const float gate = __fmul_rn(__fmul_rn(g[i][half], EXL3_NORMALIZATION), gs[half]);
-                const float up = __fmul_rn(__fmul_rn(u[i][half], EXL3_NORMALIZATION), us[half]);
+            for (uint32_t j = 0; j < 8u; j++) {
+                g[j] = loads[i][j / 4u][j % 4u];
+                u[j] = loads[i][2u + j / 4u][j % 4u];
+            }
+            row_hadamard128(g, lane);
+            row_hadamard128(u, lane);
+#pragma unroll
+            for (uint32_t j = 0; j < 8u; j++) {
+                const float gate = __fmul_rn(__fmul_rn(g[j], EXL3_NORMALIZATION), gs[j]);
+                const float up = __fmul_rn(__fmul_rn(u[j], EXL3_NORMALIZATION), us[j]);
                 const float bounded_gate = limit > 0.0f ? fminf(gate, limit) : gate;
                 const float bounded_up = limit > 0.0f ? fminf(fmaxf(up, -limit), limit) : up;
                 const float hidden = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
-                v[half] = __fmul_rn(hidden, ds[half]);
+                v[j] = __fmul_rn(hidden, ds[j]);
             }
-            wave_hadamard128(v[0], v[1], lane);
-            if (first + i < chunk.pair_count) {
-                uint16_t *operand = operands + place[i] * I;
-                operand[channel] = float_to_half_bits(__fmul_rn(v[0], EXL3_NORMALIZATION));
-                operand[channel + WAVE] = float_to_half_bits(__fmul_rn(v[1], EXL3_NORMALIZATION));
+            row_hadamard128(v, lane);
+#pragma unroll
+            for (uint32_t j = 0; j < 8u; j++) {
+                v[j] = __fmul_rn(v[j], EXL3_NORMALIZATION);
+            }
+            if (first + i < last_column) {
+                *(uint4_t *)(operands + place[i] * I + channel) = pack_half8(v);
             }
         }
     }
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_activate, exl3_tcp_record);
 
-/* launch 6: grid (hidden / 128, row_count), block 64: a row's pairs in slot order */
+/* launch 6: grid (ceil(hidden / 512), row_count), block 64: a row's pairs in slot order */
 extern "C" __global__ void exl3_tcp_combine(struct exl3_tcp_record record, unsigned char *arena)
 {
     const tcp_shape shape = tcp_shape_of(record);
     const unsigned char *workspace = arena + record.workspace_offset;
-    const uint32_t lane = threadIdx.x, channel = blockIdx.x * EXL3_TRANSFORM + lane, row = blockIdx.y;
+    uint32_t channel;
+    if (!tcp_lane_channels(shape.hidden, channel)) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x, row = blockIdx.y;
     const uint32_t H = shape.hidden, I = shape.intermediate;
     const struct router_pick *picks = (const struct router_pick *)(arena + record.picks_offset) + (uint64_t)row * shape.picks;
     const uint32_t *place_of = (const uint32_t *)(workspace + shape.layout.place_of);
     const float *down = (const float *)(workspace + shape.layout.down);
-    float sum0 = 0.0f, sum1 = 0.0f;
+    float sum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t slot = 0; slot < shape.picks; slot++) {
         const struct router_pick pick = picks[slot];
         const uint64_t place = place_of[row * shape.picks + slot];
         const uint16_t *svh = (const uint16_t *)(arena + tcp_matrix_of(record, arena, pick.expert, 2u) +
                                                  exl3_code_bytes(I, H, tcp_bits_x2(record, arena, pick.expert, 2u))) + I;
-        float v0 = down[place * H + channel], v1 = down[place * H + channel + WAVE];
-        wave_hadamard128(v0, v1, lane);
-        const float y0 = __fmul_rn(__fmul_rn(__fmul_rn(v0, EXL3_NORMALIZATION), half_bits_to_float(svh[channel])), pick.route_weight);
-        const float y1 = __fmul_rn(__fmul_rn(__fmul_rn(v1, EXL3_NORMALIZATION), half_bits_to_float(svh[channel + WAVE])), pick.route_weight);
-        sum0 = __fadd_rn(sum0, y0);
-        sum1 = __fadd_rn(sum1, y1);
+        const float4_t *products = (const float4_t *)(down + place * H + channel);
+        const float4_t low = products[0], high = products[1];
+        float v[8] = {low[0], low[1], low[2], low[3], high[0], high[1], high[2], high[3]}, scale[8];
+        unpack_half8(*(const uint4_t *)(svh + channel), scale);
+        row_hadamard128(v, lane);
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; j++) {
+            sum[j] = __fadd_rn(sum[j], __fmul_rn(__fmul_rn(__fmul_rn(v[j], EXL3_NORMALIZATION), scale[j]), pick.route_weight));
+        }
     }
-    float *out = (float *)(arena + record.output_offset) + (uint64_t)row * H;
-    out[channel] = sum0;
-    out[channel + WAVE] = sum1;
+    float4_t *out = (float4_t *)((float *)(arena + record.output_offset) + (uint64_t)row * H + channel);
+    out[0] = (float4_t){sum[0], sum[1], sum[2], sum[3]};
+    out[1] = (float4_t){sum[4], sum[5], sum[6], sum[7]};
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_combine, exl3_tcp_record);

@@ -194,10 +194,11 @@ static result_status tcp_prepare(const struct exl3_tcp_record *record, uint64_t 
     static const char *const names[EXL3_TCP_LAUNCHES] = {"exl3_tcp_count",    "exl3_tcp_place", "exl3_tcp_operands", "exl3_tcp_gemm",
                                                          "exl3_tcp_activate", "exl3_tcp_gemm",  "exl3_tcp_combine"};
     const uint32_t blocks = (uint32_t)((rows + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS), capacity = layout.chunk_capacity;
-    const uint32_t grid_x[EXL3_TCP_LAUNCHES] = {blocks, blocks, H / 128u, (I + EXL3_TCP_BLOCK_OUTPUTS - 1u) / EXL3_TCP_BLOCK_OUTPUTS,
-                                                I / 128u, (H + EXL3_TCP_BLOCK_OUTPUTS - 1u) / EXL3_TCP_BLOCK_OUTPUTS, H / 128u};
+    /* an element-wise launch's wavefront takes four blocks of 128 channels */
+    const uint32_t grid_x[EXL3_TCP_LAUNCHES] = {blocks, blocks, (H + 511u) / 512u, (I + EXL3_TCP_BLOCK_OUTPUTS - 1u) / EXL3_TCP_BLOCK_OUTPUTS,
+                                                (I + 511u) / 512u, (H + EXL3_TCP_BLOCK_OUTPUTS - 1u) / EXL3_TCP_BLOCK_OUTPUTS, (H + 511u) / 512u};
     const uint32_t grid_y[EXL3_TCP_LAUNCHES] = {1u, 1u, capacity, capacity, capacity, capacity, record->row_count};
-    const uint32_t grid_z[EXL3_TCP_LAUNCHES] = {1u, 1u, 2u, 2u, 1u, 1u, 1u};
+    const uint32_t grid_z[EXL3_TCP_LAUNCHES] = {1u, 1u, EXL3_TCP_COLUMN_PARTS, 2u, EXL3_TCP_COLUMN_PARTS, 1u, 1u};
     const uint32_t threads[EXL3_TCP_LAUNCHES] = {512u, 512u, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS};
     struct kernel_launch launches[EXL3_TCP_LAUNCHES];
     for (uint32_t index = 0; index < EXL3_TCP_LAUNCHES; index++) {

@@ -336,6 +336,8 @@ ANEMONE_INLINE uint64_t exl3_tc_workspace_bytes(uint64_t pairs, uint64_t hidden,
  * the combine of a row's pairs in slot order. */
 #define EXL3_TCP_KERNEL_FILE "kernel_exl3_tcp"
 #define EXL3_TCP_CHUNK_PAIRS 160u  /* columns of one GEMM block: pairs of one expert (ten MFMA column blocks) */
+#define EXL3_TCP_PART_COLUMNS 16u /* pairs of a chunk a block of the element-wise launches (operands, activate) takes */
+#define EXL3_TCP_COLUMN_PARTS ((EXL3_TCP_CHUNK_PAIRS + EXL3_TCP_PART_COLUMNS - 1u) / EXL3_TCP_PART_COLUMNS)
 #define EXL3_TCP_BLOCK_OUTPUTS 256u /* outputs of one GEMM block: four wavefronts of four tiles */
 #define EXL3_TCP_LAUNCHES 7u
 #define EXL3_TCP_MOST_LAUNCHES 8u  /* the reference's bound of its own forms */

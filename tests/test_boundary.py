@@ -367,8 +367,8 @@ def test_tcp_prepare_geometry_and_refusals(fake):
     assert names == ["exl3_tcp_count", "exl3_tcp_place", "exl3_tcp_operands", "exl3_tcp_gemm", "exl3_tcp_activate", "exl3_tcp_gemm",
                      "exl3_tcp_combine"]
     capacity = 4096 * 8 // amd.EXL3_TCP_CHUNK_PAIRS + 256
-    assert [list(launches[i].grid) for i in range(7)] == [[11, 1, 1], [11, 1, 1], [32, capacity, 2], [8, capacity, 2], [16, capacity, 1],
-                                                           [16, capacity, 1], [32, 4096, 1]]
+    assert [list(launches[i].grid) for i in range(7)] == [[11, 1, 1], [11, 1, 1], [8, capacity, 10], [8, capacity, 2], [4, capacity, 10],
+                                                               [16, capacity, 1], [8, 4096, 1]]  # element-wise launches: 512 channels a wavefront, 16 pairs a block
     assert [launches[i].block[0] for i in range(7)] == [512, 512, 64, 256, 64, 256, 64]
     records = [amd.Exl3TcpRecord.from_buffer_copy(bytes(launches[i].argument)[:112]) for i in range(7)]
     assert [r.pass_ for r in records] == [0, 0, 0, 0, 0, 3, 0] and all(launches[i].argument_byte_count == 112 for i in range(7))

@@ -100,6 +100,20 @@ def test_prefill_layer_against_oracle(amd, card, hidden, inner, experts_n, picks
     assert int(chunks[:used, 2].sum()) == pairs and chunks[:used, 2].max() <= most
     assert np.array_equal(chunks[:used, 1], np.concatenate([[0], np.cumsum(chunks[:used, 2])[:-1]]))
     say("  chunks %d, the longest run %d pairs" % (used, counts.max()))
+    # the operands are bit-defined: fp16(H128(bf16 x, fp16 suh) / sqrt(128)), by place, gate then up. The down pass has
+    # taken the first array since; run the route and the operands once more and read both
+    card.run(launches[0:3])
+    operands = card.download(layer.tcp_workspace_offset + layout["operands"], 2 * pairs * hidden * 2, np.uint16).reshape(2, pairs, hidden)
+    for place in sorted(set(list(range(0, pairs, max(1, pairs // 40))) + [pairs - 1])):
+        pair = int(sorted_pairs[place])
+        e = int(experts.reshape(-1)[pair])
+        for proj in range(2):
+            cb = int(orc.orc_exl3_code_bytes(hidden, inner, int(widths[e, proj])))
+            suh = np.ascontiguousarray(matrices[e][proj][cb:cb + 2 * hidden]).view(np.uint16)
+            expect = np.zeros(hidden, dtype=np.uint16)
+            orc.orc_exl3_operand(ptr(x[pair // picks], u16p), ptr(suh, u16p), hidden, ptr(expect, u16p))
+            assert np.array_equal(operands[proj, place], expect), ("operands are bit-defined", place, proj)
+    card.run(launches)
     got = layer.output()
     want = oracle_layer(layer, x, experts, weights, matrices, widths)
     scale = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
