@@ -86,6 +86,7 @@ ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_count, exl3_tcp_record);
 extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_place(struct exl3_tcp_record record, unsigned char *arena)
 {
     __shared__ __attribute__((aligned(16))) uint32_t block_experts[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
+    __shared__ uint32_t block_places[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t chunk_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
     const tcp_shape shape = tcp_shape_of(record);
@@ -111,15 +112,21 @@ extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_place(st
     (void)block_exclusive_scan(starts, experts, scratch);
     uint32_t *sorted = (uint32_t *)(workspace + shape.layout.sorted), *place_of = (uint32_t *)(workspace + shape.layout.place_of);
     const uint32_t first_pair = blockIdx.x * ROUTER_SORT_ROWS * shape.picks;
+    /* the walk writes a pick's place into LDS alone; the two tables are written behind it, a thread a pick */
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
         uint32_t place = starts[expert] + before[expert];
         sort_walk_picks(block_experts, pairs, [&](uint32_t index, uint32_t picked) {
             if (picked == expert) {
-                sorted[place] = first_pair + index;
-                place_of[first_pair + index] = place;
+                block_places[index] = place;
                 place++;
             }
         });
+    }
+    __syncthreads();
+    for (uint32_t index = threadIdx.x; index < pairs; index += blockDim.x) {
+        const uint32_t place = block_places[index];
+        sorted[place] = first_pair + index;
+        place_of[first_pair + index] = place;
     }
     if (blockIdx.x != 0u) {
         return;

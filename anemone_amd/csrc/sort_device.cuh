@@ -24,13 +24,27 @@ __device__ static __forceinline__ uint32_t sort_block_picks(const struct router_
     return rows * picks_per_row;
 }
 
-/* Every pick of a block in order, eight at a time (two 16-byte LDS reads in flight, not one 4-byte read a step):
- * visit(index, expert). block_experts is 16-byte aligned. */
+/* Every pick of a block in order, 32 at a time (eight 16-byte LDS reads in flight, so that a walk waits for LDS once
+ * in 32 picks), then eight at a time, then one: visit(index, expert). block_experts is 16-byte aligned. */
 template <typename Visit>
 __device__ static __forceinline__ void sort_walk_picks(const uint32_t *block_experts, uint32_t pairs, Visit visit)
 {
     typedef __attribute__((ext_vector_type(4))) uint32_t four_words;
     uint32_t index = 0;
+    for (; index + 32u <= pairs; index += 32u) {
+        four_words words[8];
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; i++) {
+            words[i] = *(const four_words *)(block_experts + index + 4u * i);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; i++) {
+            visit(index + 4u * i, words[i].x);
+            visit(index + 4u * i + 1u, words[i].y);
+            visit(index + 4u * i + 2u, words[i].z);
+            visit(index + 4u * i + 3u, words[i].w);
+        }
+    }
     for (; index + 8u <= pairs; index += 8u) {
         const four_words low = *(const four_words *)(block_experts + index), high = *(const four_words *)(block_experts + index + 4u);
         visit(index, low.x);
