@@ -614,8 +614,12 @@ class Exl3Layer:
         r.widths_offset, r.hidden, r.pairs_per_row = self.widths_offset, self.H, self.P
         return r
 
-    def tc_launches(self):
+    def tc_launches(self, shared_offset=None):
+        """The fused decode's launches; with shared_offset the combine adds each row's sum to the shared expert's
+        bfloat16 rows there, in place, and leaves the float32 output alone."""
         record = self.tc_record()
+        if shared_offset is not None:
+            record.shared_sum, record.shared_offset = 1, shared_offset
         launches = launches_of(EXL3_TC_LAUNCHES)
         check(self.card.lib.exl3_tc_prepare(C.byref(record), self.card.arena_bytes, backend_table(), self.card.handle, launches), "exl3_tc_prepare")
         return launches

@@ -275,6 +275,14 @@ extern "C" __global__ void exl3_tc_combine(struct exl3_tc_record record, unsigne
         sum0 = __fadd_rn(sum0, y0);
         sum1 = __fadd_rn(sum1, y1);
     }
+    if (record.shared_sum != 0u) {
+        /* the sum joins the shared expert's bfloat16 row, in place: bfloat16(sum + row), one rounding of the float32
+         * addition's result (source/kernel_exl3_tc.cu:468-471 of the reference); output_offset is not written */
+        uint16_t *shared = (uint16_t *)(arena + record.shared_offset) + (uint64_t)row * H;
+        shared[channel] = float_to_bf16(__fadd_rn(sum0, bf16_to_float(shared[channel])));
+        shared[channel + WAVE] = float_to_bf16(__fadd_rn(sum1, bf16_to_float(shared[channel + WAVE])));
+        return;
+    }
     float *out = (float *)(arena + record.output_offset) + (uint64_t)row * H;
     out[channel] = sum0;
     out[channel + WAVE] = sum1;

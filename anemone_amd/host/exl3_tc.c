@@ -41,8 +41,12 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
                EXL3_TC_MOST_ROWS, MOST_GRID_ROWS);
         return STATUS_INVALID_ARGUMENT;
     }
-    if (record->rotation != 0 || record->shared_sum != 0) {
-        REFUSE("%s: expert rotation and the shared-expert sum are tensor-parallel forms this library does not build", what);
+    if (record->shared_sum > 1u) {
+        REFUSE("%s: shared_sum %u: 0 (the sums to output_offset) or 1 (added to the shared expert's rows in place)", what, record->shared_sum);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if (record->rotation != 0) {
+        REFUSE("%s: expert rotation is a tensor-parallel form this library does not build", what);
         return STATUS_UNSUPPORTED;
     }
     if (I == 0 || I % EXL3_TRANSFORM != 0 || hidden % EXL3_TRANSFORM != 0 || hidden % (32u * EXL3_TC_GATE_UP_SLICES) != 0 ||
@@ -66,8 +70,9 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
         {"the rows", {record->hidden_offset, (uint64_t)record->row_count * hidden * 2u}, (uint64_t)record->row_count * hidden * 2u, false},
         {"the workspace", {record->workspace_offset, workspace}, workspace, false},
         {"the output", {record->output_offset, (uint64_t)record->row_count * hidden * 4u}, (uint64_t)record->row_count * hidden * 4u, false},
+        {"the shared expert's rows", {record->shared_offset, (uint64_t)record->row_count * hidden * 2u}, (uint64_t)record->row_count * hidden * 2u, false},
     };
-    if (!ranges_are_valid(what, ranges, 4, arena_byte_count) || record->workspace_offset % 256u != 0 ||
+    if (!ranges_are_valid(what, ranges, record->shared_sum != 0u ? 5u : 4u, arena_byte_count) || record->workspace_offset % 256u != 0 ||
         (mixed && record->widths_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0)) {
         if (record->workspace_offset % 256u != 0) {
             REFUSE("%s: the workspace begins off a multiple of 256", what);

@@ -299,8 +299,8 @@ struct exl3_tc_record {
     float activation_limit;    /* the SwiGLU limit; 0: none */
     uint32_t pass;             /* the products launches: 0 gate and up, 1 down; the others 0 */
     uint32_t rotation;         /* must be 0: a tensor-parallel feature, not built */
-    uint32_t shared_sum;       /* must be 0 */
-    uint64_t shared_offset;    /* unused */
+    uint32_t shared_sum;       /* 0: each row's sum float32 at output_offset; 1: added to the shared expert's rows, in place */
+    uint64_t shared_offset;    /* shared_sum 1: read and written: bfloat16 [row_count][hidden], bfloat16(sum + row) */
     /* extension */
     uint64_t widths_offset;
     uint32_t hidden;           /* 0: 5120 */

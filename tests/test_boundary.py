@@ -180,13 +180,18 @@ def test_tc_prepare_geometry_and_refusals(fake):
     passes = [amd.Exl3TcRecord.from_buffer_copy(bytes(l.argument)[:88]).pass_ for l in launches]
     assert passes == [0, 0, 0, 1, 0]
     assert amd.exl3_tc_workspace_bytes(64, 4096, 2048) == 64 * 4096 * 4 + 8 * 2 * 64 * 2048 * 4 + 4 * 64 * 4096 * 4
-    for changes, status in [(dict(row_count=0), 1), (dict(row_count=65), 1), (dict(rotation=1), 7), (dict(shared_sum=1), 7),
+    for changes, status in [(dict(row_count=0), 1), (dict(row_count=65), 1), (dict(rotation=1), 7), (dict(shared_sum=2), 1),
+                            (dict(shared_sum=1, shared_offset=ARENA - 4096), 1), (dict(shared_sum=1, shared_offset=1 << 20), 1),
                             (dict(intermediate=2000), 7), (dict(bits_x2=7), 7), (dict(bits_x2=0), 1), (dict(pass_=1), 1),
                             (dict(workspace_offset=(2 << 20) + 16), 1), (dict(output_offset=2 << 20), 1),
                             (dict(activation_limit=-1.0), 1)]:
         untouched = amd.launches_of(5)
         assert lib.exl3_tc_prepare(C.byref(tc_record(**changes)), ARENA, fake.address, fake.card, untouched) == status, changes
         assert not any(bytes(untouched))
+    # the sum into the shared expert's rows: its own range, checked like the others
+    joined = amd.launches_of(5)
+    assert lib.exl3_tc_prepare(C.byref(tc_record(shared_sum=1, shared_offset=3 << 29)), ARENA, fake.address, fake.card, joined) == 0
+    assert amd.Exl3TcRecord.from_buffer_copy(bytes(joined[4].argument)[:88]).shared_sum == 1
     # hidden 0 and pairs_per_row 0 stand for the reference's 5120 and 6
     default = amd.launches_of(5)
     assert lib.exl3_tc_prepare(C.byref(tc_record(hidden=0, pairs_per_row=0, intermediate=640, job_capacity=48)), ARENA,

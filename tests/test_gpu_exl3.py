@@ -199,6 +199,19 @@ def test_chain_and_fused_decode_against_oracle(amd, card, width_choices, rows, l
     fused = layer.output()[:live]
     assert np.max(np.abs(fused - want)) <= 4e-3 * scale, "fused decode output"
     say("  fused max err / rms", float(np.max(np.abs(fused - want)) / scale))
+    # the combine's other form: the same sums added to the shared expert's bfloat16 rows, in place, one rounding;
+    # the float32 output is then not written
+    shared = to_bf16(normals(0x5A7ED, rows * hidden) * float(scale)).reshape(rows, hidden)
+    shared[0, :4] = [0x0000, 0x8000, 0x7F80, 0x7FC0]
+    shared_offset = card.place(shared)
+    card.upload(layer.out_offset, np.full(rows * hidden * 4, 0xEE, dtype=np.uint8))
+    card.run(layer.tc_launches(shared_offset))
+    joined = card.download(shared_offset, rows * hidden * 2, np.uint16).reshape(rows, hidden)
+    expect = to_bf16(fused + bf16_to_f32(shared[:live]))
+    both_nan = np.isnan(bf16_to_f32(joined[:live])) & np.isnan(bf16_to_f32(expect))
+    assert np.array_equal(joined[:live][~both_nan], expect[~both_nan]), "sum + shared row, rounded once"
+    assert np.array_equal(joined[live:], shared[live:]), "rows past the live ones keep their values (a sum of nothing is +0)"
+    assert np.all(card.download(layer.out_offset, rows * hidden * 4, np.uint8) == 0xEE)
     # a row alone keeps its bits: the step of one row against row 0 of the step of all
     if live > 1:
         layer.set_rows(x, 1)
