@@ -62,18 +62,10 @@ __device__ static __forceinline__ uint16_t float_to_half_bits(float value)
 }
 
 /* e^x by a fixed sequence of float32 operations: k = nearest(x log2 e), r = x - k ln 2 in two pieces, a degree-6
- * polynomial in fma form, scaling by ldexp. Written without contraction so that host and card agree bit for bit. */
-__device__ static __forceinline__ float det_expf(float x)
+ * polynomial in fma form, scaling by ldexp. Written without contraction so that host and card agree bit for bit.
+ * det_exp_sequence is the sequence alone, for an x it is defined for (-104 <= x <= 88.8 in det_expf). */
+__device__ static __forceinline__ float det_exp_sequence(float x)
 {
-    if (x != x) {
-        return x;
-    }
-    if (x > 88.8f) {
-        return __builtin_huge_valf();
-    }
-    if (x < -104.0f) {
-        return 0.0f;
-    }
     const float k = __builtin_rintf(__fmul_rn(x, 1.44269502162933349609375f));
     float r = __fmaf_rn(k, -0.693145751953125f, x);
     r = __fmaf_rn(k, -1.42860676533018704503775e-06f, r);
@@ -87,6 +79,32 @@ __device__ static __forceinline__ float det_expf(float x)
     float y = __fmaf_rn(p, r2, r);
     y = __fadd_rn(y, 1.0f);
     return ldexpf(y, (int)k);
+}
+
+__device__ static __forceinline__ float det_expf(float x)
+{
+    if (x != x) {
+        return x;
+    }
+    if (x > 88.8f) {
+        return __builtin_huge_valf();
+    }
+    if (x < -104.0f) {
+        return 0.0f;
+    }
+    return det_exp_sequence(x);
+}
+
+/* gate / (1 + e^(-gate)): the bits of __fdiv_rn(gate, __fadd_rn(1.0f, det_expf(-gate))) for every float32 gate (a NaN
+ * for a NaN), without det_expf's three tests, each of which is a branch of its own and a wait for its comparison in a
+ * kernel's epilogue. The sequence's argument is held inside [-104, 89.5] instead: above 88.8 the sequence overflows to
+ * infinity by itself (k >= 128 and, where k = 128, r > 0.08, so the polynomial is above 1); below -104 det_expf gives 0
+ * and the sequence at -104 something below 2^-148, and 1 plus either is 1; a NaN gate divides to a NaN whatever the
+ * denominator. The library's arithmetic_selfcheck kernel compares the two over all 2^32 gates. */
+__device__ static __forceinline__ float det_silu(float gate)
+{
+    const float x = __builtin_amdgcn_fmed3f(-gate, -104.0f, 89.5f);
+    return __fdiv_rn(gate, __fadd_rn(1.0f, det_exp_sequence(x)));
 }
 
 /* One block of 128 values across a wavefront: lane l holds values l (v0) and l + 64 (v1). Seven stages, the

@@ -37,17 +37,15 @@ extern "C" __global__ void __launch_bounds__(LINEAR_ELEMENT_THREADS)
         largest = fmaxf(largest, __shfl_xor(largest, (int)distance, 8));
     }
     const uint32_t code_exponent = quantize_exponent_code(largest);
-    uint32_t code[4], operand[4];
-#pragma unroll
-    for (uint32_t i = 0; i < 4u; i++) {
-        quantize_code(bits[i], code_exponent, code[i], operand[i]);
-    }
     /* the word's bytes j = 0 .. 3 hold values +0 (j = 0), +8 (1), +1 (2), +9 (3); its operands' halfwords 2 r + h hold
      * value + h + 8 r */
+    const uint32_t in_word_order[4] = {bits[0], bits[2], bits[1], bits[3]};
+    uint32_t codes, carried[4];
+    quantize_codes4(in_word_order, code_exponent, codes, carried);
     const uint32_t word = quantize_word_of(l, s, t);
-    *(uint32_t *)(arena + arguments.codes_offset + vector * arguments.width + word) = code[0] | (code[2] << 8) | (code[1] << 16) | (code[3] << 24);
+    *(uint32_t *)(arena + arguments.codes_offset + vector * arguments.width + word) = codes;
     *(uint2_t *)((uint16_t *)(arena + arguments.operands_offset) + vector * arguments.width + word) =
-        (uint2_t){operand[0] | (operand[1] << 16), operand[2] | (operand[3] << 16)};
+        (uint2_t){quantize_operand_pair(carried[0], carried[2], code_exponent), quantize_operand_pair(carried[1], carried[3], code_exponent)};
     if (q % 8u == 0u) {
         (arena + arguments.exponents_offset)[vector * (arguments.width / 32u) + first / 32u] = (unsigned char)code_exponent;
     }

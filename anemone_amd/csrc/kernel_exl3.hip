@@ -203,7 +203,7 @@ extern "C" __global__ void exl3_activate(struct exl3_expert_record record, unsig
         for (uint32_t i = 0; i < 2u; i++) {
             const float bounded_gate = fminf(gate[i], limit);
             const float bounded_up = fminf(fmaxf(up[i], -limit), limit);
-            hidden[i] = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
+            hidden[i] = __fmul_rn(det_silu(bounded_gate), bounded_up);
         }
         uint16_t *hidden_out = (uint16_t *)(arena + record.hidden_offset) + (uint64_t)pair * I;
         hidden_out[channel] = float_to_bf16(hidden[0]);

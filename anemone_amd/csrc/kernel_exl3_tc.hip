@@ -177,7 +177,7 @@ extern "C" __global__ void exl3_tc_activate(struct exl3_tc_record record, unsign
             const float up = __fmul_rn(__fmul_rn(u[i], EXL3_NORMALIZATION), us[i]);
             const float bounded_gate = limit > 0.0f ? fminf(gate, limit) : gate;
             const float bounded_up = limit > 0.0f ? fminf(fmaxf(up, -limit), limit) : up;
-            const float hidden = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
+            const float hidden = __fmul_rn(det_silu(bounded_gate), bounded_up);
             v[i] = __fmul_rn(hidden, ds[i]);
         }
         wave_hadamard128(v[0], v[1], lane);

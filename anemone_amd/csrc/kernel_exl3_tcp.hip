@@ -494,7 +494,7 @@ extern "C" __global__ void exl3_tcp_activate(struct exl3_tcp_record record, unsi
                 const float up = __fmul_rn(__fmul_rn(u[j], EXL3_NORMALIZATION), us[j]);
                 const float bounded_gate = limit > 0.0f ? fminf(gate, limit) : gate;
                 const float bounded_up = limit > 0.0f ? fminf(fmaxf(up, -limit), limit) : up;
-                const float hidden = __fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up);
+                const float hidden = __fmul_rn(det_silu(bounded_gate), bounded_up);
                 v[j] = __fmul_rn(hidden, ds[j]);
             }
             row_hadamard128(v, lane);

@@ -268,14 +268,14 @@ extern "C" __global__ void trunk_hidden_entry(struct trunk_hidden_arguments argu
 #pragma unroll
         for (uint32_t v = 0; v < HYPER_VALUES_PER_THREAD; v++) {
             const float bounded_gate = fminf(g[v], limit), bounded_up = fminf(fmaxf(u[v], -limit), limit);
-            h[v] = __fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), 1.0f);
+            h[v] = __fmul_rn(__fmul_rn(det_silu(bounded_gate), bounded_up), 1.0f);
         }
         *(uint4_t *)hidden = join_pack(h);
         return;
     }
     for (uint32_t v = 0; v < HYPER_VALUES_PER_THREAD && first + v < arguments.width; v++) {
         const float bounded_gate = fminf(bf16_to_float(gate[v]), limit), bounded_up = fminf(fmaxf(bf16_to_float(up[v]), -limit), limit);
-        hidden[v] = float_to_bf16(__fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), 1.0f));
+        hidden[v] = float_to_bf16(__fmul_rn(__fmul_rn(det_silu(bounded_gate), bounded_up), 1.0f));
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_TRUNK_LINEAR, trunk_hidden_entry, trunk_hidden_arguments);

@@ -89,7 +89,7 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
                     const float gate = bf16_to_float(float_to_bf16(gate_sum)), up = bf16_to_float(float_to_bf16(up_sum));
                     const float bounded_gate = fminf(gate, limit);
                     const float bounded_up = fminf(fmaxf(up, -limit), limit);
-                    const float value = __fmul_rn(__fmul_rn(__fdiv_rn(bounded_gate, __fadd_rn(1.0f, det_expf(-bounded_gate))), bounded_up), weight);
+                    const float value = __fmul_rn(__fmul_rn(det_silu(bounded_gate), bounded_up), weight);
                     bits[j][n][v] = float_to_bf16(value);
                     largest[j] = fmaxf(largest[j], fabsf(bf16_to_float((uint16_t)bits[j][n][v])));
                 }
@@ -138,18 +138,16 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
             uint16_t *operands = (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width;
 #pragma unroll
             for (uint32_t n = 0; n < STRIP; n++) {
-                uint32_t code[4], operand[4];
-#pragma unroll
-                for (uint32_t v = 0; v < 4u; v++) {
-                    quantize_code(bits[j][n][v], code_exponent, code[v], operand[v]);
-                }
+                uint32_t own, carried[4];
+                quantize_codes4(bits[j][n], code_exponent, own, carried);
                 const uint32_t load = (tile0 + n) / 4u, step = (tile0 + n) % 4u, t = 2u * (g % 2u);
                 const uint32_t word0 = quantize_word_of(load, step, t), word1 = quantize_word_of(load, step, t + 1u);
-                const uint32_t half0 = (code[0] | (code[1] << 16)) << (8u * upper), half1 = (code[2] | (code[3] << 16)) << (8u * upper);
-                const uint32_t other = (uint32_t)__shfl_xor((int)(upper != 0u ? half0 : half1), 32, WAVE);
-                *(uint32_t *)(codes + (upper != 0u ? word1 : word0)) = (upper != 0u ? half1 : half0) | other;
-                *(uint32_t *)(operands + word0 + 2u * upper) = operand[0] | (operand[1] << 16);
-                *(uint32_t *)(operands + word1 + 2u * upper) = operand[2] | (operand[3] << 16);
+                /* word0 is (a0, b0, a1, b1) and word1 (a2, b2, a3, b3) of the codes a of the lower lane and b of the
+                 * upper: each takes the other's four and stores one of the words */
+                const uint32_t other = (uint32_t)__shfl_xor((int)own, 32, WAVE);
+                *(uint32_t *)(codes + (upper != 0u ? word1 : word0)) = __builtin_amdgcn_perm(other, own, upper != 0u ? 0x03070206u : 0x05010400u);
+                *(uint32_t *)(operands + word0 + 2u * upper) = quantize_operand_pair(carried[0], carried[1], code_exponent);
+                *(uint32_t *)(operands + word1 + 2u * upper) = quantize_operand_pair(carried[2], carried[3], code_exponent);
             }
             if (g == 0u && first_output % 32u == 0u) {
                 (arena + arguments.hidden_exponents_offset)[pair * (width / 32u) + first_output / 32u] = (unsigned char)code_exponent;

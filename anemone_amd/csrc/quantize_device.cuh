@@ -17,8 +17,10 @@ __device__ static __forceinline__ uint32_t quantize_exponent_code(float largest)
     return ((ratio >> 23) & 255u) + ((ratio & 0x7FFFFFu) != 0u ? 1u : 0u);
 }
 
-/* one bfloat16 value under its block's scale code: its E4M3 code (to nearest even, clamped at 448) and its operand */
-__device__ static __forceinline__ void quantize_code(uint32_t bits, uint32_t code_exponent, uint32_t &code_out, uint32_t &operand_out)
+/* one bfloat16 value under its block's scale code: its E4M3 code (to nearest even, clamped at 448) and its operand.
+ * The definition, in plain arithmetic; the kernels use quantize_codes4 below, which the library's arithmetic_selfcheck
+ * kernel compares with it over every value and every scale code. */
+__device__ static __forceinline__ void quantize_code_defined(uint32_t bits, uint32_t code_exponent, uint32_t &code_out, uint32_t &operand_out)
 {
     const float value = bf16_to_float((uint16_t)bits);
     const float scaled = __fmul_rn(value, __uint_as_float((254u - code_exponent) << 23)); /* exact: a power of two */
@@ -31,6 +33,49 @@ __device__ static __forceinline__ void quantize_code(uint32_t bits, uint32_t cod
     /* the operand: units x 2^(field - 130) x 2^(c - 127) x 2^100, exact, its upper half a bfloat16 */
     const float carried = __fmul_rn((float)units, __uint_as_float((field + code_exponent - 30u) << 23));
     operand_out = (code_exponent <= 146u ? __float_as_uint(carried) >> 16 : 0x7F80u) | (sign << 8);
+}
+
+/* Four values of one block at once, by the card's own conversions: the scaled value, limited to 448 in magnitude (a
+ * NaN becomes 448) under the value's sign, goes through v_cvt_pk_fp8_f32 (E4M3, to nearest even, subnormals of 2^-9);
+ * the operand is the code converted back (v_cvt_pk_f32_fp8) times 2^(c - 27), exact, whose upper half is the
+ * bfloat16. codes: byte i the code of bits[i]; carried[i]: the operand of bits[i] in the upper half of the word, to be
+ * paired by quantize_operand_pair. */
+__device__ static __forceinline__ void quantize_codes4(const uint32_t (&bits)[4], uint32_t code_exponent, uint32_t &codes, uint32_t (&carried)[4])
+{
+    const float down = __uint_as_float((254u - code_exponent) << 23);
+    const float up = __uint_as_float(((code_exponent <= 146u ? code_exponent : 146u) + 100u) << 23);
+    float held[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; i++) {
+        const uint32_t value = bits[i] << 16;
+        const float magnitude = fminf(fabsf(__fmul_rn(__uint_as_float(value), down)), 448.0f);
+        held[i] = __uint_as_float((__float_as_uint(magnitude) & 0x7FFFFFFFu) | (value & 0x80000000u));
+    }
+    int packed = __builtin_amdgcn_cvt_pk_fp8_f32(held[0], held[1], 0, false);
+    packed = __builtin_amdgcn_cvt_pk_fp8_f32(held[2], held[3], packed, true);
+    codes = (uint32_t)packed;
+    const auto low = __builtin_amdgcn_cvt_pk_f32_fp8(packed, false), high = __builtin_amdgcn_cvt_pk_f32_fp8(packed, true);
+    carried[0] = __float_as_uint(__fmul_rn(low[0], up));
+    carried[1] = __float_as_uint(__fmul_rn(low[1], up));
+    carried[2] = __float_as_uint(__fmul_rn(high[0], up));
+    carried[3] = __float_as_uint(__fmul_rn(high[1], up));
+}
+
+/* two operands as one word (first in the low half); a scale code above 146 makes every operand an infinity of its sign */
+__device__ static __forceinline__ uint32_t quantize_operand_pair(uint32_t first, uint32_t second, uint32_t code_exponent)
+{
+    const uint32_t pair = __builtin_amdgcn_perm(second, first, 0x07060302u);
+    return code_exponent <= 146u ? pair : (pair & 0x80008000u) | 0x7F807F80u;
+}
+
+/* one value by the same route (the three others zero) */
+__device__ static __forceinline__ void quantize_code(uint32_t bits, uint32_t code_exponent, uint32_t &code_out, uint32_t &operand_out)
+{
+    const uint32_t four[4] = {bits, 0u, 0u, 0u};
+    uint32_t codes, carried[4];
+    quantize_codes4(four, code_exponent, codes, carried);
+    code_out = codes & 0xFFu;
+    operand_out = quantize_operand_pair(carried[0], 0u, code_exponent) & 0xFFFFu;
 }
 
 /* where the values of a vector go: value `index` = 64 load + 16 step + u lies in word ((4 load + t) 4 + step) with
