@@ -180,6 +180,25 @@ class ExpertJoinArguments(C.Structure):
                 ("comb_offset", u64), ("row_sums_offset", u64), ("pairs_per_row", u32), ("reserved_zero", u32)]
 
 
+class DenseLinearKernels(C.Structure):
+    _fields_ = [("products", u32 * 8)]
+
+
+class DenseLinearDescription(C.Structure):
+    _fields_ = [("weights", Range), ("rows", Range), ("output", Range), ("step", Range), ("output_size", u32), ("input_size", u32),
+                ("row_count", u32), ("weight_type", u32), ("output_type", u32), ("flags", u32), ("output_scale", f32),
+                ("epsilon", f32), ("cone_layer", u32)]
+
+
+class HyperKernelsRecord(C.Structure):
+    _fields_ = [(name, u32) for name in ("mix_finish", "final_collapse", "post", "embed", "draft_inputs", "final_kept")]
+
+
+class HyperSiteDescription(C.Structure):
+    _fields_ = [(name, Range) for name in ("streams", "carried_pre", "mixes", "scale", "base", "norm_weight", "post", "comb", "hidden",
+                                           "output", "routed_sums")] + [("row_count", u32), ("reserved_zero", u32)]
+
+
 class LinearWideKernels(C.Structure):
     _fields_ = [("wide_expert_gate_up", u32), ("wide_expert_down", u32), ("wide_expert_gate_up_e4m3", u32), ("wide_expert_down_e4m3", u32),
                 ("wide_expert_gate_up_b128", u32), ("wide_expert_down_b128", u32)]
@@ -254,6 +273,10 @@ def library():
             "linear_trunk_quantized_prepare": [C.POINTER(TrunkQuantizedDescription), u64, C.POINTER(LinearKernels), launch_p],
             "linear_shared_expert_prepare": [C.POINTER(SharedExpertDescription), u64, C.POINTER(LinearKernels), launch_p],
             "expert_join_prepare": [C.POINTER(ExpertJoinDescription), u64, C.POINTER(ExpertFusedKernels), launch_p],
+            "dense_linear_kernels_prepare": [vp, vp, C.POINTER(DenseLinearKernels)],
+            "dense_linear_prepare": [C.POINTER(DenseLinearDescription), u64, C.POINTER(DenseLinearKernels), launch_p],
+            "hyper_kernels_prepare": [vp, vp, C.POINTER(HyperKernelsRecord)],
+            "hyper_site_prepare": [C.POINTER(HyperSiteDescription), u64, C.POINTER(HyperKernelsRecord), launch_p],
             "expert_post_prepare": [C.POINTER(ExpertJoinDescription), u64, u32, launch_p],
             "expert_shared_join_prepare": [C.POINTER(ExpertSharedJoinDescription), u64, C.POINTER(LinearKernels),
                                            C.POINTER(ExpertFusedKernels), launch_p],
@@ -799,6 +822,68 @@ class Fp4Layer:
 LINEAR_WIDE_GROUP_BLOCKS, LINEAR_WIDE_TILE_BLOCKS, LINEAR_INTERLEAVED_CHUNK_BLOCKS, LINEAR_INTERLEAVED_TILE_BLOCKS = 0, 1, 2, 3
 LINEAR_MAXIMUM_ROWS = 8
 MODEL_STREAMS = 4
+
+
+DENSE_BFLOAT16, DENSE_FLOAT32, DENSE_ROW_SCALE = 0, 1, 1
+MODEL_MIXES, MODEL_NORM_EPSILON = 24, 1e-20
+
+
+class SiteFront:
+    """The step ahead of a layer's routed experts, as the launches the reference's fused site front stands for: the mix
+    project (the dense product of the site's float32 mix weights [24][4 width] with the streams as its rows, scaled by
+    the row's reciprocal root mean square), the mix finish (pre, post and comb by Sinkhorn, the collapse of the streams
+    with the carried pre and its norm: the sublayer's input) and, behind the sublayer, the post. The router's scores in
+    the dense product's order are scores_launch. Arrays live in the arena of `card`."""
+
+    def __init__(self, card, rows, width, mix_weights, scale, base, norm_weight_bf16, hidden_range=None):
+        self.card, self.rows, self.width = card, rows, width
+        self.constants = {"mix_weights": np.ascontiguousarray(mix_weights, dtype=np.float32), "scale": np.ascontiguousarray(scale, dtype=np.float32),
+                          "base": np.ascontiguousarray(base, dtype=np.float32), "norm_weight": np.ascontiguousarray(norm_weight_bf16, dtype=np.uint16)}
+        assert self.constants["mix_weights"].shape == (MODEL_MIXES, MODEL_STREAMS * width)
+        self.ranges = {name: Range(card.place(array, 256), array.nbytes) for name, array in self.constants.items()}
+        sizes = {"streams": rows * MODEL_STREAMS * width * 2, "carried_pre": rows * MODEL_STREAMS * 4, "mixes": rows * MODEL_MIXES * 4,
+                 "post": rows * MODEL_STREAMS * 4, "comb": rows * MODEL_STREAMS * MODEL_STREAMS * 4, "output": rows * width * 2,
+                 "routed_sums": rows * width * 4}
+        if hidden_range is None:
+            sizes["hidden"] = rows * width * 2
+        else:
+            self.ranges["hidden"] = hidden_range
+        self.ranges.update({name: Range(card.reserve(size), size) for name, size in sizes.items()})
+        self.dense_kernels, self.hyper_kernels = DenseLinearKernels(), HyperKernelsRecord()
+        check(card.lib.dense_linear_kernels_prepare(backend_table(), card.handle, C.byref(self.dense_kernels)), "dense_linear_kernels_prepare")
+        check(card.lib.hyper_kernels_prepare(backend_table(), card.handle, C.byref(self.hyper_kernels)), "hyper_kernels_prepare")
+
+    def set_streams(self, streams_bf16, carried_pre):
+        self.card.upload(self.ranges["streams"].byte_offset, np.ascontiguousarray(streams_bf16, dtype=np.uint16))
+        self.card.upload(self.ranges["carried_pre"].byte_offset, np.ascontiguousarray(carried_pre, dtype=np.float32))
+
+    def dense_launch(self, weights, rows_range, output, output_size, input_size, weight_type, output_type=DENSE_FLOAT32, flags=0, scale=1.0,
+                     epsilon=0.0, rows=None):
+        d = DenseLinearDescription()
+        d.weights, d.rows, d.output, d.step = weights, rows_range, output, Range(0, 0)
+        d.output_size, d.input_size, d.row_count = output_size, input_size, self.rows if rows is None else rows
+        d.weight_type, d.output_type, d.flags, d.output_scale, d.epsilon = weight_type, output_type, flags, scale, epsilon
+        launch = launches_of(1)
+        check(self.card.lib.dense_linear_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.dense_kernels), launch), "dense_linear_prepare")
+        return launch
+
+    def mix_project_launch(self, rows=None):
+        return self.dense_launch(self.ranges["mix_weights"], self.ranges["streams"], self.ranges["mixes"], MODEL_MIXES, MODEL_STREAMS * self.width,
+                                 DENSE_FLOAT32, DENSE_FLOAT32, DENSE_ROW_SCALE, 1.0, MODEL_NORM_EPSILON, rows)
+
+    def site_launches(self, rows=None, combined=False):
+        """[the mix finish, the post] (hyper_site_prepare)."""
+        d = HyperSiteDescription()
+        for name in ("streams", "carried_pre", "mixes", "scale", "base", "norm_weight", "post", "comb", "hidden", "output"):
+            setattr(d, name, self.ranges[name])
+        d.routed_sums = self.ranges["routed_sums"] if combined else Range(0, 0)
+        d.row_count, d.reserved_zero = self.rows if rows is None else rows, self.width
+        launches = launches_of(2)
+        check(self.card.lib.hyper_site_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.hyper_kernels), launches), "hyper_site_prepare")
+        return launches
+
+    def read(self, name, dtype=np.uint8):
+        return self.card.download(self.ranges[name].byte_offset, self.ranges[name].byte_count, dtype)
 
 
 class SharedExpert:

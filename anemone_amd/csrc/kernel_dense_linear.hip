@@ -1,0 +1,157 @@
+/*
+ * kernel_dense_linear.hip -- the dense products of a step of 1 to 8 rows on gfx950: y = W x for a matrix as the
+ * checkpoint stores it (bfloat16 or float32, row-major) and bfloat16 rows: a site's mix project (float32
+ * [24][4 width], with the row's scale) and the router's scores of the site front's order. Entry names, record and
+ * arithmetic follow the reference (include/anemone/dense_linear_records.h:10-30, source/kernel_dense_linear.cu:40-175):
+ *   - thread t of 256 takes the chunks t, t + 256, ... of 8 inputs; its chain of an output and a row runs from +0 in
+ *     ascending input order, fmaf(weight, value, chain), both widened exactly;
+ *   - a group of 32 threads adds its chains by exchanges at distance 16 down to 1, then the 8 groups' sums are added
+ *     from +0 in ascending order;
+ *   - DENSE_ROW_SCALE: the sum times r(q (1 / input_size) + epsilon), q the row's squares (fmaf(value, value, q)) added
+ *     in the same order; r is the float32 nearest the reciprocal square root (the reference takes its card's rsqrtf);
+ *   - a float32 output is the value times output_scale; a bfloat16 one is rounded, multiplied and rounded again.
+ * DENSE_STEP_ROWS and DENSE_CONE_ROWS (the head's and the prefill cone's rows) are not built: the host refuses them.
+ *
+ * Work mapping: a wavefront holds two of the definition's groups of 32 (an exchange at a distance below 32 stays inside
+ * its half); a thread asks for all its chunks' weights ahead (a step's matrices are 2 to 4 MB: the launch is a few
+ * round trips to memory, not a stream), the rows come from the caches (every block reads the same rows).
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kernel_registry.h"
+#include "exl3_device.cuh"
+
+#define DENSE_GROUP_LANES 32u
+#define DENSE_GROUPS (DENSE_THREADS_VALUE / DENSE_GROUP_LANES)
+
+__device__ static __forceinline__ float dense_group_sum(float value)
+{
+#pragma unroll
+    for (uint32_t distance = DENSE_GROUP_LANES / 2u; distance != 0u; distance /= 2u) {
+        value = __fadd_rn(value, __shfl_xor(value, (int)distance, (int)DENSE_GROUP_LANES));
+    }
+    return value;
+}
+
+/* the float32 nearest 1 / sqrt(operand): both steps are correctly rounded in double, whose 53 places decide a tie */
+__device__ static __forceinline__ float dense_reciprocal_root(float operand)
+{
+    return (float)(1.0 / __dsqrt_rn((double)operand));
+}
+
+template <uint32_t TYPE, uint32_t ROWS, uint32_t OUTPUTS>
+__device__ static __forceinline__ void dense_linear(const struct dense_linear_arguments &arguments, unsigned char *arena)
+{
+    __shared__ float group_sums[DENSE_GROUPS][OUTPUTS + 1u][ROWS];
+    const uint32_t thread = threadIdx.x, inputs = arguments.input_size, chunks = inputs / DENSE_CHUNK_INPUTS;
+    const uint32_t first_output = blockIdx.x * OUTPUTS;
+    const bool scaled = (arguments.flags & DENSE_ROW_SCALE) != 0u;
+    const uint16_t *rows = (const uint16_t *)(arena + arguments.rows_offset);
+    float chain[OUTPUTS][ROWS], squares[ROWS];
+#pragma unroll
+    for (uint32_t r = 0; r < ROWS; r++) {
+        squares[r] = 0.0f;
+#pragma unroll
+        for (uint32_t o = 0; o < OUTPUTS; o++) {
+            chain[o][r] = 0.0f;
+        }
+    }
+    for (uint32_t chunk = thread; chunk < chunks; chunk += DENSE_THREADS_VALUE) {
+        float values[ROWS][DENSE_CHUNK_INPUTS];
+#pragma unroll
+        for (uint32_t r = 0; r < ROWS; r++) {
+            /* a column from row_count on reads row 0 and is stored nowhere */
+            const uint32_t row = r < arguments.row_count ? r : 0u;
+            unpack_bf16x8(*(const uint4_t *)(rows + (uint64_t)row * inputs + chunk * DENSE_CHUNK_INPUTS), values[r]);
+            if (scaled) {
+#pragma unroll
+                for (uint32_t i = 0; i < DENSE_CHUNK_INPUTS; i++) {
+                    squares[r] = __fmaf_rn(values[r][i], values[r][i], squares[r]);
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t o = 0; o < OUTPUTS; o++) {
+            float weights[DENSE_CHUNK_INPUTS];
+            const uint64_t at = (uint64_t)(first_output + o) * inputs + chunk * DENSE_CHUNK_INPUTS;
+            if constexpr (TYPE == DENSE_FLOAT32) {
+                const float4_t low = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at);
+                const float4_t high = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at + 4u);
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; i++) {
+                    weights[i] = low[i];
+                    weights[4u + i] = high[i];
+                }
+            } else {
+                unpack_bf16x8(*(const uint4_t *)((const uint16_t *)(arena + arguments.weights_offset) + at), weights);
+            }
+#pragma unroll
+            for (uint32_t r = 0; r < ROWS; r++) {
+#pragma unroll
+                for (uint32_t i = 0; i < DENSE_CHUNK_INPUTS; i++) {
+                    chain[o][r] = __fmaf_rn(weights[i], values[r][i], chain[o][r]);
+                }
+            }
+        }
+    }
+    const uint32_t group = thread / DENSE_GROUP_LANES, lane = thread % DENSE_GROUP_LANES;
+#pragma unroll
+    for (uint32_t r = 0; r < ROWS; r++) {
+#pragma unroll
+        for (uint32_t o = 0; o < OUTPUTS; o++) {
+            const float sum = dense_group_sum(chain[o][r]);
+            if (lane == 0u) {
+                group_sums[group][o][r] = sum;
+            }
+        }
+        if (scaled) {
+            const float sum = dense_group_sum(squares[r]);
+            if (lane == 0u) {
+                group_sums[group][OUTPUTS][r] = sum;
+            }
+        }
+    }
+    __syncthreads();
+    if (thread >= OUTPUTS * ROWS) {
+        return;
+    }
+    const uint32_t o = thread / ROWS, r = thread % ROWS;
+    if (r >= arguments.row_count) {
+        return;
+    }
+    float sum = 0.0f, square_sum = 0.0f;
+#pragma unroll
+    for (uint32_t g = 0; g < DENSE_GROUPS; g++) {
+        sum = __fadd_rn(sum, group_sums[g][o][r]);
+        if (scaled) {
+            square_sum = __fadd_rn(square_sum, group_sums[g][OUTPUTS][r]);
+        }
+    }
+    if (scaled) {
+        const float operand = __fadd_rn(__fmul_rn(square_sum, __fdiv_rn(1.0f, (float)inputs)), arguments.epsilon);
+        sum = __fmul_rn(sum, dense_reciprocal_root(operand));
+    }
+    const uint64_t index = (uint64_t)r * arguments.output_size + first_output + o;
+    if (arguments.output_type == DENSE_FLOAT32) {
+        ((float *)(arena + arguments.output_offset))[index] = __fmul_rn(sum, arguments.output_scale);
+    } else {
+        ((uint16_t *)(arena + arguments.output_offset))[index] = float_to_bf16(__fmul_rn(bf16_to_float(float_to_bf16(sum)), arguments.output_scale));
+    }
+}
+
+#define DENSE_STAMP(name, type, rows, outputs, form)                                                                                  \
+    extern "C" __global__ void __launch_bounds__(DENSE_THREADS_VALUE)                                                                 \
+        dense_linear_##name##_##rows##form(struct dense_linear_arguments arguments, unsigned char *arena)                             \
+    {                                                                                                                                 \
+        dense_linear<type, rows, outputs>(arguments, arena);                                                                          \
+    }                                                                                                                                 \
+    ANEMONE_KERNEL(KERNEL_FILE_DENSE_LINEAR, dense_linear_##name##_##rows##form, dense_linear_arguments);
+DENSE_STAMP(bfloat16, DENSE_BFLOAT16, 1, DENSE_OUTPUTS_PER_BLOCK, )
+DENSE_STAMP(bfloat16, DENSE_BFLOAT16, 8, DENSE_OUTPUTS_PER_BLOCK, )
+DENSE_STAMP(float32, DENSE_FLOAT32, 1, DENSE_OUTPUTS_PER_BLOCK, )
+DENSE_STAMP(float32, DENSE_FLOAT32, 8, DENSE_OUTPUTS_PER_BLOCK, )
+DENSE_STAMP(bfloat16, DENSE_BFLOAT16, 1, 1u, _narrow)
+DENSE_STAMP(bfloat16, DENSE_BFLOAT16, 8, 1u, _narrow)
+DENSE_STAMP(float32, DENSE_FLOAT32, 1, 1u, _narrow)
+DENSE_STAMP(float32, DENSE_FLOAT32, 8, 1u, _narrow)

@@ -441,4 +441,76 @@ uint64_t linear_jobs_byte_count(uint64_t job_count);                         /* 
 #ifdef __cplusplus
 }
 #endif
+
+/* ---- the launches a block's site front stands for (the step ahead of the routed experts) ----
+ * The reference merges a site's mix project, its mix finish, the router's scores, the select and the quantization of
+ * the sublayer's input into one launch (include/anemone/site_front.h:2-20, site_front_records.h:10-37), which writes
+ * "the same bits: only launches merge". Built here: the launches themselves, each the reference's own entry point --
+ * the dense product (include/anemone/dense_linear.h:27-99, source/dense_linear.c) and the site's mix finish and post
+ * (include/anemone/hyper_connection.h:25-71, source/hyper_connection.c); the select and the quantizer are router.h's
+ * and linear.h's above. */
+struct dense_linear_kernels {
+    uint32_t products[DENSE_INSTANCES]; /* [form][type][one row, 8]: dense_linear_<type>_<R>, then _narrow */
+};
+MUST_CHECK result_status dense_linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                                      struct dense_linear_kernels *kernels_out);
+
+/* include/anemone/dense_linear.h:70-99 of the reference. Refused with STATUS_INVALID_ARGUMENT: a NULL argument, a
+ * type outside the enumeration, a flag outside DENSE_FLAGS, an output_size that is no multiple of
+ * DENSE_OUTPUTS_PER_BLOCK or an input_size that is no multiple of DENSE_CHUNK_INPUTS, 0 rows, a range that breaks the
+ * range rules; with STATUS_UNSUPPORTED: more than LINEAR_MAXIMUM_ROWS rows (the wide launches), DENSE_STEP_ROWS and
+ * DENSE_CONE_ROWS. */
+struct dense_linear_description {
+    struct linear_range weights; /* read: [output_size][input_size] of weight_type, exactly */
+    struct linear_range rows;    /* read: bf16 [row_count][input_size] */
+    struct linear_range output;  /* written: [row_count][output_size] of output_type */
+    struct linear_range step;    /* no bytes */
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t row_count;
+    uint32_t weight_type; /* enum dense_type_code */
+    uint32_t output_type;
+    uint32_t flags;       /* DENSE_ROW_SCALE or 0 */
+    float output_scale;   /* 1 for none */
+    float epsilon;        /* of DENSE_ROW_SCALE */
+    uint32_t cone_layer;  /* 0 */
+};
+MUST_CHECK result_status dense_linear_prepare(const struct dense_linear_description *description, uint64_t arena_byte_count,
+                                              const struct dense_linear_kernels *kernels, struct kernel_launch *launch_out);
+
+/* include/anemone/hyper_connection.h:25-38: the handles of kernel_hyper_connection; the final collapse, the embedding
+ * and the draft's two are not built and stay BACKEND_NO_KERNEL. */
+struct hyper_kernels_record {
+    uint32_t mix_finish;
+    uint32_t final_collapse;
+    uint32_t post;
+    uint32_t embed;
+    uint32_t draft_inputs;
+    uint32_t final_kept;
+};
+MUST_CHECK result_status hyper_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                               struct hyper_kernels_record *kernels_out);
+
+/* A site of a block (include/anemone/hyper_connection.h:40-71): its mix finish, between its mix project and its
+ * sublayer, and its post after the sublayer, with the combine where routed_sums has bytes (the FFN site). 1 to
+ * LINEAR_MAXIMUM_ROWS rows. */
+enum hyper_site_launch { HYPER_SITE_MIX_FINISH = 0, HYPER_SITE_POST = 1, HYPER_SITE_LAUNCH_COUNT = 2 };
+struct hyper_site_description {
+    struct linear_range streams;     /* read and written: bf16 [row_count][4][width] */
+    struct linear_range carried_pre; /* read and written: float32 [row_count][4] */
+    struct linear_range mixes;       /* read: float32 [row_count][24] */
+    struct linear_range scale;       /* read: float32 [3], exactly */
+    struct linear_range base;        /* read: float32 [24], exactly */
+    struct linear_range norm_weight; /* read: bf16 [width], exactly */
+    struct linear_range post;        /* written, then read: float32 [row_count][4] */
+    struct linear_range comb;        /* written, then read: float32 [row_count][4][4] */
+    struct linear_range hidden;      /* written: bf16 [row_count][width], the sublayer's input */
+    struct linear_range output;      /* read: bf16 [row_count][width], the sublayer's output or the shared expert's */
+    struct linear_range routed_sums; /* read: float32 [row_count][width], or no bytes */
+    uint32_t row_count;
+    uint32_t reserved_zero;          /* extension: the streams' width, a multiple of 1,024 up to 8,192; 0 stands for 5,120 */
+};
+MUST_CHECK result_status hyper_site_prepare(const struct hyper_site_description *description, uint64_t arena_byte_count,
+                                            const struct hyper_kernels_record *kernels, struct kernel_launch *launches_out);
+
 #endif

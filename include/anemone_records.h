@@ -618,4 +618,64 @@ struct expert_shared_join_arguments {
 };
 ANEMONE_RECORD_HAS(expert_shared_join_arguments, 96);
 
+/* ---- the launches a site front stands for: the mix finish and the dense product ----
+ * include/anemone/hyper_connection_records.h:46-84 and include/anemone/dense_linear_records.h:56-148 of the reference. */
+#define KERNEL_HYPER_MIX_FINISH "hyper_mix_finish"
+#define MODEL_MIXES 24u                 /* (2 + streams) x streams: pre, post, comb */
+#define MODEL_HYPER_EPSILON 1e-6f
+#define MODEL_NORM_EPSILON 1e-20f
+#define MODEL_SINKHORN_ITERATIONS 20u
+#define HYPER_SCALES 3u                 /* pre, post, comb */
+#define HYPER_FINISH_MOST_THREADS 1024u /* a row's values over 8: the widths 256 .. 8192 in whole groups of 32 threads */
+
+/* Launch: grid (1, rows), block width / 8: a thread eight values of the row; the width is what the block covers (the
+ * reference fixes 5,120 and adds a group of 32 threads for Sinkhorn: here the first sixteen threads do it behind the
+ * barrier). */
+struct hyper_finish_arguments {
+    uint64_t streams_offset; /* read: bf16 [row][4][width] */
+    uint64_t pre_offset;     /* float32 [row][4]: the carried pre, read; then the site's, written */
+    uint64_t mixes_offset;   /* read: float32 [row][24] */
+    uint64_t scale_offset;   /* read: float32 [3] */
+    uint64_t base_offset;    /* read: float32 [24] */
+    uint64_t post_offset;    /* written: float32 [row][4] */
+    uint64_t comb_offset;    /* written: float32 [row][4][4] */
+    uint64_t weight_offset;  /* read: the norm's, bf16 [width] */
+    uint64_t hidden_offset;  /* written: bf16 [row][width] */
+};
+ANEMONE_RECORD_HAS(hyper_finish_arguments, 72);
+
+#define KERNEL_FILE_DENSE_LINEAR "kernel_dense_linear"
+#define KERNEL_DENSE_LINEAR_STEM "dense_linear_"
+#define DENSE_OUTPUTS_PER_BLOCK 4u
+#define DENSE_NARROW_BELOW_BLOCKS 256u /* fewer blocks than this: a block owns one output, so that more units read */
+#define DENSE_CHUNK_INPUTS 8u
+#define DENSE_THREADS_VALUE 256u
+#define DENSE_ROW_SCALE 0x1u
+#define DENSE_STEP_ROWS 0x2u /* not built: the head's */
+#define DENSE_CONE_ROWS 0x4u /* not built: the prefill cone's */
+#define DENSE_FLAGS (DENSE_ROW_SCALE | DENSE_STEP_ROWS | DENSE_CONE_ROWS)
+enum dense_type_code { DENSE_BFLOAT16 = 0, DENSE_FLOAT32 = 1, DENSE_TYPE_COUNT = 2 };
+#define DENSE_FORMS 2u          /* four outputs a block, then one (narrow) */
+#define DENSE_INSTANCES 8u      /* forms by types by row counts: [form][type][one row, 8] */
+#define DENSE_FORM_INSTANCES 4u
+#define DENSE_ROW_INSTANCES 2u
+
+/* Launch: function dense_linear_<type>_<R>[_narrow], R 1 for one row and 8 for 2 to 8; grid (output_size / outputs of
+ * a block, 1), block 256. */
+struct dense_linear_arguments {
+    uint64_t weights_offset; /* read: [output_size][input_size] of the instance's type */
+    uint64_t rows_offset;    /* read: bf16 [row_count][input_size] */
+    uint64_t output_offset;  /* written: [row_count][output_size] of output_type */
+    uint64_t step_offset;    /* not read (DENSE_STEP_ROWS and _CONE_ROWS are not built) */
+    uint32_t output_size;
+    uint32_t input_size;
+    uint32_t row_count;
+    uint32_t output_type;    /* enum dense_type_code */
+    uint32_t flags;          /* DENSE_ROW_SCALE or 0 */
+    float output_scale;
+    float epsilon;           /* of DENSE_ROW_SCALE */
+    uint32_t cone_layer;     /* 0 */
+};
+ANEMONE_RECORD_HAS(dense_linear_arguments, 64);
+
 #endif

@@ -81,6 +81,13 @@ def _load_oracle():
         "orc_hyper_post": (None, [u16p, f32p, f32p, u16p, f32p, u32, u16p]),
         "orc_expert_join": (None, [u16p, u16p, u16p, f32p, f32p, f32p, u32, u32, u32]),
         "orc_trunk_hidden": (None, [u16p, u16p, f32, u32, u16p]),
+        "orc_reciprocal_root": (f32, [f32]),
+        "orc_dense_linear": (i32, [u32, vp, u32, u32, u32, f32, f32, u32, u16p, u32, vp]),
+        "orc_hyper_sinkhorn": (None, [f32p, f32p, f32p, f32p, f32p, f32p]),
+        "orc_hyper_mix_finish": (None, [u16p, f32p, f32p, f32p, f32p, u16p, u32, f32p, f32p, u16p]),
+        "orc_hyper_collapse": (None, [u16p, f32p, u32, u16p]),
+        "orc_hyper_norm_operand": (f32, [u16p, u32]),
+        "orc_hyper_norm_with": (None, [u16p, u16p, f32, u32, u16p]),
     }
     for name, (restype, argtypes) in sig.items():
         fn = getattr(lib, name)
@@ -141,6 +148,23 @@ def _load_ref():
     if hasattr(lib, "test_hyper_post"):
         lib.test_hyper_post.restype = None
         lib.test_hyper_post.argtypes = [u16p, f32p, f32p, u16p, f32p, u16p]
+        lib.test_hyper_sinkhorn.restype = None
+        lib.test_hyper_sinkhorn.argtypes = [f32p, f32p, f32p, f32p, f32p, f32p]
+        lib.test_hyper_collapse.restype = None
+        lib.test_hyper_collapse.argtypes = [u16p, f32p, u16p]
+        lib.test_hyper_norm_operand.restype = f32
+        lib.test_hyper_norm_operand.argtypes = [u16p]
+        lib.test_hyper_reciprocal_root.restype = f32
+        lib.test_hyper_reciprocal_root.argtypes = [f32]
+        lib.test_hyper_norm_with.restype = None
+        lib.test_hyper_norm_with.argtypes = [u16p, u16p, f32, u16p]
+        lib.test_hyper_float_places.restype = u32
+        lib.test_hyper_float_places.argtypes = [f32, f32]
+    if hasattr(lib, "test_dense_reference"):
+        lib.test_dense_reference.restype = None
+        lib.test_dense_reference.argtypes = [u32, C.c_void_p, u32, u32, f32, u16p, u32, u32, u32, f64p, f64p]
+        lib.test_dense_output_holds.restype = C.c_bool
+        lib.test_dense_output_holds.argtypes = [u32, f32, C.c_void_p, C.c_uint64, C.c_double, C.c_double]
     return lib
 
 

@@ -705,3 +705,83 @@ def test_block128_prepare_geometry_and_refusals(fake):
     assert lib.linear_wide_experts_block128_prepare(C.byref(wide_experts_description(amd.WEIGHT_FORMAT_E4M3_SCALED)), arena, C.byref(linear),
                                                     C.byref(wide_kernels), three) == 1
     assert not any(bytes(three))
+
+
+def site_description(rows=8, width=4096, combined=True, **changes):
+    d = amd.HyperSiteDescription()
+    at, w = 1 << 20, width if width != 0 else 5120
+    sizes = {"streams": rows * 4 * w * 2, "carried_pre": rows * 16, "mixes": rows * 96, "scale": 12, "base": 96, "norm_weight": w * 2,
+             "post": rows * 16, "comb": rows * 64, "hidden": rows * w * 2, "output": rows * w * 2, "routed_sums": rows * w * 4}
+    for name, size in sizes.items():
+        setattr(d, name, amd.Range(at, size))
+        at += (size + 255) // 256 * 256
+    if not combined:
+        d.routed_sums = amd.Range(0, 0)
+    d.row_count, d.reserved_zero = rows, width
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d
+
+
+def dense_description(outputs=24, inputs=16384, rows=8, weight_type=1, output_type=1, flags=1, **changes):
+    d = amd.DenseLinearDescription()
+    d.weights = amd.Range(1 << 20, outputs * inputs * (4 if weight_type == 1 else 2))
+    d.rows = amd.Range(1 << 28, rows * inputs * 2)
+    d.output = amd.Range(1 << 29, rows * outputs * (4 if output_type == 1 else 2))
+    d.output_size, d.input_size, d.row_count, d.weight_type, d.output_type, d.flags = outputs, inputs, rows, weight_type, output_type, flags
+    d.output_scale, d.epsilon = 1.0, 1e-20
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d
+
+
+def test_site_front_launches_geometry_and_refusals(fake):
+    """The dense product and the hyper site: the reference's entry points (include/anemone/dense_linear.h:70-99,
+    include/anemone/hyper_connection.h:40-71), instances, geometry and refusals."""
+    lib = amd.library()
+    arena = 8 << 30
+    dense, hyper = amd.DenseLinearKernels(), amd.HyperKernelsRecord()
+    assert lib.dense_linear_kernels_prepare(fake.address, fake.card, C.byref(dense)) == 0
+    assert lib.hyper_kernels_prepare(fake.address, fake.card, C.byref(hyper)) == 0
+    names = [fake.handles[handle][1] for handle in dense.products]
+    assert names == ["dense_linear_bfloat16_1", "dense_linear_bfloat16_8", "dense_linear_float32_1", "dense_linear_float32_8",
+                     "dense_linear_bfloat16_1_narrow", "dense_linear_bfloat16_8_narrow", "dense_linear_float32_1_narrow", "dense_linear_float32_8_narrow"]
+    assert fake.handles[hyper.mix_finish] == ("kernel_hyper_connection", "hyper_mix_finish") and fake.handles[hyper.post][1] == "hyper_post_entry"
+    assert hyper.final_collapse == hyper.embed == hyper.draft_inputs == hyper.final_kept == amd.BACKEND_NO_KERNEL
+    table = kernel_table()
+    assert table[("kernel_dense_linear", "dense_linear_float32_8_narrow")] == 64 and table[("kernel_hyper_connection", "hyper_mix_finish")] == 72
+    launch = amd.launches_of(1)
+    # the mix project: 24 outputs are fewer than 256 blocks of four: the narrow form, a block an output
+    assert lib.dense_linear_prepare(C.byref(dense_description()), arena, C.byref(dense), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "dense_linear_float32_8_narrow" and list(launch[0].grid) == [24, 1, 1] and launch[0].block[0] == 256
+    assert launch[0].argument_byte_count == 64
+    one = dense_description(outputs=4096, inputs=2048, rows=1, weight_type=0, output_type=0, flags=0)
+    assert lib.dense_linear_prepare(C.byref(one), arena, C.byref(dense), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "dense_linear_bfloat16_1" and list(launch[0].grid) == [1024, 1, 1]
+    untouched = amd.launches_of(1)
+    for changes, status in [(dict(row_count=0), 1), (dict(row_count=9), 7), (dict(flags=3), 7), (dict(flags=8), 1), (dict(weight_type=2), 1),
+                            (dict(output_size=26), 1), (dict(input_size=16388), 1), (dict(cone_layer=1), 7),
+                            (dict(weights=amd.Range(1 << 20, 24 * 16384 * 4 + 16)), 1), (dict(output=amd.Range((1 << 20) + 256, 1024)), 1)]:
+        assert lib.dense_linear_prepare(C.byref(dense_description(**changes)), arena, C.byref(dense), untouched) == status, changes
+        assert not any(bytes(untouched))
+    # a site: the mix finish and the post
+    launches = amd.launches_of(2)
+    d = site_description()
+    assert lib.hyper_site_prepare(C.byref(d), arena, C.byref(hyper), launches) == 0
+    assert [fake.handles[l.kernel][1] for l in launches] == ["hyper_mix_finish", "hyper_post_entry"]
+    assert list(launches[0].grid) == [1, 8, 1] and launches[0].block[0] == 512 and launches[0].argument_byte_count == 72
+    assert list(launches[1].grid) == [4, 8, 1] and launches[1].block[0] == 128 and launches[1].argument_byte_count == 48
+    import struct
+    finish = struct.unpack("<9Q", bytes(launches[0].argument)[:72])
+    assert finish == tuple(getattr(d, name).byte_offset for name in ("streams", "carried_pre", "mixes", "scale", "base", "post", "comb", "norm_weight", "hidden"))
+    post = struct.unpack("<5QII", bytes(launches[1].argument)[:48])
+    assert post == (d.streams.byte_offset, d.post.byte_offset, d.comb.byte_offset, d.output.byte_offset, d.routed_sums.byte_offset, 1, 0)
+    plain = site_description(combined=False, width=0, rows=3)  # the attention site's post; the reference's width
+    assert lib.hyper_site_prepare(C.byref(plain), arena, C.byref(hyper), launches) == 0
+    assert launches[0].block[0] == 640 and list(launches[1].grid) == [5, 3, 1]
+    assert struct.unpack("<5QII", bytes(launches[1].argument)[:48])[4:] == (0, 0, 0)
+    untouched = amd.launches_of(2)
+    for changes in (dict(row_count=0), dict(row_count=9), dict(reserved_zero=4100), dict(reserved_zero=9216), dict(scale=amd.Range(1 << 30, 16)),
+                    dict(mixes=amd.Range((1 << 20) + 64, 1024)), dict(hidden=amd.Range((8 << 30) - 256, 8 * 4096 * 2))):
+        assert lib.hyper_site_prepare(C.byref(site_description(**changes)), arena, C.byref(hyper), untouched) == 1, changes
+        assert not any(bytes(untouched))

@@ -1,0 +1,164 @@
+"""GPU checks, through the C ABI, of the launches a site front stands for (the step ahead of the routed experts): the
+dense product (a site's mix project with the row's scale; the router's scores in that order) and the hyper site's mix
+finish and post, against the CPU oracle (oracle/orc_site.c, which tests/test_oracle_site.py pins to the reference's own
+host oracles). Everything is held bit for bit: the products' sums (the definition fixes every chain and tree), the
+mixes, pre, post and comb (the exponential and the reciprocal root are this build's fixed functions on both sides), the
+collapse, its norm, and the streams behind the post."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+from _oracle import f32p, normals, orc, ptr, to_bf16, u16p
+
+pytestmark = pytest.mark.gpu
+STREAMS, MIXES = 4, 24
+
+
+def say(*words):
+    print(*words, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def amd():
+    import anemone_amd
+    return anemone_amd
+
+
+@pytest.fixture(scope="module")
+def card(amd):
+    card = amd.Card(1 << 30)
+    yield card
+    card.close()
+
+
+@pytest.fixture(autouse=True)
+def fresh_arena(card):
+    card.cursor = 256
+    yield
+
+
+def front_of(amd, card, rows, width, seed, spread=1.0):
+    mix_weights = (normals(seed, MIXES * STREAMS * width) * 0.02).astype(np.float32).reshape(MIXES, STREAMS * width)
+    scale = (np.abs(normals(seed + 1, 3)) + 0.2).astype(np.float32)
+    base = (normals(seed + 2, MIXES) * 0.5).astype(np.float32)
+    norm_weight = to_bf16(normals(seed + 3, width) * 0.1 + 1.0)
+    front = amd.SiteFront(card, rows, width, mix_weights, scale, base, norm_weight)
+    streams = to_bf16(normals(seed + 4, rows * STREAMS * width) * spread).reshape(rows, STREAMS, width)
+    carried = (np.abs(normals(seed + 5, rows * STREAMS)) * 0.4 + 0.05).astype(np.float32).reshape(rows, STREAMS)
+    front.set_streams(streams, carried)
+    return front, streams, carried
+
+
+def oracle_dense(weight_type, weights, rows, flags, epsilon, scale, output_type):
+    outputs, inputs = weights.shape
+    out = np.zeros((rows.shape[0], outputs), np.float32 if output_type == 1 else np.uint16)
+    assert orc.orc_dense_linear(weight_type, weights.ctypes.data_as(C.c_void_p), outputs, inputs, flags, epsilon, scale, output_type,
+                                ptr(rows, u16p), rows.shape[0], out.ctypes.data_as(C.c_void_p)) == 0
+    return out
+
+
+@pytest.mark.parametrize("rows,width,live", [(8, 4096, 8), (1, 5120, 1), (5, 1024, 3), (2, 8192, 2)])
+def test_mix_project_and_finish_bit_for_bit(amd, card, rows, width, live):
+    say("site front: mix project, finish", rows, width, live)
+    front, streams, carried = front_of(amd, card, rows, width, 10 * rows + width)
+    for name in ("mixes", "post", "comb", "hidden"):
+        card.upload(front.ranges[name].byte_offset, np.full(front.ranges[name].byte_count, 0xEE, dtype=np.uint8))
+    card.run(front.mix_project_launch(live))
+    mixes = front.read("mixes", np.float32).reshape(rows, MIXES)
+    want_mixes = oracle_dense(1, front.constants["mix_weights"], np.ascontiguousarray(streams[:live].reshape(live, -1)), 1, 1e-20, 1.0, 1)
+    assert np.array_equal(mixes[:live].view(np.uint32), want_mixes.view(np.uint32))
+    assert np.all(mixes[live:].view(np.uint32) == 0xEEEEEEEE)
+    card.run(front.site_launches(live)[:1])
+    pre, post, comb = front.read("carried_pre", np.float32).reshape(rows, 4), front.read("post", np.float32).reshape(rows, 4), front.read("comb", np.float32).reshape(rows, 16)
+    hidden = front.read("hidden", np.uint16).reshape(rows, width)
+    for r in range(live):
+        want_pre, want_post, want_comb, want_hidden = carried[r].copy(), np.zeros(4, np.float32), np.zeros(16, np.float32), np.zeros(width, np.uint16)
+        orc.orc_hyper_mix_finish(ptr(np.ascontiguousarray(streams[r]), u16p), ptr(want_pre, f32p), ptr(np.ascontiguousarray(want_mixes[r]), f32p),
+                                 ptr(front.constants["scale"], f32p), ptr(front.constants["base"], f32p), ptr(front.constants["norm_weight"], u16p),
+                                 width, ptr(want_post, f32p), ptr(want_comb, f32p), ptr(want_hidden, u16p))
+        assert np.array_equal(pre[r].view(np.uint32), want_pre.view(np.uint32)), ("pre", r)
+        assert np.array_equal(post[r].view(np.uint32), want_post.view(np.uint32)), ("post", r)
+        assert np.array_equal(comb[r].view(np.uint32), want_comb.view(np.uint32)), ("comb", r)
+        assert np.array_equal(hidden[r], want_hidden), ("hidden", r, np.flatnonzero(hidden[r] != want_hidden)[:8])
+    assert np.array_equal(pre[live:], carried[live:]) and np.all(hidden[live:] == 0xEEEE)
+    say("  comb's columns sum to", comb[0].reshape(4, 4).sum(axis=0))
+
+
+def test_finish_with_specials_in_the_streams(amd, card):
+    """Infinities, not-a-numbers, signed zeros and the largest values among the streams; mixes that drive the
+    exponentials to their ends."""
+    say("site front: specials")
+    rows, width = 4, 1024
+    front, streams, carried = front_of(amd, card, rows, width, 5)
+    streams[0, 0, :8] = [0x7F80, 0xFF80, 0x7FC1, 0x8000, 0x0000, 0x0001, 0x8001, 0x7F7F]
+    streams[1] = to_bf16(normals(3, STREAMS * width) * 1e-30).reshape(STREAMS, width)
+    streams[2] = to_bf16(normals(4, STREAMS * width) * 1e18).reshape(STREAMS, width)
+    front.set_streams(streams, carried)
+    mixes = (normals(6, rows * MIXES) * 3.0).astype(np.float32).reshape(rows, MIXES)
+    mixes[1] *= 100.0
+    mixes[2, :8] = [200.0, -200.0, 1e30, -1e30, 90.0, -90.0, 0.0, -0.0]
+    mixes[3, 8:] = 0.0
+    card.upload(front.ranges["mixes"].byte_offset, mixes)
+    card.run(front.site_launches()[:1])
+    pre, post, comb = front.read("carried_pre", np.float32).reshape(rows, 4), front.read("post", np.float32).reshape(rows, 4), front.read("comb", np.float32).reshape(rows, 16)
+    hidden = front.read("hidden", np.uint16).reshape(rows, width)
+    for r in range(rows):
+        want_pre, want_post, want_comb, want_hidden = carried[r].copy(), np.zeros(4, np.float32), np.zeros(16, np.float32), np.zeros(width, np.uint16)
+        orc.orc_hyper_mix_finish(ptr(np.ascontiguousarray(streams[r]), u16p), ptr(want_pre, f32p), ptr(np.ascontiguousarray(mixes[r]), f32p),
+                                 ptr(front.constants["scale"], f32p), ptr(front.constants["base"], f32p), ptr(front.constants["norm_weight"], u16p),
+                                 width, ptr(want_post, f32p), ptr(want_comb, f32p), ptr(want_hidden, u16p))
+        for name, got, want in (("pre", pre[r], want_pre), ("post", post[r], want_post), ("comb", comb[r], want_comb)):
+            same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+            assert np.all(same), (name, r, got, want)
+        assert np.array_equal(hidden[r], want_hidden), ("hidden", r)
+
+
+@pytest.mark.parametrize("weight_type,outputs,inputs,rows,output_type,scale", [(0, 256, 4096, 8, 1, 1.0), (0, 384, 5120, 1, 1, 1.0),
+                                                                              (0, 2048, 1024, 3, 0, 0.125), (1, 64, 264, 2, 0, 1.0)])
+def test_dense_products_bit_for_bit(amd, card, weight_type, outputs, inputs, rows, output_type, scale):
+    """The router's scores in the dense product's order (bfloat16 weights, float32 out) and the other forms: four outputs
+    a block and one, one row and several, a bfloat16 output with a scale."""
+    say("dense product", weight_type, outputs, inputs, rows, output_type, scale)
+    front, _, _ = front_of(amd, card, 1, 1024, 9)
+    raw = normals(11, outputs * inputs) * 0.05
+    weights = raw.astype(np.float32).reshape(outputs, inputs) if weight_type == 1 else to_bf16(raw).reshape(outputs, inputs)
+    x = to_bf16(normals(12, rows * inputs)).reshape(rows, inputs)
+    w_range = amd.Range(card.place(weights, 256), weights.nbytes)
+    x_range = amd.Range(card.place(x, 256), x.nbytes)
+    out_bytes = rows * outputs * (4 if output_type == 1 else 2)
+    out_range = amd.Range(card.reserve(out_bytes), out_bytes)
+    card.run(front.dense_launch(w_range, x_range, out_range, outputs, inputs, weight_type, output_type, 0, scale, 0.0, rows))
+    got = card.download(out_range.byte_offset, out_bytes, np.float32 if output_type == 1 else np.uint16).reshape(rows, outputs)
+    want = oracle_dense(weight_type, weights, x, 0, 0.0, scale, output_type)
+    view = np.uint32 if output_type == 1 else np.uint16
+    assert np.array_equal(got.view(view), want.view(view))
+
+
+def test_site_from_streams_to_streams(amd, card):
+    """A whole site around a stand-in sublayer: mix project, mix finish, then the post with the combine, the streams
+    against the oracle's post of the oracle's pre-sublayer state."""
+    say("site front: a whole site")
+    rows, width = 8, 4096
+    front, streams, carried = front_of(amd, card, rows, width, 21)
+    output = to_bf16(normals(31, rows * width)).reshape(rows, width)
+    sums = (normals(32, rows * width) * 2.0).astype(np.float32).reshape(rows, width)
+    card.upload(front.ranges["output"].byte_offset, output)
+    card.upload(front.ranges["routed_sums"].byte_offset, sums)
+    finish, post = front.site_launches(combined=True)
+    launches = amd.launches_of(3)
+    launches[0], launches[1], launches[2] = front.mix_project_launch()[0], finish, post
+    card.run(launches)
+    got = front.read("streams", np.uint16).reshape(rows, STREAMS, width)
+    want_mixes = oracle_dense(1, front.constants["mix_weights"], np.ascontiguousarray(streams.reshape(rows, -1)), 1, 1e-20, 1.0, 1)
+    for r in range(rows):
+        pre, post_of, comb, hidden = carried[r].copy(), np.zeros(4, np.float32), np.zeros(16, np.float32), np.zeros(width, np.uint16)
+        orc.orc_hyper_mix_finish(ptr(np.ascontiguousarray(streams[r]), u16p), ptr(pre, f32p), ptr(np.ascontiguousarray(want_mixes[r]), f32p),
+                                 ptr(front.constants["scale"], f32p), ptr(front.constants["base"], f32p), ptr(front.constants["norm_weight"], u16p),
+                                 width, ptr(post_of, f32p), ptr(comb, f32p), ptr(hidden, u16p))
+        want = np.zeros((STREAMS, width), np.uint16)
+        orc.orc_hyper_post(ptr(np.ascontiguousarray(streams[r]), u16p), ptr(post_of, f32p), ptr(comb, f32p), ptr(np.ascontiguousarray(output[r]), u16p),
+                           ptr(np.ascontiguousarray(sums[r]), f32p), width, ptr(want, u16p))
+        assert np.array_equal(got[r], want), r
