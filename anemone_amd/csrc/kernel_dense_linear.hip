@@ -13,8 +13,11 @@
  * DENSE_STEP_ROWS and DENSE_CONE_ROWS (the head's and the prefill cone's rows) are not built: the host refuses them.
  *
  * Work mapping: a wavefront holds two of the definition's groups of 32 (an exchange at a distance below 32 stays inside
- * its half); a thread asks for all its chunks' weights ahead (a step's matrices are 2 to 4 MB: the launch is a few
- * round trips to memory, not a stream), the rows come from the caches (every block reads the same rows).
+ * its half). A step's matrices are 2 to 4 MB: the launch is a few round trips to memory, not a stream, so what counts is
+ * how many blocks there are and how many loads each keeps in flight. A block takes the rows ROWS blockIdx.y .. + ROWS - 1
+ * (the reference's launches have one row of blocks; here the host may give a matrix of few outputs, the mix project's 24,
+ * a block a row and an output, the one-row instance on a grid (outputs, rows): 192 blocks in place of 24, the same
+ * operations for every output); the chunk loop of the one-row instance is unrolled four times.
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -45,7 +48,7 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
 {
     __shared__ float group_sums[DENSE_GROUPS][OUTPUTS + 1u][ROWS];
     const uint32_t thread = threadIdx.x, inputs = arguments.input_size, chunks = inputs / DENSE_CHUNK_INPUTS;
-    const uint32_t first_output = blockIdx.x * OUTPUTS;
+    const uint32_t first_output = blockIdx.x * OUTPUTS, first_row = blockIdx.y * ROWS;
     const bool scaled = (arguments.flags & DENSE_ROW_SCALE) != 0u;
     const uint16_t *rows = (const uint16_t *)(arena + arguments.rows_offset);
     float chain[OUTPUTS][ROWS], squares[ROWS];
@@ -57,12 +60,13 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
             chain[o][r] = 0.0f;
         }
     }
+#pragma unroll(ROWS == 1u ? 4 : 1)
     for (uint32_t chunk = thread; chunk < chunks; chunk += DENSE_THREADS_VALUE) {
         float values[ROWS][DENSE_CHUNK_INPUTS];
 #pragma unroll
         for (uint32_t r = 0; r < ROWS; r++) {
             /* a column from row_count on reads row 0 and is stored nowhere */
-            const uint32_t row = r < arguments.row_count ? r : 0u;
+            const uint32_t row = first_row + r < arguments.row_count ? first_row + r : 0u;
             unpack_bf16x8(*(const uint4_t *)(rows + (uint64_t)row * inputs + chunk * DENSE_CHUNK_INPUTS), values[r]);
             if (scaled) {
 #pragma unroll
@@ -117,7 +121,7 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
         return;
     }
     const uint32_t o = thread / ROWS, r = thread % ROWS;
-    if (r >= arguments.row_count) {
+    if (first_row + r >= arguments.row_count) {
         return;
     }
     float sum = 0.0f, square_sum = 0.0f;
@@ -132,7 +136,7 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
         const float operand = __fadd_rn(__fmul_rn(square_sum, __fdiv_rn(1.0f, (float)inputs)), arguments.epsilon);
         sum = __fmul_rn(sum, dense_reciprocal_root(operand));
     }
-    const uint64_t index = (uint64_t)r * arguments.output_size + first_output + o;
+    const uint64_t index = (uint64_t)(first_row + r) * arguments.output_size + first_output + o;
     if (arguments.output_type == DENSE_FLOAT32) {
         ((float *)(arena + arguments.output_offset))[index] = __fmul_rn(sum, arguments.output_scale);
     } else {

@@ -5,7 +5,7 @@
  * include/anemone/hyper_connection.h:6-71).
  *
  *   launch        kernel                                grid                               block
- *   dense         dense_linear_<type>_<R>[_narrow]      (outputs / (4 or 1), 1, 1)         256
+ *   dense         dense_linear_<type>_<R>[_narrow]      (outputs / (4 or 1), 1 or rows, 1) 256
  *   mix finish    hyper_mix_finish                      (1, rows, 1)                       width / 8
  *   post          hyper_post_entry                      (width / 1024, rows, 1)            128
  */
@@ -15,6 +15,7 @@
 #include "prepare_common.h"
 
 #define SITE_DEFAULT_WIDTH 5120u
+#define DENSE_BY_ROW_MOST_BLOCKS 1024u
 #define SITE_MOST_WIDTH 8192u
 #define SITE_WIDTH_STEP (HYPER_VALUES_PER_THREAD * HYPER_PIECE_THREADS)
 
@@ -78,8 +79,11 @@ result_status dense_linear_prepare(const struct dense_linear_description *descri
     }
     /* fewer than DENSE_NARROW_BELOW_BLOCKS blocks of four outputs: a block owns one, the same operations for every output */
     const uint32_t form = description->output_size / DENSE_OUTPUTS_PER_BLOCK < DENSE_NARROW_BELOW_BLOCKS ? 1u : 0u;
+    /* few outputs and several rows (a site's 24 mixes): a block a row and an output, the one-row instance on a grid of
+     * (outputs, rows), so that eight times the units are at work; every output's operations are the same */
+    const bool by_row = form != 0u && description->row_count > 1u && description->output_size * description->row_count <= DENSE_BY_ROW_MOST_BLOCKS;
     const uint32_t kernel = kernels->products[form * DENSE_FORM_INSTANCES + description->weight_type * DENSE_ROW_INSTANCES +
-                                              (description->row_count > 1u ? 1u : 0u)];
+                                              (description->row_count > 1u && !by_row ? 1u : 0u)];
     if (kernel == BACKEND_NO_KERNEL) {
         REFUSE("%s: its kernel is not prepared", what);
         return STATUS_INVALID_ARGUMENT;
@@ -87,8 +91,8 @@ result_status dense_linear_prepare(const struct dense_linear_description *descri
     const struct dense_linear_arguments record = {description->weights.byte_offset, description->rows.byte_offset, description->output.byte_offset, 0,
                                                   description->output_size, description->input_size, description->row_count,
                                                   description->output_type, description->flags, description->output_scale, description->epsilon, 0};
-    launch_fill(launch_out, kernel, description->output_size / (form != 0u ? 1u : DENSE_OUTPUTS_PER_BLOCK), 1, 1, DENSE_THREADS_VALUE, 0,
-                &record, sizeof record);
+    launch_fill(launch_out, kernel, description->output_size / (form != 0u ? 1u : DENSE_OUTPUTS_PER_BLOCK), by_row ? description->row_count : 1, 1,
+                DENSE_THREADS_VALUE, 0, &record, sizeof record);
     return STATUS_OK;
 }
 

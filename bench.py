@@ -134,7 +134,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         parts = [layer.projection_launch()[0]] + routing + [layer.quantize_launch()[0]] + [experts[i] for i in range(4)]
         names = ["router_projection"] + routing_names + ["activation_quantize", "expert_gate_up", "activation_quantize(hidden)",
                                                          "expert_down", "expert_row_sum_entry"]
-    shared = None
+    shared = front = None
     if arguments.site and block128:
         raise SystemExit("--site takes the reference's scaling: the shared expert's kernels read E8M0 scales of 32 values")
     if arguments.site:
@@ -152,6 +152,16 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         if rows <= amd.LINEAR_MAXIMUM_ROWS:  # a thin step: the shared expert's down and the join in one launch
             parts = parts[:-1] + [four[i] for i in range(3)] + [shared.shared_join_launch()[0]]
             names = names[:-1] + ["trunk_gate_up", "trunk_hidden", "activation_quantize(shared)", "expert_shared_join"]
+            # and the step ahead of the router: the site's mix project and mix finish, whose hidden rows (the collapse of
+            # the streams with the carried pre, normed) are the rows the router and the quantizer then read
+            front = amd.SiteFront(card, rows, HIDDEN, (workloads.normals(base + 910, 24 * 4 * HIDDEN) * 0.02).reshape(24, 4 * HIDDEN),
+                                  [1.0, 1.0, 1.0], workloads.normals(base + 911, 24) * 0.5, workloads.to_bf16(np.ones(HIDDEN)),
+                                  hidden_range=amd.Range(layer.x_offset, rows * HIDDEN * 2))
+            for name in ("streams", "post", "comb"):  # the join reads the post and comb the finish writes
+                front.ranges[name] = shared.ranges[name]
+            card.upload(front.ranges["carried_pre"].byte_offset, np.full((rows, 4), 0.25, dtype=np.float32))
+            parts = [front.mix_project_launch()[0], front.site_launches()[0]] + parts
+            names = ["dense_linear(mix project)", "hyper_mix_finish"] + names
         else:
             parts = parts[:-1] + [four[i] for i in range(4)] + [shared.join_launch()[0]]
             names = names[:-1] + ["trunk_gate_up", "trunk_hidden", "activation_quantize(shared)", "trunk_down", "expert_join"]
@@ -221,6 +231,10 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
             "join_traffic": MEASURED_TRAFFIC_BYTES.get(("expert_join", rows)),
             "trunk_gate_up_us": trunk_us, "trunk_gate_up_GBps": 2 * shared_matrix_bytes / (trunk_us * 1e-6) / 1e9,
             "trunk_gate_up_TFLOPs": 2.0 * rows * 2 * HIDDEN * INNER / (trunk_us * 1e-6) / 1e12}
+        if front is not None:
+            result["config"]["site"]["launches"] = "the site's mix project and mix finish ahead of the router, the shared expert (E4M3 weights) and the shared join"
+            result["config"]["site"]["front_us"] = float(per_launch[0] + per_launch[1])
+            result["config"]["site"]["mix_project_GBps"] = 24 * 4 * HIDDEN * 4 / (float(per_launch[0]) * 1e-6) / 1e9
     key = ("%s_%s" % ("fp8" if fp8 else "fp4", "prefill" if prefill else "decode"), rows)
     if block128:
         key = (key[0] + "_block128", rows)
@@ -251,6 +265,28 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         import _oracle as o
         threads = min(os.cpu_count() or 1, 16)
         sample = min(rows, 4)
+        if front is not None:
+            # one step from the site's first state: the rows are then the front's (the collapse of the streams, normed),
+            # post and comb its Sinkhorn's, and the job table that step's
+            shared.set_site(site_streams, site_post, site_comb)
+            card.upload(front.ranges["carried_pre"].byte_offset, np.full((rows, 4), 0.25, dtype=np.float32))
+            card.run(step)
+            live = layer.jobs()
+            live = live[live["row_count"] > 0]
+            flat = np.ascontiguousarray(site_streams.reshape(rows, -1))
+            mixes = np.zeros((rows, 24), dtype=np.float32)
+            assert o.orc.orc_dense_linear(1, front.constants["mix_weights"].ctypes.data_as(C.c_void_p), 24, 4 * HIDDEN, 1, 1e-20, 1.0, 1,
+                                          o.ptr(flat, o.u16p), rows, mixes.ctypes.data_as(C.c_void_p)) == 0
+            x, site_post, site_comb = np.zeros((rows, HIDDEN), dtype=np.uint16), np.zeros((rows, 4), dtype=np.float32), np.zeros((rows, 4, 4), dtype=np.float32)
+            for r in range(rows):
+                pre = np.full(4, 0.25, dtype=np.float32)
+                row_hidden, row_post, row_comb = np.zeros(HIDDEN, dtype=np.uint16), np.zeros(4, dtype=np.float32), np.zeros(16, dtype=np.float32)
+                o.orc.orc_hyper_mix_finish(o.ptr(np.ascontiguousarray(site_streams[r]), o.u16p), o.ptr(pre, o.f32p), o.ptr(np.ascontiguousarray(mixes[r]), o.f32p),
+                                           o.ptr(front.constants["scale"], o.f32p), o.ptr(front.constants["base"], o.f32p),
+                                           o.ptr(front.constants["norm_weight"], o.u16p), HIDDEN, o.ptr(row_post, o.f32p), o.ptr(row_comb, o.f32p),
+                                           o.ptr(row_hidden, o.u16p))
+                x[r], site_post[r], site_comb[r] = row_hidden, row_post, row_comb.reshape(4, 4)
+            assert np.array_equal(card.download(layer.x_offset, rows * HIDDEN * 2, np.uint16).reshape(rows, HIDDEN), x), "the front's rows are the oracle's bits"
         experts_of = np.zeros((rows, PICKS), dtype=np.uint32)
         weights_of = np.zeros((rows, PICKS), dtype=np.float32)
         if prefill:
@@ -281,8 +317,9 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         if shared is None:
             got = layer.read("row_output", np.float32).reshape(rows, HIDDEN)[:sample]
         else:  # one step from the streams' first values
-            shared.set_site(site_streams, site_post, site_comb)
-            card.run(step)
+            if front is None:
+                shared.set_site(site_streams, site_post, site_comb)
+                card.run(step)
             got = shared.read("row_sums", np.float32).reshape(rows, HIDDEN)[:sample]
             got_streams = o.bf16_to_f32(shared.read("streams", np.uint16).reshape(rows, 4, HIDDEN)[:sample].reshape(-1)).astype(np.float64)
             wanted = o.bf16_to_f32(want_streams.reshape(-1)).astype(np.float64)
@@ -464,7 +501,7 @@ def main():
                         workloads.exl3_matrix_bytes(HIDDEN, INNER, int(widths[e, 1])) for e in distinct)
     down_bytes = sum(workloads.exl3_matrix_bytes(INNER, HIDDEN, int(widths[e, 2])) for e in distinct)
     step_bytes = gate_up_bytes + down_bytes + ROWS * HIDDEN * 2 + ROWS * HIDDEN * 4
-    gate_up_us = float(per_launch[3])
+    gate_up_us = float(per_launch[names.index("exl3_tc_products(gate/up)")])
     achieved = gate_up_bytes / (gate_up_us * 1e-6) / 1e9
 
     result = {

@@ -753,7 +753,11 @@ def test_site_front_launches_geometry_and_refusals(fake):
     launch = amd.launches_of(1)
     # the mix project: 24 outputs are fewer than 256 blocks of four: the narrow form, a block an output
     assert lib.dense_linear_prepare(C.byref(dense_description()), arena, C.byref(dense), launch) == 0
-    assert fake.handles[launch[0].kernel][1] == "dense_linear_float32_8_narrow" and list(launch[0].grid) == [24, 1, 1] and launch[0].block[0] == 256
+    assert fake.handles[launch[0].kernel][1] == "dense_linear_float32_1_narrow" and list(launch[0].grid) == [24, 8, 1] and launch[0].block[0] == 256
+    scores = dense_description(outputs=256, inputs=4096, weight_type=0, flags=0)  # the router's: too many blocks for a block a row
+    assert lib.dense_linear_prepare(C.byref(scores), arena, C.byref(dense), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "dense_linear_bfloat16_8_narrow" and list(launch[0].grid) == [256, 1, 1]
+    assert lib.dense_linear_prepare(C.byref(dense_description()), arena, C.byref(dense), launch) == 0
     assert launch[0].argument_byte_count == 64
     one = dense_description(outputs=4096, inputs=2048, rows=1, weight_type=0, output_type=0, flags=0)
     assert lib.dense_linear_prepare(C.byref(one), arena, C.byref(dense), launch) == 0
@@ -785,3 +789,4 @@ def test_site_front_launches_geometry_and_refusals(fake):
                     dict(mixes=amd.Range((1 << 20) + 64, 1024)), dict(hidden=amd.Range((8 << 30) - 256, 8 * 4096 * 2))):
         assert lib.hyper_site_prepare(C.byref(site_description(**changes)), arena, C.byref(hyper), untouched) == 1, changes
         assert not any(bytes(untouched))
+
