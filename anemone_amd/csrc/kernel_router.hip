@@ -67,15 +67,17 @@ __device__ static __forceinline__ float router_affinity(float score, uint32_t ki
  * A block takes PROJECTION_EXPERTS experts and up to PROJECTION_ROWS rows: it stages the weights and the rows in
  * chunks of PROJECTION_CHUNK inputs through LDS with 16-byte coalesced loads (the next chunk in flight while this
  * one is consumed); a thread owns chains 2 j and 2 j + 1 of one expert for every row, so the fma order of a chain
- * is the definition's whatever the staging. grid (ceil(E / 8), ceil(rows / 4)), block 128. */
-#define PROJECTION_ROWS 4u
+ * is the definition's whatever the staging. grid (ceil(E / 8), ceil(rows / 4)), block 128; or, for a thin step, grid
+ * (ceil(E / 8), rows): a row a block (the rows a block takes are what its grid leaves it, four or one), a quarter of
+ * the fused multiply-adds a block and four times the blocks: the launch is a few round trips to memory either way. */
+#define PROJECTION_MOST_ROWS 4u
 #define PROJECTION_EXPERTS 8u
 #define PROJECTION_CHUNK 1024u
 #define PROJECTION_W_LOADS (PROJECTION_EXPERTS * PROJECTION_CHUNK * 2u / 16u / PROJECTION_THREADS)
-#define PROJECTION_X_LOADS (PROJECTION_ROWS * PROJECTION_CHUNK * 2u / 16u / PROJECTION_THREADS)
-extern "C" __global__ void __launch_bounds__(PROJECTION_THREADS)
-    router_projection(struct router_projection_arguments arguments, unsigned char *arena)
+template <uint32_t PROJECTION_ROWS>
+__device__ static __forceinline__ void router_projection_block(const struct router_projection_arguments &arguments, unsigned char *arena)
 {
+    constexpr uint32_t PROJECTION_X_LOADS = PROJECTION_ROWS * PROJECTION_CHUNK * 2u / 16u / PROJECTION_THREADS;
     __shared__ __attribute__((aligned(16))) uint16_t w_tile[PROJECTION_EXPERTS][PROJECTION_CHUNK];
     __shared__ __attribute__((aligned(16))) uint16_t x_tile[PROJECTION_ROWS][PROJECTION_CHUNK];
     const uint32_t H = arguments.hidden, thread = threadIdx.x;
@@ -151,6 +153,16 @@ extern "C" __global__ void __launch_bounds__(PROJECTION_THREADS)
         if (pair == 0u && expert < arguments.expert_count && first_row + r < arguments.row_count) {
             ((float *)(arena + arguments.output_offset))[(uint64_t)(first_row + r) * arguments.expert_count + expert] = __fadd_rn(0.0f, sum);
         }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(PROJECTION_THREADS)
+    router_projection(struct router_projection_arguments arguments, unsigned char *arena)
+{
+    if (gridDim.y >= arguments.row_count) { /* the same in every block: a row a block */
+        router_projection_block<1u>(arguments, arena);
+    } else {
+        router_projection_block<PROJECTION_MOST_ROWS>(arguments, arena);
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_projection, router_projection_arguments);

@@ -25,6 +25,7 @@
 #define PROJECTION_THREADS 128u
 #define PROJECTION_OUTPUTS 8u /* experts a block */
 #define PROJECTION_ROWS 4u    /* rows a block takes at once */
+#define PROJECTION_BY_ROW_MOST_BLOCKS 1024u
 
 result_status router_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                      struct router_kernels_record *kernels_out)
@@ -254,8 +255,12 @@ result_status router_projection_prepare(const struct router_projection_descripti
                     sizeof record);
         return STATUS_OK;
     }
-    launch_fill(launch_out, kernels->projection, (description->expert_count + PROJECTION_OUTPUTS - 1u) / PROJECTION_OUTPUTS,
-                (description->row_count + PROJECTION_ROWS - 1u) / PROJECTION_ROWS, 1, PROJECTION_THREADS, 0, &record, sizeof record);
+    /* a thin step: a row a block (the kernel takes the rows its grid leaves it: four a block, or one) */
+    const uint32_t expert_blocks = (description->expert_count + PROJECTION_OUTPUTS - 1u) / PROJECTION_OUTPUTS;
+    const bool by_row = description->row_count <= LINEAR_MAXIMUM_ROWS && expert_blocks * description->row_count <= PROJECTION_BY_ROW_MOST_BLOCKS;
+    launch_fill(launch_out, kernels->projection, expert_blocks,
+                by_row ? description->row_count : (description->row_count + PROJECTION_ROWS - 1u) / PROJECTION_ROWS, 1, PROJECTION_THREADS, 0,
+                &record, sizeof record);
     return STATUS_OK;
 }
 
