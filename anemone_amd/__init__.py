@@ -181,7 +181,7 @@ class ExpertJoinArguments(C.Structure):
 
 
 class DenseLinearKernels(C.Structure):
-    _fields_ = [("products", u32 * 8)]
+    _fields_ = [("products", u32 * 8), ("wide_products", u32 * 2)]
 
 
 class DenseLinearDescription(C.Structure):

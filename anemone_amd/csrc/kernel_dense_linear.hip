@@ -11,6 +11,8 @@
  *     in the same order; r is the float32 nearest the reciprocal square root (the reference takes its card's rsqrtf);
  *   - a float32 output is the value times output_scale; a bfloat16 one is rounded, multiplied and rounded again.
  * DENSE_STEP_ROWS and DENSE_CONE_ROWS (the head's and the prefill cone's rows) are not built: the host refuses them.
+ * More than 8 rows: the rows in groups of 8 on grid[1] (dense_linear_<type>_8_wide, 8 outputs a block, or the 8-row
+ * instance of 4 outputs where the outputs do not divide).
  *
  * Work mapping: a wavefront holds two of the definition's groups of 32 (an exchange at a distance below 32 stays inside
  * its half). A step's matrices are 2 to 4 MB: the launch is a few round trips to memory, not a stream, so what counts is
@@ -159,3 +161,8 @@ DENSE_STAMP(bfloat16, DENSE_BFLOAT16, 1, 1u, _narrow)
 DENSE_STAMP(bfloat16, DENSE_BFLOAT16, 8, 1u, _narrow)
 DENSE_STAMP(float32, DENSE_FLOAT32, 1, 1u, _narrow)
 DENSE_STAMP(float32, DENSE_FLOAT32, 8, 1u, _narrow)
+/* a step of more rows (a prefill chunk's): groups of 8 rows on grid[1], a block 8 outputs of its group, so that a group's
+ * rows are read once for eight outputs; every output's bits are those of the launch of 8 rows of its group
+ * (dense_linear_<type>_wide_<O> of the reference, include/anemone/dense_linear_records.h:31-37) */
+DENSE_STAMP(bfloat16, DENSE_BFLOAT16, 8, DENSE_WIDE_OUTPUTS, _wide)
+DENSE_STAMP(float32, DENSE_FLOAT32, 8, DENSE_WIDE_OUTPUTS, _wide)

@@ -6,6 +6,7 @@
  *
  *   launch        kernel                                grid                               block
  *   dense         dense_linear_<type>_<R>[_narrow]      (outputs / (4 or 1), 1 or rows, 1) 256
+ *   dense, wide   dense_linear_<type>_8_wide            (outputs / 8, ceil(rows / 8), 1)   256
  *   mix finish    hyper_mix_finish                      (1, rows, 1)                       width / 8
  *   post          hyper_post_entry                      (width / 1024, rows, 1)            128
  */
@@ -15,7 +16,7 @@
 #include "prepare_common.h"
 
 #define SITE_DEFAULT_WIDTH 5120u
-#define DENSE_BY_ROW_MOST_BLOCKS 1024u
+#define DENSE_BY_ROW_MOST_BLOCKS 4096u /* a block a row and an output while that leaves at most so many blocks */
 #define SITE_MOST_WIDTH 8192u
 #define SITE_WIDTH_STEP (HYPER_VALUES_PER_THREAD * HYPER_PIECE_THREADS)
 
@@ -42,6 +43,16 @@ result_status dense_linear_kernels_prepare(const struct backend_operations *back
             return status;
         }
     }
+    for (uint32_t type = 0; type < DENSE_TYPE_COUNT; type++) {
+        char name[56];
+        (void)snprintf(name, sizeof name, "%s%s_8_wide", KERNEL_DENSE_LINEAR_STEM, dense_type_names[type]);
+        const result_status status =
+            backend->kernel_prepare(card, KERNEL_FILE_DENSE_LINEAR, name, sizeof(struct dense_linear_arguments), &kernels.wide_products[type]);
+        if (status != STATUS_OK) {
+            REFUSE("the kernels of the dense products: %s is not prepared: %s", name, status_text(status));
+            return status;
+        }
+    }
     *kernels_out = kernels;
     return STATUS_OK;
 }
@@ -62,9 +73,12 @@ result_status dense_linear_prepare(const struct dense_linear_description *descri
                DENSE_FLAGS, DENSE_OUTPUTS_PER_BLOCK, DENSE_CHUNK_INPUTS);
         return STATUS_INVALID_ARGUMENT;
     }
-    if (description->row_count > LINEAR_MAXIMUM_ROWS || (description->flags & (DENSE_STEP_ROWS | DENSE_CONE_ROWS)) != 0u ||
-        description->cone_layer != 0u || description->step.byte_count != 0u) {
-        REFUSE("%s: the wide launches (more than %u rows), the head's step rows and the cone's rows are not built", what, LINEAR_MAXIMUM_ROWS);
+    if (description->row_count > DENSE_MOST_ROWS * LINEAR_MAXIMUM_ROWS) {
+        REFUSE("%s: at most %u rows", what, DENSE_MOST_ROWS * LINEAR_MAXIMUM_ROWS);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    if ((description->flags & (DENSE_STEP_ROWS | DENSE_CONE_ROWS)) != 0u || description->cone_layer != 0u || description->step.byte_count != 0u) {
+        REFUSE("%s: the head's step rows and the cone's rows are not built", what);
         return STATUS_UNSUPPORTED;
     }
     const uint64_t weight_bytes = description->weight_type == DENSE_FLOAT32 ? 4u : 2u, output_bytes = description->output_type == DENSE_FLOAT32 ? 4u : 2u;
@@ -77,20 +91,36 @@ result_status dense_linear_prepare(const struct dense_linear_description *descri
     if (!ranges_are_valid(what, ranges, 3, arena_byte_count)) {
         return STATUS_INVALID_ARGUMENT;
     }
+    const struct dense_linear_arguments record = {description->weights.byte_offset, description->rows.byte_offset, description->output.byte_offset, 0,
+                                                  description->output_size, description->input_size, description->row_count,
+                                                  description->output_type, description->flags, description->output_scale, description->epsilon, 0};
+    const bool few_blocks = description->output_size / DENSE_OUTPUTS_PER_BLOCK < DENSE_NARROW_BELOW_BLOCKS &&
+                            (uint64_t)description->output_size * description->row_count <=
+                                (description->row_count > LINEAR_MAXIMUM_ROWS ? DENSE_BY_ROW_MOST_BLOCKS : DENSE_BY_ROW_MOST_BLOCKS / 4u);
+    if (description->row_count > LINEAR_MAXIMUM_ROWS && !few_blocks) {
+        /* a wide launch: groups of 8 rows on grid[1]; 8 outputs a block where they divide, else the 8-row instance's 4 */
+        const bool eight = description->output_size % DENSE_WIDE_OUTPUTS == 0u;
+        const uint32_t wide = eight ? kernels->wide_products[description->weight_type]
+                                    : kernels->products[description->weight_type * DENSE_ROW_INSTANCES + 1u];
+        if (wide == BACKEND_NO_KERNEL) {
+            REFUSE("%s: its kernel is not prepared", what);
+            return STATUS_INVALID_ARGUMENT;
+        }
+        launch_fill(launch_out, wide, description->output_size / (eight ? DENSE_WIDE_OUTPUTS : DENSE_OUTPUTS_PER_BLOCK),
+                    (description->row_count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS, 1, DENSE_THREADS_VALUE, 0, &record, sizeof record);
+        return STATUS_OK;
+    }
     /* fewer than DENSE_NARROW_BELOW_BLOCKS blocks of four outputs: a block owns one, the same operations for every output */
     const uint32_t form = description->output_size / DENSE_OUTPUTS_PER_BLOCK < DENSE_NARROW_BELOW_BLOCKS ? 1u : 0u;
-    /* few outputs and several rows (a site's 24 mixes): a block a row and an output, the one-row instance on a grid of
-     * (outputs, rows), so that eight times the units are at work; every output's operations are the same */
-    const bool by_row = form != 0u && description->row_count > 1u && description->output_size * description->row_count <= DENSE_BY_ROW_MOST_BLOCKS;
+    /* few outputs and several rows (a site's 24 mixes, up to some 170 rows): a block a row and an output, the one-row
+     * instance on a grid of (outputs, rows), so that many units are at work; every output's operations are the same */
+    const bool by_row = form != 0u && description->row_count > 1u && few_blocks;
     const uint32_t kernel = kernels->products[form * DENSE_FORM_INSTANCES + description->weight_type * DENSE_ROW_INSTANCES +
                                               (description->row_count > 1u && !by_row ? 1u : 0u)];
     if (kernel == BACKEND_NO_KERNEL) {
         REFUSE("%s: its kernel is not prepared", what);
         return STATUS_INVALID_ARGUMENT;
     }
-    const struct dense_linear_arguments record = {description->weights.byte_offset, description->rows.byte_offset, description->output.byte_offset, 0,
-                                                  description->output_size, description->input_size, description->row_count,
-                                                  description->output_type, description->flags, description->output_scale, description->epsilon, 0};
     launch_fill(launch_out, kernel, description->output_size / (form != 0u ? 1u : DENSE_OUTPUTS_PER_BLOCK), by_row ? description->row_count : 1, 1,
                 DENSE_THREADS_VALUE, 0, &record, sizeof record);
     return STATUS_OK;
@@ -127,8 +157,8 @@ result_status hyper_site_prepare(const struct hyper_site_description *descriptio
         return STATUS_INVALID_ARGUMENT;
     }
     const uint32_t width = description->reserved_zero != 0u ? description->reserved_zero : SITE_DEFAULT_WIDTH, rows = description->row_count;
-    if (rows == 0u || rows > LINEAR_MAXIMUM_ROWS || width % SITE_WIDTH_STEP != 0u || width > SITE_MOST_WIDTH) {
-        REFUSE("%s: 1 to %u rows of a width in whole %u up to %u", what, LINEAR_MAXIMUM_ROWS, SITE_WIDTH_STEP, SITE_MOST_WIDTH);
+    if (rows == 0u || rows > DENSE_MOST_ROWS || width % SITE_WIDTH_STEP != 0u || width > SITE_MOST_WIDTH) {
+        REFUSE("%s: 1 to %u rows of a width in whole %u up to %u", what, DENSE_MOST_ROWS, SITE_WIDTH_STEP, SITE_MOST_WIDTH);
         return STATUS_INVALID_ARGUMENT;
     }
     const bool combined = description->routed_sums.byte_count != 0u;

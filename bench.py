@@ -152,19 +152,19 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         if rows <= amd.LINEAR_MAXIMUM_ROWS:  # a thin step: the shared expert's down and the join in one launch
             parts = parts[:-1] + [four[i] for i in range(3)] + [shared.shared_join_launch()[0]]
             names = names[:-1] + ["trunk_gate_up", "trunk_hidden", "activation_quantize(shared)", "expert_shared_join"]
-            # and the step ahead of the router: the site's mix project and mix finish, whose hidden rows (the collapse of
-            # the streams with the carried pre, normed) are the rows the router and the quantizer then read
-            front = amd.SiteFront(card, rows, HIDDEN, (workloads.normals(base + 910, 24 * 4 * HIDDEN) * 0.02).reshape(24, 4 * HIDDEN),
-                                  [1.0, 1.0, 1.0], workloads.normals(base + 911, 24) * 0.5, workloads.to_bf16(np.ones(HIDDEN)),
-                                  hidden_range=amd.Range(layer.x_offset, rows * HIDDEN * 2))
-            for name in ("streams", "post", "comb"):  # the join reads the post and comb the finish writes
-                front.ranges[name] = shared.ranges[name]
-            card.upload(front.ranges["carried_pre"].byte_offset, np.full((rows, 4), 0.25, dtype=np.float32))
-            parts = [front.mix_project_launch()[0], front.site_launches()[0]] + parts
-            names = ["dense_linear(mix project)", "hyper_mix_finish"] + names
         else:
             parts = parts[:-1] + [four[i] for i in range(4)] + [shared.join_launch()[0]]
             names = names[:-1] + ["trunk_gate_up", "trunk_hidden", "activation_quantize(shared)", "trunk_down", "expert_join"]
+        # and the step ahead of the router: the site's mix project and mix finish, whose hidden rows (the collapse of the
+        # streams with the carried pre, normed) are the rows the router and the quantizer then read
+        front = amd.SiteFront(card, rows, HIDDEN, (workloads.normals(base + 910, 24 * 4 * HIDDEN) * 0.02).reshape(24, 4 * HIDDEN),
+                              [1.0, 1.0, 1.0], workloads.normals(base + 911, 24) * 0.5, workloads.to_bf16(np.ones(HIDDEN)),
+                              hidden_range=amd.Range(layer.x_offset, rows * HIDDEN * 2))
+        for name in ("streams", "post", "comb"):  # the join reads the post and comb the finish writes
+            front.ranges[name] = shared.ranges[name]
+        card.upload(front.ranges["carried_pre"].byte_offset, np.full((rows, 4), 0.25, dtype=np.float32))
+        parts = [front.mix_project_launch()[0], front.site_launches()[0]] + parts
+        names = ["dense_linear(mix project)", "hyper_mix_finish"] + names
     step = amd.launches_of(len(parts))
     for i, launch in enumerate(parts):
         step[i] = launch
@@ -232,7 +232,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
             "trunk_gate_up_us": trunk_us, "trunk_gate_up_GBps": 2 * shared_matrix_bytes / (trunk_us * 1e-6) / 1e9,
             "trunk_gate_up_TFLOPs": 2.0 * rows * 2 * HIDDEN * INNER / (trunk_us * 1e-6) / 1e12}
         if front is not None:
-            result["config"]["site"]["launches"] = "the site's mix project and mix finish ahead of the router, the shared expert (E4M3 weights) and the shared join"
+            result["config"]["site"]["launches"] = "the site's mix project and mix finish ahead of the router, the shared expert (E4M3 weights) and the join"
             result["config"]["site"]["front_us"] = float(per_launch[0] + per_launch[1])
             result["config"]["site"]["mix_project_GBps"] = 24 * 4 * HIDDEN * 4 / (float(per_launch[0]) * 1e-6) / 1e9
     key = ("%s_%s" % ("fp8" if fp8 else "fp4", "prefill" if prefill else "decode"), rows)
@@ -271,14 +271,18 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
             shared.set_site(site_streams, site_post, site_comb)
             card.upload(front.ranges["carried_pre"].byte_offset, np.full((rows, 4), 0.25, dtype=np.float32))
             card.run(step)
-            live = layer.jobs()
-            live = live[live["row_count"] > 0]
-            flat = np.ascontiguousarray(site_streams.reshape(rows, -1))
-            mixes = np.zeros((rows, 24), dtype=np.float32)
+            if prefill:
+                picks = wide.read("picks", np.dtype([("expert", "<u4"), ("route_weight", "<f4")])).reshape(rows, PICKS)
+            else:
+                live = layer.jobs() if wide is None else wide.read("jobs", amd.JOB_DTYPE)
+                live = live[live["row_count"] > 0]
+            checked = rows if rows <= 64 else sample  # the rows the oracle's front computes
+            flat = np.ascontiguousarray(site_streams[:checked].reshape(checked, -1))
+            mixes = np.zeros((checked, 24), dtype=np.float32)
             assert o.orc.orc_dense_linear(1, front.constants["mix_weights"].ctypes.data_as(C.c_void_p), 24, 4 * HIDDEN, 1, 1e-20, 1.0, 1,
-                                          o.ptr(flat, o.u16p), rows, mixes.ctypes.data_as(C.c_void_p)) == 0
+                                          o.ptr(flat, o.u16p), checked, mixes.ctypes.data_as(C.c_void_p)) == 0
             x, site_post, site_comb = np.zeros((rows, HIDDEN), dtype=np.uint16), np.zeros((rows, 4), dtype=np.float32), np.zeros((rows, 4, 4), dtype=np.float32)
-            for r in range(rows):
+            for r in range(checked):
                 pre = np.full(4, 0.25, dtype=np.float32)
                 row_hidden, row_post, row_comb = np.zeros(HIDDEN, dtype=np.uint16), np.zeros(4, dtype=np.float32), np.zeros(16, dtype=np.float32)
                 o.orc.orc_hyper_mix_finish(o.ptr(np.ascontiguousarray(site_streams[r]), o.u16p), o.ptr(pre, o.f32p), o.ptr(np.ascontiguousarray(mixes[r]), o.f32p),
@@ -286,7 +290,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                                            o.ptr(front.constants["norm_weight"], o.u16p), HIDDEN, o.ptr(row_post, o.f32p), o.ptr(row_comb, o.f32p),
                                            o.ptr(row_hidden, o.u16p))
                 x[r], site_post[r], site_comb[r] = row_hidden, row_post, row_comb.reshape(4, 4)
-            assert np.array_equal(card.download(layer.x_offset, rows * HIDDEN * 2, np.uint16).reshape(rows, HIDDEN), x), "the front's rows are the oracle's bits"
+            assert np.array_equal(card.download(layer.x_offset, rows * HIDDEN * 2, np.uint16).reshape(rows, HIDDEN)[:checked], x[:checked]), \
+                "the front's rows are the oracle's bits"
         experts_of = np.zeros((rows, PICKS), dtype=np.uint32)
         weights_of = np.zeros((rows, PICKS), dtype=np.float32)
         if prefill:

@@ -451,6 +451,7 @@ uint64_t linear_jobs_byte_count(uint64_t job_count);                         /* 
  * and linear.h's above. */
 struct dense_linear_kernels {
     uint32_t products[DENSE_INSTANCES]; /* [form][type][one row, 8]: dense_linear_<type>_<R>, then _narrow */
+    uint32_t wide_products[DENSE_TYPE_COUNT]; /* dense_linear_<type>_8_wide: more than 8 rows, 8 outputs a block */
 };
 MUST_CHECK result_status dense_linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                       struct dense_linear_kernels *kernels_out);
@@ -458,8 +459,8 @@ MUST_CHECK result_status dense_linear_kernels_prepare(const struct backend_opera
 /* include/anemone/dense_linear.h:70-99 of the reference. Refused with STATUS_INVALID_ARGUMENT: a NULL argument, a
  * type outside the enumeration, a flag outside DENSE_FLAGS, an output_size that is no multiple of
  * DENSE_OUTPUTS_PER_BLOCK or an input_size that is no multiple of DENSE_CHUNK_INPUTS, 0 rows, a range that breaks the
- * range rules; with STATUS_UNSUPPORTED: more than LINEAR_MAXIMUM_ROWS rows (the wide launches), DENSE_STEP_ROWS and
- * DENSE_CONE_ROWS. */
+ * range rules, more than DENSE_MOST_ROWS rows; with STATUS_UNSUPPORTED: DENSE_STEP_ROWS and DENSE_CONE_ROWS. More than
+ * LINEAR_MAXIMUM_ROWS rows: a wide launch, groups of 8 rows on grid[1], every output's bits those of its group's launch. */
 struct dense_linear_description {
     struct linear_range weights; /* read: [output_size][input_size] of weight_type, exactly */
     struct linear_range rows;    /* read: bf16 [row_count][input_size] */
@@ -493,7 +494,7 @@ MUST_CHECK result_status hyper_kernels_prepare(const struct backend_operations *
 
 /* A site of a block (include/anemone/hyper_connection.h:40-71): its mix finish, between its mix project and its
  * sublayer, and its post after the sublayer, with the combine where routed_sums has bytes (the FFN site). 1 to
- * LINEAR_MAXIMUM_ROWS rows. */
+ * 65535 rows (a thin step's, or a prefill chunk's: a row's bits are its own). */
 enum hyper_site_launch { HYPER_SITE_MIX_FINISH = 0, HYPER_SITE_POST = 1, HYPER_SITE_LAUNCH_COUNT = 2 };
 struct hyper_site_description {
     struct linear_range streams;     /* read and written: bf16 [row_count][4][width] */

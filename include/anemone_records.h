@@ -659,6 +659,8 @@ enum dense_type_code { DENSE_BFLOAT16 = 0, DENSE_FLOAT32 = 1, DENSE_TYPE_COUNT =
 #define DENSE_INSTANCES 8u      /* forms by types by row counts: [form][type][one row, 8] */
 #define DENSE_FORM_INSTANCES 4u
 #define DENSE_ROW_INSTANCES 2u
+#define DENSE_WIDE_OUTPUTS 8u /* outputs of a block of dense_linear_<type>_8_wide: steps of more than 8 rows, groups of 8 on grid[1] */
+#define DENSE_MOST_ROWS 65535u
 
 /* Launch: function dense_linear_<type>_<R>[_narrow], R 1 for one row and 8 for 2 to 8; grid (output_size / outputs of
  * a block, 1), block 256. */

@@ -762,8 +762,18 @@ def test_site_front_launches_geometry_and_refusals(fake):
     one = dense_description(outputs=4096, inputs=2048, rows=1, weight_type=0, output_type=0, flags=0)
     assert lib.dense_linear_prepare(C.byref(one), arena, C.byref(dense), launch) == 0
     assert fake.handles[launch[0].kernel][1] == "dense_linear_bfloat16_1" and list(launch[0].grid) == [1024, 1, 1]
+    # more rows: groups of 8 on grid[1], 8 outputs a block where they divide
+    many = dense_description(rows=8192)
+    assert lib.dense_linear_prepare(C.byref(many), arena, C.byref(dense), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "dense_linear_float32_8_wide" and list(launch[0].grid) == [3, 1024, 1]
+    odd = dense_description(outputs=20, rows=370)
+    assert lib.dense_linear_prepare(C.byref(odd), arena, C.byref(dense), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "dense_linear_float32_8" and list(launch[0].grid) == [5, 47, 1]
+    middling = dense_description(rows=32)  # few outputs, some rows: still a block a row and an output
+    assert lib.dense_linear_prepare(C.byref(middling), arena, C.byref(dense), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "dense_linear_float32_1_narrow" and list(launch[0].grid) == [24, 32, 1]
     untouched = amd.launches_of(1)
-    for changes, status in [(dict(row_count=0), 1), (dict(row_count=9), 7), (dict(flags=3), 7), (dict(flags=8), 1), (dict(weight_type=2), 1),
+    for changes, status in [(dict(row_count=0), 1), (dict(row_count=600000), 1), (dict(flags=3), 7), (dict(flags=8), 1), (dict(weight_type=2), 1),
                             (dict(output_size=26), 1), (dict(input_size=16388), 1), (dict(cone_layer=1), 7),
                             (dict(weights=amd.Range(1 << 20, 24 * 16384 * 4 + 16)), 1), (dict(output=amd.Range((1 << 20) + 256, 1024)), 1)]:
         assert lib.dense_linear_prepare(C.byref(dense_description(**changes)), arena, C.byref(dense), untouched) == status, changes
@@ -784,8 +794,11 @@ def test_site_front_launches_geometry_and_refusals(fake):
     assert lib.hyper_site_prepare(C.byref(plain), arena, C.byref(hyper), launches) == 0
     assert launches[0].block[0] == 640 and list(launches[1].grid) == [5, 3, 1]
     assert struct.unpack("<5QII", bytes(launches[1].argument)[:48])[4:] == (0, 0, 0)
+    chunk = site_description(rows=2048)
+    assert lib.hyper_site_prepare(C.byref(chunk), arena, C.byref(hyper), launches) == 0
+    assert list(launches[0].grid) == [1, 2048, 1] and list(launches[1].grid) == [4, 2048, 1]
     untouched = amd.launches_of(2)
-    for changes in (dict(row_count=0), dict(row_count=9), dict(reserved_zero=4100), dict(reserved_zero=9216), dict(scale=amd.Range(1 << 30, 16)),
+    for changes in (dict(row_count=0), dict(row_count=70000), dict(reserved_zero=4100), dict(reserved_zero=9216), dict(scale=amd.Range(1 << 30, 16)),
                     dict(mixes=amd.Range((1 << 20) + 64, 1024)), dict(hidden=amd.Range((8 << 30) - 256, 8 * 4096 * 2))):
         assert lib.hyper_site_prepare(C.byref(site_description(**changes)), arena, C.byref(hyper), untouched) == 1, changes
         assert not any(bytes(untouched))

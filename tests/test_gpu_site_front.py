@@ -60,7 +60,7 @@ def oracle_dense(weight_type, weights, rows, flags, epsilon, scale, output_type)
     return out
 
 
-@pytest.mark.parametrize("rows,width,live", [(8, 4096, 8), (1, 5120, 1), (5, 1024, 3), (2, 8192, 2)])
+@pytest.mark.parametrize("rows,width,live", [(8, 4096, 8), (1, 5120, 1), (5, 1024, 3), (2, 8192, 2), (37, 1024, 37), (300, 2048, 291)])
 def test_mix_project_and_finish_bit_for_bit(amd, card, rows, width, live):
     say("site front: mix project, finish", rows, width, live)
     front, streams, carried = front_of(amd, card, rows, width, 10 * rows + width)
@@ -117,7 +117,8 @@ def test_finish_with_specials_in_the_streams(amd, card):
 
 
 @pytest.mark.parametrize("weight_type,outputs,inputs,rows,output_type,scale", [(0, 256, 4096, 8, 1, 1.0), (0, 384, 5120, 1, 1, 1.0),
-                                                                              (0, 2048, 1024, 3, 0, 0.125), (1, 64, 264, 2, 0, 1.0)])
+                                                                              (0, 2048, 1024, 3, 0, 0.125), (1, 64, 264, 2, 0, 1.0),
+                                                                              (0, 64, 1024, 100, 1, 1.0), (1, 20, 512, 37, 0, 0.5), (1, 20, 512, 237, 0, 0.5)])
 def test_dense_products_bit_for_bit(amd, card, weight_type, outputs, inputs, rows, output_type, scale):
     """The router's scores in the dense product's order (bfloat16 weights, float32 out) and the other forms: four outputs
     a block and one, one row and several, a bfloat16 output with a scale."""
