@@ -266,7 +266,7 @@ __device__ static __forceinline__ void tcp_wait_loads()
  *   columns    the chunk's first operand row (fp16 [pair][inputs], rows of the chunk consecutive), count of them
  *   stage      LDS address of the block's two operand stages; window: of this wavefront's two weight windows
  * Lane L of an operand load lands at bytes 16 L of a 16-column group: column L / 4, slot L % 4, and asks for that
- * column's 16-byte piece (L % 4) ^ ((column / 2) % 4) of the step, so that the readers of one piece of sixteen columns
+ * column's 16-byte piece (L % 4) ^ (column / 4) of the step, so that the readers of one piece of sixteen columns
  * meet different banks. */
 template <uint32_t bits_x2, uint32_t LIVE>
 __device__ static __forceinline__ void
@@ -287,7 +287,7 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
                                          (lane / row_lanes) * row_stride + (lane % row_lanes) * 16u;
     /* operands: this wavefront brings TCP_OPERAND_PARTS of the step's 16-column groups: wave, wave + 4, ... (a group
      * past the chunk's columns lands in the stage's spare room) */
-    const uint32_t load_column = lane / 4u, load_piece = (lane % 4u) ^ ((load_column / 2u) % 4u);
+    const uint32_t load_column = lane / 4u, load_piece = (lane % 4u) ^ (load_column / 4u);
     const unsigned char *operand_source[TCP_OPERAND_PARTS]; /* a column past the chunk's last reads the first again: never stored */
 #pragma unroll
     for (uint32_t part = 0; part < TCP_OPERAND_PARTS; part++) {
@@ -295,7 +295,7 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
         operand_source[part] = (const unsigned char *)(columns + (uint64_t)(column < column_count ? column : 0u) * inputs) + load_piece * 16u;
     }
     /* where this lane reads its operand halves of column block j: column o, pieces 2 tau and 2 tau + 1, bytes 8 q .. */
-    const uint32_t swizzle = (o / 2u) % 4u;
+    const uint32_t swizzle = o / 4u;
     const uint32_t read_low = o * 64u + ((2u * tau) ^ swizzle) * 16u + 8u * q, read_high = o * 64u + ((2u * tau + 1u) ^ swizzle) * 16u + 8u * q;
 #pragma unroll
     for (uint32_t n = 0; n < TCP_WAVE_TILES; n++) {
