@@ -288,7 +288,8 @@ __device__ static __forceinline__ uint64_t wave_max_u64(uint64_t value)
 }
 
 /* One row by one wavefront: its picks by slot and their weights, written by lane 0. */
-__device__ static void router_row(const float *affinities, const float *bias, uint32_t lane, uint32_t experts,
+/* bias: the lane's values of the experts lane, lane + 64, ... (asked for before the affinities are there) */
+__device__ static void router_row(const float *affinities, const float (&bias)[ROUTER_MOST_EXPERTS / WAVE], uint32_t lane, uint32_t experts,
                                   uint32_t picks, uint32_t reference_order, float route_scale, uint32_t *chosen,
                                   float *weights)
 {
@@ -299,7 +300,7 @@ __device__ static void router_row(const float *affinities, const float *bias, ui
 #pragma unroll
     for (uint32_t place = 0; place < ROUTER_MOST_EXPERTS / WAVE; place++) {
         const uint32_t expert = lane + place * WAVE;
-        keys[place] = place < places ? router_key(__fadd_rn(affinities[expert], bias[expert]), expert) : 0ull;
+        keys[place] = place < places ? router_key(__fadd_rn(affinities[expert], bias[place]), expert) : 0ull;
     }
 #pragma unroll
     for (uint32_t pick = 0; pick < ROUTER_MOST_PICKS; pick++) {
@@ -380,6 +381,12 @@ extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
     const uint32_t live_rows = step_rows < arguments.row_count ? step_rows : arguments.row_count;
     const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const uint32_t pair = threadIdx.x, pair_count = live_rows * picks;
+    /* the lane's bias values, asked for now: they arrive while the affinities are formed */
+    float bias_of[ROUTER_MOST_EXPERTS / WAVE];
+#pragma unroll
+    for (uint32_t place = 0; place < ROUTER_MOST_EXPERTS / WAVE; place++) {
+        bias_of[place] = lane + place * WAVE < experts ? ((const float *)(arena + arguments.bias_offset))[lane + place * WAVE] : 0.0f;
+    }
     for (uint32_t index = threadIdx.x; index < live_rows * experts; index += blockDim.x) {
         const float a = router_affinity(((const float *)(arena + arguments.scores_offset))[index], arguments.affinity_kind);
         affinities[index] = a;
@@ -387,7 +394,7 @@ extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
     }
     __syncthreads();
     if (wave < live_rows) {
-        router_row(affinities + wave * experts, (const float *)(arena + arguments.bias_offset), lane, experts, picks,
+        router_row(affinities + wave * experts, bias_of, lane, experts, picks,
                    arguments.reference_order, scale, pair_experts + wave * picks, pair_weights + wave * picks);
     }
     __syncthreads();
@@ -473,6 +480,11 @@ extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
     }
     const uint32_t rows = live_rows - first_row < LINEAR_MAXIMUM_ROWS ? live_rows - first_row : LINEAR_MAXIMUM_ROWS;
     const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    float bias_of[ROUTER_MOST_EXPERTS / WAVE]; /* the lane's bias values, asked for ahead of the affinities */
+#pragma unroll
+    for (uint32_t place = 0; place < ROUTER_MOST_EXPERTS / WAVE; place++) {
+        bias_of[place] = lane + place * WAVE < experts ? ((const float *)(arena + arguments.bias_offset))[lane + place * WAVE] : 0.0f;
+    }
     for (uint32_t index = threadIdx.x; index < rows * experts; index += blockDim.x) {
         const uint64_t at = (uint64_t)first_row * experts + index;
         const float a = router_affinity(((const float *)(arena + arguments.scores_offset))[at], arguments.affinity_kind);
@@ -481,7 +493,7 @@ extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
     }
     __syncthreads();
     if (wave < rows) {
-        router_row(affinities + wave * experts, (const float *)(arena + arguments.bias_offset), lane, experts, picks,
+        router_row(affinities + wave * experts, bias_of, lane, experts, picks,
                    arguments.reference_order, arguments.route_scale, pick_experts + wave * picks, pick_weights + wave * picks);
     }
     __syncthreads();
