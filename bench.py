@@ -443,7 +443,8 @@ def main():
     parser.add_argument("--block128", action="store_true",
                         help="fp8 workloads: float32 scales of 128 x 128 weight blocks and of 128 activation values in place of the reference's E8M0 scales")
     parser.add_argument("--site", action="store_true",
-                        help="fp4/fp8 workloads: the whole FFN site, with the shared expert and the join in place of the row sum")
+                        help="fp4/fp8 workloads: the whole FFN site: the mix project and mix finish ahead of the router, the shared expert and the join "
+                             "in place of the row sum")
     parser.add_argument("--graph", action="store_true", help="time replays of the step captured as one graph (graph_capture / graph_run)")
     parser.add_argument("--calibrate", action="store_true",
                         help="run only a 1 GiB arena copy, five times: the yardstick of the traffic counters")
