@@ -163,3 +163,75 @@ def test_site_from_streams_to_streams(amd, card):
         orc.orc_hyper_post(ptr(np.ascontiguousarray(streams[r]), u16p), ptr(post_of, f32p), ptr(comb, f32p), ptr(np.ascontiguousarray(output[r]), u16p),
                            ptr(np.ascontiguousarray(sums[r]), f32p), width, ptr(want, u16p))
         assert np.array_equal(got[r], want), r
+
+
+def test_a_layer_from_streams_to_streams(amd, card):
+    """A whole FFN site of a wide step on the card, streams in and streams out: the mix project and mix finish, the
+    router and its wide select, the FP4 routed experts in their wide form, the shared expert, the join. The front's rows,
+    post and comb bit for bit the oracle's; the streams against the oracle's composition of its own stages; and the join
+    exact on the card's own pair and shared outputs."""
+    say("a layer from streams to streams")
+    from anemone_amd import workloads
+    from test_gpu_router_wide import oracle_wide
+    from _oracle import bf16_to_f32, u32p
+    E2M1, E4M3 = 3, 5
+    hidden, inner, experts_n, picks, rows = 1024, 256, 64, 4, 100
+    matrices = [[workloads.fp4_matrix(7000 + 3 * e, inner, hidden), workloads.fp4_matrix(7001 + 3 * e, inner, hidden),
+                 workloads.fp4_matrix(7002 + 3 * e, hidden, inner)] for e in range(experts_n)]
+    router = to_bf16(normals(5, experts_n * hidden) * 0.02).reshape(experts_n, hidden)
+    layer = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router)
+    shared_matrices = [workloads.fp8_matrix(61, inner, hidden), workloads.fp8_matrix(62, inner, hidden), workloads.fp8_matrix(63, hidden, inner)]
+    shared = amd.SharedExpert(layer, shared_matrices)
+    mix_weights = (normals(70, MIXES * STREAMS * hidden) * 0.02).astype(np.float32).reshape(MIXES, STREAMS * hidden)
+    scale, base = np.array([1.0, 0.8, 1.2], np.float32), (normals(71, MIXES) * 0.5).astype(np.float32)
+    norm_weight = to_bf16(normals(72, hidden) * 0.1 + 1.0)
+    front = amd.SiteFront(card, rows, hidden, mix_weights, scale, base, norm_weight, hidden_range=amd.Range(layer.x_offset, rows * hidden * 2))
+    for name in ("streams", "post", "comb"):
+        front.ranges[name] = shared.ranges[name]
+    streams = to_bf16(normals(73, rows * STREAMS * hidden)).reshape(rows, STREAMS, hidden)
+    carried = (np.abs(normals(74, rows * STREAMS)) * 0.3 + 0.1).astype(np.float32).reshape(rows, STREAMS)
+    front.set_streams(streams, carried)
+    layer.set_rows(np.zeros((rows, hidden), np.uint16))  # the rows are the front's to write
+    card.run(front.mix_project_launch())
+    card.run(front.site_launches()[:1])
+    card.run(layer.projection_launch())
+    wide = layer.wide_router()
+    card.run(wide.launches())
+    card.run(layer.quantize_launch())
+    card.run(layer.wide_expert_launches(wide)[:2])
+    card.run(shared.launches())
+    card.run(shared.join_launch())
+    # the oracle's front
+    mixes = oracle_dense(1, mix_weights, np.ascontiguousarray(streams.reshape(rows, -1)), 1, 1e-20, 1.0, 1)
+    x, post, comb = np.zeros((rows, hidden), np.uint16), np.zeros((rows, 4), np.float32), np.zeros((rows, 16), np.float32)
+    for r in range(rows):
+        pre = carried[r].copy()
+        orc.orc_hyper_mix_finish(ptr(np.ascontiguousarray(streams[r]), u16p), ptr(pre, f32p), ptr(np.ascontiguousarray(mixes[r]), f32p), ptr(scale, f32p),
+                                 ptr(base, f32p), ptr(norm_weight, u16p), hidden, ptr(post[r], f32p), ptr(comb[r], f32p), ptr(x[r], u16p))
+    assert np.array_equal(card.download(layer.x_offset, rows * hidden * 2, np.uint16).reshape(rows, hidden), x)
+    assert np.array_equal(shared.read("post", np.float32).view(np.uint32), post.reshape(-1).view(np.uint32))
+    assert np.array_equal(shared.read("comb", np.float32).view(np.uint32), comb.reshape(-1).view(np.uint32))
+    # its routed experts (the card's own routing of those rows), its shared expert, its join
+    scores = card.download(layer.scores_offset, rows * experts_n * 4, np.float32).reshape(rows, experts_n)
+    _, experts, weights, _, _, _, _ = oracle_wide(layer, scores, np.zeros(experts_n, dtype=np.float32), rows)
+    pointers = (C.c_void_p * (experts_n * 3))(*[m.ctypes.data for trio in matrices for m in trio])
+    routed_rows, routed_pairs = np.zeros((rows, hidden), dtype=np.float32), np.zeros((rows * picks, hidden), dtype=np.uint16)
+    orc.orc_linear_moe_layer(E2M1, ptr(x, u16p), rows, hidden, inner, picks, ptr(np.ascontiguousarray(experts), u32p),
+                             ptr(np.ascontiguousarray(weights), f32p), experts_n, pointers, layer.limit, ptr(routed_rows, f32p), None,
+                             ptr(routed_pairs, u16p), 8)
+    shared_pointers = (C.c_void_p * 3)(*[m.ctypes.data for m in shared_matrices])
+    one, ones = np.zeros((rows, 1), dtype=np.uint32), np.ones((rows, 1), dtype=np.float32)
+    unused, shared_output = np.zeros((rows, hidden), dtype=np.float32), np.zeros((rows, hidden), dtype=np.uint16)
+    orc.orc_linear_moe_layer(E4M3, ptr(x, u16p), rows, hidden, inner, 1, ptr(one, u32p), ptr(ones, f32p), 1, shared_pointers, layer.limit,
+                             ptr(unused, f32p), None, ptr(shared_output, u16p), 8)
+    want = streams.copy()
+    orc.orc_expert_join(ptr(routed_pairs, u16p), ptr(shared_output, u16p), ptr(want, u16p), ptr(post, f32p), ptr(comb, f32p), None, rows, picks, hidden)
+    got = bf16_to_f32(shared.read("streams", np.uint16)).astype(np.float64)
+    wanted = bf16_to_f32(want.reshape(-1)).astype(np.float64)
+    error = np.sqrt(np.mean((got - wanted) ** 2) / np.mean(wanted ** 2))
+    say("  streams rms error vs oracle: %.2e" % error)
+    assert error < 2e-2
+    exact = streams.copy()
+    pairs_card, shared_card = layer.read("pair_output", np.uint16), shared.read("output", np.uint16)
+    orc.orc_expert_join(ptr(pairs_card, u16p), ptr(shared_card, u16p), ptr(exact, u16p), ptr(post, f32p), ptr(comb, f32p), None, rows, picks, hidden)
+    assert np.array_equal(shared.read("streams", np.uint16).reshape(rows, STREAMS, hidden), exact)
