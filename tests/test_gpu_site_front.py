@@ -235,3 +235,37 @@ def test_a_layer_from_streams_to_streams(amd, card):
     pairs_card, shared_card = layer.read("pair_output", np.uint16), shared.read("output", np.uint16)
     orc.orc_expert_join(ptr(pairs_card, u16p), ptr(shared_card, u16p), ptr(exact, u16p), ptr(post, f32p), ptr(comb, f32p), None, rows, picks, hidden)
     assert np.array_equal(shared.read("streams", np.uint16).reshape(rows, STREAMS, hidden), exact)
+
+
+def test_exl3_decode_into_the_shared_rows_then_the_plain_post(amd, card):
+    """The EXL3 site of a decode step as the reference's fused decode runs it (include/anemone/exl3_tc_records.h:52-57):
+    the combine adds the routed sums to the shared expert's bfloat16 rows in place (shared_sum 1), and the site's post
+    without the combine takes those rows as the sublayer's output. Against the oracle's post of bfloat16(sum + row) of the
+    card's own sums (the float32 form of the same launches), bit for bit."""
+    say("EXL3 decode, shared sum, plain post")
+    from test_gpu_exl3 import build_layer
+    hidden, inner, experts_n, picks, rows = 1024, 256, 64, 4, 8
+    layer, _, _, _ = build_layer(amd, card, hidden, inner, experts_n, picks, rows, 5, [2, 3, 4])
+    x = to_bf16(normals(41, rows * hidden)).reshape(rows, hidden)
+    layer.set_rows(x, rows)
+    card.run(layer.projection_launch())
+    card.run(layer.select_launch(0))
+    card.run(layer.tc_launches())
+    sums = layer.output()[:rows].copy()  # float32 [rows][hidden]
+    front, streams, carried = front_of(amd, card, rows, hidden, 77)
+    shared_rows = to_bf16(normals(42, rows * hidden) * float(np.sqrt(np.mean(sums.astype(np.float64) ** 2)))).reshape(rows, hidden)
+    card.upload(front.ranges["output"].byte_offset, shared_rows)
+    post = (normals(43, rows * STREAMS) * 0.5 + 1.0).astype(np.float32).reshape(rows, STREAMS)
+    comb = (np.abs(normals(44, rows * STREAMS * STREAMS)) * 0.3).astype(np.float32).reshape(rows, STREAMS, STREAMS)
+    card.upload(front.ranges["post"].byte_offset, post)
+    card.upload(front.ranges["comb"].byte_offset, comb)
+    card.run(layer.tc_launches(front.ranges["output"].byte_offset))
+    card.run(front.site_launches(combined=False)[1:])
+    got = front.read("streams", np.uint16).reshape(rows, STREAMS, hidden)
+    summed = to_bf16(sums + (shared_rows.astype(np.uint32) << 16).view(np.float32))
+    assert np.array_equal(front.read("output", np.uint16).reshape(rows, hidden), summed)
+    for r in range(rows):
+        want = np.zeros((STREAMS, hidden), np.uint16)
+        orc.orc_hyper_post(ptr(np.ascontiguousarray(streams[r]), u16p), ptr(post[r], f32p), ptr(np.ascontiguousarray(comb[r]), f32p),
+                           ptr(np.ascontiguousarray(summed[r]), u16p), None, hidden, ptr(want, u16p))
+        assert np.array_equal(got[r], want), r
