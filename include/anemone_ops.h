@@ -19,6 +19,7 @@
 #define ANEMONE_OPS_H
 
 #include <stdbool.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "anemone_backend.h"
@@ -513,5 +514,50 @@ struct hyper_site_description {
 };
 MUST_CHECK result_status hyper_site_prepare(const struct hyper_site_description *description, uint64_t arena_byte_count,
                                             const struct hyper_kernels_record *kernels, struct kernel_launch *launches_out);
+
+/* ---- load-time EXL3 slices (include/anemone/exl3_layout.h:15-103, source/exl3_layout.c of the reference) ----
+ * A stored EXL3 matrix is [input / 16][output / 16][16 K] uint16 of codes, then suh[input], svh[output]. A slice keeps
+ * whole transforms of 128 channels on either side, so a sliced matrix is a stored EXL3 matrix of the slice's shape: its
+ * codes the code rows of the input range cut to the output range, its suh and svh the ranges' own. Nothing is decoded
+ * and no arithmetic touches a weight: the kernels of this library give, for a slice of outputs with the whole of the
+ * inputs, the bits they give for those outputs of the whole matrix (tested on the card), which is what lets a card
+ * take a share of a layer's columns. Host-only code; no device or step-loop dependency. */
+#define BB_EXL3_TP_RANKS 4u
+struct bb_exl3_matrix_slice {
+    uint32_t input_size, output_size;   /* of the whole matrix */
+    uint32_t input_begin, input_count;  /* whole transforms of 128 */
+    uint32_t output_begin, output_count;
+    uint32_t bits_per_weight;           /* a stored width this build decodes */
+    uint32_t reserved_zero;
+};
+struct bb_exl3_slice_sizes {
+    uint64_t source_bytes; /* of the whole matrix as stored */
+    uint64_t packed_bytes; /* of the slice as stored */
+};
+/* STATUS_INVALID_ARGUMENT (sizes_out unchanged) for a NULL argument, a reserved field that is not zero, a count of
+ * zero, a size, origin or count that is no multiple of 128, a range past its dimension, a width this build has no
+ * kernels for. */
+MUST_CHECK result_status bb_exl3_matrix_slice_prepare(const struct bb_exl3_matrix_slice *slice, struct bb_exl3_slice_sizes *sizes_out);
+/* The lossless copy at load. The source holds the whole matrix (source_bytes at least its stored bytes), the
+ * destination at least the slice's; the two may not overlap. Refused before a byte is written. */
+MUST_CHECK result_status bb_exl3_matrix_slice_copy(const struct bb_exl3_matrix_slice *slice, const void *source, size_t source_bytes,
+                                                   void *destination, size_t destination_bytes);
+
+enum bb_exl3_product_order { BB_EXL3_REFERENCE_ORDER = 0, BB_EXL3_EIGHT_PART_ORDER = 1 };
+/* What one of rank_count cards (1 or BB_EXL3_TP_RANKS) takes of an expert: gate and up its share of the intermediate
+ * outputs with all the inputs, down its share of the outer outputs with all the intermediate inputs: every product
+ * keeps its whole K dimension, so its K slices and their order are the whole matrix's. Metadata only: nothing here
+ * allocates, launches or moves data between cards. */
+struct bb_exl3_output_shard_plan {
+    struct bb_exl3_matrix_slice gate_up;
+    struct bb_exl3_matrix_slice down;
+    uint32_t rank_count;
+    uint32_t rank;
+    uint32_t product_slices;
+    enum bb_exl3_product_order order;
+};
+MUST_CHECK result_status bb_exl3_output_shard_prepare(uint32_t outer_size, uint32_t inner_size, uint32_t bits_per_weight, uint32_t rank_count,
+                                                      uint32_t rank, enum bb_exl3_product_order order,
+                                                      struct bb_exl3_output_shard_plan *plan_out);
 
 #endif

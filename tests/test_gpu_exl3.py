@@ -253,3 +253,52 @@ def test_single_linear_config0_shape(amd, card):
     say("  max err / rms", float(np.max(np.abs(got - want)) / rms))
     assert np.max(np.abs(got - want)) <= 2e-3 * rms  # fp16 operand rounding (2^-11 a value) dominates
 
+
+
+@pytest.mark.parametrize("width", [2, 40, 3, 4])
+def test_a_slice_of_outputs_gives_the_whole_matrix_bits(amd, card, width):
+    """The load-time slices (bb_exl3_matrix_slice_copy, include/anemone/exl3_layout.h:28-49 of the reference): a slice of
+    a matrix's outputs with all of its inputs, as its own stored matrix, through the chain's input and gate product
+    launches: the float32 products of the slice's outputs are the whole matrix's, bit for bit. This is what lets a card
+    take a share of a layer's columns."""
+    say("slice of outputs, width", width)
+    import ctypes as ct
+    inputs, outputs, begin, count = 1024, 768, 256, 384
+
+    class Slice(ct.Structure):
+        _fields_ = [(name, ct.c_uint32) for name in ("input_size", "output_size", "input_begin", "input_count", "output_begin", "output_count",
+                                                     "bits_per_weight", "reserved_zero")]
+    matrix = exl3_matrix(0x51CE0 + width, inputs, outputs, width)
+    description = Slice(inputs, outputs, 0, inputs, begin, count, width, 0)
+    sliced = np.zeros(int(orc.orc_exl3_code_bytes(inputs, count, width)) + 2 * (inputs + count), dtype=np.uint8)
+    lib = card.lib
+    lib.bb_exl3_matrix_slice_copy.restype = ct.c_int
+    lib.bb_exl3_matrix_slice_copy.argtypes = [ct.POINTER(Slice), ct.c_void_p, ct.c_size_t, ct.c_void_p, ct.c_size_t]
+    assert lib.bb_exl3_matrix_slice_copy(ct.byref(description), matrix.ctypes.data, matrix.nbytes, sliced.ctypes.data, sliced.nbytes) == 0
+    x = to_bf16(normals(0x51CE1, inputs))
+    x_at = card.place(x)
+
+    def products_of(stored, outs):
+        at = card.place(stored, 256)
+        jobs = np.zeros(1, dtype=JOB_DTYPE)
+        jobs[0]["gate_offset"] = jobs[0]["up_offset"] = jobs[0]["down_offset"] = at
+        jobs[0]["row_count"], jobs[0]["route_weight"][0] = 1, 1.0
+        record = amd.Exl3ExpertRecord()
+        record.jobs_offset = card.place(jobs.view(np.uint8))
+        record.input_offset = x_at
+        record.operands_offset = card.reserve(inputs * 4)
+        record.products_offset = record.output_offset = card.reserve(2 * max(inputs, outs) * 4)
+        record.hidden_offset = card.reserve(max(inputs, outs) * 2)
+        record.input_size, record.inner_size = inputs, outs
+        record.pair_count = record.pairs_per_row = record.job_count = 1
+        record.bits_per_weight, record.activation_limit = width, 10.0
+        launches = amd.launches_of(5)
+        amd.check(card.lib.exl3_experts_prepare(C.byref(record), card.arena_bytes, amd.backend_table(), card.handle, 950, launches), "prepare")
+        two = amd.launches_of(2)
+        two[0], two[1] = launches[0], launches[1]
+        two[0].grid[2] = two[1].grid[2] = 1  # the gate projection alone
+        card.run(two)
+        return card.download(record.products_offset, outs * 4, np.float32)
+    whole, part = products_of(matrix, outputs), products_of(sliced, count)
+    assert np.array_equal(part.view(np.uint32), whole[begin:begin + count].view(np.uint32))
+    assert np.any(part != 0)
