@@ -29,15 +29,7 @@
 
 #define DENSE_GROUP_LANES 32u
 #define DENSE_GROUPS (DENSE_THREADS_VALUE / DENSE_GROUP_LANES)
-
-__device__ static __forceinline__ float dense_group_sum(float value)
-{
-#pragma unroll
-    for (uint32_t distance = DENSE_GROUP_LANES / 2u; distance != 0u; distance /= 2u) {
-        value = __fadd_rn(value, __shfl_xor(value, (int)distance, (int)DENSE_GROUP_LANES));
-    }
-    return value;
-}
+#define DENSE_DIES 8u
 
 /* the float32 nearest 1 / sqrt(operand): both steps are correctly rounded in double, whose 53 places decide a tie */
 __device__ static __forceinline__ float dense_reciprocal_root(float operand)
@@ -50,7 +42,19 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
 {
     __shared__ float group_sums[DENSE_GROUPS][OUTPUTS + 1u][ROWS];
     const uint32_t thread = threadIdx.x, inputs = arguments.input_size, chunks = inputs / DENSE_CHUNK_INPUTS;
-    const uint32_t first_output = blockIdx.x * OUTPUTS, first_row = blockIdx.y * ROWS;
+    /* Blocks go to the card's 8 dies in turn by their linear index, and each die has its own L2. The blocks that share a
+     * group of rows (one an output group) are renumbered to follow each other on one die, so that the rows come from
+     * memory once and from that die's L2 for the other output groups: a bijection of the grid when its row groups
+     * divide by 8, the plain numbering otherwise. Which block computes an output changes nothing in its bits. */
+    uint32_t output_group = blockIdx.x, row_group = blockIdx.y;
+    if constexpr (ROWS != 1u) {
+        if (gridDim.y % DENSE_DIES == 0u) {
+            const uint32_t linear = blockIdx.x + gridDim.x * blockIdx.y, place = linear / DENSE_DIES;
+            output_group = place % gridDim.x;
+            row_group = place / gridDim.x * DENSE_DIES + linear % DENSE_DIES;
+        }
+    }
+    const uint32_t first_output = output_group * OUTPUTS, first_row = row_group * ROWS;
     const bool scaled = (arguments.flags & DENSE_ROW_SCALE) != 0u;
     const uint16_t *rows = (const uint16_t *)(arena + arguments.rows_offset);
     float chain[OUTPUTS][ROWS], squares[ROWS];
@@ -64,13 +68,39 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
     }
 #pragma unroll(ROWS == 1u ? 4 : 1)
     for (uint32_t chunk = thread; chunk < chunks; chunk += DENSE_THREADS_VALUE) {
-        float values[ROWS][DENSE_CHUNK_INPUTS];
+        /* every row's chunk is asked for before any is used: a chunk costs one trip to memory, not one a row */
+        uint4_t packed[ROWS];
 #pragma unroll
         for (uint32_t r = 0; r < ROWS; r++) {
             /* a column from row_count on reads row 0 and is stored nowhere */
             const uint32_t row = first_row + r < arguments.row_count ? first_row + r : 0u;
-            unpack_bf16x8(*(const uint4_t *)(rows + (uint64_t)row * inputs + chunk * DENSE_CHUNK_INPUTS), values[r]);
-            if (scaled) {
+            packed[r] = *(const uint4_t *)(rows + (uint64_t)row * inputs + chunk * DENSE_CHUNK_INPUTS);
+        }
+        /* and every output's weights before the first chain runs */
+        float weights[OUTPUTS][DENSE_CHUNK_INPUTS];
+#pragma unroll
+        for (uint32_t o = 0; o < OUTPUTS; o++) {
+            const uint64_t at = (uint64_t)(first_output + o) * inputs + chunk * DENSE_CHUNK_INPUTS;
+            if constexpr (TYPE == DENSE_FLOAT32) {
+                const float4_t low = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at);
+                const float4_t high = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at + 4u);
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; i++) {
+                    weights[o][i] = low[i];
+                    weights[o][4u + i] = high[i];
+                }
+            } else {
+                unpack_bf16x8(*(const uint4_t *)((const uint16_t *)(arena + arguments.weights_offset) + at), weights[o]);
+            }
+        }
+        float values[ROWS][DENSE_CHUNK_INPUTS];
+#pragma unroll
+        for (uint32_t r = 0; r < ROWS; r++) {
+            unpack_bf16x8(packed[r], values[r]);
+        }
+        if (scaled) {
+#pragma unroll
+            for (uint32_t r = 0; r < ROWS; r++) {
 #pragma unroll
                 for (uint32_t i = 0; i < DENSE_CHUNK_INPUTS; i++) {
                     squares[r] = __fmaf_rn(values[r][i], values[r][i], squares[r]);
@@ -79,42 +109,40 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
         }
 #pragma unroll
         for (uint32_t o = 0; o < OUTPUTS; o++) {
-            float weights[DENSE_CHUNK_INPUTS];
-            const uint64_t at = (uint64_t)(first_output + o) * inputs + chunk * DENSE_CHUNK_INPUTS;
-            if constexpr (TYPE == DENSE_FLOAT32) {
-                const float4_t low = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at);
-                const float4_t high = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at + 4u);
-#pragma unroll
-                for (uint32_t i = 0; i < 4u; i++) {
-                    weights[i] = low[i];
-                    weights[4u + i] = high[i];
-                }
-            } else {
-                unpack_bf16x8(*(const uint4_t *)((const uint16_t *)(arena + arguments.weights_offset) + at), weights);
-            }
 #pragma unroll
             for (uint32_t r = 0; r < ROWS; r++) {
 #pragma unroll
                 for (uint32_t i = 0; i < DENSE_CHUNK_INPUTS; i++) {
-                    chain[o][r] = __fmaf_rn(weights[i], values[r][i], chain[o][r]);
+                    chain[o][r] = __fmaf_rn(weights[o][i], values[r][i], chain[o][r]);
                 }
             }
         }
     }
     const uint32_t group = thread / DENSE_GROUP_LANES, lane = thread % DENSE_GROUP_LANES;
+    /* the exchanges of one distance for every chain before the next distance: each chain's additions are the
+     * definition's, and the exchanges of different chains are in flight together */
 #pragma unroll
-    for (uint32_t r = 0; r < ROWS; r++) {
+    for (uint32_t distance = DENSE_GROUP_LANES / 2u; distance != 0u; distance /= 2u) {
 #pragma unroll
-        for (uint32_t o = 0; o < OUTPUTS; o++) {
-            const float sum = dense_group_sum(chain[o][r]);
-            if (lane == 0u) {
-                group_sums[group][o][r] = sum;
+        for (uint32_t r = 0; r < ROWS; r++) {
+#pragma unroll
+            for (uint32_t o = 0; o < OUTPUTS; o++) {
+                chain[o][r] = __fadd_rn(chain[o][r], __shfl_xor(chain[o][r], (int)distance, (int)DENSE_GROUP_LANES));
+            }
+            if (scaled) {
+                squares[r] = __fadd_rn(squares[r], __shfl_xor(squares[r], (int)distance, (int)DENSE_GROUP_LANES));
             }
         }
-        if (scaled) {
-            const float sum = dense_group_sum(squares[r]);
-            if (lane == 0u) {
-                group_sums[group][OUTPUTS][r] = sum;
+    }
+    if (lane == 0u) {
+#pragma unroll
+        for (uint32_t r = 0; r < ROWS; r++) {
+#pragma unroll
+            for (uint32_t o = 0; o < OUTPUTS; o++) {
+                group_sums[group][o][r] = chain[o][r];
+            }
+            if (scaled) {
+                group_sums[group][OUTPUTS][r] = squares[r];
             }
         }
     }
