@@ -69,6 +69,8 @@ __device__ static __forceinline__ void join_post_values(const float (&output)[HY
     }
 }
 
+#define JOIN_SLOTS_IN_FLIGHT 8u
+
 /* The join of eight values of a row: pairs their load of the row's first pair output, a slot `stride` loads on;
  * shared_output the shared expert's output there; row_sums where their float32 sums go, or nullptr. */
 __device__ static __forceinline__ void join_values(const uint4_t *pairs, uint32_t pairs_per_row, const float (&shared_output)[HYPER_VALUES_PER_THREAD],
@@ -79,8 +81,26 @@ __device__ static __forceinline__ void join_values(const uint4_t *pairs, uint32_
     for (uint32_t v = 0; v < HYPER_VALUES_PER_THREAD; v++) {
         routed[v] = 0.0f;
     }
-#pragma unroll 8
-    for (uint32_t slot = 0; slot < pairs_per_row; slot++) {
+    /* eight slots at a time, their loads all asked for before the first is added: one trip to memory for the eight, the
+     * additions in slot order as before */
+    uint32_t slot = 0;
+    for (; slot + JOIN_SLOTS_IN_FLIGHT <= pairs_per_row; slot += JOIN_SLOTS_IN_FLIGHT) {
+        uint4_t loaded[JOIN_SLOTS_IN_FLIGHT];
+#pragma unroll
+        for (uint32_t s = 0; s < JOIN_SLOTS_IN_FLIGHT; s++) {
+            loaded[s] = pairs[(uint64_t)(slot + s) * stride];
+        }
+#pragma unroll
+        for (uint32_t s = 0; s < JOIN_SLOTS_IN_FLIGHT; s++) {
+            float pair[HYPER_VALUES_PER_THREAD];
+            join_unpack(loaded[s], pair);
+#pragma unroll
+            for (uint32_t v = 0; v < HYPER_VALUES_PER_THREAD; v++) {
+                routed[v] = __fadd_rn(routed[v], pair[v]);
+            }
+        }
+    }
+    for (; slot < pairs_per_row; slot++) {
         float pair[HYPER_VALUES_PER_THREAD];
         join_unpack(pairs[(uint64_t)slot * stride], pair);
 #pragma unroll
