@@ -3,20 +3,23 @@
  * the router's job table: five launches (operands, gate/up products, activation, down products, combine), the
  * counterpart of the reference's tensor-core MoE (source/kernel_exl3_tc.cu, include/anemone/exl3_tc_records.h).
  *
- * The arithmetic is the chain's (kernel_exl3.hip): fp16 operands from a float32 Hadamard transform, exactly decoded
- * fp16 weights, float32 MFMA sums, SwiGLU in float32, the weighted pair outputs added in slot order. What differs is
- * the work mapping: every (job, matrix, strip of eight output tiles, K slice) is an independent wavefront item that
- * streams its bytes once; K-slice partial sums are kept apart in the workspace and added in slice order by the next
+ * The arithmetic is the chain's (kernel_exl3.hip): fp16 operands from a float32 Hadamard transform, the codebook's
+ * weights (see EXACT_WEIGHTS), float32 MFMA sums, SwiGLU in float32, the weighted pair outputs added in slot order. What
+ * differs is the work mapping: every (job, matrix, strip of eight output tiles, K slice) is an independent wavefront item
+ * that streams its bytes once, from memory straight into the registers of the lanes that decode them; K-slice partial sums are kept apart in the workspace and added in slice order by the next
  * launch, so a result does not depend on scheduling, on the other rows of the step or on the grid.
  *
  * Workspace (exl3_tc_workspace_bytes): fp16 operands [2][pairs][hidden], reused as [pairs][intermediate] for the
  * down operands; float32 gate/up partials [GATE_UP_SLICES][2][pairs][intermediate]; float32 down partials
  * [DOWN_SLICES][pairs][hidden].
  */
-#include "exl3_device.cuh"
+#include "exl3_stream_device.cuh"
 #include "kernel_registry.h"
 
-#define STRIP_TILES 8u
+#define STRIP_PAIRS (EXL3_TC_STRIP_OUTPUTS / 32u) /* a strip: pairs of adjacent output tiles */
+/* false: the matrix instruction takes the codebook values before their scale and bias (1024 + b), which enter once a
+ * sum; the weights' own rounding to fp16 is then left out of the product (within the products' stated tolerance) */
+#define EXACT_WEIGHTS true
 #define PRODUCT_WAVES 4u
 #define PRODUCT_THREADS (PRODUCT_WAVES * WAVE)
 
@@ -71,42 +74,46 @@ extern "C" __global__ void exl3_tc_operands(struct exl3_tc_record record, unsign
 }
 ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_operands, exl3_tc_record);
 
-/* one wavefront item: a strip of eight output tiles by one K slice of one matrix of one job */
+/* one wavefront item: a strip of EXL3_TC_STRIP_OUTPUTS outputs by one K slice of one matrix of one job */
 template <uint32_t bits_x2>
 __device__ static __forceinline__ void tc_item(const uint32_t *codes, uint32_t inputs, uint32_t outputs,
                                                uint32_t strip, uint32_t slice, uint32_t slices,
                                                const struct expert_job_record *job, const half_t *operands,
-                                               float *partials, uint32_t *lds, uint32_t lane)
+                                               float *partials, uint32_t lane)
 {
     const uint32_t column = lane % 16u;
     const bool live = column < job->row_count;
-    const uint32_t pair = live ? job->pair_index[column] : 0u;
-    const half_t *operand = live ? operands + (uint64_t)pair * inputs : nullptr;
+    /* a column that is not live reads the first column's operand: its sums are not stored */
+    const uint32_t pair = job->pair_index[live ? column : 0u];
     const uint32_t tiles = inputs / EXL3_TILE;
-    float4_t accumulator[STRIP_TILES];
-    exl3_wave_product<bits_x2, STRIP_TILES>(codes, outputs / EXL3_TILE, strip * STRIP_TILES, tiles * slice / slices,
-                                            tiles * (slice + 1u) / slices, operand, lds, lane, accumulator);
+    float4_t accumulator[STRIP_PAIRS][2];
+    exl3_stream_product<bits_x2, STRIP_PAIRS, EXACT_WEIGHTS>(codes, outputs / EXL3_TILE, strip * 2u * STRIP_PAIRS, tiles * slice / slices,
+                                                             tiles * (slice + 1u) / slices, operands + (uint64_t)pair * inputs, lane,
+                                                             accumulator);
     if (live) {
-        float *out = partials + (uint64_t)pair * outputs + strip * (STRIP_TILES * EXL3_TILE) + 4u * (lane / 16u);
+        float *out = partials + (uint64_t)pair * outputs;
 #pragma unroll
-        for (uint32_t n = 0; n < STRIP_TILES; n++) {
-            *(float4_t *)(out + n * EXL3_TILE) = accumulator[n];
+        for (uint32_t p = 0; p < STRIP_PAIRS; p++) {
+#pragma unroll
+            for (uint32_t h = 0; h < 2u; h++) {
+                *(float4_t *)(out + exl3_stream_output(strip * 2u * STRIP_PAIRS, p, h, lane)) = accumulator[p][h];
+            }
         }
     }
 }
 
-/* launches 1 and 3: grid (outputs / 128, job_capacity, matrices * slices / 4), block 256: the block's four
- * wavefronts take four consecutive (matrix, slice) items of one strip. pass 0: gate and up; pass 1: down. */
-extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS)
+/* launches 1 and 3: grid (outputs / EXL3_TC_STRIP_OUTPUTS, job_capacity, matrices * slices / 4), block 256: the block's four
+ * wavefronts take four consecutive (matrix, slice) items of one strip. pass 0: gate and up; pass 1: down. A slice is
+ * a whole number of steps of four K tiles. */
+extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS, 4)
     exl3_tc_products(struct exl3_tc_record record, unsigned char *arena)
 {
-    __shared__ __attribute__((aligned(16))) uint32_t staging[PRODUCT_WAVES * 2u * STRIP_TILES * exl3_width<8>::tile_words];
     const struct expert_job_record *job = (const struct expert_job_record *)(arena + record.jobs_offset) + blockIdx.y;
     if (job->row_count == 0u) {
         return;
     }
     const tc_shape shape = tc_shape_of(record);
-    const uint32_t lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const bool down = record.pass != 0u;
     const uint32_t slices = down ? EXL3_TC_DOWN_SLICES : EXL3_TC_GATE_UP_SLICES;
     const uint32_t item = blockIdx.z * PRODUCT_WAVES + wave; /* projection * slices + slice */
@@ -126,13 +133,12 @@ extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS)
         partials = (float *)(workspace + exl3_tc_operand_bytes(shape.pairs, shape.hidden)) +
                    ((uint64_t)slice * 2u + projection) * shape.pairs * outputs;
     }
-    uint32_t *lds = staging + wave * (2u * STRIP_TILES * exl3_width<8>::tile_words);
     const uint32_t *codes = (const uint32_t *)(arena + matrix);
     switch (bits_x2) {
-    case 4u: tc_item<4u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
-    case 5u: tc_item<5u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
-    case 6u: tc_item<6u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
-    case 8u: tc_item<8u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lds, lane); break;
+    case 4u: tc_item<4u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
+    case 5u: tc_item<5u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
+    case 6u: tc_item<6u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
+    case 8u: tc_item<8u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
     default: break;
     }
 }

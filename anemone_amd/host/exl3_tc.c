@@ -5,12 +5,12 @@
  *
  *   launch      kernel              grid                                            block
  *   operands    exl3_tc_operands    (hidden / 128, job_capacity, 2)                 64
- *   gate/up     exl3_tc_products    (intermediate / 128, job_capacity, 2 S_gu / 4)  256   pass 0
+ *   gate/up     exl3_tc_products    (intermediate / 64, job_capacity, 2 S_gu / 4)   256   pass 0
  *   activate    exl3_tc_activate    (intermediate / 128, job_capacity, 1)           64
- *   down        exl3_tc_products    (hidden / 128, job_capacity, S_d / 4)           256   pass 1
+ *   down        exl3_tc_products    (hidden / 64, job_capacity, S_d / 4)            256   pass 1
  *   combine     exl3_tc_combine     (hidden / 128, row_count, 1)                    64
- * S_gu = EXL3_TC_GATE_UP_SLICES and S_d = EXL3_TC_DOWN_SLICES K slices; every slice is a whole number of MFMA steps
- * (32 inputs), which bounds the shapes: hidden a multiple of 32 S_gu, intermediate of 32 S_d, both of 128.
+ * S_gu = EXL3_TC_GATE_UP_SLICES and S_d = EXL3_TC_DOWN_SLICES K slices; every slice is a whole number of steps of four
+ * K tiles (64 inputs), which bounds the shapes: hidden a multiple of 64 S_gu, intermediate of 64 S_d, both of 128.
  */
 #include <math.h>
 #include <string.h>
@@ -49,10 +49,10 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
         REFUSE("%s: expert rotation is a tensor-parallel form this library does not build", what);
         return STATUS_UNSUPPORTED;
     }
-    if (I == 0 || I % EXL3_TRANSFORM != 0 || hidden % EXL3_TRANSFORM != 0 || hidden % (32u * EXL3_TC_GATE_UP_SLICES) != 0 ||
-        I % (32u * EXL3_TC_DOWN_SLICES) != 0 || I > hidden) {
+    if (I == 0 || I % EXL3_TRANSFORM != 0 || hidden % EXL3_TRANSFORM != 0 || hidden % (64u * EXL3_TC_GATE_UP_SLICES) != 0 ||
+        I % (64u * EXL3_TC_DOWN_SLICES) != 0 || I > hidden) {
         REFUSE("%s: hidden %u and intermediate %u: multiples of 128, of %u and of %u", what, hidden, I,
-               32u * EXL3_TC_GATE_UP_SLICES, 32u * EXL3_TC_DOWN_SLICES);
+               64u * EXL3_TC_GATE_UP_SLICES, 64u * EXL3_TC_DOWN_SLICES);
         return STATUS_UNSUPPORTED;
     }
     const bool mixed = record->widths_offset != 0;
@@ -81,7 +81,7 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
     }
     static const char *const names[EXL3_TC_LAUNCHES] = {"exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate",
                                                         "exl3_tc_products", "exl3_tc_combine"};
-    const uint32_t grid_x[EXL3_TC_LAUNCHES] = {hidden / 128u, I / 128u, I / 128u, hidden / 128u, hidden / 128u};
+    const uint32_t grid_x[EXL3_TC_LAUNCHES] = {hidden / 128u, I / EXL3_TC_STRIP_OUTPUTS, I / 128u, hidden / EXL3_TC_STRIP_OUTPUTS, hidden / 128u};
     const uint32_t grid_y[EXL3_TC_LAUNCHES] = {record->job_capacity, record->job_capacity, record->job_capacity,
                                                record->job_capacity, record->row_count};
     const uint32_t grid_z[EXL3_TC_LAUNCHES] = {2u, 2u * EXL3_TC_GATE_UP_SLICES / PRODUCT_WAVES, 1u,

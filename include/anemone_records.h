@@ -286,6 +286,7 @@ ANEMONE_RECORD_HAS(expert_row_sum_arguments, 24);
 #define EXL3_TC_DEFAULT_PAIRS_PER_ROW 6u
 #define EXL3_TC_GATE_UP_SLICES 8u /* K slices of a gate/up product: partial sums kept apart, added in order */
 #define EXL3_TC_DOWN_SLICES 4u
+#define EXL3_TC_STRIP_OUTPUTS 64u /* outputs of one wavefront item of the products launches */
 
 struct exl3_tc_record {
     uint64_t jobs_offset;      /* read: struct expert_job_record [job_capacity], empty ones anywhere */
