@@ -85,10 +85,10 @@ __device__ static __forceinline__ void tc_item(const uint32_t *codes, uint32_t i
     const bool live = column < job->row_count;
     /* a column that is not live reads the first column's operand: its sums are not stored */
     const uint32_t pair = job->pair_index[live ? column : 0u];
-    const uint32_t tiles = inputs / EXL3_TILE;
+    const uint32_t steps = inputs / (4u * EXL3_TILE); /* a slice is a whole number of steps of four K tiles */
     float4_t accumulator[STRIP_PAIRS][2];
-    exl3_stream_product<bits_x2, STRIP_PAIRS, EXACT_WEIGHTS>(codes, outputs / EXL3_TILE, strip * 2u * STRIP_PAIRS, tiles * slice / slices,
-                                                             tiles * (slice + 1u) / slices, operands + (uint64_t)pair * inputs, lane,
+    exl3_stream_product<bits_x2, STRIP_PAIRS, EXACT_WEIGHTS>(codes, outputs / EXL3_TILE, strip * 2u * STRIP_PAIRS, 4u * (steps * slice / slices),
+                                                             4u * (steps * (slice + 1u) / slices), operands + (uint64_t)pair * inputs, lane,
                                                              accumulator);
     if (live) {
         float *out = partials + (uint64_t)pair * outputs;

@@ -10,7 +10,7 @@
  *   down        exl3_tc_products    (hidden / 64, job_capacity, S_d / 4)            256   pass 1
  *   combine     exl3_tc_combine     (hidden / 128, row_count, 1)                    64
  * S_gu = EXL3_TC_GATE_UP_SLICES and S_d = EXL3_TC_DOWN_SLICES K slices; every slice is a whole number of steps of four
- * K tiles (64 inputs), which bounds the shapes: hidden a multiple of 64 S_gu, intermediate of 64 S_d, both of 128.
+ * K tiles (64 inputs): slice s takes the steps [steps s / S, steps (s + 1) / S). Hidden and intermediate: multiples of 128.
  */
 #include <math.h>
 #include <string.h>
@@ -49,10 +49,8 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
         REFUSE("%s: expert rotation is a tensor-parallel form this library does not build", what);
         return STATUS_UNSUPPORTED;
     }
-    if (I == 0 || I % EXL3_TRANSFORM != 0 || hidden % EXL3_TRANSFORM != 0 || hidden % (64u * EXL3_TC_GATE_UP_SLICES) != 0 ||
-        I % (64u * EXL3_TC_DOWN_SLICES) != 0 || I > hidden) {
-        REFUSE("%s: hidden %u and intermediate %u: multiples of 128, of %u and of %u", what, hidden, I,
-               64u * EXL3_TC_GATE_UP_SLICES, 64u * EXL3_TC_DOWN_SLICES);
+    if (I == 0 || I % EXL3_TRANSFORM != 0 || hidden % EXL3_TRANSFORM != 0 || I > hidden) {
+        REFUSE("%s: hidden %u and intermediate %u: multiples of 128, the intermediate size at most the hidden", what, hidden, I);
         return STATUS_UNSUPPORTED;
     }
     const bool mixed = record->widths_offset != 0;

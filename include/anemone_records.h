@@ -284,7 +284,7 @@ ANEMONE_RECORD_HAS(expert_row_sum_arguments, 24);
 #define EXL3_TC_MOST_ROWS 64u
 #define EXL3_TC_DEFAULT_HIDDEN 5120u
 #define EXL3_TC_DEFAULT_PAIRS_PER_ROW 6u
-#define EXL3_TC_GATE_UP_SLICES 8u /* K slices of a gate/up product: partial sums kept apart, added in order */
+#define EXL3_TC_GATE_UP_SLICES 4u /* K slices of a gate/up product: partial sums kept apart, added in order */
 #define EXL3_TC_DOWN_SLICES 4u
 #define EXL3_TC_STRIP_OUTPUTS 64u /* outputs of one wavefront item of the products launches */
 

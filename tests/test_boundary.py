@@ -176,7 +176,7 @@ def test_tc_prepare_geometry_and_refusals(fake):
     assert lib.exl3_tc_prepare(C.byref(tc_record()), ARENA, fake.address, fake.card, launches) == 0
     assert [fake.handles[l.kernel][1] for l in launches] == ["exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate",
                                                             "exl3_tc_products", "exl3_tc_combine"]
-    assert [list(l.grid) for l in launches] == [[32, 64, 2], [32, 64, 4], [16, 64, 1], [64, 64, 1], [32, 8, 1]]
+    assert [list(l.grid) for l in launches] == [[32, 64, 2], [32, 64, 2], [16, 64, 1], [64, 64, 1], [32, 8, 1]]
     passes = [amd.Exl3TcRecord.from_buffer_copy(bytes(l.argument)[:88]).pass_ for l in launches]
     assert passes == [0, 0, 0, 1, 0]
     assert amd.exl3_tc_workspace_bytes(64, 4096, 2048) == 64 * 4096 * 4 + 8 * 2 * 64 * 2048 * 4 + 4 * 64 * 4096 * 4
