@@ -38,31 +38,42 @@ MEASURED_TRAFFIC_BYTES = {
     ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,
     ("fp8_prefill_block128", 2048): 5386.8e6 + 67.2e6,
 }
+TRAFFIC_SOURCE = {
+    "exl3_decode": "profiles/exl3_tc_products_decode8.md", "fp4_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md",
+    "fp8_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md", "fp4_prefill": "profiles/wide_expert_fp4_fp8_prefill.md",
+    "fp8_prefill": "profiles/wide_expert_fp4_fp8_prefill.md",
+    "fp8_decode_block128": "profiles/expert_b128_fp8_block128_decode64_prefill2048.md",
+    "fp8_prefill_block128": "profiles/expert_b128_fp8_block128_decode64_prefill2048.md",
+}
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
 CONFIG = 1
 
 
-def cpu_oracle_step(orc_module, layer, x, router, matrices, widths, threads):
-    """The same step on the host cores by the CPU oracle: routing, then the experts. Returns (seconds, output)."""
+def cpu_oracle_step(orc_module, x, router, matrices, widths, threads):
+    """The same step on the host cores by the CPU oracle: routing (one C call), then the experts (one C call). Returns
+    (seconds, output, experts)."""
     import ctypes as C
     o = orc_module
     orc, ptr = o.orc, o.ptr
-    start = time.perf_counter()
-    scores = np.zeros((ROWS, EXPERTS), dtype=np.float32)
-    orc.orc_router_projection(ptr(x, o.u16p), ptr(router, o.u16p), ROWS, HIDDEN, EXPERTS, ptr(scores, o.f32p))
-    affinities = np.array([[orc.orc_router_affinity(float(s), 1) for s in row] for row in scores], dtype=np.float32)
     experts = np.zeros((ROWS, PICKS), dtype=np.uint32)
     weights = np.zeros((ROWS, PICKS), dtype=np.float32)
     bias = np.zeros(EXPERTS, dtype=np.float32)
-    for r in range(ROWS):
-        orc.orc_router_select(ptr(affinities[r], o.f32p), ptr(bias, o.f32p), EXPERTS, PICKS, 0, 1.5,
-                              ptr(experts[r], o.u32p), ptr(weights[r], o.f32p))
     pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
     out = np.zeros((ROWS, HIDDEN), dtype=np.float32)
     widths8 = np.ascontiguousarray(widths.astype(np.uint8))
+    start = time.perf_counter()
+    orc.orc_router_route(ptr(x, o.u16p), ptr(router, o.u16p), ptr(bias, o.f32p), ROWS, HIDDEN, EXPERTS, PICKS, 1, 0, 1.5, None,
+                         ptr(experts, o.u32p), ptr(weights, o.f32p))
     orc.orc_exl3_moe_layer(ptr(x, o.u16p), ROWS, HIDDEN, INNER, PICKS, ptr(experts, o.u32p), ptr(weights, o.f32p), EXPERTS,
                            pointers, ptr(widths8, o.u8p), 10.0, ptr(out, o.f32p), None, None, threads)
     return time.perf_counter() - start, out, experts
+
+
+def median_seconds(run, warmup, count):
+    """`run()` returns seconds: `warmup` calls unrecorded, then the median of `count`."""
+    for _ in range(warmup):
+        run()
+    return float(np.median([run() for _ in range(count)]))
 
 
 def queue_steps(card, step, count, graph):
@@ -205,9 +216,9 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         "value": rows * arguments.steps / seconds, "unit": "tok/s", "n_gpus": 1, "steps": arguments.steps,
         "warmup": arguments.warmup, "ms_per_step": 1000.0 * seconds / arguments.steps, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "fp8 x fp8 -> f32" if fp8 else "fp4 x fp8 -> f32", "data": "synthetic",
-        "config": {"workload": "%s_moe_decode: %d tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router, %s"
-                               % ("fp8" if fp8 else "fp4", rows, "E4M3 weights with E8M0 scales per 32 x 32" if fp8 else
-                                  "E2M1 weights with E8M0 scales per 32"),
+        "config": {"workload": "%s_moe_decode: %d tokens, H 4096, 256 experts x I 2048, top-8, %s"
+                               % ("fp8" if fp8 else "fp4", rows, "E4M3, f32 scales per 128x128 / per 128" if block128 else
+                                  "E4M3, E8M0 scales per 32x32" if fp8 else "E2M1, E8M0 scales per 32"),
                    "distinct_experts": int(len(distinct)), "jobs": int(len(live)),
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "down_GBps": matrix_bytes * len(distinct) / (down_us * 1e-6) / 1e9},
@@ -240,6 +251,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         key = (key[0] + "_block128", rows)
     if key in MEASURED_TRAFFIC_BYTES and (prefill or (arguments.gate_up_slices, arguments.down_slices) == (4, 2)):
         result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES[key]
+        result["roofline"]["traffic_source"] = TRAFFIC_SOURCE[key[0]] + " (counter bytes of the profiled run, not of this one)"
     if prefill:
         pairs = rows * PICKS
         gate_up_flops, down_flops = 2.0 * pairs * 2 * HIDDEN * INNER, 2.0 * pairs * HIDDEN * INNER
@@ -337,11 +349,46 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                                   "sample": "the first %d tokens of the same step by the CPU oracle" % sample,
                                   "seconds": cpu_seconds, "gpu_vs_oracle_rms_err": error}
     card.close()
-    print(json.dumps(result))
+    return result
 
 
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_F8_PEAK_TFLOPS = 5000.0
+
+
+def zipf_capped_load(rows, picks, experts, s):
+    """Pairs an expert of rank 0, 1, ... takes when the picks of `rows` tokens follow Zipf(s) over the experts and no
+    token picks an expert twice: rows . picks . pmf, the experts above `rows` held at `rows` and the rest scaled up."""
+    pmf = (1.0 + np.arange(experts)) ** -s
+    pmf /= pmf.sum()
+    load, capped = np.zeros(experts), np.zeros(experts, dtype=bool)
+    for _ in range(experts):
+        free = rows * picks - rows * capped.sum()
+        load = np.where(capped, rows, free * pmf / pmf[~capped].sum())
+        over = (load > rows) & ~capped
+        if not over.any():
+            break
+        capped |= over
+    return load
+
+
+def zipf_fitted_bias(workloads, x, router, ranks, target):
+    """The router's bias under which the sigmoid router's top-k loads follow `target` (by rank): ln(target share) to begin
+    with, then each expert's bias moved by the logarithm of target over realised load until the loads agree (computed
+    here on the host from float32 scores: the bias is an input of the step, the loads the card realises are reported
+    beside the target)."""
+    scores = workloads.bf16_to_f32(x).astype(np.float32) @ workloads.bf16_to_f32(router).astype(np.float32).T
+    affinities = 1.0 / (1.0 + np.exp(-scores))
+    wanted = np.zeros(EXPERTS)
+    wanted[ranks] = target
+    bias = 0.05 * np.log(wanted / wanted.max())
+    for _ in range(200):
+        top = np.argpartition(-(affinities + bias[None, :]), PICKS - 1, axis=1)[:, :PICKS]
+        realised = np.bincount(top.reshape(-1), minlength=EXPERTS).astype(np.float64)
+        if np.abs(realised - wanted).sum() / wanted.sum() < 0.02:
+            break
+        bias += 0.02 * np.log(wanted / np.maximum(realised, 0.5))
+    return (bias - bias.max()).astype(np.float32)
 
 
 def exl3_prefill(amd, workloads, arguments):
@@ -354,9 +401,13 @@ def exl3_prefill(amd, workloads, arguments):
     widths, matrices, router = workloads.exl3_moe_layer(CONFIG, HIDDEN, INNER, EXPERTS)
     x = workloads.activations(2, rows, HIDDEN)
     ranks = np.argsort(workloads.uniform01(workloads.SEED + (2 << 20) + 7, EXPERTS))
-    bias = np.zeros(EXPERTS, dtype=np.float32)
-    pmf = (1.0 + np.arange(EXPERTS)) ** -1.1
-    bias[ranks] = (arguments.zipf_strength * np.log(pmf / pmf.max())).astype(np.float32)
+    target = zipf_capped_load(rows, PICKS, EXPERTS, 1.1)  # pairs of the expert of each rank
+    if arguments.zipf_strength > 0.0:
+        bias = np.zeros(EXPERTS, dtype=np.float32)
+        pmf = (1.0 + np.arange(EXPERTS)) ** -1.1
+        bias[ranks] = (arguments.zipf_strength * np.log(pmf / pmf.max())).astype(np.float32)
+    else:
+        bias = zipf_fitted_bias(workloads, x, router, ranks, target)
     card = amd.Card(10 << 30)
     layer = amd.Exl3Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, widths, router_weights_bf16=router, bias=bias,
                           affinity_kind=amd.AFFINITY_SIGMOID, route_scale=1.5, limit=10.0)
@@ -389,10 +440,13 @@ def exl3_prefill(amd, workloads, arguments):
         "value": rows * arguments.steps / seconds, "unit": "tok/s", "n_gpus": 1, "steps": arguments.steps,
         "warmup": arguments.warmup, "ms_per_step": 1000.0 * seconds / arguments.steps, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "exl3_moe_prefill: %d tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router "
-                               "with a Zipf (s = 1.1) bias of strength %.2f, EXL3 K in {2,3,4} per tensor (%.2f bpw)"
-                               % (rows, arguments.zipf_strength, float(np.mean(widths))),
+        "config": {"workload": "exl3_moe_prefill: %d tokens, H 4096, 256 experts x I 2048, top-8, Zipf(1.1) loads (%s), %.2f bpw"
+                               % (rows, "fitted bias" if arguments.zipf_strength <= 0.0 else
+                                  "bias %.2f ln pmf" % arguments.zipf_strength, float(np.mean(widths))),
                    "pairs_of_the_busiest_expert": int(counts.max()), "experts_without_a_pair": int((counts == 0).sum()),
+                   "zipf_target_pairs_by_rank": [int(round(v)) for v in target[[0, 1, 3, 15, 63, 255]]],
+                   "realised_pairs_at_those_ranks": [int(counts[ranks[r]]) for r in (0, 1, 3, 15, 63, 255)],
+                   "load_fit_total_variation": float(np.abs(counts[ranks] - target).sum() / (2.0 * target.sum())),
                    "chunks": int(((counts + chunk - 1) // chunk).sum()),
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "down_TFLOPs": down_flops / (down_us * 1e-6) / 1e12,
@@ -424,51 +478,11 @@ def exl3_prefill(amd, workloads, arguments):
                                   "sample": "the first %d tokens of the same call by the CPU oracle, double-precision sums" % sample,
                                   "seconds": cpu_seconds, "gpu_vs_oracle_max_err_over_rms": error}
     card.close()
-    print(json.dumps(result))
+    return result
 
 
-def main():
-    parser = argparse.ArgumentParser()
-    parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=200)
-    parser.add_argument("--warmup", type=int, default=20)
-    parser.add_argument("--workload", default="exl3_decode")
-    parser.add_argument("--zipf-strength", type=float, default=0.05,
-                        help="exl3_prefill: the router's bias is this times ln(Zipf pmf): 0.05 gives loads close to Zipf (s = 1.1) "
-                             "under sigmoid affinities with no idle expert; 0.2 leaves three quarters of the experts idle")
-    parser.add_argument("--rows", type=int, default=32, help="tokens of a step (fp4_decode)")
-    parser.add_argument("--gate-up-slices", type=int, default=4)
-    parser.add_argument("--down-slices", type=int, default=2)
-    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    parser.add_argument("--block128", action="store_true",
-                        help="fp8 workloads: float32 scales of 128 x 128 weight blocks and of 128 activation values in place of the reference's E8M0 scales")
-    parser.add_argument("--site", action="store_true",
-                        help="fp4/fp8 workloads: the whole FFN site: the mix project and mix finish ahead of the router, the shared expert and the join "
-                             "in place of the row sum")
-    parser.add_argument("--graph", action="store_true", help="time replays of the step captured as one graph (graph_capture / graph_run)")
-    parser.add_argument("--calibrate", action="store_true",
-                        help="run only a 1 GiB arena copy, five times: the yardstick of the traffic counters")
-    arguments = parser.parse_args()
-    if arguments.gpus != 1:
-        print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
-        sys.exit(2)
-    if arguments.workload not in ("exl3_decode", "fp4_decode", "fp8_decode", "exl3_prefill", "fp4_prefill", "fp8_prefill"):
-        print("unknown workload %s" % arguments.workload, file=sys.stderr)
-        sys.exit(2)
-
-    import anemone_amd as amd
-    from anemone_amd import workloads
-
-    if arguments.calibrate:
-        calibrate(amd)
-        return
-    if arguments.workload == "exl3_prefill":
-        exl3_prefill(amd, workloads, arguments)
-        return
-    if arguments.workload in ("fp4_decode", "fp8_decode", "fp4_prefill", "fp8_prefill"):
-        fp4_decode(amd, workloads, arguments, fp8=arguments.workload.startswith("fp8"), prefill=arguments.workload.endswith("prefill"))
-        return
-
+def exl3_decode(amd, workloads, arguments):
+    """The workload the metric is quoted on (see the head of this file)."""
     widths, matrices, router = workloads.exl3_moe_layer(CONFIG, HIDDEN, INNER, EXPERTS)
     x = workloads.activations(CONFIG, ROWS, HIDDEN)
     card = amd.Card(4 << 30)
@@ -508,6 +522,7 @@ def main():
     down_bytes = sum(workloads.exl3_matrix_bytes(INNER, HIDDEN, int(widths[e, 2])) for e in distinct)
     step_bytes = gate_up_bytes + down_bytes + ROWS * HIDDEN * 2 + ROWS * HIDDEN * 4
     gate_up_us = float(per_launch[names.index("exl3_tc_products(gate/up)")])
+    down_us = float(per_launch[names.index("exl3_tc_products(down)")])
     achieved = gate_up_bytes / (gate_up_us * 1e-6) / 1e9
 
     result = {
@@ -523,15 +538,18 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": "exl3_moe_decode: 8 tokens, hidden 4096, 256 experts x intermediate 2048, top-8 sigmoid router, "
-                               "EXL3 K in {2,3,4} per tensor (%.2f bpw)" % float(np.mean(widths)),
+        "config": {"workload": "exl3_moe_decode: 8 tokens, H 4096, 256 experts x I 2048, top-8 sigmoid router, EXL3 K in {2,3,4} (%.2f bpw)"
+                               % float(np.mean(widths)),
                    "distinct_experts": int(len(distinct)), "step_algorithmic_bytes": int(step_bytes),
                    "step_GBps": step_bytes / seconds * arguments.steps / 1e9,
                    "host_clock_ms_per_step": 1000.0 * host_seconds / arguments.steps,
-                   "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)}},
+                   "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
+                   "down_pass": {"launch_us": down_us, "algorithmic_bytes": int(down_bytes),
+                                 "frac_of_hbm_peak": down_bytes / (down_us * 1e-6) / 1e9 / HBM_PEAK_GBS}},
         "roofline": {"bound": "hbm", "kernel": "exl3_tc_products (gate/up pass)", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES[("exl3_decode", ROWS)],
+                     "traffic_source": TRAFFIC_SOURCE["exl3_decode"] + " (counter bytes of the profiled run, not of this one)",
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
     }
 
@@ -539,16 +557,110 @@ def main():
     if not arguments.no_cpu:
         import _oracle
         threads = min(os.cpu_count() or 1, 16)
-        cpu_seconds, want, experts = cpu_oracle_step(_oracle, layer, x, router, matrices, widths, threads)
+        outputs = []
+
+        def one_step():
+            cpu_seconds, want, experts = cpu_oracle_step(_oracle, x, router, matrices, widths, threads)
+            outputs[:] = [want, experts]
+            return cpu_seconds
+        cpu_seconds = median_seconds(one_step, 1, 5)  # every step reads the experts' 0.55 GB anew: cold to the host's caches
+        want, experts = outputs
         rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
         error = float(np.max(np.abs(got - want))) / rms
         assert sorted(set(experts.reshape(-1).tolist())) == sorted(distinct.tolist()), "expert ids differ from the oracle's"
         assert error <= 4e-3, "GPU output differs from the oracle's: %g of rms" % error
         result["cpu_baseline"] = {"value": ROWS / cpu_seconds, "unit": "tok/s", "cores": threads, "kind": "port",
-                                  "sample": "1 step of the same workload (8 tokens, %d experts) by the CPU oracle, "
-                                            "double-precision sums" % len(distinct),
+                                  "sample": "the same step (8 tokens, %d experts) by the CPU oracle (routing and experts, two C calls; "
+                                            "double-precision sums): 1 warm-up, median of 5" % len(distinct),
                                   "seconds": cpu_seconds, "gpu_vs_oracle_max_err_over_rms": error}
     card.close()
+    return result
+
+
+def summary(result):
+    """What the default line keeps of a secondary workload."""
+    roofline, config = result["roofline"], result["config"]
+    keep = {"workload": config["workload"], "ms_per_step": result["ms_per_step"], "tok_s": result["value"], "steps": result["steps"],
+            "kernel": roofline["kernel"], "launch_us": roofline["launch_us"], "bound": roofline["bound"], "achieved": roofline["achieved"],
+            "peak": roofline["peak"], "unit": roofline["unit"], "frac": roofline["frac"]}
+    for name in ("algorithmic_bytes_per_launch", "algorithmic_flops_per_launch", "TFLOPs", "flop_per_byte"):
+        if name in roofline:
+            keep[name] = roofline[name]
+    for name in ("pairs_of_the_busiest_expert", "load_fit_total_variation", "chunks", "distinct_experts", "down_TFLOPs", "down_GBps"):
+        if name in config:
+            keep[name] = config[name]
+    baseline = result.get("cpu_baseline", {})
+    for name in ("gpu_vs_oracle_max_err_over_rms", "gpu_vs_oracle_rms_err"):
+        if name in baseline:
+            keep[name] = baseline[name]
+    return keep
+
+
+# the workloads of the other configurations the metric names, as the default run's config.also: (workload, rows, block128)
+ALSO = [("exl3_prefill", 4096, False), ("fp8_decode", 1, True), ("fp8_decode", 64, True), ("fp8_prefill", 2048, True),
+        ("fp8_prefill", 2048, False), ("fp4_prefill", 8192, False), ("fp4_decode", 32, False)]
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=20)
+    parser.add_argument("--workload", default="all",
+                        help="all (default): exl3_decode as the line, the other configurations' workloads in config.also; or one of "
+                             "exl3_decode, exl3_prefill, fp4_decode, fp8_decode, fp4_prefill, fp8_prefill")
+    parser.add_argument("--zipf-strength", type=float, default=0.0,
+                        help="exl3_prefill: 0 (default): the router's bias is fitted so that the experts' loads follow Zipf (s = 1.1), an "
+                             "expert at most one pair a token; above 0: the bias is this times ln(Zipf pmf)")
+    parser.add_argument("--rows", type=int, default=32, help="tokens of a step (fp4_decode)")
+    parser.add_argument("--gate-up-slices", type=int, default=4)
+    parser.add_argument("--down-slices", type=int, default=2)
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--block128", action="store_true",
+                        help="fp8 workloads: float32 scales of 128 x 128 weight blocks and of 128 activation values in place of the reference's E8M0 scales")
+    parser.add_argument("--site", action="store_true",
+                        help="fp4/fp8 workloads: the whole FFN site: the mix project and mix finish ahead of the router, the shared expert and the join "
+                             "in place of the row sum")
+    parser.add_argument("--graph", action="store_true", help="time replays of the step captured as one graph (graph_capture / graph_run)")
+    parser.add_argument("--calibrate", action="store_true",
+                        help="run only a 1 GiB arena copy, five times: the yardstick of the traffic counters")
+    arguments = parser.parse_args()
+    if arguments.gpus != 1:
+        print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
+        sys.exit(2)
+    if arguments.workload not in ("all", "exl3_decode", "fp4_decode", "fp8_decode", "exl3_prefill", "fp4_prefill", "fp8_prefill"):
+        print("unknown workload %s" % arguments.workload, file=sys.stderr)
+        sys.exit(2)
+
+    import anemone_amd as amd
+    from anemone_amd import workloads
+
+    if arguments.calibrate:
+        calibrate(amd)
+        return
+
+    def run(workload, options):
+        if workload == "exl3_decode":
+            return exl3_decode(amd, workloads, options)
+        if workload == "exl3_prefill":
+            return exl3_prefill(amd, workloads, options)
+        return fp4_decode(amd, workloads, options, fp8=workload.startswith("fp8"), prefill=workload.endswith("prefill"))
+
+    if arguments.workload != "all":
+        print(json.dumps(run(arguments.workload, arguments)))
+        return
+    result = run("exl3_decode", arguments)
+    also = []
+    for workload, rows, block128 in ALSO:
+        options = argparse.Namespace(**vars(arguments))
+        options.rows, options.block128, options.site, options.graph = rows, block128, False, False
+        prefill = workload.endswith("prefill")
+        options.steps, options.warmup = (min(arguments.steps, 5), min(arguments.warmup, 2)) if prefill else (min(arguments.steps, 20), min(arguments.warmup, 5))
+        start = time.perf_counter()
+        entry = summary(run(workload, options))
+        entry["bench_seconds"] = time.perf_counter() - start
+        also.append(entry)
+    result["config"]["also"] = also
     print(json.dumps(result))
 
 

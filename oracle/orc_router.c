@@ -230,3 +230,23 @@ void orc_router_wide_jobs(const uint32_t *experts, const float *weights, uint32_
         first_job += (taken + ORC_JOB_ROWS - 1u) / ORC_JOB_ROWS;
     }
 }
+
+/* the steps a card runs as router_projection and router_select_entry, all rows of a step */
+void orc_router_route(const uint16_t *x_bf16, const uint16_t *w_bf16, const float *bias, uint32_t rows, uint32_t hidden,
+                      uint32_t experts, uint32_t picks, int affinity_kind, int reference_order, float route_scale,
+                      float *affinities_out, uint32_t *experts_out, float *weights_out)
+{
+    float *scores = malloc((size_t)rows * experts * sizeof *scores);
+    orc_router_projection(x_bf16, w_bf16, rows, hidden, experts, scores);
+    for (size_t index = 0; index < (size_t)rows * experts; index++) {
+        scores[index] = orc_router_affinity(scores[index], affinity_kind);
+    }
+    for (uint32_t row = 0; row < rows; row++) {
+        orc_router_select(scores + (size_t)row * experts, bias, experts, picks, reference_order, route_scale,
+                          experts_out + (size_t)row * picks, weights_out + (size_t)row * picks);
+    }
+    if (affinities_out != NULL) {
+        memcpy(affinities_out, scores, (size_t)rows * experts * sizeof *scores);
+    }
+    free(scores);
+}

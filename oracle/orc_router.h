@@ -62,6 +62,12 @@ void orc_router_projection(const uint16_t *x_bf16, const uint16_t *w_bf16, uint3
 void orc_router_select(const float *affinities, const float *bias, uint32_t experts, uint32_t picks,
                        int reference_order, float route_scale, uint32_t *experts_out, float *weights_out);
 
+/* every row of a step in one call: projection, affinities (affinities_out [rows][experts], may be NULL) and the select
+ * of each row; experts_out / weights_out [rows][picks] */
+void orc_router_route(const uint16_t *x_bf16, const uint16_t *w_bf16, const float *bias, uint32_t rows, uint32_t hidden,
+                      uint32_t experts, uint32_t picks, int affinity_kind, int reference_order, float route_scale,
+                      float *affinities_out, uint32_t *experts_out, float *weights_out);
+
 /* the thin job table: row_count * picks entries, every byte written */
 void orc_router_jobs(const uint32_t *experts, const float *weights, uint32_t picks, uint32_t live_rows,
                      uint32_t row_count, uint32_t expert_count, const uint64_t *expert_offsets,

@@ -55,6 +55,7 @@ def _load_oracle():
         "orc_router_affinity": (f32, [f32, i32]),
         "orc_router_projection": (None, [u16p, u16p, u32, u32, u32, f32p]),
         "orc_router_select": (None, [f32p, f32p, u32, u32, i32, f32, u32p, f32p]),
+        "orc_router_route": (None, [u16p, u16p, f32p, u32, u32, u32, u32, i32, i32, f32, f32p, u32p, f32p]),
         "orc_router_jobs": (None, [u32p, f32p, u32, u32, u32, u32, u64p, vp]),
         "orc_router_wide_tile_count": (u32, [u32, u32, u32]),
         "orc_router_wide_job_count": (u32, [u32, u32, u32]),

@@ -225,3 +225,26 @@ def test_ref_affinity_select_jobs_and_sort():
         fn_jobs(ptr(experts, u32p), ptr(weights, f32p), *extra, 290, 300, *mid, ptr(offsets, u64p), jobs.ctypes.data)
         out.append((pairs[:290 * 6].tobytes(), runs.tobytes(), tiles.tobytes(), jobs.tobytes()))
     assert out[0] == out[1]
+
+
+def test_route_of_a_step_equals_the_calls_row_by_row():
+    """orc_router_route (projection, affinities and the select of every row in one call) against the functions it is made of."""
+    rng = np.random.default_rng(5)
+    rows, hidden, experts, picks = 5, 256, 64, 4
+    x = (rng.standard_normal((rows, hidden)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    w = ((rng.standard_normal((experts, hidden)) * 0.02).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    bias = (rng.standard_normal(experts) * 0.01).astype(np.float32)
+    for kind in (0, 1):
+        got_experts, got_weights = np.zeros((rows, picks), np.uint32), np.zeros((rows, picks), np.float32)
+        got_affinities = np.zeros((rows, experts), np.float32)
+        o.orc.orc_router_route(o.ptr(x, o.u16p), o.ptr(w, o.u16p), o.ptr(bias, o.f32p), rows, hidden, experts, picks, kind, 0, 1.5,
+                               o.ptr(got_affinities, o.f32p), o.ptr(got_experts, o.u32p), o.ptr(got_weights, o.f32p))
+        scores = np.zeros((rows, experts), np.float32)
+        o.orc.orc_router_projection(o.ptr(x, o.u16p), o.ptr(w, o.u16p), rows, hidden, experts, o.ptr(scores, o.f32p))
+        affinities = np.array([[o.orc.orc_router_affinity(float(s), kind) for s in row] for row in scores], np.float32)
+        want_experts, want_weights = np.zeros((rows, picks), np.uint32), np.zeros((rows, picks), np.float32)
+        for r in range(rows):
+            o.orc.orc_router_select(o.ptr(affinities[r], o.f32p), o.ptr(bias, o.f32p), experts, picks, 0, 1.5,
+                                    o.ptr(want_experts[r], o.u32p), o.ptr(want_weights[r], o.f32p))
+        assert got_affinities.tobytes() == affinities.tobytes()
+        assert np.array_equal(got_experts, want_experts) and got_weights.tobytes() == want_weights.tobytes()
