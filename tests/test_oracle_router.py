@@ -237,14 +237,14 @@ def test_route_of_a_step_equals_the_calls_row_by_row():
     for kind in (0, 1):
         got_experts, got_weights = np.zeros((rows, picks), np.uint32), np.zeros((rows, picks), np.float32)
         got_affinities = np.zeros((rows, experts), np.float32)
-        o.orc.orc_router_route(o.ptr(x, o.u16p), o.ptr(w, o.u16p), o.ptr(bias, o.f32p), rows, hidden, experts, picks, kind, 0, 1.5,
-                               o.ptr(got_affinities, o.f32p), o.ptr(got_experts, o.u32p), o.ptr(got_weights, o.f32p))
+        orc.orc_router_route(ptr(x, u16p), ptr(w, u16p), ptr(bias, f32p), rows, hidden, experts, picks, kind, 0, 1.5,
+                               ptr(got_affinities, f32p), ptr(got_experts, u32p), ptr(got_weights, f32p))
         scores = np.zeros((rows, experts), np.float32)
-        o.orc.orc_router_projection(o.ptr(x, o.u16p), o.ptr(w, o.u16p), rows, hidden, experts, o.ptr(scores, o.f32p))
-        affinities = np.array([[o.orc.orc_router_affinity(float(s), kind) for s in row] for row in scores], np.float32)
+        orc.orc_router_projection(ptr(x, u16p), ptr(w, u16p), rows, hidden, experts, ptr(scores, f32p))
+        affinities = np.array([[orc.orc_router_affinity(float(s), kind) for s in row] for row in scores], np.float32)
         want_experts, want_weights = np.zeros((rows, picks), np.uint32), np.zeros((rows, picks), np.float32)
         for r in range(rows):
-            o.orc.orc_router_select(o.ptr(affinities[r], o.f32p), o.ptr(bias, o.f32p), experts, picks, 0, 1.5,
-                                    o.ptr(want_experts[r], o.u32p), o.ptr(want_weights[r], o.f32p))
+            orc.orc_router_select(ptr(affinities[r], f32p), ptr(bias, f32p), experts, picks, 0, 1.5,
+                                    ptr(want_experts[r], u32p), ptr(want_weights[r], f32p))
         assert got_affinities.tobytes() == affinities.tobytes()
         assert np.array_equal(got_experts, want_experts) and got_weights.tobytes() == want_weights.tobytes()
