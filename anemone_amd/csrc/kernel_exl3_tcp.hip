@@ -9,13 +9,12 @@
  * weights, float32 MFMA sums over increasing k (one chain an output: the GEMM is not cut along k), SwiGLU in float32,
  * a row's weighted pair outputs added in slot order. A pair's result does not depend on the other pairs of the call.
  *
- * The GEMM block: 256 outputs (four wavefronts of four 16 x 16 tiles) by one chunk of at most 128 pairs of one expert.
- * A K step is 32 inputs: the chunk's operand columns (128 x 32 fp16, 8 KB) go from memory straight into LDS once a
- * block and serve all four wavefronts; each wavefront streams the two tile rows of its own strip through a private LDS
- * window, decodes each 16 x 32 weight tile once (eight weights a lane) and feeds it to eight MFMAs, one for every
- * sixteen columns. Decoding is the vector unit's work (about 4.4 instructions a weight) and the products the matrix
- * unit's (16 cycles an MFMA): at 128 columns the two take about the same time and overlap across the wavefronts of a
- * SIMD.
+ * The GEMM block: 256 outputs (four wavefronts of four 16 x 16 tiles) by one chunk of at most EXL3_TCP_CHUNK_PAIRS (160)
+ * pairs of one expert. A K step is 32 inputs: the chunk's operand columns (160 x 32 fp16, 10 KB) go from memory straight
+ * into LDS once a block and serve all four wavefronts; each wavefront streams the two tile rows of its own strip through a
+ * private LDS window, decodes each 16 x 32 weight tile once (eight weights a lane) and feeds it to up to ten MFMAs, one for
+ * every sixteen columns. Decoding is the vector unit's work (about 4.4 instructions a weight) and the products the matrix
+ * unit's (16 cycles an MFMA).
  */
 #include "exl3_device.cuh"
 #include "kernel_registry.h"

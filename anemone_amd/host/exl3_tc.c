@@ -138,7 +138,8 @@ result_status exl3_tc_prepare_paired(const struct exl3_tc_record *record, uint64
  *   activate    exl3_tcp_activate   (intermediate / 128, chunk capacity, 1)          64
  *   down        exl3_tcp_gemm       (ceil(hidden / 256), chunk capacity, 1)          256   pass EXL3_TCP_DOWN
  *   combine     exl3_tcp_combine    (hidden / 128, rows, 1)                          64
- * chunk capacity = pairs / 128 + experts: an expert's pairs cut in chunks of 128, the last ragged.
+ * chunk capacity = pairs / EXL3_TCP_CHUNK_PAIRS + experts: an expert's pairs cut in chunks of EXL3_TCP_CHUNK_PAIRS (160), the
+ * last ragged.
  */
 static result_status tcp_prepare(const struct exl3_tcp_record *record, uint64_t arena_byte_count,
                                  const struct backend_operations *backend, struct device_card *card,
@@ -162,8 +163,9 @@ static result_status tcp_prepare(const struct exl3_tcp_record *record, uint64_t 
         REFUSE("%s: rotation, halves of rows, cone layers and the two-blocks forms are forms this library does not build", what);
         return STATUS_UNSUPPORTED;
     }
-    if (H == 0 || I == 0 || I % EXL3_TRANSFORM != 0 || H % EXL3_TRANSFORM != 0) {
-        REFUSE("%s: hidden %u and intermediate %u: multiples of 128", what, H, I);
+    if (H == 0 || I == 0 || I % EXL3_TRANSFORM != 0 || H % EXL3_TRANSFORM != 0 || I > 2u * H) {
+        /* the activation writes the down operands [pairs][intermediate] over the gate and up operands [2][pairs][hidden] */
+        REFUSE("%s: hidden %u and intermediate %u: multiples of 128, the intermediate size at most twice the hidden", what, H, I);
         return STATUS_UNSUPPORTED;
     }
     const bool mixed = record->widths_offset != 0;

@@ -381,6 +381,8 @@ def test_tcp_prepare_geometry_and_refusals(fake):
     assert layout["total"] % 256 == 0 and layout["down"] - layout["gate_up"] == 2 * 32768 * 2048 * 4
     for changes, status in ((dict(row_count=0), 1), (dict(pairs_per_row=9), 1), (dict(expert_count=0), 1), (dict(pass_=1), 1),
                             (dict(rotation=1), 7), (dict(half_rows=5), 7), (dict(cone_layer=3), 7), (dict(intermediate=2000), 7),
+                            (dict(hidden=1024, intermediate=2176), 7),  # the down operands would not fit over the gate and up operands
+
                             (dict(bits_x2=7), 7), (dict(bits_x2=40), 1), (dict(workspace_offset=(256 << 20) + 16), 1),
                             (dict(workspace_offset=ARENA - 4096), 1), (dict(output_offset=2 << 20), 1)):
         untouched, n = amd.launches_of(8), C.c_uint32(99)
