@@ -19,7 +19,8 @@ LAUNCH_CHAIN, LAUNCH_SIDE, LAUNCH_RESUME, LAUNCH_JOIN, LAUNCH_SIDE_MORE = 0, 1, 
 ROUTER_SORT_ROWS = 384
 EXL3_TCP_CHUNK_PAIRS = 160
 EXL3_EXPERT_LAUNCHES, EXL3_TC_LAUNCHES = 5, 5
-EXL3_TC_GATE_UP_SLICES, EXL3_TC_DOWN_SLICES = 8, 4
+EXL3_TC_STATIC_SCRATCH_BYTES = 16 << 20
+EXL3_TC_GATE_UP_SLICES, EXL3_TC_DOWN_SLICES = 4, 4
 AFFINITY_SQRT_SOFTPLUS, AFFINITY_SIGMOID = 0, 1
 SECOND = 1_000_000_000
 

@@ -179,7 +179,7 @@ def test_tc_prepare_geometry_and_refusals(fake):
     assert [list(l.grid) for l in launches] == [[32, 64, 2], [32, 64, 2], [16, 64, 1], [64, 64, 1], [32, 8, 1]]
     passes = [amd.Exl3TcRecord.from_buffer_copy(bytes(l.argument)[:88]).pass_ for l in launches]
     assert passes == [0, 0, 0, 1, 0]
-    assert amd.exl3_tc_workspace_bytes(64, 4096, 2048) == 64 * 4096 * 4 + 8 * 2 * 64 * 2048 * 4 + 4 * 64 * 4096 * 4
+    assert amd.exl3_tc_workspace_bytes(64, 4096, 2048) == 64 * 4096 * 4 + 4 * 2 * 64 * 2048 * 4 + 4 * 64 * 4096 * 4
     for changes, status in [(dict(row_count=0), 1), (dict(row_count=65), 1), (dict(rotation=1), 7), (dict(shared_sum=2), 1),
                             (dict(shared_sum=1, shared_offset=ARENA - 4096), 1), (dict(shared_sum=1, shared_offset=1 << 20), 1),
                             (dict(intermediate=2000), 7), (dict(bits_x2=7), 7), (dict(bits_x2=0), 1), (dict(pass_=1), 1),
