@@ -15,6 +15,11 @@
  */
 #include "exl3_stream_device.cuh"
 #include "kernel_registry.h"
+#include "anemone_ops.h"
+
+#include <mutex>
+#include <stdio.h>
+#include <string.h>
 
 #define STRIP_PAIRS (EXL3_TC_STRIP_OUTPUTS / 32u) /* a strip: pairs of adjacent output tiles */
 /* false: the matrix instruction takes the codebook values before their scale and bias (1024 + b), which enter once a
@@ -294,3 +299,106 @@ extern "C" __global__ void exl3_tc_combine(struct exl3_tc_record record, unsigne
     out[channel + WAVE] = sum1;
 }
 ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_combine, exl3_tc_record);
+
+/* ---- the fused decode for callers that cannot allocate: the workspace in an array of the library's own ---- */
+
+/* Every device the library runs on holds its own copy of this array, at its own address, until the process ends. The
+ * name stands for the array in host code only as a symbol: its device address is asked for once a device. */
+static __device__ __align__(256) unsigned char scratch[EXL3_TC_STATIC_SCRATCH_BYTES];
+
+#define STATIC_MOST_DEVICES 64
+
+static result_status static_scratch_of(unsigned char **address_out)
+{
+    static std::mutex guard;
+    static unsigned char *address_of[STATIC_MOST_DEVICES];
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= STATIC_MOST_DEVICES) {
+        (void)fprintf(stderr, "anemone: exl3_tc_run_static: no current device among the first %d\n", STATIC_MOST_DEVICES);
+        return STATUS_DEVICE_ERROR;
+    }
+    std::lock_guard<std::mutex> held(guard);
+    if (address_of[device] == nullptr) {
+        unsigned char *address = nullptr;
+        const hipError_t asked = hipGetSymbolAddress((void **)&address, HIP_SYMBOL(scratch));
+        if (asked != hipSuccess || address == nullptr) {
+            (void)fprintf(stderr, "anemone: exl3_tc_run_static: hipGetSymbolAddress: %s\n", hipGetErrorString(asked));
+            return STATUS_DEVICE_ERROR;
+        }
+        address_of[device] = address;
+    }
+    *address_out = address_of[device];
+    return STATUS_OK;
+}
+
+/* kernel_prepare of a table that launches nothing: the four kernels of this file by number */
+static const char *const static_kernel_names[] = {"exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate", "exl3_tc_combine"};
+
+static result_status static_kernel_prepare(struct device_card *, const char *file, const char *function, uint32_t record_bytes,
+                                           uint32_t *kernel_out)
+{
+    if (strcmp(file, EXL3_TC_KERNEL_FILE) != 0 || record_bytes != sizeof(struct exl3_tc_record)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    for (uint32_t index = 0; index < 4u; index++) {
+        if (strcmp(function, static_kernel_names[index]) == 0) {
+            *kernel_out = index;
+            return STATUS_OK;
+        }
+    }
+    return STATUS_INVALID_ARGUMENT;
+}
+
+extern "C" result_status exl3_tc_run_static(const struct exl3_tc_record *record, void *arena_device, uint64_t arena_byte_count,
+                                            void *stream)
+{
+    if (record == nullptr || arena_device == nullptr) {
+        (void)fprintf(stderr, "anemone: exl3_tc_run_static: a missing argument\n");
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint32_t hidden = record->hidden != 0u ? record->hidden : EXL3_TC_DEFAULT_HIDDEN;
+    const uint32_t picks = record->pairs_per_row != 0u ? record->pairs_per_row : EXL3_TC_DEFAULT_PAIRS_PER_ROW;
+    const uint64_t pairs = (uint64_t)record->row_count * picks;
+    if (record->row_count > EXL3_TC_MOST_ROWS || picks > ROUTER_MOST_PICKS || hidden > (1u << 20) || record->intermediate > (1u << 20) ||
+        exl3_tc_workspace_bytes(pairs, hidden, record->intermediate) > EXL3_TC_STATIC_SCRATCH_BYTES) {
+        (void)fprintf(stderr, "anemone: exl3_tc_run_static: a step of %u rows of %u pairs, hidden %u, intermediate %u needs a workspace "
+                              "above the library's %u bytes\n", record->row_count, picks, hidden, record->intermediate,
+                      EXL3_TC_STATIC_SCRATCH_BYTES);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    unsigned char *workspace = nullptr;
+    const result_status found = static_scratch_of(&workspace);
+    if (found != STATUS_OK) {
+        return found;
+    }
+    struct backend_operations table;
+    memset(&table, 0, sizeof table);
+    table.kernel_prepare = static_kernel_prepare;
+    struct exl3_tc_record stamped = *record;
+    stamped.workspace_offset = 0u; /* checked for its alignment alone; the launches get the array's own offset below */
+    struct kernel_launch launches[EXL3_TC_LAUNCHES];
+    int placeholder = 0;
+    const result_status prepared = exl3_tc_prepare_detached(&stamped, arena_byte_count, &table, (struct device_card *)&placeholder, launches);
+    if (prepared != STATUS_OK) {
+        return prepared;
+    }
+    /* arena + offset is computed in 64 bits on the card: the difference of the two addresses names the array from the
+     * arena whichever lies higher */
+    const uint64_t offset = (uint64_t)(uintptr_t)workspace - (uint64_t)(uintptr_t)arena_device;
+    typedef void (*entry)(struct exl3_tc_record, unsigned char *);
+    const entry entries[4] = {exl3_tc_operands, exl3_tc_products, exl3_tc_activate, exl3_tc_combine};
+    for (uint32_t index = 0; index < EXL3_TC_LAUNCHES; index++) {
+        struct exl3_tc_record argument;
+        memcpy(&argument, launches[index].argument, sizeof argument);
+        argument.workspace_offset = offset;
+        hipLaunchKernelGGL(entries[launches[index].kernel], dim3(launches[index].grid[0], launches[index].grid[1], launches[index].grid[2]),
+                           dim3(launches[index].block[0], launches[index].block[1], launches[index].block[2]), 0, (hipStream_t)stream,
+                           argument, (unsigned char *)arena_device);
+        const hipError_t launched = hipGetLastError();
+        if (launched != hipSuccess) {
+            (void)fprintf(stderr, "anemone: exl3_tc_run_static: launch %u: %s\n", index, hipGetErrorString(launched));
+            return STATUS_DEVICE_ERROR;
+        }
+    }
+    return STATUS_OK;
+}

@@ -22,9 +22,10 @@
 #define PRODUCT_WAVES 4u
 #define MOST_GRID_ROWS 65535u
 
+/* detached_workspace: the workspace is not a range of the arena (exl3_tc_run_static names it by an offset of its own) */
 static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t arena_byte_count,
                                 const struct backend_operations *backend, struct device_card *card,
-                                struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
+                                struct kernel_launch launches_out[EXL3_TC_LAUNCHES], bool detached_workspace)
 {
     static const char what[] = "EXL3 fused decode";
     if (record == NULL || backend == NULL || backend->kernel_prepare == NULL || card == NULL || launches_out == NULL) {
@@ -62,15 +63,23 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
     }
     const uint64_t pairs = (uint64_t)record->row_count * picks;
     const uint64_t workspace = exl3_tc_workspace_bytes(pairs, hidden, I);
-    const struct checked_range ranges[] = {
+    struct checked_range ranges[5] = {
         {"the jobs", {record->jobs_offset, (uint64_t)record->job_capacity * sizeof(struct expert_job_record)},
          (uint64_t)record->job_capacity * sizeof(struct expert_job_record), false},
         {"the rows", {record->hidden_offset, (uint64_t)record->row_count * hidden * 2u}, (uint64_t)record->row_count * hidden * 2u, false},
-        {"the workspace", {record->workspace_offset, workspace}, workspace, false},
         {"the output", {record->output_offset, (uint64_t)record->row_count * hidden * 4u}, (uint64_t)record->row_count * hidden * 4u, false},
+        {"the workspace", {record->workspace_offset, workspace}, workspace, false},
         {"the shared expert's rows", {record->shared_offset, (uint64_t)record->row_count * hidden * 2u}, (uint64_t)record->row_count * hidden * 2u, false},
     };
-    if (!ranges_are_valid(what, ranges, record->shared_sum != 0u ? 5u : 4u, arena_byte_count) || record->workspace_offset % 256u != 0 ||
+    uint32_t range_count = 5u;
+    if (record->shared_sum == 0u) {
+        range_count = 4u;
+    }
+    if (detached_workspace) { /* the ranges of the arena alone */
+        ranges[3] = ranges[4];
+        range_count -= 1u;
+    }
+    if (!ranges_are_valid(what, ranges, range_count, arena_byte_count) || record->workspace_offset % 256u != 0 ||
         (mixed && record->widths_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0)) {
         if (record->workspace_offset % 256u != 0) {
             REFUSE("%s: the workspace begins off a multiple of 256", what);
@@ -110,21 +119,30 @@ result_status exl3_tc_prepare(const struct exl3_tc_record *record, uint64_t aren
                               const struct backend_operations *backend, struct device_card *card,
                               struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
 {
-    return tc_prepare(record, arena_byte_count, backend, card, launches_out);
+    return tc_prepare(record, arena_byte_count, backend, card, launches_out, false);
 }
 
 result_status exl3_tc_prepare_short(const struct exl3_tc_record *record, uint64_t arena_byte_count,
                                     const struct backend_operations *backend, struct device_card *card,
                                     struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
 {
-    return tc_prepare(record, arena_byte_count, backend, card, launches_out);
+    return tc_prepare(record, arena_byte_count, backend, card, launches_out, false);
 }
 
 result_status exl3_tc_prepare_paired(const struct exl3_tc_record *record, uint64_t arena_byte_count,
                                      const struct backend_operations *backend, struct device_card *card,
                                      struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
 {
-    return tc_prepare(record, arena_byte_count, backend, card, launches_out);
+    return tc_prepare(record, arena_byte_count, backend, card, launches_out, false);
+}
+
+/* The launches of exl3_tc_prepare for a workspace that is no range of the arena: every other range is checked against
+ * the arena as there, the workspace's offset only for its alignment. For exl3_tc_run_static. */
+result_status exl3_tc_prepare_detached(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                       const struct backend_operations *backend, struct device_card *card,
+                                       struct kernel_launch launches_out[EXL3_TC_LAUNCHES])
+{
+    return tc_prepare(record, arena_byte_count, backend, card, launches_out, true);
 }
 
 /*

@@ -88,6 +88,24 @@ MUST_CHECK result_status exl3_tc_prepare_paired(const struct exl3_tc_record *rec
                                                 const struct backend_operations *backend, struct device_card *card,
                                                 struct kernel_launch launches_out[EXL3_TC_LAUNCHES]);
 
+/* exl3_tc_prepare's launches for a workspace that is not a range of the arena (its offset is checked for alignment only);
+ * what exl3_tc_run_static builds its launches with */
+MUST_CHECK result_status exl3_tc_prepare_detached(const struct exl3_tc_record *record, uint64_t arena_byte_count,
+                                                  const struct backend_operations *backend, struct device_card *card,
+                                                  struct kernel_launch launches_out[EXL3_TC_LAUNCHES]);
+
+/* No counterpart in the reference. For callers that cannot allocate device memory (code under graph capture, serving
+ * loops and harnesses that forbid it): the fused decode of exl3_tc_prepare + launch_run, its five launches queued on
+ * `stream` (a hipStream_t; NULL: the default stream) of the current device, with the workspace in an array of
+ * EXL3_TC_STATIC_SCRATCH_BYTES that the library holds on every device it has run on, in place of a range of the arena.
+ * `arena_device` is the device address the record's offsets count from and `arena_byte_count` the bytes behind it that
+ * the record's ranges must lie in; record->workspace_offset is ignored. Allocates nothing and does not wait. A step
+ * whose workspace (exl3_tc_workspace_bytes) is larger than the array is refused with STATUS_INVALID_ARGUMENT. Calls on
+ * one device share that device's array: two calls whose launches overlap in time race. */
+#define EXL3_TC_STATIC_SCRATCH_BYTES (16u << 20)
+MUST_CHECK result_status exl3_tc_run_static(const struct exl3_tc_record *record, void *arena_device,
+                                            uint64_t arena_byte_count, void *stream);
+
 /* The prefill form (include/anemone/exl3_tc.h:40-59 of the reference): fills launches_out and *launch_count_out
  * (EXL3_TCP_LAUNCHES here). The reference's _base and _hybrid choose between two GEMM forms of the same bits; this
  * library has one form behind all three names. */

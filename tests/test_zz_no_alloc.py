@@ -1,0 +1,79 @@
+"""exl3_tc_run_static (the fused EXL3 decode with its workspace in an array the library holds on the device: the entry
+point for callers that cannot allocate) against exl3_tc_prepare + launch_run on the same bytes: two calls in a row,
+the second of a smaller step, each bit for bit the other entry point's output. The arena the static call reads is the
+caller's own memory (a torch tensor here), a copy of the card's arena as the select left it."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+from _oracle import normals, splitmix_words, to_bf16, exl3_matrix
+
+
+def say(*words):
+    print(*words, flush=True)
+    sys.stdout.flush()
+
+
+def one_step(amd, torch, rows, seed):
+    hidden, inner, experts_n, picks = 512, 256, 64, 4
+    width_choices = [2, 3, 4, 40]
+    draws = splitmix_words(seed, experts_n * 3) % np.uint64(len(width_choices))
+    widths = np.array(width_choices, dtype=np.uint32)[draws.astype(np.int64)].reshape(experts_n, 3)
+    matrices = [[exl3_matrix(seed * 1000 + 3 * e + 0, hidden, inner, int(widths[e, 0])),
+                 exl3_matrix(seed * 1000 + 3 * e + 1, hidden, inner, int(widths[e, 1])),
+                 exl3_matrix(seed * 1000 + 3 * e + 2, inner, hidden, int(widths[e, 2]))] for e in range(experts_n)]
+    router = to_bf16(normals(seed + 5, experts_n * hidden) * 0.02).reshape(experts_n, hidden)
+    x = to_bf16(normals(seed + 9, rows * hidden)).reshape(rows, hidden)
+    card = amd.Card(1 << 30)
+    try:
+        layer = amd.Exl3Layer(card, hidden, inner, experts_n, picks, rows, matrices, widths, router_weights_bf16=router, affinity_kind=1, limit=10.0)
+        layer.set_rows(x, rows)
+        card.run(layer.projection_launch())
+        card.run(layer.select_launch(0))
+        launches = layer.tc_launches()
+        used = (card.cursor + 255) // 256 * 256
+        before = card.download(0, used).copy()  # the arena as the select left it
+        card.run(launches)
+        want = layer.output().copy()
+        record = layer.tc_record()
+    finally:
+        card.close()
+    arena = torch.from_numpy(before).cuda()
+    out_bytes = rows * hidden * 4
+    arena[record.output_offset:record.output_offset + out_bytes] = 0xFF
+    record.workspace_offset = 0x12345600  # ignored by the static entry point
+    torch.cuda.synchronize()
+    lib = amd.library()
+    lib.exl3_tc_run_static.restype = C.c_int
+    lib.exl3_tc_run_static.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
+    status = lib.exl3_tc_run_static(C.byref(record), C.c_void_p(arena.data_ptr()), arena.numel(),
+                                    C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert status == 0, "exl3_tc_run_static answered %d" % status
+    torch.cuda.synchronize()
+    got = arena[record.output_offset:record.output_offset + out_bytes].cpu().numpy().view(np.float32).reshape(rows, hidden)
+    return got, want
+
+
+@pytest.mark.gpu
+def test_static_workspace_equals_the_arena_workspace_twice():
+    import torch
+    import anemone_amd as amd
+    for rows, seed in ((8, 41), (3, 42)):  # the second call of a smaller step: what the first left in the array must not show
+        say("exl3_tc_run_static", rows, "rows")
+        got, want = one_step(amd, torch, rows, seed)
+        assert np.all(np.isfinite(want)) and float(np.abs(want).max()) > 0.0
+        assert got.tobytes() == want.tobytes(), "the static workspace's output differs from the arena workspace's"
+
+
+def test_a_step_above_the_array_is_refused():
+    import anemone_amd as amd
+    lib = amd.library()
+    lib.exl3_tc_run_static.restype = C.c_int
+    lib.exl3_tc_run_static.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
+    record = amd.Exl3TcRecord()
+    record.row_count, record.job_capacity, record.intermediate, record.hidden, record.pairs_per_row, record.bits_x2 = 64, 512, 2048, 4096, 8, 6
+    assert amd.exl3_tc_workspace_bytes(64 * 8, 4096, 2048) > amd.EXL3_TC_STATIC_SCRATCH_BYTES
+    assert lib.exl3_tc_run_static(C.byref(record), C.c_void_p(4096), 1 << 30, None) == 1  # before any device call
+    assert lib.exl3_tc_run_static(None, C.c_void_p(4096), 1 << 30, None) == 1
