@@ -16,20 +16,18 @@
  * every sixteen columns. Decoding is the vector unit's work (about 4.4 instructions a weight) and the products the matrix
  * unit's (16 cycles an MFMA).
  */
-#include "exl3_device.cuh"
+#include "exl3_stream_device.cuh"
 #include "kernel_registry.h"
 #include "sort_device.cuh"
 
 #define TCP_SORT_THREADS 512u
 #define TCP_GEMM_WAVES 4u
 #define TCP_GEMM_THREADS (TCP_GEMM_WAVES * WAVE)
-#define TCP_WAVE_TILES 4u  /* output tiles of a wavefront: 64 outputs */
+#define TCP_WAVE_PAIRS 2u  /* pairs of adjacent output tiles of a wavefront: 64 outputs */
 #define TCP_COLUMN_BLOCKS (EXL3_TCP_CHUNK_PAIRS / 16u)
-#define TCP_STEP_INPUTS 32u
+#define TCP_STEP_INPUTS 64u
 #define TCP_BATCH 4u        /* columns the element-wise launches take at a time */
 #define TCP_WAVE_BLOCKS 4u  /* blocks of 128 channels a wavefront of an element-wise launch takes: a row of sixteen lanes each */
-#define TCP_OPERAND_PARTS ((TCP_COLUMN_BLOCKS + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES) /* 16-column groups a wavefront brings a step */
-#define TCP_STAGE_BYTES (TCP_OPERAND_PARTS * TCP_GEMM_WAVES * 1024u) /* a K step of the chunk's operand columns, in whole groups */
 
 struct tcp_shape {
     uint32_t hidden, intermediate, picks, pairs, experts;
@@ -247,137 +245,187 @@ extern "C" __global__ void exl3_tcp_operands(struct exl3_tcp_record record, unsi
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_operands, exl3_tcp_record);
 
-/* 16 bytes a lane from memory straight into LDS (lane L lands at lds_base + 16 L). Written as assembly so that the
- * compiler keeps no book on it; the waits are this file's own. */
+/*
+ * The GEMM block: 256 outputs by one chunk of at most EXL3_TCP_CHUNK_PAIRS pairs of one expert, four wavefronts of 64
+ * outputs each (two pairs of adjacent output tiles). A K step is 64 inputs (four K tiles).
+ *
+ * Weights: the codes go from memory straight into the registers of the lanes that decode them (exl3_stream_device.cuh:
+ * lane 16 g + i holds chunk i % 8 of tile i / 8 of a tile pair and of K tile g of the step); a decoded operand of eight
+ * weights a lane (output half h, input half v) feeds one matrix instruction a block of sixteen columns.
+ * Operands: a stage holds the step's 64 inputs of every column of the chunk, 128 bytes a column, its eight 16-byte pieces
+ * at the slots piece ^ ((column / 2) % 8) so that the sixteen lanes of one read (sixteen columns, one piece) meet sixteen
+ * different bank groups. Each wavefront brings a share of the stage (memory -> registers a step ahead -> LDS), one
+ * barrier a step; the reader of column block j takes piece 2 g + v of column 16 j + i as the instruction's B operand.
+ */
+/* 16 bytes a lane from memory straight into LDS (lane L lands at lds_base + 16 L), no register in between. Written as
+ * assembly: the compiler keeps no book on it, so the wait that ends a step (every load of the wavefront, then the block's
+ * barrier) is written out below. */
 __device__ static __forceinline__ void tcp_load_to_lds(const void *lane_address, uint32_t lds_base)
 {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_address), "s"(lds_base) : "memory", "m0");
 }
 
-template <uint32_t count>
-__device__ static __forceinline__ void tcp_wait_loads()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(count) : "memory");
-}
+#define TCP_STAGE_COLUMN_BYTES (TCP_STEP_INPUTS * 2u)
+#define TCP_STAGE_BYTES (EXL3_TCP_CHUNK_PAIRS * TCP_STAGE_COLUMN_BYTES)
+#define TCP_STAGE_GROUPS (EXL3_TCP_CHUNK_PAIRS / 8u) /* groups of eight columns: one 16-byte-a-lane load of a wavefront each */
+#define TCP_WAVE_GROUPS ((TCP_STAGE_GROUPS + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES)
 
-/* One wavefront of a GEMM block: its strip of TCP_WAVE_TILES output tiles against the chunk's columns, every K step.
- *   codes      the matrix's trellis, [inputs / 16][out_tiles][tile_words] uint32; strip_tile: the strip's first tile
- *   columns    the chunk's first operand row (fp16 [pair][inputs], rows of the chunk consecutive), count of them
- *   stage      LDS address of the block's two operand stages; window: of this wavefront's two weight windows
- * Lane L of an operand load lands at bytes 16 L of a 16-column group: column L / 4, slot L % 4, and asks for that
- * column's 16-byte piece (L % 4) ^ (column / 4) of the step, so that the readers of one piece of sixteen columns
- * meet different banks. */
 template <uint32_t bits_x2, uint32_t LIVE>
 __device__ static __forceinline__ void
 tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t strip_tile, uint32_t inputs,
-              const half_t *__restrict__ columns, uint32_t column_count, uint32_t stage, uint32_t window, uint32_t wave,
-              uint32_t lane, bool strip_is_live, float4_t (&accumulator)[TCP_WAVE_TILES][TCP_COLUMN_BLOCKS])
+              const half_t *__restrict__ columns, uint32_t column_count, uint32_t stages, uint32_t wave,
+              uint32_t lane, bool strip_is_live, float4_t (&accumulator)[TCP_WAVE_PAIRS][2][LIVE])
 {
-    typedef exl3_width<bits_x2> W;
-    constexpr uint32_t row_bytes = TCP_WAVE_TILES * W::tile_bytes, row_lanes = row_bytes / 16u;
-    constexpr uint32_t window_bytes = 2u * row_bytes; /* the two tile rows of a K step */
-    static_assert(row_bytes % 16u == 0u && 2u * row_lanes <= WAVE, "a step's two strip rows are one load of the wavefront");
-    const uint32_t o = lane % 16u, g = lane / 16u, tau = g / 2u, q = g % 2u;
-    const exl3_run_place run0 = exl3_run_of<bits_x2>(o, 2u * q), run1 = exl3_run_of<bits_x2>(o, 2u * q + 1u);
-    const uint64_t row_stride = (uint64_t)out_tiles * W::tile_bytes; /* bytes between K tile rows */
-    /* weights: lanes 0 .. row_lanes - 1 carry the step's first tile row, the next row_lanes its second */
-    const bool carries = lane < 2u * row_lanes && strip_is_live;
-    const unsigned char *weight_source = (const unsigned char *)codes + (uint64_t)strip_tile * W::tile_bytes +
-                                         (lane / row_lanes) * row_stride + (lane % row_lanes) * 16u;
-    /* operands: this wavefront brings TCP_OPERAND_PARTS of the step's 16-column groups: wave, wave + 4, ... (a group
-     * past the chunk's columns lands in the stage's spare room) */
-    const uint32_t load_column = lane / 4u, load_piece = (lane % 4u) ^ (load_column / 4u);
-    const unsigned char *operand_source[TCP_OPERAND_PARTS]; /* a column past the chunk's last reads the first again: never stored */
+    typedef exl3_chunk<bits_x2> C;
+    constexpr uint32_t live_groups = 2u * LIVE; /* groups of eight columns that hold a pair */
+    constexpr uint32_t wave_groups = (live_groups + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES;
+    const uint32_t g = lane / 16u, i = lane % 16u, c = i % 8u;
+    const bool odd = (c & 1u) != 0u;
+    uint32_t own, front;
+    exl3_chunk_place<bits_x2>(c, own, front);
+    const uint64_t step_stride = 4u * (uint64_t)out_tiles * C::tile_words;
+    /* a strip past the matrix reads the matrix's first strip (its sums are not stored): every wavefront runs the same loop */
+    const uint32_t *tile = codes + ((uint64_t)g * out_tiles + (strip_is_live ? strip_tile : 0u) + i / 8u) * C::tile_words;
+    /* the stage's groups this wavefront brings: wave, wave + 4, ...: lane L column 8 G + L / 8, slot L % 8 */
+    const unsigned char *operand_source[wave_groups];
 #pragma unroll
-    for (uint32_t part = 0; part < TCP_OPERAND_PARTS; part++) {
-        const uint32_t column = 16u * (wave + TCP_GEMM_WAVES * part) + load_column;
-        operand_source[part] = (const unsigned char *)(columns + (uint64_t)(column < column_count ? column : 0u) * inputs) + load_piece * 16u;
+    for (uint32_t part = 0; part < wave_groups; part++) {
+        const uint32_t group = wave + TCP_GEMM_WAVES * part, column = 8u * group + lane / 8u;
+        const uint32_t piece = (lane % 8u) ^ ((column / 2u) % 8u);
+        operand_source[part] = (const unsigned char *)(columns + (uint64_t)(column < column_count ? column : 0u) * inputs) + piece * 16u;
     }
-    /* where this lane reads its operand halves of column block j: column o, pieces 2 tau and 2 tau + 1, bytes 8 q .. */
-    const uint32_t swizzle = o / 4u;
-    const uint32_t read_low = o * 64u + ((2u * tau) ^ swizzle) * 16u + 8u * q, read_high = o * 64u + ((2u * tau + 1u) ^ swizzle) * 16u + 8u * q;
+    /* where this lane reads its B operand (v = 0, 1) of column block j: column 16 j + i, piece 2 g + v */
+    uint32_t read_at[2];
 #pragma unroll
-    for (uint32_t n = 0; n < TCP_WAVE_TILES; n++) {
+    for (uint32_t v = 0; v < 2u; v++) {
+        read_at[v] = i * TCP_STAGE_COLUMN_BYTES + (((2u * g + v) ^ ((i / 2u) % 8u)) * 16u);
+    }
 #pragma unroll
-        for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
-            accumulator[n][j] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
+#pragma unroll
+        for (uint32_t h = 0; h < 2u; h++) {
+#pragma unroll
+            for (uint32_t j = 0; j < LIVE; j++) {
+                accumulator[p][h][j] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+            }
         }
     }
     const uint32_t steps = inputs / TCP_STEP_INPUTS;
-#define TCP_ISSUE(step, buffer)                                                                                       \
-    do {                                                                                                              \
-        _Pragma("unroll") for (uint32_t part = 0; part < TCP_OPERAND_PARTS; part++)                                   \
-        {                                                                                                             \
-            tcp_load_to_lds(operand_source[part] + (uint64_t)(step) * (TCP_STEP_INPUTS * 2u),                         \
-                            stage + (buffer) * TCP_STAGE_BYTES + (wave + TCP_GEMM_WAVES * part) * 1024u);             \
-        }                                                                                                             \
-        if (carries) {                                                                                                \
-            tcp_load_to_lds(weight_source + (uint64_t)(step) * 2u * row_stride, window + (buffer) * window_bytes);    \
-        }                                                                                                             \
-    } while (0)
-    TCP_ISSUE(0u, 0u);
-    for (uint32_t step = 0; step < steps; step++) {
-        const uint32_t buffer = step % 2u;
-        if (step + 1u < steps) {
-            TCP_ISSUE(step + 1u, buffer ^ 1u);
-        }
-        /* a wavefront asks for its column groups and its weights a step, the groups alone when its strip lies past
-         * the matrix: this step's have landed once nothing but the next step's is outstanding */
-        if (step + 1u >= steps) {
-            tcp_wait_loads<0>();
-        } else if (strip_is_live) {
-            tcp_wait_loads<TCP_OPERAND_PARTS + 1u>();
-        } else {
-            tcp_wait_loads<TCP_OPERAND_PARTS>();
-        }
-        __syncthreads(); /* the other wavefronts' column groups of this step have landed as well */
-        uint2_t b_low[LIVE], b_high[LIVE]; /* the column blocks that hold a pair (LIVE of them: a constant) */
-        const uint32_t stage_base = stage + buffer * TCP_STAGE_BYTES;
+    exl3_chunk_words<bits_x2> held[2][TCP_WAVE_PAIRS];
+    /* step 0: its codes into held[0], its operand columns into stage 0 */
 #pragma unroll
-        for (uint32_t j = 0; j < LIVE; j++) {
-            b_low[j] = *(const __attribute__((address_space(3))) uint2_t *)(uintptr_t)(stage_base + j * 1024u + read_low);
-            b_high[j] = *(const __attribute__((address_space(3))) uint2_t *)(uintptr_t)(stage_base + j * 1024u + read_high);
+    for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
+        exl3_chunk_load<bits_x2>(tile + p * 2u * C::tile_words, own, front, held[0][p]);
+    }
+#pragma unroll
+    for (uint32_t part = 0; part < wave_groups; part++) {
+        if (wave + TCP_GEMM_WAVES * part < live_groups) {
+            tcp_load_to_lds(operand_source[part], stages + (wave + TCP_GEMM_WAVES * part) * 1024u);
         }
-        if (strip_is_live) {
-            const uint32_t window_base = window + buffer * window_bytes + tau * row_bytes;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    auto one_step = [&](uint32_t step, exl3_chunk_words<bits_x2> (&now)[TCP_WAVE_PAIRS], exl3_chunk_words<bits_x2> (&next)[TCP_WAVE_PAIRS]) {
+        const bool more = step + 1u < steps; /* the same in every lane */
+        const uint32_t stage = stages + (step % 2u) * TCP_STAGE_BYTES, other = stages + ((step + 1u) % 2u) * TCP_STAGE_BYTES;
+        if (more) {
+            tile += step_stride;
 #pragma unroll
-            for (uint32_t n = 0; n < TCP_WAVE_TILES; n++) {
-                const uint32_t tile_base = window_base + n * W::tile_bytes;
-                const uint32_t w00 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run0.word0);
-                const uint32_t w01 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run0.word1);
-                const uint32_t w10 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run1.word0);
-                const uint32_t w11 = *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)(tile_base + 4u * run1.word1);
-                const uint32_t f0 = __builtin_amdgcn_alignbit(w00, w01, run0.shift);
-                const uint32_t f1 = __builtin_amdgcn_alignbit(w10, w11, run1.shift);
-                uint32_t a[4];
-                exl3_decode_run<bits_x2>(f0, a[0], a[2]); /* run 0: inputs 4 q + {0, 1} and {8, 9} */
-                exl3_decode_run<bits_x2>(f1, a[1], a[3]); /* run 1: inputs 4 q + {2, 3} and {10, 11} */
-                const half8_t weights = __builtin_bit_cast(half8_t, *(const uint4_t *)a);
-                __builtin_amdgcn_s_setprio(1); /* the wavefront that feeds the matrix unit goes first at the issue */
+            for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
+                exl3_chunk_load<bits_x2>(tile + p * 2u * C::tile_words, own, front, next[p]);
+            }
 #pragma unroll
-                for (uint32_t j = 0; j < LIVE; j++) {
-                    const uint32_t b[4] = {b_low[j].x, b_low[j].y, b_high[j].x, b_high[j].y};
-                    accumulator[n][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(weights, __builtin_bit_cast(half8_t, *(const uint4_t *)b),
-                                                                               accumulator[n][j], 0, 0, 0);
+            for (uint32_t part = 0; part < wave_groups; part++) {
+                if (wave + TCP_GEMM_WAVES * part < live_groups) {
+                    tcp_load_to_lds(operand_source[part] + (uint64_t)(step + 1u) * TCP_STAGE_COLUMN_BYTES,
+                                    other + (wave + TCP_GEMM_WAVES * part) * 1024u);
                 }
-                __builtin_amdgcn_s_setprio(0);
             }
         }
-        /* this step's stage and window are read (their values are in registers or used); the step after the next may
-         * fill them once every wavefront is past this point */
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
+            exl3_chunk_align<bits_x2>(now[p], odd);
+        }
+        /* Eight operands of eight weights a lane: k = 4 v + 2 p + h (input half v outermost: its LIVE B operands are read
+         * from the stage once). An operand's LIVE matrix instructions are issued with the next operand's decoding between
+         * them, a quarter of it (two weights) behind every LIVE / 4 instructions: the decoding runs in the products' shadow. */
+        auto decode_weight = [&](uint32_t k, uint32_t w, uint32_t (&into)[4]) {
+            /* weight w = 2 t + e of operand k: symbol 8 t + 4 h + 2 v + e; the odd one completes its pair's register */
+            const uint32_t v = k / 4u, p = k / 2u % 2u, h = k % 2u, t = w / 2u, m = 8u * t + 4u * h + 2u * v + w % 2u;
+            uint32_t funnel[C::words];
+#pragma unroll
+            for (uint32_t word = 0; word < C::words; word++) {
+                funnel[word] = __builtin_amdgcn_alignbit(now[p].z[word], now[p].z[word + 1u], 16u);
+            }
+            const uint32_t product = exl3_chunk_state<bits_x2>(now[p].z, funnel, m) * EXL3_MUL1_MULTIPLIER;
+            if (w % 2u == 0u) {
+                into[t] = __builtin_amdgcn_sad_u8(product, 0u, (uint32_t)EXL3_MUL1_BASE * 0x10001u);
+            } else {
+                const uint32_t sums = __builtin_amdgcn_sad_hi_u8(product, 0u, into[t]);
+                const half2_t scale = __builtin_bit_cast(half2_t, (uint32_t)EXL3_MUL1_SCALE * 0x10001u);
+                const half2_t bias = __builtin_bit_cast(half2_t, (uint32_t)EXL3_MUL1_BIAS * 0x10001u);
+                into[t] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(half2_t, sums), scale, bias));
+            }
+        };
+        half8_t operand_b[LIVE];
+        uint32_t a[4], ahead[4];
+        auto read_operands = [&](uint32_t v) {
+#pragma unroll
+            for (uint32_t j = 0; j < LIVE; j++) {
+                operand_b[j] = __builtin_bit_cast(half8_t, *(const __attribute__((address_space(3))) uint4_t *)(uintptr_t)(stage + j * (16u * TCP_STAGE_COLUMN_BYTES) + read_at[v]));
+            }
+        };
+        read_operands(0u); /* on their way while the first operand is decoded */
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t w = 0; w < 8u; w++) {
+            decode_weight(0u, w, a);
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < 8u; k++) {
+            const uint32_t p = k / 2u % 2u, h = k % 2u;
+            if (k == 4u) {
+                read_operands(1u);
+            }
+            const uint4_t packed = {a[0], a[1], a[2], a[3]};
+            const half8_t weights = __builtin_bit_cast(half8_t, packed);
+#pragma unroll
+            for (uint32_t j = 0; j < LIVE; j++) {
+                accumulator[p][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(weights, operand_b[j], accumulator[p][h][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (k + 1u < 8u) {
+#pragma unroll
+                    for (uint32_t w = 0; w < 8u; w++) {
+                        if (w * LIVE / 8u == j) {
+                            decode_weight(k + 1u, w, ahead);
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (uint32_t t = 0; t < 4u; t++) {
+                a[t] = ahead[t];
+            }
+        }
+        /* every load of this wavefront has landed (the next step's stage among them), this step's stage is read */
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __syncthreads();
+    };
+    for (uint32_t step = 0; step < steps; step += 2u) {
+        one_step(step, held[0], held[1]);
+        if (step + 1u < steps) {
+            one_step(step + 1u, held[1], held[0]);
+        }
     }
-#undef TCP_ISSUE
 }
 
 /* launches 3 and 5: grid (ceil(outputs / 256), chunk capacity, projections), block 256.
  * pass EXL3_TCP_GATE_AND_UP: z = 0 gate, 1 up, products [z][place][intermediate]; pass EXL3_TCP_DOWN: down,
  * products [place][hidden]. */
-extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS) exl3_tcp_gemm(struct exl3_tcp_record record, unsigned char *arena)
+extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS, 2) exl3_tcp_gemm(struct exl3_tcp_record record, unsigned char *arena)
 {
     __shared__ __attribute__((aligned(16))) unsigned char stages[2u * TCP_STAGE_BYTES];
-    __shared__ __attribute__((aligned(16))) unsigned char windows[TCP_GEMM_WAVES][2u * 2u * TCP_WAVE_TILES * exl3_width<8>::tile_bytes];
     const tcp_shape shape = tcp_shape_of(record);
     unsigned char *workspace = arena + record.workspace_offset;
     const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, blockIdx.y);
@@ -394,21 +442,44 @@ extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS) exl3_tcp_gemm(str
                             ((uint64_t)(down ? 0u : projection) * shape.pairs + chunk.first_pair) * inputs;
     float *products = down ? (float *)(workspace + shape.layout.down) + (uint64_t)chunk.first_pair * outputs
                            : (float *)(workspace + shape.layout.gate_up) + ((uint64_t)projection * shape.pairs + chunk.first_pair) * outputs;
-    const uint32_t strip_tile = (blockIdx.x * EXL3_TCP_BLOCK_OUTPUTS) / EXL3_TILE + wave * TCP_WAVE_TILES;
+    const uint32_t strip_tile = (blockIdx.x * EXL3_TCP_BLOCK_OUTPUTS) / EXL3_TILE + wave * 2u * TCP_WAVE_PAIRS;
     const bool strip_is_live = strip_tile * EXL3_TILE < outputs;
-    const uint32_t stage = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)stages;
-    const uint32_t window = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)&windows[wave][0];
-    float4_t accumulator[TCP_WAVE_TILES][TCP_COLUMN_BLOCKS];
-    /* one instance a width and a count of live column blocks (4, 8 or all): the blocks past the count keep their zeros */
+    const uint32_t stage_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)stages;
+    /* one instance a width and a count of live column blocks (2, 4, 6, 8 or all): the pairs' columns and nothing past them */
     const uint32_t live_blocks = (chunk.pair_count + 15u) / 16u;
-#define TCP_GEMM_OF(bits, live) tcp_wave_gemm<bits, live>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage, window, wave, lane, strip_is_live, accumulator)
-#define TCP_GEMM_WIDTH(bits)                \
-    if (live_blocks <= 4u) {                \
-        TCP_GEMM_OF(bits, 4u);              \
-    } else if (live_blocks <= 8u) {         \
-        TCP_GEMM_OF(bits, 8u);              \
-    } else {                                \
-        TCP_GEMM_OF(bits, TCP_COLUMN_BLOCKS); \
+#define TCP_GEMM_OF(bits, live)                                                                                                   \
+    do {                                                                                                                          \
+        float4_t accumulator[TCP_WAVE_PAIRS][2][live];                                                                            \
+        tcp_wave_gemm<bits, live>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage_base, wave, lane, \
+                                  strip_is_live, accumulator);                                                                    \
+        if (strip_is_live) {                                                                                                      \
+            _Pragma("unroll") for (uint32_t j = 0; j < live; j++)                                                                 \
+            {                                                                                                                     \
+                const uint32_t column = 16u * j + lane % 16u;                                                                     \
+                if (column < chunk.pair_count) {                                                                                  \
+                    float *out = products + (uint64_t)column * outputs;                                                           \
+                    _Pragma("unroll") for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++)                                               \
+                    {                                                                                                             \
+                        _Pragma("unroll") for (uint32_t h = 0; h < 2u; h++)                                                       \
+                        {                                                                                                         \
+                            *(float4_t *)(out + exl3_stream_output(strip_tile, p, h, lane)) = accumulator[p][h][j];               \
+                        }                                                                                                         \
+                    }                                                                                                             \
+                }                                                                                                                 \
+            }                                                                                                                     \
+        }                                                                                                                         \
+    } while (0)
+#define TCP_GEMM_WIDTH(bits)                    \
+    if (live_blocks <= 2u) {                    \
+        TCP_GEMM_OF(bits, 2u);                  \
+    } else if (live_blocks <= 4u) {             \
+        TCP_GEMM_OF(bits, 4u);                  \
+    } else if (live_blocks <= 6u) {             \
+        TCP_GEMM_OF(bits, 6u);                  \
+    } else if (live_blocks <= 8u) {             \
+        TCP_GEMM_OF(bits, 8u);                  \
+    } else {                                    \
+        TCP_GEMM_OF(bits, TCP_COLUMN_BLOCKS);   \
     }
     switch (bits_x2) {
     case 4u: TCP_GEMM_WIDTH(4u) break;
@@ -419,21 +490,6 @@ extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS) exl3_tcp_gemm(str
     }
 #undef TCP_GEMM_WIDTH
 #undef TCP_GEMM_OF
-    if (!strip_is_live) {
-        return;
-    }
-    /* lane l of an accumulator: column l % 16 of its block, outputs 4 (l / 16) + i of its tile */
-#pragma unroll
-    for (uint32_t j = 0; j < TCP_COLUMN_BLOCKS; j++) {
-        const uint32_t column = 16u * j + lane % 16u;
-        if (column < chunk.pair_count) {
-            float *out = products + (uint64_t)column * outputs + strip_tile * EXL3_TILE + 4u * (lane / 16u);
-#pragma unroll
-            for (uint32_t n = 0; n < TCP_WAVE_TILES; n++) {
-                *(float4_t *)(out + n * EXL3_TILE) = accumulator[n][j];
-            }
-        }
-    }
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_gemm, exl3_tcp_record);
 
