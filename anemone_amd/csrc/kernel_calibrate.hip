@@ -27,3 +27,85 @@ extern "C" __global__ void arena_copy(struct arena_copy_arguments arguments, uns
     }
 }
 ANEMONE_KERNEL("kernel_calibrate", arena_copy, arena_copy_arguments);
+
+/* issue_rate -- the second yardstick: how often a SIMD issues one vector instruction of the kinds the EXL3 codebook is
+ * made of, and how a matrix instruction and vector instructions of one wavefront share the issue. A block is one
+ * wavefront; `kind` names the instruction, eight independent chains a lane, `iterations` trips of eight each; kinds 8
+ * to 10 are trips of four v_mfma_f32_16x16x32_f16 alone, of eight vector instructions alone, and of the four matrix
+ * instructions with two of the vector instructions behind each. The host times the launch; what is written is only there to keep the chains alive. */
+struct issue_rate_arguments {
+    uint64_t output_offset; /* written: uint32 [grid x 64] */
+    uint32_t kind;
+    uint32_t iterations;
+};
+static_assert(sizeof(struct issue_rate_arguments) == 16, "issue_rate_arguments ABI");
+
+typedef _Float16 rate_half8 __attribute__((ext_vector_type(8)));
+typedef float rate_float4 __attribute__((ext_vector_type(4)));
+
+template <uint32_t KIND>
+__device__ static __forceinline__ void issue_rate_loop(uint32_t iterations, uint32_t (&a)[8], rate_float4 (&sums)[4], rate_half8 left, rate_half8 right)
+{
+    const uint32_t multiplier = 0x83DCD12Du;
+    for (uint32_t trip = 0; trip < iterations; trip++) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; i++) {
+            if constexpr (KIND == 0u) asm volatile("v_mul_lo_u32 %0, %0, %1" : "+v"(a[i]) : "s"(multiplier));
+            if constexpr (KIND == 1u) asm volatile("v_sad_u8 %0, %0, 0, %0" : "+v"(a[i]));
+            if constexpr (KIND == 2u) asm volatile("v_bfe_u32 %0, %0, 3, 16" : "+v"(a[i]));
+            if constexpr (KIND == 3u) asm volatile("v_and_b32 %0, 0xffff, %0" : "+v"(a[i]));
+            if constexpr (KIND == 4u) asm volatile("v_pk_fma_f16 %0, %0, %1, %0" : "+v"(a[i]) : "s"(multiplier));
+            if constexpr (KIND == 5u) asm volatile("v_alignbit_b32 %0, %0, %0, 16" : "+v"(a[i]));
+            if constexpr (KIND == 6u) asm volatile("v_lshrrev_b32 %0, 3, %0" : "+v"(a[i]));
+            if constexpr (KIND == 7u) asm volatile("v_perm_b32 %0, %0, %0, %1" : "+v"(a[i]) : "s"(multiplier));
+            if constexpr (KIND >= 8u) {
+                if (KIND != 9u && i % 2u == 0u) { /* four matrix instructions a trip, each its own sums */
+                    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(sums[i / 2u]) : "v"(left), "v"(right));
+                }
+                if (KIND != 8u) {
+                    if (i % 2u == 0u) {
+                        asm volatile("v_mul_lo_u32 %0, %0, %1" : "+v"(a[i]) : "s"(multiplier));
+                    } else {
+                        asm volatile("v_sad_u8 %0, %0, 0, %0" : "+v"(a[i]));
+                    }
+                }
+            }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(64) issue_rate(struct issue_rate_arguments arguments, unsigned char *arena)
+{
+    uint32_t a[8];
+    for (uint32_t i = 0; i < 8u; i++) {
+        a[i] = threadIdx.x * 2654435761u + i;
+    }
+    rate_half8 left, right;
+    for (uint32_t i = 0; i < 8u; i++) {
+        left[i] = (_Float16)(float)(threadIdx.x % 7u + i);
+        right[i] = (_Float16)(float)i;
+    }
+    rate_float4 sums[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    switch (arguments.kind) {
+    case 0u: issue_rate_loop<0u>(arguments.iterations, a, sums, left, right); break;
+    case 1u: issue_rate_loop<1u>(arguments.iterations, a, sums, left, right); break;
+    case 2u: issue_rate_loop<2u>(arguments.iterations, a, sums, left, right); break;
+    case 3u: issue_rate_loop<3u>(arguments.iterations, a, sums, left, right); break;
+    case 4u: issue_rate_loop<4u>(arguments.iterations, a, sums, left, right); break;
+    case 5u: issue_rate_loop<5u>(arguments.iterations, a, sums, left, right); break;
+    case 6u: issue_rate_loop<6u>(arguments.iterations, a, sums, left, right); break;
+    case 7u: issue_rate_loop<7u>(arguments.iterations, a, sums, left, right); break;
+    case 8u: issue_rate_loop<8u>(arguments.iterations, a, sums, left, right); break;
+    case 9u: issue_rate_loop<9u>(arguments.iterations, a, sums, left, right); break;
+    default: issue_rate_loop<10u>(arguments.iterations, a, sums, left, right); break;
+    }
+    uint32_t kept = 0;
+    for (uint32_t i = 0; i < 8u; i++) {
+        kept ^= a[i];
+    }
+    for (uint32_t i = 0; i < 4u; i++) {
+        kept ^= (uint32_t)(sums[i][0] + sums[i][1] + sums[i][2] + sums[i][3]);
+    }
+    ((uint32_t *)(arena + arguments.output_offset))[blockIdx.x * 64u + threadIdx.x] = kept;
+}
+ANEMONE_KERNEL("kernel_calibrate", issue_rate, issue_rate_arguments);
