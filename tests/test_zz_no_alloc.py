@@ -1,7 +1,8 @@
 """exl3_tc_run_static (the fused EXL3 decode with its workspace in an array the library holds on the device: the entry
 point for callers that cannot allocate) against exl3_tc_prepare + launch_run on the same bytes: two calls in a row,
 the second of a smaller step, each bit for bit the other entry point's output. The arena the static call reads is the
-caller's own memory (a torch tensor here), a copy of the card's arena as the select left it."""
+caller's own memory (allocated here from the HIP runtime the library itself is linked to, through ctypes: one runtime in
+the process whatever ran before), a copy of the card's arena as the select left it."""
 import ctypes as C
 import sys
 
@@ -16,7 +17,16 @@ def say(*words):
     sys.stdout.flush()
 
 
-def one_step(amd, torch, rows, seed):
+def hip_runtime():
+    hip = C.CDLL("libamdhip64.so.7")  # the library's own: already loaded with it
+    hip.hipMalloc.argtypes, hip.hipMalloc.restype = [C.POINTER(C.c_void_p), C.c_size_t], C.c_int
+    hip.hipMemcpy.argtypes, hip.hipMemcpy.restype = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int], C.c_int
+    hip.hipFree.argtypes, hip.hipFree.restype = [C.c_void_p], C.c_int
+    hip.hipDeviceSynchronize.argtypes, hip.hipDeviceSynchronize.restype = [], C.c_int
+    return hip
+
+
+def one_step(amd, hip, rows, seed):
     hidden, inner, experts_n, picks = 512, 256, 64, 4
     width_choices = [2, 3, 4, 40]
     draws = splitmix_words(seed, experts_n * 3) % np.uint64(len(width_choices))
@@ -40,29 +50,34 @@ def one_step(amd, torch, rows, seed):
         record = layer.tc_record()
     finally:
         card.close()
-    arena = torch.from_numpy(before).cuda()
     out_bytes = rows * hidden * 4
-    arena[record.output_offset:record.output_offset + out_bytes] = 0xFF
+    before[record.output_offset:record.output_offset + out_bytes] = 0xFF
     record.workspace_offset = 0x12345600  # ignored by the static entry point
-    torch.cuda.synchronize()
-    lib = amd.library()
-    lib.exl3_tc_run_static.restype = C.c_int
-    lib.exl3_tc_run_static.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
-    status = lib.exl3_tc_run_static(C.byref(record), C.c_void_p(arena.data_ptr()), arena.numel(),
-                                    C.c_void_p(torch.cuda.current_stream().cuda_stream))
-    assert status == 0, "exl3_tc_run_static answered %d" % status
-    torch.cuda.synchronize()
-    got = arena[record.output_offset:record.output_offset + out_bytes].cpu().numpy().view(np.float32).reshape(rows, hidden)
+    arena = C.c_void_p()
+    assert hip.hipMalloc(C.byref(arena), before.nbytes) == 0
+    try:
+        assert hip.hipMemcpy(arena, before.ctypes.data, before.nbytes, 1) == 0
+        lib = amd.library()
+        lib.exl3_tc_run_static.restype = C.c_int
+        lib.exl3_tc_run_static.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
+        status = lib.exl3_tc_run_static(C.byref(record), arena, before.nbytes, None)  # on the null stream
+        assert status == 0, "exl3_tc_run_static answered %d" % status
+        assert hip.hipDeviceSynchronize() == 0
+        got = np.zeros((rows, hidden), np.float32)
+        assert hip.hipMemcpy(got.ctypes.data, arena.value + record.output_offset, out_bytes, 2) == 0
+    finally:
+        hip.hipFree(arena)
     return got, want
 
 
 @pytest.mark.gpu
 def test_static_workspace_equals_the_arena_workspace_twice():
-    import torch
     import anemone_amd as amd
+    amd.library()
+    hip = hip_runtime()
     for rows, seed in ((8, 41), (3, 42)):  # the second call of a smaller step: what the first left in the array must not show
         say("exl3_tc_run_static", rows, "rows")
-        got, want = one_step(amd, torch, rows, seed)
+        got, want = one_step(amd, hip, rows, seed)
         assert np.all(np.isfinite(want)) and float(np.abs(want).max()) > 0.0
         assert got.tobytes() == want.tobytes(), "the static workspace's output differs from the arena workspace's"
 
