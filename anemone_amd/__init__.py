@@ -200,6 +200,16 @@ class HyperSiteDescription(C.Structure):
                                            "output", "routed_sums")] + [("row_count", u32), ("reserved_zero", u32)]
 
 
+class SiteFrontKernels(C.Structure):
+    _fields_ = [("fronts", u32 * 8)]
+
+
+class SiteFrontDescription(C.Structure):
+    _fields_ = [(name, Range) for name in ("streams", "carried_pre", "mix_weights", "scale", "base", "norm_weight", "post", "comb", "hidden",
+                                           "codes", "exponents", "operands", "scratch")] + \
+               [("router", C.POINTER(RouterDescription)), ("router_weights", Range), ("kind", u32), ("row_count", u32), ("reserved_zero", u32)]
+
+
 class LinearWideKernels(C.Structure):
     _fields_ = [("wide_expert_gate_up", u32), ("wide_expert_down", u32), ("wide_expert_gate_up_e4m3", u32), ("wide_expert_down_e4m3", u32),
                 ("wide_expert_gate_up_b128", u32), ("wide_expert_down_b128", u32)]
@@ -278,6 +288,8 @@ def library():
             "dense_linear_prepare": [C.POINTER(DenseLinearDescription), u64, C.POINTER(DenseLinearKernels), launch_p],
             "hyper_kernels_prepare": [vp, vp, C.POINTER(HyperKernelsRecord)],
             "hyper_site_prepare": [C.POINTER(HyperSiteDescription), u64, C.POINTER(HyperKernelsRecord), launch_p],
+            "site_front_kernels_prepare": [vp, vp, C.POINTER(SiteFrontKernels)],
+            "site_front_prepare": [C.POINTER(SiteFrontDescription), u64, C.POINTER(RouterKernels), C.POINTER(SiteFrontKernels), launch_p],
             "expert_post_prepare": [C.POINTER(ExpertJoinDescription), u64, u32, launch_p],
             "expert_shared_join_prepare": [C.POINTER(ExpertSharedJoinDescription), u64, C.POINTER(LinearKernels),
                                            C.POINTER(ExpertFusedKernels), launch_p],
@@ -827,6 +839,8 @@ MODEL_STREAMS = 4
 
 DENSE_BFLOAT16, DENSE_FLOAT32, DENSE_ROW_SCALE = 0, 1, 1
 MODEL_MIXES, MODEL_NORM_EPSILON = 24, 1e-20
+SITE_FRONT_SCRATCH_BYTES, SITE_FRONT_MOST_WIDTH = 7184, 5120
+SITE_FRONT_KIND_SITE, SITE_FRONT_KIND_FFN, SITE_FRONT_KIND_INPUT, SITE_FRONT_KIND_COEFFICIENTS = 0, 1, 2, 3
 
 
 class SiteFront:
@@ -882,6 +896,51 @@ class SiteFront:
         launches = launches_of(2)
         check(self.card.lib.hyper_site_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.hyper_kernels), launches), "hyper_site_prepare")
         return launches
+
+    def front_description(self, rows=None, layer=None, order=0, kind=None):
+        """The description of the fused front of `rows` rows (site_front_prepare); with `layer` (an Exl3Layer or Fp4Layer
+        whose rows are this front's hidden range) the FFN front, whose select is the layer's. Keeps what it points at."""
+        if "scratch" not in self.ranges:
+            sizes = {"codes": self.rows * self.width, "exponents": self.rows * self.width // 32, "operands": self.rows * self.width * 2,
+                     "scratch": SITE_FRONT_SCRATCH_BYTES}
+            self.ranges.update({name: Range(self.card.reserve(size), size) for name, size in sizes.items()})
+            self.card.upload(self.ranges["scratch"].byte_offset, np.zeros(SITE_FRONT_SCRATCH_BYTES, np.uint8))
+            self.front_kernels = SiteFrontKernels()
+            check(self.card.lib.site_front_kernels_prepare(backend_table(), self.card.handle, C.byref(self.front_kernels)), "site_front_kernels_prepare")
+        d = SiteFrontDescription()
+        for name in ("streams", "carried_pre", "mix_weights", "scale", "base", "norm_weight", "post", "comb", "hidden", "codes", "exponents",
+                     "operands", "scratch"):
+            setattr(d, name, self.ranges[name])
+        d.kind = (SITE_FRONT_KIND_SITE if layer is None else SITE_FRONT_KIND_FFN) if kind is None else kind
+        d.row_count, d.reserved_zero = self.rows if rows is None else rows, self.width
+        keep = [d]
+        if layer is not None:
+            experts = layer.experts_description()
+            r = RouterDescription()
+            r.experts = C.pointer(experts)
+            r.expert_offsets = layer.expert_offsets.ctypes.data_as(C.POINTER(u64))
+            packed = getattr(layer, "packed_widths", None)
+            r.expert_widths = packed.ctypes.data_as(C.POINTER(u32)) if packed is not None and getattr(layer, "uniform_width", 1) == 0 else None
+            r.step, r.scores = Range(layer.step_offset, 16), Range(layer.scores_offset, layer.rows * layer.E * 4)
+            r.bias, r.offsets = Range(layer.bias_offset, layer.E * 4), Range(layer.offsets_offset, layer.E * 24)
+            r.affinities = Range(layer.affinities_offset, layer.rows * layer.E * 4)
+            r.order, r.expert_count, r.pick_count = order, layer.E, layer.P
+            r.affinity_kind, r.route_scale = layer.affinity_kind, layer.route_scale
+            d.router = C.pointer(r)
+            d.router_weights = Range(layer.router_offset, layer.E * layer.H * 2)
+            keep += [experts, r]
+        self.kept = keep
+        return d
+
+    def front_launch(self, rows=None, layer=None, order=0):
+        """ONE launch for the mix project, the mix finish, (with `layer`: the router's scores and its select) and the
+        quantization of the sublayer's input."""
+        d = self.front_description(rows, layer, order)
+        router_kernels = None if layer is None else C.byref(layer.router_kernels)
+        launch = launches_of(1)
+        check(self.card.lib.site_front_prepare(C.byref(d), self.card.arena_bytes, router_kernels, C.byref(self.front_kernels), launch),
+              "site_front_prepare")
+        return launch
 
     def read(self, name, dtype=np.uint8):
         return self.card.download(self.ranges[name].byte_offset, self.ranges[name].byte_count, dtype)

@@ -15,9 +15,9 @@ INCLUDE = os.path.join(ROOT, "include")
 LIBRARY = os.path.join(HERE, "libanemone_hip.so")
 BUILD = os.path.join(HERE, "build")
 
-HOST_SOURCES = ["status.c", "prepare_common.c", "weight_format.c", "exl3.c", "exl3_tc.c", "router.c", "linear.c", "expert_fused.c", "site.c", "exl3_layout.c"]
+HOST_SOURCES = ["status.c", "prepare_common.c", "weight_format.c", "exl3.c", "exl3_tc.c", "router.c", "linear.c", "expert_fused.c", "site.c", "site_front.c", "exl3_layout.c"]
 HIP_SOURCES = ["kernel_exl3.hip", "kernel_exl3_tc.hip", "kernel_exl3_tcp.hip", "kernel_router.hip", "kernel_calibrate.hip", "kernel_selfcheck.hip", "kernel_dense_linear.hip", "kernel_activation_quantize.hip", "kernel_wide_linear.hip",
-               "kernel_expert_linear.hip", "kernel_trunk_linear.hip", "kernel_hyper_connection.hip"]
+               "kernel_expert_linear.hip", "kernel_trunk_linear.hip", "kernel_hyper_connection.hip", "kernel_site_front.hip"]
 
 BACKEND_SOURCES = ["backend_hip.cpp"]  # host C++ over the HIP runtime API: no device code
 BACKEND_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include"]

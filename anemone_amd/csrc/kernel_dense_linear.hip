@@ -25,27 +25,17 @@
 #include <stdint.h>
 
 #include "kernel_registry.h"
-#include "exl3_device.cuh"
+#include "dense_device.cuh"
 
-#define DENSE_GROUP_LANES 32u
-#define DENSE_GROUPS (DENSE_THREADS_VALUE / DENSE_GROUP_LANES)
-#define DENSE_DIES 8u
-
-/* the float32 nearest 1 / sqrt(operand): both steps are correctly rounded in double, whose 53 places decide a tie */
-__device__ static __forceinline__ float dense_reciprocal_root(float operand)
-{
-    return (float)(1.0 / __dsqrt_rn((double)operand));
-}
-
+/* a kernel's block: its outputs and rows by the grid. Blocks go to the card's 8 dies in turn by their linear index, and
+ * each die has its own L2. The blocks that share a group of rows (one an output group) are renumbered to follow each other
+ * on one die, so that the rows come from memory once and from that die's L2 for the other output groups: a bijection of
+ * the grid when its row groups divide by 8, the plain numbering otherwise. Which block computes an output changes nothing
+ * in its bits. */
 template <uint32_t TYPE, uint32_t ROWS, uint32_t OUTPUTS>
 __device__ static __forceinline__ void dense_linear(const struct dense_linear_arguments &arguments, unsigned char *arena)
 {
-    __shared__ float group_sums[DENSE_GROUPS][OUTPUTS + 1u][ROWS];
-    const uint32_t thread = threadIdx.x, inputs = arguments.input_size, chunks = inputs / DENSE_CHUNK_INPUTS;
-    /* Blocks go to the card's 8 dies in turn by their linear index, and each die has its own L2. The blocks that share a
-     * group of rows (one an output group) are renumbered to follow each other on one die, so that the rows come from
-     * memory once and from that die's L2 for the other output groups: a bijection of the grid when its row groups
-     * divide by 8, the plain numbering otherwise. Which block computes an output changes nothing in its bits. */
+    __shared__ dense_group_sums<ROWS, OUTPUTS> lds;
     uint32_t output_group = blockIdx.x, row_group = blockIdx.y;
     if constexpr (ROWS != 1u) {
         if (gridDim.y % DENSE_DIES == 0u) {
@@ -54,124 +44,8 @@ __device__ static __forceinline__ void dense_linear(const struct dense_linear_ar
             row_group = place / gridDim.x * DENSE_DIES + linear % DENSE_DIES;
         }
     }
-    const uint32_t first_output = output_group * OUTPUTS, first_row = row_group * ROWS;
-    const bool scaled = (arguments.flags & DENSE_ROW_SCALE) != 0u;
-    const uint16_t *rows = (const uint16_t *)(arena + arguments.rows_offset);
-    float chain[OUTPUTS][ROWS], squares[ROWS];
-#pragma unroll
-    for (uint32_t r = 0; r < ROWS; r++) {
-        squares[r] = 0.0f;
-#pragma unroll
-        for (uint32_t o = 0; o < OUTPUTS; o++) {
-            chain[o][r] = 0.0f;
-        }
-    }
-#pragma unroll(ROWS == 1u ? 4 : 1)
-    for (uint32_t chunk = thread; chunk < chunks; chunk += DENSE_THREADS_VALUE) {
-        /* every row's chunk is asked for before any is used: a chunk costs one trip to memory, not one a row */
-        uint4_t packed[ROWS];
-#pragma unroll
-        for (uint32_t r = 0; r < ROWS; r++) {
-            /* a column from row_count on reads row 0 and is stored nowhere */
-            const uint32_t row = first_row + r < arguments.row_count ? first_row + r : 0u;
-            packed[r] = *(const uint4_t *)(rows + (uint64_t)row * inputs + chunk * DENSE_CHUNK_INPUTS);
-        }
-        /* and every output's weights before the first chain runs */
-        float weights[OUTPUTS][DENSE_CHUNK_INPUTS];
-#pragma unroll
-        for (uint32_t o = 0; o < OUTPUTS; o++) {
-            const uint64_t at = (uint64_t)(first_output + o) * inputs + chunk * DENSE_CHUNK_INPUTS;
-            if constexpr (TYPE == DENSE_FLOAT32) {
-                const float4_t low = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at);
-                const float4_t high = *(const float4_t *)((const float *)(arena + arguments.weights_offset) + at + 4u);
-#pragma unroll
-                for (uint32_t i = 0; i < 4u; i++) {
-                    weights[o][i] = low[i];
-                    weights[o][4u + i] = high[i];
-                }
-            } else {
-                unpack_bf16x8(*(const uint4_t *)((const uint16_t *)(arena + arguments.weights_offset) + at), weights[o]);
-            }
-        }
-        float values[ROWS][DENSE_CHUNK_INPUTS];
-#pragma unroll
-        for (uint32_t r = 0; r < ROWS; r++) {
-            unpack_bf16x8(packed[r], values[r]);
-        }
-        if (scaled) {
-#pragma unroll
-            for (uint32_t r = 0; r < ROWS; r++) {
-#pragma unroll
-                for (uint32_t i = 0; i < DENSE_CHUNK_INPUTS; i++) {
-                    squares[r] = __fmaf_rn(values[r][i], values[r][i], squares[r]);
-                }
-            }
-        }
-#pragma unroll
-        for (uint32_t o = 0; o < OUTPUTS; o++) {
-#pragma unroll
-            for (uint32_t r = 0; r < ROWS; r++) {
-#pragma unroll
-                for (uint32_t i = 0; i < DENSE_CHUNK_INPUTS; i++) {
-                    chain[o][r] = __fmaf_rn(weights[o][i], values[r][i], chain[o][r]);
-                }
-            }
-        }
-    }
-    const uint32_t group = thread / DENSE_GROUP_LANES, lane = thread % DENSE_GROUP_LANES;
-    /* the exchanges of one distance for every chain before the next distance: each chain's additions are the
-     * definition's, and the exchanges of different chains are in flight together */
-#pragma unroll
-    for (uint32_t distance = DENSE_GROUP_LANES / 2u; distance != 0u; distance /= 2u) {
-#pragma unroll
-        for (uint32_t r = 0; r < ROWS; r++) {
-#pragma unroll
-            for (uint32_t o = 0; o < OUTPUTS; o++) {
-                chain[o][r] = __fadd_rn(chain[o][r], __shfl_xor(chain[o][r], (int)distance, (int)DENSE_GROUP_LANES));
-            }
-            if (scaled) {
-                squares[r] = __fadd_rn(squares[r], __shfl_xor(squares[r], (int)distance, (int)DENSE_GROUP_LANES));
-            }
-        }
-    }
-    if (lane == 0u) {
-#pragma unroll
-        for (uint32_t r = 0; r < ROWS; r++) {
-#pragma unroll
-            for (uint32_t o = 0; o < OUTPUTS; o++) {
-                group_sums[group][o][r] = chain[o][r];
-            }
-            if (scaled) {
-                group_sums[group][OUTPUTS][r] = squares[r];
-            }
-        }
-    }
-    __syncthreads();
-    if (thread >= OUTPUTS * ROWS) {
-        return;
-    }
-    const uint32_t o = thread / ROWS, r = thread % ROWS;
-    if (first_row + r >= arguments.row_count) {
-        return;
-    }
-    float sum = 0.0f, square_sum = 0.0f;
-#pragma unroll
-    for (uint32_t g = 0; g < DENSE_GROUPS; g++) {
-        sum = __fadd_rn(sum, group_sums[g][o][r]);
-        if (scaled) {
-            square_sum = __fadd_rn(square_sum, group_sums[g][OUTPUTS][r]);
-        }
-    }
-    if (scaled) {
-        const float operand = __fadd_rn(__fmul_rn(square_sum, __fdiv_rn(1.0f, (float)inputs)), arguments.epsilon);
-        sum = __fmul_rn(sum, dense_reciprocal_root(operand));
-    }
-    const uint64_t index = (uint64_t)(first_row + r) * arguments.output_size + first_output + o;
-    if (arguments.output_type == DENSE_FLOAT32) {
-        ((float *)(arena + arguments.output_offset))[index] = __fmul_rn(sum, arguments.output_scale);
-    } else {
-        ((uint16_t *)(arena + arguments.output_offset))[index] = float_to_bf16(__fmul_rn(bf16_to_float(float_to_bf16(sum)), arguments.output_scale));
-    }
+    dense_linear_body<TYPE, ROWS, OUTPUTS>(arguments, arena, (const uint16_t *)(arena + arguments.rows_offset), output_group * OUTPUTS,
+                                           row_group * ROWS, threadIdx.x, true, lds);
 }
 
 #define DENSE_STAMP(name, type, rows, outputs, form)                                                                                  \

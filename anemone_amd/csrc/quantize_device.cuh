@@ -106,4 +106,40 @@ __device__ static __forceinline__ void quantize_value(uint32_t bits, uint32_t in
     }
 }
 
+/* thread q of a vector's width / 4 (four values, a word of codes) of vector `vector`: activation_quantize_entry's work of
+ * one thread; the eight threads of a block of 32 values are neighbours in one wavefront and call together */
+__device__ static __forceinline__ void activation_quantize_body(const struct activation_quantize_arguments &arguments, unsigned char *arena,
+                                                                uint32_t q, uint64_t vector)
+{
+    /* thread q = (16 l + 4 s + t) takes the four values 64 l + 16 s + 2 t + {0, 1, 8, 9}: the four codes of one word of
+     * the lane order and the four operands of one pair of words; the 32 values of a block of the quantization are those
+     * of eight neighbouring threads (s = 2 b, 2 b + 1; t = 0 .. 3) */
+    const uint32_t l = q / 16u, s = (q / 4u) % 4u, t = q % 4u, first = 64u * l + 16u * s + 2u * t;
+    if (first >= arguments.width) {
+        return; /* the width is a multiple of 64: whole groups of sixteen threads leave together */
+    }
+    const uint16_t *values = (const uint16_t *)(arena + arguments.values_offset) + vector * arguments.width + first;
+    const uint32_t near_pair = *(const uint32_t *)values, far_pair = *(const uint32_t *)(values + 8);
+    const uint32_t bits[4] = {near_pair & 0xFFFFu, near_pair >> 16, far_pair & 0xFFFFu, far_pair >> 16}; /* values +0, +1, +8, +9 */
+    float largest = fmaxf(fmaxf(fabsf(bf16_to_float((uint16_t)bits[0])), fabsf(bf16_to_float((uint16_t)bits[1]))),
+                          fmaxf(fabsf(bf16_to_float((uint16_t)bits[2])), fabsf(bf16_to_float((uint16_t)bits[3]))));
+#pragma unroll
+    for (uint32_t distance = 4u; distance != 0u; distance >>= 1u) {
+        largest = fmaxf(largest, __shfl_xor(largest, (int)distance, 8));
+    }
+    const uint32_t code_exponent = quantize_exponent_code(largest);
+    /* the word's bytes j = 0 .. 3 hold values +0 (j = 0), +8 (1), +1 (2), +9 (3); its operands' halfwords 2 r + h hold
+     * value + h + 8 r */
+    const uint32_t in_word_order[4] = {bits[0], bits[2], bits[1], bits[3]};
+    uint32_t codes, carried[4];
+    quantize_codes4(in_word_order, code_exponent, codes, carried);
+    const uint32_t word = quantize_word_of(l, s, t);
+    *(uint32_t *)(arena + arguments.codes_offset + vector * arguments.width + word) = codes;
+    *(uint2_t *)((uint16_t *)(arena + arguments.operands_offset) + vector * arguments.width + word) =
+        (uint2_t){quantize_operand_pair(carried[0], carried[2], code_exponent), quantize_operand_pair(carried[1], carried[3], code_exponent)};
+    if (q % 8u == 0u) {
+        (arena + arguments.exponents_offset)[vector * (arguments.width / 32u) + first / 32u] = (unsigned char)code_exponent;
+    }
+}
+
 #endif

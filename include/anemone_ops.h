@@ -214,6 +214,37 @@ MUST_CHECK result_status router_wide_small_prepare(const struct router_wide_desc
                                                    const struct router_kernels_record *kernels,
                                                    struct kernel_launch *launches_out);
 
+/* ---- the fused fronts of a block's sites (include/anemone/site_front.h:38-40, 42-75 of the reference) ---- */
+struct site_front_kernels {
+    uint32_t fronts[SITE_FRONT_INSTANCES]; /* site_front_1, _8, ffn_front_1, _8; the input and coefficient fronts: BACKEND_NO_KERNEL */
+};
+MUST_CHECK result_status site_front_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                                    struct site_front_kernels *kernels_out);
+struct site_front_description {
+    struct linear_range streams;     /* read: bf16 [row][4][width] */
+    struct linear_range carried_pre; /* read, then written */
+    struct linear_range mix_weights; /* read: float32 [24][4 width], exactly */
+    struct linear_range scale;       /* read: float32 [3], exactly */
+    struct linear_range base;        /* read: float32 [24], exactly */
+    struct linear_range norm_weight; /* read: bf16 [width], exactly */
+    struct linear_range post;        /* written */
+    struct linear_range comb;        /* written */
+    struct linear_range hidden;      /* written: the sublayer's input */
+    struct linear_range codes;       /* written: [row_count][width] */
+    struct linear_range exponents;   /* written: [row_count][width / 32] */
+    struct linear_range operands;    /* written: [row_count][width] */
+    struct linear_range scratch;     /* struct site_front_scratch, its counters zero */
+    const struct router_description *router; /* the FFN front's select (its scores written too), or NULL */
+    struct linear_range router_weights;      /* read by the FFN front: bf16 [experts][width], exactly */
+    uint32_t kind;                   /* enum site_front_kind; FFN exactly where router is given */
+    uint32_t row_count;
+    uint32_t reserved_zero;          /* the width; 0: 5,120 (the reference's model) */
+};
+/* fills ONE launch; the site front cut in two (SITE_FRONT_KIND_INPUT, _COEFFICIENTS) is not built: STATUS_UNSUPPORTED */
+MUST_CHECK result_status site_front_prepare(const struct site_front_description *description, uint64_t arena_byte_count,
+                                            const struct router_kernels_record *router_kernels,
+                                            const struct site_front_kernels *kernels, struct kernel_launch *launch_out);
+
 /* ---- FP4 / FP8 expert linears of the original weights (the routed part of the reference's linear.h) ---- */
 #define LINEAR_SLICE_INSTANCES 5u /* product kernels are stamped for 1, 2, 4, 8, 16 slices; gfx950 holds 1, 2, 4, 8 */
 #define LINEAR_MAXIMUM_SLICES 16u

@@ -681,4 +681,102 @@ struct dense_linear_arguments {
 };
 ANEMONE_RECORD_HAS(dense_linear_arguments, 64);
 
+/* ---- the fused fronts of a block's sites (include/anemone/site_front_records.h of the reference): a site's mix project,
+ * its mix finish and the quantization of the sublayer's input in ONE launch (site_front_<R>); the FFN front also the
+ * router's scores, in the dense product's order, and its select between the finish and the quantization
+ * (ffn_front_<R>). R = 1 for one row, 8 for 2 to 8 rows. Every output has the bits of the launches the front stands for.
+ *
+ * A front is a grid of blocks of width / 8 threads that take tickets from the scratch's first counter and their parts in
+ * the tickets' order: the rows' blocks first (a row's input from its streams and the carried pre, and its quantization:
+ * they wait for nothing), then the mix project's blocks (the last of them to publish its mixes waits for the rows' blocks,
+ * which read the pre it writes, and forms every row's post, comb and pre), then the scores' blocks (they wait for the
+ * rows' inputs; the last of them to publish its scores runs the select). A block waits only for blocks of lower tickets,
+ * which are running and wait for nothing: the grid ends whatever part of it the card holds at once. No floating-point
+ * result depends on the tickets. The last block to leave puts every counter back to zero. The input and coefficient
+ * fronts of the reference (the site front cut in two launches) are not built.
+ *
+ * The record is the reference's, 192 bytes: its router_select_arguments (80 bytes there) first, then the fourteen
+ * offsets. What this build's select takes beside the reference's members (expert count, picks a row, affinity kind, route
+ * scale) rides in the word of reference_order: bit 0 reference_order, bits 1-10 the expert count (0: 384), bits 11-14 the
+ * picks (0: 6), bit 15 the affinity kind, bits 16-31 the route scale as fp16 (0: 1.5): all zero is the reference's model. */
+#define KERNEL_FILE_SITE_FRONT "kernel_site_front"
+#define KERNEL_SITE_FRONT_STEM "site_front_"
+#define KERNEL_FFN_FRONT_STEM "ffn_front_"
+#define SITE_FRONT_ARGUMENT_BYTES 192u
+#define SITE_FRONT_SCRATCH_BYTES 7184u
+#define SITE_FRONT_MOST_WIDTH 5120u /* blocks of width / 8 threads whose 8-row dense products need 168 registers */
+#define SITE_FRONT_SCORE_OUTPUTS 4u /* experts of a block's quarter (256 threads: the dense product's block) */
+#define SITE_FRONT_MIX_OUTPUTS 2u   /* mixes of a block's quarter */
+#define SITE_FRONT_WAIT_POLLS (1u << 20) /* of a counter, some 100 ns apart; then the block gives up (scratch.gave_up) and leaves */
+enum site_front_kind {
+    SITE_FRONT_KIND_SITE = 0,
+    SITE_FRONT_KIND_FFN = 1,
+    SITE_FRONT_KIND_INPUT = 2,        /* not built */
+    SITE_FRONT_KIND_COEFFICIENTS = 3, /* not built */
+    SITE_FRONT_KINDS = 4
+};
+#define SITE_FRONT_ROW_FORMS 2u /* one row, 8 */
+#define SITE_FRONT_INSTANCES (SITE_FRONT_KINDS * SITE_FRONT_ROW_FORMS)
+
+struct site_front_select {
+    uint64_t step_offset;
+    uint64_t scores_offset;          /* the FFN front: written, then read */
+    uint64_t bias_offset;
+    uint64_t expert_offsets_offset;
+    uint64_t affinities_offset;
+    uint64_t jobs_offset;
+    uint64_t weights_offset;
+    uint64_t gate_up_last_offset;
+    uint64_t down_last_offset;
+    uint32_t row_count;              /* the site front reads nothing else of the select */
+    uint32_t reference_order_and_shape;
+};
+ANEMONE_RECORD_HAS(site_front_select, 80);
+
+ANEMONE_INLINE uint32_t site_front_shape_word(uint32_t reference_order, uint32_t expert_count, uint32_t pick_count, uint32_t affinity_kind,
+                                              uint32_t route_scale_fp16)
+{
+    return (reference_order & 1u) | ((expert_count & 1023u) << 1) | ((pick_count & 15u) << 11) | ((affinity_kind & 1u) << 15) |
+           (route_scale_fp16 << 16);
+}
+
+/* the blocks of a front of blocks of width / 8 threads: a quarter (256 threads) takes SITE_FRONT_MIX_OUTPUTS mixes or
+ * SITE_FRONT_SCORE_OUTPUTS experts, a block as many quarters as it holds whole */
+ANEMONE_INLINE uint32_t site_front_mix_blocks(uint32_t width)
+{
+    return (MODEL_MIXES / SITE_FRONT_MIX_OUTPUTS + width / 2048u - 1u) / (width / 2048u);
+}
+ANEMONE_INLINE uint32_t site_front_score_blocks(uint32_t width, uint32_t expert_count)
+{
+    return (expert_count / SITE_FRONT_SCORE_OUTPUTS + width / 2048u - 1u) / (width / 2048u);
+}
+
+struct site_front_arguments {
+    struct site_front_select select;
+    uint64_t streams_offset;        /* read: bf16 [row][4][width] */
+    uint64_t pre_offset;            /* read, then written: the carried pre, then the site's */
+    uint64_t scale_offset;          /* read: float32 [3] */
+    uint64_t base_offset;           /* read: float32 [24] */
+    uint64_t post_offset;           /* written */
+    uint64_t comb_offset;           /* written */
+    uint64_t norm_weight_offset;    /* read: bf16 [width] */
+    uint64_t hidden_offset;         /* written (and read by the FFN front's scores) */
+    uint64_t mix_weights_offset;    /* read: float32 [24][4 width] */
+    uint64_t codes_offset;          /* written: codes [row_count][width] */
+    uint64_t exponents_offset;      /* written: exponents [row_count][width / 32] */
+    uint64_t operands_offset;       /* written: operands [row_count][width] */
+    uint64_t scratch_offset;        /* struct site_front_scratch: its mixes written, its counters zero again */
+    uint64_t router_weights_offset; /* read by the FFN front: bf16 [experts][width] */
+};
+ANEMONE_RECORD_HAS(site_front_arguments, SITE_FRONT_ARGUMENT_BYTES);
+
+struct site_front_scratch {
+    uint32_t tickets, arrived, rows_ready, scored; /* zero before a launch and after it */
+    float mixes[LINEAR_MAXIMUM_ROWS][MODEL_MIXES]; /* the launch's rows' */
+    uint32_t departed;                             /* zero before a launch and after it */
+    uint32_t gave_up;                              /* blocks that waited SITE_FRONT_WAIT_POLLS polls in vain: zero on a sound card */
+    uint32_t reserved[62 + MODEL_MIXES * 8u * LINEAR_MAXIMUM_ROWS]; /* where the reference's blocks leave their partial sums */
+};
+ANEMONE_RECORD_HAS(site_front_scratch, SITE_FRONT_SCRATCH_BYTES);
+
 #endif

@@ -289,6 +289,81 @@ def test_router_prepare(fake):
     assert lib.router_select_prepare(C.byref(six), ARENA, C.byref(kernels), launch) == 0
 
 
+def front_description(fake, width=4096, rows=8, ffn=False, **changes):
+    d = amd.SiteFrontDescription()
+    at = 1 << 21
+    for name, size in (("streams", rows * 4 * width * 2), ("carried_pre", rows * 16), ("mix_weights", 24 * 4 * width * 4), ("scale", 12), ("base", 96),
+                       ("norm_weight", width * 2), ("post", rows * 16), ("comb", rows * 64), ("hidden", rows * width * 2), ("codes", rows * width),
+                       ("exponents", rows * width // 32), ("operands", rows * width * 2), ("scratch", amd.SITE_FRONT_SCRATCH_BYTES)):
+        setattr(d, name, amd.Range(at, size))
+        at += (size + 255) // 256 * 256
+    d.kind, d.row_count, d.reserved_zero = (amd.SITE_FRONT_KIND_FFN if ffn else amd.SITE_FRONT_KIND_SITE), rows, width
+    keep = []
+    if ffn:
+        router, experts, offsets = router_description(fake)
+        d.router = C.pointer(router)
+        d.router_weights = amd.Range(at, 256 * width * 2)
+        keep = [router, experts, offsets]
+    for key, value in changes.items():
+        setattr(d, key, value)
+    return d, keep
+
+
+def test_site_front_prepare(fake):
+    """One launch of blocks of width / 8 threads (the rows', the mix project's, the scores'); the FFN front's record carries the router select's record; the
+    reference's refusals (site_front.h:42-75) and this build's (the front cut in two; widths above 5,120)."""
+    lib = amd.library()
+    kernels, router_kernels = amd.SiteFrontKernels(), amd.RouterKernels()
+    assert lib.site_front_kernels_prepare(fake.address, fake.card, C.byref(kernels)) == 0
+    assert lib.router_kernels_prepare(fake.address, fake.card, C.byref(router_kernels)) == 0
+    assert [fake.handles[k][1] for k in kernels.fronts[0:4]] == ["site_front_1", "site_front_8", "ffn_front_1", "ffn_front_8"]
+    assert list(kernels.fronts[4:8]) == [amd.BACKEND_NO_KERNEL] * 4
+    launch = amd.launches_of(1)
+    d, keep = front_description(fake)
+    assert lib.site_front_prepare(C.byref(d), ARENA, None, C.byref(kernels), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "site_front_8" and list(launch[0].grid) == [8 + 6, 1, 1] and launch[0].block[0] == 512
+    assert launch[0].argument_byte_count == 192
+    record = np.frombuffer(bytes(launch[0].argument)[:192], dtype=np.uint64)
+    assert record[9] == 8 and record[10] == d.streams.byte_offset and record[22] == d.scratch.byte_offset and record[23] == 0
+    one, keep = front_description(fake, width=5120, rows=1, reserved_zero=0)
+    assert lib.site_front_prepare(C.byref(one), ARENA, None, C.byref(kernels), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "site_front_1" and list(launch[0].grid) == [1 + 6, 1, 1] and launch[0].block[0] == 640
+    f, keep = front_description(fake, ffn=True)
+    assert lib.site_front_prepare(C.byref(f), ARENA, C.byref(router_kernels), C.byref(kernels), launch) == 0
+    assert fake.handles[launch[0].kernel][1] == "ffn_front_8" and list(launch[0].grid) == [8 + 6 + 32, 1, 1]
+    select = amd.launches_of(1)
+    assert lib.router_select_prepare(C.byref(keep[0]), ARENA, C.byref(router_kernels), select) == 0
+    assert bytes(launch[0].argument)[:72] == bytes(select[0].argument)[:72], "the select's nine offsets are the front's"
+    words = np.frombuffer(bytes(launch[0].argument)[72:80], dtype=np.uint32)
+    assert words[0] == 8 and words[1] == (0 | 256 << 1 | 8 << 11 | 1 << 15 | 0x3E00 << 16)
+    assert np.frombuffer(bytes(launch[0].argument)[:192], dtype=np.uint64)[23] == f.router_weights.byte_offset
+    refusals = [(dict(kind=amd.SITE_FRONT_KIND_INPUT), False, 7), (dict(kind=amd.SITE_FRONT_KIND_COEFFICIENTS), False, 7), (dict(kind=4), False, 1),
+                (dict(row_count=0), False, 1), (dict(row_count=9), False, 1), (dict(reserved_zero=6144), False, 1), (dict(reserved_zero=1024), False, 1),
+                (dict(reserved_zero=4100), False, 1), (dict(reserved_zero=2304), False, 1), (dict(kind=amd.SITE_FRONT_KIND_FFN), False, 1), (dict(kind=amd.SITE_FRONT_KIND_SITE), True, 1),
+                (dict(hidden=amd.Range(1 << 21, 8 * 4096 * 2)), False, 1), (dict(scale=amd.Range(1 << 30, 16)), False, 1),
+                (dict(scratch=amd.Range(1 << 30, 64)), False, 1), (dict(codes=amd.Range(ARENA - 256, 8 * 4096)), False, 1),
+                (dict(row_count=4), True, 1), (dict(router_weights=amd.Range(4096, 256 * 4096 * 2)), True, 1)]
+    for changes, ffn, status in refusals:
+        bad, keep = front_description(fake, ffn=ffn, **changes)
+        untouched = amd.launches_of(1)
+        assert lib.site_front_prepare(C.byref(bad), ARENA, C.byref(router_kernels) if ffn else None, C.byref(kernels), untouched) == status, changes
+        assert not any(bytes(untouched)), changes
+    # a route scale that fp16 does not hold, a router the select refuses
+    for changes in (dict(route_scale=1.1), dict(pick_count=9)):
+        bad, keep = front_description(fake, ffn=True)
+        setattr(keep[0], *list(changes.items())[0])
+        untouched = amd.launches_of(1)
+        assert lib.site_front_prepare(C.byref(bad), ARENA, C.byref(router_kernels), C.byref(kernels), untouched) == 1 and not any(bytes(untouched))
+    # a front without its kernel, missing arguments
+    none = amd.SiteFrontKernels()
+    for i in range(8):
+        none.fronts[i] = amd.BACKEND_NO_KERNEL
+    d, keep = front_description(fake)
+    assert lib.site_front_prepare(C.byref(d), ARENA, None, C.byref(none), launch) == 1
+    assert lib.site_front_prepare(None, ARENA, None, C.byref(kernels), launch) == 1
+    assert lib.site_front_kernels_prepare(fake.address, fake.card, None) == 1
+
+
 # ---- the wide select, the prefill form, the FP4 / FP8 experts: geometry and refusals ----
 
 def wide_description(**changes):
