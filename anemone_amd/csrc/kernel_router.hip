@@ -244,36 +244,28 @@ extern "C" __global__ void __launch_bounds__(SELECT_THREADS)
     router_wide_select(struct router_wide_arguments arguments, unsigned char *arena)
 {
     __shared__ float affinities[LINEAR_MAXIMUM_ROWS * ROUTER_MOST_EXPERTS];
-    __shared__ float pick_weights[LINEAR_MAXIMUM_ROWS * ROUTER_MOST_PICKS];
-    __shared__ uint32_t pick_experts[LINEAR_MAXIMUM_ROWS * ROUTER_MOST_PICKS];
-    const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
-    const uint32_t live_rows = wide_live_rows(arguments, arena);
-    const uint32_t first_row = blockIdx.x * LINEAR_MAXIMUM_ROWS;
-    if (first_row >= live_rows) {
-        return;
-    }
-    const uint32_t rows = live_rows - first_row < LINEAR_MAXIMUM_ROWS ? live_rows - first_row : LINEAR_MAXIMUM_ROWS;
+    const uint32_t experts = arguments.expert_count, picks = arguments.pick_count, places = experts / WAVE;
     const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    float bias_of[ROUTER_MOST_EXPERTS / WAVE]; /* the lane's bias values, asked for ahead of the affinities */
+    const uint32_t row = blockIdx.x * LINEAR_MAXIMUM_ROWS + wave;
+    /* asked for together: the step's rows, the lane's bias values and scores (the row is inside the scores' array or the
+     * wavefront reads row 0's) */
+    const uint32_t live_rows = wide_live_rows(arguments, arena);
+    const uint64_t first = (uint64_t)(row < arguments.row_count ? row : 0u) * experts;
+    float bias_of[ROUTER_PLACES], scores[ROUTER_PLACES];
 #pragma unroll
-    for (uint32_t place = 0; place < ROUTER_MOST_EXPERTS / WAVE; place++) {
-        bias_of[place] = lane + place * WAVE < experts ? ((const float *)(arena + arguments.bias_offset))[lane + place * WAVE] : 0.0f;
+    for (uint32_t place = 0; place < ROUTER_PLACES; place++) {
+        bias_of[place] = place < places ? ((const float *)(arena + arguments.bias_offset))[lane + place * WAVE] : 0.0f;
+        scores[place] = place < places ? ((const float *)(arena + arguments.scores_offset))[first + lane + place * WAVE] : 0.0f;
     }
-    for (uint32_t index = threadIdx.x; index < rows * experts; index += blockDim.x) {
-        const uint64_t at = (uint64_t)first_row * experts + index;
-        const float a = router_affinity(((const float *)(arena + arguments.scores_offset))[at], arguments.affinity_kind);
-        affinities[index] = a;
-        ((float *)(arena + arguments.affinities_offset))[at] = a;
+    if (row >= live_rows) {
+        return; /* no barrier in this kernel: a wavefront is a row */
     }
-    __syncthreads();
-    if (wave < rows) {
-        router_row(affinities + wave * experts, bias_of, lane, experts, picks,
-                   arguments.reference_order, arguments.route_scale, pick_experts + wave * picks, pick_weights + wave * picks);
-    }
-    __syncthreads();
-    struct router_pick *out = (struct router_pick *)(arena + arguments.picks_offset) + (uint64_t)first_row * picks;
-    for (uint32_t index = threadIdx.x; index < rows * picks; index += blockDim.x) {
-        out[index] = (struct router_pick){pick_experts[index], pick_weights[index]};
+    struct router_pick my_pick;
+    uint32_t my_slot;
+    router_row_any(scores, bias_of, experts, affinities + wave * experts, (float *)(arena + arguments.affinities_offset) + first, lane,
+                   arguments.affinity_kind, picks, arguments.reference_order, arguments.route_scale, my_pick.expert, my_slot, my_pick.route_weight);
+    if (lane < picks) { /* lane p holds pick p */
+        ((struct router_pick *)(arena + arguments.picks_offset))[(uint64_t)row * picks + my_slot] = my_pick;
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_select, router_wide_arguments);

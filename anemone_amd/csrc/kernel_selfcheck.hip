@@ -1,6 +1,6 @@
 /*
  * kernel_selfcheck.hip -- the library's check of its own short cuts in arithmetic. Two helpers of the kernels take a
- * shorter way than the arithmetic they are defined by: det_silu (no tests around the exponential) and quantize_codes4
+ * shorter way than the arithmetic they are defined by: det_silu and det_sigmoid (no tests around the exponential) and quantize_codes4
  * (the card's FP8 conversions). This kernel runs both ways over every input there is and counts the disagreements, so
  * that a test on the card proves the two ways equal instead of sampling them. No counterpart in the reference; not on
  * the routed-expert path.
@@ -10,10 +10,11 @@
 
 #include "kernel_registry.h"
 #include "quantize_device.cuh"
+#include "router_device.cuh"
 
 struct arithmetic_selfcheck_arguments {
     uint64_t output_offset; /* written: uint32 [threads of the grid][2]: disagreements, and the first input that disagreed */
-    uint32_t check;         /* 0: det_silu over all 2^32 float32; 1: quantize_codes4 over all 2^16 values x 2^8 scale codes */
+    uint32_t check;         /* 0: det_silu over all 2^32 float32; 1: quantize_codes4 over all 2^16 values x 2^8 scale codes; 2: det_sigmoid */
     uint32_t reserved_zero;
 };
 static_assert(sizeof(struct arithmetic_selfcheck_arguments) == 16, "arithmetic_selfcheck_arguments ABI");
@@ -26,6 +27,15 @@ extern "C" __global__ void arithmetic_selfcheck(struct arithmetic_selfcheck_argu
         for (uint64_t pattern = thread; pattern < (1ull << 32); pattern += threads) {
             const float gate = __uint_as_float((uint32_t)pattern);
             const float defined = __fdiv_rn(gate, __fadd_rn(1.0f, det_expf(-gate))), taken = det_silu(gate);
+            const bool same = __float_as_uint(defined) == __float_as_uint(taken) || (defined != defined && taken != taken);
+            if (!same && disagreements++ == 0u) {
+                first = (uint32_t)pattern;
+            }
+        }
+    } else if (arguments.check == 2u) {
+        for (uint64_t pattern = thread; pattern < (1ull << 32); pattern += threads) {
+            const float score = __uint_as_float((uint32_t)pattern);
+            const float defined = __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-score))), taken = det_sigmoid(score);
             const bool same = __float_as_uint(defined) == __float_as_uint(taken) || (defined != defined && taken != taken);
             if (!same && disagreements++ == 0u) {
                 first = (uint32_t)pattern;

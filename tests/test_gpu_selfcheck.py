@@ -1,5 +1,5 @@
 """The library's check of its own arithmetic short cuts, run on the card over every input there is: det_silu against
-gate / (1 + det_expf(-gate)) for all 2^32 float32 gates, and the quantizer by the card's FP8 conversions
+gate / (1 + det_expf(-gate)) for all 2^32 float32 gates (det_sigmoid likewise against 1 / (1 + det_expf(-score))), and the quantizer by the card's FP8 conversions
 (quantize_codes4) against the quantizer's defining arithmetic (source/kernel_activation_quantize.cuh:52-133 of the
 reference, which tests/test_gpu_linear.py holds byte for byte to the CPU oracle) for all 2^16 bfloat16 values under
 all 2^8 scale codes. A disagreement names its first input."""
@@ -13,7 +13,8 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("check,what", [(0, "det_silu over all float32"), (1, "quantize_codes4 over all values and scale codes")])
+@pytest.mark.parametrize("check,what", [(0, "det_silu over all float32"), (1, "quantize_codes4 over all values and scale codes"),
+                                        (2, "det_sigmoid over all float32")])
 def test_short_cuts_equal_their_definitions(check, what):
     import anemone_amd as amd
     print("selfcheck", check, what, flush=True)
