@@ -27,6 +27,7 @@
 #define EXACT_WEIGHTS true
 #define PRODUCT_WAVES 4u
 #define PRODUCT_THREADS (PRODUCT_WAVES * WAVE)
+#define COMBINE_THREADS (ROUTER_MOST_PICKS * WAVE) /* a wavefront a slot of the row */
 
 struct tc_shape {
     uint32_t hidden, intermediate, picks, pairs;
@@ -199,92 +200,102 @@ extern "C" __global__ void exl3_tc_activate(struct exl3_tc_record record, unsign
 }
 ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_activate, exl3_tc_record);
 
-/* launch 4: grid (hidden / 128, row_count), block 64: a row's pairs in slot order */
-extern "C" __global__ void exl3_tc_combine(struct exl3_tc_record record, unsigned char *arena)
+/* launch 4: grid (hidden / 128, row_count), block 64 x ROUTER_MOST_PICKS: wavefront s takes the row's pair of slot s
+ * (its down sums in slice order, the output transform, the output scales, the route weight); wavefront 0 then adds the
+ * slots' values in slot order. A wavefront runs one instruction at a time: eight slots side by side are an eighth of
+ * the instructions one wavefront would run for the row. */
+extern "C" __global__ void __launch_bounds__(COMBINE_THREADS) exl3_tc_combine(struct exl3_tc_record record, unsigned char *arena)
 {
+    __shared__ float values[ROUTER_MOST_PICKS][EXL3_TRANSFORM];
+    __shared__ uint32_t is_held[ROUTER_MOST_PICKS];
     const tc_shape shape = tc_shape_of(record);
-    const uint32_t lane = threadIdx.x, channel = blockIdx.x * EXL3_TRANSFORM + lane, row = blockIdx.y;
+    const uint32_t lane = threadIdx.x % WAVE, slot = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const uint32_t channel = blockIdx.x * EXL3_TRANSFORM + lane, row = blockIdx.y;
     const uint32_t H = shape.hidden, I = shape.intermediate;
     const struct expert_job_record *jobs = (const struct expert_job_record *)(arena + record.jobs_offset);
     const unsigned char *workspace = arena + record.workspace_offset;
     const float *partials = (const float *)(workspace + exl3_tc_operand_bytes(shape.pairs, H) + exl3_tc_gate_up_bytes(shape.pairs, I));
-    /* the job and column that hold each of the row's pairs: every lane looks once at the jobs lane, lane + 64, ...
-     * (the eight pair indexes of a job as two 16-byte loads); a pair is held at most once, so the lane that found a
-     * slot's is read off a ballot */
-    uint32_t found[ROUTER_MOST_PICKS];
-#pragma unroll
-    for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
-        found[slot] = 0xFFFFFFFFu;
-    }
-    static_assert(LINEAR_MAXIMUM_ROWS == 8u, "a job's pair indexes are two loads of four");
-    for (uint32_t base = 0; base < record.job_capacity; base += WAVE) {
-        const uint32_t index = base + lane;
-        uint32_t mine[ROUTER_MOST_PICKS];
-#pragma unroll
-        for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
-            mine[slot] = 0xFFFFFFFFu;
-        }
-        if (index < record.job_capacity) {
-            const struct expert_job_record *job = jobs + index;
-            const uint32_t count = job->row_count;
-            const uint4_t low = *(const uint4_t *)&job->pair_index[0], high = *(const uint4_t *)&job->pair_index[4];
-            const uint32_t held[LINEAR_MAXIMUM_ROWS] = {low.x, low.y, low.z, low.w, high.x, high.y, high.z, high.w};
-#pragma unroll
-            for (uint32_t column = 0; column < LINEAR_MAXIMUM_ROWS; column++) {
-                if (column < count && held[column] / shape.picks == row) {
-                    const uint32_t slot = held[column] % shape.picks;
-#pragma unroll
-                    for (uint32_t target = 0; target < ROUTER_MOST_PICKS; target++) {
-                        mine[target] = target == slot ? index * LINEAR_MAXIMUM_ROWS + column : mine[target];
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
-            const uint64_t holders = __builtin_amdgcn_ballot_w64(mine[slot] != 0xFFFFFFFFu);
-            if (holders != 0u) { /* the same in every lane */
-                found[slot] = (uint32_t)__builtin_amdgcn_readlane((int)mine[slot], (int)__builtin_ctzll(holders));
-            }
-        }
-    }
-    /* every slot's loads are asked for before the first is used; the sums then run in slot order */
-    float partial0[ROUTER_MOST_PICKS][EXL3_TC_DOWN_SLICES], partial1[ROUTER_MOST_PICKS][EXL3_TC_DOWN_SLICES];
-    float weight[ROUTER_MOST_PICKS], scale0[ROUTER_MOST_PICKS], scale1[ROUTER_MOST_PICKS];
-#pragma unroll
-    for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
-        if (slot < shape.picks && found[slot] != 0xFFFFFFFFu) {
-            const uint32_t pair = row * shape.picks + slot;
-            const struct expert_job_record *job = jobs + found[slot] / LINEAR_MAXIMUM_ROWS;
-            weight[slot] = job->route_weight[found[slot] % LINEAR_MAXIMUM_ROWS];
-            const uint16_t *svh = (const uint16_t *)(arena + job->down_offset + exl3_code_bytes(I, H, tc_bits_x2(record, arena, job->expert, 2u))) + I;
-            scale0[slot] = half_bits_to_float(svh[channel]);
-            scale1[slot] = half_bits_to_float(svh[channel + WAVE]);
-#pragma unroll
-            for (uint32_t slice = 0; slice < EXL3_TC_DOWN_SLICES; slice++) {
-                const float *down = partials + ((uint64_t)slice * shape.pairs + pair) * H;
-                partial0[slot][slice] = down[channel];
-                partial1[slot][slice] = down[channel + WAVE];
-            }
-        }
-    }
-    float sum0 = 0.0f, sum1 = 0.0f;
-#pragma unroll
-    for (uint32_t slot = 0; slot < ROUTER_MOST_PICKS; slot++) {
-        if (slot >= shape.picks || found[slot] == 0xFFFFFFFFu) {
-            continue; /* a pair no job holds (a row beyond the live ones) adds nothing */
-        }
-        float v0 = 0.0f, v1 = 0.0f;
+    bool held = false;
+    float y0 = 0.0f, y1 = 0.0f;
+    if (slot < shape.picks) {
+        const uint32_t pair = row * shape.picks + slot;
+        /* the pair's sums are asked for first: they are inside the workspace whether a job holds the pair or not */
+        float partial0[EXL3_TC_DOWN_SLICES], partial1[EXL3_TC_DOWN_SLICES];
 #pragma unroll
         for (uint32_t slice = 0; slice < EXL3_TC_DOWN_SLICES; slice++) {
-            v0 = __fadd_rn(v0, partial0[slot][slice]);
-            v1 = __fadd_rn(v1, partial1[slot][slice]);
+            const float *down = partials + ((uint64_t)slice * shape.pairs + pair) * H;
+            partial0[slice] = down[channel];
+            partial1[slice] = down[channel + WAVE];
         }
-        wave_hadamard128(v0, v1, lane);
-        const float y0 = __fmul_rn(__fmul_rn(__fmul_rn(v0, EXL3_NORMALIZATION), scale0[slot]), weight[slot]);
-        const float y1 = __fmul_rn(__fmul_rn(__fmul_rn(v1, EXL3_NORMALIZATION), scale1[slot]), weight[slot]);
-        sum0 = __fadd_rn(sum0, y0);
-        sum1 = __fadd_rn(sum1, y1);
+        /* the job and column that hold the pair: every lane looks at the jobs lane, lane + 64, ... (what it needs of a
+         * job in four 16-byte loads asked for together); a pair is held at most once */
+        static_assert(LINEAR_MAXIMUM_ROWS == 8u && offsetof(struct expert_job_record, down_offset) == 16u &&
+                          offsetof(struct expert_job_record, pair_index) == 32u && sizeof(struct expert_job_record) == 96u,
+                      "a job from its down offset on is five loads of 16 bytes");
+        uint64_t down_offset = 0;
+        uint32_t expert = 0;
+        float weight = 0.0f;
+        for (uint32_t base = 0; base < record.job_capacity && !held; base += WAVE) {
+            const uint32_t index = base + lane;
+            bool mine = false;
+            uint64_t my_offset = 0;
+            uint32_t my_expert = 0;
+            float my_weight = 0.0f;
+            if (index < record.job_capacity) {
+                const uint4_t *job = (const uint4_t *)(jobs + index);
+                const uint4_t head = job[1], low = job[2], high = job[3], weights_low = job[4], weights_high = job[5];
+                const uint32_t count = head.z;
+                const uint32_t indexes[LINEAR_MAXIMUM_ROWS] = {low.x, low.y, low.z, low.w, high.x, high.y, high.z, high.w};
+                const uint32_t weights[LINEAR_MAXIMUM_ROWS] = {weights_low.x, weights_low.y, weights_low.z, weights_low.w,
+                                                               weights_high.x, weights_high.y, weights_high.z, weights_high.w};
+#pragma unroll
+                for (uint32_t column = 0; column < LINEAR_MAXIMUM_ROWS; column++) {
+                    const bool here = column < count && indexes[column] == pair;
+                    mine = mine || here;
+                    my_weight = here ? __uint_as_float(weights[column]) : my_weight;
+                }
+                my_offset = ((uint64_t)head.y << 32) | head.x;
+                my_expert = head.w;
+            }
+            const uint64_t holders = __builtin_amdgcn_ballot_w64(mine);
+            if (holders != 0ull) { /* the same in every lane */
+                const int holder = __builtin_ctzll(holders);
+                held = true;
+                down_offset = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(my_offset >> 32), holder) << 32) |
+                              (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)my_offset, holder);
+                expert = (uint32_t)__builtin_amdgcn_readlane((int)my_expert, holder);
+                weight = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(my_weight), holder));
+            }
+        }
+        if (held) {
+            const uint16_t *svh = (const uint16_t *)(arena + down_offset + exl3_code_bytes(I, H, tc_bits_x2(record, arena, expert, 2u))) + I;
+            const float scale0 = half_bits_to_float(svh[channel]), scale1 = half_bits_to_float(svh[channel + WAVE]);
+            float v0 = 0.0f, v1 = 0.0f;
+#pragma unroll
+            for (uint32_t slice = 0; slice < EXL3_TC_DOWN_SLICES; slice++) { /* in slice order from +0 */
+                v0 = __fadd_rn(v0, partial0[slice]);
+                v1 = __fadd_rn(v1, partial1[slice]);
+            }
+            wave_hadamard128(v0, v1, lane);
+            y0 = __fmul_rn(__fmul_rn(__fmul_rn(v0, EXL3_NORMALIZATION), scale0), weight);
+            y1 = __fmul_rn(__fmul_rn(__fmul_rn(v1, EXL3_NORMALIZATION), scale1), weight);
+        }
+    }
+    values[slot][lane] = y0;
+    values[slot][lane + WAVE] = y1;
+    if (lane == 0u) {
+        is_held[slot] = held ? 1u : 0u;
+    }
+    __syncthreads();
+    if (slot != 0u) {
+        return;
+    }
+    float sum0 = 0.0f, sum1 = 0.0f;
+    for (uint32_t other = 0; other < shape.picks; other++) {
+        if (is_held[other] != 0u) { /* a pair no job holds (a row beyond the live ones) adds nothing */
+            sum0 = __fadd_rn(sum0, values[other][lane]);
+            sum1 = __fadd_rn(sum1, values[other][lane + WAVE]);
+        }
     }
     if (record.shared_sum != 0u) {
         /* the sum joins the shared expert's bfloat16 row, in place: bfloat16(sum + row), one rounding of the float32

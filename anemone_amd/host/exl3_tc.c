@@ -8,7 +8,7 @@
  *   gate/up     exl3_tc_products    (intermediate / 64, job_capacity, 2 S_gu / 4)   256   pass 0
  *   activate    exl3_tc_activate    (intermediate / 128, job_capacity, 1)           64
  *   down        exl3_tc_products    (hidden / 64, job_capacity, S_d / 4)            256   pass 1
- *   combine     exl3_tc_combine     (hidden / 128, row_count, 1)                    64
+ *   combine     exl3_tc_combine     (hidden / 128, row_count, 1)                    512   a wavefront a slot of the row
  * S_gu = EXL3_TC_GATE_UP_SLICES and S_d = EXL3_TC_DOWN_SLICES K slices; every slice is a whole number of steps of four
  * K tiles (64 inputs): slice s takes the steps [steps s / S, steps (s + 1) / S). Hidden and intermediate: multiples of 128.
  */
@@ -93,7 +93,7 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
                                                record->job_capacity, record->row_count};
     const uint32_t grid_z[EXL3_TC_LAUNCHES] = {2u, 2u * EXL3_TC_GATE_UP_SLICES / PRODUCT_WAVES, 1u,
                                                EXL3_TC_DOWN_SLICES / PRODUCT_WAVES, 1u};
-    const uint32_t threads[EXL3_TC_LAUNCHES] = {WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS};
+    const uint32_t threads[EXL3_TC_LAUNCHES] = {WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS * ROUTER_MOST_PICKS};
     _Static_assert(2u * EXL3_TC_GATE_UP_SLICES % PRODUCT_WAVES == 0 && EXL3_TC_DOWN_SLICES % PRODUCT_WAVES == 0,
                    "a block's four wavefronts take four whole items");
     struct kernel_launch launches[EXL3_TC_LAUNCHES];
