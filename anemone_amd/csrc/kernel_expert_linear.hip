@@ -105,7 +105,7 @@ __device__ static __forceinline__ void expert_gate_up(const struct expert_gate_u
             const float g = bf16_to_float(float_to_bf16(gate[v])), u = bf16_to_float(float_to_bf16(up[v]));
             const float bounded_gate = fminf(g, limit);
             const float bounded_up = fminf(fmaxf(u, -limit), limit);
-            const float value = __fmul_rn(__fmul_rn(det_silu(bounded_gate), bounded_up), weight);
+            const float value = __fmul_rn(__fmul_rn(linear_silu(bounded_gate), bounded_up), weight);
             hidden[v] = float_to_bf16(value);
         }
         uint16_t *out = (uint16_t *)(arena + arguments.hidden_offset) + (uint64_t)pair * arguments.output_size +

@@ -11,10 +11,11 @@
 #include "kernel_registry.h"
 #include "quantize_device.cuh"
 #include "router_device.cuh"
+#include "linear_device.cuh"
 
 struct arithmetic_selfcheck_arguments {
     uint64_t output_offset; /* written: uint32 [threads of the grid][2]: disagreements, and the first input that disagreed */
-    uint32_t check;         /* 0: det_silu over all 2^32 float32; 1: quantize_codes4 over all 2^16 values x 2^8 scale codes; 2: det_sigmoid */
+    uint32_t check;         /* 0: det_silu over all 2^32 float32; 1: quantize_codes4 over all 2^16 values x 2^8 scale codes; 2: det_sigmoid; 3: linear_silu within its bound of det_silu */
     uint32_t reserved_zero;
 };
 static_assert(sizeof(struct arithmetic_selfcheck_arguments) == 16, "arithmetic_selfcheck_arguments ABI");
@@ -37,6 +38,16 @@ extern "C" __global__ void arithmetic_selfcheck(struct arithmetic_selfcheck_argu
             const float score = __uint_as_float((uint32_t)pattern);
             const float defined = __fdiv_rn(1.0f, __fadd_rn(1.0f, det_expf(-score))), taken = det_sigmoid(score);
             const bool same = __float_as_uint(defined) == __float_as_uint(taken) || (defined != defined && taken != taken);
+            if (!same && disagreements++ == 0u) {
+                first = (uint32_t)pattern;
+            }
+        }
+    } else if (arguments.check == 3u) {
+        for (uint64_t pattern = thread; pattern < (1ull << 32); pattern += threads) {
+            const float gate = __uint_as_float((uint32_t)pattern);
+            const float defined = det_silu(gate), taken = linear_silu(gate);
+            const bool same = taken == defined || fabsf(taken - defined) <= __fmaf_rn(LINEAR_SILU_BOUND, fabsf(defined), LINEAR_SILU_FLOOR) ||
+                              (defined != defined && taken != taken);
             if (!same && disagreements++ == 0u) {
                 first = (uint32_t)pattern;
             }

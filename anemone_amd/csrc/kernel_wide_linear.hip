@@ -89,7 +89,7 @@ __device__ static __forceinline__ void wide_expert_gate_up(const struct wide_exp
                     const float gate = bf16_to_float(float_to_bf16(gate_sum)), up = bf16_to_float(float_to_bf16(up_sum));
                     const float bounded_gate = fminf(gate, limit);
                     const float bounded_up = fminf(fmaxf(up, -limit), limit);
-                    const float value = __fmul_rn(__fmul_rn(det_silu(bounded_gate), bounded_up), weight);
+                    const float value = __fmul_rn(__fmul_rn(linear_silu(bounded_gate), bounded_up), weight);
                     bits[j][n][v] = float_to_bf16(value);
                     largest[j] = fmaxf(largest[j], fabsf(bf16_to_float((uint16_t)bits[j][n][v])));
                 }

@@ -36,6 +36,21 @@ __device__ static __forceinline__ void load_to_lds_4(const unsigned char *base, 
                  : "memory", "m0");
 }
 
+/* gate / (1 + e^(-gate)) of the FP4 / FP8 experts' hidden step, by the card's own exponential and reciprocal (v_exp_f32,
+ * v_rcp_f32: five instructions where the fixed float32 sequence with an IEEE division is twenty-eight). The reference
+ * takes "the card's expf" here as well (source/kernel_linear_common.cuh:195-202 there): the hidden values are held to a
+ * bound, not to bits, on either side. Within 2^-17 of det_silu's value, relatively (the rounding of gate log2(e) moves
+ * the exponential by |gate| 2^-24 ln 2: 2^-20 down to a gate of -16, 2^-17.6 at -87), plus 2^-119 (below a gate of -87.3
+ * the reciprocal is subnormal and the card gives 0 for a value of at most 1.03e-36), for every float32 gate (the library's
+ * arithmetic_selfcheck kernel runs all 2^32); a not-a-number for a not-a-number, and for -infinity as there. */
+#define LINEAR_SILU_BOUND 7.62939453125e-06f /* 2^-17 */
+#define LINEAR_SILU_FLOOR 1.50463276905252801e-36f /* 2^-119 */
+__device__ static __forceinline__ float linear_silu(float gate)
+{
+    const float e = __builtin_amdgcn_exp2f(__fmul_rn(gate, -1.44269502162933349609375f));
+    return __fmul_rn(gate, __builtin_amdgcn_rcpf(__fadd_rn(1.0f, e)));
+}
+
 /* wait until at most `count` of the wavefront's memory loads are outstanding (they retire in order); also a fence
  * for the compiler: LDS reads of a stage stay behind the wait for the loads that fill it */
 template <uint32_t count>

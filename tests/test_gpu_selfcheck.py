@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("check,what", [(0, "det_silu over all float32"), (1, "quantize_codes4 over all values and scale codes"),
-                                        (2, "det_sigmoid over all float32")])
+                                        (2, "det_sigmoid over all float32"), (3, "linear_silu within 2^-17 of det_silu over all float32")])
 def test_short_cuts_equal_their_definitions(check, what):
     import anemone_amd as amd
     print("selfcheck", check, what, flush=True)
