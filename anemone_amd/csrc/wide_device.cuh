@@ -38,12 +38,12 @@ struct wide_chain {
     bool scale_lane; /* lanes 0..15: the ones that bring the scale words of the wavefront's own column block */
     uint32_t read_at[BYTES ? 8 : 4], scale_at[STRIP], vector_at[BYTES ? 8 : 4], vector_scale_at, operand_at, shift;
 
-    __device__ __forceinline__ void issue(uint32_t stage, uint32_t at) const
+    /* the tile's columns of K step `at` into stage `stage` (every wavefront reads them: behind the barrier that ends the
+     * reads of the stage): eight groups of eight columns, two a wavefront: the column block it prepares, and that block's
+     * scale words (every wavefront issues the same number of loads: the waits count them) */
+    __device__ __forceinline__ void issue_vectors(uint32_t stage, uint32_t at) const
     {
-        const uint32_t base = window + stage * STAGE_BYTES, mine = base + wave * WAVE_BYTES;
-        /* first the tile's columns (this wavefront waits for them a step before the weights): eight groups of eight
-         * columns, two a wavefront: the column block it prepares, and that block's scale words (every wavefront issues
-         * the same number of loads: the waits count them) */
+        const uint32_t base = window + stage * STAGE_BYTES;
 #pragma unroll
         for (uint32_t part = 0; part < 2u; part++) {
             load_to_lds_16(codes + (uint64_t)at * 128u, codes_offset[part], base + VECTOR_AT + (2u * wave + part) * 1024u);
@@ -51,6 +51,13 @@ struct wide_chain {
         if (scale_lane) { /* its own sixteen columns' scale words, a lane a column: sixteen cache lines a wavefront, not 64 */
             load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT + wave * 64u);
         }
+    }
+
+    /* the wavefront's own weights and their scales of K step `at` into its part of stage `stage` (no other wavefront
+     * reads that part: once this one has read it, it may be asked for again) */
+    __device__ __forceinline__ void issue_weights(uint32_t stage, uint32_t at) const
+    {
+        const uint32_t mine = window + stage * STAGE_BYTES + wave * WAVE_BYTES;
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
 #pragma unroll
@@ -66,6 +73,12 @@ struct wide_chain {
         for (uint32_t m = 0; m < MATRICES; m++) {
             load_to_lds_4(scales[m] + (uint64_t)at * (BYTES ? 4u : 64u), scale_offset, mine + SCALES_AT + m * 256u);
         }
+    }
+
+    __device__ __forceinline__ void issue(uint32_t stage, uint32_t at) const
+    {
+        issue_vectors(stage, at); /* first: this wavefront waits for them a step before the weights */
+        issue_weights(stage, at);
     }
 
     template <typename T>
@@ -218,17 +231,30 @@ struct wide_chain {
     __device__ __forceinline__ void steps(uint32_t total, float4_t (&chain)[TILES][WIDE_COLUMN_BLOCKS]) const
     {
         if constexpr (DEPTH == 2u) {
-            /* two stages: a step's loads are asked for a step ahead, and its columns prepared once they have landed,
-             * before the barrier that opens the step */
+            /* Two stages. A wavefront's weights of a step are asked for two steps ahead, as soon as the wavefront itself has
+             * read the stage they go to (its part is its own); the tile's columns one step ahead, behind the barrier that
+             * ends every wavefront's reads of their stage; they are prepared once they have landed, before the barrier
+             * that opens their step. Outstanding at the top of step k, oldest first: the weights of k, the columns of k,
+             * the weights of k + 1. */
             issue(0u, 0u);
+            if (total > 1u) {
+                issue_weights(1u, 1u);
+            }
             for (uint32_t step = 0; step < total; step++) {
-                wait_loads<0>();
+                if (step + 1u < total) {
+                    wait_loads<WEIGHT_LOADS>();
+                } else {
+                    wait_loads<0>();
+                }
                 prepare_columns(step % 2u);
                 __syncthreads(); /* every wavefront has read the step before and brought and prepared its part of this one */
                 if (step + 1u < total) {
-                    issue((step + 1u) % 2u, step + 1u);
+                    issue_vectors((step + 1u) % 2u, step + 1u);
                 }
                 consume<LIVE>(step % 2u, chain);
+                if (step + 2u < total) {
+                    issue_weights(step % 2u, step + 2u);
+                }
             }
             return;
         }
