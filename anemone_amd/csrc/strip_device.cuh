@@ -250,14 +250,16 @@ struct strip_chain {
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + ((uint64_t)tile0 * loads + 2u * first) * 32u;
             }
             /* lane L of a 16-byte load lands at bytes 16 L of the tile's stage and asks for the piece
-             * p = L ^ (2 bit4(L) + bit5(L)) of the step: the pieces of one T (p = 32 ld + 4 G + T) then lie in
-             * different LDS banks for the readers, and every 16 lanes still read 256 contiguous bytes of memory */
-            piece_offset = 16u * (lane ^ (2u * ((lane >> 4) & 1u) + ((lane >> 5) & 1u)));
+             * p = L ^ ((L / 8) % 4) of the step: LDS has 32 banks of 4 bytes, and the pieces of one T (p = 32 ld + 4 G + T,
+             * G = 0 .. 7) then lie in eight different groups of four banks for the sixteen lanes that read them together
+             * (measured: SQ_LDS_BANK_CONFLICT of the wide gate/up launch 1.68e8 -> 1.9e7 cycles); every 16 lanes still read
+             * 256 contiguous bytes of memory */
+            piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
             /* scales: uint32 [tile][load][G]; lane L of the 4-byte load: tile L / 16, word L % 16 = 8 ld + G */
             scale_offset = (lane / 16u) * (loads * 32u) + (lane % 16u) * 4u;
 #pragma unroll
             for (uint32_t T = 0; T < 4u; T++) {
-                read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (2u * (G / 4u) + ld))) + 8u * q;
+                read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (G / 2u))) + 8u * q;
             }
 #pragma unroll
             for (uint32_t n = 0; n < STRIP; n++) {

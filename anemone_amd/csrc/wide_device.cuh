@@ -353,12 +353,14 @@ struct wide_chain {
                 words[m] = matrices[m] + (uint64_t)tile0 * steps * STEP_BYTES;
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + (uint64_t)tile0 * loads * 32u;
             }
-            piece_offset = 16u * (lane ^ (2u * ((lane >> 4) & 1u) + ((lane >> 5) & 1u)));
+            /* piece p of a tile's K step lands in slot p ^ ((p / 8) % 4): LDS has 32 banks of 4 bytes, and the eight 8-byte
+             * reads of sixteen lanes (G = 0 .. 7, twice) then fall on sixteen different banks */
+            piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
             /* lanes past the strip's tiles read its last tile's words again */
             scale_offset = (lane / 16u < STRIP ? lane / 16u : STRIP - 1u) * (loads * 32u) + (lane % 16u) * 4u;
 #pragma unroll
             for (uint32_t T = 0; T < 4u; T++) {
-                read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (2u * (G / 4u) + ld))) + 8u * q;
+                read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (G / 2u))) + 8u * q;
             }
 #pragma unroll
             for (uint32_t n = 0; n < STRIP; n++) {
