@@ -465,10 +465,19 @@ void backend_hip_card_close(struct device_card *card, uint64_t wait_limit_nanose
     if (card == nullptr) {
         return;
     }
-    (void)wait_limit_nanoseconds; /* the drain below has no limit of ours, as the reference's has none */
     {
         std::lock_guard<std::mutex> guard(card->mutex);
         (void)hipSetDevice(card->device);
+        /* unfinished work is waited for up to the limit; past it one line is logged and the drain goes on (the arena
+         * cannot be freed under a running launch) */
+        const auto deadline = std::chrono::steady_clock::now() + std::chrono::nanoseconds(wait_limit_nanoseconds);
+        while (hipStreamQuery(card->stream) == hipErrorNotReady) {
+            if (std::chrono::steady_clock::now() >= deadline) {
+                log_error("card_close", "work unfinished at the wait limit: draining the stream");
+                break;
+            }
+            std::this_thread::sleep_for(std::chrono::microseconds(50));
+        }
         if (hipStreamSynchronize(card->stream) != hipSuccess) {
             log_error("card_close", "the drain failed: the card and its arena are retained");
             return;
@@ -663,11 +672,17 @@ result_status backend_hip_launch_run_timed(struct device_card *card, const struc
     if (card_fail(card, "hipSetDevice", hipSetDevice(card->device))) {
         return STATUS_DEVICE_ERROR;
     }
-    std::vector<hipEvent_t> events(launch_count + 1u);
-    for (hipEvent_t &event : events) {
+    std::vector<hipEvent_t> events;
+    events.reserve(launch_count + 1u);
+    for (uint32_t index = 0; index <= launch_count; index++) {
+        hipEvent_t event;
         if (card_fail(card, "hipEventCreate", hipEventCreate(&event))) {
+            for (hipEvent_t created : events) {
+                (void)hipEventDestroy(created);
+            }
             return STATUS_DEVICE_ERROR;
         }
+        events.push_back(event);
     }
     result_status status = STATUS_OK;
     for (uint32_t index = 0; index < launch_count && status == STATUS_OK; index++) {

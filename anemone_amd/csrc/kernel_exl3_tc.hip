@@ -145,7 +145,20 @@ extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS, 4)
     case 5u: tc_item<5u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
     case 6u: tc_item<6u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
     case 8u: tc_item<8u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
-    default: break;
+    default:
+        /* a width this build does not decode (the prepare function refuses the one width of a record; a table's widths
+         * are the caller's): zeros, so that the launches behind this one add nothing stale */
+        if (lane % 16u < job->row_count) {
+            float *out = partials + (uint64_t)job->pair_index[lane % 16u] * outputs;
+#pragma unroll
+            for (uint32_t p = 0; p < STRIP_PAIRS; p++) {
+#pragma unroll
+                for (uint32_t h = 0; h < 2u; h++) {
+                    *(float4_t *)(out + exl3_stream_output(blockIdx.x * 2u * STRIP_PAIRS, p, h, lane)) = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+                }
+            }
+        }
+        break;
     }
 }
 ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_products, exl3_tc_record);

@@ -63,7 +63,9 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
     }
     const uint64_t pairs = (uint64_t)record->row_count * picks;
     const uint64_t workspace = exl3_tc_workspace_bytes(pairs, hidden, I);
-    struct checked_range ranges[5] = {
+    /* the table of per-matrix widths, where one is named: uint32 an expert; the record does not say how many experts there
+     * are, so what is held inside the arena and clear of what the launches write is its first word (an expert 0 there is) */
+    struct checked_range ranges[6] = {
         {"the jobs", {record->jobs_offset, (uint64_t)record->job_capacity * sizeof(struct expert_job_record)},
          (uint64_t)record->job_capacity * sizeof(struct expert_job_record), false},
         {"the rows", {record->hidden_offset, (uint64_t)record->row_count * hidden * 2u}, (uint64_t)record->row_count * hidden * 2u, false},
@@ -78,6 +80,9 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
     if (detached_workspace) { /* the ranges of the arena alone */
         ranges[3] = ranges[4];
         range_count -= 1u;
+    }
+    if (mixed) {
+        ranges[range_count++] = (struct checked_range){"the widths", {record->widths_offset, 4u}, 4u, false};
     }
     if (!ranges_are_valid(what, ranges, range_count, arena_byte_count) || record->workspace_offset % 256u != 0 ||
         (mixed && record->widths_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0)) {
@@ -206,8 +211,9 @@ static result_status tcp_prepare(const struct exl3_tcp_record *record, uint64_t 
         {"the rows", {record->hidden_offset, rows * H * 2u}, rows * H * 2u, false},
         {"the workspace", {record->workspace_offset, layout.total}, layout.total, false},
         {"the output", {record->output_offset, rows * H * 4u}, rows * H * 4u, false},
+        {"the widths", {record->widths_offset, (uint64_t)E * 4u}, (uint64_t)E * 4u, false}, /* where a table is named */
     };
-    if (!ranges_are_valid(what, ranges, 5, arena_byte_count) || record->workspace_offset % 256u != 0 ||
+    if (!ranges_are_valid(what, ranges, mixed ? 6u : 5u, arena_byte_count) || record->workspace_offset % 256u != 0 ||
         (mixed && record->widths_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0)) {
         if (record->workspace_offset % 256u != 0) {
             REFUSE("%s: the workspace begins off a multiple of 256", what);

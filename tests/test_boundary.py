@@ -184,10 +184,14 @@ def test_tc_prepare_geometry_and_refusals(fake):
                             (dict(shared_sum=1, shared_offset=ARENA - 4096), 1), (dict(shared_sum=1, shared_offset=1 << 20), 1),
                             (dict(intermediate=2000), 7), (dict(bits_x2=7), 7), (dict(bits_x2=0), 1), (dict(pass_=1), 1),
                             (dict(workspace_offset=(2 << 20) + 16), 1), (dict(output_offset=2 << 20), 1),
-                            (dict(activation_limit=-1.0), 1)]:
+                            (dict(activation_limit=-1.0), 1), (dict(widths_offset=(2 << 20) + 256), 1), (dict(widths_offset=ARENA), 1),
+                            (dict(widths_offset=4096 + 96), 1)]:
         untouched = amd.launches_of(5)
         assert lib.exl3_tc_prepare(C.byref(tc_record(**changes)), ARENA, fake.address, fake.card, untouched) == status, changes
         assert not any(bytes(untouched))
+    # a table of widths clear of the other ranges: taken
+    tabled = amd.launches_of(5)
+    assert lib.exl3_tc_prepare(C.byref(tc_record(widths_offset=16384)), ARENA, fake.address, fake.card, tabled) == 0
     # the sum into the shared expert's rows: its own range, checked like the others
     joined = amd.launches_of(5)
     assert lib.exl3_tc_prepare(C.byref(tc_record(shared_sum=1, shared_offset=3 << 29)), ARENA, fake.address, fake.card, joined) == 0
@@ -459,10 +463,15 @@ def test_tcp_prepare_geometry_and_refusals(fake):
                             (dict(hidden=1024, intermediate=2176), 7),  # the down operands would not fit over the gate and up operands
 
                             (dict(bits_x2=7), 7), (dict(bits_x2=40), 1), (dict(workspace_offset=(256 << 20) + 16), 1),
-                            (dict(workspace_offset=ARENA - 4096), 1), (dict(output_offset=2 << 20), 1)):
+                            (dict(workspace_offset=ARENA - 4096), 1), (dict(output_offset=2 << 20), 1),
+                            (dict(widths_offset=(256 << 20) + 512), 1), (dict(widths_offset=ARENA - 512), 1), (dict(widths_offset=(1 << 20) + 1024), 1)):
         untouched, n = amd.launches_of(8), C.c_uint32(99)
         assert lib.exl3_tcp_prepare(C.byref(tcp_record(**changes)), ARENA, fake.address, fake.card, untouched, C.byref(n)) == status, changes
         assert not any(bytes(untouched)) and n.value == 99
+
+
+    # a table of widths of the experts' number, clear of the other ranges: taken
+    assert lib.exl3_tcp_prepare(C.byref(tcp_record(widths_offset=48 << 20)), ARENA, fake.address, fake.card, launches, C.byref(count)) == 0
 
 
 def experts_description(fmt=amd.WEIGHT_FORMAT_E2M1_SCALED, **changes):
