@@ -210,6 +210,20 @@ class SiteFrontDescription(C.Structure):
                [("router", C.POINTER(RouterDescription)), ("router_weights", Range), ("kind", u32), ("row_count", u32), ("reserved_zero", u32)]
 
 
+class ExpertPause(C.Structure):
+    _fields_ = [("jobs_offset", u64), ("slots_offset", u64), ("slot_byte_count", u64), ("expert_byte_count", u64), ("matrix_offsets", u64 * 3),
+                ("first_host_expert", u32), ("host_expert_count", u32), ("jobs_per_row", u32), ("slot_count", u32), ("card", u32),
+                ("after_segment", u32)]
+
+
+class ExpertSlots(C.Structure):
+    _fields_ = [("fields", C.POINTER(u64)), ("pause_mark", u64), ("slot_count", u32), ("next_slot", u32)]
+
+
+class ExpertPauseUpload(C.Structure):
+    _fields_ = [("slot", u32), ("host_expert", u32)]
+
+
 class LinearWideKernels(C.Structure):
     _fields_ = [("wide_expert_gate_up", u32), ("wide_expert_down", u32), ("wide_expert_gate_up_e4m3", u32), ("wide_expert_down_e4m3", u32),
                 ("wide_expert_gate_up_b128", u32), ("wide_expert_down_b128", u32)]
@@ -288,6 +302,9 @@ def library():
             "dense_linear_prepare": [C.POINTER(DenseLinearDescription), u64, C.POINTER(DenseLinearKernels), launch_p],
             "hyper_kernels_prepare": [vp, vp, C.POINTER(HyperKernelsRecord)],
             "hyper_site_prepare": [C.POINTER(HyperSiteDescription), u64, C.POINTER(HyperKernelsRecord), launch_p],
+            "expert_pause_plan": [C.POINTER(ExpertPause), vp, u64, C.POINTER(ExpertSlots), C.POINTER(ExpertPauseUpload), C.POINTER(u32),
+                                  C.POINTER(u32)],
+            "expert_pause_run": [vp, vp, C.POINTER(ExpertPause), u32, C.POINTER(ExpertSlots), vp, vp, u64, C.POINTER(u32)],
             "site_front_kernels_prepare": [vp, vp, C.POINTER(SiteFrontKernels)],
             "site_front_prepare": [C.POINTER(SiteFrontDescription), u64, C.POINTER(RouterKernels), C.POINTER(SiteFrontKernels), launch_p],
             "expert_post_prepare": [C.POINTER(ExpertJoinDescription), u64, u32, launch_p],
@@ -529,7 +546,9 @@ class Exl3Layer:
     prepare functions."""
 
     def __init__(self, card, hidden, inner, expert_count, picks, rows, matrices, widths, router_weights_bf16=None,
-                 bias=None, affinity_kind=AFFINITY_SIGMOID, route_scale=1.5, limit=10.0):
+                 bias=None, affinity_kind=AFFINITY_SIGMOID, route_scale=1.5, limit=10.0, host_experts=()):
+        """host_experts: the experts kept in host memory (not on the card): the job table names them by tags and
+        run_pause() puts them into the card's slots (one slot a pair of a step) ahead of the experts' launches."""
         self.card, self.H, self.I, self.E, self.P, self.rows = card, hidden, inner, expert_count, picks, rows
         self.limit, self.affinity_kind, self.route_scale = limit, affinity_kind, route_scale
         self.pairs = rows * picks
@@ -537,19 +556,43 @@ class Exl3Layer:
         widths = np.asarray(widths, dtype=np.uint32).reshape(expert_count, 3)
         self.widths = widths
         self.uniform_width = int(widths[0, 0]) if np.all(widths == widths[0, 0]) else 0
-        total = sum(m.nbytes + 64 for trio in matrices for m in trio)
-        self.weights_offset = card.reserve(total, 256)
+        host_experts = list(host_experts)
+        aligned = lambda n: (n + 255) // 256 * 256
+        part_bytes = [aligned(max(matrices[e][m].nbytes for e in host_experts)) for m in range(3)] if host_experts else [0, 0, 0]
+        slot_bytes = sum(part_bytes)
+        total = aligned(sum(m.nbytes + 64 for e, trio in enumerate(matrices) if e not in host_experts for m in trio) + 256)
+        self.weights_offset = card.reserve(total + self.pairs * slot_bytes, 256)
         offsets = np.zeros((expert_count, 3), dtype=np.uint64)
         cursor = self.weights_offset
         blob = np.zeros(total, dtype=np.uint8)
         for e, trio in enumerate(matrices):
+            if e in host_experts: # a tag: the same for the three matrices
+                offsets[e, :] = self.weights_offset + total + 16 * host_experts.index(e)
+                continue
             for m, matrix in enumerate(trio):
                 cursor = (cursor + 63) // 64 * 64
                 offsets[e, m] = cursor
                 blob[cursor - self.weights_offset:cursor - self.weights_offset + matrix.nbytes] = matrix
                 cursor += matrix.nbytes
-        self.weights_bytes = total
+        self.weights_bytes = total + self.pairs * slot_bytes
         card.upload(self.weights_offset, blob)
+        if host_experts:
+            self.pause = ExpertPause()
+            self.pause.slots_offset, self.pause.slot_byte_count, self.pause.expert_byte_count = self.weights_offset + total, slot_bytes, slot_bytes
+            self.pause.matrix_offsets[0], self.pause.matrix_offsets[1], self.pause.matrix_offsets[2] = 0, part_bytes[0], part_bytes[0] + part_bytes[1]
+            self.pause.first_host_expert, self.pause.host_expert_count = 0, len(host_experts)
+            self.pause.jobs_per_row, self.pause.slot_count = picks, self.pairs
+            copies = C.c_void_p()
+            check(lib.backend_hip_staging_allocate(len(host_experts) * slot_bytes + self.pairs * 96, C.byref(copies)), "staging_allocate")
+            self.pause_staging = copies
+            view = np.ctypeslib.as_array((C.c_ubyte * (len(host_experts) * slot_bytes)).from_address(copies.value))
+            view[:] = 0
+            for i, e in enumerate(host_experts):
+                for m in range(3):
+                    at = i * slot_bytes + int(self.pause.matrix_offsets[m])
+                    view[at:at + matrices[e][m].nbytes] = matrices[e][m].view(np.uint8).reshape(-1)
+            self.slot_fields = np.zeros(2 * self.pairs, dtype=np.uint64)
+            self.slots = ExpertSlots(self.slot_fields.ctypes.data_as(C.POINTER(u64)), 0, self.pairs, 0)
         self.expert_offsets = offsets
         self.offsets_offset = card.place(offsets)
         packed = (widths[:, 0] | (widths[:, 1] << 8) | (widths[:, 2] << 16)).astype(np.uint32)
@@ -576,6 +619,15 @@ class Exl3Layer:
         self.card.upload(self.x_offset, x_bf16)
         live = self.rows if live_rows is None else live_rows
         self.card.upload(self.step_offset, step_block(live))
+
+    def run_pause(self):
+        """The layer's expert pause behind its select (expert_pause_run): the experts uploaded."""
+        self.pause.jobs_offset = self.jobs_offset
+        uploaded = u32(0)
+        jobs_staging = C.c_void_p(self.pause_staging.value + int(self.pause.host_expert_count) * int(self.pause.slot_byte_count))
+        check(self.card.lib.expert_pause_run(backend_table(), self.card.handle, C.byref(self.pause), self.rows, C.byref(self.slots), jobs_staging,
+                                             self.pause_staging, 60 * SECOND, C.byref(uploaded)), "expert_pause_run")
+        return uploaded.value
 
     def experts_description(self):
         d = RoutedExpertsDescription()

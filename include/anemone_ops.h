@@ -245,6 +245,52 @@ MUST_CHECK result_status site_front_prepare(const struct site_front_description 
                                             const struct router_kernels_record *router_kernels,
                                             const struct site_front_kernels *kernels, struct kernel_launch *launch_out);
 
+/* ---- host experts: a step's expert pauses (include/anemone/model_seam.h:193-214, source/step_experts.c:27-168 of the
+ * reference). Behind a layer's router, whose job table names a host expert i of the layer by three offsets equal to
+ * slots_offset + 16 i, each such expert is put into one of the card's slots (slot k at slots_offset + k
+ * slot_byte_count; uploaded unless a slot holds it already) and the job's offsets are pointed there; any other job keeps
+ * its offsets, all below slots_offset. ---- */
+#define EXPERT_PAUSE_MATRICES 3u
+struct expert_pause { /* model_seam.h:202-214, member for member */
+    uint64_t jobs_offset;
+    uint64_t slots_offset;
+    uint64_t slot_byte_count;
+    uint64_t expert_byte_count; /* at most slot_byte_count */
+    uint64_t matrix_offsets[EXPERT_PAUSE_MATRICES]; /* of gate, up, down inside an expert's bytes */
+    uint32_t first_host_expert;
+    uint32_t host_expert_count;
+    uint32_t jobs_per_row;
+    uint32_t slot_count; /* at least jobs_per_row times the most rows of a step */
+    uint32_t card;
+    uint32_t after_segment;
+};
+/* what the reference's step driver keeps of a card's slots between pauses (source/step_driver.h:17, 73): the caller's here */
+#define EXPERT_SLOT_FIELDS 2u
+struct expert_slots {
+    uint64_t *fields;    /* [slot_count][2]: the host expert the slot holds + 1 (0: none), the mark of the pause that took it last */
+    uint64_t pause_mark; /* of the last pause */
+    uint32_t slot_count;
+    uint32_t next_slot;  /* the slot the next upload tries first */
+};
+struct expert_pause_upload {
+    uint32_t slot;
+    uint32_t host_expert; /* of the pause's: 0 .. host_expert_count - 1 */
+};
+/* The walk over a job table in host memory: the jobs' offsets pointed into slots, the slots' state moved on, the uploads
+ * the pause owes listed in their order (uploads_out: job_count places). STATUS_DEVICE_ERROR for a job that names neither
+ * an expert on the card nor a host expert of the pause (a tag off the tags' step, beyond the layer's, matrices apart,
+ * partly a tag), as the reference answers. */
+MUST_CHECK result_status expert_pause_plan(const struct expert_pause *pause, struct expert_job_record *jobs, uint64_t job_count,
+                                           struct expert_slots *slots, struct expert_pause_upload *uploads_out,
+                                           uint32_t *upload_count_out, uint32_t *tag_count_out);
+/* The pause on a card: the job table back into jobs_staging (page-locked, jobs_per_row row_count records), the walk, the
+ * experts up from expert_copies (page-locked: the pause's host experts, expert_byte_count apart), the job table up again
+ * where a tag was in it; every copy is finished when the call returns. */
+MUST_CHECK result_status expert_pause_run(const struct backend_operations *backend, struct device_card *card,
+                                          const struct expert_pause *pause, uint32_t row_count, struct expert_slots *slots,
+                                          void *jobs_staging, const unsigned char *expert_copies, uint64_t wait_limit_nanoseconds,
+                                          uint32_t *upload_count_out);
+
 /* ---- FP4 / FP8 expert linears of the original weights (the routed part of the reference's linear.h) ---- */
 #define LINEAR_SLICE_INSTANCES 5u /* product kernels are stamped for 1, 2, 4, 8, 16 slices; gfx950 holds 1, 2, 4, 8 */
 #define LINEAR_MAXIMUM_SLICES 16u
