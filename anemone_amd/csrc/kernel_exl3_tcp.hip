@@ -69,11 +69,11 @@ extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_count(st
     const uint32_t pairs = sort_block_picks((const struct router_pick *)(arena + record.picks_offset), shape.picks, blockIdx.x,
                                             record.row_count, block_experts);
     __syncthreads();
+    __shared__ uint32_t histogram[ROUTER_MOST_EXPERTS];
+    sort_count_picks(block_experts, pairs, shape.experts, histogram);
     uint32_t *counts = (uint32_t *)(arena + record.workspace_offset + shape.layout.counts) + (uint64_t)blockIdx.x * shape.experts;
     for (uint32_t expert = threadIdx.x; expert < shape.experts; expert += blockDim.x) {
-        uint32_t count = 0;
-        sort_walk_picks(block_experts, pairs, [&](uint32_t, uint32_t picked) { count += picked == expert ? 1u : 0u; });
-        counts[expert] = count;
+        counts[expert] = histogram[expert];
     }
 }
 ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_count, exl3_tcp_record);
@@ -86,6 +86,7 @@ extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_place(st
     __shared__ uint32_t block_places[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t chunk_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
+    __shared__ uint32_t first_places[ROUTER_MOST_EXPERTS], cursors[SORT_MOST_WAVES * ROUTER_MOST_EXPERTS];
     const tcp_shape shape = tcp_shape_of(record);
     const uint32_t experts = shape.experts;
     const uint32_t blocks = (record.row_count + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
@@ -109,17 +110,12 @@ extern "C" __global__ void __launch_bounds__(TCP_SORT_THREADS) exl3_tcp_place(st
     (void)block_exclusive_scan(starts, experts, scratch);
     uint32_t *sorted = (uint32_t *)(workspace + shape.layout.sorted), *place_of = (uint32_t *)(workspace + shape.layout.place_of);
     const uint32_t first_pair = blockIdx.x * ROUTER_SORT_ROWS * shape.picks;
-    /* the walk writes a pick's place into LDS alone; the two tables are written behind it, a thread a pick */
+    /* every pick's place into LDS; the two tables are written behind it, a thread a pick */
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
-        uint32_t place = starts[expert] + before[expert];
-        sort_walk_picks(block_experts, pairs, [&](uint32_t index, uint32_t picked) {
-            if (picked == expert) {
-                block_places[index] = place;
-                place++;
-            }
-        });
+        first_places[expert] = starts[expert] + before[expert];
     }
     __syncthreads();
+    sort_place_picks(block_experts, pairs, experts, first_places, cursors, block_places);
     for (uint32_t index = threadIdx.x; index < pairs; index += blockDim.x) {
         const uint32_t place = block_places[index];
         sorted[place] = first_pair + index;

@@ -288,11 +288,11 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     if (pairs == 0u) {
         return; /* a block of no live row writes nothing; the place reads no count of it */
     }
+    __shared__ uint32_t histogram[ROUTER_MOST_EXPERTS];
+    sort_count_picks(block_experts, pairs, arguments.expert_count, histogram);
     uint32_t *counts = (uint32_t *)(arena + arguments.counts_offset) + (uint64_t)blockIdx.x * arguments.expert_count;
     for (uint32_t expert = threadIdx.x; expert < arguments.expert_count; expert += blockDim.x) {
-        uint32_t count = 0;
-        sort_walk_picks(block_experts, pairs, [&](uint32_t, uint32_t picked) { count += picked == expert ? 1u : 0u; });
-        counts[expert] = count;
+        counts[expert] = histogram[expert];
     }
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_count, router_wide_arguments);
@@ -303,25 +303,20 @@ ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_count, router_wide_arguments);
  * calls it after a barrier. */
 __device__ static __forceinline__ void wide_place_block(const struct router_wide_arguments &arguments, unsigned char *arena, uint32_t block,
                                                         const uint32_t *block_experts, uint32_t *place_of, uint32_t pairs, uint32_t *totals,
-                                                        uint32_t *starts, const uint32_t *before, uint32_t *tile_starts, uint32_t *scratch)
+                                                        uint32_t *starts, const uint32_t *before, uint32_t *tile_starts, uint32_t *scratch,
+                                                        uint32_t *first_places, uint32_t *cursors)
 {
     const uint32_t experts = arguments.expert_count, picks = arguments.pick_count;
     (void)block_exclusive_scan(starts, experts, scratch);
     const struct router_pick *all_picks = (const struct router_pick *)(arena + arguments.picks_offset);
     struct wide_pair *sorted = (struct wide_pair *)(arena + arguments.pairs_offset);
     const uint32_t first_pair = block * ROUTER_SORT_ROWS * picks;
-    /* the walk writes a pick's place into LDS and nothing else: a load of the pick's weight inside it would make every
-     * match wait for memory, one after the other; the pairs are written behind it, a thread a pick */
+    /* every pick's place into LDS; the pairs are written behind it, a thread a pick */
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
-        uint32_t place = starts[expert] + before[expert];
-        sort_walk_picks(block_experts, pairs, [&](uint32_t index, uint32_t picked) {
-            if (picked == expert) {
-                place_of[index] = place;
-                place++;
-            }
-        });
+        first_places[expert] = starts[expert] + before[expert];
     }
     __syncthreads();
+    sort_place_picks(block_experts, pairs, experts, first_places, cursors, place_of);
     for (uint32_t index = threadIdx.x; index < pairs; index += blockDim.x) {
         sorted[place_of[index]] = (struct wide_pair){first_pair + index, all_picks[first_pair + index].route_weight};
     }
@@ -371,6 +366,7 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     __shared__ uint32_t place_of[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS];
+    __shared__ uint32_t first_places[ROUTER_MOST_EXPERTS], cursors[SORT_MOST_WAVES * ROUTER_MOST_EXPERTS];
     const uint32_t experts = arguments.expert_count;
     const uint32_t live_rows = wide_live_rows(arguments, arena);
     const uint32_t live_blocks = (live_rows + ROUTER_SORT_ROWS - 1u) / ROUTER_SORT_ROWS;
@@ -392,7 +388,8 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
         tile_starts[expert] = (total + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS;
     }
     __syncthreads();
-    wide_place_block(arguments, arena, blockIdx.x, block_experts, place_of, pairs, totals, starts, before, tile_starts, scratch);
+    wide_place_block(arguments, arena, blockIdx.x, block_experts, place_of, pairs, totals, starts, before, tile_starts, scratch, first_places,
+                     cursors);
 }
 ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_wide_place, router_wide_arguments);
 
@@ -470,21 +467,21 @@ extern "C" __global__ void __launch_bounds__(WIDE_SORT_THREADS)
     __shared__ uint32_t place_of[ROUTER_SORT_ROWS * ROUTER_MOST_PICKS];
     __shared__ uint32_t totals[ROUTER_MOST_EXPERTS], starts[ROUTER_MOST_EXPERTS], before[ROUTER_MOST_EXPERTS];
     __shared__ uint32_t tile_starts[ROUTER_MOST_EXPERTS + 1u], scratch[ROUTER_MOST_EXPERTS], job_starts[ROUTER_MOST_EXPERTS + 1u];
+    __shared__ uint32_t first_places[ROUTER_MOST_EXPERTS], cursors[SORT_MOST_WAVES * ROUTER_MOST_EXPERTS];
     const uint32_t experts = arguments.expert_count;
     const uint32_t live_rows = wide_live_rows(arguments, arena);
     const uint32_t pairs = wide_block_picks(arguments, arena, 0u, live_rows, block_experts);
     __syncthreads();
+    sort_count_picks(block_experts, pairs, experts, totals);
     for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
-        uint32_t count = 0;
-        sort_walk_picks(block_experts, pairs, [&](uint32_t, uint32_t picked) { count += picked == expert ? 1u : 0u; });
-        totals[expert] = count;
+        const uint32_t count = totals[expert];
         starts[expert] = count;
         before[expert] = 0u;
         tile_starts[expert] = (count + WIDE_TILE_PAIRS - 1u) / WIDE_TILE_PAIRS;
         job_starts[expert] = (count + LINEAR_MAXIMUM_ROWS - 1u) / LINEAR_MAXIMUM_ROWS;
     }
     __syncthreads();
-    wide_place_block(arguments, arena, 0u, block_experts, place_of, pairs, totals, starts, before, tile_starts, scratch);
+    wide_place_block(arguments, arena, 0u, block_experts, place_of, pairs, totals, starts, before, tile_starts, scratch, first_places, cursors);
     __threadfence_block();
     __syncthreads(); /* the runs and the sorted pairs, written by this block, are read by its jobs */
     wide_jobs_block(arguments, arena, job_starts, scratch);

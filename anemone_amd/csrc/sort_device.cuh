@@ -1,7 +1,8 @@
 /*
  * sort_device.cuh -- what the sorts of pairs by expert share (the router's wide select and the prefill form of the
- * EXL3 experts): a block's picked experts into LDS, and a block-wide exclusive prefix sum. No atomic operation
- * anywhere: a thread owns an expert and walks the block's picks in row order.
+ * EXL3 experts): a block's picked experts into LDS, its picks counted an expert, every pick's place, and a block-wide
+ * exclusive prefix sum. The only atomic operations are integer additions in LDS that count (the same sums in any order);
+ * a pick's place among its expert's is formed from the lanes' ballots, in row order.
  */
 #ifndef SORT_DEVICE_CUH
 #define SORT_DEVICE_CUH
@@ -24,41 +25,87 @@ __device__ static __forceinline__ uint32_t sort_block_picks(const struct router_
     return rows * picks_per_row;
 }
 
-/* Every pick of a block in order, 32 at a time (eight 16-byte LDS reads in flight, so that a walk waits for LDS once
- * in 32 picks), then eight at a time, then one: visit(index, expert). block_experts is 16-byte aligned. */
-template <typename Visit>
-__device__ static __forceinline__ void sort_walk_picks(const uint32_t *block_experts, uint32_t pairs, Visit visit)
+#define SORT_WAVE 64u
+#define SORT_MOST_WAVES 8u /* of a block of the sorts: 512 threads */
+
+/* The block's picks of every expert: histogram[expert] in LDS. Integer additions in LDS: the same sums whatever their
+ * order. The whole block calls it (barriers inside); block_experts is complete before the call. */
+__device__ static __forceinline__ void sort_count_picks(const uint32_t *block_experts, uint32_t pairs, uint32_t experts, uint32_t *histogram)
 {
-    typedef __attribute__((ext_vector_type(4))) uint32_t four_words;
-    uint32_t index = 0;
-    for (; index + 32u <= pairs; index += 32u) {
-        four_words words[8];
-#pragma unroll
-        for (uint32_t i = 0; i < 8u; i++) {
-            words[i] = *(const four_words *)(block_experts + index + 4u * i);
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        histogram[expert] = 0u;
+    }
+    __syncthreads();
+    for (uint32_t index = threadIdx.x; index < pairs; index += blockDim.x) {
+        __hip_atomic_fetch_add(&histogram[block_experts[index]], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
+}
+
+/* The lanes of the wavefront that hold the same word as this lane, among the lanes where `live` (a lane that is not live
+ * gets 0): one ballot a bit of the words, `bits` of them. */
+__device__ static __forceinline__ uint64_t sort_equal_lanes(uint32_t word, bool live, uint32_t bits)
+{
+    uint64_t equal = __builtin_amdgcn_ballot_w64(live);
+    for (uint32_t bit = 0; bit < bits; bit++) {
+        const bool set = ((word >> bit) & 1u) != 0u;
+        const uint64_t holders = __builtin_amdgcn_ballot_w64(live && set);
+        equal &= set ? holders : ~holders;
+    }
+    return live ? equal : 0ull;
+}
+
+/* Every pick's place, in LDS: place_of[index] = first[expert] + the picks of the same expert before it in the block.
+ * Wavefront w of the block's `waves` takes the picks [w share, (w + 1) share) in order, 64 at a time: a pick's place is
+ * its expert's cursor plus the lanes below it that hold the same expert (ballots over the expert's bits: no lane waits
+ * for another's answer), and the first of them moves the cursor on. A wavefront's cursors begin behind the picks of the
+ * wavefronts before it, which a histogram a wavefront (LDS, integer additions) and a walk over the wavefronts by a thread
+ * an expert give. first: LDS, experts words (kept); cursors: LDS, SORT_MOST_WAVES x experts words. The whole block
+ * calls it (barriers inside). */
+__device__ static __forceinline__ void sort_place_picks(const uint32_t *block_experts, uint32_t pairs, uint32_t experts, const uint32_t *first,
+                                                        uint32_t *cursors, uint32_t *place_of)
+{
+    const uint32_t lane = threadIdx.x % SORT_WAVE, wave = threadIdx.x / SORT_WAVE, waves = blockDim.x / SORT_WAVE;
+    const uint32_t share = ((pairs + waves - 1u) / waves + SORT_WAVE - 1u) / SORT_WAVE * SORT_WAVE; /* whole groups of 64 a wavefront */
+    const uint32_t begin = wave * share < pairs ? wave * share : pairs, end = begin + share < pairs ? begin + share : pairs;
+    for (uint32_t at = threadIdx.x; at < waves * experts; at += blockDim.x) {
+        cursors[at] = 0u;
+    }
+    __syncthreads();
+    for (uint32_t index = begin + lane; index < end; index += SORT_WAVE) {
+        __hip_atomic_fetch_add(&cursors[wave * experts + block_experts[index]], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
+    for (uint32_t expert = threadIdx.x; expert < experts; expert += blockDim.x) {
+        uint32_t place = first[expert];
+        for (uint32_t other = 0; other < waves; other++) {
+            const uint32_t count = cursors[other * experts + expert];
+            cursors[other * experts + expert] = place;
+            place += count;
         }
-#pragma unroll
-        for (uint32_t i = 0; i < 8u; i++) {
-            visit(index + 4u * i, words[i].x);
-            visit(index + 4u * i + 1u, words[i].y);
-            visit(index + 4u * i + 2u, words[i].z);
-            visit(index + 4u * i + 3u, words[i].w);
+    }
+    __syncthreads();
+    uint32_t bits = 0;
+    while ((1u << bits) < experts) {
+        bits++;
+    }
+    uint32_t *mine = cursors + wave * experts;
+    for (uint32_t base = begin; base < end; base += SORT_WAVE) {
+        const uint32_t index = base + lane;
+        const bool live = index < end;
+        const uint32_t expert = live ? block_experts[index] : 0u;
+        const uint64_t equal = sort_equal_lanes(expert, live, bits);
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(equal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)equal, 0u));
+        if (live) {
+            const uint32_t cursor = mine[expert]; /* every lane of an expert reads it before the first of them writes it: LDS serves
+                                                    a wavefront's instructions in their order */
+            place_of[index] = cursor + below;
+            if (below == 0u) {
+                mine[expert] = cursor + (uint32_t)__builtin_popcountll(equal);
+            }
         }
     }
-    for (; index + 8u <= pairs; index += 8u) {
-        const four_words low = *(const four_words *)(block_experts + index), high = *(const four_words *)(block_experts + index + 4u);
-        visit(index, low.x);
-        visit(index + 1u, low.y);
-        visit(index + 2u, low.z);
-        visit(index + 3u, low.w);
-        visit(index + 4u, high.x);
-        visit(index + 5u, high.y);
-        visit(index + 6u, high.z);
-        visit(index + 7u, high.w);
-    }
-    for (; index < pairs; index++) {
-        visit(index, block_experts[index]);
-    }
+    __syncthreads();
 }
 
 /* exclusive prefix sums of values[0 .. count) in LDS, count <= ROUTER_MOST_EXPERTS, by the whole block; total returned */
