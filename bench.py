@@ -32,8 +32,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("exl3_decode", 8): 375.2e6 + 8.4e6,
     ("fp4_decode", 32): 1434.7e6 + 1.0e6,
     ("fp8_decode", 32): 2746.8e6 + 1.0e6,
-    ("fp4_prefill", 8192): 4900.2e6 + 446.0e6,
-    ("fp8_prefill", 2048): 5211.3e6 + 116.0e6,
+    ("fp4_prefill", 8192): 4777.9e6 + 447.0e6,
+    ("fp8_prefill", 2048): 5626.5e6 + 117.6e6,
     ("expert_join", 8192): 877.7e6 + 402.7e6,
     ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,
     ("fp8_prefill_block128", 2048): 5386.8e6 + 67.2e6,
