@@ -106,9 +106,12 @@ def fp4_layer(amd, card, hidden, inner, experts_n, picks, rows, distinct=4, **ke
 
 
 @pytest.mark.parametrize("rows,width,experts_n,picks,live,form", [(8, 4096, 256, 8, 8, "fp4"), (1, 4096, 256, 8, 1, "fp4"), (8, 2048, 64, 4, 5, "fp4"),
-                                                                   (6, 3072, 128, 6, 6, "exl3")])
+                                                                   (6, 3072, 128, 6, 6, "exl3"), (8, 5120, 384, 6, 8, "fp4-reference-order")])
 def test_ffn_front_equals_its_launches(amd, card, rows, width, experts_n, picks, live, form):
+    """The last case is the reference's own model: width 5,120, 384 experts, six picks in the reference's order of sums."""
     say("fused FFN front", rows, width, experts_n, picks, live, form)
+    order = 1 if form.endswith("reference-order") else 0
+    form = form.split("-")[0]
     inner = 256
     if form == "fp4":
         layer = fp4_layer(amd, card, width, inner, experts_n, picks, rows)
@@ -124,7 +127,7 @@ def test_ffn_front_equals_its_launches(amd, card, rows, width, experts_n, picks,
     streams = to_bf16(normals(73, rows * STREAMS * width)).reshape(rows, STREAMS, width)
     carried = (np.abs(normals(74, rows * STREAMS)) * 0.3 + 0.1).astype(np.float32).reshape(rows, STREAMS)
     layer.set_rows(np.zeros((rows, width), np.uint16), live)  # the rows are the front's to write; the step block's live rows
-    fused = front.front_launch(rows, layer)  # the front's rows are the select's; the step block names the live ones
+    fused = front.front_launch(rows, layer, order)  # the front's rows are the select's; the step block names the live ones
     scores_range = amd.Range(layer.scores_offset, rows * experts_n * 4)
     scores = front.dense_launch(amd.Range(layer.router_offset, experts_n * width * 2), amd.Range(layer.x_offset, rows * width * 2), scores_range,
                                 experts_n, width, amd.DENSE_BFLOAT16, amd.DENSE_FLOAT32, 0, 1.0, 0.0, rows)
@@ -145,7 +148,7 @@ def test_ffn_front_equals_its_launches(amd, card, rows, width, experts_n, picks,
         card.run(front.mix_project_launch(rows))
         card.run(front.site_launches(rows)[:1])
         card.run(scores)
-        card.run(layer.select_launch(0))
+        card.run(layer.select_launch(order))
         card.run(quantize)
 
     front.set_streams(streams, carried)
@@ -163,7 +166,7 @@ def test_ffn_front_equals_its_launches(amd, card, rows, width, experts_n, picks,
     # what the launches cost on the card, queued back to back
     array = amd.launches_of(5)
     array[0], array[1], array[2], array[3], array[4] = front.mix_project_launch(rows)[0], front.site_launches(rows)[0], scores[0], \
-        layer.select_launch(0)[0], quantize[0]
+        layer.select_launch(order)[0], quantize[0]
     for name, launches in (("separate", array), ("fused", fused)):
         times = []
         for _ in range(6):
