@@ -984,10 +984,11 @@ class SiteFront:
         self.kept = keep
         return d
 
-    def front_launch(self, rows=None, layer=None, order=0):
+    def front_launch(self, rows=None, layer=None, order=0, kind=None):
         """ONE launch for the mix project, the mix finish, (with `layer`: the router's scores and its select) and the
-        quantization of the sublayer's input."""
-        d = self.front_description(rows, layer, order)
+        quantization of the sublayer's input; with kind SITE_FRONT_KIND_INPUT or _COEFFICIENTS one of the two launches
+        the site front may be cut in (the input front first)."""
+        d = self.front_description(rows, layer, order, kind)
         router_kernels = None if layer is None else C.byref(layer.router_kernels)
         launch = launches_of(1)
         check(self.card.lib.site_front_prepare(C.byref(d), self.card.arena_bytes, router_kernels, C.byref(self.front_kernels), launch),

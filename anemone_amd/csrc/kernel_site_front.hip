@@ -1,7 +1,9 @@
 /*
  * kernel_site_front.hip -- the fused fronts of a block's sites on gfx950: site_front_<R> (a site's mix project, its mix
  * finish and the quantization of the sublayer's input in one launch) and ffn_front_<R> (the same with the router's scores
- * and its select between the finish and the quantization). Entry names, record and what is written follow the reference
+ * and its select between the finish and the quantization); input_front_<R> and then coefficient_front_<R>, the site front
+ * in two launches (the first stores hidden, codes, exponents and operands; the second the mixes, post, comb and the site's
+ * pre, and may run beside later launches up to the site's post). Entry names, record and what is written follow the reference
  * (include/anemone/site_front_records.h:10-37, source/kernel_site_front.cu): every output has the bits of the launches
  * the front stands for, because it runs their code (dense_device.cuh, hyper_device.cuh, router_device.cuh,
  * quantize_device.cuh) on the same operands in the same order.
@@ -19,6 +21,10 @@
  * A wait is thread 0 polling the counter (agent scope) with a sleep between polls, at most SITE_FRONT_WAIT_POLLS times;
  * a block whose wait runs out counts itself in gave_up, skips its part and leaves: every wave of the grid ends. The
  * last block to leave (departed) clears the counters.
+ *
+ * The two halves need no tickets and no waits: the input front is a row a block (grid rows); the coefficient front is the
+ * mix project's blocks (grid site_front_mix_blocks), the last of which to publish arrived forms post, comb and pre and
+ * clears that counter. The stream orders them: the coefficient front writes the pre that the input front read.
  */
 #include "kernel_registry.h"
 #include "dense_device.cuh"
@@ -88,6 +94,47 @@ __device__ static __forceinline__ bool front_wait(uint32_t *counter, uint32_t ta
     return *word != 0u;
 }
 
+/* a row's block: the row's input, then its quantization, a thread four values at a time */
+__device__ static __forceinline__ void front_row(const struct site_front_arguments &arguments, const struct hyper_finish_arguments &finish,
+                                                 unsigned char *arena, uint32_t row, uint32_t thread, uint32_t threads, float *group_sums)
+{
+    const uint32_t width = threads * HYPER_VALUES_PER_THREAD;
+    hyper_row_input_body(finish, arena, row, thread, threads, group_sums);
+    __syncthreads(); /* the row is written: this block's threads read it */
+    const struct activation_quantize_arguments quantize = {arguments.hidden_offset, arguments.codes_offset, arguments.exponents_offset,
+                                                           arguments.operands_offset, width};
+    for (uint32_t q = thread; q < width / 4u; q += threads) {
+        activation_quantize_body(quantize, arena, q, row);
+    }
+}
+
+/* block `block` of the mix project's: float32 [24][4 width] by the streams as rows of 4 width values, with the row's scale,
+ * SITE_FRONT_MIX_OUTPUTS mixes a quarter of 256 threads, into the scratch's mixes */
+template <uint32_t ROWS>
+__device__ static __forceinline__ void front_mix_project(const struct site_front_arguments &arguments, unsigned char *arena, uint32_t rows,
+                                                         uint32_t block, uint32_t thread, uint32_t threads,
+                                                         dense_group_sums<ROWS, SITE_FRONT_MIX_OUTPUTS> *sums)
+{
+    const uint32_t quarter = thread / DENSE_THREADS_VALUE, quarters = threads / DENSE_THREADS_VALUE;
+    const bool in_quarter = quarter < quarters;
+    struct dense_linear_arguments dense = {};
+    dense.weights_offset = arguments.mix_weights_offset;
+    dense.rows_offset = arguments.streams_offset;
+    dense.output_offset = arguments.scratch_offset + offsetof(struct site_front_scratch, mixes);
+    dense.output_size = MODEL_MIXES;
+    dense.input_size = MODEL_STREAMS * threads * HYPER_VALUES_PER_THREAD;
+    dense.row_count = rows;
+    dense.output_type = DENSE_FLOAT32;
+    dense.flags = DENSE_ROW_SCALE;
+    dense.output_scale = 1.0f;
+    dense.epsilon = MODEL_NORM_EPSILON;
+    constexpr uint32_t groups = MODEL_MIXES / SITE_FRONT_MIX_OUTPUTS;
+    const uint32_t group = block * quarters + quarter;
+    dense_linear_body<DENSE_FLOAT32, ROWS, SITE_FRONT_MIX_OUTPUTS>(dense, arena, (const uint16_t *)(arena + dense.rows_offset),
+                                                                   group * SITE_FRONT_MIX_OUTPUTS, 0u, thread % DENSE_THREADS_VALUE,
+                                                                   in_quarter && group < groups, sums[in_quarter ? quarter : 0u]);
+}
+
 template <uint32_t ROWS, bool FFN>
 __device__ static __forceinline__ void site_front(const struct site_front_arguments &arguments, unsigned char *arena)
 {
@@ -121,33 +168,11 @@ __device__ static __forceinline__ void site_front(const struct site_front_argume
                                                   arguments.norm_weight_offset, arguments.hidden_offset};
     if (ticket < rows) {
         /* a row: its input, then its quantization, a thread four values at a time */
-        const uint32_t row = ticket;
-        hyper_row_input_body(finish, arena, row, thread, threads, lds.group_sums);
-        __syncthreads(); /* the row is written: this block's threads read it */
-        const struct activation_quantize_arguments quantize = {arguments.hidden_offset, arguments.codes_offset, arguments.exponents_offset,
-                                                               arguments.operands_offset, width};
-        for (uint32_t q = thread; q < width / 4u; q += threads) {
-            activation_quantize_body(quantize, arena, q, row);
-        }
+        front_row(arguments, finish, arena, ticket, thread, threads, lds.group_sums);
         front_publish<true, false>(&scratch->rows_ready, thread, &word);
     } else if (ticket < rows + mix_blocks) {
         /* the mix project: float32 [24][4 width] by the streams as rows of 4 width values, with the row's scale */
-        struct dense_linear_arguments dense = {};
-        dense.weights_offset = arguments.mix_weights_offset;
-        dense.rows_offset = arguments.streams_offset;
-        dense.output_offset = mixes_offset;
-        dense.output_size = MODEL_MIXES;
-        dense.input_size = MODEL_STREAMS * width;
-        dense.row_count = rows;
-        dense.output_type = DENSE_FLOAT32;
-        dense.flags = DENSE_ROW_SCALE;
-        dense.output_scale = 1.0f;
-        dense.epsilon = MODEL_NORM_EPSILON;
-        constexpr uint32_t groups = MODEL_MIXES / SITE_FRONT_MIX_OUTPUTS;
-        const uint32_t group = (ticket - rows) * quarters + quarter;
-        dense_linear_body<DENSE_FLOAT32, ROWS, SITE_FRONT_MIX_OUTPUTS>(dense, arena, (const uint16_t *)(arena + dense.rows_offset),
-                                                                       group * SITE_FRONT_MIX_OUTPUTS, 0u, quarter_thread,
-                                                                       in_quarter && group < groups, lds.mixes[slot]);
+        front_mix_project<ROWS>(arguments, arena, rows, ticket - rows, thread, threads, lds.mixes);
         if (front_publish<true, true>(&scratch->arrived, thread, &word) == mix_blocks - 1u &&
             front_wait<false>(&scratch->rows_ready, rows, thread, &word, &scratch->gave_up)) {
             /* every mix is stored and every row's block has read the carried pre */
@@ -202,6 +227,48 @@ __device__ static __forceinline__ void site_front(const struct site_front_argume
     }
 }
 
+/* the site front's first half: a row a block */
+__device__ static __forceinline__ void input_front(const struct site_front_arguments &arguments, unsigned char *arena)
+{
+    __shared__ float group_sums[32];
+    const uint32_t rows = arguments.select.row_count;
+    if (gridDim.x != rows) {
+        return;
+    }
+    const struct hyper_finish_arguments finish = {arguments.streams_offset, arguments.pre_offset,
+                                                  arguments.scratch_offset + offsetof(struct site_front_scratch, mixes), arguments.scale_offset,
+                                                  arguments.base_offset, arguments.post_offset, arguments.comb_offset,
+                                                  arguments.norm_weight_offset, arguments.hidden_offset};
+    front_row(arguments, finish, arena, blockIdx.x, threadIdx.x, blockDim.x, group_sums);
+}
+
+/* its second half: the mix project's blocks; the last to publish forms every row's post, comb and pre */
+template <uint32_t ROWS>
+__device__ static __forceinline__ void coefficient_front(const struct site_front_arguments &arguments, unsigned char *arena)
+{
+    __shared__ dense_group_sums<ROWS, SITE_FRONT_MIX_OUTPUTS> sums[FRONT_MOST_QUARTERS];
+    __shared__ uint32_t word;
+    const uint32_t thread = threadIdx.x, threads = blockDim.x, rows = arguments.select.row_count;
+    const uint32_t mix_blocks = site_front_mix_blocks(threads * HYPER_VALUES_PER_THREAD);
+    struct site_front_scratch *scratch = (struct site_front_scratch *)(arena + arguments.scratch_offset);
+    if (gridDim.x != mix_blocks) {
+        return;
+    }
+    front_mix_project<ROWS>(arguments, arena, rows, blockIdx.x, thread, threads, sums);
+    if (front_publish<true, true>(&scratch->arrived, thread, &word) == mix_blocks - 1u) {
+        const struct hyper_finish_arguments finish = {arguments.streams_offset, arguments.pre_offset,
+                                                      arguments.scratch_offset + offsetof(struct site_front_scratch, mixes), arguments.scale_offset,
+                                                      arguments.base_offset, arguments.post_offset, arguments.comb_offset,
+                                                      arguments.norm_weight_offset, arguments.hidden_offset};
+        if (thread < rows * MODEL_STREAMS * MODEL_STREAMS) {
+            hyper_coefficients_body(finish, arena, thread / (MODEL_STREAMS * MODEL_STREAMS), thread % (MODEL_STREAMS * MODEL_STREAMS));
+        }
+        if (thread == 0u) {
+            scratch->arrived = 0u; /* every block has added to it */
+        }
+    }
+}
+
 #define FRONT_STAMP(name, rows, ffn)                                                                                           \
     extern "C" __global__ void __launch_bounds__(FRONT_MOST_THREADS) name##_##rows(struct site_front_arguments arguments, \
                                                                                             unsigned char *arena)              \
@@ -213,3 +280,15 @@ FRONT_STAMP(site_front, 1, false)
 FRONT_STAMP(site_front, 8, false)
 FRONT_STAMP(ffn_front, 1, true)
 FRONT_STAMP(ffn_front, 8, true)
+
+#define HALF_STAMP(name, rows, call)                                                                                           \
+    extern "C" __global__ void __launch_bounds__(FRONT_MOST_THREADS) name##_##rows(struct site_front_arguments arguments, \
+                                                                                            unsigned char *arena)              \
+    {                                                                                                                          \
+        call(arguments, arena);                                                                                                \
+    }                                                                                                                          \
+    ANEMONE_KERNEL(KERNEL_FILE_SITE_FRONT, name##_##rows, site_front_arguments);
+HALF_STAMP(input_front, 1, input_front)
+HALF_STAMP(input_front, 8, input_front)
+HALF_STAMP(coefficient_front, 1, coefficient_front<1>)
+HALF_STAMP(coefficient_front, 8, coefficient_front<8>)

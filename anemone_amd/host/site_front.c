@@ -6,6 +6,9 @@
  *   launch        kernel             grid                                                          block
  *   site front    site_front_<R>     (rows + site_front_mix_blocks, 1, 1)                          width / 8
  *   FFN front     ffn_front_<R>      (rows + site_front_mix_blocks + site_front_score_blocks, 1, 1)  width / 8
+ *   input front   input_front_<R>    (rows, 1, 1)                                                  width / 8
+ *   coefficients  coefficient_front_<R>  (site_front_mix_blocks, 1, 1)                             width / 8
+ * The input front and then the coefficient front are the site front in two launches of one stream.
  * R = 1 for one row, 8 for 2 to 8 rows. The width is a multiple of 1,024 from 2,048 to SITE_FRONT_MOST_WIDTH (a block holds
  * at least one quarter of 256 threads for the dense products and at most 640 threads). The scratch's counters are zero
  * before the first launch (whoever owns the arena clears it once); every launch leaves them zero; launches that share a
@@ -26,13 +29,11 @@ result_status site_front_kernels_prepare(const struct backend_operations *backen
         REFUSE("the kernels of the site fronts: a missing argument");
         return STATUS_INVALID_ARGUMENT;
     }
-    static const char *const names[SITE_FRONT_INSTANCES] = {"site_front_1", "site_front_8", "ffn_front_1", "ffn_front_8", NULL, NULL, NULL, NULL};
+    static const char *const names[SITE_FRONT_INSTANCES] = {"site_front_1", "site_front_8", "ffn_front_1", "ffn_front_8",
+                                                               "input_front_1", "input_front_8", "coefficient_front_1", "coefficient_front_8"};
     struct site_front_kernels kernels;
     for (uint32_t instance = 0; instance < SITE_FRONT_INSTANCES; instance++) {
         kernels.fronts[instance] = BACKEND_NO_KERNEL;
-        if (names[instance] == NULL) {
-            continue; /* the input and coefficient fronts */
-        }
         const result_status status =
             backend->kernel_prepare(card, KERNEL_FILE_SITE_FRONT, names[instance], sizeof(struct site_front_arguments), &kernels.fronts[instance]);
         if (status != STATUS_OK) {
@@ -73,10 +74,6 @@ result_status site_front_prepare(const struct site_front_description *descriptio
     if ((description->router != NULL) != ffn || (router_kernels != NULL) != ffn) {
         REFUSE("%s: a router and its kernels are given together, exactly for the FFN front", what);
         return STATUS_INVALID_ARGUMENT;
-    }
-    if (description->kind == SITE_FRONT_KIND_INPUT || description->kind == SITE_FRONT_KIND_COEFFICIENTS) {
-        REFUSE("%s: the site front cut in an input front and a coefficient front is not built", what);
-        return STATUS_UNSUPPORTED;
     }
     const uint32_t width = description->reserved_zero != 0u ? description->reserved_zero : FRONT_DEFAULT_WIDTH, rows = description->row_count;
     if (rows == 0u || rows > LINEAR_MAXIMUM_ROWS || width < FRONT_LEAST_WIDTH || width > SITE_FRONT_MOST_WIDTH || width % FRONT_WIDTH_STEP != 0u) {
@@ -169,7 +166,10 @@ result_status site_front_prepare(const struct site_front_description *descriptio
     record.operands_offset = description->operands.byte_offset;
     record.scratch_offset = description->scratch.byte_offset;
     record.router_weights_offset = ffn ? description->router_weights.byte_offset : 0u;
-    const uint32_t blocks = rows + site_front_mix_blocks(width) + (ffn ? site_front_score_blocks(width, experts) : 0u);
+    const uint32_t blocks = description->kind == SITE_FRONT_KIND_INPUT          ? rows
+                            : description->kind == SITE_FRONT_KIND_COEFFICIENTS ? site_front_mix_blocks(width)
+                                                                                : rows + site_front_mix_blocks(width) +
+                                                                                      (ffn ? site_front_score_blocks(width, experts) : 0u);
     launch_fill(launch_out, kernels->fronts[instance], blocks, 1, 1, width / HYPER_VALUES_PER_THREAD, 0, &record, sizeof record);
     return STATUS_OK;
 }

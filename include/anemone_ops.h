@@ -216,7 +216,7 @@ MUST_CHECK result_status router_wide_small_prepare(const struct router_wide_desc
 
 /* ---- the fused fronts of a block's sites (include/anemone/site_front.h:38-40, 42-75 of the reference) ---- */
 struct site_front_kernels {
-    uint32_t fronts[SITE_FRONT_INSTANCES]; /* site_front_1, _8, ffn_front_1, _8; the input and coefficient fronts: BACKEND_NO_KERNEL */
+    uint32_t fronts[SITE_FRONT_INSTANCES]; /* site_front_1, _8, ffn_front_1, _8, input_front_1, _8, coefficient_front_1, _8 */
 };
 MUST_CHECK result_status site_front_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                     struct site_front_kernels *kernels_out);
@@ -240,7 +240,7 @@ struct site_front_description {
     uint32_t row_count;
     uint32_t reserved_zero;          /* the width; 0: 5,120 (the reference's model) */
 };
-/* fills ONE launch; the site front cut in two (SITE_FRONT_KIND_INPUT, _COEFFICIENTS) is not built: STATUS_UNSUPPORTED */
+/* fills ONE launch: a whole front, or one of the two the site front is cut in (SITE_FRONT_KIND_INPUT, then _COEFFICIENTS) */
 MUST_CHECK result_status site_front_prepare(const struct site_front_description *description, uint64_t arena_byte_count,
                                             const struct router_kernels_record *router_kernels,
                                             const struct site_front_kernels *kernels, struct kernel_launch *launch_out);

@@ -692,8 +692,9 @@ ANEMONE_RECORD_HAS(dense_linear_arguments, 64);
  * which read the pre it writes, and forms every row's post, comb and pre), then the scores' blocks (they wait for the
  * rows' inputs; the last of them to publish its scores runs the select). A block waits only for blocks of lower tickets,
  * which are running and wait for nothing: the grid ends whatever part of it the card holds at once. No floating-point
- * result depends on the tickets. The last block to leave puts every counter back to zero. The input and coefficient
- * fronts of the reference (the site front cut in two launches) are not built.
+ * result depends on the tickets. The last block to leave puts every counter back to zero. The input front
+ * (the rows' blocks: a row a block, no counter) and then the coefficient front (the mix project's blocks; the last to
+ * publish forms post, comb and pre and clears that counter) are the site front in two launches of one stream.
  *
  * The record is the reference's, 192 bytes: its router_select_arguments (80 bytes there) first, then the fourteen
  * offsets. What this build's select takes beside the reference's members (expert count, picks a row, affinity kind, route
@@ -711,8 +712,8 @@ ANEMONE_RECORD_HAS(dense_linear_arguments, 64);
 enum site_front_kind {
     SITE_FRONT_KIND_SITE = 0,
     SITE_FRONT_KIND_FFN = 1,
-    SITE_FRONT_KIND_INPUT = 2,        /* not built */
-    SITE_FRONT_KIND_COEFFICIENTS = 3, /* not built */
+    SITE_FRONT_KIND_INPUT = 2,        /* the site front's first half: hidden, codes, exponents, operands */
+    SITE_FRONT_KIND_COEFFICIENTS = 3, /* its second half: the mixes, post, comb, the site's pre */
     SITE_FRONT_KINDS = 4
 };
 #define SITE_FRONT_ROW_FORMS 2u /* one row, 8 */

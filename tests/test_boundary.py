@@ -315,13 +315,13 @@ def front_description(fake, width=4096, rows=8, ffn=False, **changes):
 
 def test_site_front_prepare(fake):
     """One launch of blocks of width / 8 threads (the rows', the mix project's, the scores'); the FFN front's record carries the router select's record; the
-    reference's refusals (site_front.h:42-75) and this build's (the front cut in two; widths above 5,120)."""
+    reference's refusals (site_front.h:42-75) and this build's (widths above 5,120); the two launches the site front may be cut in."""
     lib = amd.library()
     kernels, router_kernels = amd.SiteFrontKernels(), amd.RouterKernels()
     assert lib.site_front_kernels_prepare(fake.address, fake.card, C.byref(kernels)) == 0
     assert lib.router_kernels_prepare(fake.address, fake.card, C.byref(router_kernels)) == 0
     assert [fake.handles[k][1] for k in kernels.fronts[0:4]] == ["site_front_1", "site_front_8", "ffn_front_1", "ffn_front_8"]
-    assert list(kernels.fronts[4:8]) == [amd.BACKEND_NO_KERNEL] * 4
+    assert [fake.handles[k][1] for k in kernels.fronts[4:8]] == ["input_front_1", "input_front_8", "coefficient_front_1", "coefficient_front_8"]
     launch = amd.launches_of(1)
     d, keep = front_description(fake)
     assert lib.site_front_prepare(C.byref(d), ARENA, None, C.byref(kernels), launch) == 0
@@ -332,6 +332,11 @@ def test_site_front_prepare(fake):
     one, keep = front_description(fake, width=5120, rows=1, reserved_zero=0)
     assert lib.site_front_prepare(C.byref(one), ARENA, None, C.byref(kernels), launch) == 0
     assert fake.handles[launch[0].kernel][1] == "site_front_1" and list(launch[0].grid) == [1 + 6, 1, 1] and launch[0].block[0] == 640
+    for kind, name, blocks in ((amd.SITE_FRONT_KIND_INPUT, "input_front_8", 8), (amd.SITE_FRONT_KIND_COEFFICIENTS, "coefficient_front_8", 6)):
+        half, keep = front_description(fake, kind=kind)
+        assert lib.site_front_prepare(C.byref(half), ARENA, None, C.byref(kernels), launch) == 0
+        assert fake.handles[launch[0].kernel][1] == name and list(launch[0].grid) == [blocks, 1, 1] and launch[0].block[0] == 512
+        assert bytes(launch[0].argument)[:192] == bytes(record), "the halves take the site front's record"
     f, keep = front_description(fake, ffn=True)
     assert lib.site_front_prepare(C.byref(f), ARENA, C.byref(router_kernels), C.byref(kernels), launch) == 0
     assert fake.handles[launch[0].kernel][1] == "ffn_front_8" and list(launch[0].grid) == [8 + 6 + 32, 1, 1]
@@ -341,7 +346,7 @@ def test_site_front_prepare(fake):
     words = np.frombuffer(bytes(launch[0].argument)[72:80], dtype=np.uint32)
     assert words[0] == 8 and words[1] == (0 | 256 << 1 | 8 << 11 | 1 << 15 | 0x3E00 << 16)
     assert np.frombuffer(bytes(launch[0].argument)[:192], dtype=np.uint64)[23] == f.router_weights.byte_offset
-    refusals = [(dict(kind=amd.SITE_FRONT_KIND_INPUT), False, 7), (dict(kind=amd.SITE_FRONT_KIND_COEFFICIENTS), False, 7), (dict(kind=4), False, 1),
+    refusals = [(dict(kind=amd.SITE_FRONT_KIND_INPUT), True, 1), (dict(kind=amd.SITE_FRONT_KIND_COEFFICIENTS), True, 1), (dict(kind=4), False, 1),
                 (dict(row_count=0), False, 1), (dict(row_count=9), False, 1), (dict(reserved_zero=6144), False, 1), (dict(reserved_zero=1024), False, 1),
                 (dict(reserved_zero=4100), False, 1), (dict(reserved_zero=2304), False, 1), (dict(kind=amd.SITE_FRONT_KIND_FFN), False, 1), (dict(kind=amd.SITE_FRONT_KIND_SITE), True, 1),
                 (dict(hidden=amd.Range(1 << 21, 8 * 4096 * 2)), False, 1), (dict(scale=amd.Range(1 << 30, 16)), False, 1),

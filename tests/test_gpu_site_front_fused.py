@@ -96,6 +96,43 @@ def test_site_front_equals_its_launches(amd, card, rows, width, live):
     assert all(again[name].tobytes() == want[name].tobytes() for name in SITE_OUTPUTS)
 
 
+@pytest.mark.parametrize("rows,width,live", [(8, 4096, 8), (1, 5120, 1), (5, 3072, 3)])
+def test_the_two_halves_equal_the_site_front(amd, card, rows, width, live):
+    """The input front and then the coefficient front (site_front_records.h:24-28 of the reference): the first stores hidden,
+    codes, exponents and operands and leaves pre, post and comb alone; the second the mixes, post, comb and the site's pre."""
+    say("site front in two launches", rows, width, live)
+    front, streams, carried = front_of(amd, card, rows, width, 5 * rows + width)
+    whole = front.front_launch(live)
+    first = front.front_launch(live, kind=amd.SITE_FRONT_KIND_INPUT)
+    second = front.front_launch(live, kind=amd.SITE_FRONT_KIND_COEFFICIENTS)
+    poison(card, front.ranges, SITE_OUTPUTS[1:])
+    card.run(whole)
+    want = snapshot(card, front.ranges, SITE_OUTPUTS)
+    want_scratch = front.read("scratch", np.uint8).copy()
+    front.set_streams(streams, carried)
+    before_pre = front.read("carried_pre", np.uint8).copy()
+    poison(card, front.ranges, SITE_OUTPUTS[1:])
+    card.upload(front.ranges["scratch"].byte_offset, np.zeros(amd.SITE_FRONT_SCRATCH_BYTES, np.uint8))
+    card.run(first)
+    middle = snapshot(card, front.ranges, SITE_OUTPUTS)
+    for name in ("hidden", "codes", "exponents", "operands"):
+        assert middle[name].tobytes() == want[name].tobytes(), name
+    assert middle["carried_pre"].tobytes() == before_pre.tobytes() and np.all(middle["post"] == 0xEE) and np.all(middle["comb"] == 0xEE)
+    card.run(second)
+    got = snapshot(card, front.ranges, SITE_OUTPUTS)
+    for name in SITE_OUTPUTS:
+        assert got[name].tobytes() == want[name].tobytes(), name
+    scratch = front.read("scratch", np.uint8)
+    assert not scratch[:16].any() and not scratch[16 + 768:16 + 776].any(), "the counters are zero again"
+    assert scratch[16:16 + live * MIXES * 4].tobytes() == want_scratch[16:16 + live * MIXES * 4].tobytes(), "the mixes in the scratch"
+    # again without clearing anything: the second half left its counter zero
+    front.set_streams(streams, carried)
+    card.run(first)
+    card.run(second)
+    again = snapshot(card, front.ranges, SITE_OUTPUTS)
+    assert all(again[name].tobytes() == want[name].tobytes() for name in SITE_OUTPUTS)
+
+
 def fp4_layer(amd, card, hidden, inner, experts_n, picks, rows, distinct=4, **keywords):
     from anemone_amd import workloads
     trios = [[workloads.fp4_matrix(9000 + 3 * e, inner, hidden), workloads.fp4_matrix(9001 + 3 * e, inner, hidden),
