@@ -133,22 +133,81 @@ ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_projection, router_projection_argument
  * fmaf over wide exponent ranges, subnormal products and infinities): a block is a chain, its 16 x 16 sums the chains
  * of 16 experts by 16 rows, and the eight instructions of a group of 32 inputs advance the 32 chains by one input
  * each, in the definition's order. Instruction q takes the chains 8 b + q of the blocks b = 0 .. 3, so that lane
- * (b, n) needs the inputs 32 i + 8 b + {0 .. 7} of expert n (and of row n): one 16-byte load each a group. The fold is
- * inside a lane. grid (E / 16, ceil(rows / 64)), block 256: a wavefront 16 rows. */
+ * (b, n) needs the inputs 32 i + 8 b + {0 .. 7} of expert n (and of row n): one 16-byte piece each a group. The fold is
+ * inside a lane. grid (E / 16, ceil(rows / 64)), block 256: a wavefront 16 rows.
+ *
+ * The pieces pass through LDS. Read by the lanes that use them they would be 64 bytes of each of sixteen rows an
+ * instruction, rows a power of two apart: half-used lines that fall into the same few sets of the first-level cache, and
+ * the wavefronts waited for them three quarters of their time. Instead a stage of PROJECTION_STAGE_INPUTS inputs of the
+ * block's 16 experts and 64 rows (80 rows of 256 bytes) is brought by 20 loads of a wavefront that go from memory
+ * straight into LDS, each 256 contiguous bytes of four rows; piece p of tile row R lies at slot p ^ (R % 16) of its row,
+ * so that the eight lanes of a 16-byte read (eight rows, one piece) meet eight different bank groups. Three stages: the
+ * stage two ahead is asked for behind the barrier that ends the stage before the current one. */
 typedef __attribute__((ext_vector_type(16))) float float16_t;
+#define PROJECTION_STAGE_ROW_BYTES (PROJECTION_STAGE_INPUTS * 2u)
+#define PROJECTION_STAGE_ROWS (16u + PROJECTION_TILE_ROWS)
+#define PROJECTION_STAGE_BYTES (PROJECTION_STAGE_ROWS * PROJECTION_STAGE_ROW_BYTES)
+#define PROJECTION_STAGES 3u
+#define PROJECTION_WAVE_LOADS (PROJECTION_STAGE_BYTES / 1024u / (PROJECTION_TILE_THREADS / WAVE)) /* 5 */
+
+/* a group of 32 inputs: eight instructions, each one input further on the four chains it takes */
+__device__ static __forceinline__ void projection_tile_group(const uint4_t &w_now, const uint4_t &x_now, float16_t (&chain)[8])
+{
+    const uint32_t w_words[4] = {w_now.x, w_now.y, w_now.z, w_now.w}, x_words[4] = {x_now.x, x_now.y, x_now.z, x_now.w};
+#pragma unroll
+    for (uint32_t q = 0; q < 8u; q++) {
+        const float a = __uint_as_float(q % 2u == 0u ? w_words[q / 2u] << 16 : w_words[q / 2u] & 0xFFFF0000u);
+        const float b = __uint_as_float(q % 2u == 0u ? x_words[q / 2u] << 16 : x_words[q / 2u] & 0xFFFF0000u);
+        chain[q] = __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, chain[q], 0, 0, 0);
+    }
+}
+
+/* 16 bytes a lane from memory straight into LDS (lane L lands at lds_base + 16 L). Written as assembly: the compiler keeps
+ * no book on it, so the waits for it are written out where a stage is needed. */
+__device__ static __forceinline__ void projection_load_to_lds(const void *lane_address, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_address), "s"(lds_base) : "memory", "m0");
+}
+
 extern "C" __global__ void __launch_bounds__(PROJECTION_TILE_THREADS, 2) /* two blocks a CU: two wavefronts a SIMD */
     router_projection_tiles(struct router_projection_arguments arguments, unsigned char *arena)
 {
-    const uint32_t lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, block = lane / 16u, index = lane % 16u;
+    __shared__ __attribute__((aligned(1024))) unsigned char window[PROJECTION_STAGES * PROJECTION_STAGE_BYTES];
+    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), block = lane / 16u, index = lane % 16u;
     const uint32_t H = arguments.hidden, groups = H / PROJECTION_CHAINS;
-    const uint32_t first_expert = blockIdx.x * 16u, first_row = (blockIdx.y * (PROJECTION_TILE_THREADS / WAVE) + wave) * 16u;
-    if (first_row >= arguments.row_count) {
-        return; /* the whole wavefront */
+    const uint32_t stages = groups / 4u; /* whole stages: whoever prepares the launch holds the width to a multiple of PROJECTION_STAGE_INPUTS */
+    const uint32_t first_expert = blockIdx.x * 16u, block_row = blockIdx.y * PROJECTION_TILE_ROWS, first_row = block_row + wave * 16u;
+    const uint32_t window_address = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)window;
+    /* what this wavefront brings of a stage: the loads wave, wave + 4, ...; load d is the tile rows 4 d .. 4 d + 3 (the
+     * experts' rows first, then the block's rows; a row past the last repeats the last: its sums are not stored) */
+    const unsigned char *source[PROJECTION_WAVE_LOADS];
+    uint32_t piece_bytes[PROJECTION_WAVE_LOADS];
+#pragma unroll
+    for (uint32_t part = 0; part < PROJECTION_WAVE_LOADS; part++) {
+        const uint32_t tile_row = 4u * (wave + 4u * part) + lane / 16u;
+        piece_bytes[part] = 16u * ((lane % 16u) ^ (tile_row % 16u));
+        if (tile_row < 16u) {
+            source[part] = arena + arguments.weights_offset + (uint64_t)(first_expert + tile_row) * H * 2u;
+        } else {
+            const uint32_t row = block_row + tile_row - 16u;
+            source[part] = arena + arguments.rows_offset + (uint64_t)(row < arguments.row_count ? row : arguments.row_count - 1u) * H * 2u;
+        }
     }
-    /* a row past the last repeats the last: its sums are not stored */
-    const uint32_t row = first_row + index < arguments.row_count ? first_row + index : arguments.row_count - 1u;
-    const uint4_t *w = (const uint4_t *)((const uint16_t *)(arena + arguments.weights_offset) + (uint64_t)(first_expert + index) * H + 8u * block);
-    const uint4_t *x = (const uint4_t *)((const uint16_t *)(arena + arguments.rows_offset) + (uint64_t)row * H + 8u * block);
+    auto ask = [&](uint32_t stage) {
+        const uint32_t base = window_address + (stage % PROJECTION_STAGES) * PROJECTION_STAGE_BYTES;
+#pragma unroll
+        for (uint32_t part = 0; part < PROJECTION_WAVE_LOADS; part++) {
+            projection_load_to_lds(source[part] + stage * PROJECTION_STAGE_ROW_BYTES + piece_bytes[part], base + (wave + 4u * part) * 1024u);
+        }
+    };
+    /* where lane (b, n) reads its pieces of group i of a stage: piece 4 i + b of expert n and of the wavefront's row n */
+    uint32_t w_at[4], x_at[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; i++) {
+        const uint32_t slot = 16u * ((4u * i + block) ^ index);
+        w_at[i] = index * PROJECTION_STAGE_ROW_BYTES + slot;
+        x_at[i] = (16u + 16u * wave + index) * PROJECTION_STAGE_ROW_BYTES + slot;
+    }
     float16_t chain[8];
 #pragma unroll
     for (uint32_t q = 0; q < 8u; q++) {
@@ -157,33 +216,33 @@ extern "C" __global__ void __launch_bounds__(PROJECTION_TILE_THREADS, 2) /* two 
             chain[q][v] = 0.0f;
         }
     }
-    /* PROJECTION_TILE_AHEAD groups are asked for ahead of the one in use (a group is 32 bfloat16: four 16-byte pieces
-     * on); the ring is indexed by constants: the loop is unrolled by its length */
-    uint4_t w_ring[PROJECTION_TILE_AHEAD], x_ring[PROJECTION_TILE_AHEAD];
-#pragma unroll
-    for (uint32_t ahead = 0; ahead < PROJECTION_TILE_AHEAD; ahead++) {
-        const uint32_t group = ahead < groups ? ahead : groups - 1u;
-        w_ring[ahead] = w[4u * group];
-        x_ring[ahead] = x[4u * group];
+    ask(0u);
+    if (stages > 1u) {
+        ask(1u);
     }
-    for (uint32_t first = 0; first < groups; first += PROJECTION_TILE_AHEAD) {
+    for (uint32_t stage = 0; stage < stages; stage++) {
+        /* this wavefront's loads of the stage have landed (the next stage's may be under way), then every wavefront's;
+         * behind the barrier every wavefront is through the stage before, whose window the stage two ahead takes */
+        if (stage + 1u < stages) {
+            asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PROJECTION_WAVE_LOADS) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __syncthreads();
+        if (stage + 2u < stages) {
+            ask(stage + 2u);
+        }
+        const unsigned char *now = window + (stage % PROJECTION_STAGES) * PROJECTION_STAGE_BYTES;
+        uint4_t w_now = *(const uint4_t *)(now + w_at[0]), x_now = *(const uint4_t *)(now + x_at[0]);
 #pragma unroll
-        for (uint32_t slot = 0; slot < PROJECTION_TILE_AHEAD; slot++) {
-            const uint32_t group = first + slot;
-            if (group >= groups) { /* the same in every lane */
-                break;
+        for (uint32_t i = 0; i < 4u; i++) {
+            const uint4_t w_use = w_now, x_use = x_now;
+            if (i + 1u < 4u) { /* the next group's pieces are on their way behind this group's instructions */
+                w_now = *(const uint4_t *)(now + w_at[i + 1u]);
+                x_now = *(const uint4_t *)(now + x_at[i + 1u]);
+                __builtin_amdgcn_sched_barrier(0); /* asked for here, not behind the group's instructions */
             }
-            const uint4_t w_now = w_ring[slot], x_now = x_ring[slot];
-            const uint32_t next = group + PROJECTION_TILE_AHEAD < groups ? group + PROJECTION_TILE_AHEAD : groups - 1u;
-            w_ring[slot] = w[4u * next];
-            x_ring[slot] = x[4u * next];
-            const uint32_t w_words[4] = {w_now.x, w_now.y, w_now.z, w_now.w}, x_words[4] = {x_now.x, x_now.y, x_now.z, x_now.w};
-#pragma unroll
-            for (uint32_t q = 0; q < 8u; q++) {
-                const float a = __uint_as_float(q % 2u == 0u ? w_words[q / 2u] << 16 : w_words[q / 2u] & 0xFFFF0000u);
-                const float b = __uint_as_float(q % 2u == 0u ? x_words[q / 2u] << 16 : x_words[q / 2u] & 0xFFFF0000u);
-                chain[q] = __builtin_amdgcn_mfma_f32_16x16x1f32(a, b, chain[q], 0, 0, 0);
-            }
+            projection_tile_group(w_use, x_use, chain);
         }
     }
     /* register v = 4 b + r of chain[q] is chain 8 b + q of expert 4 (lane / 16) + r and row lane % 16. The fold, as the

@@ -7,7 +7,8 @@
  *
  *   launch        kernel                grid                        block
  *   projection    router_projection     (ceil(E / 8), ceil(rows / 4), 1)   128   eight experts and four rows a block
- *                 router_projection_tiles (E / 16, ceil(rows / 64), 1)     256   257 rows and more: 16 experts by 64 rows a block
+ *                 router_projection_tiles (E / 16, ceil(rows / 64), 1)     256   257 rows and more of a width in whole 128, E in whole 16:
+ *                                                                                16 experts by 64 rows a block
  *   select        router_select_entry   (1, 1, 1)                   512   a wavefront a row
  *   wide select   router_wide_select    (ceil(rows / 8), 1, 1)      512   a wavefront a row
  *   wide count    router_wide_count     (ceil(rows / 384), 1, 1)    512   a thread an expert
@@ -249,7 +250,8 @@ result_status router_projection_prepare(const struct router_projection_descripti
         .expert_count = description->expert_count,
     };
     if (kernels->projection_tiles != BACKEND_NO_KERNEL && description->row_count >= PROJECTION_TILE_LEAST_ROWS &&
-        description->expert_count % 16u == 0) { /* many rows: the chains on the matrix unit, 16 experts by 64 rows a block */
+        description->expert_count % 16u == 0 &&
+        description->hidden % PROJECTION_STAGE_INPUTS == 0) { /* many rows: the chains on the matrix unit, 16 experts by 64 rows a block */
         launch_fill(launch_out, kernels->projection_tiles, description->expert_count / 16u,
                     (description->row_count + PROJECTION_TILE_ROWS - 1u) / PROJECTION_TILE_ROWS, 1, PROJECTION_TILE_THREADS, 0, &record,
                     sizeof record);

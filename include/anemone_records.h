@@ -108,7 +108,7 @@ ANEMONE_RECORD_HAS(wide_expert_tile, 32);
 #define PROJECTION_TILE_THREADS 256u
 #define PROJECTION_TILE_ROWS 64u   /* rows of a block of router_projection_tiles: 16 a wavefront */
 #define PROJECTION_TILE_LEAST_ROWS 257u /* fewer rows take router_projection: its blocks are smaller and more */
-#define PROJECTION_TILE_AHEAD 4u        /* groups of 32 inputs asked for ahead */
+#define PROJECTION_STAGE_INPUTS 128u     /* inputs of a stage of router_projection_tiles: the width is a whole number of them */
 #define KERNEL_ROUTER_SELECT "router_select_entry"
 #define KERNEL_ROUTER_WIDE_SELECT "router_wide_select"
 #define KERNEL_ROUTER_WIDE_COUNT "router_wide_count"

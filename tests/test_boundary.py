@@ -263,6 +263,31 @@ def router_description(fake, **changes):
     return d, experts, offsets
 
 
+def test_router_projection_prepare_geometry(fake):
+    """Which kernel takes a projection: many rows of a width in whole 128 inputs go to the matrix unit (16 experts by 64
+    rows a block); any other width, and thin steps, to router_projection (eight experts a block)."""
+    lib = amd.library()
+    kernels = amd.RouterKernels()
+    assert lib.router_kernels_prepare(fake.address, fake.card, C.byref(kernels)) == 0
+
+    def prepared(rows, hidden, experts_n):
+        d = amd.RouterProjectionDescription(amd.Range(1 << 20, experts_n * hidden * 2), amd.Range(1 << 24, rows * hidden * 2),
+                                            amd.Range(1 << 27, rows * experts_n * 4), rows, hidden, experts_n, 0)
+        launch = amd.launches_of(1)
+        status = lib.router_projection_prepare(C.byref(d), ARENA, C.byref(kernels), launch)
+        return status, (fake.handles[launch[0].kernel][1] if status == 0 else None), list(launch[0].grid), launch[0].block[0]
+
+    assert prepared(300, 512, 64) == (0, "router_projection_tiles", [4, 5, 1], 256)
+    assert prepared(4096, 4096, 256) == (0, "router_projection_tiles", [16, 64, 1], 256)
+    status, name, grid, block = prepared(300, 160, 64)  # no whole number of stages of 128 inputs
+    assert (status, name, grid) == (0, "router_projection", [8, 75, 1])
+    status, name, grid, block = prepared(300, 512, 72)  # no whole number of 16 experts
+    assert (status, name, grid) == (0, "router_projection", [9, 75, 1])
+    status, name, grid, block = prepared(8, 4096, 256)  # a thin step: a row a block
+    assert (status, name, grid) == (0, "router_projection", [32, 8, 1])
+    assert prepared(300, 48, 64)[0] == 1 and prepared(0, 512, 64)[0] == 1  # a width that is no multiple of 32; no row
+
+
 def test_router_prepare(fake):
     lib = amd.library()
     kernels = amd.RouterKernels()
