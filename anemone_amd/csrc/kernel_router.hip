@@ -141,13 +141,14 @@ ANEMONE_KERNEL(KERNEL_FILE_ROUTER, router_projection, router_projection_argument
  * the wavefronts waited for them three quarters of their time. Instead a stage of PROJECTION_STAGE_INPUTS inputs of the
  * block's 16 experts and 64 rows (80 rows of 256 bytes) is brought by 20 loads of a wavefront that go from memory
  * straight into LDS, each 256 contiguous bytes of four rows; piece p of tile row R lies at slot p ^ (R % 16) of its row,
- * so that the eight lanes of a 16-byte read (eight rows, one piece) meet eight different bank groups. Three stages: the
- * stage two ahead is asked for behind the barrier that ends the stage before the current one. */
+ * so that the eight lanes of a 16-byte read (eight rows, one piece) meet eight different bank groups. Two stages (40 KB:
+ * three blocks a CU, which measured faster than three stages and two blocks): the next stage is asked for behind the
+ * barrier that ends the stage before the current one. */
 typedef __attribute__((ext_vector_type(16))) float float16_t;
 #define PROJECTION_STAGE_ROW_BYTES (PROJECTION_STAGE_INPUTS * 2u)
 #define PROJECTION_STAGE_ROWS (16u + PROJECTION_TILE_ROWS)
 #define PROJECTION_STAGE_BYTES (PROJECTION_STAGE_ROWS * PROJECTION_STAGE_ROW_BYTES)
-#define PROJECTION_STAGES 3u
+#define PROJECTION_STAGES 2u
 #define PROJECTION_WAVE_LOADS (PROJECTION_STAGE_BYTES / 1024u / (PROJECTION_TILE_THREADS / WAVE)) /* 5 */
 
 /* a group of 32 inputs: eight instructions, each one input further on the four chains it takes */
@@ -169,7 +170,7 @@ __device__ static __forceinline__ void projection_load_to_lds(const void *lane_a
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_address), "s"(lds_base) : "memory", "m0");
 }
 
-extern "C" __global__ void __launch_bounds__(PROJECTION_TILE_THREADS, 2) /* two blocks a CU: two wavefronts a SIMD */
+extern "C" __global__ void __launch_bounds__(PROJECTION_TILE_THREADS, 3) /* three blocks a CU */
     router_projection_tiles(struct router_projection_arguments arguments, unsigned char *arena)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char window[PROJECTION_STAGES * PROJECTION_STAGE_BYTES];
@@ -217,20 +218,13 @@ extern "C" __global__ void __launch_bounds__(PROJECTION_TILE_THREADS, 2) /* two 
         }
     }
     ask(0u);
-    if (stages > 1u) {
-        ask(1u);
-    }
     for (uint32_t stage = 0; stage < stages; stage++) {
-        /* this wavefront's loads of the stage have landed (the next stage's may be under way), then every wavefront's;
-         * behind the barrier every wavefront is through the stage before, whose window the stage two ahead takes */
-        if (stage + 1u < stages) {
-            asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PROJECTION_WAVE_LOADS) : "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
+        /* this wavefront's loads of the stage have landed, then every wavefront's; behind the barrier every wavefront is
+         * through the stage before, whose window the next stage takes */
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (stage + 2u < stages) {
-            ask(stage + 2u);
+        if (stage + 1u < stages) {
+            ask(stage + 1u);
         }
         const unsigned char *now = window + (stage % PROJECTION_STAGES) * PROJECTION_STAGE_BYTES;
         uint4_t w_now = *(const uint4_t *)(now + w_at[0]), x_now = *(const uint4_t *)(now + x_at[0]);
