@@ -74,6 +74,9 @@ result_status expert_pause_plan(const struct expert_pause *pause, struct expert_
                 slots->next_slot = (slot + 1u) % slots->slot_count;
                 if (slots->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS + 1u] == mark) {
                     REFUSE("%s: none of the %u slots of card %u is free", what, slots->slot_count, pause->card);
+                    for (uint32_t named = 0; named < uploads; named++) { /* nothing went up: these hold no expert */
+                        slots->fields[(uint64_t)uploads_out[named].slot * EXPERT_SLOT_FIELDS] = 0;
+                    }
                     return STATUS_DEVICE_ERROR;
                 }
                 uploads_out[uploads++] = (struct expert_pause_upload){slot, (uint32_t)tag};
@@ -152,9 +155,6 @@ result_status expert_pause_run(const struct backend_operations *backend, struct 
                                            expert_copies + (uint64_t)uploads[index].host_expert * pause->expert_byte_count,
                                            pause->expert_byte_count, &tickets[held]);
             held += status == STATUS_OK ? 1u : 0u;
-            if (status != STATUS_OK) { /* the slot holds no expert whole */
-                slots->fields[(uint64_t)uploads[index].slot * EXPERT_SLOT_FIELDS] = 0;
-            }
         }
     }
     if (status == STATUS_OK && tag_count != 0) {
@@ -169,6 +169,13 @@ result_status expert_pause_run(const struct backend_operations *backend, struct 
     }
     const result_status waited = tickets_wait(backend, card, tickets, held, wait_limit_nanoseconds);
     status = status != STATUS_OK ? status : waited;
+    if (status != STATUS_OK) {
+        /* a copy that did not begin or did not finish: none of this pause's slots is taken to hold its expert whole (the
+         * walk named them before any copy), so a later pause brings the expert up again */
+        for (uint32_t index = 0; index < upload_count; index++) {
+            slots->fields[(uint64_t)uploads[index].slot * EXPERT_SLOT_FIELDS] = 0;
+        }
+    }
     if (upload_count_out != NULL) {
         *upload_count_out = upload_count;
     }

@@ -120,6 +120,7 @@ class CopyBackend:
     def __init__(self, arena_bytes):
         self.arena = np.zeros(arena_bytes, dtype=np.uint8)
         self.log, self.held, self.ticket = [], {}, 0
+        self.fail_upload_number = 0  # the n-th upload from now answers STATUS_DEVICE_ERROR (0: none does)
         self.callbacks = (BEGIN(self.upload), WAIT(self.wait), BEGIN(self.download))
         self.operations = (C.c_void_p * 28)()
         self.operations[7] = C.cast(self.callbacks[0], C.c_void_p)
@@ -128,6 +129,11 @@ class CopyBackend:
         self.card = C.c_void_p(0x2000)
 
     def upload(self, card, offset, source, count, ticket_out):
+        if self.fail_upload_number:
+            self.fail_upload_number -= 1
+            if self.fail_upload_number == 0:
+                self.log.append(("refused", offset, count))
+                return amd.STATUS_DEVICE_ERROR
         self.arena[offset:offset + count] = np.ctypeslib.as_array((C.c_ubyte * count).from_address(source))
         self.ticket += 1
         self.log.append(("up", offset, count))
@@ -195,3 +201,33 @@ def test_run_moves_the_experts_and_the_table():
     assert backend.log == [("down", 1024, 288)]
     assert amd.library().expert_pause_run(C.addressof(backend.operations), backend.card, C.byref(pause), 3, C.byref(slots.state), staging.ctypes.data,
                                           copies.ctypes.data, 10 ** 9, None) == amd.STATUS_INVALID_ARGUMENT  # nine jobs for six slots
+
+
+def test_a_failed_copy_leaves_none_of_the_pause_slots_held():
+    """The walk names the slots before any copy begins: when a copy fails, no slot this pause meant to fill may pass for
+    holding its expert, or a later pause would run the experts on bytes that never came."""
+    backend = CopyBackend(32768)
+    copies = np.zeros((FIRST_HOST_EXPERTS, EXPERT_BYTES), dtype=np.uint8)
+    for e in range(FIRST_HOST_EXPERTS):
+        copies[e] = (np.arange(EXPERT_BYTES) * 5 + 11 * e) % 253
+    slots, pause, staging = CardSlots(SLOTS), pause_record(0), np.zeros(SLOTS, dtype=JOB)
+
+    def run(experts):
+        jobs = jobs_of(0, experts)
+        backend.arena[pause.jobs_offset:pause.jobs_offset + 96 * len(jobs)] = table_of(jobs).view(np.uint8)
+        backend.log.clear()
+        return amd.library().expert_pause_run(C.addressof(backend.operations), backend.card, C.byref(pause), 1, C.byref(slots.state),
+                                              staging.ctypes.data, copies.ctypes.data, 10 ** 9, None)
+
+    assert run([HOST + 4, 1, 2]) == 0 and slots.held() == [4, None, None, None, None, None]
+    backend.fail_upload_number = 2
+    assert run([HOST + 4, HOST + 1, HOST + 2]) == amd.STATUS_DEVICE_ERROR
+    assert [entry[0] for entry in backend.log] == ["down", "up", "refused"], "the pause stops at the copy that fails"
+    assert slots.held() == [4, None, None, None, None, None], "the held expert stays; neither of the two named slots holds one"
+    # the next pause brings both up again, into the slots in turn
+    assert run([HOST + 4, HOST + 1, HOST + 2]) == 0
+    assert [entry[0] for entry in backend.log] == ["down", "up", "up", "up"]
+    held = {expert: slot for slot, expert in enumerate(slots.held()) if expert is not None}
+    assert set(held) == {4, 1, 2}
+    for expert, slot in held.items():
+        assert np.array_equal(backend.arena[SLOTS_OFFSET + slot * SLOT_BYTES:SLOTS_OFFSET + slot * SLOT_BYTES + EXPERT_BYTES], copies[expert])
