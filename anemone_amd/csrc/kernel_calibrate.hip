@@ -32,7 +32,9 @@ ANEMONE_KERNEL("kernel_calibrate", arena_copy, arena_copy_arguments);
  * made of, and how a matrix instruction and vector instructions of one wavefront share the issue. A block is one
  * wavefront; `kind` names the instruction, eight independent chains a lane, `iterations` trips of eight each; kinds 8
  * to 10 are trips of four v_mfma_f32_16x16x32_f16 alone, of eight vector instructions alone, and of the four matrix
- * instructions with two of the vector instructions behind each. The host times the launch; what is written is only there to keep the chains alive. */
+ * instructions with two of the vector instructions behind each; kind 11 is trips of eight v_mfma_f32_16x16x1_4b_f32 (the
+ * router's many-row projection: one fused multiply-add a sum of four 16 x 16 blocks), each on sums of its own. The host
+ * times the launch; what is written is only there to keep the chains alive. */
 struct issue_rate_arguments {
     uint64_t output_offset; /* written: uint32 [grid x 64] */
     uint32_t kind;
@@ -42,6 +44,31 @@ static_assert(sizeof(struct issue_rate_arguments) == 16, "issue_rate_arguments A
 
 typedef _Float16 rate_half8 __attribute__((ext_vector_type(8)));
 typedef float rate_float4 __attribute__((ext_vector_type(4)));
+typedef float rate_float16 __attribute__((ext_vector_type(16)));
+
+/* kind 11: `iterations` trips of eight v_mfma_f32_16x16x1_4b_f32, eight sets of sums */
+__device__ static __forceinline__ float issue_rate_blocks(uint32_t iterations, float left, float right)
+{
+    rate_float16 sums[8];
+    for (uint32_t q = 0; q < 8u; q++) {
+        for (uint32_t v = 0; v < 16u; v++) {
+            sums[q][v] = 0.0f;
+        }
+    }
+    for (uint32_t trip = 0; trip < iterations; trip++) {
+#pragma unroll
+        for (uint32_t q = 0; q < 8u; q++) {
+            asm volatile("v_mfma_f32_16x16x1_4b_f32 %0, %1, %2, %0" : "+v"(sums[q]) : "v"(left), "v"(right));
+        }
+    }
+    float kept = 0.0f;
+    for (uint32_t q = 0; q < 8u; q++) {
+        for (uint32_t v = 0; v < 16u; v++) {
+            kept += sums[q][v];
+        }
+    }
+    return kept;
+}
 
 template <uint32_t KIND>
 __device__ static __forceinline__ void issue_rate_loop(uint32_t iterations, uint32_t (&a)[8], rate_float4 (&sums)[4], rate_half8 left, rate_half8 right)
@@ -86,6 +113,11 @@ extern "C" __global__ void __launch_bounds__(64) issue_rate(struct issue_rate_ar
         right[i] = (_Float16)(float)i;
     }
     rate_float4 sums[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    if (arguments.kind == 11u) { /* the same in every lane */
+        const float kept = issue_rate_blocks(arguments.iterations, (float)(threadIdx.x % 7u) * 0.001f, 1.0f + (float)threadIdx.x * 0.002f);
+        ((uint32_t *)(arena + arguments.output_offset))[blockIdx.x * 64u + threadIdx.x] = (uint32_t)kept;
+        return;
+    }
     switch (arguments.kind) {
     case 0u: issue_rate_loop<0u>(arguments.iterations, a, sums, left, right); break;
     case 1u: issue_rate_loop<1u>(arguments.iterations, a, sums, left, right); break;

@@ -104,7 +104,8 @@ def calibrate(amd):
     # the vector unit's issue rate: one wavefront a block, `waves` wavefronts a SIMD (1,024 SIMDs), eight chains a lane
     rates = {}
     kinds = ["v_mul_lo_u32", "v_sad_u8", "v_bfe_u32", "v_and_b32", "v_pk_fma_f16", "v_alignbit_b32", "v_lshrrev_b32", "v_perm_b32",
-             "4 mfma_16x16x32_f16 a trip", "4 x (v_mul_lo_u32, v_sad_u8) a trip", "4 mfma with 2 of the 8 vector instructions behind each, a trip"]
+             "4 mfma_16x16x32_f16 a trip", "4 x (v_mul_lo_u32, v_sad_u8) a trip", "4 mfma with 2 of the 8 vector instructions behind each, a trip",
+             "v_mfma_f32_16x16x1_4b_f32"]
     iterations, out = 20000, card.reserve(64 << 20)
     probe = amd.launches_of(1)
     probe[0].kernel = card.kernel("kernel_calibrate", "issue_rate", 16)
@@ -117,7 +118,7 @@ def calibrate(amd):
             C.memmove(C.byref(probe[0], type(probe[0]).argument.offset + 8), (C.c_uint32 * 2)(kind, iterations), 8)
             card.run_timed(probe)
             microseconds = min(card.run_timed(probe)[0] for _ in range(2))
-            per = 8.0 if kind < 8 else 1.0  # instructions (or trips) a loop body
+            per = 8.0 if kind < 8 or kind == 11 else 1.0  # instructions (or trips) a loop body
             rates["%d waves a SIMD: %s" % (waves, name)] = round(microseconds * 1e-6 * 2.4e9 / (iterations * per * waves), 2)
     card.close()
     print(json.dumps({"calibrate": "arena_copy", "bytes_read": size, "bytes_written": size, "launch_us": times,
