@@ -156,7 +156,7 @@ def test_wide_small_equals_the_four_launches(amd, card, experts_n, picks, rows, 
     assert np.all(wide.read("counts", np.uint8) == 0xEE)  # the counts scratch stays unwritten
 
 
-@pytest.mark.parametrize("experts_n,rows,hidden,scale", [(64, 300, 512, 1.0), (256, 257, 1024, 1.0), (64, 321, 128, 1e-18), (128, 1000, 256, 3e18), (64, 700, 384, 1.0), (64, 300, 192, 1.0)])
+@pytest.mark.parametrize("experts_n,rows,hidden,scale", [(64, 300, 512, 1.0), (256, 257, 1024, 1.0), (64, 321, 128, 1e-18), (128, 1000, 256, 3e18), (64, 700, 384, 1.0), (64, 300, 192, 1.0), (384, 290, 5120, 1.0)])
 def test_projection_of_many_rows_bit_exact(amd, card, experts_n, rows, hidden, scale):
     """router_projection_tiles (257 rows and more: the 32 chains of a score as matrix-unit products of one input each)
     against the oracle's chains, every bit; scales that put products among the subnormals and near overflow among
