@@ -133,6 +133,41 @@ def test_the_two_halves_equal_the_site_front(amd, card, rows, width, live):
     assert all(again[name].tobytes() == want[name].tobytes() for name in SITE_OUTPUTS)
 
 
+def test_a_wait_that_cannot_end_gives_up_and_every_block_leaves(amd, card):
+    """The waits between the front's blocks are bounded. Forced from the host: the tickets' counter starts at the row count,
+    so no block takes a row and the rows' inputs never come; the block that would form the coefficients waits its bounded
+    number of polls, counts itself in gave_up and leaves without writing; the last block to leave still clears the
+    counters, and the next launch on a clean scratch is whole again."""
+    rows, width = 4, 2048
+    say("site front, a wait that cannot end", rows, width)
+    front, streams, carried = front_of(amd, card, rows, width, 77)
+    fused = front.front_launch(rows)
+    poison(card, front.ranges, SITE_OUTPUTS[1:])
+    card.run(fused)
+    want = snapshot(card, front.ranges, SITE_OUTPUTS)
+    front.set_streams(streams, carried)
+    poison(card, front.ranges, SITE_OUTPUTS[1:])
+    before_pre = front.read("carried_pre", np.uint8).copy()
+    head = np.zeros(4, dtype=np.uint32)
+    head[0] = rows  # tickets
+    card.upload(front.ranges["scratch"].byte_offset, head.view(np.uint8))
+    card.run(fused)
+    scratch = front.read("scratch", np.uint8)
+    counters, tail = scratch[:16].view(np.uint32), scratch[16 + 768:16 + 776].view(np.uint32)
+    assert not counters.any() and tail[0] == 0, "the last block to leave cleared the counters"
+    assert tail[1] == 1, "one block gave up: the one that waits for the rows before it forms the coefficients"
+    got = snapshot(card, front.ranges, SITE_OUTPUTS)
+    assert got["carried_pre"].tobytes() == before_pre.tobytes()
+    for name in SITE_OUTPUTS[1:]:
+        assert np.all(got[name] == 0xEE), name
+    # gave_up is the caller's to read and clear; then the front is whole again
+    card.upload(front.ranges["scratch"].byte_offset + 16 + 768 + 4, np.zeros(4, dtype=np.uint8))
+    card.run(fused)
+    again = snapshot(card, front.ranges, SITE_OUTPUTS)
+    assert all(again[name].tobytes() == want[name].tobytes() for name in SITE_OUTPUTS)
+    assert not front.read("scratch", np.uint8)[16 + 768:16 + 776].any()
+
+
 def fp4_layer(amd, card, hidden, inner, experts_n, picks, rows, distinct=4, **keywords):
     from anemone_amd import workloads
     trios = [[workloads.fp4_matrix(9000 + 3 * e, inner, hidden), workloads.fp4_matrix(9001 + 3 * e, inner, hidden),
