@@ -129,151 +129,197 @@ result_status expert_producer_prepare(const struct linear_routed_experts_descrip
     return STATUS_OK;
 }
 
-/* ---- the join and the shared join ---- */
-#define JOIN_ROW_VALUES (HYPER_VALUES_PER_THREAD * HYPER_PIECE_THREADS) /* values of a row a block of a join takes */
-#define JOIN_MOST_ROWS 65535u
-#define JOIN_DEFAULT_WIDTH 5120u /* the reference's model */
-enum { JOIN_RANGES = 6, DOWN_RANGES = 4 };
+/* ---- the join and the shared join ---------------------------------------------------------------------------------
+ * Written from the contract of the reference's include/anemone/expert_fused.h:63-101: what a join reads (the routed
+ * experts' pair outputs, the shared expert's rows, the four streams, the row's post and comb) and what it writes (the
+ * streams in place and, where the caller gives them room, the routed row sums). */
 
-static uint32_t join_width_of(const struct expert_join_description *join)
-{
-    return join->width == 0 ? JOIN_DEFAULT_WIDTH : join->width;
-}
+/* what a join's description comes to once read: the counts every range's size is made of */
+struct join_extent {
+    uint64_t rows;
+    uint64_t pairs;      /* rows times the picks of a row */
+    uint32_t width;      /* of a stream's row; the description's 0 stands for the reference's model */
+    uint32_t row_blocks; /* blocks that share a row: grid[0] */
+    bool stores_sums;
+};
 
-static bool join_counts_are_valid(const char *what, const struct expert_join_description *join, uint32_t most_rows)
+static const uint32_t join_block_values = HYPER_VALUES_PER_THREAD * HYPER_PIECE_THREADS;
+
+static bool join_extent_read(const char *who, const struct expert_join_description *join, uint32_t row_limit, struct join_extent *extent_out)
 {
-    const uint32_t width = join_width_of(join);
-    if (join->row_count == 0 || join->row_count > most_rows || join->pairs_per_row == 0 || width % JOIN_ROW_VALUES != 0 ||
-        (uint64_t)join->row_count * join->pairs_per_row > UINT32_MAX) {
-        REFUSE("%s: %u rows, %u pairs a row, %u wide: it takes 1 to %u rows, a pair or more, a width that is a multiple of %u", what,
-               join->row_count, join->pairs_per_row, width, most_rows, JOIN_ROW_VALUES);
+    struct join_extent extent;
+    extent.width = join->width != 0 ? join->width : 5120u;
+    extent.rows = join->row_count;
+    extent.pairs = extent.rows * join->pairs_per_row;
+    extent.row_blocks = extent.width / join_block_values;
+    extent.stores_sums = join->row_sums.byte_count != 0;
+    const bool counts_fit = extent.rows >= 1 && extent.rows <= row_limit && join->pairs_per_row >= 1 && extent.pairs <= UINT32_MAX;
+    if (!counts_fit || extent.row_blocks * join_block_values != extent.width) {
+        REFUSE("%s: the join is built for 1..%u rows of one pick or more and rows of whole %u values; asked: %u rows, %u picks, %u values",
+               who, row_limit, join_block_values, join->row_count, join->pairs_per_row, extent.width);
         return false;
     }
+    *extent_out = extent;
     return true;
 }
 
-/* the ranges of a join, the row sums last: JOIN_RANGES of them, or one fewer where it writes no row sums */
-static uint32_t join_ranges_of(const struct expert_join_description *join, struct checked_range *ranges_out)
+/* the ranges of one description, gathered as its parts name them and checked together */
+struct range_list {
+    struct checked_range item[12];
+    uint32_t used;
+};
+
+static void list_range(struct range_list *list, const char *name, struct linear_range range, uint64_t touched, bool exact)
 {
-    const uint64_t rows = join->row_count, width = join_width_of(join);
-    const struct checked_range ranges[JOIN_RANGES] = {
-        {"the pair outputs", join->pair_output, linear_values_byte_count(rows * join->pairs_per_row, width), false},
-        {"the shared expert's output", join->shared_output, linear_values_byte_count(rows, width), false},
-        {"the streams", join->streams, linear_values_byte_count(rows * MODEL_STREAMS, width), false},
-        {"the post", join->post, rows * MODEL_STREAMS * 4u, false},
-        {"the comb", join->comb, rows * MODEL_STREAMS * MODEL_STREAMS * 4u, false},
-        {"the row sums", join->row_sums, linear_sums_byte_count(rows, width), false},
-    };
-    memcpy(ranges_out, ranges, sizeof ranges);
-    return join->row_sums.byte_count != 0 ? JOIN_RANGES : JOIN_RANGES - 1u;
+    const struct checked_range entry = {name, range, touched, exact};
+    list->item[list->used++] = entry;
 }
 
-static uint64_t row_sums_offset_of(const struct expert_join_description *join)
+static void list_join_ranges(struct range_list *list, const struct expert_join_description *join, const struct join_extent *extent)
 {
-    return join->row_sums.byte_count != 0 ? join->row_sums.byte_offset : EXPERT_JOIN_NO_ROW_SUMS;
+    const uint64_t stream_rows = extent->rows * MODEL_STREAMS;
+    list_range(list, "pair_output (bfloat16, a row a pair)", join->pair_output, linear_values_byte_count(extent->pairs, extent->width), false);
+    list_range(list, "shared_output (bfloat16, a row a row)", join->shared_output, linear_values_byte_count(extent->rows, extent->width), false);
+    list_range(list, "streams (bfloat16, four rows a row)", join->streams, linear_values_byte_count(stream_rows, extent->width), false);
+    list_range(list, "post (float32, four a row)", join->post, stream_rows * sizeof(float), false);
+    list_range(list, "comb (float32, four by four a row)", join->comb, stream_rows * MODEL_STREAMS * sizeof(float), false);
+    if (extent->stores_sums) {
+        list_range(list, "row_sums (float32, a row a row)", join->row_sums, linear_sums_byte_count(extent->rows, extent->width), false);
+    }
+}
+
+static bool list_holds(const char *who, const struct range_list *list, uint64_t arena_byte_count)
+{
+    return ranges_are_valid(who, list->item, list->used, arena_byte_count);
 }
 
 result_status expert_join_prepare(const struct expert_join_description *description, uint64_t arena_byte_count,
                                   const struct expert_fused_kernels *kernels, struct kernel_launch *launch_out)
 {
-    static const char what[] = "the join of the FFN site";
-    struct checked_range ranges[JOIN_RANGES];
-    if (description == NULL || kernels == NULL || launch_out == NULL || kernels->join == BACKEND_NO_KERNEL) {
-        REFUSE("%s: a missing argument or an unprepared kernel", what);
+    static const char who[] = "expert_join_prepare";
+    if (description == NULL || kernels == NULL || launch_out == NULL) {
+        REFUSE("%s: description, kernels and launch are all needed", who);
         return STATUS_INVALID_ARGUMENT;
     }
-    if (!join_counts_are_valid(what, description, JOIN_MOST_ROWS) ||
-        !ranges_are_valid(what, ranges, join_ranges_of(description, ranges), arena_byte_count)) {
+    if (kernels->join == BACKEND_NO_KERNEL) {
+        REFUSE("%s: expert_fused_kernels_prepare has not found the join's kernel", who);
         return STATUS_INVALID_ARGUMENT;
     }
-    const struct expert_join_arguments record = {
-        description->pair_output.byte_offset, description->shared_output.byte_offset, description->streams.byte_offset,
-        description->post.byte_offset, description->comb.byte_offset, row_sums_offset_of(description), description->pairs_per_row, 0};
-    launch_fill(launch_out, kernels->join, join_width_of(description) / JOIN_ROW_VALUES, description->row_count, 1,
-                HYPER_PIECE_THREADS, 0, &record, sizeof record);
+    struct join_extent extent;
+    struct range_list list = {.used = 0};
+    if (!join_extent_read(who, description, 65535u, &extent)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    list_join_ranges(&list, description, &extent);
+    if (!list_holds(who, &list, arena_byte_count)) {
+        return STATUS_INVALID_ARGUMENT;
+    }
+    struct expert_join_arguments record;
+    memset(&record, 0, sizeof record);
+    record.pair_output_offset = description->pair_output.byte_offset;
+    record.shared_output_offset = description->shared_output.byte_offset;
+    record.streams_offset = description->streams.byte_offset;
+    record.post_offset = description->post.byte_offset;
+    record.comb_offset = description->comb.byte_offset;
+    record.row_sums_offset = extent.stores_sums ? description->row_sums.byte_offset : EXPERT_JOIN_NO_ROW_SUMS;
+    record.pairs_per_row = description->pairs_per_row;
+    launch_fill(launch_out, kernels->join, extent.row_blocks, description->row_count, 1, HYPER_PIECE_THREADS, 0, &record, sizeof record);
     return STATUS_OK;
 }
 
 result_status expert_post_prepare(const struct expert_join_description *join, uint64_t arena_byte_count, uint32_t kernel,
                                   struct kernel_launch *launch_out)
 {
-    static const char what[] = "the post of the FFN site";
-    struct checked_range ranges[JOIN_RANGES];
+    static const char who[] = "expert_post_prepare";
     if (join == NULL || launch_out == NULL || kernel == BACKEND_NO_KERNEL) {
-        REFUSE("%s: a missing argument or an unprepared kernel", what);
+        REFUSE("%s: the description, the launch and a prepared kernel are needed", who);
         return STATUS_INVALID_ARGUMENT;
     }
-    if (join->row_sums.byte_count == 0) {
-        REFUSE("%s: it reads the row sums: their range has no bytes", what);
+    struct join_extent extent;
+    struct range_list list = {.used = 0};
+    if (!join_extent_read(who, join, 65535u, &extent)) {
         return STATUS_INVALID_ARGUMENT;
     }
-    if (!join_counts_are_valid(what, join, JOIN_MOST_ROWS) || !ranges_are_valid(what, ranges, join_ranges_of(join, ranges), arena_byte_count)) {
+    if (!extent.stores_sums) {
+        REFUSE("%s: the post adds the stored row sums; this description stores none", who);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    list_join_ranges(&list, join, &extent);
+    if (!list_holds(who, &list, arena_byte_count)) {
         return STATUS_INVALID_ARGUMENT;
     }
     const struct hyper_post_arguments record = {join->streams.byte_offset, join->post.byte_offset, join->comb.byte_offset,
                                                 join->shared_output.byte_offset, join->row_sums.byte_offset, 1u, 0};
-    launch_fill(launch_out, kernel, join_width_of(join) / JOIN_ROW_VALUES, join->row_count, 1, HYPER_PIECE_THREADS, 0, &record, sizeof record);
+    launch_fill(launch_out, kernel, extent.row_blocks, join->row_count, 1, HYPER_PIECE_THREADS, 0, &record, sizeof record);
     return STATUS_OK;
+}
+
+/* the built instance of a slice count, or BUILT_INSTANCES */
+static uint32_t instance_of_slices(uint32_t slice_count)
+{
+    for (uint32_t instance = 0; instance < BUILT_INSTANCES; instance++) {
+        if (slice_counts[instance] == slice_count) {
+            return instance;
+        }
+    }
+    return BUILT_INSTANCES;
 }
 
 result_status expert_shared_join_prepare(const struct expert_shared_join_description *description, uint64_t arena_byte_count,
                                          const struct linear_kernels_record *linear_kernels, const struct expert_fused_kernels *kernels,
                                          struct kernel_launch *launch_out)
 {
-    static const char what[] = "the shared join of the FFN site";
-    struct checked_range ranges[DOWN_RANGES + JOIN_RANGES];
-    struct kernel_launch separate;
+    static const char who[] = "expert_shared_join_prepare";
     if (description == NULL || linear_kernels == NULL || kernels == NULL || launch_out == NULL) {
-        REFUSE("%s: a missing argument", what);
+        REFUSE("%s: description, both kernel records and the launch are needed", who);
         return STATUS_INVALID_ARGUMENT;
     }
     const struct expert_join_description *join = &description->join;
-    /* what the down's own launch refuses is refused here, behind its one error line; the launch is discarded */
-    struct linear_trunk_quantized_description down;
-    memset(&down, 0, sizeof down);
-    down.matrices[0] = description->down;
-    down.codes = description->codes;
-    down.exponents = description->exponents;
-    down.operands = description->operands;
-    down.outputs[0] = join->shared_output;
-    down.matrix_count = 1;
-    down.row_count = join->row_count;
-    const result_status status = linear_trunk_quantized_prepare(&down, arena_byte_count, linear_kernels, &separate);
-    if (status != STATUS_OK) {
-        return status;
+    /* The launch is the shared expert's down product with the join behind it. The product's own prepare function is asked
+     * first, on a launch that is thrown away: what it refuses is refused here under its own line. */
+    struct linear_trunk_quantized_description product;
+    struct kernel_launch thrown_away;
+    memset(&product, 0, sizeof product);
+    product.matrix_count = 1;
+    product.matrices[0] = description->down;
+    product.outputs[0] = join->shared_output;
+    product.codes = description->codes;
+    product.exponents = description->exponents;
+    product.operands = description->operands;
+    product.row_count = join->row_count;
+    const result_status product_status = linear_trunk_quantized_prepare(&product, arena_byte_count, linear_kernels, &thrown_away);
+    if (product_status != STATUS_OK) {
+        return product_status;
     }
-    uint32_t instance = 0;
-    while (instance < BUILT_INSTANCES && slice_counts[instance] != description->down.slice_count) {
-        instance++;
-    }
-    if (!join_counts_are_valid(what, join, LINEAR_MAXIMUM_ROWS) || instance == BUILT_INSTANCES ||
-        kernels->shared_join[instance] == BACKEND_NO_KERNEL) {
-        REFUSE("%s: at most %u rows, and a prepared kernel of %u slices", what, LINEAR_MAXIMUM_ROWS, description->down.slice_count);
+    struct join_extent extent;
+    const uint32_t instance = instance_of_slices(description->down.slice_count);
+    if (!join_extent_read(who, join, LINEAR_MAXIMUM_ROWS, &extent)) {
         return STATUS_INVALID_ARGUMENT;
     }
-    const struct matrix_shape_record *shape = &description->down.shape;
-    if (shape->output_size != join_width_of(join)) {
-        REFUSE("%s: down has %u outputs: the streams are %u wide", what, shape->output_size, join_width_of(join));
+    if (instance == BUILT_INSTANCES || kernels->shared_join[instance] == BACKEND_NO_KERNEL) {
+        REFUSE("%s: no prepared kernel for a down product of %u slices", who, description->down.slice_count);
         return STATUS_INVALID_ARGUMENT;
     }
-    const uint64_t rows = join->row_count;
-    const struct checked_range down_ranges[DOWN_RANGES] = {
-        {"down", description->down.stored, description->down.stored.byte_count, true},
-        {"the hidden codes", description->codes, linear_codes_byte_count(rows, shape->input_size), false},
-        {"the hidden exponents", description->exponents, linear_exponents_byte_count(rows, shape->input_size), false},
-        {"the hidden operands", description->operands, 0, false},
-    };
-    memcpy(ranges, down_ranges, sizeof down_ranges);
-    const uint32_t range_count = DOWN_RANGES + join_ranges_of(join, ranges + DOWN_RANGES);
-    if (!ranges_are_valid(what, ranges, range_count, arena_byte_count)) {
+    const uint32_t inputs = description->down.shape.input_size, outputs = description->down.shape.output_size;
+    if (outputs != extent.width) {
+        REFUSE("%s: the down matrix writes rows of %u values into streams of %u", who, outputs, extent.width);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    struct range_list list = {.used = 0};
+    list_range(&list, "down (the stored matrix)", description->down.stored, description->down.stored.byte_count, true);
+    list_range(&list, "codes of the hidden rows", description->codes, linear_codes_byte_count(extent.rows, inputs), false);
+    list_range(&list, "exponents of the hidden rows", description->exponents, linear_exponents_byte_count(extent.rows, inputs), false);
+    list_range(&list, "operands of the hidden rows", description->operands, 0, false);
+    list_join_ranges(&list, join, &extent);
+    if (!list_holds(who, &list, arena_byte_count)) {
         return STATUS_INVALID_ARGUMENT;
     }
     const struct expert_shared_join_arguments record = {
         description->down.stored.byte_offset, description->codes.byte_offset, description->exponents.byte_offset,
         description->operands.byte_offset, join->shared_output.byte_offset, join->pair_output.byte_offset, join->streams.byte_offset,
-        join->post.byte_offset, join->comb.byte_offset, row_sums_offset_of(join), shape->input_size, join->row_count,
-        join->pairs_per_row, join->width};
-    launch_fill(launch_out, kernels->shared_join[instance], (shape->output_size + TRUNK_STRIP_OUTPUTS - 1u) / TRUNK_STRIP_OUTPUTS, 1, 1,
-                64u * description->down.slice_count, 0, &record, sizeof record);
+        join->post.byte_offset, join->comb.byte_offset, extent.stores_sums ? join->row_sums.byte_offset : EXPERT_JOIN_NO_ROW_SUMS, inputs,
+        join->row_count, join->pairs_per_row, join->width};
+    const uint32_t strips = (outputs + TRUNK_STRIP_OUTPUTS - 1u) / TRUNK_STRIP_OUTPUTS;
+    launch_fill(launch_out, kernels->shared_join[instance], strips, 1, 1, 64u * description->down.slice_count, 0, &record, sizeof record);
     return STATUS_OK;
 }

@@ -1,97 +1,170 @@
 /*
- * step_experts.c -- a step's expert pauses: the routed experts a layer keeps in host memory go into the card's slots
- * between the layer's router and its experts. Host code over the backend's copies; what happens, its order and its
- * refusals follow the reference (include/anemone/model_seam.h:193-214; source/step_experts.c:27-168, whose driver-held
- * state is here a struct of the caller's, expert_slots).
+ * step_experts.c -- a step's expert pauses. A layer may keep some of its routed experts in host memory; between the
+ * layer's router and its expert launches the ones the step needs are brought into slots of the card. Written from the
+ * contract of the reference's include/anemone/model_seam.h:193-214 (what a tag is, where a slot lies, that a held expert
+ * does not go up again); the reference's step driver holds the slots' state itself (source/step_experts.c:27-168), here it
+ * is the caller's struct expert_slots.
  *
- * A job names a host expert i of its layer by three offsets equal to slots_offset + 16 i (a tag). At a pause the job
- * table comes back from the card; a first walk marks every slot that holds an expert some job names; a second gives
- * each such job that slot, or else the next slot in turn that no job of this pause marked, into which the expert's
- * bytes go up, and points the job's three offsets into the slot; the job table goes up again where a tag was in it. A
- * job of a tag marks one slot at most and a card has at least as many slots as a step has jobs, so an unmarked slot is
- * always left. expert_pause_plan is the walk alone (no card), expert_pause_run the pause on a card.
+ * expert_pause_plan is the walk over a job table in host memory and touches no card: it reads every job first and refuses
+ * a table with a broken job whole; then the slots whose expert a job names are set aside, and in the table's order each
+ * hosted job is pointed at the slot of its expert, which is the one that holds it or else the first slot from the cursor
+ * on that no job of this pause reads (the expert is then owed an upload and the cursor moves behind that slot).
+ * expert_pause_run is the pause on a card over the backend's copies.
  */
 #include <string.h>
 
 #include "prepare_common.h"
 
-#define TAG_BYTES LINEAR_OFFSET_ALIGNMENT_BYTES
-#define SLOT_PASSES 2u /* the slots that hold their expert; then the others' */
+/* a card's slots a pause can name at once: the walk keeps one bit a slot on its stack */
+#define PAUSE_MOST_SLOTS 4096u
+#define NO_SLOT UINT32_MAX
 
-static uint32_t slot_holding(const struct expert_slots *slots, uint64_t expert)
+enum job_kind { JOB_STAYS, JOB_HOSTED, JOB_BROKEN };
+
+/* What a job's three offsets say. A hosted job's are one value, slots_offset + 16 i with i among the pause's host
+ * experts; a job that stays has all three below slots_offset (or no rows); anything between the two is broken. */
+static enum job_kind job_kind_of(const struct expert_pause *pause, const struct expert_job_record *job, uint32_t *host_expert_out)
 {
-    uint32_t slot = 0;
-    while (slot < slots->slot_count && slots->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS] != expert + 1u) {
-        slot++;
+    const uint64_t floor = pause->slots_offset;
+    const bool any_above = job->gate_offset >= floor || job->up_offset >= floor || job->down_offset >= floor;
+    if (job->row_count == 0 || !any_above) {
+        return JOB_STAYS;
     }
-    return slot;
+    if (job->gate_offset < floor || job->up_offset != job->gate_offset || job->down_offset != job->gate_offset) {
+        return JOB_BROKEN;
+    }
+    const uint64_t distance = job->gate_offset - floor;
+    if (distance % LINEAR_OFFSET_ALIGNMENT_BYTES != 0 || distance / LINEAR_OFFSET_ALIGNMENT_BYTES >= pause->host_expert_count) {
+        return JOB_BROKEN;
+    }
+    *host_expert_out = (uint32_t)(distance / LINEAR_OFFSET_ALIGNMENT_BYTES);
+    return JOB_HOSTED;
+}
+
+/* the card's slots as the walk sees them: who is in a slot, and one bit a slot for "a job of this pause reads it" */
+struct slot_view {
+    uint64_t *fields;
+    uint32_t count;
+    uint64_t in_use[PAUSE_MOST_SLOTS / 64u];
+};
+
+static uint64_t *occupant(const struct slot_view *view, uint32_t slot)
+{
+    return &view->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS];
+}
+
+static uint32_t slot_of_expert(const struct slot_view *view, uint64_t expert)
+{
+    for (uint32_t slot = 0; slot < view->count; slot++) {
+        if (*occupant(view, slot) == expert + 1u) {
+            return slot;
+        }
+    }
+    return NO_SLOT;
+}
+
+static bool in_use(const struct slot_view *view, uint32_t slot)
+{
+    return (view->in_use[slot / 64u] >> (slot % 64u)) & 1u;
+}
+
+static void take(struct slot_view *view, uint32_t slot)
+{
+    view->in_use[slot / 64u] |= (uint64_t)1 << (slot % 64u);
+}
+
+/* the first slot from the cursor on, round the ring once, that no job of this pause reads */
+static uint32_t spare_slot_from(const struct slot_view *view, uint32_t cursor)
+{
+    for (uint32_t step = 0; step < view->count; step++) {
+        const uint32_t slot = (cursor + step) % view->count;
+        if (!in_use(view, slot)) {
+            return slot;
+        }
+    }
+    return NO_SLOT;
 }
 
 result_status expert_pause_plan(const struct expert_pause *pause, struct expert_job_record *jobs, uint64_t job_count,
                                 struct expert_slots *slots, struct expert_pause_upload *uploads_out, uint32_t *upload_count_out,
                                 uint32_t *tag_count_out)
 {
-    static const char what[] = "an expert pause";
-    if (pause == NULL || (jobs == NULL && job_count != 0) || slots == NULL || slots->fields == NULL || uploads_out == NULL ||
-        upload_count_out == NULL || tag_count_out == NULL) {
-        REFUSE("%s: a missing argument", what);
+    if (pause == NULL || slots == NULL || slots->fields == NULL || uploads_out == NULL || upload_count_out == NULL || tag_count_out == NULL ||
+        (job_count != 0 && jobs == NULL)) {
+        REFUSE("expert_pause_plan: every pointer is needed");
         return STATUS_INVALID_ARGUMENT;
     }
-    if (slots->slot_count == 0 || slots->slot_count != pause->slot_count || slots->next_slot >= slots->slot_count ||
-        job_count > slots->slot_count || pause->expert_byte_count > pause->slot_byte_count) {
-        REFUSE("%s: %u slots of the card for the pause's %u, no more jobs (%llu) than slots, an expert no larger than a slot", what,
-               slots->slot_count, pause->slot_count, (unsigned long long)job_count);
+    if (slots->slot_count == 0 || slots->slot_count > PAUSE_MOST_SLOTS || slots->slot_count != pause->slot_count ||
+        slots->next_slot >= slots->slot_count) {
+        REFUSE("expert_pause_plan: the state holds %u slots (cursor %u), the pause speaks of %u; 1..%u are served", slots->slot_count,
+               slots->next_slot, pause->slot_count, PAUSE_MOST_SLOTS);
         return STATUS_INVALID_ARGUMENT;
     }
-    const uint64_t mark = ++slots->pause_mark;
-    uint32_t uploads = 0, tags = 0;
-    for (uint32_t pass = 0; pass < SLOT_PASSES; pass++) {
-        for (uint64_t index = 0; index < job_count; index++) {
-            struct expert_job_record *job = &jobs[index];
-            const uint64_t base = pause->slots_offset;
-            if (job->row_count == 0 || (job->gate_offset < base && job->up_offset < base && job->down_offset < base)) {
-                continue; /* empty, or an expert on the card */
+    if (job_count > slots->slot_count || pause->expert_byte_count > pause->slot_byte_count) {
+        REFUSE("expert_pause_plan: %llu jobs must find room in %u slots and %llu bytes of an expert in a slot's %llu",
+               (unsigned long long)job_count, slots->slot_count, (unsigned long long)pause->expert_byte_count,
+               (unsigned long long)pause->slot_byte_count);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    /* 1. read every job before anything moves: a table with a broken job leaves the slots and the table as they were */
+    uint32_t hosted = 0, host_expert = 0;
+    for (uint64_t j = 0; j < job_count; j++) {
+        const enum job_kind kind = job_kind_of(pause, &jobs[j], &host_expert);
+        if (kind == JOB_BROKEN) {
+            REFUSE("expert_pause_plan: the offsets of job %llu (%llu, %llu, %llu) are not below the slots at %llu and are no tag of the "
+                   "layer's %u host experts either (card %u)",
+                   (unsigned long long)j, (unsigned long long)jobs[j].gate_offset, (unsigned long long)jobs[j].up_offset,
+                   (unsigned long long)jobs[j].down_offset, (unsigned long long)pause->slots_offset, pause->host_expert_count, pause->card);
+            return STATUS_DEVICE_ERROR;
+        }
+        hosted += kind == JOB_HOSTED;
+    }
+    struct slot_view view = {slots->fields, slots->slot_count, {0}};
+    const uint64_t stamp = slots->pause_mark + 1u;
+    /* 2. the experts already in a slot keep it: those slots are out of the spare ones' ring for this pause */
+    for (uint64_t j = 0; j < job_count && hosted != 0; j++) {
+        if (job_kind_of(pause, &jobs[j], &host_expert) == JOB_HOSTED) {
+            const uint32_t slot = slot_of_expert(&view, (uint64_t)pause->first_host_expert + host_expert);
+            if (slot != NO_SLOT) {
+                take(&view, slot);
             }
-            const uint64_t tag = (job->gate_offset - base) / TAG_BYTES; /* where the job holds one */
-            if (job->gate_offset < base || (job->gate_offset - base) % TAG_BYTES != 0 || tag >= pause->host_expert_count ||
-                job->up_offset != job->gate_offset || job->down_offset != job->gate_offset) {
-                REFUSE("%s: job %llu names neither an expert on card %u nor one of the %u in host memory", what,
-                       (unsigned long long)index, pause->card, pause->host_expert_count);
-                return STATUS_DEVICE_ERROR;
-            }
-            uint32_t slot = slot_holding(slots, pause->first_host_expert + tag);
-            if (slot < slots->slot_count) { /* the first walk marks it, the second finds it marked */
-                slots->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS + 1u] = mark;
-            }
-            if (pass == 0) {
-                continue;
-            }
-            if (slot == slots->slot_count) {
-                slot = slots->next_slot;
-                for (uint32_t tried = 1; tried < slots->slot_count && slots->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS + 1u] == mark; tried++) {
-                    slot = (slot + 1u) % slots->slot_count;
-                }
-                slots->next_slot = (slot + 1u) % slots->slot_count;
-                if (slots->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS + 1u] == mark) {
-                    REFUSE("%s: none of the %u slots of card %u is free", what, slots->slot_count, pause->card);
-                    for (uint32_t named = 0; named < uploads; named++) { /* nothing went up: these hold no expert */
-                        slots->fields[(uint64_t)uploads_out[named].slot * EXPERT_SLOT_FIELDS] = 0;
-                    }
-                    return STATUS_DEVICE_ERROR;
-                }
-                uploads_out[uploads++] = (struct expert_pause_upload){slot, (uint32_t)tag};
-                slots->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS] = pause->first_host_expert + tag + 1u;
-                slots->fields[(uint64_t)slot * EXPERT_SLOT_FIELDS + 1u] = mark;
-            }
-            const uint64_t at = base + (uint64_t)slot * pause->slot_byte_count;
-            job->gate_offset = at + pause->matrix_offsets[0];
-            job->up_offset = at + pause->matrix_offsets[1];
-            job->down_offset = at + pause->matrix_offsets[EXPERT_PAUSE_MATRICES - 1u];
-            tags++;
         }
     }
-    *upload_count_out = uploads;
-    *tag_count_out = tags;
+    /* 3. in the table's order every hosted job gets its slot, a spare one from the cursor on where its expert is in none */
+    uint32_t owed = 0, cursor = slots->next_slot;
+    for (uint64_t j = 0; j < job_count && hosted != 0; j++) {
+        struct expert_job_record *job = &jobs[j];
+        if (job_kind_of(pause, job, &host_expert) != JOB_HOSTED) {
+            continue;
+        }
+        const uint64_t expert = (uint64_t)pause->first_host_expert + host_expert;
+        uint32_t slot = slot_of_expert(&view, expert);
+        if (slot == NO_SLOT) {
+            slot = spare_slot_from(&view, cursor);
+            if (slot == NO_SLOT) { /* not reached while a table has no more jobs than the card slots */
+                REFUSE("expert_pause_plan: all %u slots of card %u are read by this pause's jobs", view.count, pause->card);
+                for (uint32_t u = 0; u < owed; u++) {
+                    *occupant(&view, uploads_out[u].slot) = 0;
+                }
+                return STATUS_DEVICE_ERROR;
+            }
+            cursor = (slot + 1u) % view.count;
+            *occupant(&view, slot) = expert + 1u;
+            take(&view, slot);
+            uploads_out[owed].slot = slot;
+            uploads_out[owed].host_expert = host_expert;
+            owed++;
+        }
+        occupant(&view, slot)[1] = stamp;
+        const uint64_t slot_base = pause->slots_offset + (uint64_t)slot * pause->slot_byte_count;
+        job->gate_offset = slot_base + pause->matrix_offsets[0];
+        job->up_offset = slot_base + pause->matrix_offsets[1];
+        job->down_offset = slot_base + pause->matrix_offsets[2];
+    }
+    slots->pause_mark = stamp;
+    slots->next_slot = cursor;
+    *upload_count_out = owed;
+    *tag_count_out = hosted;
     return STATUS_OK;
 }
 
