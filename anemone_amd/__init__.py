@@ -9,6 +9,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY_PATH = os.path.join(HERE, "libanemone_hip.so")
+PROBE_LIBRARY_PATH = os.path.join(HERE, "libanemone_probe.so")
 
 STATUS_OK, STATUS_INVALID_ARGUMENT, STATUS_OUT_OF_MEMORY = 0, 1, 2
 STATUS_DEVICE_ERROR, STATUS_TIMED_OUT, STATUS_UNSUPPORTED, STATUS_BUSY = 5, 6, 7, 8
@@ -238,6 +239,20 @@ JOB_DTYPE = np.dtype([("gate_offset", "<u8"), ("up_offset", "<u8"), ("down_offse
                       ("expert", "<u4"), ("pair_index", "<u4", (8,)), ("route_weight", "<f4", (8,))])
 
 _lib = None
+_probe_lib = None
+
+
+def probe_library():
+    """Loads libanemone_probe.so (the copy, instruction-rate and self-check kernels: measurement and tests, not part of the
+    drop-in library). Its kernel files add themselves to the backend's kernel table as the library is loaded, after which
+    Card.kernel finds them like any other."""
+    global _probe_lib
+    if _probe_lib is None:
+        library()
+        if not os.path.exists(PROBE_LIBRARY_PATH):
+            raise ImportError("%s is missing: run `python -m anemone_amd.build`" % PROBE_LIBRARY_PATH)
+        _probe_lib = C.CDLL(PROBE_LIBRARY_PATH)
+    return _probe_lib
 
 
 def library():

@@ -1,4 +1,7 @@
-"""Builds libanemone_hip.so in place: the C11 host side (gcc) and the HIP backend and kernels (hipcc, gfx950).
+"""Builds libanemone_hip.so in place: the C11 host side (gcc) and the HIP backend and kernels (hipcc, gfx950); and beside it
+libanemone_probe.so, the measurement and self-check kernels (an instruction-rate probe, a plain copy, the exhaustive
+arithmetic checks), which are evidence and tests, not part of the drop-in library: they add themselves to the backend's
+kernel table when that library is loaded.
 
     python -m anemone_amd.build [--jobs N]
 
@@ -13,11 +16,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 INCLUDE = os.path.join(ROOT, "include")
 LIBRARY = os.path.join(HERE, "libanemone_hip.so")
+PROBE_LIBRARY = os.path.join(HERE, "libanemone_probe.so")
+EXPORTS = os.path.join(HERE, "host", "exports.map")
 BUILD = os.path.join(HERE, "build")
 
 HOST_SOURCES = ["status.c", "prepare_common.c", "weight_format.c", "exl3.c", "exl3_tc.c", "router.c", "linear.c", "expert_fused.c", "site.c", "site_front.c", "step_experts.c", "exl3_layout.c"]
-HIP_SOURCES = ["kernel_exl3.hip", "kernel_exl3_tc.hip", "kernel_exl3_tcp.hip", "kernel_router.hip", "kernel_calibrate.hip", "kernel_selfcheck.hip", "kernel_dense_linear.hip", "kernel_activation_quantize.hip", "kernel_wide_linear.hip",
+HIP_SOURCES = ["kernel_exl3.hip", "kernel_exl3_tc.hip", "kernel_exl3_tcp.hip", "kernel_router.hip", "kernel_dense_linear.hip", "kernel_activation_quantize.hip", "kernel_wide_linear.hip",
                "kernel_expert_linear.hip", "kernel_trunk_linear.hip", "kernel_hyper_connection.hip", "kernel_site_front.hip"]
+PROBE_SOURCES = ["kernel_calibrate.hip", "kernel_selfcheck.hip"]
 
 BACKEND_SOURCES = ["backend_hip.cpp"]  # host C++ over the HIP runtime API: no device code
 BACKEND_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include"]
@@ -48,16 +54,19 @@ def build(jobs=8, verbose=False):
         objects.append(target)
         commands.append(["g++", *BACKEND_FLAGS, "-I", INCLUDE, "-I", os.path.join(HERE, "csrc"), "-c",
                          os.path.join(HERE, "csrc", name), "-o", target])
-    for name in HIP_SOURCES:
+    probe_objects = []
+    for name in HIP_SOURCES + PROBE_SOURCES:
         target = os.path.join(BUILD, name + ".o")
-        objects.append(target)
+        (probe_objects if name in PROBE_SOURCES else objects).append(target)
         commands.append(["hipcc", *HIP_FLAGS, "-I", INCLUDE, "-I", os.path.join(HERE, "csrc"), "-c",
                          os.path.join(HERE, "csrc", name), "-o", target])
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         for output in pool.map(run, commands):
             if verbose and output.strip():
                 print(output)
-    run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBRARY, *objects])
+    run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--version-script=" + EXPORTS, "-o", LIBRARY, *objects])
+    run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIBRARY, *probe_objects, "-L", HERE, "-lanemone_hip",
+         "-Wl,-rpath,$ORIGIN"])
     return LIBRARY
 
 

@@ -90,6 +90,7 @@ def queue_steps(card, step, count, graph):
 def calibrate(amd):
     """A copy of 1 GiB inside the arena (1 GiB read, 1 GiB written), five launches."""
     import ctypes as C
+    amd.probe_library()
     size = 1 << 30
     card = amd.Card(3 << 30)
     source, destination = card.reserve(size), card.reserve(size)

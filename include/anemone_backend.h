@@ -197,6 +197,12 @@ MUST_CHECK result_status backend_hip_launch_run_timed(struct device_card *card,
 uint32_t backend_hip_kernel_table_count(void);
 MUST_CHECK result_status backend_hip_kernel_table_entry(uint32_t index, const char **file_out,
                                                         const char **function_out, uint32_t *record_bytes_out);
+/* Adds one kernel to that table: every kernel file of the library does so for its entries before main, and a second
+ * library of kernels linked against this one (the build's libanemone_probe.so: a plain copy, an instruction-rate probe
+ * and exhaustive arithmetic checks, which are measurement and tests and stay out of the drop-in library) does so when it
+ * is loaded. host_function is the kernel's host-side handle; the strings must outlive the table. No counterpart in the
+ * reference, which finds its kernels in module images (source/backend_cuda_kernel_images.h:18-26). */
+void anemone_register_kernel(const char *file, const char *function, const void *host_function, uint32_t record_bytes);
 
 #ifdef __cplusplus
 }

@@ -19,6 +19,7 @@ def test_short_cuts_equal_their_definitions(check, what):
     import anemone_amd as amd
     print("selfcheck", check, what, flush=True)
     sys.stdout.flush()
+    amd.probe_library()
     card = amd.Card(64 << 20)
     try:
         blocks, threads = 4096, 256
