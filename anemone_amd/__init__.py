@@ -81,7 +81,8 @@ class Exl3TcRecord(C.Structure):
     _fields_ = [("jobs_offset", u64), ("hidden_offset", u64), ("workspace_offset", u64), ("output_offset", u64),
                 ("row_count", u32), ("job_capacity", u32), ("intermediate", u32), ("bits_x2", u32),
                 ("activation_limit", f32), ("pass_", u32), ("rotation", u32), ("shared_sum", u32),
-                ("shared_offset", u64), ("widths_offset", u64), ("hidden", u32), ("pairs_per_row", u32)]
+                ("shared_offset", u64), ("widths_offset", u64), ("hidden", u32), ("pairs_per_row", u32), ("expert_count", u32),
+                ("reserved_zero", u32)]
 
 
 class RouterKernels(C.Structure):
@@ -221,6 +222,10 @@ class ExpertSlots(C.Structure):
     _fields_ = [("fields", C.POINTER(u64)), ("pause_mark", u64), ("slot_count", u32), ("next_slot", u32)]
 
 
+class ExpertHostCopies(C.Structure):
+    _fields_ = [("block", C.POINTER(C.c_ubyte)), ("byte_count", u64), ("table_staging_offset", u64)]
+
+
 class ExpertPauseUpload(C.Structure):
     _fields_ = [("slot", u32), ("host_expert", u32)]
 
@@ -322,6 +327,9 @@ def library():
             "expert_pause_run": [vp, vp, C.POINTER(ExpertPause), u32, C.POINTER(ExpertSlots), vp, vp, u64, C.POINTER(u32)],
             "site_front_kernels_prepare": [vp, vp, C.POINTER(SiteFrontKernels)],
             "site_front_prepare": [C.POINTER(SiteFrontDescription), u64, C.POINTER(RouterKernels), C.POINTER(SiteFrontKernels), launch_p],
+            "site_front_check": [vp, vp, Range, vp, u64, C.POINTER(u32)],
+            "expert_host_copies_attach": [vp, C.POINTER(ExpertPause), u32, C.POINTER(u64), u64, vp, u64, u64, u64, C.POINTER(ExpertHostCopies),
+                                          C.POINTER(u64)],
             "expert_post_prepare": [C.POINTER(ExpertJoinDescription), u64, u32, launch_p],
             "expert_shared_join_prepare": [C.POINTER(ExpertSharedJoinDescription), u64, C.POINTER(LinearKernels),
                                            C.POINTER(ExpertFusedKernels), launch_p],
@@ -330,6 +338,8 @@ def library():
             function = getattr(lib, name)
             function.restype = C.c_int
             function.argtypes = argtypes
+        lib.expert_host_copies_detach.restype = None
+        lib.expert_host_copies_detach.argtypes = [vp, C.POINTER(ExpertHostCopies)]
         lib.backend_hip_card_close.restype = None
         lib.backend_hip_card_close.argtypes = [vp, u64]
         lib.backend_hip_staging_free.restype = None
@@ -597,15 +607,21 @@ class Exl3Layer:
             self.pause.matrix_offsets[0], self.pause.matrix_offsets[1], self.pause.matrix_offsets[2] = 0, part_bytes[0], part_bytes[0] + part_bytes[1]
             self.pause.first_host_expert, self.pause.host_expert_count = 0, len(host_experts)
             self.pause.jobs_per_row, self.pause.slot_count = picks, self.pairs
-            copies = C.c_void_p()
-            check(lib.backend_hip_staging_allocate(len(host_experts) * slot_bytes + self.pairs * 96, C.byref(copies)), "staging_allocate")
-            self.pause_staging = copies
-            view = np.ctypeslib.as_array((C.c_ubyte * (len(host_experts) * slot_bytes)).from_address(copies.value))
-            view[:] = 0
+            # the layer's host arena: every host expert's three matrices at the pause's matrix offsets; the page-locked copies
+            # the pauses upload from are the library's to make (expert_host_copies_attach)
+            host_arena = np.zeros(len(host_experts) * slot_bytes, dtype=np.uint8)
             for i, e in enumerate(host_experts):
                 for m in range(3):
                     at = i * slot_bytes + int(self.pause.matrix_offsets[m])
-                    view[at:at + matrices[e][m].nbytes] = matrices[e][m].view(np.uint8).reshape(-1)
+                    host_arena[at:at + matrices[e][m].nbytes] = matrices[e][m].view(np.uint8).reshape(-1)
+            host_offsets = (np.arange(len(host_experts), dtype=np.uint64) * np.uint64(slot_bytes))
+            self.host_copies, pause_offsets = ExpertHostCopies(), (u64 * 1)()
+            check(lib.expert_host_copies_attach(backend_table(), C.byref(self.pause), 1, host_offsets.ctypes.data_as(C.POINTER(u64)), len(host_experts),
+                                                host_arena.ctypes.data, host_arena.nbytes, self.pairs * 96, 64 << 30, C.byref(self.host_copies),
+                                                pause_offsets), "expert_host_copies_attach")
+            base = C.cast(self.host_copies.block, C.c_void_p).value
+            self.pause_copies = C.c_void_p(base + int(pause_offsets[0]))
+            self.pause_table_staging = C.c_void_p(base + int(self.host_copies.table_staging_offset))
             self.slot_fields = np.zeros(2 * self.pairs, dtype=np.uint64)
             self.slots = ExpertSlots(self.slot_fields.ctypes.data_as(C.POINTER(u64)), 0, self.pairs, 0)
         self.expert_offsets = offsets
@@ -635,13 +651,16 @@ class Exl3Layer:
         live = self.rows if live_rows is None else live_rows
         self.card.upload(self.step_offset, step_block(live))
 
+    def release_host_experts(self):
+        """Gives the page-locked copies back (expert_host_copies_detach): after the last pause's uploads have retired."""
+        self.card.lib.expert_host_copies_detach(backend_table(), C.byref(self.host_copies))
+
     def run_pause(self):
         """The layer's expert pause behind its select (expert_pause_run): the experts uploaded."""
         self.pause.jobs_offset = self.jobs_offset
         uploaded = u32(0)
-        jobs_staging = C.c_void_p(self.pause_staging.value + int(self.pause.host_expert_count) * int(self.pause.slot_byte_count))
-        check(self.card.lib.expert_pause_run(backend_table(), self.card.handle, C.byref(self.pause), self.rows, C.byref(self.slots), jobs_staging,
-                                             self.pause_staging, 60 * SECOND, C.byref(uploaded)), "expert_pause_run")
+        check(self.card.lib.expert_pause_run(backend_table(), self.card.handle, C.byref(self.pause), self.rows, C.byref(self.slots),
+                                             self.pause_table_staging, self.pause_copies, 60 * SECOND, C.byref(uploaded)), "expert_pause_run")
         return uploaded.value
 
     def experts_description(self):
@@ -715,6 +734,7 @@ class Exl3Layer:
         r.bits_x2 = {2: 4, 3: 6, 4: 8, 40: 5}.get(self.uniform_width, 8)
         r.activation_limit = self.limit
         r.widths_offset, r.hidden, r.pairs_per_row = self.widths_offset, self.H, self.P
+        r.expert_count = self.E if self.widths_offset else 0
         return r
 
     def tc_launches(self, shared_offset=None):

@@ -331,6 +331,8 @@ result_status wait_for(device_card *card, hipEvent_t event, uint64_t limit_ns)
 
 } // namespace
 
+extern "C" result_status exl3_tc_static_scratch_resolve(void); /* kernel_exl3_tc.hip; private to the library */
+
 extern "C" {
 
 void anemone_register_kernel(const char *file, const char *function, const void *host_function,
@@ -440,6 +442,7 @@ result_status backend_hip_card_open(uint32_t card_index, uint64_t arena_byte_cou
         return STATUS_OUT_OF_MEMORY;
     }
     bool ok = hipStreamCreateWithFlags(&card->stream, hipStreamNonBlocking) == hipSuccess;
+    ok = ok && exl3_tc_static_scratch_resolve() == STATUS_OK; /* the library's array on this device: found once, here */
     for (copy_slot &slot : card->slots) {
         slot.ticket = 0;
         ok = ok && hipEventCreateWithFlags(&slot.event, hipEventDisableTiming) == hipSuccess;

@@ -49,6 +49,9 @@ __device__ static __forceinline__ uint32_t tc_bits_x2(const struct exl3_tc_recor
     if (record.widths_offset == 0u) {
         return record.bits_x2;
     }
+    if (expert >= record.expert_count) {
+        return 0u; /* beyond the table: no width, which every launch treats as a matrix it cannot decode */
+    }
     return exl3_bits_x2(exl3_width_of(((const uint32_t *)(arena + record.widths_offset))[expert], matrix));
 }
 
@@ -353,6 +356,15 @@ static result_status static_scratch_of(unsigned char **address_out)
     }
     *address_out = address_of[device];
     return STATUS_OK;
+}
+
+/* card_open's part of the set-up: the array's address on the card's device (current when this is called) is asked for
+ * there, so that the code object is loaded and the address known before the first step; a call of exl3_tc_run_static on
+ * a device no card was opened on still resolves it itself, once, and that one call is not one to make under capture */
+extern "C" result_status exl3_tc_static_scratch_resolve(void)
+{
+    unsigned char *address = nullptr;
+    return static_scratch_of(&address);
 }
 
 /* kernel_prepare of a table that launches nothing: the four kernels of this file by number */

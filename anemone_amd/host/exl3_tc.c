@@ -63,8 +63,13 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
     }
     const uint64_t pairs = (uint64_t)record->row_count * picks;
     const uint64_t workspace = exl3_tc_workspace_bytes(pairs, hidden, I);
-    /* the table of per-matrix widths, where one is named: uint32 an expert; the record does not say how many experts there
-     * are, so what is held inside the arena and clear of what the launches write is its first word (an expert 0 there is) */
+    /* the table of per-matrix widths, where one is named: uint32 an expert, expert_count of them, inside the arena and
+     * clear of what the launches write; the kernels read no entry beyond it */
+    if (record->reserved_zero != 0 || (mixed ? record->expert_count == 0 : record->expert_count != 0)) {
+        REFUSE("%s: a widths table needs its expert count (%u), a record without one names none, and the reserved word is zero", what,
+               record->expert_count);
+        return STATUS_INVALID_ARGUMENT;
+    }
     struct checked_range ranges[6] = {
         {"the jobs", {record->jobs_offset, (uint64_t)record->job_capacity * sizeof(struct expert_job_record)},
          (uint64_t)record->job_capacity * sizeof(struct expert_job_record), false},
@@ -82,7 +87,8 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
         range_count -= 1u;
     }
     if (mixed) {
-        ranges[range_count++] = (struct checked_range){"the widths", {record->widths_offset, 4u}, 4u, false};
+        const uint64_t table_bytes = (uint64_t)record->expert_count * 4u;
+        ranges[range_count++] = (struct checked_range){"the widths", {record->widths_offset, table_bytes}, table_bytes, false};
     }
     if (!ranges_are_valid(what, ranges, range_count, arena_byte_count) || record->workspace_offset % 256u != 0 ||
         (mixed && record->widths_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0)) {

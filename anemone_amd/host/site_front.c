@@ -14,6 +14,7 @@
  * before the first launch (whoever owns the arena clears it once); every launch leaves them zero; launches that share a
  * scratch run one after the other.
  */
+#include <stddef.h>
 #include <string.h>
 
 #include "prepare_common.h"
@@ -172,4 +173,39 @@ result_status site_front_prepare(const struct site_front_description *descriptio
                                                                                       (ffn ? site_front_score_blocks(width, experts) : 0u);
     launch_fill(launch_out, kernels->fronts[instance], blocks, 1, 1, width / HYPER_VALUES_PER_THREAD, 0, &record, sizeof record);
     return STATUS_OK;
+}
+
+result_status site_front_check(const struct backend_operations *backend, struct device_card *card, struct linear_range scratch,
+                               void *staging, uint64_t wait_limit_nanoseconds, uint32_t *gave_up_out)
+{
+    if (backend == NULL || backend->download_begin == NULL || backend->upload_begin == NULL || backend->upload_wait == NULL || card == NULL ||
+        staging == NULL || scratch.byte_count < SITE_FRONT_SCRATCH_BYTES || scratch.byte_offset % LINEAR_OFFSET_ALIGNMENT_BYTES != 0) {
+        REFUSE("site_front_check: a backend with copies, a card, the front's scratch range and 8 page-locked bytes are needed");
+        return STATUS_INVALID_ARGUMENT;
+    }
+    /* the two words behind the mixes: departed (zero again once a launch has ended) and gave_up */
+    const uint64_t tail = scratch.byte_offset + offsetof(struct site_front_scratch, departed);
+    uint32_t *words = staging;
+    uint64_t ticket = 0;
+    result_status status = backend->download_begin(card, tail, words, 2 * sizeof *words, &ticket);
+    if (status == STATUS_OK) {
+        status = backend->upload_wait(card, ticket, wait_limit_nanoseconds);
+    }
+    if (status != STATUS_OK) {
+        return status;
+    }
+    const uint32_t gave_up = words[1];
+    if (gave_up_out != NULL) {
+        *gave_up_out = gave_up;
+    }
+    if (gave_up == 0) {
+        return STATUS_OK;
+    }
+    REFUSE("site_front_check: %u blocks of a fused front gave their wait up: the outputs of that launch are not whole", gave_up);
+    words[1] = 0; /* the count is read once: the next launch begins on a clean scratch */
+    status = backend->upload_begin(card, tail, words, 2 * sizeof *words, &ticket);
+    if (status == STATUS_OK) {
+        status = backend->upload_wait(card, ticket, wait_limit_nanoseconds);
+    }
+    return status != STATUS_OK ? status : STATUS_DEVICE_ERROR;
 }

@@ -254,3 +254,89 @@ result_status expert_pause_run(const struct backend_operations *backend, struct 
     }
     return status;
 }
+
+/* ---- the page-locked copies a card's pauses upload from ------------------------------------------------------------ */
+
+/* the bytes of a pause's copies, or UINT64_MAX where they leave 64 bits */
+static uint64_t pause_copy_bytes(const struct expert_pause *pause)
+{
+    return product_or_most(pause->expert_byte_count, pause->host_expert_count);
+}
+
+result_status expert_host_copies_attach(const struct backend_operations *backend, const struct expert_pause *pauses, uint32_t pause_count,
+                                        const uint64_t *host_expert_offsets, uint64_t host_expert_count, const void *host_arena,
+                                        uint64_t host_byte_count, uint64_t table_staging_bytes, uint64_t most_bytes,
+                                        struct expert_host_copies *copies_out, uint64_t *pause_offsets_out)
+{
+    if (backend == NULL || backend->staging_allocate == NULL || copies_out == NULL || (pause_count != 0 && (pauses == NULL || pause_offsets_out == NULL))) {
+        REFUSE("expert_host_copies_attach: a backend that allocates page-locked memory, the pauses and both outputs are needed");
+        return STATUS_INVALID_ARGUMENT;
+    }
+    /* first the sizes and every source range, so that a refusal has allocated and written nothing */
+    uint64_t total = 0;
+    for (uint32_t p = 0; p < pause_count; p++) {
+        const struct expert_pause *pause = &pauses[p];
+        const uint64_t bytes = pause_copy_bytes(pause);
+        const uint64_t last = (uint64_t)pause->first_host_expert + pause->host_expert_count;
+        if (pause->host_expert_count == 0 || pause->expert_byte_count == 0 || bytes == UINT64_MAX || last > host_expert_count ||
+            host_expert_offsets == NULL || host_arena == NULL) {
+            REFUSE("expert_host_copies_attach: pause %u speaks of host experts %u..%llu of %llu, %llu bytes each: none, or not all, are in the "
+                   "table of the host arena", p, pause->first_host_expert, (unsigned long long)last, (unsigned long long)host_expert_count,
+                   (unsigned long long)pause->expert_byte_count);
+            return STATUS_INVALID_ARGUMENT;
+        }
+        for (uint64_t e = pause->first_host_expert; e < last; e++) {
+            if (host_expert_offsets[e] > host_byte_count || pause->expert_byte_count > host_byte_count - host_expert_offsets[e]) {
+                REFUSE("expert_host_copies_attach: host expert %llu (%llu bytes at %llu) ends behind the host arena's %llu bytes",
+                       (unsigned long long)e, (unsigned long long)pause->expert_byte_count, (unsigned long long)host_expert_offsets[e],
+                       (unsigned long long)host_byte_count);
+                return STATUS_INVALID_ARGUMENT;
+            }
+        }
+        if (bytes > UINT64_MAX - total) {
+            return STATUS_OUT_OF_MEMORY;
+        }
+        total += bytes;
+    }
+    const uint64_t table_at = (total + 255u) / 256u * 256u;
+    if (table_staging_bytes > UINT64_MAX - table_at || table_at + table_staging_bytes > most_bytes) {
+        REFUSE("expert_host_copies_attach: %llu bytes of experts and %llu of a job table are above the %llu the caller allows",
+               (unsigned long long)total, (unsigned long long)table_staging_bytes, (unsigned long long)most_bytes);
+        return STATUS_OUT_OF_MEMORY;
+    }
+    struct expert_host_copies made = {NULL, table_at + table_staging_bytes, table_at};
+    if (made.byte_count != 0) {
+        void *block = NULL;
+        const result_status status = backend->staging_allocate(made.byte_count, &block);
+        if (status != STATUS_OK) {
+            return status;
+        }
+        if (block == NULL) {
+            return STATUS_OUT_OF_MEMORY;
+        }
+        made.block = block;
+    }
+    uint64_t at = 0;
+    for (uint32_t p = 0; p < pause_count; p++) {
+        const struct expert_pause *pause = &pauses[p];
+        pause_offsets_out[p] = at;
+        for (uint32_t e = 0; e < pause->host_expert_count; e++, at += pause->expert_byte_count) {
+            memcpy(made.block + at, (const unsigned char *)host_arena + host_expert_offsets[(uint64_t)pause->first_host_expert + e],
+                   (size_t)pause->expert_byte_count);
+        }
+    }
+    *copies_out = made;
+    return STATUS_OK;
+}
+
+void expert_host_copies_detach(const struct backend_operations *backend, struct expert_host_copies *copies)
+{
+    if (backend == NULL || copies == NULL) {
+        return;
+    }
+    if (copies->block != NULL && backend->staging_free != NULL) {
+        backend->staging_free(copies->block);
+    }
+    copies->block = NULL;
+    copies->byte_count = copies->table_staging_offset = 0;
+}

@@ -99,7 +99,10 @@ MUST_CHECK result_status exl3_tc_prepare_detached(const struct exl3_tc_record *r
  * `stream` (a hipStream_t; NULL: the default stream) of the current device, with the workspace in an array of
  * EXL3_TC_STATIC_SCRATCH_BYTES that the library holds on every device it has run on, in place of a range of the arena.
  * `arena_device` is the device address the record's offsets count from and `arena_byte_count` the bytes behind it that
- * the record's ranges must lie in; record->workspace_offset is ignored. Allocates nothing and does not wait. A step
+ * the record's ranges must lie in; record->workspace_offset is ignored. Allocates nothing and does not wait: the array's
+ * address on a device is found when card_open opens that device (which loads the library's code there); on a device no
+ * card was opened on, the first call finds it itself, and that one call may load code and must not be made under
+ * capture. A step
  * whose workspace (exl3_tc_workspace_bytes) is larger than the array is refused with STATUS_INVALID_ARGUMENT. Calls on
  * one device share that device's array: two calls whose launches overlap in time race. */
 #define EXL3_TC_STATIC_SCRATCH_BYTES (16u << 20)
@@ -244,6 +247,15 @@ struct site_front_description {
 MUST_CHECK result_status site_front_prepare(const struct site_front_description *description, uint64_t arena_byte_count,
                                             const struct router_kernels_record *router_kernels,
                                             const struct site_front_kernels *kernels, struct kernel_launch *launch_out);
+/* A fused front's blocks wait for each other a bounded number of polls (SITE_FRONT_WAIT_POLLS); one that waits in vain
+ * counts itself in the scratch's gave_up, skips its part and leaves, and the launch still ends like any other. The count is
+ * the caller's to read: this call brings it back from the card (behind every launch queued before it; staging: 8
+ * page-locked bytes), writes it to gave_up_out (may be NULL) and, where it is not zero, clears it on the card and answers
+ * STATUS_DEVICE_ERROR: what that launch wrote is not whole and the step must not go on. STATUS_OK: every block ran its
+ * part. No counterpart in the reference, whose fronts wait without a bound (source/kernel_site_front.cu). */
+MUST_CHECK result_status site_front_check(const struct backend_operations *backend, struct device_card *card,
+                                          struct linear_range scratch, void *staging, uint64_t wait_limit_nanoseconds,
+                                          uint32_t *gave_up_out);
 
 /* ---- host experts: a step's expert pauses (include/anemone/model_seam.h:193-214, source/step_experts.c:27-168 of the
  * reference). Behind a layer's router, whose job table names a host expert i of the layer by three offsets equal to
@@ -290,6 +302,28 @@ MUST_CHECK result_status expert_pause_run(const struct backend_operations *backe
                                           const struct expert_pause *pause, uint32_t row_count, struct expert_slots *slots,
                                           void *jobs_staging, const unsigned char *expert_copies, uint64_t wait_limit_nanoseconds,
                                           uint32_t *upload_count_out);
+
+/* The page-locked copies the pauses of one card upload from: what the reference's step driver makes when host experts are
+ * attached to it (include/anemone/step.h:55, 189; source/step_experts.c:170-240 of the reference: every host expert the
+ * pauses name is copied once out of the host arena into memory from the backend's staging_allocate, a pause's experts
+ * side by side, expert_byte_count apart). Here the block also holds, behind the experts and on a multiple of 256,
+ * table_staging_bytes for the job table expert_pause_run brings back. pause_offsets_out[p] is where pause p's copies
+ * begin: expert_pause_run takes block + pause_offsets_out[p] as expert_copies and block + table_staging_offset as
+ * jobs_staging. host_expert_offsets [host_expert_count] are byte offsets into host_arena (host_byte_count bytes).
+ * STATUS_INVALID_ARGUMENT: a pause without host experts, experts beyond the table or the arena; STATUS_OUT_OF_MEMORY:
+ * more than most_bytes in all, or the backend's answer. A refusal allocates nothing and leaves both outputs untouched. */
+struct expert_host_copies {
+    unsigned char *block;          /* page-locked; NULL: nothing attached */
+    uint64_t byte_count;           /* of the block */
+    uint64_t table_staging_offset; /* in the block */
+};
+MUST_CHECK result_status expert_host_copies_attach(const struct backend_operations *backend, const struct expert_pause *pauses,
+                                                   uint32_t pause_count, const uint64_t *host_expert_offsets,
+                                                   uint64_t host_expert_count, const void *host_arena, uint64_t host_byte_count,
+                                                   uint64_t table_staging_bytes, uint64_t most_bytes,
+                                                   struct expert_host_copies *copies_out, uint64_t *pause_offsets_out);
+/* gives the block back to the backend (when every upload from it has retired) and clears the record */
+void expert_host_copies_detach(const struct backend_operations *backend, struct expert_host_copies *copies);
 
 /* ---- FP4 / FP8 expert linears of the original weights (the routed part of the reference's linear.h) ---- */
 #define LINEAR_SLICE_INSTANCES 5u /* product kernels are stamped for 1, 2, 4, 8, 16 slices; gfx950 holds 1, 2, 4, 8 */

@@ -23,7 +23,7 @@
  *     router_select_arguments  80 B  (router_records.h:98-110)   + expert_count, pick_count, affinity_kind, route_scale
  *     router_wide_arguments    120 B (router_records.h:117-134)  + the same four
  *     exl3_expert_record       80 B  (exl3_records.h:144-159)    + widths_offset
- *     exl3_tc_record           72 B  (exl3_tc_records.h:40-58)   + widths_offset, hidden, pairs_per_row
+ *     exl3_tc_record           72 B  (exl3_tc_records.h:40-58)   + widths_offset, hidden, pairs_per_row, expert_count
  *     exl3_tcp_record          88 B  (exl3_tc_records.h:244-262) + widths_offset, hidden, pairs_per_row, expert_count
  * widths_offset: 0, or the arena offset of uint32 [expert_count], entry e = gate | up << 8 | down << 16, the stored
  * widths of expert e's three matrices (per-matrix widths: one layer mixes K = 2, 3, 4). When it is 0 every matrix
@@ -306,8 +306,10 @@ struct exl3_tc_record {
     uint64_t widths_offset;
     uint32_t hidden;           /* 0: 5120 */
     uint32_t pairs_per_row;    /* 0: 6 */
+    uint32_t expert_count;     /* entries of the table at widths_offset (needed with it; else 0): a job of an expert beyond it adds nothing */
+    uint32_t reserved_zero;
 };
-ANEMONE_RECORD_HAS(exl3_tc_record, 88);
+ANEMONE_RECORD_HAS(exl3_tc_record, 96);
 
 /* workspace of the fused decode: fp16 operands [2][pairs][hidden] (later [pairs][intermediate]), float32 gate/up
  * partial products [GATE_UP_SLICES][2][pairs][intermediate], float32 down partials [DOWN_SLICES][pairs][hidden] */

@@ -61,7 +61,7 @@ def test_kernel_table_matches_the_records():
     assert table[("kernel_exl3", "exl3_reconstruct")] == C.sizeof(amd.Exl3ReconstructRecord) == 32
     assert table[("kernel_exl3", "exl3_input")] == C.sizeof(amd.Exl3ExpertRecord) == 88
     assert table[("kernel_exl3", "exl3_row_sum")] == C.sizeof(amd.RowSumArguments) == 24
-    assert table[("kernel_exl3_tc", "exl3_tc_products")] == C.sizeof(amd.Exl3TcRecord) == 88
+    assert table[("kernel_exl3_tc", "exl3_tc_products")] == C.sizeof(amd.Exl3TcRecord) == 96
     for width in ("k2", "k2_5", "k3", "k4", "mixed"):
         assert ("kernel_exl3", "exl3_gate_up_" + width) in table and ("kernel_exl3", "exl3_down_" + width) in table
     assert table[("kernel_router", "router_select_entry")] == 96
@@ -177,25 +177,28 @@ def test_tc_prepare_geometry_and_refusals(fake):
     assert [fake.handles[l.kernel][1] for l in launches] == ["exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate",
                                                             "exl3_tc_products", "exl3_tc_combine"]
     assert [list(l.grid) for l in launches] == [[32, 64, 2], [32, 64, 2], [16, 64, 1], [64, 64, 1], [32, 8, 1]]
-    passes = [amd.Exl3TcRecord.from_buffer_copy(bytes(l.argument)[:88]).pass_ for l in launches]
+    passes = [amd.Exl3TcRecord.from_buffer_copy(bytes(l.argument)[:96]).pass_ for l in launches]
     assert passes == [0, 0, 0, 1, 0]
     assert amd.exl3_tc_workspace_bytes(64, 4096, 2048) == 64 * 4096 * 4 + 4 * 2 * 64 * 2048 * 4 + 4 * 64 * 4096 * 4
     for changes, status in [(dict(row_count=0), 1), (dict(row_count=65), 1), (dict(rotation=1), 7), (dict(shared_sum=2), 1),
                             (dict(shared_sum=1, shared_offset=ARENA - 4096), 1), (dict(shared_sum=1, shared_offset=1 << 20), 1),
                             (dict(intermediate=2000), 7), (dict(bits_x2=7), 7), (dict(bits_x2=0), 1), (dict(pass_=1), 1),
                             (dict(workspace_offset=(2 << 20) + 16), 1), (dict(output_offset=2 << 20), 1),
-                            (dict(activation_limit=-1.0), 1), (dict(widths_offset=(2 << 20) + 256), 1), (dict(widths_offset=ARENA), 1),
-                            (dict(widths_offset=4096 + 96), 1)]:
+                            (dict(activation_limit=-1.0), 1), (dict(widths_offset=(2 << 20) + 256, expert_count=256), 1),
+                            (dict(widths_offset=ARENA, expert_count=256), 1), (dict(widths_offset=4096 + 96, expert_count=256), 1),
+                            # the table is checked for every expert's entry, not its first: its tail in the jobs, or past the arena
+                            (dict(widths_offset=4096 - 1008, expert_count=256), 1), (dict(widths_offset=ARENA - 1008, expert_count=256), 1),
+                            (dict(widths_offset=16384), 1), (dict(expert_count=256), 1), (dict(reserved_zero=1), 1)]:
         untouched = amd.launches_of(5)
         assert lib.exl3_tc_prepare(C.byref(tc_record(**changes)), ARENA, fake.address, fake.card, untouched) == status, changes
         assert not any(bytes(untouched))
     # a table of widths clear of the other ranges: taken
     tabled = amd.launches_of(5)
-    assert lib.exl3_tc_prepare(C.byref(tc_record(widths_offset=16384)), ARENA, fake.address, fake.card, tabled) == 0
+    assert lib.exl3_tc_prepare(C.byref(tc_record(widths_offset=16384, expert_count=256)), ARENA, fake.address, fake.card, tabled) == 0
     # the sum into the shared expert's rows: its own range, checked like the others
     joined = amd.launches_of(5)
     assert lib.exl3_tc_prepare(C.byref(tc_record(shared_sum=1, shared_offset=3 << 29)), ARENA, fake.address, fake.card, joined) == 0
-    assert amd.Exl3TcRecord.from_buffer_copy(bytes(joined[4].argument)[:88]).shared_sum == 1
+    assert amd.Exl3TcRecord.from_buffer_copy(bytes(joined[4].argument)[:96]).shared_sum == 1
     # hidden 0 and pairs_per_row 0 stand for the reference's 5120 and 6
     default = amd.launches_of(5)
     assert lib.exl3_tc_prepare(C.byref(tc_record(hidden=0, pairs_per_row=0, intermediate=640, job_capacity=48)), ARENA,

@@ -165,3 +165,61 @@ def test_wide_experts_of_the_original_weights(amd, workloads, form, rows):
     say("  rms error of the sampled rows %.2e" % error)
     assert error <= 2e-2
     assert np.all(np.isfinite(got)) and float(np.abs(got).max()) < 1e4, "every row of the step is written and bounded"
+
+
+@pytest.mark.parametrize("form,rows", [("fp8_block128", 1), ("fp8_block128", 64), ("fp4", 32)])
+def test_job_table_experts_of_the_original_weights(amd, workloads, form, rows):
+    """The decode form (the router's job table, expert_gate_up_<S> / expert_down_<S> with the K slices of the measured runs)
+    at the full shape: 1 and 64 rows of FP8 with float32 block scales, 32 rows of FP4; four sampled rows against the
+    oracle's layer."""
+    say("full shape: job-table", form, rows, "rows")
+    fp8 = form != "fp4"
+    distinct_generated = 4 if fp8 else 16
+    base = workloads.SEED + ((3 if fp8 else 4) << 20)
+    matrix = workloads.fp8_block128_matrix if fp8 else workloads.fp4_matrix
+    trios = [[matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
+              matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
+    matrices = [trios[e % distinct_generated] for e in range(EXPERTS)]
+    router = workloads.to_bf16(workloads.normals(base + 2, EXPERTS * HIDDEN) * 0.02).reshape(EXPERTS, HIDDEN)
+    x = workloads.activations(4, rows, HIDDEN)
+    card = amd.Card(((9 if fp8 else 5) << 30) + rows * (1 << 18))
+    try:
+        layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router, gate_up_slices=4, down_slices=2,
+                             weight_format=amd.WEIGHT_FORMAT_E4M3_BLOCK128 if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED)
+        layer.set_rows(x, rows)
+        wide = layer.wide_router() if rows > 8 else None
+        routing = layer.select_launch(0) if wide is None else wide.launches(small=True)
+        experts_launches = layer.expert_launches(wide)
+        card.run(layer.projection_launch())
+        card.run(routing)
+        card.run(layer.quantize_launch())
+        card.run(experts_launches)
+        jobs = layer.jobs() if wide is None else wide.read("jobs", amd.JOB_DTYPE)
+        got = layer.read("row_output", np.float32).reshape(rows, HIDDEN)
+    finally:
+        card.close()
+    live = jobs[jobs["row_count"] > 0]
+    experts_of, weights_of = np.zeros((rows, PICKS), np.uint32), np.zeros((rows, PICKS), np.float32)
+    seen = np.zeros(rows * PICKS, dtype=int)
+    for job in live:
+        for c in range(job["row_count"]):
+            experts_of.reshape(-1)[job["pair_index"][c]] = job["expert"]
+            weights_of.reshape(-1)[job["pair_index"][c]] = job["route_weight"][c]
+            seen[job["pair_index"][c]] += 1
+    assert np.all(seen == 1), "every pair of the step is in exactly one job"
+    # the picks are the oracle's: ids and weight bits of the sampled rows
+    sample = np.unique(np.array([0, rows // 3, rows // 2, rows - 1]))
+    want_experts, want_weights = np.zeros((len(sample), PICKS), np.uint32), np.zeros((len(sample), PICKS), np.float32)
+    bias = np.zeros(EXPERTS, np.float32)
+    o.orc.orc_router_route(o.ptr(np.ascontiguousarray(x[sample]), o.u16p), o.ptr(router, o.u16p), o.ptr(bias, o.f32p), len(sample), HIDDEN, EXPERTS,
+                           PICKS, layer.affinity_kind, 0, layer.route_scale, None, o.ptr(want_experts, o.u32p), o.ptr(want_weights, o.f32p))
+    assert np.array_equal(np.sort(experts_of[sample], axis=1), np.sort(want_experts, axis=1))
+    pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
+    want = np.zeros((len(sample), HIDDEN), dtype=np.float32)
+    o.orc.orc_linear_moe_layer(6 if fp8 else 3, o.ptr(np.ascontiguousarray(x[sample]), o.u16p), len(sample), HIDDEN, INNER, PICKS,
+                               o.ptr(np.ascontiguousarray(experts_of[sample]), o.u32p), o.ptr(np.ascontiguousarray(weights_of[sample]), o.f32p),
+                               EXPERTS, pointers, 10.0, o.ptr(want, o.f32p), None, None, 16)
+    error = float(np.sqrt(np.mean((got[sample] - want) ** 2) / np.mean(want.astype(np.float64) ** 2)))
+    say("  rms error of the sampled rows %.2e" % error)
+    assert error <= 2e-2
+    assert np.all(np.isfinite(got)) and float(np.abs(got).max()) < 1e4

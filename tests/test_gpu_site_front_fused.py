@@ -160,8 +160,12 @@ def test_a_wait_that_cannot_end_gives_up_and_every_block_leaves(amd, card):
     assert got["carried_pre"].tobytes() == before_pre.tobytes()
     for name in SITE_OUTPUTS[1:]:
         assert np.all(got[name] == 0xEE), name
-    # gave_up is the caller's to read and clear; then the front is whole again
-    card.upload(front.ranges["scratch"].byte_offset + 16 + 768 + 4, np.zeros(4, dtype=np.uint8))
+    # gave_up is the caller's to read: site_front_check reports it as a device error and clears it; then the front is whole again
+    import ctypes as C
+    count = C.c_uint32(0)
+    assert card.lib.site_front_check(amd.backend_table(), card.handle, front.ranges["scratch"], card.staging, 10 ** 10,
+                                     C.byref(count)) == amd.STATUS_DEVICE_ERROR and count.value == 1
+    assert card.lib.site_front_check(amd.backend_table(), card.handle, front.ranges["scratch"], card.staging, 10 ** 10, C.byref(count)) == 0
     card.run(fused)
     again = snapshot(card, front.ranges, SITE_OUTPUTS)
     assert all(again[name].tobytes() == want[name].tobytes() for name in SITE_OUTPUTS)

@@ -231,3 +231,98 @@ def test_a_failed_copy_leaves_none_of_the_pause_slots_held():
     assert set(held) == {4, 1, 2}
     for expert, slot in held.items():
         assert np.array_equal(backend.arena[SLOTS_OFFSET + slot * SLOT_BYTES:SLOTS_OFFSET + slot * SLOT_BYTES + EXPERT_BYTES], copies[expert])
+
+
+def test_site_front_check_reads_and_clears_the_count_of_blocks_that_gave_up():
+    """site_front_check over the stand-in backend: a clean scratch answers STATUS_OK and moves nothing up; a scratch whose
+    gave_up counts blocks answers STATUS_DEVICE_ERROR, reports the count and leaves it zero on the card."""
+    backend = CopyBackend(16384)
+    scratch = amd.Range(1024, 7184)  # SITE_FRONT_SCRATCH_BYTES
+    tail = 1024 + 16 + 8 * 24 * 4  # behind the four counters and the mixes of eight rows: departed, gave_up
+    staging = np.zeros(2, dtype=np.uint32)
+    count = C.c_uint32(99)
+    lib = amd.library()
+    assert lib.site_front_check(C.addressof(backend.operations), backend.card, scratch, staging.ctypes.data, 10 ** 9, C.byref(count)) == 0
+    assert count.value == 0 and backend.log == [("down", tail, 8)]
+    backend.arena[tail + 4:tail + 8] = np.array([3], dtype=np.uint32).view(np.uint8)
+    backend.arena[tail - 4:tail] = 0x77
+    backend.log.clear()
+    assert lib.site_front_check(C.addressof(backend.operations), backend.card, scratch, staging.ctypes.data, 10 ** 9,
+                                C.byref(count)) == amd.STATUS_DEVICE_ERROR
+    assert count.value == 3 and backend.log == [("down", tail, 8), ("up", tail, 8)]
+    assert not backend.arena[tail:tail + 8].any() and np.all(backend.arena[tail - 4:tail] == 0x77)
+    assert lib.site_front_check(C.addressof(backend.operations), backend.card, scratch, staging.ctypes.data, 10 ** 9, None) == 0
+    assert lib.site_front_check(C.addressof(backend.operations), backend.card, amd.Range(1024, 64), staging.ctypes.data, 10 ** 9,
+                                None) == amd.STATUS_INVALID_ARGUMENT
+
+
+# ---- the page-locked copies (expert_host_copies_attach) over a stand-in for the backend's staging memory ----
+
+ALLOCATE = C.CFUNCTYPE(C.c_int, C.c_uint64, C.POINTER(C.c_void_p))
+FREE = C.CFUNCTYPE(None, C.c_void_p)
+
+
+class StagingBackend:
+    def __init__(self):
+        self.blocks, self.freed, self.fail_staging_allocation = {}, [], False
+        self.callbacks = (ALLOCATE(self.allocate), FREE(self.free))
+        self.operations = (C.c_void_p * 28)()
+        self.operations[5] = C.cast(self.callbacks[0], C.c_void_p)
+        self.operations[6] = C.cast(self.callbacks[1], C.c_void_p)
+
+    def allocate(self, count, out):
+        if self.fail_staging_allocation:
+            return amd.STATUS_OUT_OF_MEMORY
+        block = np.full(count, 0xCD, dtype=np.uint8)
+        self.blocks[block.ctypes.data] = block
+        out[0] = block.ctypes.data
+        return 0
+
+    def free(self, address):
+        self.freed.append(address)
+
+
+def test_host_copies_attach_copies_every_expert_once_and_refuses_whole():
+    lib = amd.library()
+    backend = StagingBackend()
+    rng = np.random.default_rng(11)
+    host_arena = rng.integers(0, 256, size=4096, dtype=np.uint8)
+    offsets = np.array([0, 512, 100, 1800, 3000, 2400, 3600], dtype=np.uint64)  # in no order, as a loader may leave them
+    pauses = (amd.ExpertPause * 2)()
+    pauses[0].first_host_expert, pauses[0].host_expert_count, pauses[0].expert_byte_count = 0, 3, 200
+    pauses[1].first_host_expert, pauses[1].host_expert_count, pauses[1].expert_byte_count = 3, 4, 96
+
+    def attach(table_bytes=288, most=1 << 20, arena_bytes=host_arena.nbytes, count=len(offsets), pause_count=2):
+        copies, starts = amd.ExpertHostCopies(), (C.c_uint64 * 2)(77, 77)
+        status = lib.expert_host_copies_attach(C.addressof(backend.operations), pauses, pause_count, offsets.ctypes.data_as(C.POINTER(C.c_uint64)), count,
+                                               host_arena.ctypes.data, arena_bytes, table_bytes, most, C.byref(copies), starts)
+        return status, copies, list(starts)
+
+    status, copies, starts = attach()
+    assert status == 0 and starts == [0, 600] and copies.table_staging_offset == 1024 and copies.byte_count == 1024 + 288
+    block = backend.blocks[C.cast(copies.block, C.c_void_p).value]
+    for e in range(3):
+        assert np.array_equal(block[200 * e:200 * e + 200], host_arena[int(offsets[e]):int(offsets[e]) + 200])
+    for e in range(4):
+        assert np.array_equal(block[600 + 96 * e:600 + 96 * e + 96], host_arena[int(offsets[3 + e]):int(offsets[3 + e]) + 96])
+    assert np.all(block[984:] == 0xCD), "nothing is written behind the experts"
+    lib.expert_host_copies_detach(C.addressof(backend.operations), C.byref(copies))
+    assert backend.freed == [block.ctypes.data] and not copies.block and copies.byte_count == 0
+    lib.expert_host_copies_detach(C.addressof(backend.operations), C.byref(copies))  # again: nothing to give back
+    assert len(backend.freed) == 1
+    # refusals allocate nothing and leave the outputs as they were
+    before = len(backend.blocks)
+    for keywords, want in ((dict(arena_bytes=3600 + 95), amd.STATUS_INVALID_ARGUMENT), (dict(count=6), amd.STATUS_INVALID_ARGUMENT),
+                           (dict(most=1024 + 287), amd.STATUS_OUT_OF_MEMORY)):
+        status, copies, starts = attach(**keywords)
+        assert status == want and not copies.block and starts == [77, 77] and len(backend.blocks) == before, keywords
+    pauses[1].host_expert_count = 0
+    assert attach()[0] == amd.STATUS_INVALID_ARGUMENT  # a pause without host experts
+    pauses[1].host_expert_count = 4
+    backend.fail_staging_allocation = True
+    status, copies, starts = attach()
+    assert status == amd.STATUS_OUT_OF_MEMORY and not copies.block and starts == [77, 77]
+    # no pauses and no table: nothing to allocate, an empty record
+    backend.fail_staging_allocation = False
+    status, copies, _ = attach(table_bytes=0, pause_count=0)
+    assert status == 0 and not copies.block and copies.byte_count == 0 and len(backend.blocks) == before

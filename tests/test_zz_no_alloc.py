@@ -23,10 +23,14 @@ def hip_runtime():
     hip.hipMemcpy.argtypes, hip.hipMemcpy.restype = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int], C.c_int
     hip.hipFree.argtypes, hip.hipFree.restype = [C.c_void_p], C.c_int
     hip.hipDeviceSynchronize.argtypes, hip.hipDeviceSynchronize.restype = [], C.c_int
+    hip.hipMemGetInfo.argtypes, hip.hipMemGetInfo.restype = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)], C.c_int
+    hip.hipStreamCreate.argtypes, hip.hipStreamCreate.restype = [C.POINTER(C.c_void_p)], C.c_int
+    hip.hipStreamSynchronize.argtypes, hip.hipStreamSynchronize.restype = [C.c_void_p], C.c_int
+    hip.hipStreamDestroy.argtypes, hip.hipStreamDestroy.restype = [C.c_void_p], C.c_int
     return hip
 
 
-def one_step(amd, hip, rows, seed):
+def one_step(amd, hip, rows, seed, own_stream=False):
     hidden, inner, experts_n, picks = 512, 256, 64, 4
     width_choices = [2, 3, 4, 40]
     draws = splitmix_words(seed, experts_n * 3) % np.uint64(len(width_choices))
@@ -60,9 +64,18 @@ def one_step(amd, hip, rows, seed):
         lib = amd.library()
         lib.exl3_tc_run_static.restype = C.c_int
         lib.exl3_tc_run_static.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
-        status = lib.exl3_tc_run_static(C.byref(record), arena, before.nbytes, None)  # on the null stream
+        stream = C.c_void_p()  # NULL: the null stream
+        if own_stream:
+            assert hip.hipStreamCreate(C.byref(stream)) == 0
+        free_before, free_after, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        assert hip.hipDeviceSynchronize() == 0 and hip.hipMemGetInfo(C.byref(free_before), C.byref(total)) == 0
+        status = lib.exl3_tc_run_static(C.byref(record), arena, before.nbytes, stream)
         assert status == 0, "exl3_tc_run_static answered %d" % status
-        assert hip.hipDeviceSynchronize() == 0
+        assert (hip.hipStreamSynchronize(stream) if own_stream else hip.hipDeviceSynchronize()) == 0
+        assert hip.hipMemGetInfo(C.byref(free_after), C.byref(total)) == 0
+        assert free_after.value == free_before.value, "the call changed the device's free memory: %d -> %d" % (free_before.value, free_after.value)
+        if own_stream:
+            assert hip.hipStreamDestroy(stream) == 0
         got = np.zeros((rows, hidden), np.float32)
         assert hip.hipMemcpy(got.ctypes.data, arena.value + record.output_offset, out_bytes, 2) == 0
     finally:
@@ -75,9 +88,9 @@ def test_static_workspace_equals_the_arena_workspace_twice():
     import anemone_amd as amd
     amd.library()
     hip = hip_runtime()
-    for rows, seed in ((8, 41), (3, 42)):  # the second call of a smaller step: what the first left in the array must not show
-        say("exl3_tc_run_static", rows, "rows")
-        got, want = one_step(amd, hip, rows, seed)
+    for rows, seed, own_stream in ((8, 41, False), (3, 42, True)):  # the second call of a smaller step: what the first left in the array must not show
+        say("exl3_tc_run_static", rows, "rows", "on a stream of the test's" if own_stream else "on the null stream")
+        got, want = one_step(amd, hip, rows, seed, own_stream)
         assert np.all(np.isfinite(want)) and float(np.abs(want).max()) > 0.0
         assert got.tobytes() == want.tobytes(), "the static workspace's output differs from the arena workspace's"
 
