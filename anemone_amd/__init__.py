@@ -14,6 +14,7 @@ PROBE_LIBRARY_PATH = os.path.join(HERE, "libanemone_probe.so")
 STATUS_OK, STATUS_INVALID_ARGUMENT, STATUS_OUT_OF_MEMORY = 0, 1, 2
 STATUS_DEVICE_ERROR, STATUS_TIMED_OUT, STATUS_UNSUPPORTED, STATUS_BUSY = 5, 6, 7, 8
 WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED, WEIGHT_FORMAT_E4M3_BLOCK128 = 2, 3, 5, 6
+WEIGHT_FORMAT_E2M1_GFX950, WEIGHT_FORMAT_E4M3_GFX950 = 7, 8  # the two _SCALED formats in gfx950's own lane order
 ARITHMETIC_CLASS_GFX950 = 950
 BACKEND_NO_KERNEL = 0xFFFFFFFF
 LAUNCH_CHAIN, LAUNCH_SIDE, LAUNCH_RESUME, LAUNCH_JOIN, LAUNCH_SIDE_MORE = 0, 1, 2, 3, 4  # kernel_launch.branch
@@ -235,6 +236,10 @@ class LinearWideKernels(C.Structure):
                 ("wide_expert_gate_up_b128", u32), ("wide_expert_down_b128", u32)]
 
 
+class LinearNativeKernels(C.Structure):
+    _fields_ = [("native_expert_gate_up", u32), ("native_expert_down", u32), ("native_expert_gate_up_e4m3", u32), ("native_expert_down_e4m3", u32)]
+
+
 class QuantizeDescription(C.Structure):
     _fields_ = [("values", Range), ("codes", Range), ("exponents", Range), ("operands", Range), ("width", u32),
                 ("row_count", u32)]
@@ -312,6 +317,11 @@ def library():
             "linear_wide_kernels_prepare": [vp, vp, u32, C.POINTER(LinearWideKernels)],
             "linear_wide_experts_prepare": [C.POINTER(LinearWideExpertsDescription), u64, C.POINTER(LinearKernels),
                                             C.POINTER(LinearWideKernels), launch_p],
+            "linear_native_kernels_prepare": [vp, vp, u32, C.POINTER(LinearNativeKernels)],
+            "linear_native_experts_prepare": [C.POINTER(LinearWideExpertsDescription), u64, C.POINTER(LinearKernels),
+                                              C.POINTER(LinearNativeKernels), launch_p],
+            "weight_format_gfx950_pack": [C.c_int, C.POINTER(Shape), vp, u64, vp, u64],
+            "weight_format_gfx950_unpack": [C.c_int, C.POINTER(Shape), vp, u64, vp, u64],
             "expert_fused_kernels_prepare": [vp, vp, u32, C.POINTER(ExpertFusedKernels)],
             "expert_producer_prepare": [C.POINTER(RoutedExpertsDescription), Range, u64, C.POINTER(LinearKernels),
                                         C.POINTER(ExpertFusedKernels), launch_p],
@@ -362,6 +372,26 @@ def status_text(status):
 def check(status, what):
     if status != STATUS_OK:
         raise AnemoneError(what, status)
+
+
+def gfx950_pack(weight_format, outputs, inputs, stored):
+    """A matrix of the reference's E2M1_SCALED / E4M3_SCALED bytes in gfx950's lane order (weight_format names the GFX950
+    format): the library's load-time re-lay-out, weight_format_gfx950_pack."""
+    stored = np.ascontiguousarray(stored, dtype=np.uint8)
+    packed = np.empty_like(stored)
+    shape = Shape(outputs, inputs, 8 if weight_format == WEIGHT_FORMAT_E4M3_GFX950 else 4, 0)
+    check(library().weight_format_gfx950_pack(weight_format, C.byref(shape), stored.ctypes.data, stored.nbytes, packed.ctypes.data, packed.nbytes),
+          "weight_format_gfx950_pack")
+    return packed
+
+
+def gfx950_unpack(weight_format, outputs, inputs, packed):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    stored = np.empty_like(packed)
+    shape = Shape(outputs, inputs, 8 if weight_format == WEIGHT_FORMAT_E4M3_GFX950 else 4, 0)
+    check(library().weight_format_gfx950_unpack(weight_format, C.byref(shape), packed.ctypes.data, packed.nbytes, stored.ctypes.data, stored.nbytes),
+          "weight_format_gfx950_unpack")
+    return stored
 
 
 def backend_table():
@@ -782,7 +812,9 @@ class Exl3Layer:
 
 class Fp4Layer:
     """One MoE layer of the original FP4 weights (WEIGHT_FORMAT_E2M1_SCALED; or, with weight_format, of FP8 weights,
-    WEIGHT_FORMAT_E4M3_SCALED; stored bytes as the reference's packs hold them) in a card's arena, with the scratch ranges of a step of at most `rows` rows: the quantizer of the rows,
+    WEIGHT_FORMAT_E4M3_SCALED; stored bytes as the reference's packs hold them; with WEIGHT_FORMAT_E2M1_GFX950 or
+    WEIGHT_FORMAT_E4M3_GFX950 the matrices, given in the reference's bytes, go through the library's load-time re-lay-out
+    first) in a card's arena, with the scratch ranges of a step of at most `rows` rows: the quantizer of the rows,
     the router's select, and the four launches of the routed experts."""
 
     def __init__(self, card, hidden, inner, expert_count, picks, rows, matrices, router_weights_bf16=None,
@@ -790,7 +822,15 @@ class Fp4Layer:
                  weight_format=WEIGHT_FORMAT_E2M1_SCALED):
         self.card, self.H, self.I, self.E, self.P, self.rows = card, hidden, inner, expert_count, picks, rows
         self.weight_format = weight_format
-        self.bits = 8 if weight_format in (WEIGHT_FORMAT_E4M3_SCALED, WEIGHT_FORMAT_E4M3_BLOCK128) else 4
+        self.bits = 8 if weight_format in (WEIGHT_FORMAT_E4M3_SCALED, WEIGHT_FORMAT_E4M3_BLOCK128, WEIGHT_FORMAT_E4M3_GFX950) else 4
+        self.native = weight_format in (WEIGHT_FORMAT_E2M1_GFX950, WEIGHT_FORMAT_E4M3_GFX950)
+        if self.native:  # a matrix that lies at several experts' places is packed once
+            packed = {}
+            for trio in matrices:
+                for m, matrix in enumerate(trio):
+                    if id(matrix) not in packed:
+                        packed[id(matrix)] = gfx950_pack(weight_format, *((inner, hidden) if m < 2 else (hidden, inner)), matrix)
+            matrices = [[packed[id(matrix)] for matrix in trio] for trio in matrices]
         self.block128 = weight_format == WEIGHT_FORMAT_E4M3_BLOCK128
         self.limit, self.affinity_kind, self.route_scale = limit, affinity_kind, route_scale
         self.gate_up_slices, self.down_slices = gate_up_slices, down_slices
@@ -892,6 +932,15 @@ class Fp4Layer:
         d.experts = self.experts_description(wide)
         d.experts.gate_up_slice_count = d.experts.down_slice_count = 1
         d.tiles, d.pairs, d.tile_count = wide.ranges["tiles"], wide.ranges["pairs"], wide.tile_count
+        if self.native:
+            if not hasattr(self, "native_kernels"):
+                self.native_kernels = LinearNativeKernels()
+                check(self.card.lib.linear_native_kernels_prepare(backend_table(), self.card.handle, ARITHMETIC_CLASS_GFX950,
+                                                                  C.byref(self.native_kernels)), "linear_native_kernels_prepare")
+            launches = launches_of(3)
+            check(self.card.lib.linear_native_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), C.byref(self.native_kernels),
+                                                              launches), "linear_native_experts_prepare")
+            return launches
         launches = launches_of(4 if self.block128 else 3)
         prepare = self.card.lib.linear_wide_experts_block128_prepare if self.block128 else self.card.lib.linear_wide_experts_prepare
         check(prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), C.byref(self.wide_kernels), launches), "linear_wide_experts_prepare")

@@ -565,11 +565,12 @@ result_status linear_wide_kernels_prepare(const struct backend_operations *backe
  * own between the products); else those of the reference's formats (three) */
 static result_status wide_experts_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
                                           const struct linear_kernels_record *linear_kernels,
-                                          const struct linear_wide_kernels_record *kernels, bool block128,
-                                          struct kernel_launch *launches_out)
+                                          const struct linear_wide_kernels_record *kernels, const struct linear_native_kernels_record *native_kernels,
+                                          bool block128, struct kernel_launch *launches_out)
 {
-    const char *what = block128 ? "the wide routed experts of float32 block scales" : "the wide routed experts";
-    if (description == NULL || linear_kernels == NULL || kernels == NULL || launches_out == NULL) {
+    const bool native = native_kernels != NULL; /* experts in gfx950's lane order: the same launches by the native kernels */
+    const char *what = native ? "the wide routed experts in gfx950's lane order" : block128 ? "the wide routed experts of float32 block scales" : "the wide routed experts";
+    if (description == NULL || linear_kernels == NULL || (kernels == NULL && !native) || launches_out == NULL) {
         REFUSE("%s: a missing argument", what);
         return STATUS_INVALID_ARGUMENT;
     }
@@ -580,16 +581,18 @@ static result_status wide_experts_prepare(const struct linear_wide_experts_descr
         REFUSE("%s: a weight format of %u", what, (uint32_t)experts->weight_format);
         return STATUS_INVALID_ARGUMENT;
     }
-    const bool bytes = experts->weight_format == WEIGHT_FORMAT_E4M3_SCALED || block128;
+    const enum weight_format_code nibbles_format = native ? WEIGHT_FORMAT_E2M1_GFX950 : WEIGHT_FORMAT_E2M1_SCALED;
+    const enum weight_format_code bytes_format = native ? WEIGHT_FORMAT_E4M3_GFX950 : WEIGHT_FORMAT_E4M3_SCALED;
+    const bool bytes = experts->weight_format == bytes_format || block128;
     const uint32_t strip_outputs = bytes ? LINEAR_STRIP_OUTPUTS / 2u : LINEAR_STRIP_OUTPUTS;
     uint64_t gate_up_bytes = 0, down_bytes = 0;
-    if (description->reserved_zero != 0 || experts->reserved_zero != 0 || (experts->weight_format != WEIGHT_FORMAT_E2M1_SCALED && !bytes) ||
+    if (description->reserved_zero != 0 || experts->reserved_zero != 0 || (experts->weight_format != nibbles_format && !bytes) ||
         format == NULL || format->stored_byte_count(gate_up, &gate_up_bytes) != STATUS_OK ||
         format->stored_byte_count(down, &down_bytes) != STATUS_OK || gate_up->input_size % 128u != 0 || down->input_size % 128u != 0 ||
         down->input_size != gate_up->output_size || gate_up->output_size < strip_outputs || down->output_size < strip_outputs ||
         gate_up->output_size % 32u != 0) {
         REFUSE("%s: matrices of format %u or %u in shapes it stores, inputs a multiple of 128, gate/up outputs of 32, at least %u outputs, "
-               "down reading what gate and up write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, (uint32_t)WEIGHT_FORMAT_E4M3_SCALED, strip_outputs);
+               "down reading what gate and up write", what, (uint32_t)nibbles_format, (uint32_t)bytes_format, strip_outputs);
         return STATUS_INVALID_ARGUMENT;
     }
     if (experts->gate_up_slice_count != 1u || experts->down_slice_count != 1u) {
@@ -597,8 +600,17 @@ static result_status wide_experts_prepare(const struct linear_wide_experts_descr
                experts->down_slice_count);
         return STATUS_INVALID_ARGUMENT;
     }
-    const uint32_t gate_up_kernel = block128 ? kernels->wide_expert_gate_up_b128 : bytes ? kernels->wide_expert_gate_up_e4m3 : kernels->wide_expert_gate_up;
-    const uint32_t down_kernel = block128 ? kernels->wide_expert_down_b128 : bytes ? kernels->wide_expert_down_e4m3 : kernels->wide_expert_down;
+    uint32_t gate_up_kernel, down_kernel, gate_up_window, down_window;
+    if (native) {
+        gate_up_kernel = bytes ? native_kernels->native_expert_gate_up_e4m3 : native_kernels->native_expert_gate_up;
+        down_kernel = bytes ? native_kernels->native_expert_down_e4m3 : native_kernels->native_expert_down;
+        gate_up_window = down_window = NATIVE_WINDOW_BYTES(bytes ? NATIVE_E4M3_COLUMN_BLOCKS : NATIVE_E2M1_COLUMN_BLOCKS);
+    } else {
+        gate_up_kernel = block128 ? kernels->wide_expert_gate_up_b128 : bytes ? kernels->wide_expert_gate_up_e4m3 : kernels->wide_expert_gate_up;
+        down_kernel = block128 ? kernels->wide_expert_down_b128 : bytes ? kernels->wide_expert_down_e4m3 : kernels->wide_expert_down;
+        gate_up_window = bytes ? WIDE_GATE_UP_E4M3_WINDOW_BYTES : WIDE_GATE_UP_WINDOW_BYTES;
+        down_window = bytes ? WIDE_DOWN_E4M3_WINDOW_BYTES : WIDE_DOWN_WINDOW_BYTES;
+    }
     if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL || linear_kernels->expert_row_sum == BACKEND_NO_KERNEL ||
         (block128 && linear_kernels->activation_quantize_128 == BACKEND_NO_KERNEL)) {
         REFUSE("%s: a kernel of the chain is not prepared", what);
@@ -644,7 +656,7 @@ static result_status wide_experts_prepare(const struct linear_wide_experts_descr
     uint32_t at = 0;
     launch_fill(&launches[at++], gate_up_kernel,
                 (gate_up->output_size + gate_up_outputs - 1u) / gate_up_outputs, description->tile_count, 1,
-                WIDE_BLOCK_THREADS, bytes ? WIDE_GATE_UP_E4M3_WINDOW_BYTES : WIDE_GATE_UP_WINDOW_BYTES, &gate_up_record, sizeof gate_up_record);
+                WIDE_BLOCK_THREADS, gate_up_window, &gate_up_record, sizeof gate_up_record);
     if (block128) { /* the hidden values, which the gate/up launch left where the operands go, to their codes and scales */
         const struct activation_quantize_arguments quantize_record = {
             experts->hidden_operands.byte_offset, experts->hidden_codes.byte_offset, experts->hidden_exponents.byte_offset,
@@ -654,7 +666,7 @@ static result_status wide_experts_prepare(const struct linear_wide_experts_descr
                     LINEAR_ELEMENT_THREADS, 0, &quantize_record, sizeof quantize_record);
     }
     launch_fill(&launches[at++], down_kernel, (down->output_size + block_outputs - 1u) / block_outputs,
-                description->tile_count, 1, WIDE_BLOCK_THREADS, bytes ? WIDE_DOWN_E4M3_WINDOW_BYTES : WIDE_DOWN_WINDOW_BYTES, &down_record, sizeof down_record);
+                description->tile_count, 1, WIDE_BLOCK_THREADS, down_window, &down_record, sizeof down_record);
     launch_fill(&launches[at++], linear_kernels->expert_row_sum,
                 (down->output_size + ROW_SUM_BLOCK_OUTPUTS - 1u) / ROW_SUM_BLOCK_OUTPUTS, (uint32_t)rows, 1, LINEAR_ELEMENT_THREADS, 0,
                 &row_sum_record, sizeof row_sum_record);
@@ -666,12 +678,52 @@ result_status linear_wide_experts_prepare(const struct linear_wide_experts_descr
                                           const struct linear_kernels_record *linear_kernels,
                                           const struct linear_wide_kernels_record *kernels, struct kernel_launch *launches_out)
 {
-    return wide_experts_prepare(description, arena_byte_count, linear_kernels, kernels, false, launches_out);
+    return wide_experts_prepare(description, arena_byte_count, linear_kernels, kernels, NULL, false, launches_out);
 }
 
 result_status linear_wide_experts_block128_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
                                                    const struct linear_kernels_record *linear_kernels,
                                                    const struct linear_wide_kernels_record *kernels, struct kernel_launch *launches_out)
 {
-    return wide_experts_prepare(description, arena_byte_count, linear_kernels, kernels, true, launches_out);
+    return wide_experts_prepare(description, arena_byte_count, linear_kernels, kernels, NULL, true, launches_out);
+}
+
+/* ---- the same launches for experts stored in gfx950's lane order ---- */
+
+result_status linear_native_kernels_prepare(const struct backend_operations *backend, struct device_card *card, uint32_t arithmetic_class,
+                                            struct linear_native_kernels_record *kernels_out)
+{
+    if (backend == NULL || backend->kernel_prepare == NULL || card == NULL || kernels_out == NULL || arithmetic_class != ARITHMETIC_CLASS_GFX950) {
+        REFUSE("linear_native_kernels_prepare: a backend, a card of class %u and a record to fill are needed", ARITHMETIC_CLASS_GFX950);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    static const struct {
+        const char *name;
+        uint32_t record_bytes;
+    } wanted[4] = {{KERNEL_NATIVE_EXPERT_GATE_UP_STEM "1", sizeof(struct wide_expert_gate_up_arguments)},
+                   {KERNEL_NATIVE_EXPERT_DOWN_STEM "1", sizeof(struct wide_expert_down_arguments)},
+                   {KERNEL_NATIVE_EXPERT_GATE_UP_STEM "e4m3_1", sizeof(struct wide_expert_gate_up_arguments)},
+                   {KERNEL_NATIVE_EXPERT_DOWN_STEM "e4m3_1", sizeof(struct wide_expert_down_arguments)}};
+    uint32_t handles[4];
+    _Static_assert(sizeof(struct linear_native_kernels_record) == sizeof handles, "a handle a member, in the members' order");
+    for (uint32_t i = 0; i < 4u; i++) {
+        const result_status status = backend->kernel_prepare(card, KERNEL_FILE_NATIVE_LINEAR, wanted[i].name, wanted[i].record_bytes, &handles[i]);
+        if (status != STATUS_OK) {
+            REFUSE("linear_native_kernels_prepare: %s: %s", wanted[i].name, status_text(status));
+            return status;
+        }
+    }
+    memcpy(kernels_out, handles, sizeof handles);
+    return STATUS_OK;
+}
+
+result_status linear_native_experts_prepare(const struct linear_wide_experts_description *description, uint64_t arena_byte_count,
+                                            const struct linear_kernels_record *linear_kernels,
+                                            const struct linear_native_kernels_record *kernels, struct kernel_launch *launches_out)
+{
+    if (kernels == NULL) {
+        REFUSE("linear_native_experts_prepare: the native kernels' record is needed");
+        return STATUS_INVALID_ARGUMENT;
+    }
+    return wide_experts_prepare(description, arena_byte_count, linear_kernels, NULL, kernels, false, launches_out);
 }

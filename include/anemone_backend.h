@@ -52,7 +52,14 @@ enum weight_format_code {
     /* extension, no counterpart in the reference: E4M3 codes in E4M3_SCALED's lane order [out/16][in/32][lane][16], then
      * one float32 scale for every 128 outputs x 128 inputs, [out/128][in/128]; its vectors are quantized 128 values a
      * float32 scale */
-    WEIGHT_FORMAT_E4M3_BLOCK128 = 6
+    WEIGHT_FORMAT_E4M3_BLOCK128 = 6,
+    /* extensions, no counterpart in the reference: the two formats above whose name ends in _SCALED, the same weights and
+     * scale codes, laid out in the lane order of gfx950's own matrix instruction (v_mfma_scale_f32_16x16x128_f8f6f4 on
+     * wavefronts of 64) as the reference's are in the order of its cards' (include/anemone/weight_format_seam.h:22-46: "a
+     * new format is a new entry here, its kernels in every backend, and its reference decode among the tests"). Made at
+     * load time from the reference's bytes by weight_format_gfx950_pack (anemone_ops.h), which also states the lay-out. */
+    WEIGHT_FORMAT_E2M1_GFX950 = 7,
+    WEIGHT_FORMAT_E4M3_GFX950 = 8
 };
 
 #define BACKEND_MAXIMUM_CARDS 16

@@ -47,6 +47,27 @@ struct weight_format_operations {
 const struct weight_format_operations *weight_format_operations_of(enum weight_format_code format);
 extern const struct weight_format_operations exl3_weight_operations;
 
+/* Load-time re-lay-out between the reference's lane order and gfx950's (host only: bytes move, no weight or scale code
+ * changes; no allocation). A matrix [outputs][inputs], outputs a multiple of 16 (32 for E4M3), inputs of 128, is tiles of
+ * 16 outputs by K steps of 128 inputs. In a GFX950 format the tiles follow each other, a tile's K steps follow each
+ * other, and a K step is the 64 lanes' A operand of v_mfma_scale_f32_16x16x128_f8f6f4, lane 16 g + o holding output o:
+ *   E2M1_GFX950  16 bytes a lane: nibble n (0: low) of byte b of word T is input 32 g + 16 n + 2 T + {0, 8, 1, 9}[b] of
+ *                the step; behind all tiles the scale codes, one byte a lane a K step a tile ([tile][step][lane]): the
+ *                E8M0 code of output o, inputs 32 g .. 32 g + 31. Bytes: outputs inputs / 2 + outputs inputs / 32.
+ *   E4M3_GFX950  32 bytes a lane as two halves of 1,024 bytes a step ([half][lane][16]): byte c of word v (0 .. 7; half
+ *                v / 4) is input 64 (v / 4) + 16 g + 8 (c % 2) + 2 (v % 4) + c / 2; behind all tiles the scale codes as
+ *                E4M3_SCALED stores them (a row of inputs / 32 for every 32 outputs). Bytes: E4M3_SCALED's.
+ * The byte a lane's register holds is the byte the reference-format kernels of this library form there from the
+ * reference's lay-out, so both formats' kernels run the same sums. pack: from E2M1_SCALED to E2M1_GFX950 or from
+ * E4M3_SCALED to E4M3_GFX950 (`format` names the GFX950 format); unpack: back. The two byte counts must be the
+ * formats' stored_byte_count of the shape and the buffers apart; else STATUS_INVALID_ARGUMENT and nothing is written. */
+MUST_CHECK result_status weight_format_gfx950_pack(enum weight_format_code format, const struct matrix_shape_record *shape,
+                                                   const void *reference_bytes, uint64_t reference_byte_count, void *packed_out,
+                                                   uint64_t packed_byte_count);
+MUST_CHECK result_status weight_format_gfx950_unpack(enum weight_format_code format, const struct matrix_shape_record *shape,
+                                                     const void *packed_bytes, uint64_t packed_byte_count, void *reference_out,
+                                                     uint64_t reference_byte_count);
+
 enum linear_order_code { LINEAR_ORDER_FIXED = 0, LINEAR_ORDER_REFERENCE = 1 };
 
 /* ---- EXL3 chain ---- */
@@ -561,6 +582,23 @@ MUST_CHECK result_status linear_wide_experts_block128_prepare(const struct linea
                                                               uint64_t arena_byte_count, const struct linear_kernels_record *linear_kernels,
                                                               const struct linear_wide_kernels_record *kernels,
                                                               struct kernel_launch *launches_out);
+
+/* The wide form of experts stored in gfx950's lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950; no counterpart in the
+ * reference): linear_wide_experts_prepare's description, three launches and outputs -- bit for bit those of the same
+ * matrices in the reference's lay-out -- by the kernels of kernel_native_linear.hip, whose weights go from memory into
+ * the matrix instruction's registers. */
+struct linear_native_kernels_record {
+    uint32_t native_expert_gate_up; /* E2M1_GFX950, one slice */
+    uint32_t native_expert_down;
+    uint32_t native_expert_gate_up_e4m3; /* E4M3_GFX950 */
+    uint32_t native_expert_down_e4m3;
+};
+MUST_CHECK result_status linear_native_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
+                                                       uint32_t arithmetic_class, struct linear_native_kernels_record *kernels_out);
+MUST_CHECK result_status linear_native_experts_prepare(const struct linear_wide_experts_description *description,
+                                                       uint64_t arena_byte_count, const struct linear_kernels_record *linear_kernels,
+                                                       const struct linear_native_kernels_record *kernels,
+                                                       struct kernel_launch *launches_out);
 
 uint64_t linear_values_byte_count(uint64_t vector_count, uint64_t width);    /* bfloat16 [vector][width] */
 uint64_t linear_codes_byte_count(uint64_t vector_count, uint64_t width);     /* E4M3 [vector][width] */

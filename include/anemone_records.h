@@ -490,6 +490,14 @@ ANEMONE_RECORD_HAS(expert_gate_up_quantize_arguments, 96);
 #define WIDE_GATE_UP_E4M3_WINDOW_BYTES 53760u /* of wide_expert_gate_up_e4m3_<S>: two stages */
 #define WIDE_DOWN_WINDOW_BYTES 51712u     /* of wide_expert_down_<S>: two stages */
 #define WIDE_DOWN_E4M3_WINDOW_BYTES 51712u /* of wide_expert_down_e4m3_<S>: two stages */
+/* the kernels of the same launches for experts of WEIGHT_FORMAT_E2M1_GFX950 / _E4M3_GFX950: the same records */
+#define KERNEL_FILE_NATIVE_LINEAR "kernel_native_linear"
+#define KERNEL_NATIVE_EXPERT_GATE_UP_STEM "native_expert_gate_up_"
+#define KERNEL_NATIVE_EXPERT_DOWN_STEM "native_expert_down_"
+#define NATIVE_E2M1_COLUMN_BLOCKS 4u /* a block of the E2M1_GFX950 launches: one tile of the wide select (64 pairs) */
+#define NATIVE_E4M3_COLUMN_BLOCKS 8u /* of the E4M3_GFX950 launches: two tiles of one expert (128 pairs), read once */
+/* dynamic LDS: two stages of a K step of the block's columns (128 bytes of codes a column, 4 of scale codes) */
+#define NATIVE_WINDOW_BYTES(column_blocks) (2u * ((column_blocks) * 2048u + (column_blocks) * 64u))
 struct wide_expert_gate_up_arguments {
     uint64_t tiles_offset;            /* read: struct wide_expert_tile [tile_count] */
     uint64_t pairs_offset;            /* read: struct wide_pair [pair_count] */

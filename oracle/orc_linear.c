@@ -14,10 +14,21 @@
 
 #define BLOCK 32u
 
+static int holds_nibbles(int format)
+{
+    return format == ORC_FORMAT_E2M1_SCALED || format == ORC_FORMAT_E2M1_GFX950;
+}
+
 static int shape_is_stored(int format, uint32_t outputs, uint32_t inputs)
 {
     if (outputs == 0u || inputs == 0u || outputs % 16u != 0u) {
         return 0;
+    }
+    if (format == ORC_FORMAT_E2M1_GFX950) {
+        return inputs % 128u == 0u;
+    }
+    if (format == ORC_FORMAT_E4M3_GFX950) {
+        return inputs % 128u == 0u && outputs % 32u == 0u;
     }
     if (format == ORC_FORMAT_E2M1_SCALED) {
         return inputs % 64u == 0u;
@@ -33,7 +44,7 @@ static int shape_is_stored(int format, uint32_t outputs, uint32_t inputs)
 
 uint64_t orc_linear_scale_count(int format, uint32_t outputs, uint32_t inputs)
 {
-    if (format == ORC_FORMAT_E2M1_SCALED) {
+    if (holds_nibbles(format)) {
         return (uint64_t)outputs * (inputs / BLOCK);
     }
     if (format == ORC_FORMAT_E4M3_BLOCK128) {
@@ -45,7 +56,7 @@ uint64_t orc_linear_scale_count(int format, uint32_t outputs, uint32_t inputs)
 uint64_t orc_linear_stored_bytes(int format, uint32_t outputs, uint32_t inputs)
 {
     const uint64_t weights = (uint64_t)outputs * inputs;
-    return (format == ORC_FORMAT_E2M1_SCALED ? weights / 2u : weights) + orc_linear_scale_count(format, outputs, inputs);
+    return (holds_nibbles(format) ? weights / 2u : weights) + orc_linear_scale_count(format, outputs, inputs);
 }
 
 /* ---- lay-out: walk the stored words and ask which weight lies in each ---- */
@@ -57,6 +68,56 @@ int orc_linear_lay_out(int format, uint32_t outputs, uint32_t inputs, const uint
         return -1;
     }
     const uint32_t tiles = outputs / 16u;
+    if (format == ORC_FORMAT_E2M1_GFX950 || format == ORC_FORMAT_E4M3_GFX950) {
+        /* walk the stored bytes of the definition and ask which weight lies in each */
+        static const uint32_t input_of_byte[4] = {0, 8, 1, 9};
+        const uint32_t steps = inputs / 128u;
+        uint64_t at = 0;
+        for (uint32_t tile = 0; tile < tiles; tile++) {
+            for (uint32_t step = 0; step < steps; step++) {
+                if (format == ORC_FORMAT_E2M1_GFX950) {
+                    for (uint32_t lane = 0; lane < 64u; lane++) {
+                        for (uint32_t T = 0; T < 4u; T++) {
+                            for (uint32_t b = 0; b < 4u; b++, at++) {
+                                uint32_t byte = 0;
+                                for (uint32_t n = 0; n < 2u; n++) {
+                                    const uint32_t input = 128u * step + 32u * (lane / 16u) + 16u * n + 2u * T + input_of_byte[b];
+                                    const uint32_t code = codes[(uint64_t)(16u * tile + lane % 16u) * inputs + input];
+                                    if (code > 15u) {
+                                        return -1;
+                                    }
+                                    byte |= code << (4u * n);
+                                }
+                                stored[at] = (uint8_t)byte;
+                            }
+                        }
+                    }
+                } else {
+                    for (uint32_t half = 0; half < 2u; half++) {
+                        for (uint32_t lane = 0; lane < 64u; lane++) {
+                            for (uint32_t k = 0; k < 16u; k++, at++) {
+                                const uint32_t v = 4u * half + k / 4u, c = k % 4u;
+                                const uint32_t input = 128u * step + 64u * (v / 4u) + 16u * (lane / 16u) + 8u * (c % 2u) + 2u * (v % 4u) + c / 2u;
+                                stored[at] = codes[(uint64_t)(16u * tile + lane % 16u) * inputs + input];
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        if (format == ORC_FORMAT_E4M3_GFX950) {
+            memcpy(stored + at, scale_codes, orc_linear_scale_count(format, outputs, inputs));
+            return 0;
+        }
+        for (uint32_t tile = 0; tile < tiles; tile++) {
+            for (uint32_t step = 0; step < steps; step++) {
+                for (uint32_t lane = 0; lane < 64u; lane++, at++) {
+                    stored[at] = scale_codes[(uint64_t)(16u * tile + lane % 16u) * (inputs / BLOCK) + 4u * step + lane / 16u];
+                }
+            }
+        }
+        return 0;
+    }
     if (format == ORC_FORMAT_E2M1_SCALED) {
         const uint32_t loads = inputs / 64u;
         uint64_t at = 0;
@@ -123,6 +184,22 @@ int orc_linear_read(int format, uint32_t outputs, uint32_t inputs, const uint8_t
         return -1;
     }
     const uint32_t tile = output / 16u, in_tile = output % 16u, g = in_tile % 8u, far_output = in_tile / 8u;
+    if (format == ORC_FORMAT_E2M1_GFX950) {
+        /* input = 128 step + 32 G + 16 n + r with r = 2 T + {0, 8, 1, 9}[b]: r below 8 is 2 T + (0 or 1), else 2 T + (8 or 9) */
+        const uint32_t steps = inputs / 128u, step = input / 128u, G = (input % 128u) / 32u, n = (input % 32u) / 16u, r = input % 16u;
+        const uint32_t T = (r % 8u) / 2u, b = 2u * (r % 2u) + r / 8u, lane = 16u * G + in_tile;
+        *code_out = (stored[(((uint64_t)tile * steps + step) * 64u + lane) * 16u + 4u * T + b] >> (4u * n)) & 15u;
+        *scale_out = stored[(uint64_t)outputs * inputs / 2u + ((uint64_t)tile * steps + step) * 64u + lane];
+        return 0;
+    }
+    if (format == ORC_FORMAT_E4M3_GFX950) {
+        /* input = 128 step + 64 half + 16 G + r with r = 8 (c % 2) + 2 (v % 4) + c / 2 */
+        const uint32_t steps = inputs / 128u, step = input / 128u, half = (input % 128u) / 64u, G = (input % 64u) / 16u, r = input % 16u;
+        const uint32_t word = (r % 8u) / 2u, c = 2u * (r % 2u) + r / 8u, lane = 16u * G + in_tile;
+        *code_out = stored[((uint64_t)tile * steps + step) * 2048u + half * 1024u + lane * 16u + word * 4u + c];
+        *scale_out = stored[(uint64_t)outputs * inputs + (uint64_t)(output / 32u) * (inputs / BLOCK) + input / BLOCK];
+        return 0;
+    }
     if (format == ORC_FORMAT_E2M1_SCALED) {
         const uint32_t loads = inputs / 64u, load = input / 64u, within = input % 64u;
         const uint32_t step = within / 16u, j = within % 16u;
@@ -235,7 +312,7 @@ static void tile_values(int format, uint32_t outputs, uint32_t inputs, const uin
             uint32_t code, scale;
             (void)orc_linear_read(format, outputs, inputs, stored, 16u * tile + o, input, &code, &scale);
             values_out[(uint64_t)o * inputs + input] =
-                (float)(format == ORC_FORMAT_E2M1_SCALED ? orc_e2m1_value(code) : orc_e4m3_value(code));
+                (float)(holds_nibbles(format) ? orc_e2m1_value(code) : orc_e4m3_value(code));
             if (input % BLOCK == 0u) {
                 scale_exponents_out[o * (inputs / BLOCK) + input / BLOCK] = (int)scale - 127;
             }

@@ -32,6 +32,16 @@
 #define ORC_FORMAT_E4M3_SCALED 5
 #define ORC_FORMAT_E4M3_BLOCK128 6 /* no reference counterpart: E4M3 codes in E4M3_SCALED's lane order, then one float32
                                     * scale for every 128 outputs x 128 inputs, [outputs / 128][inputs / 128] */
+/* no reference counterpart either: the two _SCALED formats' weights and scale codes in the lane order of gfx950's matrix
+ * instruction. A matrix is tiles of 16 outputs by K steps of 128 inputs, tile after tile, step after step; a step is 64
+ * lanes, lane 16 g + o holding output o of the tile.
+ *   E2M1_GFX950: 16 bytes a lane; nibble n (0: low) of byte b of word T is input 32 g + 16 n + 2 T + {0, 8, 1, 9}[b] of
+ *     the step; behind all tiles one scale byte a lane a step a tile: the E8M0 code of output o, inputs 32 g .. + 31.
+ *   E4M3_GFX950: 32 bytes a lane, as two halves [half][lane][16]; byte c of word v (half v / 4) is input
+ *     64 (v / 4) + 16 g + 8 (c % 2) + 2 (v % 4) + c / 2; the scale codes as E4M3_SCALED's.
+ * Inputs a multiple of 128; outputs of 16 (E2M1) or 32 (E4M3). */
+#define ORC_FORMAT_E2M1_GFX950 7
+#define ORC_FORMAT_E4M3_GFX950 8
 
 uint64_t orc_linear_stored_bytes(int format, uint32_t outputs, uint32_t inputs);
 uint64_t orc_linear_scale_count(int format, uint32_t outputs, uint32_t inputs);
