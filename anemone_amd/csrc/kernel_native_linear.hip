@@ -86,11 +86,19 @@ __device__ static __forceinline__ void native_vectors_of(const struct wide_pair 
 }
 
 /* grid (ceil(output_size / (4 strips)), tile_count), block 256; a strip is STRIP tiles of gate and STRIP of up */
+/* sets of weight registers and stages of columns: 4-bit weights 3 and 2 (156 registers: three wavefronts a SIMD; with a
+ * third stage 177, and two wavefronts measured 8 % slower, held to 168 by spills 38 % slower); one-byte weights 4 and 3
+ * (6 and 3 measured the same) */
+template <bool BYTES>
+struct native_depths {
+    static constexpr uint32_t SLOTS = BYTES ? 4u : 3u, DEPTH = BYTES ? NATIVE_E4M3_STAGES : NATIVE_E2M1_STAGES;
+};
+
 template <bool BYTES, uint32_t STRIP, uint32_t GROUP>
 __device__ static __forceinline__ void native_expert_gate_up(const struct wide_expert_gate_up_arguments &arguments, unsigned char *arena)
 {
     constexpr uint32_t COLUMN_BLOCKS = 4u * GROUP;
-    typedef native_chain<2, BYTES, STRIP, COLUMN_BLOCKS> chain_type;
+    typedef native_chain<2, BYTES, STRIP, COLUMN_BLOCKS, native_depths<BYTES>::SLOTS, native_depths<BYTES>::DEPTH> chain_type;
     constexpr uint32_t TILES = chain_type::TILES;
     static_assert(STRIP == 1u || STRIP == 2u, "a quantizer block of 32 outputs is one strip or two");
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
@@ -124,7 +132,7 @@ template <bool BYTES, uint32_t GROUP>
 __device__ static __forceinline__ void native_expert_down(const struct wide_expert_down_arguments &arguments, unsigned char *arena)
 {
     constexpr uint32_t COLUMN_BLOCKS = 4u * GROUP;
-    typedef native_chain<1, BYTES, (BYTES ? 2u : 4u), COLUMN_BLOCKS> chain_type;
+    typedef native_chain<1, BYTES, (BYTES ? 2u : 4u), COLUMN_BLOCKS, native_depths<BYTES>::SLOTS, native_depths<BYTES>::DEPTH> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -154,27 +162,31 @@ __device__ static __forceinline__ void native_expert_down(const struct wide_expe
 }
 
 /* E2M1_GFX950 experts: a block is one tile of pairs by 128 outputs of gate and up (256 of down); E4M3_GFX950 experts: two
- * tiles by 64 (128 of down). The LDS window is dynamic shared memory: NATIVE_WINDOW_BYTES(column blocks). */
-extern "C" __global__ void __launch_bounds__(NATIVE_THREADS) native_expert_gate_up_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
+ * tiles by 64 (128 of down). The LDS window is dynamic shared memory: NATIVE_WINDOW_BYTES(column blocks, stages). */
+#define NATIVE_E2M1_WAVES 3 /* 168 registers */
+extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E2M1_WAVES) native_expert_gate_up_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
 {
-    native_expert_gate_up<false, 2u, 1u>(arguments, arena);
+    native_expert_gate_up<false, 2u, NATIVE_E2M1_COLUMN_BLOCKS / 4u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_gate_up_1, wide_expert_gate_up_arguments);
-extern "C" __global__ void __launch_bounds__(NATIVE_THREADS) native_expert_down_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
+extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E2M1_WAVES) native_expert_down_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
 {
-    native_expert_down<false, 1u>(arguments, arena);
+    native_expert_down<false, NATIVE_E2M1_COLUMN_BLOCKS / 4u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_down_1, wide_expert_down_arguments);
-extern "C" __global__ void __launch_bounds__(NATIVE_THREADS) native_expert_gate_up_e4m3_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
+#define NATIVE_E4M3_WAVES 2 /* wavefronts a SIMD the launch is compiled for: 256 registers */
+extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E4M3_WAVES) native_expert_gate_up_e4m3_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
 {
-    native_expert_gate_up<true, 1u, 2u>(arguments, arena);
+    native_expert_gate_up<true, 1u, NATIVE_E4M3_COLUMN_BLOCKS / 4u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_gate_up_e4m3_1, wide_expert_gate_up_arguments);
-extern "C" __global__ void __launch_bounds__(NATIVE_THREADS) native_expert_down_e4m3_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
+extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E4M3_WAVES) native_expert_down_e4m3_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
 {
-    native_expert_down<true, 2u>(arguments, arena);
+    native_expert_down<true, NATIVE_E4M3_COLUMN_BLOCKS / 4u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_down_e4m3_1, wide_expert_down_arguments);
 
-static_assert(native_chain<2, false, 2u, 4u>::WINDOW_BYTES == NATIVE_WINDOW_BYTES(4u) && native_chain<1, true, 2u, 8u>::WINDOW_BYTES == NATIVE_WINDOW_BYTES(8u),
+static_assert(native_chain<2, false, 2u, NATIVE_E2M1_COLUMN_BLOCKS, 3u, NATIVE_E2M1_STAGES>::WINDOW_BYTES == NATIVE_WINDOW_BYTES(NATIVE_E2M1_COLUMN_BLOCKS, NATIVE_E2M1_STAGES) &&
+                  native_chain<1, true, 2u, NATIVE_E4M3_COLUMN_BLOCKS, 4u, NATIVE_E4M3_STAGES>::WINDOW_BYTES == NATIVE_WINDOW_BYTES(NATIVE_E4M3_COLUMN_BLOCKS, NATIVE_E4M3_STAGES),
               "the windows the host asks for are the kernels'");
+

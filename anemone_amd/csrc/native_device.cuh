@@ -8,7 +8,7 @@
  * by LDS DMA, turned into the B operand's order in place by the wavefront that brought them.
  *
  * A block is COLUMN_BLOCKS x 16 columns (pairs of one expert) by four wavefronts' strips of weight tiles. A wavefront
- * keeps three sets of weight registers: while step s is multiplied, the loads of s + 1 and s + 2 are on their way.
+ * keeps several sets of weight registers: while one step is multiplied, the loads of the steps behind it are on their way.
  */
 #ifndef NATIVE_DEVICE_CUH
 #define NATIVE_DEVICE_CUH
@@ -17,19 +17,30 @@
 
 #define NATIVE_WAVES 4u
 #define NATIVE_THREADS (NATIVE_WAVES * WAVE)
-#define NATIVE_SLOTS 3u
 
 /* memory into registers, 16 bytes or one byte a lane: the address is a base common to the wavefront plus the lane's own
  * byte offset (plus 1,024: the second half of a tile of one-byte weights). Assembly, like the loads into LDS beside which
- * they are counted: the compiler keeps no book on them, native_landed is the wait. */
+ * they are counted: the compiler keeps no book on them, native_landed is the wait. ONCE: the bytes are read by this
+ * block alone (an expert's one-byte weights in a block that holds all its pairs): asked for as a stream, so that they do
+ * not push the columns, which every block of the expert reads, out of the level-2 cache. */
+template <bool ONCE>
 __device__ static __forceinline__ void load_16(uint4_t &into, const unsigned char *base, uint32_t lane_offset)
 {
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
+    if constexpr (ONCE) {
+        asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
+    } else {
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
+    }
 }
 
+template <bool ONCE>
 __device__ static __forceinline__ void load_16_second(uint4_t &into, const unsigned char *base, uint32_t lane_offset)
 {
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
+    if constexpr (ONCE) {
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024 nt" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
+    } else {
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
+    }
 }
 
 __device__ static __forceinline__ void load_1(uint32_t &into, const unsigned char *base, uint32_t lane_offset)
@@ -49,7 +60,9 @@ __device__ static __forceinline__ void native_landed(uint32_t &value)
     asm volatile("" : "+v"(value));
 }
 
-template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES, uint32_t COLUMN_BLOCKS>
+/* SLOTS: sets of weight registers a wavefront keeps (the weights of SLOTS - 1 steps are on their way while one is
+ * multiplied); DEPTH: stages of columns in LDS, likewise */
+template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES, uint32_t COLUMN_BLOCKS, uint32_t SLOTS, uint32_t DEPTH>
 struct native_chain {
     static_assert(COLUMN_BLOCKS == 4u || COLUMN_BLOCKS == 8u, "a wavefront brings one or two column blocks");
     static constexpr uint32_t STRIP = STRIP_TILES;
@@ -59,11 +72,10 @@ struct native_chain {
     static constexpr uint32_t WAVE_BLOCKS = COLUMN_BLOCKS / NATIVE_WAVES;     /* column blocks a wavefront brings and prepares */
     static constexpr uint32_t VECTOR_BYTES = COLUMN_BLOCKS * 2048u;            /* a K step of the block's columns' codes */
     static constexpr uint32_t STAGE_BYTES = VECTOR_BYTES + COLUMN_BLOCKS * 64u; /* and their scale words behind them */
-    static constexpr uint32_t DEPTH = 2u;
     static constexpr uint32_t WINDOW_BYTES = DEPTH * STAGE_BYTES;
     static constexpr uint32_t VECTOR_LOADS = 2u * WAVE_BLOCKS + 1u;
     static constexpr uint32_t WEIGHT_LOADS = TILES * HALVES + TILES;
-    static_assert(VECTOR_LOADS + 2u * WEIGHT_LOADS < 64u, "vmcnt has six bits");
+    static_assert((DEPTH - 1u) * VECTOR_LOADS + (SLOTS - 1u) * WEIGHT_LOADS < 64u, "vmcnt has six bits");
 
     struct slot {
         uint4_t words[TILES][HALVES];
@@ -71,6 +83,7 @@ struct native_chain {
     };
 
     const unsigned char *words[MATRICES], *scales[MATRICES], *codes, *exponents;
+    uint32_t step_stride; /* from a tile's K step to its next */
     uint32_t window, wave, word_offset[STRIP], scale_offset[STRIP], codes_offset[WAVE_BLOCKS][2], exponents_offset;
     uint32_t vector_at[BYTES ? 8 : 4], vector_scale_at, operand_at;
     bool scale_lane;
@@ -108,12 +121,12 @@ struct native_chain {
     {
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
-            const unsigned char *step_words = words[m] + (uint64_t)at * STEP_BYTES;
+            const unsigned char *step_words = words[m] + (uint64_t)at * step_stride;
 #pragma unroll
             for (uint32_t n = 0; n < STRIP; n++) {
-                load_16(into.words[m * STRIP + n][0], step_words, word_offset[n]);
+                load_16<BYTES>(into.words[m * STRIP + n][0], step_words, word_offset[n]);
                 if constexpr (BYTES) {
-                    load_16_second(into.words[m * STRIP + n][1], step_words, word_offset[n]);
+                    load_16_second<BYTES>(into.words[m * STRIP + n][1], step_words, word_offset[n]);
                 }
             }
         }
@@ -177,21 +190,29 @@ struct native_chain {
         uint32_t b_at = base + operand_at, b_scale_at = base + VECTOR_BYTES + vector_scale_at;
         asm volatile("" : "+v"(b_at), "+v"(b_scale_at));
         __builtin_amdgcn_s_setprio(1);
+        /* a column block's operand is read while the block before it is multiplied: two blocks' registers, not LIVE */
+        uint4_t low = lds_read<uint4_t>(b_at), high = lds_read<uint4_t>(b_at + 1024u);
+        uint32_t scale_b = lds_read<unsigned char>(b_scale_at);
 #pragma unroll
         for (uint32_t j = 0; j < LIVE; j++) {
-            const uint4_t low = lds_read<uint4_t>(b_at + j * 2048u), high = lds_read<uint4_t>(b_at + j * 2048u + 1024u);
             const int8_vector b = {(int)low.x, (int)low.y, (int)low.z, (int)low.w, (int)high.x, (int)high.y, (int)high.z, (int)high.w};
-            const uint32_t scale_b = lds_read<unsigned char>(b_scale_at + j * 64u);
+            const uint32_t scale_now = scale_b;
+            asm volatile("" ::: "memory"); /* the reads below stay below the reads above, and above those of the next block */
+            if (j + 1u < LIVE) {
+                low = lds_read<uint4_t>(b_at + (j + 1u) * 2048u);
+                high = lds_read<uint4_t>(b_at + (j + 1u) * 2048u + 1024u);
+                scale_b = lds_read<unsigned char>(b_scale_at + (j + 1u) * 64u);
+            }
 #pragma unroll
             for (uint32_t t = 0; t < TILES; t++) {
                 if constexpr (BYTES) {
                     const uint4_t first = set.words[t][0], second = set.words[t][HALVES - 1u];
                     const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
-                    chain[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[t][j], 0, 0, 0, (int)set.scale[t], 0, (int)scale_b);
+                    chain[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[t][j], 0, 0, 0, (int)set.scale[t], 0, (int)scale_now);
                 } else {
                     const uint4_t w = set.words[t][0];
                     const int8_vector a = {(int)w.x, (int)w.y, (int)w.z, (int)w.w, 0, 0, 0, 0};
-                    chain[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[t][j], 4, 0, 0, (int)set.scale[t], 0, (int)scale_b);
+                    chain[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[t][j], 4, 0, 0, (int)set.scale[t], 0, (int)scale_now);
                 }
             }
         }
@@ -199,48 +220,109 @@ struct native_chain {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stage is read before the next barrier */
     }
 
-    /* K step `step` of `total` out of set `now`; `behind` is the set step - 1 used, which step + 2 takes.
-     * Loads in the order they are asked for: ... columns of `step`, weights of step + 1 | columns of step + 1, weights of
-     * step + 2. At the top everything up to the columns of `step` has landed once no more than the weights of step + 1
-     * are outstanding; the weights of `step` were asked for before those columns. */
-    template <uint32_t LIVE>
-    __device__ __forceinline__ void one_step(uint32_t step, uint32_t total, slot &now, slot &behind,
-                                             float4_t (&chain)[TILES][COLUMN_BLOCKS]) const
+    /* How many loads may be outstanding at the top of K step `step` for its columns and weights to have landed. Loads in
+     * the order they are asked for: the columns of steps 0 .. DEPTH - 2, the weights of steps 0 .. SLOTS - 2, then, in
+     * every step j, the columns of step j + DEPTH - 1 and behind them the weights of step j + SLOTS - 1 (where the chain
+     * has such steps). The count is of the loads of later steps asked for behind the later of the two. */
+    __device__ static __forceinline__ uint32_t when_columns(uint32_t k)
     {
-        if (step + 1u < total) {
-            wait_loads<WEIGHT_LOADS>();
+        return k < DEPTH - 1u ? k : 64u * (1u + k - (DEPTH - 1u));
+    }
+
+    __device__ static __forceinline__ uint32_t when_weights(uint32_t k)
+    {
+        return k < SLOTS - 1u ? DEPTH - 1u + k : 64u * (1u + k - (SLOTS - 1u)) + 1u;
+    }
+
+    __device__ static __forceinline__ uint32_t loads_behind(uint32_t step, uint32_t total)
+    {
+        static_assert(SLOTS >= DEPTH && DEPTH >= 2u && SLOTS + DEPTH < 64u, "the weights are asked for at least as far ahead as the columns");
+        const uint32_t mine = when_columns(step) > when_weights(step) ? when_columns(step) : when_weights(step);
+        const uint32_t now = 64u * (1u + step); /* what steps before this one asked for lies below this */
+        uint32_t count = 0;
+#pragma unroll
+        for (uint32_t ahead = 1; ahead < SLOTS; ahead++) {
+            const uint32_t k = step + ahead;
+            if (k < total) {
+                count += when_columns(k) > mine && when_columns(k) < now ? VECTOR_LOADS : 0u;
+                count += when_weights(k) > mine && when_weights(k) < now ? WEIGHT_LOADS : 0u;
+            }
+        }
+        return count;
+    }
+
+    /* s_waitcnt takes its count as a constant: one instruction a count that loads_behind can come to */
+    template <uint32_t WEIGHTS = 0, uint32_t VECTORS = 0>
+    __device__ static __forceinline__ void wait_behind(uint32_t count)
+    {
+        if (count == WEIGHTS * WEIGHT_LOADS + VECTORS * VECTOR_LOADS) {
+            wait_loads<WEIGHTS * WEIGHT_LOADS + VECTORS * VECTOR_LOADS>();
+            return;
+        }
+        if constexpr (VECTORS + 1u < DEPTH - 1u) {
+            wait_behind<WEIGHTS, VECTORS + 1u>(count);
+        } else if constexpr (WEIGHTS + 1u < SLOTS) {
+            wait_behind<WEIGHTS + 1u, 0u>(count);
         } else {
-            wait_loads<0>();
+            wait_loads<0>(); /* not reached: every count is one of the above */
         }
-        landed(now);
-        prepare_columns(step % 2u);
+    }
+
+    /* K step `step` of `total` out of set K of the wavefront's sets of weight registers; the weights of step
+     * `step` + SLOTS - 1 take the set the step before this one used */
+    template <uint32_t LIVE, uint32_t K>
+    __device__ __forceinline__ void one_step(uint32_t step, uint32_t total, slot (&sets)[SLOTS], float4_t (&chain)[TILES][COLUMN_BLOCKS]) const
+    {
+        wait_behind(loads_behind(step, total));
+        landed(sets[K]);
+        /* where the sets and the stages go round together the stage is a constant of the instance */
+        const uint32_t stage = SLOTS % DEPTH == 0u ? K % DEPTH : step % DEPTH;
+        prepare_columns(stage);
         __syncthreads(); /* every wavefront has read the step before and prepared its columns of this one */
-        if (step + 1u < total) {
-            issue_vectors((step + 1u) % 2u, step + 1u);
+        if (step + DEPTH - 1u < total) {
+            issue_vectors((stage + DEPTH - 1u) % DEPTH, step + DEPTH - 1u);
         }
-        if (step + 2u < total) {
-            issue_weights(behind, step + 2u);
+        if (step + SLOTS - 1u < total) {
+            issue_weights(sets[(K + SLOTS - 1u) % SLOTS], step + SLOTS - 1u);
         }
-        consume<LIVE>(step % 2u, now, chain);
+        consume<LIVE>(stage, sets[K], chain);
+    }
+
+    template <uint32_t LIVE, uint32_t K>
+    __device__ __forceinline__ void round_of_steps(uint32_t step, uint32_t total, slot (&sets)[SLOTS], float4_t (&chain)[TILES][COLUMN_BLOCKS]) const
+    {
+        if (step + K < total) {
+            one_step<LIVE, K>(step + K, total, sets, chain);
+        }
+        if constexpr (K + 1u < SLOTS) {
+            round_of_steps<LIVE, K + 1u>(step, total, sets, chain);
+        }
+    }
+
+    template <uint32_t K>
+    __device__ __forceinline__ void first_weights(uint32_t total, slot (&sets)[SLOTS]) const
+    {
+        if (K < total) {
+            issue_weights(sets[K], K);
+        }
+        if constexpr (K + 2u < SLOTS) {
+            first_weights<K + 1u>(total, sets);
+        }
     }
 
     template <uint32_t LIVE>
     __device__ __forceinline__ void steps(uint32_t total, float4_t (&chain)[TILES][COLUMN_BLOCKS]) const
     {
-        slot set0, set1, set2;
-        issue_vectors(0u, 0u);
-        issue_weights(set0, 0u);
-        if (total > 1u) {
-            issue_weights(set1, 1u);
+        slot sets[SLOTS];
+#pragma unroll
+        for (uint32_t k = 0; k + 1u < DEPTH; k++) {
+            if (k < total) {
+                issue_vectors(k, k);
+            }
         }
-        for (uint32_t step = 0; step < total; step += NATIVE_SLOTS) {
-            one_step<LIVE>(step, total, set0, set2, chain);
-            if (step + 1u < total) {
-                one_step<LIVE>(step + 1u, total, set1, set0, chain);
-            }
-            if (step + 2u < total) {
-                one_step<LIVE>(step + 2u, total, set2, set1, chain);
-            }
+        first_weights<0>(total, sets);
+        for (uint32_t step = 0; step < total; step += SLOTS) {
+            round_of_steps<LIVE, 0>(step, total, sets, chain);
         }
     }
 
@@ -282,6 +364,7 @@ struct native_chain {
         const uint32_t tile0 = strip * STRIP + STRIP <= tiles ? strip * STRIP : tiles - STRIP;
         tile0_out = tile0;
         const uint32_t tile_bytes = steps * STEP_BYTES;
+        step_stride = STEP_BYTES;
         window = window_address;
         wave = wave_index;
         codes = vector_codes;

@@ -35,12 +35,11 @@ __device__ static __forceinline__ void wide_gate_up_finish(const struct wide_exp
     const bool strip_is_live = first_output < width; /* else: a strip wholly past the matrix (its tiles were the strip's before it) */
     const float limit = arguments.activation_limit;
     const uint32_t g = lane / 16u, upper = g / 2u;
-    uint32_t bits[COLUMN_BLOCKS][STRIP][4];
-    float largest[COLUMN_BLOCKS];
-#pragma unroll
-    for (uint32_t j = 0; j < COLUMN_BLOCKS; j++) {
+    /* column block j: the hidden values of the lane's rows of its column, and the largest magnitude of the column's 16
+     * STRIP values of this strip (the same in the column's four lanes) */
+    const auto hidden_of = [&](uint32_t j, uint32_t (&bits)[STRIP][4]) -> float {
         const uint32_t column = 16u * j + lane % 16u;
-        largest[j] = 0.0f;
+        float largest = 0.0f;
         if (column < pair_count && strip_is_live) { /* the same in the four lanes of a column */
             const float weight = pairs[column].route_weight;
 #pragma unroll
@@ -52,8 +51,8 @@ __device__ static __forceinline__ void wide_gate_up_finish(const struct wide_exp
                     const float bounded_gate = fminf(gate, limit);
                     const float bounded_up = fminf(fmaxf(up, -limit), limit);
                     const float value = __fmul_rn(__fmul_rn(linear_silu(bounded_gate), bounded_up), weight);
-                    bits[j][n][v] = float_to_bf16(value);
-                    largest[j] = fmaxf(largest[j], fabsf(bf16_to_float((uint16_t)bits[j][n][v])));
+                    bits[n][v] = float_to_bf16(value);
+                    largest = fmaxf(largest, fabsf(bf16_to_float((uint16_t)bits[n][v])));
                 }
             }
             if constexpr (B128) {
@@ -62,12 +61,57 @@ __device__ static __forceinline__ void wide_gate_up_finish(const struct wide_exp
                 uint16_t *values = (uint16_t *)(arena + arguments.hidden_operands_offset) + (uint64_t)pairs[column].pair_index * width;
 #pragma unroll
                 for (uint32_t n = 0; n < STRIP; n++) {
-                    *(uint2_t *)(values + (tile0 + n) * 16u + 4u * g) = (uint2_t){bits[j][n][0] | (bits[j][n][1] << 16), bits[j][n][2] | (bits[j][n][3] << 16)};
+                    *(uint2_t *)(values + (tile0 + n) * 16u + 4u * g) = (uint2_t){bits[n][0] | (bits[n][1] << 16), bits[n][2] | (bits[n][3] << 16)};
                 }
             }
-            largest[j] = fmaxf(largest[j], __shfl_xor(largest[j], 16, WAVE));
-            largest[j] = fmaxf(largest[j], __shfl_xor(largest[j], 32, WAVE));
+            largest = fmaxf(largest, __shfl_xor(largest, 16, WAVE));
+            largest = fmaxf(largest, __shfl_xor(largest, 32, WAVE));
         }
+        return largest;
+    };
+    /* column block j: the quantizer's step on those values under the block's largest magnitude, and its stores */
+    const auto store_of = [&](uint32_t j, const uint32_t (&bits)[STRIP][4], float largest) {
+        const uint32_t column = 16u * j + lane % 16u;
+        if (column < pair_count) {
+            const uint64_t pair = pairs[column].pair_index;
+            const uint32_t code_exponent = quantize_exponent_code(largest);
+            unsigned char *codes = arena + arguments.hidden_codes_offset + pair * width;
+            uint16_t *operands = (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width;
+#pragma unroll
+            for (uint32_t n = 0; n < STRIP; n++) {
+                uint32_t own, carried[4];
+                quantize_codes4(bits[n], code_exponent, own, carried);
+                const uint32_t load = (tile0 + n) / 4u, step = (tile0 + n) % 4u, t = 2u * (g % 2u);
+                const uint32_t word0 = quantize_word_of(load, step, t), word1 = quantize_word_of(load, step, t + 1u);
+                /* word0 is (a0, b0, a1, b1) and word1 (a2, b2, a3, b3) of the codes a of the lower lane and b of the
+                 * upper: each takes the other's four and stores one of the words */
+                const uint32_t other = (uint32_t)__shfl_xor((int)own, 32, WAVE);
+                *(uint32_t *)(codes + (upper != 0u ? word1 : word0)) = __builtin_amdgcn_perm(other, own, upper != 0u ? 0x03070206u : 0x05010400u);
+                *(uint32_t *)(operands + word0 + 2u * upper) = quantize_operand_pair(carried[0], carried[1], code_exponent);
+                *(uint32_t *)(operands + word1 + 2u * upper) = quantize_operand_pair(carried[2], carried[3], code_exponent);
+            }
+            if (g == 0u && first_output % 32u == 0u) {
+                (arena + arguments.hidden_exponents_offset)[pair * (width / 32u) + first_output / 32u] = (unsigned char)code_exponent;
+            }
+        }
+    };
+    if constexpr (STRIP == 2u && !B128) {
+        /* a quantizer block is this wavefront's own: a column block at a time, its values in eight registers */
+#pragma unroll
+        for (uint32_t j = 0; j < COLUMN_BLOCKS; j++) {
+            uint32_t bits[STRIP][4];
+            const float largest = hidden_of(j, bits);
+            if (strip_is_live) {
+                store_of(j, bits, largest);
+            }
+        }
+        return;
+    }
+    uint32_t bits[COLUMN_BLOCKS][STRIP][4];
+    float largest[COLUMN_BLOCKS];
+#pragma unroll
+    for (uint32_t j = 0; j < COLUMN_BLOCKS; j++) {
+        largest[j] = hidden_of(j, bits[j]);
     }
     if constexpr (B128) {
         return;
@@ -92,29 +136,7 @@ __device__ static __forceinline__ void wide_gate_up_finish(const struct wide_exp
     }
 #pragma unroll
     for (uint32_t j = 0; j < COLUMN_BLOCKS; j++) {
-        const uint32_t column = 16u * j + lane % 16u;
-        if (column < pair_count) {
-            const uint64_t pair = pairs[column].pair_index;
-            const uint32_t code_exponent = quantize_exponent_code(largest[j]);
-            unsigned char *codes = arena + arguments.hidden_codes_offset + pair * width;
-            uint16_t *operands = (uint16_t *)(arena + arguments.hidden_operands_offset) + pair * width;
-#pragma unroll
-            for (uint32_t n = 0; n < STRIP; n++) {
-                uint32_t own, carried[4];
-                quantize_codes4(bits[j][n], code_exponent, own, carried);
-                const uint32_t load = (tile0 + n) / 4u, step = (tile0 + n) % 4u, t = 2u * (g % 2u);
-                const uint32_t word0 = quantize_word_of(load, step, t), word1 = quantize_word_of(load, step, t + 1u);
-                /* word0 is (a0, b0, a1, b1) and word1 (a2, b2, a3, b3) of the codes a of the lower lane and b of the
-                 * upper: each takes the other's four and stores one of the words */
-                const uint32_t other = (uint32_t)__shfl_xor((int)own, 32, WAVE);
-                *(uint32_t *)(codes + (upper != 0u ? word1 : word0)) = __builtin_amdgcn_perm(other, own, upper != 0u ? 0x03070206u : 0x05010400u);
-                *(uint32_t *)(operands + word0 + 2u * upper) = quantize_operand_pair(carried[0], carried[1], code_exponent);
-                *(uint32_t *)(operands + word1 + 2u * upper) = quantize_operand_pair(carried[2], carried[3], code_exponent);
-            }
-            if (g == 0u && first_output % 32u == 0u) {
-                (arena + arguments.hidden_exponents_offset)[pair * (width / 32u) + first_output / 32u] = (unsigned char)code_exponent;
-            }
-        }
+        store_of(j, bits[j], largest[j]);
     }
 }
 

@@ -604,7 +604,8 @@ static result_status wide_experts_prepare(const struct linear_wide_experts_descr
     if (native) {
         gate_up_kernel = bytes ? native_kernels->native_expert_gate_up_e4m3 : native_kernels->native_expert_gate_up;
         down_kernel = bytes ? native_kernels->native_expert_down_e4m3 : native_kernels->native_expert_down;
-        gate_up_window = down_window = NATIVE_WINDOW_BYTES(bytes ? NATIVE_E4M3_COLUMN_BLOCKS : NATIVE_E2M1_COLUMN_BLOCKS);
+        gate_up_window = down_window = bytes ? NATIVE_WINDOW_BYTES(NATIVE_E4M3_COLUMN_BLOCKS, NATIVE_E4M3_STAGES)
+                                             : NATIVE_WINDOW_BYTES(NATIVE_E2M1_COLUMN_BLOCKS, NATIVE_E2M1_STAGES);
     } else {
         gate_up_kernel = block128 ? kernels->wide_expert_gate_up_b128 : bytes ? kernels->wide_expert_gate_up_e4m3 : kernels->wide_expert_gate_up;
         down_kernel = block128 ? kernels->wide_expert_down_b128 : bytes ? kernels->wide_expert_down_e4m3 : kernels->wide_expert_down;

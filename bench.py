@@ -138,6 +138,9 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     distinct_generated = 4 if fp8 else 16
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
     block128 = fp8 and arguments.block128  # float32 scales of 128 x 128 blocks and of 128 values (the usual FP8 block scaling)
+    native = getattr(arguments, "native", False)  # the weights in gfx950's own lane order (a load-time re-lay-out of the same bytes)
+    if native and (block128 or not prefill):
+        raise SystemExit("--native: the wide (prefill) launches of the reference's scalings take it")
     matrix = workloads.fp8_block128_matrix if block128 else workloads.fp8_matrix if fp8 else workloads.fp4_matrix
     trios = [[matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
               matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
@@ -147,8 +150,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     card = amd.Card(((9 if fp8 else 5) << 30) + rows * (1 << 18))
     layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router,
                          gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices,
-                         weight_format=amd.WEIGHT_FORMAT_E4M3_BLOCK128 if block128 else amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else
-                         amd.WEIGHT_FORMAT_E2M1_SCALED)
+                         weight_format=(amd.WEIGHT_FORMAT_E4M3_GFX950 if fp8 else amd.WEIGHT_FORMAT_E2M1_GFX950) if native else
+                         amd.WEIGHT_FORMAT_E4M3_BLOCK128 if block128 else amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED)
     layer.set_rows(x, rows)
     wide = layer.wide_router() if rows > 8 or prefill else None  # more than eight rows: the wide select sorts the pairs by expert
     small = wide is not None and rows <= amd.ROUTER_SORT_ROWS and not prefill  # count, place and jobs in one block
@@ -239,7 +242,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         "scaling": "weak", "vs_baseline": None, "dtype": "fp8 x fp8 -> f32" if fp8 else "fp4 x fp8 -> f32", "data": "synthetic",
         "config": {"workload": "%s_moe_decode: %d tokens, H 4096, 256 experts x I 2048, top-8, %s"
                                % ("fp8" if fp8 else "fp4", rows, "E4M3, f32 scales per 128x128 / per 128" if block128 else
-                                  "E4M3, E8M0 scales per 32x32" if fp8 else "E2M1, E8M0 scales per 32"),
+                                  "E4M3, E8M0 scales per 32x32" if fp8 else "E2M1, E8M0 scales per 32") + (", gfx950 lane order" if native else ""),
                    "distinct_experts": int(len(distinct)), "jobs": int(len(live)),
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "down_GBps": matrix_bytes * len(distinct) / (down_us * 1e-6) / 1e9},
@@ -270,6 +273,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     key = ("%s_%s" % ("fp8" if fp8 else "fp4", "prefill" if prefill else "decode"), rows)
     if block128:
         key = (key[0] + "_block128", rows)
+    if native:
+        key = (key[0] + "_native", rows)
     if key in MEASURED_TRAFFIC_BYTES and (prefill or (arguments.gate_up_slices, arguments.down_slices) == (4, 2)):
         result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES[key]
         result["roofline"]["traffic_source"] = TRAFFIC_SOURCE[key[0]] + " (counter bytes of the profiled run, not of this one)"
@@ -284,7 +289,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         result["config"]["step_TFLOPs"] = (gate_up_flops + down_flops) / (seconds / arguments.steps) / 1e12
         # the products are MFMAs of FP8 activations (with FP4 or FP8 weights): the FP8 rate is the instruction's peak.
         # What bounds the launch is read off its arithmetic intensity against the card's balance of the two peaks.
-        kernel = "wide_expert_gate_up_%s1" % ("b128_" if block128 else "e4m3_" if fp8 else "")
+        kernel = ("native_expert_gate_up_%s1" if native else "wide_expert_gate_up_%s1") % ("b128_" if block128 else "e4m3_" if fp8 else "")
         if gate_up_flops / gate_up_bytes >= MFMA_F8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9):
             result["roofline"] = {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_F8_PEAK_TFLOPS, "unit": "TFLOP/s",
                                   "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": result["roofline"]["traffic"],
@@ -337,6 +342,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
         want = np.zeros((sample, HIDDEN), dtype=np.float32)
         want_pairs = np.zeros((sample * PICKS, HIDDEN), dtype=np.uint16)
         start = time.perf_counter()
+        # the oracle reads the reference's bytes, from which the card's native lay-out was made
         o.orc.orc_linear_moe_layer(6 if block128 else 5 if fp8 else 3, o.ptr(np.ascontiguousarray(x[:sample]), o.u16p), sample, HIDDEN, INNER, PICKS,
                                    o.ptr(np.ascontiguousarray(experts_of[:sample]), o.u32p),
                                    o.ptr(np.ascontiguousarray(weights_of[:sample]), o.f32p), EXPERTS, pointers, 10.0,
@@ -639,6 +645,9 @@ def main():
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--block128", action="store_true",
                         help="fp8 workloads: float32 scales of 128 x 128 weight blocks and of 128 activation values in place of the reference's E8M0 scales")
+    parser.add_argument("--native", action="store_true",
+                        help="fp4_prefill / fp8_prefill: the experts' weights in gfx950's own lane order (WEIGHT_FORMAT_E2M1_GFX950 / _E4M3_GFX950, "
+                             "made from the same bytes by the library's load-time re-lay-out)")
     parser.add_argument("--site", action="store_true",
                         help="fp4/fp8 workloads: the whole FFN site: the mix project and mix finish ahead of the router, the shared expert and the join "
                              "in place of the row sum")
