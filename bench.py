@@ -590,7 +590,7 @@ def exl3_decode(amd, workloads, arguments):
             cpu_seconds, want, experts = cpu_oracle_step(_oracle, x, router, matrices, widths, threads)
             outputs[:] = [want, experts]
             return cpu_seconds
-        cpu_seconds = median_seconds(one_step, 1, 5)  # every step reads the experts' 0.55 GB anew: cold to the host's caches
+        cpu_seconds = median_seconds(one_step, 4, 20)  # every step reads the experts' 0.55 GB anew: cold to the host's caches
         want, experts = outputs
         rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
         error = float(np.max(np.abs(got - want))) / rms
@@ -598,9 +598,80 @@ def exl3_decode(amd, workloads, arguments):
         assert error <= 4e-3, "GPU output differs from the oracle's: %g of rms" % error
         result["cpu_baseline"] = {"value": ROWS / cpu_seconds, "unit": "tok/s", "cores": threads, "kind": "port",
                                   "sample": "the same step (8 tokens, %d experts) by the CPU oracle (routing and experts, two C calls; "
-                                            "double-precision sums): 1 warm-up, median of 5" % len(distinct),
+                                            "double-precision sums): 4 warm-ups, median of 20" % len(distinct),
                                   "seconds": cpu_seconds, "gpu_vs_oracle_max_err_over_rms": error}
     card.close()
+    return result
+
+
+def exl3_linear(amd, workloads, arguments):
+    """BASELINE's configuration 0: one EXL3 linear y = (((x.suh)Hb)T)Hb.svh at 4096 x 4096, K = 4, batch 1, as the chain's
+    input, product and finish launches on one job, beside the CPU oracle's same product on one host core. Algorithmic
+    bytes: the stored matrix (codes, suh, svh), the bfloat16 input and the float32 output: 8,429,568."""
+    import ctypes as C
+    n, width = 4096, 4
+    matrix = workloads.exl3_matrix(workloads.SEED, n, n, width)
+    x = workloads.to_bf16(workloads.normals(workloads.SEED + 1, n))
+    card = amd.Card(1 << 30)
+    at = card.place(matrix, 256)
+    jobs = np.zeros(1, dtype=amd.JOB_DTYPE)
+    jobs[0]["gate_offset"] = jobs[0]["up_offset"] = jobs[0]["down_offset"] = at
+    jobs[0]["row_count"], jobs[0]["route_weight"][0] = 1, 1.0
+    record = amd.Exl3ExpertRecord()
+    record.jobs_offset = card.place(jobs.view(np.uint8))
+    record.input_offset = card.place(x)
+    record.operands_offset = card.reserve(n * 4)
+    record.products_offset = record.output_offset = card.reserve(n * 8)
+    record.hidden_offset = card.reserve(n * 2)
+    record.input_size = record.inner_size = n
+    record.pair_count = record.pairs_per_row = record.job_count = 1
+    record.bits_per_weight, record.activation_limit = width, 10.0
+    launches = amd.launches_of(5)
+    amd.check(card.lib.exl3_experts_prepare(C.byref(record), card.arena_bytes, amd.backend_table(), card.handle, 950, launches), "exl3_experts_prepare")
+    step = amd.launches_of(3)
+    step[0], step[1], step[2] = launches[0], launches[3], launches[4]  # input, the product of one matrix, finish
+    step[0].grid[2] = 1
+    names = ["exl3_input", "exl3_down_k4", "exl3_finish"]
+    queue_steps(card, step, arguments.warmup, None)
+    card.wait()
+    device_us = card.measure(lambda: queue_steps(card, step, arguments.steps, None))
+    per_launch = np.zeros(3)
+    for _ in range(arguments.steps):
+        per_launch += np.array(card.run_timed(step))
+    per_launch /= arguments.steps
+    seconds = device_us * 1e-6
+    algorithmic = workloads.exl3_matrix_bytes(n, n, width) + n * 2 + n * 4
+    product_us = float(per_launch[1])
+    achieved = algorithmic / (product_us * 1e-6) / 1e9
+    result = {
+        "metric": "MoE layer tok/s; decode HBM GB/s & prefill MFMA % of peak, 1 GPU", "value": arguments.steps / seconds, "unit": "tok/s",
+        "n_gpus": 1, "steps": arguments.steps, "warmup": arguments.warmup, "ms_per_step": 1000.0 * seconds / arguments.steps,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "exl3_linear: one matrix 4096 x 4096, K 4, batch 1 (BASELINE configuration 0)",
+                   "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
+                   "step_GBps": algorithmic / (seconds / arguments.steps) / 1e9},
+        "roofline": {"bound": "hbm", "kernel": "exl3_down_k4 (the product launch)", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": int(algorithmic), "launch_us": product_us},
+    }
+    got = card.download(record.output_offset, n * 4, np.float32)
+    card.close()
+    if not arguments.no_cpu:
+        import _oracle as o
+        xs = o.bf16_to_f32(x).astype(np.float64)
+        want = np.zeros(n)
+
+        def once():
+            start = time.perf_counter()
+            o.orc.orc_exl3_linear_f64(o.ptr(matrix, o.u8p), n, n, width, o.ptr(xs, o.f64p), o.ptr(want, o.f64p))
+            return time.perf_counter() - start
+        cpu_seconds = median_seconds(once, 4, 20)
+        rms = float(np.sqrt(np.mean(want ** 2)))
+        error = float(np.max(np.abs(got - want))) / rms
+        assert error <= 2e-3, "GPU output differs from the oracle's: %g of rms" % error
+        result["cpu_baseline"] = {"value": 1.0 / cpu_seconds, "unit": "tok/s", "cores": 1, "kind": "port",
+                                  "sample": "the same product by the CPU oracle (orc_exl3_linear_f64, one thread, double-precision sums): "
+                                            "4 warm-ups, median of 20", "seconds": cpu_seconds, "GBps": algorithmic / cpu_seconds / 1e9,
+                                  "gpu_vs_oracle_max_err_over_rms": error}
     return result
 
 
@@ -620,12 +691,21 @@ def summary(result):
     for name in ("gpu_vs_oracle_max_err_over_rms", "gpu_vs_oracle_rms_err"):
         if name in baseline:
             keep[name] = baseline[name]
+    if config["workload"].startswith("exl3_linear"):
+        keep["launch_us_all"] = config["launch_us"]
+        keep["cpu_baseline"] = baseline
     return keep
 
 
 # the workloads of the other configurations the metric names, as the default run's config.also: (workload, rows, block128)
-ALSO = [("exl3_prefill", 4096, False), ("fp8_decode", 1, True), ("fp8_decode", 64, True), ("fp8_prefill", 2048, True),
-        ("fp8_prefill", 2048, False), ("fp4_prefill", 8192, False), ("fp4_decode", 32, False)]
+ALSO = [("exl3_linear", 1, False, False), ("exl3_prefill", 4096, False, False), ("fp8_decode", 1, True, False), ("fp8_decode", 64, True, False),
+        ("fp8_prefill", 2048, True, False), ("fp8_prefill", 2048, False, False), ("fp8_prefill", 2048, False, True),
+        ("fp4_prefill", 8192, False, False), ("fp4_prefill", 8192, False, True), ("fp4_decode", 32, False, False)]
+# the other configurations' headline fractions as scalars of config (beside config.also, which holds the whole lines)
+HEADLINES = {("exl3_linear", False, False): "exl3_linear_hbm_frac", ("exl3_prefill", False, False): "exl3_prefill_mfma_frac",
+             ("fp8_prefill", True, False): "fp8_block128_prefill_hbm_frac", ("fp8_prefill", False, False): "fp8_prefill_hbm_frac",
+             ("fp8_prefill", False, True): "fp8_gfx950_prefill_hbm_frac", ("fp4_prefill", False, False): "fp4_prefill_mfma_frac",
+             ("fp4_prefill", False, True): "fp4_gfx950_prefill_mfma_frac", ("fp4_decode", False, False): "fp4_decode32_hbm_frac"}
 
 
 def main():
@@ -635,7 +715,7 @@ def main():
     parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--workload", default="all",
                         help="all (default): exl3_decode as the line, the other configurations' workloads in config.also; or one of "
-                             "exl3_decode, exl3_prefill, fp4_decode, fp8_decode, fp4_prefill, fp8_prefill")
+                             "exl3_decode, exl3_linear, exl3_prefill, fp4_decode, fp8_decode, fp4_prefill, fp8_prefill")
     parser.add_argument("--zipf-strength", type=float, default=0.0,
                         help="exl3_prefill: 0 (default): the router's bias is fitted so that the experts' loads follow Zipf (s = 1.1), an "
                              "expert at most one pair a token; above 0: the bias is this times ln(Zipf pmf)")
@@ -658,7 +738,7 @@ def main():
     if arguments.gpus != 1:
         print("bench.py measures one GPU: this build holds no multi-GPU code (--gpus %d refused)" % arguments.gpus, file=sys.stderr)
         sys.exit(2)
-    if arguments.workload not in ("all", "exl3_decode", "fp4_decode", "fp8_decode", "exl3_prefill", "fp4_prefill", "fp8_prefill"):
+    if arguments.workload not in ("all", "exl3_decode", "exl3_linear", "fp4_decode", "fp8_decode", "exl3_prefill", "fp4_prefill", "fp8_prefill"):
         print("unknown workload %s" % arguments.workload, file=sys.stderr)
         sys.exit(2)
 
@@ -674,6 +754,8 @@ def main():
             return exl3_decode(amd, workloads, options)
         if workload == "exl3_prefill":
             return exl3_prefill(amd, workloads, options)
+        if workload == "exl3_linear":
+            return exl3_linear(amd, workloads, options)
         return fp4_decode(amd, workloads, options, fp8=workload.startswith("fp8"), prefill=workload.endswith("prefill"))
 
     if arguments.workload != "all":
@@ -681,15 +763,19 @@ def main():
         return
     result = run("exl3_decode", arguments)
     also = []
-    for workload, rows, block128 in ALSO:
+    for workload, rows, block128, native in ALSO:
         options = argparse.Namespace(**vars(arguments))
-        options.rows, options.block128, options.site, options.graph = rows, block128, False, False
+        options.rows, options.block128, options.native, options.site, options.graph = rows, block128, native, False, False
         prefill = workload.endswith("prefill")
         options.steps, options.warmup = (min(arguments.steps, 5), min(arguments.warmup, 2)) if prefill else (min(arguments.steps, 20), min(arguments.warmup, 5))
         start = time.perf_counter()
         entry = summary(run(workload, options))
         entry["bench_seconds"] = time.perf_counter() - start
         also.append(entry)
+        if (workload, block128, native) in HEADLINES:
+            result["config"][HEADLINES[(workload, block128, native)]] = entry["frac"]
+        if workload == "fp8_decode":
+            result["config"]["fp8_block128_decode%d_hbm_frac" % rows] = entry["frac"]
     result["config"]["also"] = also
     print(json.dumps(result))
 

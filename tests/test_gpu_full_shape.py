@@ -126,10 +126,13 @@ def test_prefill_of_4096_rows(amd, workloads, exl3_layer_tensors):
     assert error <= 4e-3
 
 
-@pytest.mark.parametrize("form,rows", [("fp4", 8192), ("fp8", 2048), ("fp8_block128", 2048)])
-def test_wide_experts_of_the_original_weights(amd, workloads, form, rows):
-    say("full shape: wide", form, rows, "rows")
-    fp8, block128 = form != "fp4", form == "fp8_block128"
+WIDE_RESULTS = {}  # form -> (picks, row outputs, hidden codes): a lay-out's run is kept for the other lay-out's comparison
+
+
+def run_wide_form(amd, workloads, form, rows):
+    if form in WIDE_RESULTS:
+        return WIDE_RESULTS[form]
+    fp8, block128, native = form.startswith("fp8"), form == "fp8_block128", form.endswith("_gfx950")
     distinct_generated = 4 if fp8 else 16
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
     matrix = workloads.fp8_block128_matrix if block128 else workloads.fp8_matrix if fp8 else workloads.fp4_matrix
@@ -138,11 +141,12 @@ def test_wide_experts_of_the_original_weights(amd, workloads, form, rows):
     matrices = [trios[e % distinct_generated] for e in range(EXPERTS)]
     router = workloads.to_bf16(workloads.normals(base + 2, EXPERTS * HIDDEN) * 0.02).reshape(EXPERTS, HIDDEN)
     x = workloads.activations(4, rows, HIDDEN)
+    weight_format = (amd.WEIGHT_FORMAT_E4M3_GFX950 if fp8 else amd.WEIGHT_FORMAT_E2M1_GFX950) if native else \
+        amd.WEIGHT_FORMAT_E4M3_BLOCK128 if block128 else amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED
     card = amd.Card(((9 if fp8 else 5) << 30) + rows * (1 << 18))
     try:
         layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router, gate_up_slices=4, down_slices=2,
-                             weight_format=amd.WEIGHT_FORMAT_E4M3_BLOCK128 if block128 else amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else
-                             amd.WEIGHT_FORMAT_E2M1_SCALED)
+                             weight_format=weight_format)
         layer.set_rows(x, rows)
         wide = layer.wide_router()
         experts_launches = layer.wide_expert_launches(wide)
@@ -152,12 +156,28 @@ def test_wide_experts_of_the_original_weights(amd, workloads, form, rows):
         card.run(experts_launches)
         picks = wide.read("picks", np.dtype([("expert", "<u4"), ("route_weight", "<f4")])).reshape(rows, PICKS)
         got = layer.read("row_output", np.float32).reshape(rows, HIDDEN)
+        hidden_codes = layer.read("hidden_codes").copy()
     finally:
         card.close()
+    WIDE_RESULTS[form] = (x, matrices, picks, got, hidden_codes)
+    return WIDE_RESULTS[form]
+
+
+@pytest.mark.parametrize("form,rows", [("fp4", 8192), ("fp8", 2048), ("fp8_block128", 2048), ("fp4_gfx950", 8192), ("fp8_gfx950", 2048)])
+def test_wide_experts_of_the_original_weights(amd, workloads, form, rows):
+    say("full shape: wide", form, rows, "rows")
+    fp8, block128, native = form.startswith("fp8"), form == "fp8_block128", form.endswith("_gfx950")
+    x, matrices, picks, got, hidden_codes = run_wide_form(amd, workloads, form, rows)
+    if native:
+        # gfx950's lay-out of the same matrices: every byte the launches write is the reference lay-out's (the same sums)
+        _, _, want_picks, want, want_codes = run_wide_form(amd, workloads, form[:3], rows)
+        assert want_picks.tobytes() == picks.tobytes()
+        assert got.tobytes() == want.tobytes(), "the row outputs differ from the reference lay-out's"
+        assert hidden_codes.tobytes() == want_codes.tobytes(), "the hidden codes differ from the reference lay-out's"
     sample = np.array([0, 1, 2, rows // 2, rows - 3, rows - 2, rows - 1])
     experts = np.ascontiguousarray(picks["expert"][sample])
     weights = np.ascontiguousarray(picks["route_weight"][sample])
-    pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])
+    pointers = (C.c_void_p * (EXPERTS * 3))(*[m.ctypes.data for trio in matrices for m in trio])  # the reference's bytes: the re-lay-out's source
     want = np.zeros((len(sample), HIDDEN), dtype=np.float32)
     o.orc.orc_linear_moe_layer(6 if block128 else 5 if fp8 else 3, o.ptr(np.ascontiguousarray(x[sample]), o.u16p), len(sample), HIDDEN, INNER, PICKS,
                                o.ptr(experts, o.u32p), o.ptr(weights, o.f32p), EXPERTS, pointers, 10.0, o.ptr(want, o.f32p), None, None, 16)
