@@ -48,6 +48,11 @@ __device__ static __forceinline__ void load_1(uint32_t &into, const unsigned cha
     asm volatile("global_load_ubyte %0, %1, %2" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
 }
 
+__device__ static __forceinline__ void load_4(uint32_t &into, const unsigned char *base, uint32_t lane_offset)
+{
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(into) : "v"(lane_offset), "s"(base) : "memory");
+}
+
 /* behind wait_loads: the value the load left in the register is this statement's result, so that nothing that uses it
  * can be placed ahead of the wait */
 __device__ static __forceinline__ void native_landed(uint4_t &value)
@@ -74,18 +79,23 @@ struct native_chain {
     static constexpr uint32_t STAGE_BYTES = VECTOR_BYTES + COLUMN_BLOCKS * 64u; /* and their scale words behind them */
     static constexpr uint32_t WINDOW_BYTES = DEPTH * STAGE_BYTES;
     static constexpr uint32_t VECTOR_LOADS = 2u * WAVE_BLOCKS + 1u;
-    static constexpr uint32_t WEIGHT_LOADS = TILES * HALVES + TILES;
+    /* scale codes: of one-byte weights a byte a lane a tile (a row of 32 outputs' codes, as the reference stores them); of
+     * 4-bit weights a word a lane a matrix: its bytes are the codes of the lane's row and inputs in the four tiles of a group
+     * of 64 outputs, which the matrix instruction picks by number */
+    static constexpr uint32_t SCALE_LOADS = BYTES ? TILES : MATRICES;
+    static constexpr uint32_t WEIGHT_LOADS = TILES * HALVES + SCALE_LOADS;
+    static_assert(BYTES || STRIP == 2u || STRIP == 4u, "a strip of 4-bit weights is half a group of four tiles, or a whole one");
     static_assert((DEPTH - 1u) * VECTOR_LOADS + (SLOTS - 1u) * WEIGHT_LOADS < 64u, "vmcnt has six bits");
 
     struct slot {
         uint4_t words[TILES][HALVES];
-        uint32_t scale[TILES];
+        uint32_t scale[SCALE_LOADS];
     };
 
     const unsigned char *words[MATRICES], *scales[MATRICES], *codes, *exponents;
     uint32_t step_stride; /* from a tile's K step to its next */
     uint32_t window, wave, word_offset[STRIP], scale_offset[STRIP], codes_offset[WAVE_BLOCKS][2], exponents_offset;
-    uint32_t vector_at[BYTES ? 8 : 4], vector_scale_at, operand_at;
+    uint32_t vector_at[BYTES ? 8 : 4], vector_scale_at, operand_at, scale_shift;
     bool scale_lane;
 
     template <typename T>
@@ -132,10 +142,14 @@ struct native_chain {
         }
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
-            const unsigned char *step_scales = scales[m] + (uint64_t)at * (BYTES ? 4u : 64u);
+            const unsigned char *step_scales = scales[m] + (uint64_t)at * (BYTES ? 4u : 256u);
+            if constexpr (BYTES) {
 #pragma unroll
-            for (uint32_t n = 0; n < STRIP; n++) {
-                load_1(into.scale[m * STRIP + n], step_scales, scale_offset[n]);
+                for (uint32_t n = 0; n < STRIP; n++) {
+                    load_1(into.scale[m * STRIP + n], step_scales, scale_offset[n]);
+                }
+            } else {
+                load_4(into.scale[m], step_scales, scale_offset[0]);
             }
         }
     }
@@ -148,7 +162,10 @@ struct native_chain {
             for (uint32_t h = 0; h < HALVES; h++) {
                 native_landed(set.words[t][h]);
             }
-            native_landed(set.scale[t]);
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < SCALE_LOADS; k++) {
+            native_landed(set.scale[k]);
         }
     }
 
@@ -181,6 +198,26 @@ struct native_chain {
         }
     }
 
+    /* tile T and the tiles behind it of the wavefront's strip against column block j (the number of the scale code's byte
+     * is part of the instruction: a constant) */
+    template <uint32_t T>
+    __device__ static __forceinline__ void multiply_tiles(const slot &set, const uint32_t (&scale_a)[SCALE_LOADS], const int8_vector &b,
+                                                          uint32_t scale_b, uint32_t j, float4_t (&chain)[TILES][COLUMN_BLOCKS])
+    {
+        if constexpr (BYTES) {
+            const uint4_t first = set.words[T][0], second = set.words[T][HALVES - 1u];
+            const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
+            chain[T][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[T][j], 0, 0, 0, (int)scale_a[T], 0, (int)scale_b);
+        } else {
+            const uint4_t w = set.words[T][0];
+            const int8_vector a = {(int)w.x, (int)w.y, (int)w.z, (int)w.w, 0, 0, 0, 0};
+            chain[T][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[T][j], 4, 0, T % STRIP, (int)scale_a[T / STRIP], 0, (int)scale_b);
+        }
+        if constexpr (T + 1u < TILES) {
+            multiply_tiles<T + 1u>(set, scale_a, b, scale_b, j, chain);
+        }
+    }
+
     /* one K step of LIVE column blocks from a stage's columns and a set of weight registers */
     template <uint32_t LIVE>
     __device__ __forceinline__ void consume(uint32_t stage, const slot &set, float4_t (&chain)[TILES][COLUMN_BLOCKS]) const
@@ -189,6 +226,11 @@ struct native_chain {
         asm volatile("" : "+s"(base));
         uint32_t b_at = base + operand_at, b_scale_at = base + VECTOR_BYTES + vector_scale_at;
         asm volatile("" : "+v"(b_at), "+v"(b_scale_at));
+        uint32_t scale_a[SCALE_LOADS];
+#pragma unroll
+        for (uint32_t k = 0; k < SCALE_LOADS; k++) { /* 4-bit weights, two tiles a strip: the group's upper two tiles' codes down */
+            scale_a[k] = BYTES ? set.scale[k] : set.scale[k] >> scale_shift;
+        }
         __builtin_amdgcn_s_setprio(1);
         /* a column block's operand is read while the block before it is multiplied: two blocks' registers, not LIVE */
         uint4_t low = lds_read<uint4_t>(b_at), high = lds_read<uint4_t>(b_at + 1024u);
@@ -203,18 +245,7 @@ struct native_chain {
                 high = lds_read<uint4_t>(b_at + (j + 1u) * 2048u + 1024u);
                 scale_b = lds_read<unsigned char>(b_scale_at + (j + 1u) * 64u);
             }
-#pragma unroll
-            for (uint32_t t = 0; t < TILES; t++) {
-                if constexpr (BYTES) {
-                    const uint4_t first = set.words[t][0], second = set.words[t][HALVES - 1u];
-                    const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
-                    chain[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[t][j], 0, 0, 0, (int)set.scale[t], 0, (int)scale_now);
-                } else {
-                    const uint4_t w = set.words[t][0];
-                    const int8_vector a = {(int)w.x, (int)w.y, (int)w.z, (int)w.w, 0, 0, 0, 0};
-                    chain[t][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[t][j], 4, 0, 0, (int)set.scale[t], 0, (int)scale_now);
-                }
-            }
+            multiply_tiles<0>(set, scale_a, b, scale_now, j, chain);
         }
         __builtin_amdgcn_s_setprio(0);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stage is read before the next barrier */
@@ -374,14 +405,14 @@ struct native_chain {
             words[m] = matrices[m] + (uint64_t)tile0 * tile_bytes;
             if constexpr (BYTES) { /* the scale codes as the reference stores them: a row of inputs / 32 bytes for every 32 outputs */
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs + (uint64_t)(tile0 / 2u) * (inputs / 32u);
-            } else { /* a byte a lane a tile's K step */
-                scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + (uint64_t)tile0 * steps * 64u;
+            } else { /* a word a lane a K step of a group of four tiles */
+                scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + (uint64_t)(tile0 / 4u) * steps * 256u;
             }
         }
 #pragma unroll
         for (uint32_t n = 0; n < STRIP; n++) {
             word_offset[n] = n * tile_bytes + 16u * lane;
-            scale_offset[n] = BYTES ? ((tile0 + n) / 2u - tile0 / 2u) * (inputs / 32u) + g : n * steps * 64u + lane;
+            scale_offset[n] = BYTES ? ((tile0 + n) / 2u - tile0 / 2u) * (inputs / 32u) + g : 4u * lane;
         }
 #pragma unroll
         for (uint32_t i = 0; i < WAVE_BLOCKS; i++) {
@@ -407,6 +438,7 @@ struct native_chain {
         }
         vector_scale_at = 4u * o + g;
         operand_at = 16u * lane;
+        scale_shift = 8u * (tile0 % 4u);
     }
 };
 

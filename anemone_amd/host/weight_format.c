@@ -62,7 +62,7 @@ static result_status exl3_bytes(const struct matrix_shape_record *shape, uint64_
 /* the GFX950 formats hold what their _SCALED counterparts hold, in whole K steps of 128 inputs */
 static result_status e2m1_gfx950_bytes(const struct matrix_shape_record *shape, uint64_t *out)
 {
-    if (shape == NULL || shape->input_size % 128u != 0) {
+    if (shape == NULL || shape->input_size % 128u != 0 || shape->output_size % 64u != 0) {
         return STATUS_INVALID_ARGUMENT;
     }
     return e2m1_bytes(shape, out);
@@ -116,6 +116,13 @@ static uint32_t word_at(const unsigned char *bytes, uint64_t word)
     return value;
 }
 
+/* where E2M1_GFX950 holds the scale code of a lane of a tile's K step: the tiles in groups of four (64 outputs), a group's
+ * K step 64 lanes x 4 bytes, byte tile % 4 */
+static uint64_t e2m1_gfx950_scale_at(uint32_t tile, uint32_t step, uint32_t steps, uint32_t lane)
+{
+    return (((uint64_t)(tile / 4u) * steps + step) * 64u + lane) * 4u + tile % 4u;
+}
+
 /* E2M1: a K step's lane 16 g + o takes, for each of its four words T, the words `2 (g % 2)` and `2 (g % 2) + 1` of the
  * reference's lane 4 (o % 8) + T of load 2 step + g / 2: its output's nibbles of the first below those of the second */
 static void e2m1_to_gfx950(uint32_t outputs, uint32_t inputs, const unsigned char *from, unsigned char *to)
@@ -135,7 +142,7 @@ static void e2m1_to_gfx950(uint32_t outputs, uint32_t inputs, const unsigned cha
                     const uint32_t word = low | (high << 4);
                     memcpy(to + ((((uint64_t)tile * steps + step) * 64u + lane) * 4u + T) * 4u, &word, sizeof word);
                 }
-                to_scales[((uint64_t)tile * steps + step) * 64u + lane] = from_scales[(load * 8u + o % 8u) * 4u + 2u * (g % 2u) + o / 8u];
+                to_scales[e2m1_gfx950_scale_at(tile, step, steps, lane)] = from_scales[(load * 8u + o % 8u) * 4u + 2u * (g % 2u) + o / 8u];
             }
         }
     }
@@ -164,7 +171,7 @@ static void e2m1_from_gfx950(uint32_t outputs, uint32_t inputs, const unsigned c
                     to[word * 4u + bit / 8u] |= (unsigned char)(code << (bit % 8u));
                 }
                 const uint64_t load = (uint64_t)tile * loads + 2u * step + g / 2u;
-                to_scales[(load * 8u + o % 8u) * 4u + 2u * (g % 2u) + o / 8u] = from_scales[((uint64_t)tile * steps + step) * 64u + lane];
+                to_scales[(load * 8u + o % 8u) * 4u + 2u * (g % 2u) + o / 8u] = from_scales[e2m1_gfx950_scale_at(tile, step, steps, lane)];
             }
         }
     }

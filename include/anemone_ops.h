@@ -48,12 +48,14 @@ const struct weight_format_operations *weight_format_operations_of(enum weight_f
 extern const struct weight_format_operations exl3_weight_operations;
 
 /* Load-time re-lay-out between the reference's lane order and gfx950's (host only: bytes move, no weight or scale code
- * changes; no allocation). A matrix [outputs][inputs], outputs a multiple of 16 (32 for E4M3), inputs of 128, is tiles of
+ * changes; no allocation). A matrix [outputs][inputs], outputs a multiple of 64 (32 for E4M3), inputs of 128, is tiles of
  * 16 outputs by K steps of 128 inputs. In a GFX950 format the tiles follow each other, a tile's K steps follow each
  * other, and a K step is the 64 lanes' A operand of v_mfma_scale_f32_16x16x128_f8f6f4, lane 16 g + o holding output o:
  *   E2M1_GFX950  16 bytes a lane: nibble n (0: low) of byte b of word T is input 32 g + 16 n + 2 T + {0, 8, 1, 9}[b] of
- *                the step; behind all tiles the scale codes, one byte a lane a K step a tile ([tile][step][lane]): the
- *                E8M0 code of output o, inputs 32 g .. 32 g + 31. Bytes: outputs inputs / 2 + outputs inputs / 32.
+ *                the step; behind all tiles the scale codes, the tiles in groups of four (outputs a multiple of 64): a
+ *                group's K step is a word a lane ([group][step][lane][4]), byte n the E8M0 code of output o of the
+ *                group's tile n, inputs 32 g .. 32 g + 31: a wavefront's strip of two or four tiles takes its codes with
+ *                one load and the matrix instruction picks the byte. Bytes: outputs inputs / 2 + outputs inputs / 32.
  *   E4M3_GFX950  32 bytes a lane as two halves of 1,024 bytes a step ([half][lane][16]): byte c of word v (0 .. 7; half
  *                v / 4) is input 64 (v / 4) + 16 g + 8 (c % 2) + 2 (v % 4) + c / 2; behind all tiles the scale codes as
  *                E4M3_SCALED stores them (a row of inputs / 32 for every 32 outputs). Bytes: E4M3_SCALED's.

@@ -25,7 +25,7 @@ static int shape_is_stored(int format, uint32_t outputs, uint32_t inputs)
         return 0;
     }
     if (format == ORC_FORMAT_E2M1_GFX950) {
-        return inputs % 128u == 0u;
+        return inputs % 128u == 0u && outputs % 64u == 0u;
     }
     if (format == ORC_FORMAT_E4M3_GFX950) {
         return inputs % 128u == 0u && outputs % 32u == 0u;
@@ -109,10 +109,12 @@ int orc_linear_lay_out(int format, uint32_t outputs, uint32_t inputs, const uint
             memcpy(stored + at, scale_codes, orc_linear_scale_count(format, outputs, inputs));
             return 0;
         }
-        for (uint32_t tile = 0; tile < tiles; tile++) {
+        for (uint32_t group = 0; group < tiles / 4u; group++) { /* a word a lane a K step of a group of four tiles */
             for (uint32_t step = 0; step < steps; step++) {
-                for (uint32_t lane = 0; lane < 64u; lane++, at++) {
-                    stored[at] = scale_codes[(uint64_t)(16u * tile + lane % 16u) * (inputs / BLOCK) + 4u * step + lane / 16u];
+                for (uint32_t lane = 0; lane < 64u; lane++) {
+                    for (uint32_t n = 0; n < 4u; n++, at++) {
+                        stored[at] = scale_codes[(uint64_t)(16u * (4u * group + n) + lane % 16u) * (inputs / BLOCK) + 4u * step + lane / 16u];
+                    }
                 }
             }
         }
@@ -189,7 +191,7 @@ int orc_linear_read(int format, uint32_t outputs, uint32_t inputs, const uint8_t
         const uint32_t steps = inputs / 128u, step = input / 128u, G = (input % 128u) / 32u, n = (input % 32u) / 16u, r = input % 16u;
         const uint32_t T = (r % 8u) / 2u, b = 2u * (r % 2u) + r / 8u, lane = 16u * G + in_tile;
         *code_out = (stored[(((uint64_t)tile * steps + step) * 64u + lane) * 16u + 4u * T + b] >> (4u * n)) & 15u;
-        *scale_out = stored[(uint64_t)outputs * inputs / 2u + ((uint64_t)tile * steps + step) * 64u + lane];
+        *scale_out = stored[(uint64_t)outputs * inputs / 2u + ((((uint64_t)(tile / 4u) * steps + step) * 64u + lane) * 4u + tile % 4u)];
         return 0;
     }
     if (format == ORC_FORMAT_E4M3_GFX950) {

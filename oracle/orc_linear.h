@@ -36,10 +36,11 @@
  * instruction. A matrix is tiles of 16 outputs by K steps of 128 inputs, tile after tile, step after step; a step is 64
  * lanes, lane 16 g + o holding output o of the tile.
  *   E2M1_GFX950: 16 bytes a lane; nibble n (0: low) of byte b of word T is input 32 g + 16 n + 2 T + {0, 8, 1, 9}[b] of
- *     the step; behind all tiles one scale byte a lane a step a tile: the E8M0 code of output o, inputs 32 g .. + 31.
+ *     the step; behind all tiles the scale codes, the tiles in groups of four: a word a lane a step a group, byte n the
+ *     E8M0 code of output o of the group's tile n, inputs 32 g .. + 31.
  *   E4M3_GFX950: 32 bytes a lane, as two halves [half][lane][16]; byte c of word v (half v / 4) is input
  *     64 (v / 4) + 16 g + 8 (c % 2) + 2 (v % 4) + c / 2; the scale codes as E4M3_SCALED's.
- * Inputs a multiple of 128; outputs of 16 (E2M1) or 32 (E4M3). */
+ * Inputs a multiple of 128; outputs of 64 (E2M1) or 32 (E4M3). */
 #define ORC_FORMAT_E2M1_GFX950 7
 #define ORC_FORMAT_E4M3_GFX950 8
 
