@@ -141,7 +141,9 @@ class LinearKernels(C.Structure):
                 ("trunk_linear_quantized", u32 * 5), ("trunk_linear_bfloat16", u32 * 5), ("trunk_hidden", u32),
                 ("trunk_linear_quantized_wide", u32 * 5), ("trunk_linear_bfloat16_wide", u32 * 5),
                 ("trunk_linear_quantized_interleaved", u32), ("expert_gate_up_e4m3", u32 * 5), ("expert_down_e4m3", u32 * 5),
-                ("expert_gate_up_b128", u32 * 5), ("expert_down_b128", u32 * 5), ("activation_quantize_128", u32)]
+                ("expert_gate_up_b128", u32 * 5), ("expert_down_b128", u32 * 5), ("activation_quantize_128", u32),
+                ("expert_gate_up_gfx950", u32 * 5), ("expert_down_gfx950", u32 * 5), ("expert_gate_up_e4m3_gfx950", u32 * 5),
+                ("expert_down_e4m3_gfx950", u32 * 5)]
 
 
 class ExpertFusedKernels(C.Structure):

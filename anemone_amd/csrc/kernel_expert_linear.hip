@@ -40,11 +40,11 @@
 
 
 /* gate and up: block = S wavefronts (slices of the inputs); grid (ceil(output_size / 64), jobs) */
-template <uint32_t S, bool BYTES, bool B128 = false>
+template <uint32_t S, bool BYTES, bool B128 = false, bool NATIVE = false>
 __device__ static __forceinline__ void expert_gate_up(const struct expert_gate_up_arguments &arguments,
                                                       unsigned char *arena, uint16_t *strip_hidden = nullptr)
 {
-    typedef strip_chain<2, BYTES, B128> chain_type;
+    typedef strip_chain<2, BYTES, B128, NATIVE> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP;
     __shared__ __attribute__((aligned(16))) unsigned char window[S][chain_type::WINDOW_BYTES];
     static_assert(chain_type::WINDOW_BYTES >= TILES * WAVE * 16u, "a wavefront's sums fit its idle window");
@@ -194,10 +194,10 @@ __device__ static __forceinline__ void expert_gate_up_quantize(const struct expe
 }
 
 /* down: block = S wavefronts; grid (ceil(output_size / 64), jobs) */
-template <uint32_t S, bool BYTES, bool B128 = false>
+template <uint32_t S, bool BYTES, bool B128 = false, bool NATIVE = false>
 __device__ static __forceinline__ void expert_down(const struct expert_down_arguments &arguments, unsigned char *arena)
 {
-    typedef strip_chain<1, BYTES, B128> chain_type;
+    typedef strip_chain<1, BYTES, B128, NATIVE> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP;
     __shared__ __attribute__((aligned(16))) unsigned char window[S][chain_type::WINDOW_BYTES];
     static_assert(chain_type::WINDOW_BYTES >= TILES * WAVE * 16u, "a wavefront's sums fit its idle window");
@@ -256,7 +256,9 @@ __device__ static __forceinline__ void expert_down(const struct expert_down_argu
  * entries take WEIGHT_FORMAT_E4M3_SCALED experts (a format the reference stores and lays out but multiplies in its
  * trunk alone: no counterpart among its expert kernels); same records, same rounding points. The _b128_ entries take
  * WEIGHT_FORMAT_E4M3_BLOCK128 experts (E4M3 codes with one float32 scale for every 128 x 128 block, vectors quantized a
- * 128 values with float32 scales, read where the records name the exponents: no counterpart in the reference). */
+ * 128 values with float32 scales, read where the records name the exponents: no counterpart in the reference). The
+ * _gfx950_ entries take experts stored in the card's own lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950: no
+ * counterpart in the reference) and give the sums of the same matrices in the reference's lay-out, bit for bit. */
 #define EXPERT_ENTRIES(S)                                                                                         \
     extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
         expert_gate_up_##S(struct expert_gate_up_arguments arguments, unsigned char *arena)                      \
@@ -305,7 +307,31 @@ __device__ static __forceinline__ void expert_down(const struct expert_down_argu
     {                                                                                                             \
         expert_down<S, true, true>(arguments, arena);                                                             \
     }                                                                                                             \
-    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_b128_##S, expert_down_arguments)
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_b128_##S, expert_down_arguments);                       \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_gate_up_gfx950_##S(struct expert_gate_up_arguments arguments, unsigned char *arena)               \
+    {                                                                                                             \
+        expert_gate_up<S, false, false, true>(arguments, arena);                                                  \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_gate_up_gfx950_##S, expert_gate_up_arguments);               \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_down_gfx950_##S(struct expert_down_arguments arguments, unsigned char *arena)                     \
+    {                                                                                                             \
+        expert_down<S, false, false, true>(arguments, arena);                                                     \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_gfx950_##S, expert_down_arguments);                     \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_gate_up_e4m3_gfx950_##S(struct expert_gate_up_arguments arguments, unsigned char *arena)          \
+    {                                                                                                             \
+        expert_gate_up<S, true, false, true>(arguments, arena);                                                   \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_gate_up_e4m3_gfx950_##S, expert_gate_up_arguments);          \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_down_e4m3_gfx950_##S(struct expert_down_arguments arguments, unsigned char *arena)                \
+    {                                                                                                             \
+        expert_down<S, true, false, true>(arguments, arena);                                                      \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_e4m3_gfx950_##S, expert_down_arguments)
 EXPERT_ENTRIES(1);
 EXPERT_ENTRIES(2);
 EXPERT_ENTRIES(4);

@@ -17,9 +17,14 @@
 /* B128 (one-byte weights alone): the scales are float32, one for every 128 outputs x 128 inputs of a matrix and one for
  * every 128 values of a vector, in place of the E8M0 codes; a K step's MFMA then runs from zero with scales of one and its
  * sums enter the chain by one fused multiply-add with the product of the two scales. */
-template <uint32_t MATRICES, bool BYTES, bool B128 = false>
+/* NATIVE: the matrices are stored in gfx950's lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950): a lane's 16 bytes of
+ * a tile's K step (and, of one-byte weights, the 16 bytes 1,024 further) are its A operand as they lie, so a stage's
+ * tiles are read with one or two 16-byte LDS reads and no arithmetic; the scale codes of 4-bit weights are a word a lane
+ * for the strip's four tiles (a group of 64 outputs), its byte picked by the matrix instruction. */
+template <uint32_t MATRICES, bool BYTES, bool B128 = false, bool NATIVE = false>
 struct strip_chain {
     static_assert(BYTES || !B128, "float32 scales go with one-byte weights");
+    static_assert(!NATIVE || !B128, "gfx950's lane order is built for the formats of E8M0 scale codes");
     static constexpr uint32_t STRIP = BYTES ? 2u : 4u; /* tiles of a strip: 4 KB of every matrix a stage either way */
     static constexpr uint32_t STEP_BYTES = BYTES ? BYTE_STEP_BYTES : NIBBLE_STEP_BYTES;
     static constexpr uint32_t TILE_LOADS = STEP_BYTES / 1024u; /* 16-byte-a-lane loads of a tile's step */
@@ -66,7 +71,7 @@ struct strip_chain {
         }
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
-            load_to_lds_4(scales[m] + (uint64_t)at * (BYTES ? 4u : 64u), scale_offset, base + SCALES_AT + m * 256u);
+            load_to_lds_4(scales[m] + (uint64_t)at * (BYTES ? 4u : NATIVE ? 256u : 64u), scale_offset, base + SCALES_AT + m * 256u);
         }
         load_to_lds_16(codes + (uint64_t)at * 128u, codes_offset, base + VECTOR_AT);
         load_to_lds_4(exponents + (uint64_t)at * 4u, exponents_offset, base + VECTOR_SCALE_AT);
@@ -76,6 +81,27 @@ struct strip_chain {
     __device__ static __forceinline__ T lds_read(uint32_t address)
     {
         return *(const __attribute__((address_space(3))) T *)(uintptr_t)address;
+    }
+
+    /* tile T of a stage and the tiles behind it, stored in gfx950's lane order (the number of the scale code's byte in
+     * its word is part of the instruction: a constant) */
+    template <uint32_t T>
+    __device__ __forceinline__ void native_tiles(uint32_t base, const int8_vector &b, uint32_t scale_b, float4_t (&chain)[TILES]) const
+    {
+        const uint4_t first = lds_read<uint4_t>(base + T * STEP_BYTES + piece_offset);
+        if constexpr (BYTES) {
+            const uint4_t second = lds_read<uint4_t>(base + T * STEP_BYTES + 1024u + piece_offset);
+            const uint32_t scale_a = lds_read<unsigned char>(base + SCALES_AT + (T / STRIP) * 256u + scale_at[T % STRIP]);
+            const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
+            chain[T] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[T], 0, 0, 0, (int)scale_a, 0, (int)scale_b);
+        } else {
+            const uint32_t scale_a = lds_read<uint32_t>(base + SCALES_AT + (T / STRIP) * 256u + scale_offset);
+            const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, 0, 0, 0, 0};
+            chain[T] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[T], 4, 0, T % STRIP, (int)scale_a, 0, (int)scale_b);
+        }
+        if constexpr (T + 1u < TILES) {
+            native_tiles<T + 1u>(base, b, scale_b, chain);
+        }
     }
 
     __device__ __forceinline__ void consume(uint32_t stage, float4_t (&chain)[TILES]) const
@@ -101,6 +127,11 @@ struct strip_chain {
             float_scale_b = lds_read<float>(base + VECTOR_SCALE_AT + vector_scale_at);
         } else {
             scale_b = lds_read<unsigned char>(base + VECTOR_SCALE_AT + vector_scale_at);
+        }
+        if constexpr (NATIVE) {
+            native_tiles<0>(base, b, scale_b, chain);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            return;
         }
 #pragma unroll
         for (uint32_t tile = 0; tile < TILES; tile++) {
@@ -223,7 +254,7 @@ struct strip_chain {
             }
             /* lane L of a load lands at slot L and asks for the piece L ^ (bits 3, 4 of L, as a number): the pieces
              * (group, G, t) of one t then lie in different banks for the readers */
-            piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
+            piece_offset = NATIVE ? 16u * lane : 16u * (lane ^ ((lane >> 3) & 3u)); /* gfx950's order: as stored */
             /* the strip's tiles lie in one or two rows of scales (32 outputs a row): lanes past them ask for the last again,
              * so that a load touches two cache lines and not one a lane */
             const uint32_t rows_needed = (tile0 + STRIP - 1u) / 2u - row0;
@@ -249,23 +280,36 @@ struct strip_chain {
                 words[m] = matrices[m] + ((uint64_t)tile0 * steps + first) * STEP_BYTES;
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + ((uint64_t)tile0 * loads + 2u * first) * 32u;
             }
-            /* lane L of a 16-byte load lands at bytes 16 L of the tile's stage and asks for the piece
-             * p = L ^ ((L / 8) % 4) of the step: LDS has 32 banks of 4 bytes, and the pieces of one T (p = 32 ld + 4 G + T,
-             * G = 0 .. 7) then lie in eight different groups of four banks for the sixteen lanes that read them together
-             * (measured: SQ_LDS_BANK_CONFLICT of the wide gate/up launch 1.68e8 -> 1.9e7 cycles); every 16 lanes still read
-             * 256 contiguous bytes of memory */
-            piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
-            /* scales: uint32 [tile][load][G]; lane L of the 4-byte load: tile L / 16, word L % 16 = 8 ld + G */
-            scale_offset = (lane / 16u) * (loads * 32u) + (lane % 16u) * 4u;
+            if constexpr (NATIVE) {
+                /* WEIGHT_FORMAT_E2M1_GFX950: words [tile][K step][lane][16 bytes]; scale codes uint32
+                 * [group of four tiles][K step][lane], byte n of a word the code of tile n of the group. The format holds
+                 * whole groups (outputs a multiple of 64), so a strip is one. */
 #pragma unroll
-            for (uint32_t T = 0; T < 4u; T++) {
-                read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (G / 2u))) + 8u * q;
-            }
+                for (uint32_t m = 0; m < MATRICES; m++) {
+                    scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + ((uint64_t)(tile0 / 4u) * steps + first) * 256u;
+                }
+                piece_offset = 16u * lane;
+                scale_offset = 4u * lane;
+                shift = 0;
+            } else {
+                /* lane L of a 16-byte load lands at bytes 16 L of the tile's stage and asks for the piece
+                 * p = L ^ ((L / 8) % 4) of the step: LDS has 32 banks of 4 bytes, and the pieces of one T (p = 32 ld + 4 G + T,
+                 * G = 0 .. 7) then lie in eight different groups of four banks for the sixteen lanes that read them together
+                 * (measured: SQ_LDS_BANK_CONFLICT of the wide gate/up launch 1.68e8 -> 1.9e7 cycles); every 16 lanes still read
+                 * 256 contiguous bytes of memory */
+                piece_offset = 16u * (lane ^ ((lane >> 3) & 3u));
+                /* scales: uint32 [tile][load][G]; lane L of the 4-byte load: tile L / 16, word L % 16 = 8 ld + G */
+                scale_offset = (lane / 16u) * (loads * 32u) + (lane % 16u) * 4u;
 #pragma unroll
-            for (uint32_t n = 0; n < STRIP; n++) {
-                scale_at[n] = n * 64u + (8u * ld + G) * 4u + 2u * q + parity;
+                for (uint32_t T = 0; T < 4u; T++) {
+                    read_at[T] = 16u * (32u * ld + 4u * G + (T ^ (G / 2u))) + 8u * q;
+                }
+#pragma unroll
+                for (uint32_t n = 0; n < STRIP; n++) {
+                    scale_at[n] = n * 64u + (8u * ld + G) * 4u + 2u * q + parity;
+                }
+                shift = 4u * parity;
             }
-            shift = 4u * parity;
         }
         /* the vectors: lane L of the 16-byte load holds slot L % 8 of column L / 8 and asks for that column's piece
          * (L % 8) ^ (L / 8) of the step, so that one piece of all columns lies in different banks; lane L of the

@@ -107,6 +107,11 @@ result_status expert_producer_prepare(const struct linear_routed_experts_descrip
         return STATUS_INVALID_ARGUMENT;
     }
     const bool bytes = description->weight_format == WEIGHT_FORMAT_E4M3_SCALED;
+    if (!bytes && description->weight_format != WEIGHT_FORMAT_E2M1_SCALED) {
+        REFUSE("%s: experts of format %u: the producer is built for formats %u and %u (the others take the launches it stands for)", what,
+               (uint32_t)description->weight_format, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, (uint32_t)WEIGHT_FORMAT_E4M3_SCALED);
+        return STATUS_INVALID_ARGUMENT;
+    }
     uint32_t instance = 0;
     while (instance < BUILT_INSTANCES && slice_counts[instance] != description->gate_up_slice_count) {
         instance++;

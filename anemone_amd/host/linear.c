@@ -90,6 +90,23 @@ result_status linear_kernels_prepare(const struct backend_operations *backend, s
                                              &kernels.expert_down_b128[instance]);
         }
     }
+    for (uint32_t instance = 0; status == STATUS_OK && instance < BUILT_INSTANCES; instance++) {
+        /* the same four families of the formats in gfx950's lane order */
+        const struct {
+            const char *stem, *infix;
+            uint32_t record_bytes, *handle;
+        } native[] = {
+            {KERNEL_EXPERT_GATE_UP_STEM, "gfx950_", sizeof(struct expert_gate_up_arguments), &kernels.expert_gate_up_gfx950[instance]},
+            {KERNEL_EXPERT_DOWN_STEM, "gfx950_", sizeof(struct expert_down_arguments), &kernels.expert_down_gfx950[instance]},
+            {KERNEL_EXPERT_GATE_UP_STEM, "e4m3_gfx950_", sizeof(struct expert_gate_up_arguments), &kernels.expert_gate_up_e4m3_gfx950[instance]},
+            {KERNEL_EXPERT_DOWN_STEM, "e4m3_gfx950_", sizeof(struct expert_down_arguments), &kernels.expert_down_e4m3_gfx950[instance]},
+        };
+        for (uint32_t k = 0; status == STATUS_OK && k < sizeof native / sizeof native[0]; k++) {
+            char name[56];
+            (void)snprintf(name, sizeof name, "%s%s%u", native[k].stem, native[k].infix, slice_counts[instance]);
+            status = backend->kernel_prepare(card, KERNEL_FILE_EXPERT_LINEAR, name, native[k].record_bytes, native[k].handle);
+        }
+    }
     if (status == STATUS_OK) {
         status = backend->kernel_prepare(card, KERNEL_FILE_ACTIVATION_QUANTIZE, KERNEL_ACTIVATION_QUANTIZE_128,
                                          sizeof(struct activation_quantize_arguments), &kernels.activation_quantize_128);
@@ -231,16 +248,18 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     uint64_t gate_up_bytes = 0, down_bytes = 0;
     uint32_t gate_up_instance = 0, down_instance = 0;
     const bool block128 = description->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128;
-    const bool bytes = description->weight_format == WEIGHT_FORMAT_E4M3_SCALED || block128;
+    const bool native = description->weight_format == WEIGHT_FORMAT_E2M1_GFX950 || description->weight_format == WEIGHT_FORMAT_E4M3_GFX950;
+    const bool bytes = description->weight_format == WEIGHT_FORMAT_E4M3_SCALED || description->weight_format == WEIGHT_FORMAT_E4M3_GFX950 || block128;
+    const bool nibbles = description->weight_format == WEIGHT_FORMAT_E2M1_SCALED || description->weight_format == WEIGHT_FORMAT_E2M1_GFX950;
     const uint32_t strip_outputs = bytes ? LINEAR_STRIP_OUTPUTS / 2u : LINEAR_STRIP_OUTPUTS;
-    if (description->reserved_zero != 0 || (description->weight_format != WEIGHT_FORMAT_E2M1_SCALED && !bytes) || format == NULL ||
+    if (description->reserved_zero != 0 || (!nibbles && !bytes) || format == NULL ||
         format->stored_byte_count(gate_up, &gate_up_bytes) != STATUS_OK ||
         format->stored_byte_count(down, &down_bytes) != STATUS_OK || gate_up->input_size % 128u != 0 ||
         down->input_size % 128u != 0 || down->input_size != gate_up->output_size ||
         gate_up->output_size < strip_outputs || down->output_size < strip_outputs) {
-        REFUSE("%s: matrices of format %u or %u in shapes it stores, inputs a multiple of 128, at least %u outputs, down "
+        REFUSE("%s: matrices of format %u, %u, %u, %u or %u in shapes it stores, inputs a multiple of 128, at least %u outputs, down "
                "reading what gate and up write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, (uint32_t)WEIGHT_FORMAT_E4M3_SCALED,
-               strip_outputs);
+               (uint32_t)WEIGHT_FORMAT_E4M3_BLOCK128, (uint32_t)WEIGHT_FORMAT_E2M1_GFX950, (uint32_t)WEIGHT_FORMAT_E4M3_GFX950, strip_outputs);
         return STATUS_INVALID_ARGUMENT;
     }
     if (!instance_of(description->gate_up_slice_count, gate_up->input_size, &gate_up_instance) ||
@@ -249,12 +268,17 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
                description->gate_up_slice_count, description->down_slice_count);
         return STATUS_INVALID_ARGUMENT;
     }
-    const uint32_t gate_up_kernel = block128 ? kernels->expert_gate_up_b128[gate_up_instance]
-                                    : bytes  ? kernels->expert_gate_up_e4m3[gate_up_instance]
-                                             : kernels->expert_gate_up[gate_up_instance];
-    const uint32_t down_kernel = block128 ? kernels->expert_down_b128[down_instance]
-                                 : bytes  ? kernels->expert_down_e4m3[down_instance]
-                                          : kernels->expert_down[down_instance];
+    const uint32_t *const gate_up_family = block128          ? kernels->expert_gate_up_b128
+                                           : native && bytes ? kernels->expert_gate_up_e4m3_gfx950
+                                           : native          ? kernels->expert_gate_up_gfx950
+                                           : bytes           ? kernels->expert_gate_up_e4m3
+                                                             : kernels->expert_gate_up;
+    const uint32_t *const down_family = block128          ? kernels->expert_down_b128
+                                        : native && bytes ? kernels->expert_down_e4m3_gfx950
+                                        : native          ? kernels->expert_down_gfx950
+                                        : bytes           ? kernels->expert_down_e4m3
+                                                          : kernels->expert_down;
+    const uint32_t gate_up_kernel = gate_up_family[gate_up_instance], down_kernel = down_family[down_instance];
     const uint32_t quantize_kernel = block128 ? kernels->activation_quantize_128 : kernels->activation_quantize;
     const uint32_t quantize_block_values = block128 ? QUANTIZE_128_BLOCK_VALUES : QUANTIZE_BLOCK_VALUES;
     if (gate_up_kernel == BACKEND_NO_KERNEL || down_kernel == BACKEND_NO_KERNEL ||

@@ -139,8 +139,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
     block128 = fp8 and arguments.block128  # float32 scales of 128 x 128 blocks and of 128 values (the usual FP8 block scaling)
     native = getattr(arguments, "native", False)  # the weights in gfx950's own lane order (a load-time re-lay-out of the same bytes)
-    if native and (block128 or not prefill):
-        raise SystemExit("--native: the wide (prefill) launches of the reference's scalings take it")
+    if native and block128:
+        raise SystemExit("--native: the formats of the reference's scalings (E8M0 codes) have a gfx950 lane order")
     matrix = workloads.fp8_block128_matrix if block128 else workloads.fp8_matrix if fp8 else workloads.fp4_matrix
     trios = [[matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
               matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
@@ -246,7 +246,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
                    "distinct_experts": int(len(distinct)), "jobs": int(len(live)),
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "down_GBps": matrix_bytes * len(distinct) / (down_us * 1e-6) / 1e9},
-        "roofline": {"bound": "hbm", "kernel": "expert_gate_up_%s%d" % ("b128_" if block128 else "e4m3_" if fp8 else "", arguments.gate_up_slices),
+        "roofline": {"bound": "hbm", "kernel": "expert_gate_up_%s%s%d" % ("b128_" if block128 else "e4m3_" if fp8 else "", "gfx950_" if native else "", arguments.gate_up_slices),
                      "achieved": gate_up_bytes / (gate_up_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": int(gate_up_bytes), "launch_us": gate_up_us},
@@ -726,7 +726,7 @@ def main():
     parser.add_argument("--block128", action="store_true",
                         help="fp8 workloads: float32 scales of 128 x 128 weight blocks and of 128 activation values in place of the reference's E8M0 scales")
     parser.add_argument("--native", action="store_true",
-                        help="fp4_prefill / fp8_prefill: the experts' weights in gfx950's own lane order (WEIGHT_FORMAT_E2M1_GFX950 / _E4M3_GFX950, "
+                        help="fp4 and fp8 workloads: the experts' weights in gfx950's own lane order (WEIGHT_FORMAT_E2M1_GFX950 / _E4M3_GFX950, "
                              "made from the same bytes by the library's load-time re-lay-out)")
     parser.add_argument("--site", action="store_true",
                         help="fp4/fp8 workloads: the whole FFN site: the mix project and mix finish ahead of the router, the shared expert and the join "

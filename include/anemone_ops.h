@@ -370,6 +370,11 @@ struct linear_kernels_record { /* include/anemone/linear.h:121-132 of the refere
     uint32_t expert_gate_up_b128[LINEAR_SLICE_INSTANCES];
     uint32_t expert_down_b128[LINEAR_SLICE_INSTANCES];
     uint32_t activation_quantize_128;
+    /* extension: experts stored in gfx950's lane order, WEIGHT_FORMAT_E2M1_GFX950 and WEIGHT_FORMAT_E4M3_GFX950 */
+    uint32_t expert_gate_up_gfx950[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_down_gfx950[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_gate_up_e4m3_gfx950[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_down_e4m3_gfx950[LINEAR_SLICE_INSTANCES];
 };
 MUST_CHECK result_status linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                 uint32_t arithmetic_class, struct linear_kernels_record *kernels_out);
@@ -416,9 +421,10 @@ enum linear_routed_experts_launch {
     LINEAR_ROUTED_EXPERTS_ROW_SUM = 3,  /* expert_row_sum_entry: pair_output to row_output */
     LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT = 4
 };
-/* launches_out: LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT launches; weight_format E2M1_SCALED, or (extensions) E4M3_SCALED or
- * E4M3_BLOCK128: the latter's exponent ranges hold float32 scales of 128 values (the same bytes), its quantizer launch
- * is activation_quantize_128_entry, its shapes are multiples of 128 */
+/* launches_out: LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT launches; weight_format E2M1_SCALED, or (extensions) E4M3_SCALED,
+ * E4M3_BLOCK128 (its exponent ranges hold float32 scales of 128 values (the same bytes), its quantizer launch is
+ * activation_quantize_128_entry, its shapes are multiples of 128), E2M1_GFX950 or E4M3_GFX950 (the outputs of the same
+ * matrices stored as E2M1_SCALED or E4M3_SCALED, bit for bit) */
 MUST_CHECK result_status linear_routed_experts_prepare(const struct linear_routed_experts_description *description,
                                                        uint64_t arena_byte_count,
                                                        const struct linear_kernels_record *kernels,

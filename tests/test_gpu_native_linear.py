@@ -131,3 +131,48 @@ def test_native_layer_against_oracle(amd, card, fmt):
     error = np.sqrt(np.mean((row_output - want) ** 2) / np.mean(want.astype(np.float64) ** 2))
     say("  layer rms error vs oracle: %.2e" % error)
     assert error < 2e-2
+
+
+def run_jobs(card, layer, x, live):
+    layer.set_rows(x, live)
+    card.run(layer.projection_launch())
+    card.run(layer.select_launch(0))
+    card.run(layer.quantize_launch())
+    for name in ("hidden",) + NAMES:
+        card.upload(layer.ranges[name].byte_offset, np.full(layer.ranges[name].byte_count, 0xEE, dtype=np.uint8))
+    card.run(layer.expert_launches())
+    return [layer.read(name).copy() for name in ("hidden",) + NAMES], layer.jobs().copy()
+
+
+@pytest.mark.parametrize("hidden,inner,picks,rows,live,fmt,gate_up_slices,down_slices", [
+    (512, 256, 4, 8, 8, E2M1, 4, 2),     # the slice counts the card's order takes
+    (512, 256, 4, 8, 7, E2M1, 1, 1),     # one chain; a row beyond the live ones
+    (1024, 512, 8, 3, 3, E2M1, 8, 4),
+    (640, 384, 2, 5, 5, E2M1, 2, 1),     # five K steps over two slices: chains of two and three steps
+    (512, 256, 4, 8, 8, E4M3, 4, 2),
+    (640, 384, 8, 2, 2, E4M3, 1, 2),     # 40 tiles of the gate product: strips of two
+    (1024, 512, 1, 8, 5, E4M3, 8, 4),
+])
+def test_native_job_table_kernels_equal_the_reference_lay_out(amd, card, hidden, inner, picks, rows, live, fmt, gate_up_slices, down_slices):
+    """The job-table kernels (a thin step's) of the formats in gfx950's lane order, expert_gate_up_gfx950_<S> and its like:
+    byte for byte what the reference-format kernels of the same slice counts write for the same matrices."""
+    say("native job-table kernels", hidden, inner, picks, rows, live, fmt, gate_up_slices, down_slices)
+    experts_n = 64
+    matrices = matrices_of(hidden, inner, experts_n, 41, fmt, distinct=16)
+    router = to_bf16(normals(43, experts_n * hidden) * 0.02).reshape(experts_n, hidden)
+    x = to_bf16(normals(47, rows * hidden)).reshape(rows, hidden)
+    reference = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router, weight_format=fmt,
+                             gate_up_slices=gate_up_slices, down_slices=down_slices)
+    want, want_jobs = run_jobs(card, reference, x, live)
+    native = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router,
+                          weight_format=E2M1_GFX950 if fmt == E2M1 else E4M3_GFX950, gate_up_slices=gate_up_slices, down_slices=down_slices)
+    got, got_jobs = run_jobs(card, native, x, live)
+    assert np.array_equal(want_jobs["expert"], got_jobs["expert"]) and np.array_equal(want_jobs["pair_index"], got_jobs["pair_index"])
+    pairs = live * picks
+    for name, a, b in zip(("hidden",) + NAMES, want, got):
+        per = a.size // (rows if name == "row_output" else rows * picks)
+        count = (live if name == "row_output" else pairs) * per
+        differing = np.flatnonzero(a.reshape(-1)[:count] != b.reshape(-1)[:count])
+        say("  %s: %d of %d bytes differ" % (name, differing.size, count))
+        assert differing.size == 0, (name, differing[:8], per)
+        assert a.reshape(-1)[:count].tobytes() != bytes([0xEE]) * count, "the launches wrote"
