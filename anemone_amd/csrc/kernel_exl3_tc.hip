@@ -112,20 +112,24 @@ __device__ static __forceinline__ void tc_item(const uint32_t *codes, uint32_t i
 }
 
 /* launches 1 and 3: grid (outputs / EXL3_TC_STRIP_OUTPUTS, job_capacity, matrices * slices / 4), block 256: the block's four
- * wavefronts take four consecutive (matrix, slice) items of one strip. pass 0: gate and up; pass 1: down. A slice is
+ * wavefronts take four consecutive (matrix, slice) items of one strip (a strip of fewer than four items: the items of
+ * adjacent strips, the grid's x that many times smaller and its z 1). pass 0: gate and up; pass 1: down. A slice is
  * a whole number of steps of four K tiles. */
-extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS, 4)
-    exl3_tc_products(struct exl3_tc_record record, unsigned char *arena)
+__device__ static __forceinline__ void tc_products_block(const struct exl3_tc_record &record, unsigned char *arena, uint32_t block_x,
+                                                         uint32_t block_y, uint32_t block_z, uint32_t lane, uint32_t wave)
 {
-    const struct expert_job_record *job = (const struct expert_job_record *)(arena + record.jobs_offset) + blockIdx.y;
+    const struct expert_job_record *job = (const struct expert_job_record *)(arena + record.jobs_offset) + block_y;
     if (job->row_count == 0u) {
         return;
     }
     const tc_shape shape = tc_shape_of(record);
-    const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const bool down = record.pass != 0u;
     const uint32_t slices = down ? EXL3_TC_DOWN_SLICES : EXL3_TC_GATE_UP_SLICES;
-    const uint32_t item = blockIdx.z * PRODUCT_WAVES + wave; /* projection * slices + slice */
+    /* a strip's items: projection * slices + slice; fewer than a block's wavefronts: the block takes adjacent strips */
+    const uint32_t strip_items = (down ? 1u : 2u) * slices;
+    const uint32_t place = block_z * PRODUCT_WAVES + wave;
+    const uint32_t item = strip_items >= PRODUCT_WAVES ? place : place % strip_items;
+    const uint32_t strip = strip_items >= PRODUCT_WAVES ? block_x : block_x * (PRODUCT_WAVES / strip_items) + place / strip_items;
     const uint32_t projection = item / slices, slice = item % slices;
     const uint32_t inputs = down ? shape.intermediate : shape.hidden;
     const uint32_t outputs = down ? shape.hidden : shape.intermediate;
@@ -144,10 +148,10 @@ extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS, 4)
     }
     const uint32_t *codes = (const uint32_t *)(arena + matrix);
     switch (bits_x2) {
-    case 4u: tc_item<4u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
-    case 5u: tc_item<5u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
-    case 6u: tc_item<6u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
-    case 8u: tc_item<8u>(codes, inputs, outputs, blockIdx.x, slice, slices, job, operands, partials, lane); break;
+    case 4u: tc_item<4u>(codes, inputs, outputs, strip, slice, slices, job, operands, partials, lane); break;
+    case 5u: tc_item<5u>(codes, inputs, outputs, strip, slice, slices, job, operands, partials, lane); break;
+    case 6u: tc_item<6u>(codes, inputs, outputs, strip, slice, slices, job, operands, partials, lane); break;
+    case 8u: tc_item<8u>(codes, inputs, outputs, strip, slice, slices, job, operands, partials, lane); break;
     default:
         /* a width this build does not decode (the prepare function refuses the one width of a record; a table's widths
          * are the caller's): zeros, so that the launches behind this one add nothing stale */
@@ -157,12 +161,18 @@ extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS, 4)
             for (uint32_t p = 0; p < STRIP_PAIRS; p++) {
 #pragma unroll
                 for (uint32_t h = 0; h < 2u; h++) {
-                    *(float4_t *)(out + exl3_stream_output(blockIdx.x * 2u * STRIP_PAIRS, p, h, lane)) = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+                    *(float4_t *)(out + exl3_stream_output(strip * 2u * STRIP_PAIRS, p, h, lane)) = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
                 }
             }
         }
         break;
     }
+}
+
+extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS, 4)
+    exl3_tc_products(struct exl3_tc_record record, unsigned char *arena)
+{
+    tc_products_block(record, arena, blockIdx.x, blockIdx.y, blockIdx.z, threadIdx.x % WAVE, __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE));
 }
 ANEMONE_KERNEL(EXL3_TC_KERNEL_FILE, exl3_tc_products, exl3_tc_record);
 

@@ -99,14 +99,25 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
     }
     static const char *const names[EXL3_TC_LAUNCHES] = {"exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate",
                                                         "exl3_tc_products", "exl3_tc_combine"};
-    const uint32_t grid_x[EXL3_TC_LAUNCHES] = {hidden / 128u, I / EXL3_TC_STRIP_OUTPUTS, I / 128u, hidden / EXL3_TC_STRIP_OUTPUTS, hidden / 128u};
+    /* a block's four wavefronts take four items: of one strip (its matrices x slices a multiple of four: z blocks a strip)
+     * or of adjacent strips (a divisor of four: that many strips a block) */
+    enum { GATE_UP_ITEMS = 2u * EXL3_TC_GATE_UP_SLICES, DOWN_ITEMS = EXL3_TC_DOWN_SLICES };
+    _Static_assert((GATE_UP_ITEMS % PRODUCT_WAVES == 0 || PRODUCT_WAVES % GATE_UP_ITEMS == 0) &&
+                   (DOWN_ITEMS % PRODUCT_WAVES == 0 || PRODUCT_WAVES % DOWN_ITEMS == 0), "a block's four wavefronts take four whole items");
+    const uint32_t gate_up_strips = GATE_UP_ITEMS >= PRODUCT_WAVES ? 1u : PRODUCT_WAVES / GATE_UP_ITEMS;
+    const uint32_t down_strips = DOWN_ITEMS >= PRODUCT_WAVES ? 1u : PRODUCT_WAVES / DOWN_ITEMS;
+    if (I % (EXL3_TC_STRIP_OUTPUTS * gate_up_strips) != 0 || hidden % (EXL3_TC_STRIP_OUTPUTS * down_strips) != 0) {
+        REFUSE("%s: sizes that are no whole number of the products' blocks (%u and %u outputs)", what,
+               EXL3_TC_STRIP_OUTPUTS * gate_up_strips, EXL3_TC_STRIP_OUTPUTS * down_strips);
+        return STATUS_INVALID_ARGUMENT;
+    }
+    const uint32_t grid_x[EXL3_TC_LAUNCHES] = {hidden / 128u, I / (EXL3_TC_STRIP_OUTPUTS * gate_up_strips), I / 128u,
+                                               hidden / (EXL3_TC_STRIP_OUTPUTS * down_strips), hidden / 128u};
     const uint32_t grid_y[EXL3_TC_LAUNCHES] = {record->job_capacity, record->job_capacity, record->job_capacity,
                                                record->job_capacity, record->row_count};
-    const uint32_t grid_z[EXL3_TC_LAUNCHES] = {2u, 2u * EXL3_TC_GATE_UP_SLICES / PRODUCT_WAVES, 1u,
-                                               EXL3_TC_DOWN_SLICES / PRODUCT_WAVES, 1u};
+    const uint32_t grid_z[EXL3_TC_LAUNCHES] = {2u, (GATE_UP_ITEMS + PRODUCT_WAVES - 1u) / PRODUCT_WAVES, 1u,
+                                               (DOWN_ITEMS + PRODUCT_WAVES - 1u) / PRODUCT_WAVES, 1u};
     const uint32_t threads[EXL3_TC_LAUNCHES] = {WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS, PRODUCT_THREADS, WAVE_THREADS * ROUTER_MOST_PICKS};
-    _Static_assert(2u * EXL3_TC_GATE_UP_SLICES % PRODUCT_WAVES == 0 && EXL3_TC_DOWN_SLICES % PRODUCT_WAVES == 0,
-                   "a block's four wavefronts take four whole items");
     struct kernel_launch launches[EXL3_TC_LAUNCHES];
     for (uint32_t index = 0; index < EXL3_TC_LAUNCHES; index++) {
         uint32_t kernel = BACKEND_NO_KERNEL;

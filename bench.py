@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 # same counter reads for a 1 GiB copy), for the workloads at the sizes profiled: constants of those runs (the summaries
 # under profiles/ hold the commands and the counts), reported as roofline.traffic when a run has the same sizes
 MEASURED_TRAFFIC_BYTES = {
-    ("exl3_decode", 8): 375.2e6 + 8.4e6,
+    ("exl3_decode", 8): 375.1e6 + 4.2e6,
     ("fp4_decode", 32): 1434.7e6 + 1.0e6,
     ("fp8_decode", 32): 2746.8e6 + 1.0e6,
     ("fp4_prefill", 8192): 4777.9e6 + 447.0e6,
@@ -37,6 +37,10 @@ MEASURED_TRAFFIC_BYTES = {
     ("expert_join", 8192): 877.7e6 + 402.7e6,
     ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,
     ("fp8_prefill_block128", 2048): 5386.8e6 + 67.2e6,
+    ("fp4_prefill_native", 8192): 5870.2e6 + 450.7e6,
+    ("fp8_prefill_native", 2048): 4711.2e6 + 113.3e6,
+    ("fp4_decode_native", 32): 1434.2e6 + 1.0e6,
+    ("fp8_decode_native", 32): 2746.7e6 + 1.0e6,
 }
 TRAFFIC_SOURCE = {
     "exl3_decode": "profiles/exl3_tc_products_decode8.md", "fp4_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md",
@@ -44,6 +48,8 @@ TRAFFIC_SOURCE = {
     "fp8_prefill": "profiles/wide_expert_fp4_fp8_prefill.md",
     "fp8_decode_block128": "profiles/expert_b128_fp8_block128_decode64_prefill2048.md",
     "fp8_prefill_block128": "profiles/expert_b128_fp8_block128_decode64_prefill2048.md",
+    "fp4_prefill_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md", "fp8_prefill_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md",
+    "fp4_decode_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md", "fp8_decode_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md",
 }
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
 CONFIG = 1
@@ -581,6 +587,28 @@ def exl3_decode(amd, workloads, arguments):
     }
 
     got = layer.output()
+    if arguments.cached_what_if:
+        # how much of a products pass is memory: the five launches of the fused decode alone, with the job table as the
+        # select wrote it and with every job's matrices taken from the first expert of the same width (9 matrices, which
+        # the caches hold), in turns
+        table = jobs.copy()
+        first = {}
+        for j in range(len(table)):
+            if table[j]["row_count"] > 0:
+                for m, name in enumerate(("gate_offset", "up_offset", "down_offset")):
+                    table[j][name] = first.setdefault((m, int(widths[int(table[j]["expert"]), m])), int(table[j][name]))
+        turns = {"as_routed": [], "one_expert_a_width": []}
+        for _ in range(4):
+            for name, which in (("as_routed", jobs), ("one_expert_a_width", table)):
+                card.upload(layer.jobs_offset, which.view(np.uint8))
+                for _ in range(5):
+                    card.run_timed(fused)
+                spent = np.zeros(amd.EXL3_TC_LAUNCHES)
+                for _ in range(arguments.steps):
+                    spent += np.array(card.run_timed(fused))
+                turns[name].append([round(float(us), 2) for us in (spent / arguments.steps)[[1, 3]]])
+        card.upload(layer.jobs_offset, jobs.view(np.uint8))
+        result["config"]["cached_what_if"] = {"launch_us_gate_up_and_down_a_turn": turns, "distinct_matrices": len(first)}
     if not arguments.no_cpu:
         import _oracle
         threads = min(os.cpu_count() or 1, 16)
@@ -728,6 +756,9 @@ def main():
     parser.add_argument("--native", action="store_true",
                         help="fp4 and fp8 workloads: the experts' weights in gfx950's own lane order (WEIGHT_FORMAT_E2M1_GFX950 / _E4M3_GFX950, "
                              "made from the same bytes by the library's load-time re-lay-out)")
+    parser.add_argument("--cached-what-if", action="store_true",
+                        help="exl3_decode: also time the fused decode's launches with every job's matrices taken from one expert of "
+                             "the same width (the bytes come from the caches): what of a products pass is memory")
     parser.add_argument("--site", action="store_true",
                         help="fp4/fp8 workloads: the whole FFN site: the mix project and mix finish ahead of the router, the shared expert and the join "
                              "in place of the row sum")

@@ -496,9 +496,7 @@ ANEMONE_RECORD_HAS(expert_gate_up_quantize_arguments, 96);
 #define KERNEL_NATIVE_EXPERT_DOWN_STEM "native_expert_down_"
 #define NATIVE_E2M1_COLUMN_BLOCKS 4u /* a block of the E2M1_GFX950 launches: one tile of the wide select (64 pairs) */
 #define NATIVE_E4M3_COLUMN_BLOCKS 8u /* of the E4M3_GFX950 launches: two tiles of one expert (128 pairs), read once */
-#ifndef NATIVE_E2M1_STAGES
-#define NATIVE_E2M1_STAGES 2u
-#endif /* stages of columns in LDS: a K step in use, the next on its way */
+#define NATIVE_E2M1_STAGES 2u /* stages of columns in LDS: a K step in use, the next on its way */
 #define NATIVE_E4M3_STAGES 3u
 /* dynamic LDS: the stages of a K step of the block's columns (128 bytes of codes a column, 4 of scale codes) */
 #define NATIVE_WINDOW_BYTES(column_blocks, stages) ((stages) * ((column_blocks) * 2048u + (column_blocks) * 64u))
