@@ -300,7 +300,8 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
             result["roofline"] = {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_F8_PEAK_TFLOPS, "unit": "TFLOP/s",
                                   "frac": achieved / MFMA_F8_PEAK_TFLOPS, "traffic": result["roofline"]["traffic"],
                                   "algorithmic_flops_per_launch": gate_up_flops,
-                                  "launch_us": gate_up_us}
+                                  "launch_us": gate_up_us, **({"traffic_source": result["roofline"]["traffic_source"]}
+                                                              if "traffic_source" in result["roofline"] else {})}
         else:
             result["roofline"]["kernel"] = kernel  # the matrices' bytes of the distinct experts against the memory's peak
             result["roofline"]["TFLOPs"] = achieved
@@ -709,7 +710,7 @@ def summary(result):
     keep = {"workload": config["workload"], "ms_per_step": result["ms_per_step"], "tok_s": result["value"], "steps": result["steps"],
             "kernel": roofline["kernel"], "launch_us": roofline["launch_us"], "bound": roofline["bound"], "achieved": roofline["achieved"],
             "peak": roofline["peak"], "unit": roofline["unit"], "frac": roofline["frac"]}
-    for name in ("algorithmic_bytes_per_launch", "algorithmic_flops_per_launch", "TFLOPs", "flop_per_byte"):
+    for name in ("algorithmic_bytes_per_launch", "algorithmic_flops_per_launch", "TFLOPs", "flop_per_byte", "traffic", "traffic_source"):
         if name in roofline:
             keep[name] = roofline[name]
     for name in ("pairs_of_the_busiest_expert", "load_fit_total_variation", "chunks", "distinct_experts", "down_TFLOPs", "down_GBps"):
@@ -725,15 +726,16 @@ def summary(result):
     return keep
 
 
-# the workloads of the other configurations the metric names, as the default run's config.also: (workload, rows, block128)
+# the workloads of the other configurations the metric names, as the default run's config.also: (workload, rows, block128, gfx950 lane order)
 ALSO = [("exl3_linear", 1, False, False), ("exl3_prefill", 4096, False, False), ("fp8_decode", 1, True, False), ("fp8_decode", 64, True, False),
         ("fp8_prefill", 2048, True, False), ("fp8_prefill", 2048, False, False), ("fp8_prefill", 2048, False, True),
-        ("fp4_prefill", 8192, False, False), ("fp4_prefill", 8192, False, True), ("fp4_decode", 32, False, False)]
+        ("fp4_prefill", 8192, False, False), ("fp4_prefill", 8192, False, True), ("fp4_decode", 32, False, False), ("fp4_decode", 32, False, True)]
 # the other configurations' headline fractions as scalars of config (beside config.also, which holds the whole lines)
 HEADLINES = {("exl3_linear", False, False): "exl3_linear_hbm_frac", ("exl3_prefill", False, False): "exl3_prefill_mfma_frac",
              ("fp8_prefill", True, False): "fp8_block128_prefill_hbm_frac", ("fp8_prefill", False, False): "fp8_prefill_hbm_frac",
              ("fp8_prefill", False, True): "fp8_gfx950_prefill_hbm_frac", ("fp4_prefill", False, False): "fp4_prefill_mfma_frac",
-             ("fp4_prefill", False, True): "fp4_gfx950_prefill_mfma_frac", ("fp4_decode", False, False): "fp4_decode32_hbm_frac"}
+             ("fp4_prefill", False, True): "fp4_gfx950_prefill_mfma_frac", ("fp4_decode", False, False): "fp4_decode32_hbm_frac",
+             ("fp4_decode", False, True): "fp4_gfx950_decode32_hbm_frac"}
 
 
 def main():
