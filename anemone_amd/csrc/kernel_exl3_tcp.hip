@@ -10,11 +10,11 @@
  * a row's weighted pair outputs added in slot order. A pair's result does not depend on the other pairs of the call.
  *
  * The GEMM block: 256 outputs (four wavefronts of four 16 x 16 tiles) by one chunk of at most EXL3_TCP_CHUNK_PAIRS (160)
- * pairs of one expert. A K step is 32 inputs: the chunk's operand columns (160 x 32 fp16, 10 KB) go from memory straight
- * into LDS once a block and serve all four wavefronts; each wavefront streams the two tile rows of its own strip through a
- * private LDS window, decodes each 16 x 32 weight tile once (eight weights a lane) and feeds it to up to ten MFMAs, one for
- * every sixteen columns. Decoding is the vector unit's work (about 4.4 instructions a weight) and the products the matrix
- * unit's (16 cycles an MFMA).
+ * pairs of one expert. A K step is 64 inputs: the chunk's operand columns (160 x 64 fp16, 20 KB) go from memory straight
+ * into LDS once a block and serve all four wavefronts; each wavefront's codes go from memory into the registers of the
+ * lanes that decode them, a decoded operand of eight weights a lane feeds up to five matrix instructions of 32 x 32
+ * outputs, one for every 32 columns. Decoding is the vector unit's work (about 3.7 instructions a weight) and the
+ * products the matrix unit's (32 cycles an instruction).
  */
 #include "exl3_stream_device.cuh"
 #include "kernel_registry.h"
@@ -24,8 +24,9 @@
 #define TCP_GEMM_WAVES 4u
 #define TCP_GEMM_THREADS (TCP_GEMM_WAVES * WAVE)
 #define TCP_WAVE_PAIRS 2u  /* pairs of adjacent output tiles of a wavefront: 64 outputs */
-#define TCP_COLUMN_BLOCKS (EXL3_TCP_CHUNK_PAIRS / 16u)
+#define TCP_COLUMN_BLOCKS (EXL3_TCP_CHUNK_PAIRS / 16u) /* of sixteen columns: two a block of the matrix instruction's 32 */
 #define TCP_STEP_INPUTS 64u
+#define TCP_DIES 8u         /* the card's dies (XCDs), each with a level-2 cache of its own: blocks are dealt to them in turn */
 #define TCP_BATCH 4u        /* columns the element-wise launches take at a time */
 #define TCP_WAVE_BLOCKS 4u  /* blocks of 128 channels a wavefront of an element-wise launch takes: a row of sixteen lanes each */
 
@@ -245,13 +246,13 @@ ANEMONE_KERNEL(EXL3_TCP_KERNEL_FILE, exl3_tcp_operands, exl3_tcp_record);
  * The GEMM block: 256 outputs by one chunk of at most EXL3_TCP_CHUNK_PAIRS pairs of one expert, four wavefronts of 64
  * outputs each (two pairs of adjacent output tiles). A K step is 64 inputs (four K tiles).
  *
- * Weights: the codes go from memory straight into the registers of the lanes that decode them (exl3_stream_device.cuh:
- * lane 16 g + i holds chunk i % 8 of tile i / 8 of a tile pair and of K tile g of the step); a decoded operand of eight
- * weights a lane (output half h, input half v) feeds one matrix instruction a block of sixteen columns.
+ * Weights: the codes go from memory straight into the registers of the lanes that decode them, by the stream product's
+ * decode (exl3_stream_device.cuh) under the assignment of chunks to lanes that tcp_wave_gemm states; a decoded operand
+ * of eight weights a lane (output half h, input half v) feeds one matrix instruction a block of 32 columns.
  * Operands: a stage holds the step's 64 inputs of every column of the chunk, 128 bytes a column, its eight 16-byte pieces
- * at the slots piece ^ ((column / 2) % 8) so that the sixteen lanes of one read (sixteen columns, one piece) meet sixteen
- * different bank groups. Each wavefront brings a share of the stage (memory -> registers a step ahead -> LDS), one
- * barrier a step; the reader of column block j takes piece 2 g + v of column 16 j + i as the instruction's B operand.
+ * at the slots piece ^ ((column / 2) % 8) so that sixteen lanes of one read (sixteen columns, one piece) meet sixteen
+ * different bank groups. Each wavefront brings a share of the stage by LDS DMA a step ahead, one barrier a step; the
+ * reader of column block j takes piece 4 s + 2 (lane / 32) + v of column 32 j + lane % 32 as the instruction's B operand.
  */
 /* 16 bytes a lane from memory straight into LDS (lane L lands at lds_base + 16 L), no register in between. Written as
  * assembly: the compiler keeps no book on it, so the wait that ends a step (every load of the wavefront, then the block's
@@ -266,22 +267,31 @@ __device__ static __forceinline__ void tcp_load_to_lds(const void *lane_address,
 #define TCP_STAGE_GROUPS (EXL3_TCP_CHUNK_PAIRS / 8u) /* groups of eight columns: one 16-byte-a-lane load of a wavefront each */
 #define TCP_WAVE_GROUPS ((TCP_STAGE_GROUPS + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES)
 
+/* A wavefront's product of 64 outputs by the chunk's columns on the matrix instruction of 32 x 32 outputs
+ * (v_mfma_f32_32x32x16_f16: A lane l row l % 32, k = 8 (l / 32) + e; B lane l column l % 32, the same k; D lane l
+ * column l % 32, register r row r % 4 + 8 (r / 4) + 4 (l / 32); measured on the card). Lane 16 g + i decodes chunk i % 8 of output tile i / 8 + 2 (g % 2) of the
+ * wavefront's four and of K tile 2 s + g / 2 of the step's four (s = 0, 1: the step's halves), so the 32 rows of an
+ * instruction (h, v) are output (i % 8) + 8 h of those four tiles and its sixteen k are inputs 8 v .. + 7 of the two K
+ * tiles of half s: what a lane decodes, and how, is the stream product's; a decoded operand feeds LIVE instructions of
+ * twice the work each. LIVE: blocks of 32 columns. */
+typedef float float16v_t __attribute__((ext_vector_type(16)));
+
 template <uint32_t bits_x2, uint32_t LIVE>
 __device__ static __forceinline__ void
 tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t strip_tile, uint32_t inputs,
-              const half_t *__restrict__ columns, uint32_t column_count, uint32_t stages, uint32_t wave,
-              uint32_t lane, bool strip_is_live, float4_t (&accumulator)[TCP_WAVE_PAIRS][2][LIVE])
+                const half_t *__restrict__ columns, uint32_t column_count, uint32_t stages, uint32_t wave,
+                uint32_t lane, bool strip_is_live, float16v_t (&accumulator)[2][LIVE])
 {
     typedef exl3_chunk<bits_x2> C;
-    constexpr uint32_t live_groups = 2u * LIVE; /* groups of eight columns that hold a pair */
+    constexpr uint32_t live_groups = 4u * LIVE; /* groups of eight columns that hold a pair */
     constexpr uint32_t wave_groups = (live_groups + TCP_GEMM_WAVES - 1u) / TCP_GEMM_WAVES;
-    const uint32_t g = lane / 16u, i = lane % 16u, c = i % 8u;
+    const uint32_t g = lane / 16u, i = lane % 16u, c = i % 8u, upper = lane / 32u, row = lane % 32u;
     const bool odd = (c & 1u) != 0u;
     uint32_t own, front;
     exl3_chunk_place<bits_x2>(c, own, front);
-    const uint64_t step_stride = 4u * (uint64_t)out_tiles * C::tile_words;
+    const uint64_t step_stride = 4u * (uint64_t)out_tiles * C::tile_words, half_stride = 2u * (uint64_t)out_tiles * C::tile_words;
     /* a strip past the matrix reads the matrix's first strip (its sums are not stored): every wavefront runs the same loop */
-    const uint32_t *tile = codes + ((uint64_t)g * out_tiles + (strip_is_live ? strip_tile : 0u) + i / 8u) * C::tile_words;
+    const uint32_t *tile = codes + ((uint64_t)(g / 2u) * out_tiles + (strip_is_live ? strip_tile : 0u) + i / 8u + 2u * (g % 2u)) * C::tile_words;
     /* the stage's groups this wavefront brings: wave, wave + 4, ...: lane L column 8 G + L / 8, slot L % 8 */
     const unsigned char *operand_source[wave_groups];
 #pragma unroll
@@ -290,28 +300,30 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
         const uint32_t piece = (lane % 8u) ^ ((column / 2u) % 8u);
         operand_source[part] = (const unsigned char *)(columns + (uint64_t)(column < column_count ? column : 0u) * inputs) + piece * 16u;
     }
-    /* where this lane reads its B operand (v = 0, 1) of column block j: column 16 j + i, piece 2 g + v */
-    uint32_t read_at[2];
+    /* where this lane reads its B operand (half s, inputs v) of column block j: column 32 j + row, piece 4 s + 2 upper + v */
+    uint32_t read_at[2][2];
 #pragma unroll
-    for (uint32_t v = 0; v < 2u; v++) {
-        read_at[v] = i * TCP_STAGE_COLUMN_BYTES + (((2u * g + v) ^ ((i / 2u) % 8u)) * 16u);
+    for (uint32_t s = 0; s < 2u; s++) {
+#pragma unroll
+        for (uint32_t v = 0; v < 2u; v++) {
+            read_at[s][v] = row * TCP_STAGE_COLUMN_BYTES + (((4u * s + 2u * upper + v) ^ ((row / 2u) % 8u)) * 16u);
+        }
     }
 #pragma unroll
-    for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
+    for (uint32_t h = 0; h < 2u; h++) {
 #pragma unroll
-        for (uint32_t h = 0; h < 2u; h++) {
+        for (uint32_t j = 0; j < LIVE; j++) {
 #pragma unroll
-            for (uint32_t j = 0; j < LIVE; j++) {
-                accumulator[p][h][j] = (float4_t){0.0f, 0.0f, 0.0f, 0.0f};
+            for (uint32_t r = 0; r < 16u; r++) {
+                accumulator[h][j][r] = 0.0f;
             }
         }
     }
     const uint32_t steps = inputs / TCP_STEP_INPUTS;
-    exl3_chunk_words<bits_x2> held[2][TCP_WAVE_PAIRS];
-    /* step 0: its codes into held[0], its operand columns into stage 0 */
+    exl3_chunk_words<bits_x2> held[2][2];
 #pragma unroll
-    for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
-        exl3_chunk_load<bits_x2>(tile + p * 2u * C::tile_words, own, front, held[0][p]);
+    for (uint32_t s = 0; s < 2u; s++) {
+        exl3_chunk_load<bits_x2>(tile + s * half_stride, own, front, held[0][s]);
     }
 #pragma unroll
     for (uint32_t part = 0; part < wave_groups; part++) {
@@ -321,14 +333,14 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    auto one_step = [&](uint32_t step, exl3_chunk_words<bits_x2> (&now)[TCP_WAVE_PAIRS], exl3_chunk_words<bits_x2> (&next)[TCP_WAVE_PAIRS]) {
+    auto one_step = [&](uint32_t step, exl3_chunk_words<bits_x2> (&now)[2], exl3_chunk_words<bits_x2> (&next)[2]) {
         const bool more = step + 1u < steps; /* the same in every lane */
         const uint32_t stage = stages + (step % 2u) * TCP_STAGE_BYTES, other = stages + ((step + 1u) % 2u) * TCP_STAGE_BYTES;
         if (more) {
             tile += step_stride;
 #pragma unroll
-            for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
-                exl3_chunk_load<bits_x2>(tile + p * 2u * C::tile_words, own, front, next[p]);
+            for (uint32_t s = 0; s < 2u; s++) {
+                exl3_chunk_load<bits_x2>(tile + s * half_stride, own, front, next[s]);
             }
 #pragma unroll
             for (uint32_t part = 0; part < wave_groups; part++) {
@@ -339,21 +351,20 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
             }
         }
 #pragma unroll
-        for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++) {
-            exl3_chunk_align<bits_x2>(now[p], odd);
+        for (uint32_t s = 0; s < 2u; s++) {
+            exl3_chunk_align<bits_x2>(now[s], odd);
         }
-        /* Eight operands of eight weights a lane: k = 4 v + 2 p + h (input half v outermost: its LIVE B operands are read
-         * from the stage once). An operand's LIVE matrix instructions are issued with the next operand's decoding between
-         * them, a quarter of it (two weights) behind every LIVE / 4 instructions: the decoding runs in the products' shadow. */
+        /* Eight operands of eight weights a lane: k = 4 s + 2 v + h (the B operands of (s, v) serve both h and are read a
+         * pair of operands ahead). An operand's LIVE matrix instructions are issued with the next operand's decoding
+         * between them: the decoding runs in the products' shadow. */
         auto decode_weight = [&](uint32_t k, uint32_t w, uint32_t (&into)[4]) {
-            /* weight w = 2 t + e of operand k: symbol 8 t + 4 h + 2 v + e; the odd one completes its pair's register */
-            const uint32_t v = k / 4u, p = k / 2u % 2u, h = k % 2u, t = w / 2u, m = 8u * t + 4u * h + 2u * v + w % 2u;
+            const uint32_t s = k / 4u, v = k / 2u % 2u, h = k % 2u, t = w / 2u, m = 8u * t + 4u * h + 2u * v + w % 2u;
             uint32_t funnel[C::words];
 #pragma unroll
             for (uint32_t word = 0; word < C::words; word++) {
-                funnel[word] = __builtin_amdgcn_alignbit(now[p].z[word], now[p].z[word + 1u], 16u);
+                funnel[word] = __builtin_amdgcn_alignbit(now[s].z[word], now[s].z[word + 1u], 16u);
             }
-            const uint32_t product = exl3_chunk_state<bits_x2>(now[p].z, funnel, m) * EXL3_MUL1_MULTIPLIER;
+            const uint32_t product = exl3_chunk_state<bits_x2>(now[s].z, funnel, m) * EXL3_MUL1_MULTIPLIER;
             if (w % 2u == 0u) {
                 into[t] = __builtin_amdgcn_sad_u8(product, 0u, (uint32_t)EXL3_MUL1_BASE * 0x10001u);
             } else {
@@ -363,12 +374,12 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
                 into[t] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(half2_t, sums), scale, bias));
             }
         };
-        half8_t operand_b[LIVE];
+        half8_t operand_b[2][LIVE];
         uint32_t a[4], ahead[4];
-        auto read_operands = [&](uint32_t v) {
+        auto read_operands = [&](uint32_t k) { /* those of operands k and k + 1 */
 #pragma unroll
             for (uint32_t j = 0; j < LIVE; j++) {
-                operand_b[j] = __builtin_bit_cast(half8_t, *(const __attribute__((address_space(3))) uint4_t *)(uintptr_t)(stage + j * (16u * TCP_STAGE_COLUMN_BYTES) + read_at[v]));
+                operand_b[k / 2u % 2u][j] = __builtin_bit_cast(half8_t, *(const __attribute__((address_space(3))) uint4_t *)(uintptr_t)(stage + j * (32u * TCP_STAGE_COLUMN_BYTES) + read_at[k / 4u][k / 2u % 2u]));
             }
         };
         read_operands(0u); /* on their way while the first operand is decoded */
@@ -379,15 +390,15 @@ tcp_wave_gemm(const uint32_t *__restrict__ codes, uint32_t out_tiles, uint32_t s
         }
 #pragma unroll
         for (uint32_t k = 0; k < 8u; k++) {
-            const uint32_t p = k / 2u % 2u, h = k % 2u;
-            if (k == 4u) {
-                read_operands(1u);
+            const uint32_t h = k % 2u;
+            if (k % 2u == 0u && k + 2u < 8u) {
+                read_operands(k + 2u);
             }
             const uint4_t packed = {a[0], a[1], a[2], a[3]};
             const half8_t weights = __builtin_bit_cast(half8_t, packed);
 #pragma unroll
             for (uint32_t j = 0; j < LIVE; j++) {
-                accumulator[p][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(weights, operand_b[j], accumulator[p][h][j], 0, 0, 0);
+                accumulator[h][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(weights, operand_b[k / 2u % 2u][j], accumulator[h][j], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 if (k + 1u < 8u) {
 #pragma unroll
@@ -424,13 +435,24 @@ extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS, 2) exl3_tcp_gemm(
     __shared__ __attribute__((aligned(16))) unsigned char stages[2u * TCP_STAGE_BYTES];
     const tcp_shape shape = tcp_shape_of(record);
     unsigned char *workspace = arena + record.workspace_offset;
-    const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, blockIdx.y);
+    /* Which (strip of 256 outputs, chunk, projection) this block takes. The card deals blocks to its eight dies in turn by
+     * their number x + gx (y + gy z), so die c holds the blocks whose x % 8 is c. Every output strip of a chunk reads the
+     * chunk's operand columns: the blocks of eight consecutive rows m = y + gy z of the grid are re-assigned so that those
+     * a die holds among them are all the strips of one (chunk, projection), which then come from memory into that die's
+     * level-2 cache once (a grid whose x is no multiple of eight, and the rows past the last whole eight, stay as dealt). */
+    uint32_t strip = blockIdx.x, place = blockIdx.y + gridDim.y * blockIdx.z;
+    const uint32_t places = gridDim.y * gridDim.z;
+    if (gridDim.x % TCP_DIES == 0u && place < places / TCP_DIES * TCP_DIES) {
+        strip = (place % TCP_DIES) * (gridDim.x / TCP_DIES) + blockIdx.x / TCP_DIES;
+        place = place / TCP_DIES * TCP_DIES + blockIdx.x % TCP_DIES;
+    }
+    const struct exl3_tcp_chunk chunk = tcp_chunk_of(shape, workspace, place % gridDim.y);
     if (chunk.pair_count == 0u) {
         return;
     }
     const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const bool down = record.pass == EXL3_TCP_DOWN;
-    const uint32_t projection = down ? 2u : blockIdx.z;
+    const uint32_t projection = down ? 2u : place / gridDim.y;
     const uint32_t inputs = down ? shape.intermediate : shape.hidden, outputs = down ? shape.hidden : shape.intermediate;
     const uint32_t bits_x2 = tcp_bits_x2(record, arena, chunk.expert, projection);
     const uint32_t *codes = (const uint32_t *)(arena + tcp_matrix_of(record, arena, chunk.expert, projection));
@@ -438,27 +460,31 @@ extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS, 2) exl3_tcp_gemm(
                             ((uint64_t)(down ? 0u : projection) * shape.pairs + chunk.first_pair) * inputs;
     float *products = down ? (float *)(workspace + shape.layout.down) + (uint64_t)chunk.first_pair * outputs
                            : (float *)(workspace + shape.layout.gate_up) + ((uint64_t)projection * shape.pairs + chunk.first_pair) * outputs;
-    const uint32_t strip_tile = (blockIdx.x * EXL3_TCP_BLOCK_OUTPUTS) / EXL3_TILE + wave * 2u * TCP_WAVE_PAIRS;
+    const uint32_t strip_tile = (strip * EXL3_TCP_BLOCK_OUTPUTS) / EXL3_TILE + wave * 2u * TCP_WAVE_PAIRS;
     const bool strip_is_live = strip_tile * EXL3_TILE < outputs;
     const uint32_t stage_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)stages;
-    /* one instance a width and a count of live column blocks (2, 4, 6, 8 or all): the pairs' columns and nothing past them */
     const uint32_t live_blocks = (chunk.pair_count + 15u) / 16u;
+    /* one instance a width and a count of live blocks of 32 columns (1 to 5): the pairs' columns and nothing past them */
 #define TCP_GEMM_OF(bits, live)                                                                                                   \
     do {                                                                                                                          \
-        float4_t accumulator[TCP_WAVE_PAIRS][2][live];                                                                            \
+        float16v_t accumulator[2][live];                                                                                          \
         tcp_wave_gemm<bits, live>(codes, outputs / EXL3_TILE, strip_tile, inputs, columns, chunk.pair_count, stage_base, wave, lane, \
-                                  strip_is_live, accumulator);                                                                    \
+                                    strip_is_live, accumulator);                                                                  \
         if (strip_is_live) {                                                                                                      \
             _Pragma("unroll") for (uint32_t j = 0; j < live; j++)                                                                 \
             {                                                                                                                     \
-                const uint32_t column = 16u * j + lane % 16u;                                                                     \
+                const uint32_t column = 32u * j + lane % 32u;                                                                     \
                 if (column < chunk.pair_count) {                                                                                  \
                     float *out = products + (uint64_t)column * outputs;                                                           \
-                    _Pragma("unroll") for (uint32_t p = 0; p < TCP_WAVE_PAIRS; p++)                                               \
+                    _Pragma("unroll") for (uint32_t h = 0; h < 2u; h++)                                                           \
                     {                                                                                                             \
-                        _Pragma("unroll") for (uint32_t h = 0; h < 2u; h++)                                                       \
+                        _Pragma("unroll") for (uint32_t q = 0; q < 4u; q++)                                                       \
                         {                                                                                                         \
-                            *(float4_t *)(out + exl3_stream_output(strip_tile, p, h, lane)) = accumulator[p][h][j];               \
+                            const uint32_t first_row = 8u * q + 4u * (lane / 32u);                                                \
+                            const uint32_t output = EXL3_TILE * (strip_tile + first_row % 16u / 8u + 2u * (first_row / 16u)) +    \
+                                                    first_row % 8u + 8u * h;                                                      \
+                            *(float4_t *)(out + output) = (float4_t){accumulator[h][j][4u * q], accumulator[h][j][4u * q + 1u],   \
+                                                                     accumulator[h][j][4u * q + 2u], accumulator[h][j][4u * q + 3u]}; \
                         }                                                                                                         \
                     }                                                                                                             \
                 }                                                                                                                 \
@@ -467,15 +493,15 @@ extern "C" __global__ void __launch_bounds__(TCP_GEMM_THREADS, 2) exl3_tcp_gemm(
     } while (0)
 #define TCP_GEMM_WIDTH(bits)                    \
     if (live_blocks <= 2u) {                    \
-        TCP_GEMM_OF(bits, 2u);                  \
+        TCP_GEMM_OF(bits, 1u);                  \
     } else if (live_blocks <= 4u) {             \
-        TCP_GEMM_OF(bits, 4u);                  \
+        TCP_GEMM_OF(bits, 2u);                  \
     } else if (live_blocks <= 6u) {             \
-        TCP_GEMM_OF(bits, 6u);                  \
+        TCP_GEMM_OF(bits, 3u);                  \
     } else if (live_blocks <= 8u) {             \
-        TCP_GEMM_OF(bits, 8u);                  \
+        TCP_GEMM_OF(bits, 4u);                  \
     } else {                                    \
-        TCP_GEMM_OF(bits, TCP_COLUMN_BLOCKS);   \
+        TCP_GEMM_OF(bits, TCP_COLUMN_BLOCKS / 2u); \
     }
     switch (bits_x2) {
     case 4u: TCP_GEMM_WIDTH(4u) break;
