@@ -174,7 +174,7 @@ extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E2M1_WAVES) 
     native_expert_down<false, NATIVE_E2M1_COLUMN_BLOCKS / 4u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_down_1, wide_expert_down_arguments);
-#define NATIVE_E4M3_WAVES 2 /* wavefronts a SIMD the launch is compiled for: 256 registers */
+#define NATIVE_E4M3_WAVES 3 /* 168 registers (the down launch took 170 left to itself, and two wavefronts a SIMD: 487 against 461 us) */
 extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E4M3_WAVES) native_expert_gate_up_e4m3_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
 {
     native_expert_gate_up<true, 1u, NATIVE_E4M3_COLUMN_BLOCKS / 4u>(arguments, arena);
