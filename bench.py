@@ -37,13 +37,14 @@ MEASURED_TRAFFIC_BYTES = {
     ("expert_join", 8192): 877.7e6 + 402.7e6,
     ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,
     ("fp8_prefill_block128", 2048): 5386.8e6 + 67.2e6,
-    ("fp4_prefill_native", 8192): 5870.2e6 + 450.7e6,
+    ("fp4_prefill_native", 8192): 5530.8e6 + 415.4e6,
+    ("exl3_prefill", 4096): 2858.6e6 + 538.5e6,
     ("fp8_prefill_native", 2048): 4711.2e6 + 113.3e6,
     ("fp4_decode_native", 32): 1434.2e6 + 1.0e6,
     ("fp8_decode_native", 32): 2746.7e6 + 1.0e6,
 }
 TRAFFIC_SOURCE = {
-    "exl3_decode": "profiles/exl3_tc_products_decode8.md", "fp4_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md",
+    "exl3_decode": "profiles/exl3_tc_products_decode8.md", "exl3_prefill": "profiles/exl3_tcp_gemm_prefill4096.md", "fp4_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md",
     "fp8_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md", "fp4_prefill": "profiles/wide_expert_fp4_fp8_prefill.md",
     "fp8_prefill": "profiles/wide_expert_fp4_fp8_prefill.md",
     "fp8_decode_block128": "profiles/expert_b128_fp8_block128_decode64_prefill2048.md",
@@ -489,6 +490,9 @@ def exl3_prefill(amd, workloads, arguments):
                      "unit": "TFLOP/s", "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": None,
                      "algorithmic_flops_per_launch": gate_up_flops, "launch_us": gate_up_us},
     }
+    if ("exl3_prefill", rows) in MEASURED_TRAFFIC_BYTES and arguments.zipf_strength <= 0.0:
+        result["roofline"]["traffic"] = MEASURED_TRAFFIC_BYTES[("exl3_prefill", rows)]
+        result["roofline"]["traffic_source"] = TRAFFIC_SOURCE["exl3_prefill"] + " (counter bytes of the profiled run, not of this one)"
     if not arguments.no_cpu:
         import ctypes as C
         import _oracle as o
