@@ -33,8 +33,10 @@ ANEMONE_KERNEL("kernel_calibrate", arena_copy, arena_copy_arguments);
  * wavefront; `kind` names the instruction, eight independent chains a lane, `iterations` trips of eight each; kinds 8
  * to 10 are trips of four v_mfma_f32_16x16x32_f16 alone, of eight vector instructions alone, and of the four matrix
  * instructions with two of the vector instructions behind each; kind 11 is trips of eight v_mfma_f32_16x16x1_4b_f32 (the
- * router's many-row projection: one fused multiply-add a sum of four 16 x 16 blocks), each on sums of its own. The host
- * times the launch; what is written is only there to keep the chains alive. */
+ * router's many-row projection: one fused multiply-add a sum of four 16 x 16 blocks), each on sums of its own; kinds 12
+ * to 15 are trips of ten v_mfma_f32_32x32x16_f16 (the EXL3 prefill GEMM's), each on sums of its own, with 0, 7, 14 and 30 of
+ * the codebook's vector instructions behind each: how far a wavefront's decoding runs beside its matrix instructions. The
+ * host times the launch; what is written is only there to keep the chains alive. */
 struct issue_rate_arguments {
     uint64_t output_offset; /* written: uint32 [grid x 64] */
     uint32_t kind;
@@ -63,6 +65,38 @@ __device__ static __forceinline__ float issue_rate_blocks(uint32_t iterations, f
     }
     float kept = 0.0f;
     for (uint32_t q = 0; q < 8u; q++) {
+        for (uint32_t v = 0; v < 16u; v++) {
+            kept += sums[q][v];
+        }
+    }
+    return kept;
+}
+
+/* kinds 12 to 15: `iterations` trips of ten v_mfma_f32_32x32x16_f16 with BEHIND vector instructions behind each */
+template <uint32_t BEHIND>
+__device__ static __forceinline__ float issue_rate_beside(uint32_t iterations, uint32_t (&a)[8], rate_half8 left, rate_half8 right)
+{
+    rate_float16 sums[10];
+    for (uint32_t q = 0; q < 10u; q++) {
+        for (uint32_t v = 0; v < 16u; v++) {
+            sums[q][v] = 0.0f;
+        }
+    }
+    const uint32_t multiplier = 0x83DCD12Du;
+    for (uint32_t trip = 0; trip < iterations; trip++) {
+#pragma unroll
+        for (uint32_t q = 0; q < 10u; q++) {
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(sums[q]) : "v"(left), "v"(right));
+#pragma unroll
+            for (uint32_t n = 0; n < BEHIND; n++) {
+                if (n % 3u == 0u) asm volatile("v_mul_lo_u32 %0, %0, %1" : "+v"(a[n % 8u]) : "s"(multiplier));
+                if (n % 3u == 1u) asm volatile("v_bfe_u32 %0, %0, 3, 16" : "+v"(a[n % 8u]));
+                if (n % 3u == 2u) asm volatile("v_sad_u8 %0, %0, 0, %0" : "+v"(a[n % 8u]));
+            }
+        }
+    }
+    float kept = 0.0f;
+    for (uint32_t q = 0; q < 10u; q++) {
         for (uint32_t v = 0; v < 16u; v++) {
             kept += sums[q][v];
         }
@@ -116,6 +150,21 @@ extern "C" __global__ void __launch_bounds__(64) issue_rate(struct issue_rate_ar
     if (arguments.kind == 11u) { /* the same in every lane */
         const float kept = issue_rate_blocks(arguments.iterations, (float)(threadIdx.x % 7u) * 0.001f, 1.0f + (float)threadIdx.x * 0.002f);
         ((uint32_t *)(arena + arguments.output_offset))[blockIdx.x * 64u + threadIdx.x] = (uint32_t)kept;
+        return;
+    }
+    if (arguments.kind >= 12u) { /* the same in every lane */
+        float kept = 0.0f;
+        switch (arguments.kind) {
+        case 12u: kept = issue_rate_beside<0u>(arguments.iterations, a, left, right); break;
+        case 13u: kept = issue_rate_beside<7u>(arguments.iterations, a, left, right); break;
+        case 14u: kept = issue_rate_beside<14u>(arguments.iterations, a, left, right); break;
+        default: kept = issue_rate_beside<30u>(arguments.iterations, a, left, right); break;
+        }
+        uint32_t word = (uint32_t)kept;
+        for (uint32_t i = 0; i < 8u; i++) {
+            word ^= a[i];
+        }
+        ((uint32_t *)(arena + arguments.output_offset))[blockIdx.x * 64u + threadIdx.x] = word;
         return;
     }
     switch (arguments.kind) {

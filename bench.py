@@ -113,7 +113,8 @@ def calibrate(amd):
     rates = {}
     kinds = ["v_mul_lo_u32", "v_sad_u8", "v_bfe_u32", "v_and_b32", "v_pk_fma_f16", "v_alignbit_b32", "v_lshrrev_b32", "v_perm_b32",
              "4 mfma_16x16x32_f16 a trip", "4 x (v_mul_lo_u32, v_sad_u8) a trip", "4 mfma with 2 of the 8 vector instructions behind each, a trip",
-             "v_mfma_f32_16x16x1_4b_f32"]
+             "v_mfma_f32_16x16x1_4b_f32", "v_mfma_f32_32x32x16_f16 alone", "v_mfma_f32_32x32x16_f16 with 7 vector instructions behind it",
+             "v_mfma_f32_32x32x16_f16 with 14 vector instructions behind it", "v_mfma_f32_32x32x16_f16 with 30 vector instructions behind it"]
     iterations, out = 20000, card.reserve(64 << 20)
     probe = amd.launches_of(1)
     probe[0].kernel = card.kernel("kernel_calibrate", "issue_rate", 16)
@@ -123,11 +124,12 @@ def calibrate(amd):
         probe[0].grid[0], probe[0].grid[1], probe[0].grid[2] = 1024 * waves, 1, 1
         for kind, name in enumerate(kinds):
             C.memmove(probe[0].argument, (C.c_uint64 * 1)(out), 8)
-            C.memmove(C.byref(probe[0], type(probe[0]).argument.offset + 8), (C.c_uint32 * 2)(kind, iterations), 8)
+            trips = iterations if kind < 12 else iterations // 4
+            C.memmove(C.byref(probe[0], type(probe[0]).argument.offset + 8), (C.c_uint32 * 2)(kind, trips), 8)
             card.run_timed(probe)
             microseconds = min(card.run_timed(probe)[0] for _ in range(2))
-            per = 8.0 if kind < 8 or kind == 11 else 1.0  # instructions (or trips) a loop body
-            rates["%d waves a SIMD: %s" % (waves, name)] = round(microseconds * 1e-6 * 2.4e9 / (iterations * per * waves), 2)
+            per = 8.0 if kind < 8 or kind == 11 else 10.0 if kind >= 12 else 1.0  # instructions (or trips) a loop body
+            rates["%d waves a SIMD: %s" % (waves, name)] = round(microseconds * 1e-6 * 2.4e9 / (trips * per * waves), 2)
     card.close()
     print(json.dumps({"calibrate": "arena_copy", "bytes_read": size, "bytes_written": size, "launch_us": times,
                       "GBps_read_plus_write": 2 * size / (min(times) * 1e-6) / 1e9,
