@@ -510,7 +510,7 @@ def test_tcp_prepare_geometry_and_refusals(fake):
 def experts_description(fmt=amd.WEIGHT_FORMAT_E2M1_SCALED, **changes):
     rows, P, H, I = 8, 8, 4096, 2048
     pairs = rows * P
-    bits = 8 if fmt in (amd.WEIGHT_FORMAT_E4M3_SCALED, amd.WEIGHT_FORMAT_E4M3_BLOCK128) else 4
+    bits = 8 if fmt in (amd.WEIGHT_FORMAT_E4M3_SCALED, amd.WEIGHT_FORMAT_E4M3_BLOCK128, amd.WEIGHT_FORMAT_E4M3_GFX950) else 4
     d = amd.RoutedExpertsDescription()
     cursor = [4096]
 
@@ -824,6 +824,54 @@ def test_block128_prepare_geometry_and_refusals(fake):
     assert lib.linear_wide_experts_block128_prepare(C.byref(wide_experts_description(amd.WEIGHT_FORMAT_E4M3_SCALED)), arena, C.byref(linear),
                                                     C.byref(wide_kernels), three) == 1
     assert not any(bytes(three))
+
+
+def test_gfx950_formats_prepare_geometry_and_refusals(fake):
+    """The formats in gfx950's lane order (7, 8): the job-table launches by the expert_*_gfx950_<S> kernels on the
+    reference formats' grids, the wide form by linear_native_experts_prepare alone, the producer refused."""
+    lib = amd.library()
+    arena = 8 << 30
+    linear, wide_kernels, native = amd.LinearKernels(), amd.LinearWideKernels(), amd.LinearNativeKernels()
+    assert lib.linear_kernels_prepare(fake.address, fake.card, 950, C.byref(linear)) == 0
+    assert lib.linear_wide_kernels_prepare(fake.address, fake.card, 950, C.byref(wide_kernels)) == 0
+    assert lib.linear_native_kernels_prepare(fake.address, fake.card, 950, C.byref(native)) == 0
+    assert fake.handles[linear.expert_gate_up_gfx950[0]][1] == "expert_gate_up_gfx950_1"
+    assert fake.handles[linear.expert_down_e4m3_gfx950[3]][1] == "expert_down_e4m3_gfx950_8" and linear.expert_gate_up_gfx950[4] == amd.BACKEND_NO_KERNEL
+    assert fake.handles[native.native_expert_gate_up][1] == "native_expert_gate_up_1" and fake.handles[native.native_expert_down_e4m3][1] == "native_expert_down_e4m3_1"
+    for fmt, like, names in ((amd.WEIGHT_FORMAT_E2M1_GFX950, amd.WEIGHT_FORMAT_E2M1_SCALED, ["expert_gate_up_gfx950_4", "expert_down_gfx950_2"]),
+                             (amd.WEIGHT_FORMAT_E4M3_GFX950, amd.WEIGHT_FORMAT_E4M3_SCALED, ["expert_gate_up_e4m3_gfx950_4", "expert_down_e4m3_gfx950_2"])):
+        launches, reference = amd.launches_of(4), amd.launches_of(4)
+        assert lib.linear_routed_experts_prepare(C.byref(experts_description(fmt)), ARENA, C.byref(linear), launches) == 0
+        assert lib.linear_routed_experts_prepare(C.byref(experts_description(like)), ARENA, C.byref(linear), reference) == 0
+        assert [fake.handles[launches[i].kernel][1] for i in (0, 2)] == names
+        assert fake.handles[launches[1].kernel][1] == "activation_quantize_entry" and fake.handles[launches[3].kernel][1] == "expert_row_sum_entry"
+        for ours, theirs in zip(launches, reference):  # the grids, blocks and records of the reference format's launches
+            assert list(ours.grid) == list(theirs.grid) and list(ours.block) == list(theirs.block)
+            assert bytes(ours.argument) == bytes(theirs.argument)
+        # the wide form: its own prepare takes these formats, the reference formats' prepare does not, and the other way round
+        three, untouched = amd.launches_of(3), amd.launches_of(4)
+        description = wide_experts_description(fmt)
+        assert lib.linear_native_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(native), three) == 0
+        assert fake.handles[three[0].kernel][1].startswith("native_expert_gate_up") and fake.handles[three[2].kernel][1] == "expert_row_sum_entry"
+        assert three[0].dynamic_shared_byte_count > 0 and three[0].block[0] == 256
+        assert lib.linear_wide_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(wide_kernels), untouched) == 1
+        assert lib.linear_native_experts_prepare(C.byref(wide_experts_description(like)), arena, C.byref(linear), C.byref(native), untouched) == 1
+        assert not any(bytes(untouched))
+    # E2M1_GFX950 stores whole groups of four tiles: outputs in whole 64
+    odd = amd.launches_of(4)
+    assert lib.linear_routed_experts_prepare(C.byref(experts_description(amd.WEIGHT_FORMAT_E2M1_GFX950, gate_up_shape=amd.Shape(2048 + 32, 4096, 4, 0),
+                                                                         down_shape=amd.Shape(4096, 2048 + 32, 4, 0))), ARENA, C.byref(linear), odd) == 1
+    assert not any(bytes(odd))
+    # the producer is built for the reference's two formats
+    fused = amd.ExpertFusedKernels()
+    assert lib.expert_fused_kernels_prepare(fake.address, fake.card, 950, C.byref(fused)) == 0
+    one = amd.launches_of(1)
+    for fmt in (amd.WEIGHT_FORMAT_E2M1_GFX950, amd.WEIGHT_FORMAT_E4M3_GFX950, amd.WEIGHT_FORMAT_E4M3_BLOCK128):
+        d = experts_description(fmt)
+        arrivals = amd.Range(6 << 30, 64 * (2048 // 32) * 4)
+        assert lib.expert_producer_prepare(C.byref(d), arrivals, arena, C.byref(linear), C.byref(fused), one) == 1, fmt
+        assert not any(bytes(one))
+    assert lib.expert_producer_prepare(C.byref(experts_description()), amd.Range(6 << 30, 64 * (2048 // 32) * 4), arena, C.byref(linear), C.byref(fused), one) == 0
 
 
 def site_description(rows=8, width=4096, combined=True, **changes):
