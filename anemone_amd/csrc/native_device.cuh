@@ -16,6 +16,10 @@
 #include "linear_device.cuh"
 
 #define NATIVE_WAVES 4u
+/* one-byte weights: a step's next weights are asked for at its top, ahead of the columns' preparation and the barrier
+ * (gate/up 953 -> 933 us, down 462 -> 456); 4-bit weights: in the middle of its matrix instructions (at the top: gate/up
+ * 1 % shorter, down 3 % longer) */
+#define NATIVE_WEIGHTS_FIRST_OF(bytes) (bytes)
 #define NATIVE_THREADS (NATIVE_WAVES * WAVE)
 
 /* memory into registers, 16 bytes or one byte a lane: the address is a base common to the wavefront plus the lane's own
@@ -218,9 +222,10 @@ struct native_chain {
         }
     }
 
-    /* one K step of LIVE column blocks from a stage's columns and a set of weight registers */
-    template <uint32_t LIVE>
-    __device__ __forceinline__ void consume(uint32_t stage, const slot &set, float4_t (&chain)[TILES][COLUMN_BLOCKS]) const
+    /* one K step of LIVE column blocks from a stage's columns and a set of weight registers; `between` runs behind the
+     * middle column block's matrix instructions */
+    template <uint32_t LIVE, typename BETWEEN>
+    __device__ __forceinline__ void consume(uint32_t stage, const slot &set, float4_t (&chain)[TILES][COLUMN_BLOCKS], BETWEEN between) const
     {
         uint32_t base = window + stage * STAGE_BYTES;
         asm volatile("" : "+s"(base));
@@ -246,6 +251,9 @@ struct native_chain {
                 scale_b = lds_read<unsigned char>(b_scale_at + (j + 1u) * 64u);
             }
             multiply_tiles<0>(set, scale_a, b, scale_now, j, chain);
+            if (j == (LIVE - 1u) / 2u) {
+                between();
+            }
         }
         __builtin_amdgcn_s_setprio(0);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stage is read before the next barrier */
@@ -254,15 +262,16 @@ struct native_chain {
     /* How many loads may be outstanding at the top of K step `step` for its columns and weights to have landed. Loads in
      * the order they are asked for: the columns of steps 0 .. DEPTH - 2, the weights of steps 0 .. SLOTS - 2, then, in
      * every step j, the columns of step j + DEPTH - 1 and behind them the weights of step j + SLOTS - 1 (where the chain
-     * has such steps). The count is of the loads of later steps asked for behind the later of the two. */
+     * has such steps; with WEIGHTS_FIRST the weights, then the columns). The count is of the loads of later steps asked for behind the later of the two. */
+    static constexpr bool WEIGHTS_FIRST = NATIVE_WEIGHTS_FIRST_OF(BYTES); /* inside a step: the weights asked for ahead of the columns */
     __device__ static __forceinline__ uint32_t when_columns(uint32_t k)
     {
-        return k < DEPTH - 1u ? k : 64u * (1u + k - (DEPTH - 1u));
+        return k < DEPTH - 1u ? k : 64u * (1u + k - (DEPTH - 1u)) + (WEIGHTS_FIRST ? 1u : 0u);
     }
 
     __device__ static __forceinline__ uint32_t when_weights(uint32_t k)
     {
-        return k < SLOTS - 1u ? DEPTH - 1u + k : 64u * (1u + k - (SLOTS - 1u)) + 1u;
+        return k < SLOTS - 1u ? DEPTH - 1u + k : 64u * (1u + k - (SLOTS - 1u)) + (WEIGHTS_FIRST ? 0u : 1u);
     }
 
     __device__ static __forceinline__ uint32_t loads_behind(uint32_t step, uint32_t total)
@@ -306,6 +315,14 @@ struct native_chain {
     {
         wait_behind(loads_behind(step, total));
         landed(sets[K]);
+        const auto ask = [&]() {
+            if (step + SLOTS - 1u < total) {
+                issue_weights(sets[(K + SLOTS - 1u) % SLOTS], step + SLOTS - 1u);
+            }
+        };
+        if constexpr (WEIGHTS_FIRST) {
+            ask(); /* into the set the step before this one used: nothing of the block's is waited for */
+        }
         /* where the sets and the stages go round together the stage is a constant of the instance */
         const uint32_t stage = SLOTS % DEPTH == 0u ? K % DEPTH : step % DEPTH;
         prepare_columns(stage);
@@ -313,10 +330,17 @@ struct native_chain {
         if (step + DEPTH - 1u < total) {
             issue_vectors((stage + DEPTH - 1u) % DEPTH, step + DEPTH - 1u);
         }
-        if (step + SLOTS - 1u < total) {
-            issue_weights(sets[(K + SLOTS - 1u) % SLOTS], step + SLOTS - 1u);
+        /* 4-bit weights: the next weights are asked for in the middle of the step's matrix instructions (a launch 1.7 %
+         * shorter than asking ahead of them: the requests spread over the step); one-byte weights in the middle: a quarter
+         * slower */
+        if constexpr (WEIGHTS_FIRST) {
+            consume<LIVE>(stage, sets[K], chain, []() {});
+        } else if constexpr (BYTES) {
+            ask();
+            consume<LIVE>(stage, sets[K], chain, []() {});
+        } else {
+            consume<LIVE>(stage, sets[K], chain, ask);
         }
-        consume<LIVE>(stage, sets[K], chain);
     }
 
     template <uint32_t LIVE, uint32_t K>
