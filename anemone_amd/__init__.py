@@ -15,6 +15,7 @@ STATUS_OK, STATUS_INVALID_ARGUMENT, STATUS_OUT_OF_MEMORY = 0, 1, 2
 STATUS_DEVICE_ERROR, STATUS_TIMED_OUT, STATUS_UNSUPPORTED, STATUS_BUSY = 5, 6, 7, 8
 WEIGHT_FORMAT_EXL3, WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E4M3_SCALED, WEIGHT_FORMAT_E4M3_BLOCK128 = 2, 3, 5, 6
 WEIGHT_FORMAT_E2M1_GFX950, WEIGHT_FORMAT_E4M3_GFX950 = 7, 8  # the two _SCALED formats in gfx950's own lane order
+WEIGHT_FORMAT_E4M3_BLOCK128_GFX950 = 9  # E4M3_BLOCK128's codes in E4M3_GFX950's lane order, its float32 scales as they are
 ARITHMETIC_CLASS_GFX950 = 950
 BACKEND_NO_KERNEL = 0xFFFFFFFF
 LAUNCH_CHAIN, LAUNCH_SIDE, LAUNCH_RESUME, LAUNCH_JOIN, LAUNCH_SIDE_MORE = 0, 1, 2, 3, 4  # kernel_launch.branch
@@ -143,7 +144,7 @@ class LinearKernels(C.Structure):
                 ("trunk_linear_quantized_interleaved", u32), ("expert_gate_up_e4m3", u32 * 5), ("expert_down_e4m3", u32 * 5),
                 ("expert_gate_up_b128", u32 * 5), ("expert_down_b128", u32 * 5), ("activation_quantize_128", u32),
                 ("expert_gate_up_gfx950", u32 * 5), ("expert_down_gfx950", u32 * 5), ("expert_gate_up_e4m3_gfx950", u32 * 5),
-                ("expert_down_e4m3_gfx950", u32 * 5)]
+                ("expert_down_e4m3_gfx950", u32 * 5), ("expert_gate_up_b128_gfx950", u32 * 5), ("expert_down_b128_gfx950", u32 * 5)]
 
 
 class ExpertFusedKernels(C.Structure):
@@ -239,7 +240,8 @@ class LinearWideKernels(C.Structure):
 
 
 class LinearNativeKernels(C.Structure):
-    _fields_ = [("native_expert_gate_up", u32), ("native_expert_down", u32), ("native_expert_gate_up_e4m3", u32), ("native_expert_down_e4m3", u32)]
+    _fields_ = [("native_expert_gate_up", u32), ("native_expert_down", u32), ("native_expert_gate_up_e4m3", u32), ("native_expert_down_e4m3", u32),
+                ("native_expert_gate_up_b128", u32), ("native_expert_down_b128", u32)]
 
 
 class QuantizeDescription(C.Structure):
@@ -377,11 +379,11 @@ def check(status, what):
 
 
 def gfx950_pack(weight_format, outputs, inputs, stored):
-    """A matrix of the reference's E2M1_SCALED / E4M3_SCALED bytes in gfx950's lane order (weight_format names the GFX950
-    format): the library's load-time re-lay-out, weight_format_gfx950_pack."""
+    """A matrix of the reference's E2M1_SCALED / E4M3_SCALED bytes (or of E4M3_BLOCK128's) in gfx950's lane order
+    (weight_format names the GFX950 format): the library's load-time re-lay-out, weight_format_gfx950_pack."""
     stored = np.ascontiguousarray(stored, dtype=np.uint8)
     packed = np.empty_like(stored)
-    shape = Shape(outputs, inputs, 8 if weight_format == WEIGHT_FORMAT_E4M3_GFX950 else 4, 0)
+    shape = Shape(outputs, inputs, 4 if weight_format == WEIGHT_FORMAT_E2M1_GFX950 else 8, 0)
     check(library().weight_format_gfx950_pack(weight_format, C.byref(shape), stored.ctypes.data, stored.nbytes, packed.ctypes.data, packed.nbytes),
           "weight_format_gfx950_pack")
     return packed
@@ -390,7 +392,7 @@ def gfx950_pack(weight_format, outputs, inputs, stored):
 def gfx950_unpack(weight_format, outputs, inputs, packed):
     packed = np.ascontiguousarray(packed, dtype=np.uint8)
     stored = np.empty_like(packed)
-    shape = Shape(outputs, inputs, 8 if weight_format == WEIGHT_FORMAT_E4M3_GFX950 else 4, 0)
+    shape = Shape(outputs, inputs, 4 if weight_format == WEIGHT_FORMAT_E2M1_GFX950 else 8, 0)
     check(library().weight_format_gfx950_unpack(weight_format, C.byref(shape), packed.ctypes.data, packed.nbytes, stored.ctypes.data, stored.nbytes),
           "weight_format_gfx950_unpack")
     return stored
@@ -814,9 +816,9 @@ class Exl3Layer:
 
 class Fp4Layer:
     """One MoE layer of the original FP4 weights (WEIGHT_FORMAT_E2M1_SCALED; or, with weight_format, of FP8 weights,
-    WEIGHT_FORMAT_E4M3_SCALED; stored bytes as the reference's packs hold them; with WEIGHT_FORMAT_E2M1_GFX950 or
-    WEIGHT_FORMAT_E4M3_GFX950 the matrices, given in the reference's bytes, go through the library's load-time re-lay-out
-    first) in a card's arena, with the scratch ranges of a step of at most `rows` rows: the quantizer of the rows,
+    WEIGHT_FORMAT_E4M3_SCALED; stored bytes as the reference's packs hold them; with WEIGHT_FORMAT_E2M1_GFX950,
+    WEIGHT_FORMAT_E4M3_GFX950 or WEIGHT_FORMAT_E4M3_BLOCK128_GFX950 the matrices, given in the reference's bytes (in
+    E4M3_BLOCK128's for the last), go through the library's load-time re-lay-out first) in a card's arena, with the scratch ranges of a step of at most `rows` rows: the quantizer of the rows,
     the router's select, and the four launches of the routed experts."""
 
     def __init__(self, card, hidden, inner, expert_count, picks, rows, matrices, router_weights_bf16=None,
@@ -824,8 +826,8 @@ class Fp4Layer:
                  weight_format=WEIGHT_FORMAT_E2M1_SCALED):
         self.card, self.H, self.I, self.E, self.P, self.rows = card, hidden, inner, expert_count, picks, rows
         self.weight_format = weight_format
-        self.bits = 8 if weight_format in (WEIGHT_FORMAT_E4M3_SCALED, WEIGHT_FORMAT_E4M3_BLOCK128, WEIGHT_FORMAT_E4M3_GFX950) else 4
-        self.native = weight_format in (WEIGHT_FORMAT_E2M1_GFX950, WEIGHT_FORMAT_E4M3_GFX950)
+        self.bits = 4 if weight_format in (WEIGHT_FORMAT_E2M1_SCALED, WEIGHT_FORMAT_E2M1_GFX950) else 8
+        self.native = weight_format in (WEIGHT_FORMAT_E2M1_GFX950, WEIGHT_FORMAT_E4M3_GFX950, WEIGHT_FORMAT_E4M3_BLOCK128_GFX950)
         if self.native:  # a matrix that lies at several experts' places is packed once
             packed = {}
             for trio in matrices:
@@ -833,7 +835,7 @@ class Fp4Layer:
                     if id(matrix) not in packed:
                         packed[id(matrix)] = gfx950_pack(weight_format, *((inner, hidden) if m < 2 else (hidden, inner)), matrix)
             matrices = [[packed[id(matrix)] for matrix in trio] for trio in matrices]
-        self.block128 = weight_format == WEIGHT_FORMAT_E4M3_BLOCK128
+        self.block128 = weight_format in (WEIGHT_FORMAT_E4M3_BLOCK128, WEIGHT_FORMAT_E4M3_BLOCK128_GFX950)
         self.limit, self.affinity_kind, self.route_scale = limit, affinity_kind, route_scale
         self.gate_up_slices, self.down_slices = gate_up_slices, down_slices
         self.pairs = rows * picks
@@ -939,7 +941,7 @@ class Fp4Layer:
                 self.native_kernels = LinearNativeKernels()
                 check(self.card.lib.linear_native_kernels_prepare(backend_table(), self.card.handle, ARITHMETIC_CLASS_GFX950,
                                                                   C.byref(self.native_kernels)), "linear_native_kernels_prepare")
-            launches = launches_of(3)
+            launches = launches_of(4 if self.block128 else 3)
             check(self.card.lib.linear_native_experts_prepare(C.byref(d), self.card.arena_bytes, C.byref(self.kernels), C.byref(self.native_kernels),
                                                               launches), "linear_native_experts_prepare")
             return launches

@@ -257,8 +257,8 @@ __device__ static __forceinline__ void expert_down(const struct expert_down_argu
  * trunk alone: no counterpart among its expert kernels); same records, same rounding points. The _b128_ entries take
  * WEIGHT_FORMAT_E4M3_BLOCK128 experts (E4M3 codes with one float32 scale for every 128 x 128 block, vectors quantized a
  * 128 values with float32 scales, read where the records name the exponents: no counterpart in the reference). The
- * _gfx950_ entries take experts stored in the card's own lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950: no
- * counterpart in the reference) and give the sums of the same matrices in the reference's lay-out, bit for bit. */
+ * _gfx950_ entries take experts stored in the card's own lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950,
+ * _E4M3_BLOCK128_GFX950: no counterpart in the reference) and give the sums of the same matrices in the reference's lay-out, bit for bit. */
 #define EXPERT_ENTRIES(S)                                                                                         \
     extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
         expert_gate_up_##S(struct expert_gate_up_arguments arguments, unsigned char *arena)                      \
@@ -331,7 +331,19 @@ __device__ static __forceinline__ void expert_down(const struct expert_down_argu
     {                                                                                                             \
         expert_down<S, true, false, true>(arguments, arena);                                                      \
     }                                                                                                             \
-    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_e4m3_gfx950_##S, expert_down_arguments)
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_e4m3_gfx950_##S, expert_down_arguments);                \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_gate_up_b128_gfx950_##S(struct expert_gate_up_arguments arguments, unsigned char *arena)          \
+    {                                                                                                             \
+        expert_gate_up<S, true, true, true>(arguments, arena);                                                    \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_gate_up_b128_gfx950_##S, expert_gate_up_arguments);          \
+    extern "C" __global__ void __launch_bounds__(S * WAVE)                                                        \
+        expert_down_b128_gfx950_##S(struct expert_down_arguments arguments, unsigned char *arena)                \
+    {                                                                                                             \
+        expert_down<S, true, true, true>(arguments, arena);                                                       \
+    }                                                                                                             \
+    ANEMONE_KERNEL(KERNEL_FILE_EXPERT_LINEAR, expert_down_b128_gfx950_##S, expert_down_arguments)
 EXPERT_ENTRIES(1);
 EXPERT_ENTRIES(2);
 EXPERT_ENTRIES(4);

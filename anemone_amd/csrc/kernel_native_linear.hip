@@ -111,18 +111,25 @@ __device__ static __forceinline__ void native_vectors_of(const struct wide_pair 
 
 /* grid (ceil(output_size / (4 strips)), tile_count), block 256; a strip is STRIP tiles of gate and STRIP of up */
 /* sets of weight registers and stages of columns: 4-bit weights 3 and 2 (156 registers: three wavefronts a SIMD; with a
- * third stage 177, and two wavefronts measured 8 % slower, held to 168 by spills 38 % slower); one-byte weights 4 and 3
- * (6 and 3 measured the same) */
-template <bool BYTES>
+ * third stage 177, and two wavefronts measured 8 % slower, held to 168 by spills 38 % slower); one-byte weights 3 and 3
+ * (150 registers; 4 and 3, at 168, and 6 and 3 measured the same) */
+/* float32 block scales: a step's products start from zero and are added times the scales, which takes registers the
+ * E8M0 forms leave free. Three sets of weight registers for either product; gate/up two wavefronts a SIMD (901 us a
+ * launch of 2048 tokens, against 915 to 940 with four sets, and 1065 with four sets held to 168 registers by spills),
+ * down three (459 us, against 484 at two wavefronts and 529 with four sets) */
+#define NATIVE_B128_SLOTS 3u
+#define NATIVE_B128_GATE_UP_WAVES 2
+#define NATIVE_B128_DOWN_WAVES 2
+template <bool BYTES, bool B128 = false>
 struct native_depths {
-    static constexpr uint32_t SLOTS = BYTES ? 4u : 3u, DEPTH = BYTES ? NATIVE_E4M3_STAGES : NATIVE_E2M1_STAGES;
+    static constexpr uint32_t SLOTS = 3u, DEPTH = BYTES ? NATIVE_E4M3_STAGES : NATIVE_E2M1_STAGES;
 };
 
-template <bool BYTES, uint32_t STRIP, uint32_t GROUP>
+template <bool BYTES, uint32_t STRIP, uint32_t GROUP, bool B128 = false>
 __device__ static __forceinline__ void native_expert_gate_up(const struct wide_expert_gate_up_arguments &arguments, unsigned char *arena)
 {
     constexpr uint32_t COLUMN_BLOCKS = 4u * GROUP;
-    typedef native_chain<2, BYTES, STRIP, COLUMN_BLOCKS, native_depths<BYTES>::SLOTS, native_depths<BYTES>::DEPTH> chain_type;
+    typedef native_chain<2, BYTES, STRIP, COLUMN_BLOCKS, native_depths<BYTES, B128>::SLOTS, native_depths<BYTES, B128>::DEPTH, B128> chain_type;
     constexpr uint32_t TILES = chain_type::TILES;
     static_assert(STRIP == 1u || STRIP == 2u, "a quantizer block of 32 outputs is one strip or two");
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
@@ -150,14 +157,14 @@ __device__ static __forceinline__ void native_expert_gate_up(const struct wide_e
         }
     }
     chain_of.whole(arguments.input_size / 128u, (pair_count + 15u) / 16u, chain);
-    wide_gate_up_finish<STRIP, COLUMN_BLOCKS, false>(arguments, arena, window, pairs, pair_count, block_strip, tile0, wave, lane, chain);
+    wide_gate_up_finish<STRIP, COLUMN_BLOCKS, B128>(arguments, arena, window, pairs, pair_count, block_strip, tile0, wave, lane, chain);
 }
 
-template <bool BYTES, uint32_t GROUP>
+template <bool BYTES, uint32_t GROUP, bool B128 = false>
 __device__ static __forceinline__ void native_expert_down(const struct wide_expert_down_arguments &arguments, unsigned char *arena)
 {
     constexpr uint32_t COLUMN_BLOCKS = 4u * GROUP;
-    typedef native_chain<1, BYTES, (BYTES ? 2u : 4u), COLUMN_BLOCKS, native_depths<BYTES>::SLOTS, native_depths<BYTES>::DEPTH> chain_type;
+    typedef native_chain<1, BYTES, (BYTES ? 2u : 4u), COLUMN_BLOCKS, native_depths<BYTES, B128>::SLOTS, native_depths<BYTES, B128>::DEPTH, B128> chain_type;
     constexpr uint32_t TILES = chain_type::TILES, STRIP = chain_type::STRIP;
     extern __shared__ __attribute__((aligned(16))) unsigned char window[];
     const uint32_t lane = threadIdx.x % WAVE, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
@@ -200,7 +207,7 @@ extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E2M1_WAVES) 
     native_expert_down<false, NATIVE_E2M1_COLUMN_BLOCKS / 4u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_down_1, wide_expert_down_arguments);
-#define NATIVE_E4M3_WAVES 3 /* 168 registers (the down launch took 170 left to itself, and two wavefronts a SIMD: 487 against 461 us) */
+#define NATIVE_E4M3_WAVES 3 /* 150 and 152 registers (with four sets of weight registers the down launch took 170 left to itself, and at two wavefronts a SIMD 487 against 461 us) */
 extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E4M3_WAVES) native_expert_gate_up_e4m3_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
 {
     native_expert_gate_up<true, 1u, NATIVE_E4M3_COLUMN_BLOCKS / 4u>(arguments, arena);
@@ -211,6 +218,20 @@ extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_E4M3_WAVES) 
     native_expert_down<true, NATIVE_E4M3_COLUMN_BLOCKS / 4u>(arguments, arena);
 }
 ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_down_e4m3_1, wide_expert_down_arguments);
+
+/* E4M3_BLOCK128_GFX950 experts (float32 scales of 128 x 128 blocks, columns of 128-value float32 scales): the E4M3_GFX950
+ * launches' shape; the gate/up launch leaves the hidden VALUES where the record names the hidden operands, and their
+ * quantizer (activation_quantize_128_entry) is a launch of its own */
+extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_B128_GATE_UP_WAVES) native_expert_gate_up_b128_1(struct wide_expert_gate_up_arguments arguments, unsigned char *arena)
+{
+    native_expert_gate_up<true, 1u, NATIVE_E4M3_COLUMN_BLOCKS / 4u, true>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_gate_up_b128_1, wide_expert_gate_up_arguments);
+extern "C" __global__ void __launch_bounds__(NATIVE_THREADS, NATIVE_B128_DOWN_WAVES) native_expert_down_b128_1(struct wide_expert_down_arguments arguments, unsigned char *arena)
+{
+    native_expert_down<true, NATIVE_E4M3_COLUMN_BLOCKS / 4u, true>(arguments, arena);
+}
+ANEMONE_KERNEL(KERNEL_FILE_NATIVE_LINEAR, native_expert_down_b128_1, wide_expert_down_arguments);
 
 static_assert(native_chain<2, false, 2u, NATIVE_E2M1_COLUMN_BLOCKS, 3u, NATIVE_E2M1_STAGES>::WINDOW_BYTES == NATIVE_WINDOW_BYTES(NATIVE_E2M1_COLUMN_BLOCKS, NATIVE_E2M1_STAGES) &&
                   native_chain<1, true, 2u, NATIVE_E4M3_COLUMN_BLOCKS, 4u, NATIVE_E4M3_STAGES>::WINDOW_BYTES == NATIVE_WINDOW_BYTES(NATIVE_E4M3_COLUMN_BLOCKS, NATIVE_E4M3_STAGES),

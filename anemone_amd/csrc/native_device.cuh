@@ -24,7 +24,9 @@
 
 /* memory into registers, 16 bytes or one byte a lane: the address is a base common to the wavefront plus the lane's own
  * byte offset (plus 1,024: the second half of a tile of one-byte weights). Assembly, like the loads into LDS beside which
- * they are counted: the compiler keeps no book on them, native_landed is the wait. ONCE: the bytes are read by this
+ * they are counted: the compiler keeps no book on them, native_landed is the wait (so a kernel of these loads must spill
+ * no vector register: one saved between its load and the wait is saved before it is filled, and the build refuses such
+ * a kernel). ONCE: the bytes are read by this
  * block alone (an expert's one-byte weights in a block that holds all its pairs): asked for as a stream, so that they do
  * not push the columns, which every block of the expert reads, out of the level-2 cache. */
 template <bool ONCE>
@@ -71,8 +73,13 @@ __device__ static __forceinline__ void native_landed(uint32_t &value)
 
 /* SLOTS: sets of weight registers a wavefront keeps (the weights of SLOTS - 1 steps are on their way while one is
  * multiplied); DEPTH: stages of columns in LDS, likewise */
-template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES, uint32_t COLUMN_BLOCKS, uint32_t SLOTS, uint32_t DEPTH>
+/* B128 (one-byte weights alone): float32 scales, one for every 128 outputs x 128 inputs of a matrix and one for every 128
+ * values of a column, in place of the E8M0 codes (the same bytes a K step: a word where four codes were): a K step's
+ * matrix instruction runs from zero with scale codes of one and its sums enter the chain by one fused multiply-add with
+ * the product of the two scales, as the reference-order kernels of that scaling add them */
+template <uint32_t MATRICES, bool BYTES, uint32_t STRIP_TILES, uint32_t COLUMN_BLOCKS, uint32_t SLOTS, uint32_t DEPTH, bool B128 = false>
 struct native_chain {
+    static_assert(BYTES || !B128, "float32 scales go with one-byte weights");
     static_assert(COLUMN_BLOCKS == 4u || COLUMN_BLOCKS == 8u, "a wavefront brings one or two column blocks");
     static constexpr uint32_t STRIP = STRIP_TILES;
     static constexpr uint32_t TILES = MATRICES * STRIP;
@@ -86,7 +93,7 @@ struct native_chain {
     /* scale codes: of one-byte weights a byte a lane a tile (a row of 32 outputs' codes, as the reference stores them); of
      * 4-bit weights a word a lane a matrix: its bytes are the codes of the lane's row and inputs in the four tiles of a group
      * of 64 outputs, which the matrix instruction picks by number */
-    static constexpr uint32_t SCALE_LOADS = BYTES ? TILES : MATRICES;
+    static constexpr uint32_t SCALE_LOADS = BYTES && !B128 ? TILES : MATRICES;
     static constexpr uint32_t WEIGHT_LOADS = TILES * HALVES + SCALE_LOADS;
     static_assert(BYTES || STRIP == 2u || STRIP == 4u, "a strip of 4-bit weights is half a group of four tiles, or a whole one");
     static_assert((DEPTH - 1u) * VECTOR_LOADS + (SLOTS - 1u) * WEIGHT_LOADS < 64u, "vmcnt has six bits");
@@ -147,12 +154,12 @@ struct native_chain {
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
             const unsigned char *step_scales = scales[m] + (uint64_t)at * (BYTES ? 4u : 256u);
-            if constexpr (BYTES) {
+            if constexpr (BYTES && !B128) {
 #pragma unroll
                 for (uint32_t n = 0; n < STRIP; n++) {
                     load_1(into.scale[m * STRIP + n], step_scales, scale_offset[n]);
                 }
-            } else {
+            } else { /* a word a lane of a group of four tiles' codes, or the strip's one float32 scale in every lane */
                 load_4(into.scale[m], step_scales, scale_offset[0]);
             }
         }
@@ -208,7 +215,16 @@ struct native_chain {
     __device__ static __forceinline__ void multiply_tiles(const slot &set, const uint32_t (&scale_a)[SCALE_LOADS], const int8_vector &b,
                                                           uint32_t scale_b, uint32_t j, float4_t (&chain)[TILES][COLUMN_BLOCKS])
     {
-        if constexpr (BYTES) {
+        if constexpr (B128) {
+            const uint4_t first = set.words[T][0], second = set.words[T][HALVES - 1u];
+            const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
+            const float scale = __fmul_rn(__uint_as_float(scale_a[T / STRIP]), __uint_as_float(scale_b));
+            const float4_t step = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, (float4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0, 127, 0, 127);
+#pragma unroll
+            for (uint32_t v = 0; v < 4u; v++) {
+                chain[T][j][v] = __fmaf_rn(step[v], scale, chain[T][j][v]);
+            }
+        } else if constexpr (BYTES) {
             const uint4_t first = set.words[T][0], second = set.words[T][HALVES - 1u];
             const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
             chain[T][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, chain[T][j], 0, 0, 0, (int)scale_a[T], 0, (int)scale_b);
@@ -239,7 +255,7 @@ struct native_chain {
         __builtin_amdgcn_s_setprio(1);
         /* a column block's operand is read while the block before it is multiplied: two blocks' registers, not LIVE */
         uint4_t low = lds_read<uint4_t>(b_at), high = lds_read<uint4_t>(b_at + 1024u);
-        uint32_t scale_b = lds_read<unsigned char>(b_scale_at);
+        uint32_t scale_b = B128 ? lds_read<uint32_t>(b_scale_at) : lds_read<unsigned char>(b_scale_at); /* a code, or a float32's bits */
 #pragma unroll
         for (uint32_t j = 0; j < LIVE; j++) {
             const int8_vector b = {(int)low.x, (int)low.y, (int)low.z, (int)low.w, (int)high.x, (int)high.y, (int)high.z, (int)high.w};
@@ -248,7 +264,7 @@ struct native_chain {
             if (j + 1u < LIVE) {
                 low = lds_read<uint4_t>(b_at + (j + 1u) * 2048u);
                 high = lds_read<uint4_t>(b_at + (j + 1u) * 2048u + 1024u);
-                scale_b = lds_read<unsigned char>(b_scale_at + (j + 1u) * 64u);
+                scale_b = B128 ? lds_read<uint32_t>(b_scale_at + (j + 1u) * 64u) : lds_read<unsigned char>(b_scale_at + (j + 1u) * 64u);
             }
             multiply_tiles<0>(set, scale_a, b, scale_now, j, chain);
             if (j == (LIVE - 1u) / 2u) {
@@ -427,7 +443,9 @@ struct native_chain {
 #pragma unroll
         for (uint32_t m = 0; m < MATRICES; m++) {
             words[m] = matrices[m] + (uint64_t)tile0 * tile_bytes;
-            if constexpr (BYTES) { /* the scale codes as the reference stores them: a row of inputs / 32 bytes for every 32 outputs */
+            if constexpr (B128) { /* float32 [outputs / 128][inputs / 128] behind the codes: the strip's row, a word a K step */
+                scales[m] = matrices[m] + (uint64_t)outputs * inputs + (uint64_t)(tile0 / 8u) * (inputs / 32u);
+            } else if constexpr (BYTES) { /* the scale codes as the reference stores them: a row of inputs / 32 bytes for every 32 outputs */
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs + (uint64_t)(tile0 / 2u) * (inputs / 32u);
             } else { /* a word a lane a K step of a group of four tiles */
                 scales[m] = matrices[m] + (uint64_t)outputs * inputs / 2u + (uint64_t)(tile0 / 4u) * steps * 256u;
@@ -436,7 +454,7 @@ struct native_chain {
 #pragma unroll
         for (uint32_t n = 0; n < STRIP; n++) {
             word_offset[n] = n * tile_bytes + 16u * lane;
-            scale_offset[n] = BYTES ? ((tile0 + n) / 2u - tile0 / 2u) * (inputs / 32u) + g : 4u * lane;
+            scale_offset[n] = B128 ? 0u : BYTES ? ((tile0 + n) / 2u - tile0 / 2u) * (inputs / 32u) + g : 4u * lane;
         }
 #pragma unroll
         for (uint32_t i = 0; i < WAVE_BLOCKS; i++) {
@@ -460,7 +478,7 @@ struct native_chain {
                 vector_at[part] = group_bytes + 16u * (8u * column + (piece ^ column ^ (o / 8u))) + 8u * (g / 2u);
             }
         }
-        vector_scale_at = 4u * o + g;
+        vector_scale_at = B128 ? 4u * o : 4u * o + g;
         operand_at = 16u * lane;
         scale_shift = 8u * (tile0 % 4u);
     }

@@ -20,11 +20,11 @@
 /* NATIVE: the matrices are stored in gfx950's lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950): a lane's 16 bytes of
  * a tile's K step (and, of one-byte weights, the 16 bytes 1,024 further) are its A operand as they lie, so a stage's
  * tiles are read with one or two 16-byte LDS reads and no arithmetic; the scale codes of 4-bit weights are a word a lane
- * for the strip's four tiles (a group of 64 outputs), its byte picked by the matrix instruction. */
+ * for the strip's four tiles (a group of 64 outputs), its byte picked by the matrix instruction; with B128 the scales are
+ * E4M3_BLOCK128's float32 words where they are. */
 template <uint32_t MATRICES, bool BYTES, bool B128 = false, bool NATIVE = false>
 struct strip_chain {
     static_assert(BYTES || !B128, "float32 scales go with one-byte weights");
-    static_assert(!NATIVE || !B128, "gfx950's lane order is built for the formats of E8M0 scale codes");
     static constexpr uint32_t STRIP = BYTES ? 2u : 4u; /* tiles of a strip: 4 KB of every matrix a stage either way */
     static constexpr uint32_t STEP_BYTES = BYTES ? BYTE_STEP_BYTES : NIBBLE_STEP_BYTES;
     static constexpr uint32_t TILE_LOADS = STEP_BYTES / 1024u; /* 16-byte-a-lane loads of a tile's step */
@@ -89,7 +89,16 @@ struct strip_chain {
     __device__ __forceinline__ void native_tiles(uint32_t base, const int8_vector &b, uint32_t scale_b, float4_t (&chain)[TILES]) const
     {
         const uint4_t first = lds_read<uint4_t>(base + T * STEP_BYTES + piece_offset);
-        if constexpr (BYTES) {
+        if constexpr (B128) { /* scale_b: the bits of the column's float32 scale */
+            const uint4_t second = lds_read<uint4_t>(base + T * STEP_BYTES + 1024u + piece_offset);
+            const float scale = __fmul_rn(lds_read<float>(base + SCALES_AT + (T / STRIP) * 256u), __uint_as_float(scale_b));
+            const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
+            const float4_t step = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, (float4_t){0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0, 127, 0, 127);
+#pragma unroll
+            for (uint32_t v = 0; v < 4u; v++) {
+                chain[T][v] = __fmaf_rn(step[v], scale, chain[T][v]);
+            }
+        } else if constexpr (BYTES) {
             const uint4_t second = lds_read<uint4_t>(base + T * STEP_BYTES + 1024u + piece_offset);
             const uint32_t scale_a = lds_read<unsigned char>(base + SCALES_AT + (T / STRIP) * 256u + scale_at[T % STRIP]);
             const int8_vector a = {(int)first.x, (int)first.y, (int)first.z, (int)first.w, (int)second.x, (int)second.y, (int)second.z, (int)second.w};
@@ -129,7 +138,7 @@ struct strip_chain {
             scale_b = lds_read<unsigned char>(base + VECTOR_SCALE_AT + vector_scale_at);
         }
         if constexpr (NATIVE) {
-            native_tiles<0>(base, b, scale_b, chain);
+            native_tiles<0>(base, b, B128 ? __float_as_uint(float_scale_b) : scale_b, chain);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             return;
         }

@@ -100,6 +100,8 @@ result_status linear_kernels_prepare(const struct backend_operations *backend, s
             {KERNEL_EXPERT_DOWN_STEM, "gfx950_", sizeof(struct expert_down_arguments), &kernels.expert_down_gfx950[instance]},
             {KERNEL_EXPERT_GATE_UP_STEM, "e4m3_gfx950_", sizeof(struct expert_gate_up_arguments), &kernels.expert_gate_up_e4m3_gfx950[instance]},
             {KERNEL_EXPERT_DOWN_STEM, "e4m3_gfx950_", sizeof(struct expert_down_arguments), &kernels.expert_down_e4m3_gfx950[instance]},
+            {KERNEL_EXPERT_GATE_UP_STEM, "b128_gfx950_", sizeof(struct expert_gate_up_arguments), &kernels.expert_gate_up_b128_gfx950[instance]},
+            {KERNEL_EXPERT_DOWN_STEM, "b128_gfx950_", sizeof(struct expert_down_arguments), &kernels.expert_down_b128_gfx950[instance]},
         };
         for (uint32_t k = 0; status == STATUS_OK && k < sizeof native / sizeof native[0]; k++) {
             char name[56];
@@ -247,8 +249,9 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
     const struct weight_format_operations *format = weight_format_operations_of(description->weight_format);
     uint64_t gate_up_bytes = 0, down_bytes = 0;
     uint32_t gate_up_instance = 0, down_instance = 0;
-    const bool block128 = description->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128;
-    const bool native = description->weight_format == WEIGHT_FORMAT_E2M1_GFX950 || description->weight_format == WEIGHT_FORMAT_E4M3_GFX950;
+    const bool block128 = description->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128 || description->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128_GFX950;
+    const bool native = description->weight_format == WEIGHT_FORMAT_E2M1_GFX950 || description->weight_format == WEIGHT_FORMAT_E4M3_GFX950 ||
+                        description->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128_GFX950;
     const bool bytes = description->weight_format == WEIGHT_FORMAT_E4M3_SCALED || description->weight_format == WEIGHT_FORMAT_E4M3_GFX950 || block128;
     const bool nibbles = description->weight_format == WEIGHT_FORMAT_E2M1_SCALED || description->weight_format == WEIGHT_FORMAT_E2M1_GFX950;
     const uint32_t strip_outputs = bytes ? LINEAR_STRIP_OUTPUTS / 2u : LINEAR_STRIP_OUTPUTS;
@@ -257,9 +260,9 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
         format->stored_byte_count(down, &down_bytes) != STATUS_OK || gate_up->input_size % 128u != 0 ||
         down->input_size % 128u != 0 || down->input_size != gate_up->output_size ||
         gate_up->output_size < strip_outputs || down->output_size < strip_outputs) {
-        REFUSE("%s: matrices of format %u, %u, %u, %u or %u in shapes it stores, inputs a multiple of 128, at least %u outputs, down "
+        REFUSE("%s: matrices of format %u, %u or %u to %u in shapes it stores, inputs a multiple of 128, at least %u outputs, down "
                "reading what gate and up write", what, (uint32_t)WEIGHT_FORMAT_E2M1_SCALED, (uint32_t)WEIGHT_FORMAT_E4M3_SCALED,
-               (uint32_t)WEIGHT_FORMAT_E4M3_BLOCK128, (uint32_t)WEIGHT_FORMAT_E2M1_GFX950, (uint32_t)WEIGHT_FORMAT_E4M3_GFX950, strip_outputs);
+               (uint32_t)WEIGHT_FORMAT_E4M3_BLOCK128, (uint32_t)WEIGHT_FORMAT_E4M3_BLOCK128_GFX950, strip_outputs);
         return STATUS_INVALID_ARGUMENT;
     }
     if (!instance_of(description->gate_up_slice_count, gate_up->input_size, &gate_up_instance) ||
@@ -268,12 +271,14 @@ result_status linear_routed_experts_prepare(const struct linear_routed_experts_d
                description->gate_up_slice_count, description->down_slice_count);
         return STATUS_INVALID_ARGUMENT;
     }
-    const uint32_t *const gate_up_family = block128          ? kernels->expert_gate_up_b128
+    const uint32_t *const gate_up_family = block128 && native ? kernels->expert_gate_up_b128_gfx950
+                                           : block128        ? kernels->expert_gate_up_b128
                                            : native && bytes ? kernels->expert_gate_up_e4m3_gfx950
                                            : native          ? kernels->expert_gate_up_gfx950
                                            : bytes           ? kernels->expert_gate_up_e4m3
                                                              : kernels->expert_gate_up;
-    const uint32_t *const down_family = block128          ? kernels->expert_down_b128
+    const uint32_t *const down_family = block128 && native ? kernels->expert_down_b128_gfx950
+                                        : block128        ? kernels->expert_down_b128
                                         : native && bytes ? kernels->expert_down_e4m3_gfx950
                                         : native          ? kernels->expert_down_gfx950
                                         : bytes           ? kernels->expert_down_e4m3
@@ -601,7 +606,7 @@ static result_status wide_experts_prepare(const struct linear_wide_experts_descr
     const struct linear_routed_experts_description *experts = &description->experts;
     const struct matrix_shape_record *gate_up = &experts->gate_up_shape, *down = &experts->down_shape;
     const struct weight_format_operations *format = weight_format_operations_of(experts->weight_format);
-    if (block128 != (experts->weight_format == WEIGHT_FORMAT_E4M3_BLOCK128)) {
+    if (block128 != (experts->weight_format == (native ? WEIGHT_FORMAT_E4M3_BLOCK128_GFX950 : WEIGHT_FORMAT_E4M3_BLOCK128))) {
         REFUSE("%s: a weight format of %u", what, (uint32_t)experts->weight_format);
         return STATUS_INVALID_ARGUMENT;
     }
@@ -626,8 +631,10 @@ static result_status wide_experts_prepare(const struct linear_wide_experts_descr
     }
     uint32_t gate_up_kernel, down_kernel, gate_up_window, down_window;
     if (native) {
-        gate_up_kernel = bytes ? native_kernels->native_expert_gate_up_e4m3 : native_kernels->native_expert_gate_up;
-        down_kernel = bytes ? native_kernels->native_expert_down_e4m3 : native_kernels->native_expert_down;
+        gate_up_kernel = block128 ? native_kernels->native_expert_gate_up_b128
+                         : bytes  ? native_kernels->native_expert_gate_up_e4m3
+                                  : native_kernels->native_expert_gate_up;
+        down_kernel = block128 ? native_kernels->native_expert_down_b128 : bytes ? native_kernels->native_expert_down_e4m3 : native_kernels->native_expert_down;
         gate_up_window = down_window = bytes ? NATIVE_WINDOW_BYTES(NATIVE_E4M3_COLUMN_BLOCKS, NATIVE_E4M3_STAGES)
                                              : NATIVE_WINDOW_BYTES(NATIVE_E2M1_COLUMN_BLOCKS, NATIVE_E2M1_STAGES);
     } else {
@@ -725,13 +732,15 @@ result_status linear_native_kernels_prepare(const struct backend_operations *bac
     static const struct {
         const char *name;
         uint32_t record_bytes;
-    } wanted[4] = {{KERNEL_NATIVE_EXPERT_GATE_UP_STEM "1", sizeof(struct wide_expert_gate_up_arguments)},
+    } wanted[6] = {{KERNEL_NATIVE_EXPERT_GATE_UP_STEM "1", sizeof(struct wide_expert_gate_up_arguments)},
                    {KERNEL_NATIVE_EXPERT_DOWN_STEM "1", sizeof(struct wide_expert_down_arguments)},
                    {KERNEL_NATIVE_EXPERT_GATE_UP_STEM "e4m3_1", sizeof(struct wide_expert_gate_up_arguments)},
-                   {KERNEL_NATIVE_EXPERT_DOWN_STEM "e4m3_1", sizeof(struct wide_expert_down_arguments)}};
-    uint32_t handles[4];
+                   {KERNEL_NATIVE_EXPERT_DOWN_STEM "e4m3_1", sizeof(struct wide_expert_down_arguments)},
+                   {KERNEL_NATIVE_EXPERT_GATE_UP_STEM "b128_1", sizeof(struct wide_expert_gate_up_arguments)},
+                   {KERNEL_NATIVE_EXPERT_DOWN_STEM "b128_1", sizeof(struct wide_expert_down_arguments)}};
+    uint32_t handles[6];
     _Static_assert(sizeof(struct linear_native_kernels_record) == sizeof handles, "a handle a member, in the members' order");
-    for (uint32_t i = 0; i < 4u; i++) {
+    for (uint32_t i = 0; i < 6u; i++) {
         const result_status status = backend->kernel_prepare(card, KERNEL_FILE_NATIVE_LINEAR, wanted[i].name, wanted[i].record_bytes, &handles[i]);
         if (status != STATUS_OK) {
             REFUSE("linear_native_kernels_prepare: %s: %s", wanted[i].name, status_text(status));
@@ -750,5 +759,6 @@ result_status linear_native_experts_prepare(const struct linear_wide_experts_des
         REFUSE("linear_native_experts_prepare: the native kernels' record is needed");
         return STATUS_INVALID_ARGUMENT;
     }
-    return wide_experts_prepare(description, arena_byte_count, linear_kernels, NULL, kernels, false, launches_out);
+    const bool block128 = description != NULL && description->experts.weight_format == WEIGHT_FORMAT_E4M3_BLOCK128_GFX950;
+    return wide_experts_prepare(description, arena_byte_count, linear_kernels, NULL, kernels, block128, launches_out);
 }

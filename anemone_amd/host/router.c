@@ -169,7 +169,8 @@ result_status router_select_prepare(const struct router_description *description
         experts->job_count != experts->row_count * P ||
         (experts->weight_format != WEIGHT_FORMAT_E2M1_SCALED && experts->weight_format != WEIGHT_FORMAT_E4M3_SCALED &&
          experts->weight_format != WEIGHT_FORMAT_EXL3 && experts->weight_format != WEIGHT_FORMAT_E4M3_BLOCK128 &&
-         experts->weight_format != WEIGHT_FORMAT_E2M1_GFX950 && experts->weight_format != WEIGHT_FORMAT_E4M3_GFX950) ||
+         experts->weight_format != WEIGHT_FORMAT_E2M1_GFX950 && experts->weight_format != WEIGHT_FORMAT_E4M3_GFX950 &&
+         experts->weight_format != WEIGHT_FORMAT_E4M3_BLOCK128_GFX950) ||
         !(description->route_scale > 0.0f)) {
         REFUSE("%s: the select writes 1 to %u rows of %u pairs, a job a pair, with a route scale above zero", what,
                LINEAR_MAXIMUM_ROWS, P);
@@ -293,7 +294,8 @@ static result_status wide_launches(const struct router_wide_description *descrip
     if (R == 0 || R > ROUTER_WIDE_MOST_ROWS || !(description->route_scale > 0.0f) ||
         (description->weight_format != WEIGHT_FORMAT_E2M1_SCALED && description->weight_format != WEIGHT_FORMAT_E4M3_SCALED &&
          description->weight_format != WEIGHT_FORMAT_EXL3 && description->weight_format != WEIGHT_FORMAT_E4M3_BLOCK128 &&
-         description->weight_format != WEIGHT_FORMAT_E2M1_GFX950 && description->weight_format != WEIGHT_FORMAT_E4M3_GFX950)) {
+         description->weight_format != WEIGHT_FORMAT_E2M1_GFX950 && description->weight_format != WEIGHT_FORMAT_E4M3_GFX950 &&
+         description->weight_format != WEIGHT_FORMAT_E4M3_BLOCK128_GFX950)) {
         REFUSE("%s: 1 to %u rows, a route scale above zero, experts of a format the path holds", what, ROUTER_WIDE_MOST_ROWS);
         return STATUS_INVALID_ARGUMENT;
     }

@@ -82,6 +82,7 @@ static const struct weight_format_operations e4m3_block128_operations = {"e4m3_b
 const struct weight_format_operations exl3_weight_operations = {"exl3", exl3_bytes};
 static const struct weight_format_operations e2m1_gfx950_operations = {"e2m1_gfx950", e2m1_gfx950_bytes};
 static const struct weight_format_operations e4m3_gfx950_operations = {"e4m3_gfx950", e4m3_gfx950_bytes};
+static const struct weight_format_operations e4m3_block128_gfx950_operations = {"e4m3_block128_gfx950", e4m3_block128_bytes}; /* whole blocks of 128 x 128 either way */
 
 const struct weight_format_operations *weight_format_operations_of(enum weight_format_code format)
 {
@@ -92,6 +93,7 @@ const struct weight_format_operations *weight_format_operations_of(enum weight_f
     case WEIGHT_FORMAT_E4M3_BLOCK128: return &e4m3_block128_operations;
     case WEIGHT_FORMAT_E2M1_GFX950: return &e2m1_gfx950_operations;
     case WEIGHT_FORMAT_E4M3_GFX950: return &e4m3_gfx950_operations;
+    case WEIGHT_FORMAT_E4M3_BLOCK128_GFX950: return &e4m3_block128_gfx950_operations;
     default: return NULL;
     }
 }
@@ -179,7 +181,7 @@ static void e2m1_from_gfx950(uint32_t outputs, uint32_t inputs, const unsigned c
 
 /* E4M3: byte c of word v of lane 16 g + o is byte 8 (g % 2) + 4 (c % 2) + 2 (c / 2) + o / 8 of the reference's lane
  * 4 (o % 8) + v % 4 of the group 4 step + 2 (v / 4) + g / 2; the scale codes stay where they are */
-static void e4m3_between(uint32_t outputs, uint32_t inputs, const unsigned char *from, unsigned char *to, bool to_gfx950)
+static void e4m3_between(uint32_t outputs, uint32_t inputs, const unsigned char *from, unsigned char *to, bool to_gfx950, uint64_t scale_bytes)
 {
     const uint32_t tiles = outputs / 16u, steps = inputs / 128u, groups = inputs / 32u;
     for (uint32_t tile = 0; tile < tiles; tile++) {
@@ -202,21 +204,23 @@ static void e4m3_between(uint32_t outputs, uint32_t inputs, const unsigned char 
         }
     }
     const uint64_t codes = (uint64_t)outputs * inputs;
-    memcpy(to + codes, from + codes, (size_t)((uint64_t)((outputs + 31u) / 32u) * groups));
+    memcpy(to + codes, from + codes, (size_t)scale_bytes); /* E8M0 rows or float32 blocks: where they are */
 }
 
 static result_status gfx950_move(enum weight_format_code format, const struct matrix_shape_record *shape, const void *from, uint64_t from_bytes,
                                  void *to, uint64_t to_bytes, bool to_gfx950)
 {
     const struct weight_format_operations *operations =
-        format == WEIGHT_FORMAT_E2M1_GFX950 || format == WEIGHT_FORMAT_E4M3_GFX950 ? weight_format_operations_of(format) : NULL;
+        format == WEIGHT_FORMAT_E2M1_GFX950 || format == WEIGHT_FORMAT_E4M3_GFX950 || format == WEIGHT_FORMAT_E4M3_BLOCK128_GFX950
+            ? weight_format_operations_of(format)
+            : NULL;
     uint64_t bytes = 0;
     if (operations == NULL || from == NULL || to == NULL || operations->stored_byte_count(shape, &bytes) != STATUS_OK || from_bytes != bytes ||
         to_bytes != bytes || !apart(from, from_bytes, to, to_bytes)) {
         return STATUS_INVALID_ARGUMENT; /* the _SCALED counterpart's byte count is the same for every shape both store */
     }
-    if (format == WEIGHT_FORMAT_E4M3_GFX950) {
-        e4m3_between(shape->output_size, shape->input_size, from, to, to_gfx950);
+    if (format == WEIGHT_FORMAT_E4M3_GFX950 || format == WEIGHT_FORMAT_E4M3_BLOCK128_GFX950) {
+        e4m3_between(shape->output_size, shape->input_size, from, to, to_gfx950, bytes - (uint64_t)shape->output_size * shape->input_size);
     } else if (to_gfx950) {
         e2m1_to_gfx950(shape->output_size, shape->input_size, from, to);
     } else {

@@ -40,6 +40,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("fp4_prefill_native", 8192): 5530.8e6 + 415.4e6,
     ("exl3_prefill", 4096): 2858.6e6 + 538.5e6,
     ("fp8_prefill_native", 2048): 4711.2e6 + 113.3e6,
+    ("fp8_prefill_block128_native", 2048): 4693.9e6 + 67.1e6,
     ("fp4_decode_native", 32): 1434.2e6 + 1.0e6,
     ("fp8_decode_native", 32): 2746.7e6 + 1.0e6,
 }
@@ -50,6 +51,7 @@ TRAFFIC_SOURCE = {
     "fp8_decode_block128": "profiles/expert_b128_fp8_block128_decode64_prefill2048.md",
     "fp8_prefill_block128": "profiles/expert_b128_fp8_block128_decode64_prefill2048.md",
     "fp4_prefill_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md", "fp8_prefill_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md",
+    "fp8_prefill_block128_native": "profiles/native_expert_b128_gfx950_prefill2048.md",
     "fp4_decode_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md", "fp8_decode_native": "profiles/native_expert_fp4_fp8_gfx950_lane_order.md",
 }
 HIDDEN, INNER, EXPERTS, PICKS, ROWS = 4096, 2048, 256, 8, 8
@@ -148,8 +150,6 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
     block128 = fp8 and arguments.block128  # float32 scales of 128 x 128 blocks and of 128 values (the usual FP8 block scaling)
     native = getattr(arguments, "native", False)  # the weights in gfx950's own lane order (a load-time re-lay-out of the same bytes)
-    if native and block128:
-        raise SystemExit("--native: the formats of the reference's scalings (E8M0 codes) have a gfx950 lane order")
     matrix = workloads.fp8_block128_matrix if block128 else workloads.fp8_matrix if fp8 else workloads.fp4_matrix
     trios = [[matrix(base + 16 + 3 * e + 0, INNER, HIDDEN), matrix(base + 16 + 3 * e + 1, INNER, HIDDEN),
               matrix(base + 16 + 3 * e + 2, HIDDEN, INNER)] for e in range(distinct_generated)]
@@ -159,7 +159,7 @@ def fp4_decode(amd, workloads, arguments, fp8=False, prefill=False):
     card = amd.Card(((9 if fp8 else 5) << 30) + rows * (1 << 18))
     layer = amd.Fp4Layer(card, HIDDEN, INNER, EXPERTS, PICKS, rows, matrices, router_weights_bf16=router,
                          gate_up_slices=arguments.gate_up_slices, down_slices=arguments.down_slices,
-                         weight_format=(amd.WEIGHT_FORMAT_E4M3_GFX950 if fp8 else amd.WEIGHT_FORMAT_E2M1_GFX950) if native else
+                         weight_format=(amd.WEIGHT_FORMAT_E4M3_BLOCK128_GFX950 if block128 else amd.WEIGHT_FORMAT_E4M3_GFX950 if fp8 else amd.WEIGHT_FORMAT_E2M1_GFX950) if native else
                          amd.WEIGHT_FORMAT_E4M3_BLOCK128 if block128 else amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED)
     layer.set_rows(x, rows)
     wide = layer.wide_router() if rows > 8 or prefill else None  # more than eight rows: the wide select sorts the pairs by expert
@@ -734,11 +734,12 @@ def summary(result):
 
 # the workloads of the other configurations the metric names, as the default run's config.also: (workload, rows, block128, gfx950 lane order)
 ALSO = [("exl3_linear", 1, False, False), ("exl3_prefill", 4096, False, False), ("fp8_decode", 1, True, False), ("fp8_decode", 64, True, False),
-        ("fp8_prefill", 2048, True, False), ("fp8_prefill", 2048, False, False), ("fp8_prefill", 2048, False, True),
+        ("fp8_prefill", 2048, True, False), ("fp8_prefill", 2048, True, True), ("fp8_prefill", 2048, False, False), ("fp8_prefill", 2048, False, True),
         ("fp4_prefill", 8192, False, False), ("fp4_prefill", 8192, False, True), ("fp4_decode", 32, False, False), ("fp4_decode", 32, False, True)]
 # the other configurations' headline fractions as scalars of config (beside config.also, which holds the whole lines)
 HEADLINES = {("exl3_linear", False, False): "exl3_linear_hbm_frac", ("exl3_prefill", False, False): "exl3_prefill_mfma_frac",
-             ("fp8_prefill", True, False): "fp8_block128_prefill_hbm_frac", ("fp8_prefill", False, False): "fp8_prefill_hbm_frac",
+             ("fp8_prefill", True, False): "fp8_block128_prefill_hbm_frac", ("fp8_prefill", True, True): "fp8_block128_gfx950_prefill_hbm_frac",
+             ("fp8_prefill", False, False): "fp8_prefill_hbm_frac",
              ("fp8_prefill", False, True): "fp8_gfx950_prefill_hbm_frac", ("fp4_prefill", False, False): "fp4_prefill_mfma_frac",
              ("fp4_prefill", False, True): "fp4_gfx950_prefill_mfma_frac", ("fp4_decode", False, False): "fp4_decode32_hbm_frac",
              ("fp4_decode", False, True): "fp4_gfx950_decode32_hbm_frac"}

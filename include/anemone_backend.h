@@ -59,7 +59,9 @@ enum weight_format_code {
      * new format is a new entry here, its kernels in every backend, and its reference decode among the tests"). Made at
      * load time from the reference's bytes by weight_format_gfx950_pack (anemone_ops.h), which also states the lay-out. */
     WEIGHT_FORMAT_E2M1_GFX950 = 7,
-    WEIGHT_FORMAT_E4M3_GFX950 = 8
+    WEIGHT_FORMAT_E4M3_GFX950 = 8,
+    /* and E4M3_BLOCK128 likewise: its codes in E4M3_GFX950's order, its float32 scales where they are */
+    WEIGHT_FORMAT_E4M3_BLOCK128_GFX950 = 9
 };
 
 #define BACKEND_MAXIMUM_CARDS 16

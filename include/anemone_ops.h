@@ -59,9 +59,11 @@ extern const struct weight_format_operations exl3_weight_operations;
  *   E4M3_GFX950  32 bytes a lane as two halves of 1,024 bytes a step ([half][lane][16]): byte c of word v (0 .. 7; half
  *                v / 4) is input 64 (v / 4) + 16 g + 8 (c % 2) + 2 (v % 4) + c / 2; behind all tiles the scale codes as
  *                E4M3_SCALED stores them (a row of inputs / 32 for every 32 outputs). Bytes: E4M3_SCALED's.
+ *   E4M3_BLOCK128_GFX950  E4M3_GFX950's bytes of codes; behind them E4M3_BLOCK128's float32 scales [outputs / 128][inputs /
+ *                128] (outputs and inputs multiples of 128). Bytes: E4M3_BLOCK128's.
  * The byte a lane's register holds is the byte the reference-format kernels of this library form there from the
- * reference's lay-out, so both formats' kernels run the same sums. pack: from E2M1_SCALED to E2M1_GFX950 or from
- * E4M3_SCALED to E4M3_GFX950 (`format` names the GFX950 format); unpack: back. The two byte counts must be the
+ * reference's lay-out, so both formats' kernels run the same sums. pack: from E2M1_SCALED to E2M1_GFX950, from
+ * E4M3_SCALED to E4M3_GFX950 or from E4M3_BLOCK128 to E4M3_BLOCK128_GFX950 (`format` names the GFX950 format); unpack: back. The two byte counts must be the
  * formats' stored_byte_count of the shape and the buffers apart; else STATUS_INVALID_ARGUMENT and nothing is written. */
 MUST_CHECK result_status weight_format_gfx950_pack(enum weight_format_code format, const struct matrix_shape_record *shape,
                                                    const void *reference_bytes, uint64_t reference_byte_count, void *packed_out,
@@ -375,6 +377,8 @@ struct linear_kernels_record { /* include/anemone/linear.h:121-132 of the refere
     uint32_t expert_down_gfx950[LINEAR_SLICE_INSTANCES];
     uint32_t expert_gate_up_e4m3_gfx950[LINEAR_SLICE_INSTANCES];
     uint32_t expert_down_e4m3_gfx950[LINEAR_SLICE_INSTANCES];
+    uint32_t expert_gate_up_b128_gfx950[LINEAR_SLICE_INSTANCES]; /* WEIGHT_FORMAT_E4M3_BLOCK128_GFX950 */
+    uint32_t expert_down_b128_gfx950[LINEAR_SLICE_INSTANCES];
 };
 MUST_CHECK result_status linear_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                 uint32_t arithmetic_class, struct linear_kernels_record *kernels_out);
@@ -423,8 +427,8 @@ enum linear_routed_experts_launch {
 };
 /* launches_out: LINEAR_ROUTED_EXPERTS_LAUNCH_COUNT launches; weight_format E2M1_SCALED, or (extensions) E4M3_SCALED,
  * E4M3_BLOCK128 (its exponent ranges hold float32 scales of 128 values (the same bytes), its quantizer launch is
- * activation_quantize_128_entry, its shapes are multiples of 128), E2M1_GFX950 or E4M3_GFX950 (the outputs of the same
- * matrices stored as E2M1_SCALED or E4M3_SCALED, bit for bit) */
+ * activation_quantize_128_entry, its shapes are multiples of 128), E2M1_GFX950, E4M3_GFX950 or E4M3_BLOCK128_GFX950 (the
+ * outputs of the same matrices stored as E2M1_SCALED, E4M3_SCALED or E4M3_BLOCK128, bit for bit) */
 MUST_CHECK result_status linear_routed_experts_prepare(const struct linear_routed_experts_description *description,
                                                        uint64_t arena_byte_count,
                                                        const struct linear_kernels_record *kernels,
@@ -591,15 +595,18 @@ MUST_CHECK result_status linear_wide_experts_block128_prepare(const struct linea
                                                               const struct linear_wide_kernels_record *kernels,
                                                               struct kernel_launch *launches_out);
 
-/* The wide form of experts stored in gfx950's lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950; no counterpart in the
- * reference): linear_wide_experts_prepare's description, three launches and outputs -- bit for bit those of the same
- * matrices in the reference's lay-out -- by the kernels of kernel_native_linear.hip, whose weights go from memory into
- * the matrix instruction's registers. */
+/* The wide form of experts stored in gfx950's lane order (WEIGHT_FORMAT_E2M1_GFX950, _E4M3_GFX950, _E4M3_BLOCK128_GFX950; no
+ * counterpart in the reference): linear_wide_experts_prepare's description, three launches (E4M3_BLOCK128_GFX950: the four
+ * of linear_wide_experts_block128_prepare, LINEAR_WIDE_EXPERTS_BLOCK128_LAUNCH_COUNT) and outputs -- bit for bit those of
+ * the same matrices in the reference's lay-out -- by the kernels of kernel_native_linear.hip, whose weights go from
+ * memory into the matrix instruction's registers. */
 struct linear_native_kernels_record {
     uint32_t native_expert_gate_up; /* E2M1_GFX950, one slice */
     uint32_t native_expert_down;
     uint32_t native_expert_gate_up_e4m3; /* E4M3_GFX950 */
     uint32_t native_expert_down_e4m3;
+    uint32_t native_expert_gate_up_b128; /* E4M3_BLOCK128_GFX950 */
+    uint32_t native_expert_down_b128;
 };
 MUST_CHECK result_status linear_native_kernels_prepare(const struct backend_operations *backend, struct device_card *card,
                                                        uint32_t arithmetic_class, struct linear_native_kernels_record *kernels_out);

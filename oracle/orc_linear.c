@@ -19,6 +19,16 @@ static int holds_nibbles(int format)
     return format == ORC_FORMAT_E2M1_SCALED || format == ORC_FORMAT_E2M1_GFX950;
 }
 
+static int holds_float_scales(int format)
+{
+    return format == ORC_FORMAT_E4M3_BLOCK128 || format == ORC_FORMAT_E4M3_BLOCK128_GFX950;
+}
+
+static int bytes_in_lane_order(int format)
+{
+    return format == ORC_FORMAT_E4M3_GFX950 || format == ORC_FORMAT_E4M3_BLOCK128_GFX950;
+}
+
 static int shape_is_stored(int format, uint32_t outputs, uint32_t inputs)
 {
     if (outputs == 0u || inputs == 0u || outputs % 16u != 0u) {
@@ -36,7 +46,7 @@ static int shape_is_stored(int format, uint32_t outputs, uint32_t inputs)
     if (format == ORC_FORMAT_E4M3_SCALED) {
         return inputs % 32u == 0u;
     }
-    if (format == ORC_FORMAT_E4M3_BLOCK128) {
+    if (holds_float_scales(format)) {
         return inputs % 128u == 0u && outputs % 128u == 0u;
     }
     return 0;
@@ -47,7 +57,7 @@ uint64_t orc_linear_scale_count(int format, uint32_t outputs, uint32_t inputs)
     if (holds_nibbles(format)) {
         return (uint64_t)outputs * (inputs / BLOCK);
     }
-    if (format == ORC_FORMAT_E4M3_BLOCK128) {
+    if (holds_float_scales(format)) {
         return (uint64_t)(outputs / 128u) * (inputs / 128u) * 4u; /* float32 scales, counted in bytes */
     }
     return (uint64_t)((outputs + 31u) / 32u) * (inputs / BLOCK);
@@ -68,7 +78,7 @@ int orc_linear_lay_out(int format, uint32_t outputs, uint32_t inputs, const uint
         return -1;
     }
     const uint32_t tiles = outputs / 16u;
-    if (format == ORC_FORMAT_E2M1_GFX950 || format == ORC_FORMAT_E4M3_GFX950) {
+    if (format == ORC_FORMAT_E2M1_GFX950 || bytes_in_lane_order(format)) {
         /* walk the stored bytes of the definition and ask which weight lies in each */
         static const uint32_t input_of_byte[4] = {0, 8, 1, 9};
         const uint32_t steps = inputs / 128u;
@@ -105,7 +115,7 @@ int orc_linear_lay_out(int format, uint32_t outputs, uint32_t inputs, const uint
                 }
             }
         }
-        if (format == ORC_FORMAT_E4M3_GFX950) {
+        if (bytes_in_lane_order(format)) { /* the scale codes, or the float32 scales, as they come */
             memcpy(stored + at, scale_codes, orc_linear_scale_count(format, outputs, inputs));
             return 0;
         }
@@ -194,11 +204,15 @@ int orc_linear_read(int format, uint32_t outputs, uint32_t inputs, const uint8_t
         *scale_out = stored[(uint64_t)outputs * inputs / 2u + ((((uint64_t)(tile / 4u) * steps + step) * 64u + lane) * 4u + tile % 4u)];
         return 0;
     }
-    if (format == ORC_FORMAT_E4M3_GFX950) {
+    if (bytes_in_lane_order(format)) {
         /* input = 128 step + 64 half + 16 G + r with r = 8 (c % 2) + 2 (v % 4) + c / 2 */
         const uint32_t steps = inputs / 128u, step = input / 128u, half = (input % 128u) / 64u, G = (input % 64u) / 16u, r = input % 16u;
         const uint32_t word = (r % 8u) / 2u, c = 2u * (r % 2u) + r / 8u, lane = 16u * G + in_tile;
         *code_out = stored[((uint64_t)tile * steps + step) * 2048u + half * 1024u + lane * 16u + word * 4u + c];
+        if (holds_float_scales(format)) {
+            memcpy(scale_out, stored + (uint64_t)outputs * inputs + ((uint64_t)(output / 128u) * steps + step) * 4u, 4u);
+            return 0;
+        }
         *scale_out = stored[(uint64_t)outputs * inputs + (uint64_t)(output / 32u) * (inputs / BLOCK) + input / BLOCK];
         return 0;
     }
@@ -368,12 +382,11 @@ int orc_linear_products(int format, uint32_t outputs, uint32_t inputs, const uin
     return 0;
 }
 
-int orc_linear_products_128(uint32_t outputs, uint32_t inputs, const uint8_t *stored, uint32_t first, uint32_t count,
-                            const uint8_t *fed_codes, const float *fed_scales, uint32_t vectors, double *sums_out,
-                            double *magnitude_out)
+int orc_linear_products_128_of(int format, uint32_t outputs, uint32_t inputs, const uint8_t *stored, uint32_t first,
+                               uint32_t count, const uint8_t *fed_codes, const float *fed_scales, uint32_t vectors,
+                               double *sums_out, double *magnitude_out)
 {
-    const int format = ORC_FORMAT_E4M3_BLOCK128;
-    if (!shape_is_stored(format, outputs, inputs) || first + count > outputs) {
+    if (!holds_float_scales(format) || !shape_is_stored(format, outputs, inputs) || first + count > outputs) {
         return -1;
     }
     const uint32_t blocks = inputs / 128u;
@@ -409,6 +422,14 @@ int orc_linear_products_128(uint32_t outputs, uint32_t inputs, const uint8_t *st
     free(values);
     free(scales);
     return 0;
+}
+
+int orc_linear_products_128(uint32_t outputs, uint32_t inputs, const uint8_t *stored, uint32_t first, uint32_t count,
+                            const uint8_t *fed_codes, const float *fed_scales, uint32_t vectors, double *sums_out,
+                            double *magnitude_out)
+{
+    return orc_linear_products_128_of(ORC_FORMAT_E4M3_BLOCK128, outputs, inputs, stored, first, count, fed_codes, fed_scales,
+                                      vectors, sums_out, magnitude_out);
 }
 
 static double bf16_last_place(uint16_t bits)
@@ -540,7 +561,7 @@ struct linear_layer {
  * scale arrays have the same bytes either way: width / 32 a vector) */
 static void layer_quantize(int format, const uint16_t *values, uint32_t width, uint8_t *codes, uint8_t *scales)
 {
-    if (format == ORC_FORMAT_E4M3_BLOCK128) {
+    if (holds_float_scales(format)) {
         orc_act_quantize_128(values, width, codes, (float *)(void *)scales);
     } else {
         (void)orc_act_quantize(values, width, codes, scales);
@@ -550,8 +571,8 @@ static void layer_quantize(int format, const uint16_t *values, uint32_t width, u
 static void layer_products(int format, uint32_t outputs, uint32_t inputs, const uint8_t *stored, const uint8_t *codes,
                            const uint8_t *scales, uint32_t vectors, double *sums)
 {
-    if (format == ORC_FORMAT_E4M3_BLOCK128) {
-        (void)orc_linear_products_128(outputs, inputs, stored, 0, outputs, codes, (const float *)(const void *)scales, vectors, sums, NULL);
+    if (holds_float_scales(format)) {
+        (void)orc_linear_products_128_of(format, outputs, inputs, stored, 0, outputs, codes, (const float *)(const void *)scales, vectors, sums, NULL);
     } else {
         (void)orc_linear_products(format, outputs, inputs, stored, 0, outputs, codes, scales, vectors, sums, NULL);
     }

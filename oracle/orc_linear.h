@@ -43,6 +43,9 @@
  * Inputs a multiple of 128; outputs of 64 (E2M1) or 32 (E4M3). */
 #define ORC_FORMAT_E2M1_GFX950 7
 #define ORC_FORMAT_E4M3_GFX950 8
+/* E4M3_BLOCK128's codes in E4M3_GFX950's lane order, then E4M3_BLOCK128's float32 scales as they are;
+ * inputs and outputs a multiple of 128 */
+#define ORC_FORMAT_E4M3_BLOCK128_GFX950 9
 
 uint64_t orc_linear_stored_bytes(int format, uint32_t outputs, uint32_t inputs);
 uint64_t orc_linear_scale_count(int format, uint32_t outputs, uint32_t inputs);
@@ -93,6 +96,10 @@ void orc_fp8_block128_products(uint32_t outputs, uint32_t inputs, const uint8_t 
 int orc_linear_products_128(uint32_t outputs, uint32_t inputs, const uint8_t *stored, uint32_t first, uint32_t count,
                             const uint8_t *fed_codes, const float *fed_scales, uint32_t vectors, double *sums_out,
                             double *magnitude_out);
+/* the same for either format of float32 scales (ORC_FORMAT_E4M3_BLOCK128, ORC_FORMAT_E4M3_BLOCK128_GFX950) */
+int orc_linear_products_128_of(int format, uint32_t outputs, uint32_t inputs, const uint8_t *stored, uint32_t first,
+                               uint32_t count, const uint8_t *fed_codes, const float *fed_scales, uint32_t vectors,
+                               double *sums_out, double *magnitude_out);
 
 /* One whole FP4/FP8 routed-expert layer (formats of the reference, per-32 scales), double-precision products with
  * the kernels' rounding points (format 6: float32 scales per 128, quantizer orc_act_quantize_128): quantize x per row, gate/up products -> bf16, hidden step -> bf16, quantize the

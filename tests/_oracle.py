@@ -70,6 +70,7 @@ def _load_oracle():
         "orc_operands_lay_out": (None, [u8p, u8p, u32, u16p]),
         "orc_linear_products": (i32, [i32, u32, u32, u8p, u32, u32, u8p, u8p, u32, f64p, f64p]),
         "orc_linear_products_128": (i32, [u32, u32, u8p, u32, u32, u8p, f32p, u32, f64p, f64p]),
+        "orc_linear_products_128_of": (i32, [i32, u32, u32, u8p, u32, u32, u8p, f32p, u32, f64p, f64p]),
         "orc_linear_within_tolerance": (i32, [C.c_uint16, C.c_double, C.c_double, u32, u32]),
         "orc_linear_within_allowance": (i32, [C.c_uint16, C.c_double, C.c_double, u32, u32, C.c_double]),
         "orc_hidden_value": (C.c_double, [C.c_double] * 4),

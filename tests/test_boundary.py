@@ -510,7 +510,7 @@ def test_tcp_prepare_geometry_and_refusals(fake):
 def experts_description(fmt=amd.WEIGHT_FORMAT_E2M1_SCALED, **changes):
     rows, P, H, I = 8, 8, 4096, 2048
     pairs = rows * P
-    bits = 8 if fmt in (amd.WEIGHT_FORMAT_E4M3_SCALED, amd.WEIGHT_FORMAT_E4M3_BLOCK128, amd.WEIGHT_FORMAT_E4M3_GFX950) else 4
+    bits = 4 if fmt in (amd.WEIGHT_FORMAT_E2M1_SCALED, amd.WEIGHT_FORMAT_E2M1_GFX950) else 8
     d = amd.RoutedExpertsDescription()
     cursor = [4096]
 
@@ -827,7 +827,7 @@ def test_block128_prepare_geometry_and_refusals(fake):
 
 
 def test_gfx950_formats_prepare_geometry_and_refusals(fake):
-    """The formats in gfx950's lane order (7, 8): the job-table launches by the expert_*_gfx950_<S> kernels on the
+    """The formats in gfx950's lane order (7, 8, 9): the job-table launches by the expert_*_gfx950_<S> kernels on the
     reference formats' grids, the wide form by linear_native_experts_prepare alone, the producer refused."""
     lib = amd.library()
     arena = 8 << 30
@@ -838,23 +838,32 @@ def test_gfx950_formats_prepare_geometry_and_refusals(fake):
     assert fake.handles[linear.expert_gate_up_gfx950[0]][1] == "expert_gate_up_gfx950_1"
     assert fake.handles[linear.expert_down_e4m3_gfx950[3]][1] == "expert_down_e4m3_gfx950_8" and linear.expert_gate_up_gfx950[4] == amd.BACKEND_NO_KERNEL
     assert fake.handles[native.native_expert_gate_up][1] == "native_expert_gate_up_1" and fake.handles[native.native_expert_down_e4m3][1] == "native_expert_down_e4m3_1"
+    assert fake.handles[linear.expert_gate_up_b128_gfx950[1]][1] == "expert_gate_up_b128_gfx950_2" and fake.handles[native.native_expert_down_b128][1] == "native_expert_down_b128_1"
     for fmt, like, names in ((amd.WEIGHT_FORMAT_E2M1_GFX950, amd.WEIGHT_FORMAT_E2M1_SCALED, ["expert_gate_up_gfx950_4", "expert_down_gfx950_2"]),
-                             (amd.WEIGHT_FORMAT_E4M3_GFX950, amd.WEIGHT_FORMAT_E4M3_SCALED, ["expert_gate_up_e4m3_gfx950_4", "expert_down_e4m3_gfx950_2"])):
+                             (amd.WEIGHT_FORMAT_E4M3_GFX950, amd.WEIGHT_FORMAT_E4M3_SCALED, ["expert_gate_up_e4m3_gfx950_4", "expert_down_e4m3_gfx950_2"]),
+                             (amd.WEIGHT_FORMAT_E4M3_BLOCK128_GFX950, amd.WEIGHT_FORMAT_E4M3_BLOCK128, ["expert_gate_up_b128_gfx950_4", "expert_down_b128_gfx950_2"])):
+        block128 = fmt == amd.WEIGHT_FORMAT_E4M3_BLOCK128_GFX950
         launches, reference = amd.launches_of(4), amd.launches_of(4)
         assert lib.linear_routed_experts_prepare(C.byref(experts_description(fmt)), ARENA, C.byref(linear), launches) == 0
         assert lib.linear_routed_experts_prepare(C.byref(experts_description(like)), ARENA, C.byref(linear), reference) == 0
         assert [fake.handles[launches[i].kernel][1] for i in (0, 2)] == names
-        assert fake.handles[launches[1].kernel][1] == "activation_quantize_entry" and fake.handles[launches[3].kernel][1] == "expert_row_sum_entry"
+        assert fake.handles[launches[1].kernel][1] == ("activation_quantize_128_entry" if block128 else "activation_quantize_entry")
+        assert fake.handles[launches[3].kernel][1] == "expert_row_sum_entry"
         for ours, theirs in zip(launches, reference):  # the grids, blocks and records of the reference format's launches
             assert list(ours.grid) == list(theirs.grid) and list(ours.block) == list(theirs.block)
             assert bytes(ours.argument) == bytes(theirs.argument)
         # the wide form: its own prepare takes these formats, the reference formats' prepare does not, and the other way round
-        three, untouched = amd.launches_of(3), amd.launches_of(4)
+        three, untouched = amd.launches_of(4), amd.launches_of(4)
         description = wide_experts_description(fmt)
         assert lib.linear_native_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(native), three) == 0
-        assert fake.handles[three[0].kernel][1].startswith("native_expert_gate_up") and fake.handles[three[2].kernel][1] == "expert_row_sum_entry"
+        assert fake.handles[three[0].kernel][1].startswith("native_expert_gate_up") and fake.handles[three[3 if block128 else 2].kernel][1] == "expert_row_sum_entry"
+        if block128:  # the hidden values' quantizer is a launch of its own, as in the E4M3_BLOCK128 wide form
+            assert [fake.handles[three[i].kernel][1] for i in (0, 1, 2)] == ["native_expert_gate_up_b128_1", "activation_quantize_128_entry", "native_expert_down_b128_1"]
+        else:
+            assert not any(bytes(three[3]))
         assert three[0].dynamic_shared_byte_count > 0 and three[0].block[0] == 256
         assert lib.linear_wide_experts_prepare(C.byref(description), arena, C.byref(linear), C.byref(wide_kernels), untouched) == 1
+        assert lib.linear_wide_experts_block128_prepare(C.byref(description), arena, C.byref(linear), C.byref(wide_kernels), untouched) == 1
         assert lib.linear_native_experts_prepare(C.byref(wide_experts_description(like)), arena, C.byref(linear), C.byref(native), untouched) == 1
         assert not any(bytes(untouched))
     # E2M1_GFX950 stores whole groups of four tiles: outputs in whole 64
@@ -866,7 +875,7 @@ def test_gfx950_formats_prepare_geometry_and_refusals(fake):
     fused = amd.ExpertFusedKernels()
     assert lib.expert_fused_kernels_prepare(fake.address, fake.card, 950, C.byref(fused)) == 0
     one = amd.launches_of(1)
-    for fmt in (amd.WEIGHT_FORMAT_E2M1_GFX950, amd.WEIGHT_FORMAT_E4M3_GFX950, amd.WEIGHT_FORMAT_E4M3_BLOCK128):
+    for fmt in (amd.WEIGHT_FORMAT_E2M1_GFX950, amd.WEIGHT_FORMAT_E4M3_GFX950, amd.WEIGHT_FORMAT_E4M3_BLOCK128, amd.WEIGHT_FORMAT_E4M3_BLOCK128_GFX950):
         d = experts_description(fmt)
         arrivals = amd.Range(6 << 30, 64 * (2048 // 32) * 4)
         assert lib.expert_producer_prepare(C.byref(d), arrivals, arena, C.byref(linear), C.byref(fused), one) == 1, fmt
@@ -970,3 +979,17 @@ def test_site_front_launches_geometry_and_refusals(fake):
         assert lib.hyper_site_prepare(C.byref(site_description(**changes)), arena, C.byref(hyper), untouched) == 1, changes
         assert not any(bytes(untouched))
 
+
+
+def test_the_build_refuses_a_spilling_kernel_of_hand_issued_loads():
+    """anemone_amd/build.py reads the compiler's resource remarks of the kernels whose loads the compiler keeps no book on
+    (csrc/native_device.cuh) and names those that spill a vector register."""
+    from anemone_amd import build
+    remark = "/x/kernel_native_linear.hip:%d:1: remark: %s [-Rpass-analysis=kernel-resource-usage]"
+    lines = []
+    for at, (name, sgprs, vgprs) in enumerate([("native_expert_gate_up_1", 0, 0), ("native_expert_down_b128_1", 3, 14), ("native_expert_down_1", 9, 0)]):
+        lines += [remark % (at, "Function Name: " + name), remark % (at, "    VGPRs: 168"), remark % (at, "    ScratchSize [bytes/lane]: %d" % (4 * vgprs)),
+                  remark % (at, "    SGPRs Spill: %d" % sgprs), remark % (at, "    VGPRs Spill: %d" % vgprs)]
+    assert build.spilling_kernels("\n".join(lines + ["warning: something else"])) == [("native_expert_down_b128_1", 14)]
+    assert build.spilling_kernels("") == []
+    assert "kernel_native_linear.hip" in build.NO_SPILL_SOURCES and set(build.NO_SPILL_SOURCES) <= set(build.HIP_SOURCES)

@@ -132,7 +132,7 @@ WIDE_RESULTS = {}  # form -> (picks, row outputs, hidden codes): a lay-out's run
 def run_wide_form(amd, workloads, form, rows):
     if form in WIDE_RESULTS:
         return WIDE_RESULTS[form]
-    fp8, block128, native = form.startswith("fp8"), form == "fp8_block128", form.endswith("_gfx950")
+    fp8, block128, native = form.startswith("fp8"), form.startswith("fp8_block128"), form.endswith("_gfx950")
     distinct_generated = 4 if fp8 else 16
     base = workloads.SEED + ((3 if fp8 else 4) << 20)
     matrix = workloads.fp8_block128_matrix if block128 else workloads.fp8_matrix if fp8 else workloads.fp4_matrix
@@ -141,7 +141,7 @@ def run_wide_form(amd, workloads, form, rows):
     matrices = [trios[e % distinct_generated] for e in range(EXPERTS)]
     router = workloads.to_bf16(workloads.normals(base + 2, EXPERTS * HIDDEN) * 0.02).reshape(EXPERTS, HIDDEN)
     x = workloads.activations(4, rows, HIDDEN)
-    weight_format = (amd.WEIGHT_FORMAT_E4M3_GFX950 if fp8 else amd.WEIGHT_FORMAT_E2M1_GFX950) if native else \
+    weight_format = (amd.WEIGHT_FORMAT_E4M3_BLOCK128_GFX950 if block128 else amd.WEIGHT_FORMAT_E4M3_GFX950 if fp8 else amd.WEIGHT_FORMAT_E2M1_GFX950) if native else \
         amd.WEIGHT_FORMAT_E4M3_BLOCK128 if block128 else amd.WEIGHT_FORMAT_E4M3_SCALED if fp8 else amd.WEIGHT_FORMAT_E2M1_SCALED
     card = amd.Card(((9 if fp8 else 5) << 30) + rows * (1 << 18))
     try:
@@ -163,14 +163,15 @@ def run_wide_form(amd, workloads, form, rows):
     return WIDE_RESULTS[form]
 
 
-@pytest.mark.parametrize("form,rows", [("fp4", 8192), ("fp8", 2048), ("fp8_block128", 2048), ("fp4_gfx950", 8192), ("fp8_gfx950", 2048)])
+@pytest.mark.parametrize("form,rows", [("fp4", 8192), ("fp8", 2048), ("fp8_block128", 2048), ("fp4_gfx950", 8192), ("fp8_gfx950", 2048),
+                                       ("fp8_block128_gfx950", 2048)])
 def test_wide_experts_of_the_original_weights(amd, workloads, form, rows):
     say("full shape: wide", form, rows, "rows")
-    fp8, block128, native = form.startswith("fp8"), form == "fp8_block128", form.endswith("_gfx950")
+    fp8, block128, native = form.startswith("fp8"), form.startswith("fp8_block128"), form.endswith("_gfx950")
     x, matrices, picks, got, hidden_codes = run_wide_form(amd, workloads, form, rows)
     if native:
         # gfx950's lay-out of the same matrices: every byte the launches write is the reference lay-out's (the same sums)
-        _, _, want_picks, want, want_codes = run_wide_form(amd, workloads, form[:3], rows)
+        _, _, want_picks, want, want_codes = run_wide_form(amd, workloads, form[:-len("_gfx950")], rows)
         assert want_picks.tobytes() == picks.tobytes()
         assert got.tobytes() == want.tobytes(), "the row outputs differ from the reference lay-out's"
         assert hidden_codes.tobytes() == want_codes.tobytes(), "the hidden codes differ from the reference lay-out's"

@@ -1,5 +1,5 @@
 """GPU parity of the wide routed experts whose weights lie in gfx950's own lane order (WEIGHT_FORMAT_E2M1_GFX950,
-WEIGHT_FORMAT_E4M3_GFX950; the matrices go through the library's load-time re-lay-out, weight_format_gfx950_pack), through
+WEIGHT_FORMAT_E4M3_GFX950, WEIGHT_FORMAT_E4M3_BLOCK128_GFX950; the matrices go through the library's load-time re-lay-out, weight_format_gfx950_pack), through
 the C ABI: byte for byte the outputs of the same layer in the reference's lay-out (kernel_wide_linear.hip's launches,
 which tests/test_gpu_wide_linear.py holds byte for byte to the job-table kernels and those to the oracle), and the
 layer's rows against the CPU oracle reading the re-laid-out bytes itself."""
@@ -13,7 +13,8 @@ from _oracle import f32p, normals, orc, ptr, to_bf16, u16p, u32p
 
 pytestmark = pytest.mark.gpu
 
-E2M1, E4M3, E2M1_GFX950, E4M3_GFX950 = 3, 5, 7, 8
+E2M1, E4M3, B128, E2M1_GFX950, E4M3_GFX950, B128_GFX950 = 3, 5, 6, 7, 8, 9
+NATIVE_OF = {E2M1: E2M1_GFX950, E4M3: E4M3_GFX950, B128: B128_GFX950}
 NAMES = ("hidden_codes", "hidden_exponents", "hidden_operands", "pair_output", "row_output")
 
 
@@ -43,7 +44,7 @@ def fresh_arena(card):
 
 def matrices_of(hidden, inner, experts_n, seed, fmt, distinct=8):
     from anemone_amd import workloads
-    matrix = workloads.fp4_matrix if fmt == E2M1 else workloads.fp8_matrix
+    matrix = workloads.fp4_matrix if fmt == E2M1 else workloads.fp8_block128_matrix if fmt == B128 else workloads.fp8_matrix
     trios = [[matrix(seed * 1000 + 3 * e + 0, inner, hidden), matrix(seed * 1000 + 3 * e + 1, inner, hidden),
               matrix(seed * 1000 + 3 * e + 2, hidden, inner)] for e in range(distinct)]
     return [trios[e % distinct] for e in range(experts_n)]
@@ -73,6 +74,10 @@ def run_wide(card, layer, x, live):
     (512, 256, 64, 8, 1500, 1401, E4M3),  # blocks of two tiles of one expert, a run's odd last tile alone
     (512, 256, 64, 8, 6000, 5999, E4M3),  # runs of a dozen tiles: the places of a run's tiles by the lanes' look back
     (512, 256, 64, 1, 4300, 4300, -E4M3), # one expert takes every row: a run of 68 tiles, the look back goes round again
+    (512, 256, 64, 4, 300, 300, B128),    # float32 scales of 128 x 128 blocks: the quantizer between the two products
+    (640, 384, 64, 2, 450, 449, B128),
+    (512, 256, 64, 8, 1500, 1401, B128),
+    (512, 256, 64, 1, 4300, 4300, -B128),
 ])
 def test_native_equals_the_reference_lay_out_byte_for_byte(amd, card, hidden, inner, experts_n, picks, rows, live, fmt):
     say("native experts", hidden, inner, experts_n, picks, rows, live, fmt)
@@ -89,7 +94,7 @@ def test_native_equals_the_reference_lay_out_byte_for_byte(amd, card, hidden, in
     counts = np.bincount(wide.read("picks", np.dtype([("expert", "<u4"), ("route_weight", "<f4")]))["expert"][:live * picks], minlength=experts_n)
     say("  pairs of the busiest expert:", int(counts.max()))
     native = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router,
-                          weight_format=E2M1_GFX950 if fmt == E2M1 else E4M3_GFX950)
+                          weight_format=NATIVE_OF[fmt])
     card.upload(native.bias_offset, bias)
     got, _ = run_wide(card, native, x, live)
     pairs = live * picks
@@ -102,18 +107,20 @@ def test_native_equals_the_reference_lay_out_byte_for_byte(amd, card, hidden, in
         assert a.reshape(-1)[:count].tobytes() != bytes([0xEE]) * count, "the launches wrote"
     if live < rows:  # nothing is written for the pairs of the rows beyond the live ones
         for name, b in zip(NAMES[:4], got[:4]):
+            if fmt == B128 and name in ("hidden_codes", "hidden_exponents"):
+                continue  # the quantizer of 128 values a scale is a launch over every pair the step has room for
             per = b.size // (rows * picks)
             assert np.all(b.reshape(-1)[pairs * per:] == 0xEE), name
 
 
-@pytest.mark.parametrize("fmt", [E2M1, E4M3])
+@pytest.mark.parametrize("fmt", [E2M1, E4M3, B128])
 def test_native_layer_against_oracle(amd, card, fmt):
     """The layer in gfx950's lay-out against the CPU oracle reading the SAME re-laid-out bytes (its own reading of the
     format, oracle/orc_linear.c) with the picks the card made."""
     say("native layer against the oracle", fmt)
     from test_gpu_router_wide import oracle_wide
     hidden, inner, experts_n, picks, rows, live = 512, 256, 64, 4, 150, 143
-    native_format = E2M1_GFX950 if fmt == E2M1 else E4M3_GFX950
+    native_format = NATIVE_OF[fmt]
     matrices = matrices_of(hidden, inner, experts_n, 33, fmt, distinct=64)
     router = to_bf16(normals(5, experts_n * hidden) * 0.02).reshape(experts_n, hidden)
     layer = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router, weight_format=native_format)
@@ -152,6 +159,10 @@ def run_jobs(card, layer, x, live):
     (512, 256, 4, 8, 8, E4M3, 4, 2),
     (640, 384, 8, 2, 2, E4M3, 1, 2),     # 40 tiles of the gate product: strips of two
     (1024, 512, 1, 8, 5, E4M3, 8, 4),
+    (512, 256, 4, 8, 8, B128, 4, 2),
+    (640, 384, 8, 2, 2, B128, 1, 2),
+    (1024, 512, 1, 8, 5, B128, 8, 4),
+    (640, 384, 2, 5, 5, B128, 2, 1),
 ])
 def test_native_job_table_kernels_equal_the_reference_lay_out(amd, card, hidden, inner, picks, rows, live, fmt, gate_up_slices, down_slices):
     """The job-table kernels (a thin step's) of the formats in gfx950's lane order, expert_gate_up_gfx950_<S> and its like:
@@ -165,7 +176,7 @@ def test_native_job_table_kernels_equal_the_reference_lay_out(amd, card, hidden,
                              gate_up_slices=gate_up_slices, down_slices=down_slices)
     want, want_jobs = run_jobs(card, reference, x, live)
     native = amd.Fp4Layer(card, hidden, inner, experts_n, picks, rows, matrices, router_weights_bf16=router,
-                          weight_format=E2M1_GFX950 if fmt == E2M1 else E4M3_GFX950, gate_up_slices=gate_up_slices, down_slices=down_slices)
+                          weight_format=NATIVE_OF[fmt], gate_up_slices=gate_up_slices, down_slices=down_slices)
     got, got_jobs = run_jobs(card, native, x, live)
     assert np.array_equal(want_jobs["expert"], got_jobs["expert"]) and np.array_equal(want_jobs["pair_index"], got_jobs["pair_index"])
     pairs = live * picks
@@ -175,4 +186,5 @@ def test_native_job_table_kernels_equal_the_reference_lay_out(amd, card, hidden,
         differing = np.flatnonzero(a.reshape(-1)[:count] != b.reshape(-1)[:count])
         say("  %s: %d of %d bytes differ" % (name, differing.size, count))
         assert differing.size == 0, (name, differing[:8], per)
-        assert a.reshape(-1)[:count].tobytes() != bytes([0xEE]) * count, "the launches wrote"
+        if not (fmt == B128 and name == "hidden_operands"):  # the quantizer of 128 values a scale writes no operands
+            assert a.reshape(-1)[:count].tobytes() != bytes([0xEE]) * count, "the launches wrote"
