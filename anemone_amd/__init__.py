@@ -239,6 +239,37 @@ class LinearWideKernels(C.Structure):
                 ("wide_expert_gate_up_b128", u32), ("wide_expert_down_b128", u32)]
 
 
+class PackTensor(C.Structure):
+    """A tensor record as a pack stores it (include/anemone_descriptor.h: struct pack_tensor, 64 bytes)."""
+    _fields_ = [("byte_offset_in_extent", u64), ("byte_count", u64), ("extent_index", u32), ("name_byte_offset", u32), ("name_byte_count", u32),
+                ("element_type", u32), ("dimension_count", u32), ("dimensions", u32 * 4), ("weight_format", u32), ("bits_per_weight", u32),
+                ("reserved_zero", u32 * 1)]
+
+
+PACK_TENSOR_DTYPE = np.dtype([("byte_offset_in_extent", "<u8"), ("byte_count", "<u8"), ("extent_index", "<u4"), ("name_byte_offset", "<u4"),
+                              ("name_byte_count", "<u4"), ("element_type", "<u4"), ("dimension_count", "<u4"), ("dimensions", "<u4", (4,)),
+                              ("weight_format", "<u4"), ("bits_per_weight", "<u4"), ("reserved_zero", "<u4", (1,))])
+
+
+class Exl3PackView(C.Structure):
+    _fields_ = [("header_digest", u64), ("file_byte_count", u64), ("tensors", C.c_void_p), ("name_bytes", C.c_void_p), ("tensor_count", u32),
+                ("name_byte_count", u32)]
+
+
+class Exl3DescriptorMatrix(C.Structure):
+    _fields_ = [("kind", C.c_char_p), ("outputs", u32), ("inputs", u32)]
+
+
+class Exl3EstablishedPack(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("header_digest", u64), ("file_byte_count", u64)]
+
+
+class Exl3DescriptorModel(C.Structure):
+    _fields_ = [("model_type", C.c_char_p), ("layers", u32), ("experts_per_layer", u32), ("hidden", u32), ("intermediate", u32),
+                ("matrices", Exl3DescriptorMatrix * 3), ("established", C.POINTER(Exl3EstablishedPack)), ("established_count", u32),
+                ("routes_per_row", u32), ("cone_first_layer", u32)]
+
+
 class LinearNativeKernels(C.Structure):
     _fields_ = [("native_expert_gate_up", u32), ("native_expert_down", u32), ("native_expert_gate_up_e4m3", u32), ("native_expert_down_e4m3", u32),
                 ("native_expert_gate_up_b128", u32), ("native_expert_down_b128", u32)]
@@ -345,6 +376,8 @@ def library():
             "expert_host_copies_attach": [vp, C.POINTER(ExpertPause), u32, C.POINTER(u64), u64, vp, u64, u64, u64, C.POINTER(ExpertHostCopies),
                                           C.POINTER(u64)],
             "expert_post_prepare": [C.POINTER(ExpertJoinDescription), u64, u32, launch_p],
+            "exl3_descriptor_check": [C.c_char_p, C.POINTER(Exl3PackView), C.POINTER(Exl3DescriptorModel), C.c_char_p, u64, C.c_bool],
+            "exl3_descriptor_tc_check": [C.c_char_p, C.POINTER(Exl3DescriptorModel), u32, u32],
             "expert_shared_join_prepare": [C.POINTER(ExpertSharedJoinDescription), u64, C.POINTER(LinearKernels),
                                            C.POINTER(ExpertFusedKernels), launch_p],
         }
@@ -363,6 +396,8 @@ def library():
         lib.backend_hip_kernel_table_count.restype = u32
         lib.exl3_scratch_byte_count.restype = u64
         lib.exl3_scratch_byte_count.argtypes = [u32, u32]
+        lib.anemone_sha256.restype = None
+        lib.anemone_sha256.argtypes = [vp, u64, vp]
         lib.exl3_width_name.restype = C.c_char_p
         lib.exl3_width_name.argtypes = [u32]
         _lib = lib

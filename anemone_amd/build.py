@@ -20,7 +20,7 @@ PROBE_LIBRARY = os.path.join(HERE, "libanemone_probe.so")
 EXPORTS = os.path.join(HERE, "host", "exports.map")
 BUILD = os.path.join(HERE, "build")
 
-HOST_SOURCES = ["status.c", "prepare_common.c", "weight_format.c", "exl3.c", "exl3_tc.c", "router.c", "linear.c", "expert_fused.c", "site.c", "site_front.c", "step_experts.c", "exl3_layout.c"]
+HOST_SOURCES = ["status.c", "prepare_common.c", "weight_format.c", "exl3.c", "exl3_tc.c", "router.c", "linear.c", "expert_fused.c", "site.c", "site_front.c", "step_experts.c", "exl3_layout.c", "sha256.c", "json_tree.c", "exl3_descriptor.c"]
 HIP_SOURCES = ["kernel_exl3.hip", "kernel_exl3_tc.hip", "kernel_exl3_tcp.hip", "kernel_router.hip", "kernel_dense_linear.hip", "kernel_activation_quantize.hip", "kernel_wide_linear.hip", "kernel_native_linear.hip",
                "kernel_expert_linear.hip", "kernel_trunk_linear.hip", "kernel_hyper_connection.hip", "kernel_site_front.hip"]
 PROBE_SOURCES = ["kernel_calibrate.hip", "kernel_selfcheck.hip"]

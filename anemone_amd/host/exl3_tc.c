@@ -22,6 +22,30 @@
 #define PRODUCT_WAVES 4u
 #define MOST_GRID_ROWS 65535u
 
+/* a block's four wavefronts take four items: of one strip (its matrices x slices a multiple of four: z blocks a strip)
+ * or of adjacent strips (a divisor of four: that many strips a block) */
+enum { GATE_UP_ITEMS = 2u * EXL3_TC_GATE_UP_SLICES, DOWN_ITEMS = EXL3_TC_DOWN_SLICES };
+_Static_assert((GATE_UP_ITEMS % PRODUCT_WAVES == 0 || PRODUCT_WAVES % GATE_UP_ITEMS == 0) &&
+               (DOWN_ITEMS % PRODUCT_WAVES == 0 || PRODUCT_WAVES % DOWN_ITEMS == 0), "a block's four wavefronts take four whole items");
+#define GATE_UP_STRIPS (GATE_UP_ITEMS >= PRODUCT_WAVES ? 1u : PRODUCT_WAVES / GATE_UP_ITEMS)
+#define DOWN_STRIPS (DOWN_ITEMS >= PRODUCT_WAVES ? 1u : PRODUCT_WAVES / DOWN_ITEMS)
+
+/* why the fused decode's launches do not take a layer of these sizes (the prefill launches take every layer they take,
+ * and an intermediate size up to twice the hidden); NULL when they do */
+const char *exl3_tc_geometry_refusal(uint32_t hidden, uint32_t intermediate)
+{
+    if (hidden == 0 || intermediate == 0 || intermediate % EXL3_TRANSFORM != 0 || hidden % EXL3_TRANSFORM != 0) {
+        return "the sizes are multiples of 128";
+    }
+    if (intermediate > hidden) {
+        return "the intermediate size is at most the hidden size";
+    }
+    if (intermediate % (EXL3_TC_STRIP_OUTPUTS * GATE_UP_STRIPS) != 0 || hidden % (EXL3_TC_STRIP_OUTPUTS * DOWN_STRIPS) != 0) {
+        return "the sizes are whole numbers of the products' blocks";
+    }
+    return NULL;
+}
+
 /* detached_workspace: the workspace is not a range of the arena (exl3_tc_run_static names it by an offset of its own) */
 static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t arena_byte_count,
                                 const struct backend_operations *backend, struct device_card *card,
@@ -99,13 +123,7 @@ static result_status tc_prepare(const struct exl3_tc_record *record, uint64_t ar
     }
     static const char *const names[EXL3_TC_LAUNCHES] = {"exl3_tc_operands", "exl3_tc_products", "exl3_tc_activate",
                                                         "exl3_tc_products", "exl3_tc_combine"};
-    /* a block's four wavefronts take four items: of one strip (its matrices x slices a multiple of four: z blocks a strip)
-     * or of adjacent strips (a divisor of four: that many strips a block) */
-    enum { GATE_UP_ITEMS = 2u * EXL3_TC_GATE_UP_SLICES, DOWN_ITEMS = EXL3_TC_DOWN_SLICES };
-    _Static_assert((GATE_UP_ITEMS % PRODUCT_WAVES == 0 || PRODUCT_WAVES % GATE_UP_ITEMS == 0) &&
-                   (DOWN_ITEMS % PRODUCT_WAVES == 0 || PRODUCT_WAVES % DOWN_ITEMS == 0), "a block's four wavefronts take four whole items");
-    const uint32_t gate_up_strips = GATE_UP_ITEMS >= PRODUCT_WAVES ? 1u : PRODUCT_WAVES / GATE_UP_ITEMS;
-    const uint32_t down_strips = DOWN_ITEMS >= PRODUCT_WAVES ? 1u : PRODUCT_WAVES / DOWN_ITEMS;
+    const uint32_t gate_up_strips = GATE_UP_STRIPS, down_strips = DOWN_STRIPS;
     if (I % (EXL3_TC_STRIP_OUTPUTS * gate_up_strips) != 0 || hidden % (EXL3_TC_STRIP_OUTPUTS * down_strips) != 0) {
         REFUSE("%s: sizes that are no whole number of the products' blocks (%u and %u outputs)", what,
                EXL3_TC_STRIP_OUTPUTS * gate_up_strips, EXL3_TC_STRIP_OUTPUTS * down_strips);

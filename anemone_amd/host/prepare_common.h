@@ -37,4 +37,7 @@ void launch_fill(struct kernel_launch *launch, uint32_t kernel, uint32_t grid_x,
 /* a * b, or UINT64_MAX where the product leaves 64 bits */
 uint64_t product_or_most(uint64_t a, uint64_t b);
 
+/* exl3_tc.c: why the fused EXL3 launches do not take a layer of these sizes, NULL when they do */
+const char *exl3_tc_geometry_refusal(uint32_t hidden, uint32_t intermediate);
+
 #endif
