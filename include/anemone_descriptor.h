@@ -52,7 +52,9 @@ extern "C" {
 #define EXL3_DESCRIPTOR_MATRIX_KINDS 3u /* a routed expert's matrices: gate, up, down */
 #define EXL3_DESCRIPTOR_OPT_IN "--exl3_unrated_map=1"
 
-/* A tensor record as a pack stores it (include/anemone/pack.h:131-146 of the reference; 64 bytes, little-endian) */
+/* A tensor record as a pack stores it (include/anemone/pack.h:131-146 of the reference; 64 bytes, little-endian). A
+ * translation unit that also includes the reference's pack.h includes it first: its struct is then the one used. */
+#ifndef PACK_H
 #define PACK_MAXIMUM_DIMENSIONS 4
 struct pack_tensor {
     uint64_t byte_offset_in_extent;
@@ -67,6 +69,10 @@ struct pack_tensor {
     uint32_t bits_per_weight; /* EXL3: the stored width (K, or 16 K + 8 for a half K) */
     uint32_t reserved_zero[1];
 };
+#endif
+#ifndef __cplusplus
+_Static_assert(sizeof(struct pack_tensor) == 64, "a tensor record as the file stores it");
+#endif
 
 /* What the check reads of an open pack (pack.h:68-82 header fields; :176-186 accessors). The records are sorted by name
  * as unsigned bytes, a shorter name before a longer one it begins (pack.h:17-18); the check verifies that and that
