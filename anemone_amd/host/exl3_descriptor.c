@@ -413,63 +413,66 @@ static bool widths_rule(struct check *check, uint32_t widths, const struct exl3_
            fail(check, STATUS_INVALID_ARGUMENT, "widths: %" PRIu32 " layers, but the model has %" PRIu32, layer_count, model->layers);
 }
 
-struct file_bytes {
-    char *bytes; /* kept files only */
-    uint64_t count;
-    unsigned char digest[SHA256_DIGEST_BYTES];
+/* a file opened for one pass over its bytes */
+struct opened_file {
+    int descriptor;
+    uint64_t size;
 };
 
-/* a regular file of at most most_bytes, read once and hashed; kept whole when `keeps`, else hashed a piece at a time */
-static bool file_read(struct check *check, const char *path, const char *what, uint64_t most_bytes, bool keeps, struct file_bytes *file_out)
+/* opens what must be a regular file of at most most_bytes; `what` names it in a line */
+static bool regular_open(struct check *check, const char *path, const char *what, uint64_t most_bytes, struct opened_file *file_out)
 {
-    /* O_NONBLOCK: a FIFO at the path must not hold the open before it is seen to be no regular file */
-    const int descriptor = open(path, O_RDONLY | O_CLOEXEC | O_NONBLOCK | O_NOCTTY);
     struct stat about;
-    if (descriptor < 0 || fstat(descriptor, &about) != 0) {
+    /* not blocking: a FIFO at the path must not hold the open before it is seen to be no regular file */
+    file_out->descriptor = open(path, O_RDONLY | O_NONBLOCK | O_NOCTTY | O_CLOEXEC);
+    if (file_out->descriptor < 0) {
+        return fail(check, STATUS_INPUT_OUTPUT_ERROR, "%s: cannot be opened (%s)", what, strerror(errno));
+    }
+    if (fstat(file_out->descriptor, &about) != 0) {
         const int error = errno;
-        if (descriptor >= 0) {
-            (void)close(descriptor);
-        }
+        (void)close(file_out->descriptor);
         return fail(check, STATUS_INPUT_OUTPUT_ERROR, "%s: cannot be opened (%s)", what, strerror(error));
     }
-    const uint64_t size = (uint64_t)about.st_size;
-    if (!S_ISREG(about.st_mode) || size > most_bytes) {
-        (void)close(descriptor);
+    if (!S_ISREG(about.st_mode) || (uint64_t)about.st_size > most_bytes) {
+        (void)close(file_out->descriptor);
         return fail(check, STATUS_INVALID_ARGUMENT, "%s: no regular file of at most %" PRIu64 " bytes", what, most_bytes);
     }
-    char *buffer = malloc(keeps ? (size_t)size + 1u : HASH_PIECE_BYTES);
-    if (buffer == NULL) {
-        (void)close(descriptor);
-        return fail(check, STATUS_OUT_OF_MEMORY, "%s: no memory to read it into", what);
-    }
+    file_out->size = (uint64_t)about.st_size;
+    return true;
+}
+
+/* one pass over an opened file, which is closed: its SHA-256, and its bytes into `kept` (size + 1 bytes, a NUL behind
+ * them) when that is not NULL; else a piece at a time through a buffer of the pass's own */
+static bool hashed_through(struct check *check, struct opened_file *file, const char *what, char *kept, unsigned char digest_out[SHA256_DIGEST_BYTES])
+{
+    char *piece = kept != NULL ? NULL : malloc(HASH_PIECE_BYTES);
     struct sha256_stream stream;
+    uint64_t taken = 0;
+    bool is_whole = kept != NULL || piece != NULL;
+    const bool has_memory = is_whole;
     sha256_begin(&stream);
-    uint64_t done = 0;
-    while (done < size) {
-        char *into = keeps ? buffer + done : buffer;
-        const uint64_t left = size - done;
-        const size_t asked = keeps || left < HASH_PIECE_BYTES ? (size_t)left : HASH_PIECE_BYTES;
-        const ssize_t got = pread(descriptor, into, asked, (off_t)done);
-        if (got <= 0) {
-            break;
+    while (is_whole && taken < file->size) {
+        char *into = kept != NULL ? kept + taken : piece;
+        const uint64_t left = file->size - taken;
+        const ssize_t got = read(file->descriptor, into, left < HASH_PIECE_BYTES ? (size_t)left : HASH_PIECE_BYTES);
+        is_whole = got > 0;
+        if (is_whole) {
+            sha256_feed(&stream, into, (uint64_t)got);
+            taken += (uint64_t)got;
         }
-        sha256_feed(&stream, into, (uint64_t)got);
-        done += (uint64_t)got;
     }
-    (void)close(descriptor);
-    if (done < size) {
-        free(buffer);
+    (void)close(file->descriptor);
+    free(piece);
+    if (!has_memory) {
+        return fail(check, STATUS_OUT_OF_MEMORY, "%s: no memory to read it through", what);
+    }
+    if (!is_whole) {
         return fail(check, STATUS_INPUT_OUTPUT_ERROR, "%s: cannot be read whole", what);
     }
-    sha256_finish(&stream, file_out->digest);
-    file_out->count = size;
-    if (keeps) {
-        buffer[size] = '\0';
-        file_out->bytes = buffer;
-    } else {
-        free(buffer);
-        file_out->bytes = NULL;
+    if (kept != NULL) {
+        kept[file->size] = '\0';
     }
+    sha256_finish(&stream, digest_out);
     return true;
 }
 
@@ -526,9 +529,10 @@ static bool quality_rule(struct check *check, uint32_t quality, const char *map,
     memcpy(record, text, text_count);
     record[text_count] = '\0';
     (void)snprintf(named, sizeof named, "quality.record %s", record);
-    struct file_bytes capture = {0};
-    if (!file_read(check, record, named, (uint64_t)INT64_MAX, false, &capture) ||
-        !digest_is(check, found[2], "quality.sha256", capture.digest, "the record's")) {
+    struct opened_file capture;
+    unsigned char capture_digest[SHA256_DIGEST_BYTES];
+    if (!regular_open(check, record, named, (uint64_t)INT64_MAX, &capture) || !hashed_through(check, &capture, named, NULL, capture_digest) ||
+        !digest_is(check, found[2], "quality.sha256", capture_digest, "the record's")) {
         return false;
     }
     (void)snprintf(words_out, words_bytes, "recorded (%s)", record);
@@ -536,7 +540,7 @@ static bool quality_rule(struct check *check, uint32_t quality, const char *map,
 }
 
 /* every rule, in the order of the file's members; the line of a descriptor that holds once all do */
-static bool descriptor_rules(struct check *check, const struct file_bytes *file, const char *map, const struct exl3_pack_view *pack,
+static bool descriptor_rules(struct check *check, const unsigned char file_digest[SHA256_DIGEST_BYTES], const char *map, const struct exl3_pack_view *pack,
                              const struct exl3_descriptor_model *model, const char *tables, uint64_t table_byte_count, bool admits_unrated)
 {
     const struct json_tree *tree = check->tree;
@@ -630,7 +634,7 @@ static bool descriptor_rules(struct check *check, const struct file_bytes *file,
             used += written > 0 ? (size_t)written : 0u;
         }
     }
-    hexadecimal(file->digest, sidecar_digest);
+    hexadecimal(file_digest, sidecar_digest);
     (void)fprintf(stderr, "anemone: exl3 descriptor %s (sha256 %s) holds: model %s, quantiser %.*s, widths %s, quality %s\n", check->sidecar,
                   sidecar_digest, model->model_type, (int)(source_count < 400u ? source_count : 400u), source, widths_words, quality_words);
     return true;
@@ -659,53 +663,76 @@ static bool absent_rule(struct check *check, const struct exl3_pack_view *pack, 
     return true;
 }
 
+/* what the check needs of its arguments before it looks at any file */
+static bool arguments_are_usable(const char *map_path, const struct exl3_pack_view *pack, const struct exl3_descriptor_model *model, const char *tables,
+                                 uint64_t table_byte_count)
+{
+    if (map_path == NULL || pack == NULL || model == NULL || (table_byte_count != 0 && tables == NULL)) {
+        return false;
+    }
+    bool usable = model->model_type != NULL && model->layers != 0 && model->experts_per_layer != 0 &&
+                  (model->established_count == 0 || model->established != NULL);
+    for (uint32_t k = 0; usable && k < EXL3_DESCRIPTOR_MATRIX_KINDS; k++) {
+        usable = model->matrices[k].kind != NULL;
+    }
+    return usable;
+}
+
 result_status exl3_descriptor_check(const char *map_path, const struct exl3_pack_view *pack, const struct exl3_descriptor_model *model,
                                     const char *tables, uint64_t table_byte_count, bool admits_unrated)
 {
-    if (map_path == NULL || pack == NULL || model == NULL || model->model_type == NULL || model->layers == 0 || model->experts_per_layer == 0 ||
-        (model->established == NULL && model->established_count != 0) || (tables == NULL && table_byte_count != 0)) {
+    if (!arguments_are_usable(map_path, pack, model, tables, table_byte_count)) {
         return STATUS_INVALID_ARGUMENT;
-    }
-    for (uint32_t k = 0; k < EXL3_DESCRIPTOR_MATRIX_KINDS; k++) {
-        if (model->matrices[k].kind == NULL) {
-            return STATUS_INVALID_ARGUMENT;
-        }
     }
     if (!view_is_sound(pack)) {
         REFUSE("exl3 descriptor: the pack's tensor records are not sorted by name inside their name bytes");
         return STATUS_INVALID_ARGUMENT;
     }
-    char real[PATH_MAX], sidecar[PATH_MAX];
-    const char *map = realpath(map_path, real) != NULL ? real : map_path;
-    const int length = snprintf(sidecar, sizeof sidecar, "%s" EXL3_DESCRIPTOR_SUFFIX, map);
-    if (length < 0 || (size_t)length >= sizeof sidecar) {
+    /* the sidecar lies beside the map the path leads to; beside the path as given when it leads nowhere */
+    char resolved[PATH_MAX], sidecar[PATH_MAX];
+    const char *map = realpath(map_path, resolved);
+    if (map == NULL) {
+        map = map_path;
+    }
+    if (strlen(map) + sizeof EXL3_DESCRIPTOR_SUFFIX > sizeof sidecar) {
         REFUSE("exl3 descriptor: the map's path %.200s... leaves no room for its sidecar's", map);
         return STATUS_INVALID_ARGUMENT;
     }
+    (void)snprintf(sidecar, sizeof sidecar, "%s%s", map, EXL3_DESCRIPTOR_SUFFIX);
     struct check check = {.sidecar = sidecar, .status = STATUS_OK};
-    struct stat link;
+    struct stat entry;
     /* nothing at the path, not even a link (a link to nothing fails at its open), or nothing can be: a name too long */
-    if (lstat(sidecar, &link) != 0 && (errno == ENOENT || errno == ENAMETOOLONG)) {
-        return absent_rule(&check, pack, model, admits_unrated) ? STATUS_OK : check.status;
+    const bool is_absent = lstat(sidecar, &entry) != 0 && (errno == ENOENT || errno == ENAMETOOLONG);
+    if (is_absent) {
+        (void)absent_rule(&check, pack, model, admits_unrated);
+        return check.status;
     }
-    struct file_bytes file = {0};
-    if (!file_read(&check, sidecar, "the file", EXL3_DESCRIPTOR_MOST_BYTES, true, &file)) {
+    struct opened_file file;
+    unsigned char digest[SHA256_DIGEST_BYTES];
+    if (!regular_open(&check, sidecar, "the file", EXL3_DESCRIPTOR_MOST_BYTES, &file)) {
+        return check.status;
+    }
+    char *text = malloc((size_t)file.size + 1u);
+    if (text == NULL) {
+        (void)close(file.descriptor);
+        (void)fail(&check, STATUS_OUT_OF_MEMORY, "the file: no memory to read it into");
         return check.status;
     }
     struct json_tree tree = {0};
-    const enum json_tree_status read = json_tree_read(file.bytes, (size_t)file.count, &tree);
-    if (read == JSON_TREE_NO_MEMORY) {
-        (void)fail(&check, STATUS_OUT_OF_MEMORY, "no memory to check it in");
-    } else if (read != JSON_TREE_READ) {
-        (void)fail(&check, STATUS_INVALID_ARGUMENT, "the file is not one JSON object");
-    } else {
-        check.tree = &tree;
-        if (!descriptor_rules(&check, &file, map, pack, model, tables, table_byte_count, admits_unrated) && check.status == STATUS_OK) {
-            check.status = STATUS_INVALID_ARGUMENT;
+    if (hashed_through(&check, &file, "the file", text, digest)) {
+        switch (json_tree_read(text, (size_t)file.size, &tree)) {
+        case JSON_TREE_NO_MEMORY: (void)fail(&check, STATUS_OUT_OF_MEMORY, "no memory to check it in"); break;
+        case JSON_TREE_NOT_JSON: (void)fail(&check, STATUS_INVALID_ARGUMENT, "the file is not one JSON object"); break;
+        case JSON_TREE_READ:
+            check.tree = &tree;
+            if (!descriptor_rules(&check, digest, map, pack, model, tables, table_byte_count, admits_unrated) && check.status == STATUS_OK) {
+                check.status = STATUS_INVALID_ARGUMENT; /* not reached: every rule that fails leaves its status */
+            }
+            json_tree_free(&tree);
+            break;
         }
-        json_tree_free(&tree);
     }
-    free(file.bytes);
+    free(text);
     return check.status;
 }
 
