@@ -13,7 +13,6 @@
 #include "exl3_device.cuh"
 #include "kernel_registry.h"
 
-#define STRIP_TILES 8u
 #define PRODUCT_WAVES EXL3_PRODUCT_SLICES
 #define PRODUCT_THREADS (PRODUCT_WAVES * WAVE)
 
@@ -77,8 +76,10 @@ extern "C" __global__ void exl3_input(struct exl3_expert_record record, unsigned
 }
 ANEMONE_KERNEL(EXL3_KERNEL_FILE, exl3_input, exl3_expert_record);
 
-/* Products of one job: block = four wavefronts = the four K slices of one strip of eight output tiles. */
-template <uint32_t bits_x2, bool down>
+/* Products of one job: block = four wavefronts = the four K slices of one strip of STRIP_TILES output tiles (eight; one
+ * in the thin instances, which a launch of few jobs takes so that its blocks cover the card: the same slices and the
+ * same order of sums, so the same bits). */
+template <uint32_t bits_x2, bool down, uint32_t STRIP_TILES>
 __device__ static __forceinline__ void chain_product(const struct exl3_expert_record &record, unsigned char *arena,
                                                      const struct expert_job_record *job, uint32_t *staging,
                                                      float *partial)
@@ -128,7 +129,7 @@ __device__ static __forceinline__ void chain_product(const struct exl3_expert_re
     }
 }
 
-template <uint32_t fixed_bits_x2, bool down>
+template <uint32_t fixed_bits_x2, bool down, uint32_t STRIP_TILES>
 __device__ static __forceinline__ void chain_product_entry(const struct exl3_expert_record &record,
                                                            unsigned char *arena)
 {
@@ -143,10 +144,10 @@ __device__ static __forceinline__ void chain_product_entry(const struct exl3_exp
         bits_x2 = exl3_bits_x2(chain_width(record, arena, job->expert, down ? 2u : blockIdx.z));
     }
     switch (bits_x2) {
-    case 4u: chain_product<4u, down>(record, arena, job, staging, partial); break;
-    case 5u: chain_product<5u, down>(record, arena, job, staging, partial); break;
-    case 6u: chain_product<6u, down>(record, arena, job, staging, partial); break;
-    case 8u: chain_product<8u, down>(record, arena, job, staging, partial); break;
+    case 4u: chain_product<4u, down, STRIP_TILES>(record, arena, job, staging, partial); break;
+    case 5u: chain_product<5u, down, STRIP_TILES>(record, arena, job, staging, partial); break;
+    case 6u: chain_product<6u, down, STRIP_TILES>(record, arena, job, staging, partial); break;
+    case 8u: chain_product<8u, down, STRIP_TILES>(record, arena, job, staging, partial); break;
     default: break;
     }
 }
@@ -155,15 +156,27 @@ __device__ static __forceinline__ void chain_product_entry(const struct exl3_exp
     extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS)                                            \
         exl3_gate_up_##name(struct exl3_expert_record record, unsigned char *arena)                         \
     {                                                                                                        \
-        chain_product_entry<bits_x2, false>(record, arena);                                                  \
+        chain_product_entry<bits_x2, false, EXL3_STRIP_TILES>(record, arena);                                \
     }                                                                                                        \
     ANEMONE_KERNEL(EXL3_KERNEL_FILE, exl3_gate_up_##name, exl3_expert_record);                               \
     extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS)                                            \
         exl3_down_##name(struct exl3_expert_record record, unsigned char *arena)                            \
     {                                                                                                        \
-        chain_product_entry<bits_x2, true>(record, arena);                                                   \
+        chain_product_entry<bits_x2, true, EXL3_STRIP_TILES>(record, arena);                                 \
     }                                                                                                        \
-    ANEMONE_KERNEL(EXL3_KERNEL_FILE, exl3_down_##name, exl3_expert_record)
+    ANEMONE_KERNEL(EXL3_KERNEL_FILE, exl3_down_##name, exl3_expert_record);                                  \
+    extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS)                                            \
+        exl3_gate_up_##name##_thin(struct exl3_expert_record record, unsigned char *arena)                  \
+    {                                                                                                        \
+        chain_product_entry<bits_x2, false, EXL3_THIN_STRIP_TILES>(record, arena);                           \
+    }                                                                                                        \
+    ANEMONE_KERNEL(EXL3_KERNEL_FILE, exl3_gate_up_##name##_thin, exl3_expert_record);                        \
+    extern "C" __global__ void __launch_bounds__(PRODUCT_THREADS)                                            \
+        exl3_down_##name##_thin(struct exl3_expert_record record, unsigned char *arena)                     \
+    {                                                                                                        \
+        chain_product_entry<bits_x2, true, EXL3_THIN_STRIP_TILES>(record, arena);                            \
+    }                                                                                                        \
+    ANEMONE_KERNEL(EXL3_KERNEL_FILE, exl3_down_##name##_thin, exl3_expert_record)
 EXL3_PRODUCT_ENTRIES(k2, 4u);
 EXL3_PRODUCT_ENTRIES(k2_5, 5u);
 EXL3_PRODUCT_ENTRIES(k3, 6u);

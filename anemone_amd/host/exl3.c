@@ -8,6 +8,7 @@
  *   gate/up         exl3_gate_up_<k>|_mixed     (inner_size / 128, jobs, 2)           256  4 K slices x 8 output tiles
  *   activate        exl3_activate               (inner_size / 128, jobs, 1)           64
  *   down            exl3_down_<k>|_mixed        (input_size / 128, jobs, 1)           256
+ *   (a product launch of fewer than EXL3_THIN_BELOW_BLOCKS such blocks: the _thin instance, x = size / 16)
  *   finish          exl3_finish                 (input_size / 128, jobs, 1)           64
  *   row sum         exl3_row_sum                (ceil(width / 256), rows, 1)          256
  *
@@ -122,17 +123,21 @@ static result_status chain_prepare(const struct exl3_expert_record *record, uint
     }
     char gate_up_name[40], down_name[40];
     const char *width = mixed ? "mixed" : exl3_width_name(exl3_bits_x2(record->bits_per_weight));
-    (void)snprintf(gate_up_name, sizeof gate_up_name, "exl3_gate_up_%s", width);
-    (void)snprintf(down_name, sizeof down_name, "exl3_down_%s", width);
+    /* a product launch of few blocks (a job or two) takes the instances of one output tile a block: eight times the
+     * blocks, the same sums */
+    const bool thin_gate_up = (uint64_t)record->inner_size / STRIP_OUTPUTS * record->job_count * 2u < EXL3_THIN_BELOW_BLOCKS;
+    const bool thin_down = (uint64_t)record->input_size / STRIP_OUTPUTS * record->job_count < EXL3_THIN_BELOW_BLOCKS;
+    (void)snprintf(gate_up_name, sizeof gate_up_name, "exl3_gate_up_%s%s", width, thin_gate_up ? "_thin" : "");
+    (void)snprintf(down_name, sizeof down_name, "exl3_down_%s%s", width, thin_down ? "_thin" : "");
     const struct {
         const char *name;
-        uint32_t width, threads, projections;
+        uint32_t width, threads, projections, block_outputs;
     } stages[EXL3_EXPERT_LAUNCHES] = {
-        {"exl3_input", record->input_size, WAVE_THREADS, 2u},
-        {gate_up_name, record->inner_size, PRODUCT_THREADS, 2u},
-        {"exl3_activate", record->inner_size, WAVE_THREADS, 1u},
-        {down_name, record->input_size, PRODUCT_THREADS, 1u},
-        {"exl3_finish", record->input_size, WAVE_THREADS, 1u},
+        {"exl3_input", record->input_size, WAVE_THREADS, 2u, EXL3_TRANSFORM},
+        {gate_up_name, record->inner_size, PRODUCT_THREADS, 2u, (thin_gate_up ? EXL3_THIN_STRIP_TILES : EXL3_STRIP_TILES) * EXL3_TILE},
+        {"exl3_activate", record->inner_size, WAVE_THREADS, 1u, EXL3_TRANSFORM},
+        {down_name, record->input_size, PRODUCT_THREADS, 1u, (thin_down ? EXL3_THIN_STRIP_TILES : EXL3_STRIP_TILES) * EXL3_TILE},
+        {"exl3_finish", record->input_size, WAVE_THREADS, 1u, EXL3_TRANSFORM},
     };
     struct kernel_launch launches[EXL3_EXPERT_LAUNCHES];
     for (uint32_t stage = 0; stage < EXL3_EXPERT_LAUNCHES; stage++) {
@@ -145,8 +150,9 @@ static result_status chain_prepare(const struct exl3_expert_record *record, uint
         if (kernel == BACKEND_NO_KERNEL) {
             return STATUS_UNSUPPORTED;
         }
-        _Static_assert(STRIP_OUTPUTS == EXL3_TRANSFORM, "a strip of outputs and a transform block are both 128 wide");
-        launch_fill(&launches[stage], kernel, stages[stage].width / EXL3_TRANSFORM, record->job_count,
+        _Static_assert(STRIP_OUTPUTS == EXL3_STRIP_TILES * EXL3_TILE && STRIP_OUTPUTS == EXL3_TRANSFORM,
+                       "a strip of outputs and a transform block are both 128 wide");
+        launch_fill(&launches[stage], kernel, stages[stage].width / stages[stage].block_outputs, record->job_count,
                     stages[stage].projections, stages[stage].threads, 0, record, sizeof *record);
     }
     memcpy(launches_out, launches, sizeof launches);

@@ -666,7 +666,7 @@ def exl3_linear(amd, workloads, arguments):
     step = amd.launches_of(3)
     step[0], step[1], step[2] = launches[0], launches[3], launches[4]  # input, the product of one matrix, finish
     step[0].grid[2] = 1
-    names = ["exl3_input", "exl3_down_k4", "exl3_finish"]
+    names = ["exl3_input", "exl3_down_k4_thin", "exl3_finish"]  # one job: the product kernel of one output tile a block
     queue_steps(card, step, arguments.warmup, None)
     card.wait()
     device_us = card.measure(lambda: queue_steps(card, step, arguments.steps, None))
@@ -685,7 +685,7 @@ def exl3_linear(amd, workloads, arguments):
         "config": {"workload": "exl3_linear: one matrix 4096 x 4096, K 4, batch 1 (BASELINE configuration 0)",
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "step_GBps": algorithmic / (seconds / arguments.steps) / 1e9},
-        "roofline": {"bound": "hbm", "kernel": "exl3_down_k4 (the product launch)", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "roofline": {"bound": "hbm", "kernel": "exl3_down_k4_thin (the product launch)", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": int(algorithmic), "launch_us": product_us},
     }
     got = card.download(record.output_offset, n * 4, np.float32)

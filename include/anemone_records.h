@@ -202,6 +202,9 @@ ANEMONE_RECORD_HAS(router_wide_arguments, 136);
 #define EXL3_NORMALIZATION 0.08838834764831845f
 #define EXL3_EXPERT_LAUNCHES 5u
 #define EXL3_PRODUCT_SLICES 4u
+#define EXL3_STRIP_TILES 8u      /* output tiles of a block of the chain's product launches: 128 outputs */
+#define EXL3_THIN_STRIP_TILES 1u /* of the _thin instances, which a launch of fewer than EXL3_THIN_BELOW_BLOCKS blocks takes */
+#define EXL3_THIN_BELOW_BLOCKS 256u
 
 #ifdef __cplusplus
 #define ANEMONE_INLINE __host__ __device__ static constexpr inline

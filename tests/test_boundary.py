@@ -130,6 +130,16 @@ def test_chain_prepare_geometry(fake):
     mixed = amd.launches_of(5)
     assert lib.exl3_experts_prepare(C.byref(chain_record(widths_offset=1 << 30)), ARENA, fake.address, fake.card, 950, mixed) == 0
     assert fake.handles[mixed[1].kernel][1] == "exl3_gate_up_mixed" and fake.handles[mixed[3].kernel][1] == "exl3_down_mixed"
+    # product launches of fewer than 256 blocks take the instances of one output tile a block (eight times the blocks)
+    for jobs, pairs, names, grids in ((1, 8, ["exl3_gate_up_k3_thin", "exl3_down_k3_thin"], [[128, 1, 2], [256, 1, 1]]),
+                                      (7, 8, ["exl3_gate_up_k3_thin", "exl3_down_k3_thin"], [[128, 7, 2], [256, 7, 1]]),
+                                      (8, 8, ["exl3_gate_up_k3", "exl3_down_k3"], [[16, 8, 2], [32, 8, 1]])):
+        few = amd.launches_of(5)
+        assert lib.exl3_experts_prepare(C.byref(chain_record(job_count=jobs, pair_count=pairs)), ARENA, fake.address, fake.card, 950, few) == 0
+        assert [fake.handles[few[i].kernel][1] for i in (1, 3)] == names and [list(few[i].grid) for i in (1, 3)] == grids
+        assert [list(few[i].grid) for i in (0, 2, 4)] == [[32, jobs, 2], [16, jobs, 1], [32, jobs, 1]]
+    assert lib.exl3_experts_prepare(C.byref(chain_record(job_count=1, pair_count=8, widths_offset=1 << 30)), ARENA, fake.address, fake.card, 950, mixed) == 0
+    assert fake.handles[mixed[1].kernel][1] == "exl3_gate_up_mixed_thin" and fake.handles[mixed[3].kernel][1] == "exl3_down_mixed_thin"
     assert lib.exl3_scratch_byte_count(64, 4096) == 64 * 4096 * 12
     assert lib.exl3_width_name(6) == b"k3" and lib.exl3_width_name(5) == b"k2_5" and lib.exl3_width_name(7) is None
 

@@ -256,6 +256,45 @@ def test_single_linear_config0_shape(amd, card):
 
 
 @pytest.mark.parametrize("width", [2, 40, 3, 4])
+def test_thin_product_instances_give_the_same_bits(amd, card, width):
+    """A chain of one or two jobs takes the product kernels of one output tile a block (exl3_gate_up_<k>_thin,
+    exl3_down_<k>_thin: anemone_amd/host/exl3.c); the same chain with room for 64 jobs (the others empty) takes the
+    kernels of eight tiles a block. Same K slices, same order of sums: every float32 product and output bit for bit."""
+    say("thin product instances, width", width)
+    hidden, inner, pairs = 512, 256, 2
+    matrices = [exl3_matrix(0x7100 + width * 8 + m, *((inner, hidden) if m < 2 else (hidden, inner)), width) for m in range(3)]
+    places = [card.place(m, 256) for m in matrices]
+    x = to_bf16(normals(0x7200 + width, pairs * hidden)).reshape(pairs, hidden)
+    outputs = []
+    for job_count in (1, 64):
+        jobs = np.zeros(job_count, dtype=JOB_DTYPE)
+        jobs[0]["gate_offset"], jobs[0]["up_offset"], jobs[0]["down_offset"] = places
+        jobs[0]["row_count"] = pairs
+        jobs[0]["pair_index"][:pairs] = np.arange(pairs)
+        jobs[0]["route_weight"][:pairs] = [0.75, 1.5]
+        record = amd.Exl3ExpertRecord()
+        record.jobs_offset = card.place(jobs.view(np.uint8))
+        record.input_offset = card.place(x)
+        record.operands_offset = card.reserve(pairs * hidden * 4)
+        record.products_offset = record.output_offset = card.reserve(pairs * hidden * 8)
+        record.hidden_offset = card.reserve(pairs * inner * 2)
+        record.input_size, record.inner_size = hidden, inner
+        record.pair_count, record.pairs_per_row, record.job_count = pairs, 1, job_count
+        record.bits_per_weight, record.activation_limit = width, 10.0
+        launches = amd.launches_of(5)
+        amd.check(card.lib.exl3_experts_prepare(C.byref(record), card.arena_bytes, amd.backend_table(), card.handle, 950, launches), "prepare")
+        assert list(launches[1].grid) == ([inner // 16, 1, 2] if job_count == 1 else [inner // 128, 64, 2])
+        card.upload(record.output_offset, np.full(pairs * hidden * 8, 0xEE, dtype=np.uint8))
+        card.run(launches[0:2])
+        products = card.download(record.products_offset, 2 * pairs * inner * 4, np.uint32).copy()
+        card.run(launches[2:5])
+        outputs.append((products, card.download(record.output_offset, pairs * hidden * 4, np.uint32).copy()))
+    assert np.array_equal(outputs[0][0], outputs[1][0]), "the gate and up products"
+    assert np.array_equal(outputs[0][1], outputs[1][1]), "the outputs"
+    assert not np.all(outputs[0][1] == 0xEEEEEEEE)
+
+
+@pytest.mark.parametrize("width", [2, 40, 3, 4])
 def test_a_slice_of_outputs_gives_the_whole_matrix_bits(amd, card, width):
     """The load-time slices (bb_exl3_matrix_slice_copy, include/anemone/exl3_layout.h:28-49 of the reference): a slice of
     a matrix's outputs with all of its inputs, as its own stored matrix, through the chain's input and gate product
