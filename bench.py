@@ -30,6 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # under profiles/ hold the commands and the counts), reported as roofline.traffic when a run has the same sizes
 MEASURED_TRAFFIC_BYTES = {
     ("exl3_decode", 8): 375.1e6 + 4.2e6,
+    ("exl3_linear", 1): 8.495e6 + 0.016e6,
     ("fp4_decode", 32): 1434.7e6 + 1.0e6,
     ("fp8_decode", 32): 2746.8e6 + 1.0e6,
     ("fp4_prefill", 8192): 4777.9e6 + 447.0e6,
@@ -45,6 +46,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("fp8_decode_native", 32): 2746.7e6 + 1.0e6,
 }
 TRAFFIC_SOURCE = {
+    "exl3_linear": "profiles/exl3_down_k4_thin_single_linear.md",
     "exl3_decode": "profiles/exl3_tc_products_decode8.md", "exl3_prefill": "profiles/exl3_tcp_gemm_prefill4096.md", "fp4_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md",
     "fp8_decode": "profiles/expert_gate_up_fp4_fp8_decode32.md", "fp4_prefill": "profiles/wide_expert_fp4_fp8_prefill.md",
     "fp8_prefill": "profiles/wide_expert_fp4_fp8_prefill.md",
@@ -686,7 +688,9 @@ def exl3_linear(amd, workloads, arguments):
                    "launch_us": {name: round(float(us), 2) for name, us in zip(names, per_launch)},
                    "step_GBps": algorithmic / (seconds / arguments.steps) / 1e9},
         "roofline": {"bound": "hbm", "kernel": "exl3_down_k4_thin (the product launch)", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": int(algorithmic), "launch_us": product_us},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES[("exl3_linear", 1)],
+                     "traffic_source": TRAFFIC_SOURCE["exl3_linear"] + " (counter bytes of the profiled run, not of this one)",
+                     "algorithmic_bytes_per_launch": int(algorithmic), "launch_us": product_us},
     }
     got = card.download(record.output_offset, n * 4, np.float32)
     card.close()
