@@ -739,7 +739,9 @@ def summary(result):
 # the workloads of the other configurations the metric names, as the default run's config.also: (workload, rows, block128, gfx950 lane order)
 ALSO = [("exl3_linear", 1, False, False), ("exl3_prefill", 4096, False, False), ("fp8_decode", 1, True, False), ("fp8_decode", 64, True, False),
         ("fp8_prefill", 2048, True, False), ("fp8_prefill", 2048, True, True), ("fp8_prefill", 2048, False, False), ("fp8_prefill", 2048, False, True),
-        ("fp4_prefill", 8192, False, False), ("fp4_prefill", 8192, False, True), ("fp4_decode", 32, False, False), ("fp4_decode", 32, False, True)]
+        ("fp4_prefill", 8192, False, False), ("fp4_prefill", 8192, False, True), ("fp4_decode", 32, False, False), ("fp4_decode", 32, False, True),
+        # configuration 4 is reported against the FP8 run of configuration 3 on the same inputs: that scaling at its sizes
+        ("fp8_prefill", 8192, True, True), ("fp8_decode", 32, True, False)]
 # the other configurations' headline fractions as scalars of config (beside config.also, which holds the whole lines)
 HEADLINES = {("exl3_linear", False, False): "exl3_linear_hbm_frac", ("exl3_prefill", False, False): "exl3_prefill_mfma_frac",
              ("fp8_prefill", True, False): "fp8_block128_prefill_hbm_frac", ("fp8_prefill", True, True): "fp8_block128_gfx950_prefill_hbm_frac",
@@ -816,10 +818,14 @@ def main():
         entry = summary(run(workload, options))
         entry["bench_seconds"] = time.perf_counter() - start
         also.append(entry)
-        if (workload, block128, native) in HEADLINES:
+        if (workload, block128, native) in HEADLINES and not (workload == "fp8_prefill" and rows != 2048):
             result["config"][HEADLINES[(workload, block128, native)]] = entry["frac"]
         if workload == "fp8_decode":
             result["config"]["fp8_block128_decode%d_hbm_frac" % rows] = entry["frac"]
+    # the FP4 layer's steps against the FP8 layer's (float32 block scales) on the same rows: tokens a second, FP4 over FP8
+    rate = {(w, r, b, n): e["tok_s"] for (w, r, b, n), e in zip(ALSO, also)}
+    result["config"]["fp4_over_fp8_prefill8192_tok_s"] = rate[("fp4_prefill", 8192, False, True)] / rate[("fp8_prefill", 8192, True, True)]
+    result["config"]["fp4_over_fp8_decode32_tok_s"] = rate[("fp4_decode", 32, False, True)] / rate[("fp8_decode", 32, True, False)]
     result["config"]["also"] = also
     print(json.dumps(result))
 
