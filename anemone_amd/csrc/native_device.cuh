@@ -14,6 +14,7 @@
 #define NATIVE_DEVICE_CUH
 
 #include "linear_device.cuh"
+#include "native_waits.h"
 
 #define NATIVE_WAVES 4u
 /* one-byte weights: a step's next weights are asked for at its top, ahead of the columns' preparation and the barrier
@@ -275,36 +276,12 @@ struct native_chain {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the stage is read before the next barrier */
     }
 
-    /* How many loads may be outstanding at the top of K step `step` for its columns and weights to have landed. Loads in
-     * the order they are asked for: the columns of steps 0 .. DEPTH - 2, the weights of steps 0 .. SLOTS - 2, then, in
-     * every step j, the columns of step j + DEPTH - 1 and behind them the weights of step j + SLOTS - 1 (where the chain
-     * has such steps; with WEIGHTS_FIRST the weights, then the columns). The count is of the loads of later steps asked for behind the later of the two. */
+    /* how many loads may be outstanding at the top of a K step for its columns and weights to have landed: native_waits.h */
     static constexpr bool WEIGHTS_FIRST = NATIVE_WEIGHTS_FIRST_OF(BYTES); /* inside a step: the weights asked for ahead of the columns */
-    __device__ static __forceinline__ uint32_t when_columns(uint32_t k)
-    {
-        return k < DEPTH - 1u ? k : 64u * (1u + k - (DEPTH - 1u)) + (WEIGHTS_FIRST ? 1u : 0u);
-    }
-
-    __device__ static __forceinline__ uint32_t when_weights(uint32_t k)
-    {
-        return k < SLOTS - 1u ? DEPTH - 1u + k : 64u * (1u + k - (SLOTS - 1u)) + (WEIGHTS_FIRST ? 0u : 1u);
-    }
-
+    typedef native_waits<SLOTS, DEPTH, WEIGHTS_FIRST, VECTOR_LOADS, WEIGHT_LOADS> waits;
     __device__ static __forceinline__ uint32_t loads_behind(uint32_t step, uint32_t total)
     {
-        static_assert(SLOTS >= DEPTH && DEPTH >= 2u && SLOTS + DEPTH < 64u, "the weights are asked for at least as far ahead as the columns");
-        const uint32_t mine = when_columns(step) > when_weights(step) ? when_columns(step) : when_weights(step);
-        const uint32_t now = 64u * (1u + step); /* what steps before this one asked for lies below this */
-        uint32_t count = 0;
-#pragma unroll
-        for (uint32_t ahead = 1; ahead < SLOTS; ahead++) {
-            const uint32_t k = step + ahead;
-            if (k < total) {
-                count += when_columns(k) > mine && when_columns(k) < now ? VECTOR_LOADS : 0u;
-                count += when_weights(k) > mine && when_weights(k) < now ? WEIGHT_LOADS : 0u;
-            }
-        }
-        return count;
+        return waits::loads_behind(step, total);
     }
 
     /* s_waitcnt takes its count as a constant: one instruction a count that loads_behind can come to */
