@@ -397,6 +397,9 @@ def test_the_readers_grammar_is_json_loads(capfd, place):
     m = model_of(layers=1, experts_per_layer=2)
     base = json.dumps(small_descriptor())
     expect(capfd, place, p, base, OK, "widths K3 6", model=m)
+    # as the converter writes it (tools/convert/make_virtual_pack.py:350 of the reference): json.dumps(descriptor, indent=1) and a line feed
+    expect(capfd, place, p, json.dumps(small_descriptor(), indent=1) + "\n", OK, "widths K3 6", model=m)
+    expect(capfd, place, p, json.dumps(small_descriptor(), indent=1, ensure_ascii=False, sort_keys=True) + "\n", OK, "widths K3 6", model=m)
     slot = '"architectures": []'
     assert slot in base
     accepted = ['[1, -0, 1.5e+3, -2E-7, 0.0, NaN, Infinity, -Infinity, true, false, null]', '"\\u00e9\\ud83d\\ude00\\"\\\\\\/\\b\\f\\n\\r\\t"', '"é\U0001F600"',
