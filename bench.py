@@ -38,9 +38,9 @@ MEASURED_TRAFFIC_BYTES = {
     ("expert_join", 8192): 877.7e6 + 402.7e6,
     ("fp8_decode_block128", 64): 3713.0e6 + 2.1e6,
     ("fp8_prefill_block128", 2048): 5386.8e6 + 67.2e6,
-    ("fp4_prefill_native", 8192): 5530.8e6 + 415.4e6,
+    ("fp4_prefill_native", 8192): 5500.8e6 + 421.1e6,
     ("exl3_prefill", 4096): 2858.6e6 + 538.5e6,
-    ("fp8_prefill_native", 2048): 4711.2e6 + 113.3e6,
+    ("fp8_prefill_native", 2048): 4711.8e6 + 113.5e6,
     ("fp8_prefill_block128_native", 2048): 4693.9e6 + 67.1e6,
     ("fp4_decode_native", 32): 1434.2e6 + 1.0e6,
     ("fp8_decode_native", 32): 2746.7e6 + 1.0e6,
