@@ -449,7 +449,7 @@ def test_wide_router_prepare(fake):
     assert names == ["router_wide_select", "router_wide_count", "router_wide_place", "router_wide_jobs"]
     assert [list(l.grid) for l in launches] == [[512, 1, 1], [11, 1, 1], [11, 1, 1], [1, 1, 1]]
     assert all(l.block[0] == 512 and l.argument_byte_count == 136 for l in launches)
-    assert amd.wide_tile_count(4096, 8, 256) == 768 and amd.wide_job_count(4096, 8, 256) == 4320  # the survey's figures
+    assert amd.wide_tile_count(4096, 8, 256) == 768 and amd.wide_job_count(4096, 8, 256) == 4320  # 32768 pairs over 256 experts: at most pairs / 64 + experts tiles and (pairs + 7 experts) / 8 jobs
     for changes in (dict(row_count=0), dict(row_count=70000), dict(expert_count=100), dict(pick_count=0), dict(route_scale=-1.0),
                     dict(reserved_zero=1), dict(weight_format=1), dict(jobs=amd.Range(1 << 27, 96))):
         bad, keep = wide_description(**changes)
