@@ -78,6 +78,16 @@ def run_wide(card, layer, x, live):
     (640, 384, 64, 2, 450, 449, B128),
     (512, 256, 64, 8, 1500, 1401, B128),
     (512, 256, 64, 1, 4300, 4300, -B128),
+    # chains of one, two and three K steps: fewer steps than sets of weight registers and stages of columns
+    (128, 128, 64, 4, 300, 300, E2M1),
+    (256, 128, 64, 4, 300, 297, E2M1),
+    (384, 256, 64, 2, 500, 500, E2M1),
+    (128, 128, 64, 4, 600, 600, E4M3),
+    (256, 128, 64, 8, 300, 300, E4M3),
+    (384, 256, 64, 2, 500, 499, E4M3),
+    (128, 128, 64, 4, 600, 600, B128),
+    (256, 128, 64, 8, 300, 299, B128),
+    (384, 256, 64, 2, 500, 500, B128),
 ])
 def test_native_equals_the_reference_lay_out_byte_for_byte(amd, card, hidden, inner, experts_n, picks, rows, live, fmt):
     say("native experts", hidden, inner, experts_n, picks, rows, live, fmt)
@@ -163,6 +173,10 @@ def run_jobs(card, layer, x, live):
     (640, 384, 8, 2, 2, B128, 1, 2),
     (1024, 512, 1, 8, 5, B128, 8, 4),
     (640, 384, 2, 5, 5, B128, 2, 1),
+    (128, 128, 4, 8, 8, E2M1, 1, 1),     # one K step
+    (256, 128, 4, 8, 7, E4M3, 2, 1),     # two K steps over two slices: a step a chain
+    (128, 128, 2, 6, 6, B128, 1, 1),
+    (384, 256, 8, 4, 4, E2M1, 1, 2),
 ])
 def test_native_job_table_kernels_equal_the_reference_lay_out(amd, card, hidden, inner, picks, rows, live, fmt, gate_up_slices, down_slices):
     """The job-table kernels (a thin step's) of the formats in gfx950's lane order, expert_gate_up_gfx950_<S> and its like:
