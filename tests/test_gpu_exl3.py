@@ -255,21 +255,25 @@ def test_single_linear_config0_shape(amd, card):
 
 
 
-@pytest.mark.parametrize("width", [2, 40, 3, 4])
+@pytest.mark.parametrize("width", [2, 40, 3, 4, (3, 2, 4)])
 def test_thin_product_instances_give_the_same_bits(amd, card, width):
     """A chain of one or two jobs takes the product kernels of one output tile a block (exl3_gate_up_<k>_thin,
     exl3_down_<k>_thin: anemone_amd/host/exl3.c); the same chain with room for 64 jobs (the others empty) takes the
     kernels of eight tiles a block. Same K slices, same order of sums: every float32 product and output bit for bit."""
     say("thin product instances, width", width)
     hidden, inner, pairs = 512, 256, 2
-    matrices = [exl3_matrix(0x7100 + width * 8 + m, *((inner, hidden) if m < 2 else (hidden, inner)), width) for m in range(3)]
+    widths = width if isinstance(width, tuple) else (width,) * 3  # a tuple: a width a matrix, through the record's widths table
+    mixed = isinstance(width, tuple)
+    width = widths[0]
+    matrices = [exl3_matrix(0x7100 + widths[m] * 8 + m, *((inner, hidden) if m < 2 else (hidden, inner)), widths[m]) for m in range(3)]
+    widths_at = card.place(np.full(4, widths[0] | widths[1] << 8 | widths[2] << 16, dtype=np.uint32)) if mixed else 0
     places = [card.place(m, 256) for m in matrices]
     x = to_bf16(normals(0x7200 + width, pairs * hidden)).reshape(pairs, hidden)
     outputs = []
     for job_count in (1, 64):
         jobs = np.zeros(job_count, dtype=JOB_DTYPE)
         jobs[0]["gate_offset"], jobs[0]["up_offset"], jobs[0]["down_offset"] = places
-        jobs[0]["row_count"] = pairs
+        jobs[0]["row_count"], jobs[0]["expert"] = pairs, 3
         jobs[0]["pair_index"][:pairs] = np.arange(pairs)
         jobs[0]["route_weight"][:pairs] = [0.75, 1.5]
         record = amd.Exl3ExpertRecord()
@@ -280,7 +284,7 @@ def test_thin_product_instances_give_the_same_bits(amd, card, width):
         record.hidden_offset = card.reserve(pairs * inner * 2)
         record.input_size, record.inner_size = hidden, inner
         record.pair_count, record.pairs_per_row, record.job_count = pairs, 1, job_count
-        record.bits_per_weight, record.activation_limit = width, 10.0
+        record.bits_per_weight, record.activation_limit, record.widths_offset = width, 10.0, widths_at
         launches = amd.launches_of(5)
         amd.check(card.lib.exl3_experts_prepare(C.byref(record), card.arena_bytes, amd.backend_table(), card.handle, 950, launches), "prepare")
         assert list(launches[1].grid) == ([inner // 16, 1, 2] if job_count == 1 else [inner // 128, 64, 2])
