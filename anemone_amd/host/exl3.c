@@ -83,10 +83,12 @@ static result_status chain_prepare(const struct exl3_expert_record *record, uint
                ARITHMETIC_CLASS_GFX950);
         return STATUS_INVALID_ARGUMENT;
     }
-    if (record->reserved_zero != 0 || record->pair_count == 0 || record->pairs_per_row == 0 ||
-        record->pair_count % record->pairs_per_row != 0 || record->output_offset != record->products_offset ||
-        record->job_count == 0 || record->job_count > MOST_GRID_ROWS || record->inner_size > record->input_size ||
-        !isfinite(record->activation_limit) || !(record->activation_limit > 0.0f)) {
+    const bool whole_rows = record->pairs_per_row >= 1u && record->pair_count >= 1u && record->pair_count % record->pairs_per_row == 0u;
+    const bool jobs_fit_a_grid = record->job_count >= 1u && record->job_count <= MOST_GRID_ROWS;
+    const bool sums_in_place = record->products_offset == record->output_offset; /* the finish launch overwrites the products it reads */
+    const bool limit_holds = isfinite(record->activation_limit) && record->activation_limit > 0.0f;
+    if (!whole_rows || !jobs_fit_a_grid || !sums_in_place || !limit_holds || record->input_size < record->inner_size ||
+        record->reserved_zero != 0) {
         REFUSE("%s: counts, the in-place output rule or the activation limit", what);
         return STATUS_INVALID_ARGUMENT;
     }

@@ -3,17 +3,18 @@
 
 const char *status_text(result_status status)
 {
-    static const char *const phrases[STATUS_COUNT] = {
-        [STATUS_OK] = "ok",
-        [STATUS_INVALID_ARGUMENT] = "invalid argument",
-        [STATUS_OUT_OF_MEMORY] = "out of memory",
-        [STATUS_INPUT_OUTPUT_ERROR] = "input/output error",
-        [STATUS_CORRUPT_PACK] = "corrupt pack",
-        [STATUS_DEVICE_ERROR] = "device error",
-        [STATUS_TIMED_OUT] = "timed out",
-        [STATUS_UNSUPPORTED] = "unsupported",
-        [STATUS_BUSY_VALUE] = "busy",
-        [STATUS_INJECTED_FAULT] = "injected fault",
-    };
-    return (unsigned)status < STATUS_COUNT ? phrases[status] : "unknown status";
+    switch (status) {
+    case STATUS_OK: return "ok";
+    case STATUS_INVALID_ARGUMENT: return "invalid argument";
+    case STATUS_OUT_OF_MEMORY: return "out of memory";
+    case STATUS_INPUT_OUTPUT_ERROR: return "input/output error";
+    case STATUS_CORRUPT_PACK: return "corrupt pack";
+    case STATUS_DEVICE_ERROR: return "device error";
+    case STATUS_TIMED_OUT: return "timed out";
+    case STATUS_UNSUPPORTED: return "unsupported";
+    case STATUS_BUSY_VALUE: return "busy";
+    case STATUS_INJECTED_FAULT: return "injected fault";
+    case STATUS_COUNT: break; /* not a status */
+    }
+    return "unknown status";
 }
